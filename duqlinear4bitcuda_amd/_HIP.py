@@ -1,0 +1,287 @@
+"""Tensor-level ops with the names and signatures of the reference's pybind11 module
+``qlinear4bit._CUDA`` (src/export/bindings.cpp:768-932), for the Linear4bit path.
+
+Each op checks its tensors the way the reference binding does (contiguous, on a GPU,
+same device, matching sizes), allocates its output with ``torch.empty`` on the input's
+device, and calls the C ABI on the current torch stream.  Argument errors raise
+``RuntimeError`` as ``torch::check*`` does in the reference.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+_QUANT_COL_K = 10
+
+
+def _stream(t: torch.Tensor):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _check(name, *tensors):
+    dev = None
+    for i, t in enumerate(tensors):
+        if not isinstance(t, torch.Tensor):
+            raise RuntimeError(f"{name}: argument #{i} is not a tensor")
+        if not t.is_contiguous():
+            raise RuntimeError(f"{name}: expected argument #{i} to be contiguous")
+        if not t.is_cuda:
+            raise RuntimeError(f"{name}: expected argument #{i} to be on a GPU device, got {t.device}")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise RuntimeError(f"{name}: expected all tensors on {dev}, argument #{i} is on {t.device}")
+
+
+def _check_size0(name, t, what, n):
+    if t.dim() < 1 or t.size(0) != n:
+        raise RuntimeError(f"{name}: expected {what} to have size {n} at dimension 0, got {tuple(t.shape)}")
+
+
+def _check_dtype(name, t, what, dtype):
+    if t.dtype != dtype:
+        raise RuntimeError(f"{name}: expected {what} to have dtype {dtype}, got {t.dtype}")
+
+
+def _ptr(t):
+    return t.data_ptr() if t is not None else None
+
+
+def matmul(A: torch.Tensor, B: torch.Tensor) -> torch.Tensor:
+    """int4Unpack(A) @ int4Unpack(B)^T -> int32 [M, N] (bindings.cpp:10-26)."""
+    _check("matmul", A, B)
+    _check_dtype("matmul", A, "A", torch.uint8)
+    _check_dtype("matmul", B, "B", torch.uint8)
+    M, N, K = A.size(0), B.size(0), A.size(1) * 2
+    if B.size(1) != A.size(1):
+        raise RuntimeError(f"matmul: packed K differs: A {tuple(A.shape)} vs B {tuple(B.shape)}")
+    C = torch.empty((M, N), dtype=torch.int32, device=A.device)
+    with torch.cuda.device(A.device):
+        st = _lib.load().duq_matmul_host_4bit(_ptr(A), _ptr(B), M, N, K, _ptr(C), _stream(A))
+    _lib.check(st, "matmul")
+    return C
+
+
+def sym_quant(x: torch.Tensor, scale: torch.Tensor, qmax: int = 6) -> torch.Tensor:
+    """int4Pack(clamp(rint(x / scale), -8, qmax)) -> uint8 [M, ceil(K/2)] (bindings.cpp:88-105).
+    ``qmax`` defaults to 6, the bound the reference device kernel really applies
+    (include/common.h:53-54)."""
+    _check("sym_quant", x, scale)
+    _check_dtype("sym_quant", x, "x", torch.float16)
+    _check_dtype("sym_quant", scale, "scale", torch.float16)
+    _check_size0("sym_quant", scale, "scale", x.size(0))
+    rows, cols = x.size(0), x.size(1)
+    cd = (cols + 1) // 2
+    q = torch.empty((rows, cd), dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        st = _lib.load().duq_sym_quant_host_qmax(_ptr(x), _ptr(scale), rows, cols, cd, qmax, _ptr(q), _stream(x))
+    _lib.check(st, "sym_quant")
+    return q
+
+
+def sym_dual_quant(x, scale_1, scale_2):
+    """bindings.cpp:107-127."""
+    _check("sym_dual_quant", x, scale_1, scale_2)
+    for t, n in ((x, "x"), (scale_1, "scale_1"), (scale_2, "scale_2")):
+        _check_dtype("sym_dual_quant", t, n, torch.float16)
+    _check_size0("sym_dual_quant", scale_1, "scale_1", x.size(0))
+    _check_size0("sym_dual_quant", scale_2, "scale_2", x.size(0))
+    rows, cols = x.size(0), x.size(1)
+    cd = (cols + 1) // 2
+    q = torch.empty((rows, cd), dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        st = _lib.load().duq_sym_dual_quant_host(_ptr(x), _ptr(scale_1), _ptr(scale_2), rows, cols, cd, _ptr(q),
+                                                 _stream(x))
+    _lib.check(st, "sym_dual_quant")
+    return q
+
+
+def asym_quant(x, scale, zeros):
+    """bindings.cpp:221-243."""
+    _check("asym_quant", x, scale, zeros)
+    for t, n in ((x, "x"), (scale, "scale"), (zeros, "zeros")):
+        _check_dtype("asym_quant", t, n, torch.float16)
+    _check_size0("asym_quant", scale, "scale", x.size(0))
+    _check_size0("asym_quant", zeros, "zeros", x.size(0))
+    rows, cols = x.size(0), x.size(1)
+    cd = (cols + 1) // 2
+    q = torch.empty((rows, cd), dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        st = _lib.load().duq_asym_quant_host(_ptr(x), _ptr(scale), _ptr(zeros), rows, cols, cd, _ptr(q), _stream(x))
+    _lib.check(st, "asym_quant")
+    return q
+
+
+def asym_dual_quant(x, scale_1, zeros_1, scale_2, zeros_2):
+    """bindings.cpp:393-421 (whose body forgets to return q; this one returns it)."""
+    ts = (x, scale_1, zeros_1, scale_2, zeros_2)
+    _check("asym_dual_quant", *ts)
+    for t, n in zip(ts, ("x", "scale_1", "zeros_1", "scale_2", "zeros_2")):
+        _check_dtype("asym_dual_quant", t, n, torch.float16)
+        if t is not x:
+            _check_size0("asym_dual_quant", t, n, x.size(0))
+    rows, cols = x.size(0), x.size(1)
+    cd = (cols + 1) // 2
+    q = torch.empty((rows, cd), dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        st = _lib.load().duq_asym_dual_quant_host(_ptr(x), _ptr(scale_1), _ptr(zeros_1), _ptr(scale_2),
+                                                  _ptr(zeros_2), rows, cols, cd, _ptr(q), _stream(x))
+    _lib.check(st, "asym_dual_quant")
+    return q
+
+
+def _check_bits(name, bits):
+    if bits != 32:
+        raise RuntimeError(f"{name}: Unsupported data type")  # bindings.cpp:159-167
+
+
+def sym_dequant(q, scale_row, scale_col, bits: int = 32):
+    """bindings.cpp:130-170."""
+    _check("sym_dequant", q, scale_row, scale_col)
+    _check_dtype("sym_dequant", q, "q", torch.int32)
+    _check_dtype("sym_dequant", scale_row, "scale_row", torch.float16)
+    _check_dtype("sym_dequant", scale_col, "scale_col", torch.float16)
+    rows, cols = q.size(0), q.size(1)
+    _check_size0("sym_dequant", scale_row, "scale_row", rows)
+    _check_size0("sym_dequant", scale_col, "scale_col", cols)
+    _check_bits("sym_dequant", bits)
+    x = torch.empty(q.shape, dtype=torch.float16, device=q.device)
+    with torch.cuda.device(q.device):
+        st = _lib.load().duq_sym_dequant_host(_ptr(q), _ptr(scale_row), _ptr(scale_col), rows, cols, _ptr(x),
+                                              _stream(q))
+    _lib.check(st, "sym_dequant")
+    return x
+
+
+def sym_dual_dequant(q, scale_row, scale_col_1, scale_col_2, bits: int = 32):
+    """bindings.cpp:172-217."""
+    ts = (q, scale_row, scale_col_1, scale_col_2)
+    _check("sym_dual_dequant", *ts)
+    _check_dtype("sym_dual_dequant", q, "q", torch.int32)
+    for t, n in zip(ts[1:], ("scale_row", "scale_col_1", "scale_col_2")):
+        _check_dtype("sym_dual_dequant", t, n, torch.float16)
+    rows, cols = q.size(0), q.size(1)
+    _check_size0("sym_dual_dequant", scale_row, "scale_row", rows)
+    _check_size0("sym_dual_dequant", scale_col_1, "scale_col_1", cols)
+    _check_size0("sym_dual_dequant", scale_col_2, "scale_col_2", cols)
+    _check_bits("sym_dual_dequant", bits)
+    x = torch.empty(q.shape, dtype=torch.float16, device=q.device)
+    with torch.cuda.device(q.device):
+        st = _lib.load().duq_sym_dual_dequant_host(_ptr(q), _ptr(scale_row), _ptr(scale_col_1), _ptr(scale_col_2),
+                                                   rows, cols, _ptr(x), _stream(q))
+    _lib.check(st, "sym_dual_dequant")
+    return x
+
+
+def asym_dequant(q, scale_row, zeros_row, scale_col, zeros_col, bits: int = 32):
+    """bindings.cpp:268-307."""
+    ts = (q, scale_row, zeros_row, scale_col, zeros_col)
+    _check("asym_dequant", *ts)
+    _check_dtype("asym_dequant", q, "q", torch.int32)
+    for t, n in zip(ts[1:], ("scale_row", "zeros_row", "scale_col", "zeros_col")):
+        _check_dtype("asym_dequant", t, n, torch.float16)
+    rows, cols = q.size(0), q.size(1)
+    _check_size0("asym_dequant", scale_row, "scale_row", rows)
+    _check_size0("asym_dequant", zeros_row, "zeros_row", rows)
+    _check_size0("asym_dequant", scale_col, "scale_col", cols)
+    _check_size0("asym_dequant", zeros_col, "zeros_col", cols)
+    _check_bits("asym_dequant", bits)
+    x = torch.empty(q.shape, dtype=torch.float16, device=q.device)
+    with torch.cuda.device(q.device):
+        st = _lib.load().duq_asym_dequant_host(_ptr(q), _ptr(scale_row), _ptr(zeros_row), _ptr(scale_col),
+                                               _ptr(zeros_col), rows, cols, _ptr(x), _stream(q))
+    _lib.check(st, "asym_dequant")
+    return x
+
+
+def asym_dual_dequant(q, scale_row, zeros_row, scale_col_1, zeros_col_1, scale_col_2, zeros_col_2, bits: int = 32):
+    """bindings.cpp:423-467."""
+    ts = (q, scale_row, zeros_row, scale_col_1, zeros_col_1, scale_col_2, zeros_col_2)
+    _check("asym_dual_dequant", *ts)
+    _check_dtype("asym_dual_dequant", q, "q", torch.int32)
+    names = ("scale_row", "zeros_row", "scale_col_1", "zeros_col_1", "scale_col_2", "zeros_col_2")
+    for t, n in zip(ts[1:], names):
+        _check_dtype("asym_dual_dequant", t, n, torch.float16)
+    rows, cols = q.size(0), q.size(1)
+    for t, n in zip(ts[1:3], names[:2]):
+        _check_size0("asym_dual_dequant", t, n, rows)
+    for t, n in zip(ts[3:], names[2:]):
+        _check_size0("asym_dual_dequant", t, n, cols)
+    _check_bits("asym_dual_dequant", bits)
+    x = torch.empty(q.shape, dtype=torch.float16, device=q.device)
+    with torch.cuda.device(q.device):
+        st = _lib.load().duq_asym_dual_dequant_host(_ptr(q), _ptr(scale_row), _ptr(zeros_row), _ptr(scale_col_1),
+                                                    _ptr(zeros_col_1), _ptr(scale_col_2), _ptr(zeros_col_2), rows,
+                                                    cols, _ptr(x), _stream(q))
+    _lib.check(st, "asym_dual_dequant")
+    return x
+
+
+def get_dual_quant_col_k() -> int:
+    """bindings.cpp:471-473."""
+    return _QUANT_COL_K
+
+
+# ---- additions over the reference module: fused ops -----------------------------------
+
+def quantize_rows_sym(x: torch.Tensor, clip: float = 1.0, qmax: int = 6):
+    """One-pass SymQuantizer (qlinear4bit/nn/quantizer.py:10-16): returns (q uint8 [M,K/2],
+    scales fp16 [M,1]).  Requires K % 32 == 0."""
+    _check("quantize_rows_sym", x)
+    _check_dtype("quantize_rows_sym", x, "x", torch.float16)
+    rows, cols = x.size(0), x.size(1)
+    q = torch.empty((rows, cols // 2), dtype=torch.uint8, device=x.device)
+    s = torch.empty((rows, 1), dtype=torch.float16, device=x.device)
+    with torch.cuda.device(x.device):
+        st = _lib.load().duq_quantize_rows_sym(_ptr(x), rows, cols, float(clip), qmax, _ptr(q), _ptr(s), _stream(x))
+    _lib.check(st, "quantize_rows_sym")
+    return q, s
+
+
+def quantize_rows_asym(x: torch.Tensor):
+    """One-pass AsymQuantizer (qlinear4bit/nn/quantizer.py:24-35): returns (q, scale [M,1],
+    zeros [M,1]).  Requires K % 32 == 0."""
+    _check("quantize_rows_asym", x)
+    _check_dtype("quantize_rows_asym", x, "x", torch.float16)
+    rows, cols = x.size(0), x.size(1)
+    q = torch.empty((rows, cols // 2), dtype=torch.uint8, device=x.device)
+    s = torch.empty((rows, 1), dtype=torch.float16, device=x.device)
+    z = torch.empty((rows, 1), dtype=torch.float16, device=x.device)
+    with torch.cuda.device(x.device):
+        st = _lib.load().duq_quantize_rows_asym(_ptr(x), rows, cols, _ptr(q), _ptr(s), _ptr(z), _stream(x))
+    _lib.check(st, "quantize_rows_asym")
+    return q, s, z
+
+
+EPI_SYM, EPI_ASYM, EPI_SYM_DUAL, EPI_ASYM_DUAL = 0, 1, 2, 3
+
+
+def linear4bit_forward(mode, xq, scale_x, zeros_x, w, w_scale_1, w_zeros_1=None, w_scale_2=None, w_zeros_2=None,
+                       bias=None):
+    """matmul + dequant (+ bias) in one launch; bit-identical to the separate ops.
+    All tensors 2-D / 1-D-viewable and contiguous; returns fp16 [M, N]."""
+    present = [t for t in (xq, scale_x, zeros_x, w, w_scale_1, w_zeros_1, w_scale_2, w_zeros_2, bias) if t is not None]
+    _check("linear4bit_forward", *present)
+    _check_dtype("linear4bit_forward", xq, "xq", torch.uint8)
+    _check_dtype("linear4bit_forward", w, "w", torch.uint8)
+    for t in present:
+        if t is not xq and t is not w:
+            _check_dtype("linear4bit_forward", t, "scale/zero/bias", torch.float16)
+    M, N, K = xq.size(0), w.size(0), xq.size(1) * 2
+    if w.size(1) != xq.size(1):
+        raise RuntimeError(f"linear4bit_forward: packed K differs: x {tuple(xq.shape)} vs w {tuple(w.shape)}")
+    _check_size0("linear4bit_forward", scale_x.view(-1), "scale_x", M)
+    for t, n in ((w_scale_1, "w_scale_1"), (w_zeros_1, "w_zeros_1"), (w_scale_2, "w_scale_2"),
+                 (w_zeros_2, "w_zeros_2"), (bias, "bias")):
+        if t is not None:
+            _check_size0("linear4bit_forward", t.view(-1), n, N)
+    if zeros_x is not None:
+        _check_size0("linear4bit_forward", zeros_x.view(-1), "zeros_x", M)
+    y = torch.empty((M, N), dtype=torch.float16, device=xq.device)
+    with torch.cuda.device(xq.device):
+        st = _lib.load().duq_linear4bit_forward(mode, _ptr(xq), _ptr(scale_x), _ptr(zeros_x), _ptr(w), _ptr(w_scale_1),
+                                                _ptr(w_zeros_1), _ptr(w_scale_2), _ptr(w_zeros_2), _ptr(bias), M, N, K,
+                                                _ptr(y), _stream(xq))
+    _lib.check(st, "linear4bit_forward")
+    return y

@@ -1,0 +1,190 @@
+// extern "C" boundary of libduq_hip.so: argument validation, then the launchers.
+// Nothing here allocates, synchronises, throws or keeps state.
+#include "../../include/duq_hip.h"
+#include "duq_launch.h"
+
+namespace {
+
+inline hipStream_t as_stream(duq_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+inline bool aligned(const void *p, uintptr_t a) { return reinterpret_cast<uintptr_t>(p) % a == 0; }
+
+int check_quant_shape(uint32_t rows, uint32_t colsSrc, uint32_t colsDst)
+{
+    (void)rows;
+    if (colsDst != (colsSrc + 1) / 2) return DUQ_E_SHAPE;
+    return DUQ_OK;
+}
+
+int check_qmax(int32_t qmax) { return (qmax >= 0 && qmax <= 7) ? DUQ_OK : DUQ_E_MODE; }
+
+int check_gemm(const void *A, const void *B, uint32_t M, uint32_t N, uint32_t K)
+{
+    if (M == 0 || N == 0) return DUQ_OK;
+    if (!A || !B) return DUQ_E_NULL;
+    if (K % 64 != 0) return DUQ_E_KALIGN;
+    if (K > 131008u) return DUQ_E_TOO_LARGE;
+    if (!aligned(A, 16) || !aligned(B, 16)) return DUQ_E_ALIGN;
+    return DUQ_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int duq_abi_version(void) { return 1; }
+
+const char *duq_status_string(int status)
+{
+    switch (status) {
+    case DUQ_OK: return "ok";
+    case DUQ_E_NULL: return "a required pointer is NULL";
+    case DUQ_E_SHAPE: return "inconsistent dimensions";
+    case DUQ_E_KALIGN: return "K must be a multiple of 64 (packed row length a multiple of 32 bytes)";
+    case DUQ_E_MODE: return "unknown epilogue mode or unsupported qmax";
+    case DUQ_E_ALIGN: return "pointer alignment requirement not met";
+    case DUQ_E_TOO_LARGE: return "dimension too large";
+    default: break;
+    }
+    if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));
+    return "unknown status";
+}
+
+int duq_get_dual_quant_col_k(void) { return DUQ_QUANT_COL_K; }
+
+int duq_sym_quant_host_qmax(const duq_half *x, const duq_half *scale, uint32_t rows, uint32_t colsSrc,
+                            uint32_t colsDst, int32_t qmax, uint8_t *q, duq_stream_t stream)
+{
+    if (int e = check_quant_shape(rows, colsSrc, colsDst)) return e;
+    if (int e = check_qmax(qmax)) return e;
+    if (rows == 0 || colsSrc == 0) return DUQ_OK;
+    if (!x || !scale || !q) return DUQ_E_NULL;
+    return duq::launch_sym_quant(x, scale, rows, colsSrc, colsDst, qmax, q, as_stream(stream));
+}
+
+int duq_sym_quant_host(const duq_half *x, const duq_half *scale, uint32_t rows, uint32_t colsSrc, uint32_t colsDst,
+                       uint8_t *q, duq_stream_t stream)
+{
+    return duq_sym_quant_host_qmax(x, scale, rows, colsSrc, colsDst, DUQ_QMAX_SYM_DEVICE, q, stream);
+}
+
+int duq_sym_dual_quant_host(const duq_half *x, const duq_half *scale_1, const duq_half *scale_2, uint32_t rows,
+                            uint32_t colsSrc, uint32_t colsDst, uint8_t *q, duq_stream_t stream)
+{
+    if (int e = check_quant_shape(rows, colsSrc, colsDst)) return e;
+    if (rows == 0 || colsSrc == 0) return DUQ_OK;
+    if (!x || !scale_1 || !scale_2 || !q) return DUQ_E_NULL;
+    return duq::launch_sym_dual_quant(x, scale_1, scale_2, rows, colsSrc, colsDst, DUQ_QMAX_SYM_DEVICE, q,
+                                      as_stream(stream));
+}
+
+int duq_asym_quant_host(const duq_half *x, const duq_half *scale, const duq_half *zeros, uint32_t rows,
+                        uint32_t colsSrc, uint32_t colsDst, uint8_t *q, duq_stream_t stream)
+{
+    if (int e = check_quant_shape(rows, colsSrc, colsDst)) return e;
+    if (rows == 0 || colsSrc == 0) return DUQ_OK;
+    if (!x || !scale || !zeros || !q) return DUQ_E_NULL;
+    return duq::launch_asym_quant(x, scale, zeros, rows, colsSrc, colsDst, q, as_stream(stream));
+}
+
+int duq_asym_dual_quant_host(const duq_half *x, const duq_half *scale_1, const duq_half *zeros_1,
+                             const duq_half *scale_2, const duq_half *zeros_2, uint32_t rows, uint32_t colsSrc,
+                             uint32_t colsDst, uint8_t *q, duq_stream_t stream)
+{
+    if (int e = check_quant_shape(rows, colsSrc, colsDst)) return e;
+    if (rows == 0 || colsSrc == 0) return DUQ_OK;
+    if (!x || !scale_1 || !zeros_1 || !scale_2 || !zeros_2 || !q) return DUQ_E_NULL;
+    return duq::launch_asym_dual_quant(x, scale_1, zeros_1, scale_2, zeros_2, rows, colsSrc, colsDst, q,
+                                       as_stream(stream));
+}
+
+int duq_quantize_rows_sym(const duq_half *x, uint32_t rows, uint32_t cols, float clip, int32_t qmax, uint8_t *q,
+                          duq_half *scale, duq_stream_t stream)
+{
+    if (int e = check_qmax(qmax)) return e;
+    if (rows == 0 || cols == 0) return DUQ_OK;
+    if (!x || !q || !scale) return DUQ_E_NULL;
+    if (cols % 32 != 0) return DUQ_E_SHAPE;
+    if (!aligned(x, 16) || !aligned(q, 16)) return DUQ_E_ALIGN;
+    return duq::launch_quantize_rows_sym(x, rows, cols, clip, qmax, q, scale, as_stream(stream));
+}
+
+int duq_quantize_rows_asym(const duq_half *x, uint32_t rows, uint32_t cols, uint8_t *q, duq_half *scale,
+                           duq_half *zeros, duq_stream_t stream)
+{
+    if (rows == 0 || cols == 0) return DUQ_OK;
+    if (!x || !q || !scale || !zeros) return DUQ_E_NULL;
+    if (cols % 32 != 0) return DUQ_E_SHAPE;
+    if (!aligned(x, 16) || !aligned(q, 16)) return DUQ_E_ALIGN;
+    return duq::launch_quantize_rows_asym(x, rows, cols, q, scale, zeros, as_stream(stream));
+}
+
+int duq_matmul_host_4bit(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N, uint32_t K, int32_t *C,
+                         duq_stream_t stream)
+{
+    if (int e = check_gemm(A, B, M, N, K)) return e;
+    if (M == 0 || N == 0) return DUQ_OK;
+    if (!C) return DUQ_E_NULL;
+    return duq::launch_gemm_s4(A, B, M, N, K, C, nullptr, nullptr, as_stream(stream));
+}
+
+int duq_sym_dequant_host(const int32_t *q, const duq_half *scale_row, const duq_half *scale_col, uint32_t rows,
+                         uint32_t cols, duq_half *x, duq_stream_t stream)
+{
+    if (rows == 0 || cols == 0) return DUQ_OK;
+    if (!q || !scale_row || !scale_col || !x) return DUQ_E_NULL;
+    duq::Epilogue e{DUQ_EPI_SYM, scale_row, nullptr, scale_col, nullptr, nullptr, nullptr, nullptr};
+    return duq::launch_dequant(q, e, rows, cols, x, as_stream(stream));
+}
+
+int duq_sym_dual_dequant_host(const int32_t *q, const duq_half *scale_row, const duq_half *scale_col_1,
+                              const duq_half *scale_col_2, uint32_t rows, uint32_t cols, duq_half *x,
+                              duq_stream_t stream)
+{
+    if (rows == 0 || cols == 0) return DUQ_OK;
+    if (!q || !scale_row || !scale_col_1 || !scale_col_2 || !x) return DUQ_E_NULL;
+    duq::Epilogue e{DUQ_EPI_SYM_DUAL, scale_row, nullptr, scale_col_1, nullptr, scale_col_2, nullptr, nullptr};
+    return duq::launch_dequant(q, e, rows, cols, x, as_stream(stream));
+}
+
+int duq_asym_dequant_host(const int32_t *q, const duq_half *scale_row, const duq_half *zeros_row,
+                          const duq_half *scale_col, const duq_half *zeros_col, uint32_t rows, uint32_t cols,
+                          duq_half *x, duq_stream_t stream)
+{
+    if (rows == 0 || cols == 0) return DUQ_OK;
+    if (!q || !scale_row || !zeros_row || !scale_col || !zeros_col || !x) return DUQ_E_NULL;
+    duq::Epilogue e{DUQ_EPI_ASYM, scale_row, zeros_row, scale_col, zeros_col, nullptr, nullptr, nullptr};
+    return duq::launch_dequant(q, e, rows, cols, x, as_stream(stream));
+}
+
+int duq_asym_dual_dequant_host(const int32_t *q, const duq_half *scale_row, const duq_half *zeros_row,
+                               const duq_half *scale_col_1, const duq_half *zeros_col_1, const duq_half *scale_col_2,
+                               const duq_half *zeros_col_2, uint32_t rows, uint32_t cols, duq_half *x,
+                               duq_stream_t stream)
+{
+    if (rows == 0 || cols == 0) return DUQ_OK;
+    if (!q || !scale_row || !zeros_row || !scale_col_1 || !zeros_col_1 || !scale_col_2 || !zeros_col_2 || !x)
+        return DUQ_E_NULL;
+    duq::Epilogue e{DUQ_EPI_ASYM_DUAL, scale_row, zeros_row, scale_col_1, zeros_col_1, scale_col_2, zeros_col_2,
+                    nullptr};
+    return duq::launch_dequant(q, e, rows, cols, x, as_stream(stream));
+}
+
+int duq_linear4bit_forward(int32_t mode, const uint8_t *xq, const duq_half *scale_x, const duq_half *zeros_x,
+                           const uint8_t *w, const duq_half *w_scale_1, const duq_half *w_zeros_1,
+                           const duq_half *w_scale_2, const duq_half *w_zeros_2, const duq_half *bias, uint32_t M,
+                           uint32_t N, uint32_t K, duq_half *y, duq_stream_t stream)
+{
+    if (mode < DUQ_EPI_SYM || mode > DUQ_EPI_ASYM_DUAL) return DUQ_E_MODE;
+    if (int e = check_gemm(xq, w, M, N, K)) return e;
+    if (M == 0 || N == 0) return DUQ_OK;
+    if (!scale_x || !w_scale_1 || !y) return DUQ_E_NULL;
+    const bool asym = mode == DUQ_EPI_ASYM || mode == DUQ_EPI_ASYM_DUAL;
+    const bool dual = mode == DUQ_EPI_SYM_DUAL || mode == DUQ_EPI_ASYM_DUAL;
+    if (asym && (!zeros_x || !w_zeros_1)) return DUQ_E_NULL;
+    if (dual && !w_scale_2) return DUQ_E_NULL;
+    if (asym && dual && !w_zeros_2) return DUQ_E_NULL;
+    duq::Epilogue e{mode, scale_x, zeros_x, w_scale_1, w_zeros_1, w_scale_2, w_zeros_2, bias};
+    return duq::launch_gemm_s4(xq, w, M, N, K, nullptr, &e, y, as_stream(stream));
+}
+
+}  // extern "C"

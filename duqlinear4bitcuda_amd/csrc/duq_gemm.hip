@@ -1,0 +1,382 @@
+// Packed-int4 x packed-int4 -> int32 GEMM for gfx950 on v_mfma_i32_16x16x64_i8, with the
+// fp16 dequant epilogue fused in (or raw int32 accumulators out).
+//
+//   C[m,n] = sum_k s4(A[m,k]) * s4(B[n,k])        (src/kernels/gemm.cu:8-43 of the reference)
+//
+// Nibble -> byte: for a packed word w, (w & 0xF0F0F0F0) holds the four odd-k nibbles as
+// bytes equal to 16*s4 (sign included), ((w << 4) & 0xF0F0F0F0) the four even-k ones.
+// Both operands are expanded the same way, so every MFMA product is 256*a*b and the
+// accumulator is 256*C exactly; one arithmetic shift by 8 recovers C.  |C| <= 64*K, so
+// 256*|C| stays below 2^31 for K <= 131008.  Integer accumulation is order-free, so the
+// k order inside a tile only has to be the same for A and B.
+//
+// Two kernels:
+//  * tile kernel (prefill, M > 16): BM x BN x 128 tiles, 4 wavefronts (2 x 2), packed
+//    nibbles are expanded to bytes on the way from global memory into LDS, LDS rows are
+//    padded to 144 B so that the 128-bit fragment reads are bank-conflict free, LDS is
+//    double buffered and the next tile's global loads are in flight during the MFMAs.
+//    The weight operand goes to the MFMA "A" side, so each lane ends up with four
+//    consecutive output columns of one row and stores them as one vector.
+//  * skinny kernel (decode, M <= 16): HBM-bound weight streaming.  One workgroup owns 16
+//    output columns, its wavefronts split K, every lane issues all of its 128-bit weight
+//    loads before the first MFMA, fragments go from global memory straight to registers
+//    (no LDS for operands), partial sums meet in LDS once at the end.
+#include "duq_epilogue.h"
+#include "duq_launch.h"
+
+namespace duq {
+
+constexpr uint32_t kNibbleMask = 0xF0F0F0F0u;
+
+struct GemmParams {
+    const uint8_t *A;  // activations [M, K/2]
+    const uint8_t *B;  // weights     [N, K/2]
+    uint32_t M, N, K;
+    int32_t *C;        // int32 out (EPI < 0)
+    uint16_t *y;       // fp16 out  (EPI >= 0)
+    Epilogue epi;
+    uint32_t tiles_m, tiles_n;
+};
+
+__device__ __forceinline__ void expand_nibbles(const v4u w, v4u &even, v4u &odd)
+{
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        even[i] = (w[i] << 4) & kNibbleMask;
+        odd[i] = w[i] & kNibbleMask;
+    }
+}
+
+// Workgroup id -> tile id.  Consecutive workgroup ids land on consecutive XCDs (8 of them,
+// each with its own L2), so ids are regrouped to give every XCD one contiguous range of
+// tiles; tiles inside a range walk down a band of 8 tile-rows first, which keeps the A and
+// B panels an XCD touches compact.
+__device__ __forceinline__ void tile_of_block(uint32_t bid, uint32_t tiles_m, uint32_t tiles_n, uint32_t &tm,
+                                              uint32_t &tn)
+{
+    const uint32_t ntiles = tiles_m * tiles_n;
+    const uint32_t per = ntiles / 8, rem = ntiles % 8;
+    const uint32_t xcd = bid % 8, local = bid / 8;
+    const uint32_t logical = xcd < rem ? xcd * (per + 1) + local : rem * (per + 1) + (xcd - rem) * per + local;
+    constexpr uint32_t GM = 8;
+    const uint32_t per_band = GM * tiles_n;
+    const uint32_t band = logical / per_band;
+    const uint32_t first_m = band * GM;
+    const uint32_t band_h = min(tiles_m - first_m, GM);
+    const uint32_t in_band = logical % per_band;
+    tm = first_m + in_band % band_h;
+    tn = in_band / band_h;
+}
+
+// Store four consecutive output columns of one row.
+template <int EPI, bool BIAS>
+__device__ __forceinline__ void store_quad(const GemmParams &p, uint32_t m, uint32_t n0, v4i acc, bool vec_ok)
+{
+    if (m >= p.M || n0 >= p.N) return;
+    if (EPI < 0) {
+        int32_t *dst = p.C + (uint64_t)m * p.N + n0;
+        if (vec_ok && n0 + 3 < p.N) {
+            *reinterpret_cast<v4i *>(dst) = acc;
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (n0 + r < p.N) dst[r] = acc[r];
+        }
+    } else {
+        constexpr int MODE = EPI < 0 ? 0 : EPI;
+        const f16 s_row = bits_to_f16(p.epi.s_row[m]);
+        const f16 z_row = (MODE == 1 || MODE == 3) ? bits_to_f16(p.epi.z_row[m]) : (f16)0;
+        uint16_t out[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const uint32_t n = min(n0 + r, p.N - 1);
+            const ColParams c = load_col<MODE, BIAS>(p.epi.s_col_1, p.epi.z_col_1, p.epi.s_col_2, p.epi.z_col_2,
+                                                     p.epi.bias, n);
+            out[r] = dequant_one<MODE, BIAS>(acc[r], s_row, z_row, c);
+        }
+        uint16_t *dst = p.y + (uint64_t)m * p.N + n0;
+        if (vec_ok && n0 + 3 < p.N) {
+            *reinterpret_cast<v2u *>(dst) = v2u{(uint32_t)out[0] | ((uint32_t)out[1] << 16),
+                                                (uint32_t)out[2] | ((uint32_t)out[3] << 16)};
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (n0 + r < p.N) dst[r] = out[r];
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// tile kernel
+// ---------------------------------------------------------------------------------
+constexpr int kBK = 128;           // k elements per tile step (64 packed bytes per row)
+constexpr int kLdsStride = 144;    // bytes per LDS row: 128 expanded bytes + 16 pad
+
+template <int BM, int BN, int EPI, bool BIAS>
+__global__ __launch_bounds__(256) void gemm_s4_tile_kernel(GemmParams p)
+{
+    constexpr int WTM = BM / 2, WTN = BN / 2;  // per-wavefront tile
+    constexpr int TM = WTM / 16, TN = WTN / 16;
+    constexpr int NA = BM / 64, NB = BN / 64;  // 16-byte global pieces per thread
+    static_assert(BM % 64 == 0 && BN % 64 == 0, "tile shape");
+
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2][(BM + BN) * kLdsStride];
+
+    uint32_t tile_m, tile_n;
+    tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+    const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u, wave = tid >> 6;
+    const uint32_t wm = wave >> 1, wn = wave & 1u;
+    const uint32_t l16 = lane & 15u, g = lane >> 4;
+    const uint32_t kbytes = p.K >> 1;
+    const uint32_t nk = (p.K + kBK - 1) / kBK;
+
+    // global source of each 16-byte piece this thread moves (row clamped to stay in bounds)
+    const uint8_t *srcA[NA];
+    const uint8_t *srcB[NB];
+    uint32_t ldsA[NA], ldsB[NB];
+    const uint32_t pj = tid & 3u;  // which 16-byte piece of the 64-byte row segment
+#pragma unroll
+    for (int i = 0; i < NA; ++i) {
+        const uint32_t row = (tid >> 2) + i * 64;
+        const uint32_t gm = min(m0 + row, p.M - 1);
+        srcA[i] = p.A + (uint64_t)gm * kbytes + pj * 16;
+        ldsA[i] = row * kLdsStride + pj * 32;
+    }
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+        const uint32_t row = (tid >> 2) + i * 64;
+        const uint32_t gn = min(n0 + row, p.N - 1);
+        srcB[i] = p.B + (uint64_t)gn * kbytes + pj * 16;
+        ldsB[i] = (BM + row) * kLdsStride + pj * 32;
+    }
+
+    v4u ga[NA], gb[NB];
+    auto load_tile = [&](uint32_t kt) {
+        const uint32_t koff = kt * (kBK / 2);
+        const bool ok = koff + pj * 16 < kbytes;  // K % 64 == 0: a piece is all in or all out
+#pragma unroll
+        for (int i = 0; i < NA; ++i)
+            ga[i] = ok ? *reinterpret_cast<const v4u *>(srcA[i] + koff) : v4u{0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int i = 0; i < NB; ++i)
+            gb[i] = ok ? *reinterpret_cast<const v4u *>(srcB[i] + koff) : v4u{0u, 0u, 0u, 0u};
+    };
+    auto store_tile = [&](uint32_t buf) {
+        uint8_t *base = lds[buf];
+#pragma unroll
+        for (int i = 0; i < NA; ++i) {
+            v4u ev, od;
+            expand_nibbles(ga[i], ev, od);
+            *reinterpret_cast<v4u *>(base + ldsA[i]) = ev;
+            *reinterpret_cast<v4u *>(base + ldsA[i] + 16) = od;
+        }
+#pragma unroll
+        for (int i = 0; i < NB; ++i) {
+            v4u ev, od;
+            expand_nibbles(gb[i], ev, od);
+            *reinterpret_cast<v4u *>(base + ldsB[i]) = ev;
+            *reinterpret_cast<v4u *>(base + ldsB[i] + 16) = od;
+        }
+    };
+
+    v4i acc[TN][TM];
+#pragma unroll
+    for (int a = 0; a < TN; ++a)
+#pragma unroll
+        for (int b = 0; b < TM; ++b) acc[a][b] = v4i{0, 0, 0, 0};
+
+    // fragment rows of this lane inside the LDS tile
+    const uint32_t fragX = (wm * WTM + l16) * kLdsStride + g * 16;         // activations
+    const uint32_t fragW = (BM + wn * WTN + l16) * kLdsStride + g * 16;    // weights
+
+    load_tile(0);
+    store_tile(0);
+    __syncthreads();
+
+    for (uint32_t kt = 0; kt < nk; ++kt) {
+        const uint32_t cur = kt & 1u;
+        const bool more = kt + 1 < nk;
+        if (more) load_tile(kt + 1);
+
+        const uint8_t *base = lds[cur];
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            v4i fx[TM], fw[TN];
+#pragma unroll
+            for (int b = 0; b < TM; ++b)
+                fx[b] = *reinterpret_cast<const v4i *>(base + fragX + b * 16 * kLdsStride + s * 64);
+#pragma unroll
+            for (int a = 0; a < TN; ++a)
+                fw[a] = *reinterpret_cast<const v4i *>(base + fragW + a * 16 * kLdsStride + s * 64);
+#pragma unroll
+            for (int a = 0; a < TN; ++a)
+#pragma unroll
+                for (int b = 0; b < TM; ++b)
+                    acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fw[a], fx[b], acc[a][b], 0, 0, 0);
+        }
+
+        if (more) store_tile(cur ^ 1u);
+        __syncthreads();
+    }
+
+    // lane holds, for every (a, b): rows n = 4*g + r of the weight fragment, column m = l16
+    const bool vec_ok = (EPI < 0) ? (p.N % 4 == 0 && reinterpret_cast<uintptr_t>(p.C) % 16 == 0)
+                                  : (p.N % 4 == 0 && reinterpret_cast<uintptr_t>(p.y) % 8 == 0);
+#pragma unroll
+    for (int b = 0; b < TM; ++b)
+#pragma unroll
+        for (int a = 0; a < TN; ++a) {
+            v4i v = acc[a][b];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) v[r] >>= 8;
+            store_quad<EPI, BIAS>(p, m0 + wm * WTM + b * 16 + l16, n0 + wn * WTN + a * 16 + g * 4, v, vec_ok);
+        }
+}
+
+// ---------------------------------------------------------------------------------
+// skinny kernel (M <= 16)
+// ---------------------------------------------------------------------------------
+// Workgroup = WAVES wavefronts, 16 output columns.  Wavefront w owns the k range
+// [w*kw, (w+1)*kw) with kw = ceil(K/64/WAVES)*64 elements, walked in steps of 128 k (64 B
+// per row): lane (l16, g) loads bytes [g*16, g*16+16) of the 64-byte segment of weight
+// row n0+l16 and of activation row l16, expands both and issues two MFMAs (even k, odd k).
+constexpr int kSkinnyUnroll = 8;  // 128-bit loads in flight per operand per lane
+
+template <int WAVES, int EPI, bool BIAS>
+__global__ __launch_bounds__(WAVES * 64) void gemm_s4_skinny_kernel(GemmParams p)
+{
+    __shared__ v4i part[WAVES][64];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u, wave = tid >> 6;
+    const uint32_t l16 = lane & 15u, g = lane >> 4;
+    const uint32_t n0 = blockIdx.x * 16;
+    const uint32_t kbytes = p.K >> 1;
+    const uint32_t segs = kbytes / 64 + ((kbytes % 64) ? 1 : 0);  // 64-byte segments per row
+    const uint32_t per_wave = (segs + WAVES - 1) / WAVES;
+    const uint32_t seg_begin = wave * per_wave;
+    const uint32_t seg_end = min(seg_begin + per_wave, segs);
+
+    const uint32_t wrow = min(n0 + l16, p.N - 1);
+    const bool xrow_ok = l16 < p.M;
+    const uint8_t *wsrc = p.B + (uint64_t)wrow * kbytes + g * 16;
+    const uint8_t *xsrc = p.A + (uint64_t)(xrow_ok ? l16 : 0) * kbytes + g * 16;
+
+    v4i acc = v4i{0, 0, 0, 0};
+    for (uint32_t s0 = seg_begin; s0 < seg_end; s0 += kSkinnyUnroll) {
+        v4u w[kSkinnyUnroll], x[kSkinnyUnroll];
+#pragma unroll
+        for (int u = 0; u < kSkinnyUnroll; ++u) {
+            const uint32_t off = (s0 + u) * 64;
+            const bool ok = (s0 + u) < seg_end && off + g * 16 < kbytes;
+            w[u] = ok ? __builtin_nontemporal_load(reinterpret_cast<const v4u *>(wsrc + off)) : v4u{0u, 0u, 0u, 0u};
+            x[u] = (ok && xrow_ok) ? *reinterpret_cast<const v4u *>(xsrc + off) : v4u{0u, 0u, 0u, 0u};
+        }
+#pragma unroll
+        for (int u = 0; u < kSkinnyUnroll; ++u) {
+            v4u we, wo, xe, xo;
+            expand_nibbles(w[u], we, wo);
+            expand_nibbles(x[u], xe, xo);
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i, we), __builtin_bit_cast(v4i, xe),
+                                                        acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i, wo), __builtin_bit_cast(v4i, xo),
+                                                        acc, 0, 0, 0);
+        }
+    }
+
+    if (WAVES > 1) {
+        part[wave][lane] = acc;
+        __syncthreads();
+        if (wave != 0) return;
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) {
+            const v4i o = part[w][lane];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[r] += o[r];
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) acc[r] >>= 8;
+    const bool vec_ok = (EPI < 0) ? (p.N % 4 == 0 && reinterpret_cast<uintptr_t>(p.C) % 16 == 0)
+                                  : (p.N % 4 == 0 && reinterpret_cast<uintptr_t>(p.y) % 8 == 0);
+    store_quad<EPI, BIAS>(p, l16, n0 + g * 4, acc, vec_ok);
+}
+
+// ---------------------------------------------------------------------------------
+// dispatch
+// ---------------------------------------------------------------------------------
+template <int EPI, bool BIAS>
+static void launch_epi(GemmParams &p, hipStream_t stream)
+{
+    if (p.M <= 16) {
+        const dim3 grid((p.N + 15) / 16);
+        const uint32_t segs = (p.K / 2 + 63) / 64;
+        // enough wavefronts per workgroup that each walks about one unrolled step of K
+        if (segs <= 4 * kSkinnyUnroll)
+            hipLaunchKernelGGL((gemm_s4_skinny_kernel<4, EPI, BIAS>), grid, dim3(256), 0, stream, p);
+        else if (segs <= 8 * kSkinnyUnroll)
+            hipLaunchKernelGGL((gemm_s4_skinny_kernel<8, EPI, BIAS>), grid, dim3(512), 0, stream, p);
+        else
+            hipLaunchKernelGGL((gemm_s4_skinny_kernel<16, EPI, BIAS>), grid, dim3(1024), 0, stream, p);
+        return;
+    }
+    // largest tile that still yields at least one workgroup per CU (256 CUs); small
+    // problems take the small tile to spread over the chip.
+    auto tiles = [&](uint32_t bm, uint32_t bn) { return ((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn); };
+    if (tiles(128, 256) >= 256 && p.M > 64) {
+        p.tiles_m = (p.M + 127) / 128;
+        p.tiles_n = (p.N + 255) / 256;
+        hipLaunchKernelGGL((gemm_s4_tile_kernel<128, 256, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0,
+                           stream, p);
+    } else if (tiles(128, 128) >= 256 && p.M > 64) {
+        p.tiles_m = (p.M + 127) / 128;
+        p.tiles_n = (p.N + 127) / 128;
+        hipLaunchKernelGGL((gemm_s4_tile_kernel<128, 128, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0,
+                           stream, p);
+    } else {
+        p.tiles_m = (p.M + 63) / 64;
+        p.tiles_n = (p.N + 63) / 64;
+        hipLaunchKernelGGL((gemm_s4_tile_kernel<64, 64, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0,
+                           stream, p);
+    }
+}
+
+int launch_gemm_s4(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N, uint32_t K, int32_t *out_acc,
+                   const Epilogue *epi, uint16_t *y, hipStream_t stream)
+{
+    if (M == 0 || N == 0) return 0;
+    GemmParams p{};
+    p.A = A;
+    p.B = B;
+    p.M = M;
+    p.N = N;
+    p.K = K;
+    p.C = out_acc;
+    p.y = y;
+    if (epi) p.epi = *epi;
+    if (out_acc) {
+        launch_epi<-1, false>(p, stream);
+    } else {
+        const bool bias = epi->bias != nullptr;
+#define DUQ_GEMM(MODE)                             \
+    case MODE:                                     \
+        if (bias)                                  \
+            launch_epi<MODE, true>(p, stream);     \
+        else                                       \
+            launch_epi<MODE, false>(p, stream);    \
+        break;
+        switch (epi->mode) {
+            DUQ_GEMM(0)
+            DUQ_GEMM(1)
+            DUQ_GEMM(2)
+            DUQ_GEMM(3)
+        default:
+            return (int)hipErrorInvalidValue;
+        }
+#undef DUQ_GEMM
+    }
+    return (int)hipGetLastError();
+}
+
+}  // namespace duq

@@ -1,0 +1,44 @@
+// Host-side launchers implemented by the .hip files; the extern "C" layer in
+// duq_abi.hip validates arguments and forwards here.  All return a hipError_t as int.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <algorithm>
+
+namespace duq {
+
+int launch_sym_quant(const uint16_t *x, const uint16_t *scale, uint32_t rows, uint32_t colsSrc, uint32_t colsDst,
+                     int qmax, uint8_t *q, hipStream_t stream);
+int launch_sym_dual_quant(const uint16_t *x, const uint16_t *s1, const uint16_t *s2, uint32_t rows,
+                          uint32_t colsSrc, uint32_t colsDst, int qmax, uint8_t *q, hipStream_t stream);
+int launch_asym_quant(const uint16_t *x, const uint16_t *scale, const uint16_t *zeros, uint32_t rows,
+                      uint32_t colsSrc, uint32_t colsDst, uint8_t *q, hipStream_t stream);
+int launch_asym_dual_quant(const uint16_t *x, const uint16_t *s1, const uint16_t *z1, const uint16_t *s2,
+                           const uint16_t *z2, uint32_t rows, uint32_t colsSrc, uint32_t colsDst, uint8_t *q,
+                           hipStream_t stream);
+int launch_quantize_rows_sym(const uint16_t *x, uint32_t rows, uint32_t cols, float clip, int qmax, uint8_t *q,
+                             uint16_t *scale, hipStream_t stream);
+int launch_quantize_rows_asym(const uint16_t *x, uint32_t rows, uint32_t cols, uint8_t *q, uint16_t *scale,
+                              uint16_t *zeros, hipStream_t stream);
+
+// Epilogue description shared by the stand-alone dequant kernels and the fused GEMM.
+// mode: 0 sym, 1 asym, 2 sym-dual, 3 asym-dual (DUQ_EPI_* of the public header).
+struct Epilogue {
+    int mode;
+    const uint16_t *s_row;   // [rows]
+    const uint16_t *z_row;   // [rows]  asym modes
+    const uint16_t *s_col_1; // [cols]
+    const uint16_t *z_col_1; // [cols]  asym modes
+    const uint16_t *s_col_2; // [cols]  dual modes
+    const uint16_t *z_col_2; // [cols]  asym-dual
+    const uint16_t *bias;    // [cols] or nullptr
+};
+
+int launch_dequant(const int32_t *acc, const Epilogue &epi, uint32_t rows, uint32_t cols, uint16_t *y,
+                   hipStream_t stream);
+
+// GEMM: out_acc != nullptr -> int32 accumulators [M,N]; else fused epilogue into y.
+int launch_gemm_s4(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N, uint32_t K, int32_t *out_acc,
+                   const Epilogue *epi, uint16_t *y, hipStream_t stream);
+
+}  // namespace duq

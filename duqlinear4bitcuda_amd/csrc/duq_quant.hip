@@ -1,0 +1,375 @@
+// Per-token int4 quantizers for gfx950.
+//
+// Two families:
+//  * given-scale kernels, one per reference launcher (sym, sym-dual, asym, asym-dual):
+//    stream x once, 8 binary16 elements (one 128-bit load) -> one packed 32-bit word per
+//    lane step, fully coalesced; a scalar kernel covers odd / unaligned shapes;
+//  * fused row kernels that also compute the per-token scale (and zero): the row is
+//    read from HBM once into registers, the |x| max (or min and max) is reduced with
+//    wavefront shuffles (plus one LDS hop when several wavefronts share a row), and
+//    the packed nibbles are written with 128-bit stores.
+//
+// Arithmetic follows the reference kernels operator by operator:
+//   sym  : src/kernels/quant.cu:11-45     asym : src/kernels/quant.cu:99-132
+//   dual : src/kernels/quant2.cu:9-45, 101-139
+//   scale: qlinear4bit/nn/quantizer.py:13, 27-31
+#include "duq_device.h"
+#include "duq_launch.h"
+
+namespace duq {
+
+enum QuantKind { kSym = 0, kSymDual = 1, kAsym = 2, kAsymDual = 3 };
+
+struct QuantParams {
+    const uint16_t *x;
+    const uint16_t *s1;  // scale / scale_1   [rows]
+    const uint16_t *z1;  // zeros / zeros_1   [rows] (asym kinds)
+    const uint16_t *s2;  // scale_2           [rows] (dual kinds)
+    const uint16_t *z2;  // zeros_2           [rows] (asym dual)
+    uint8_t *q;
+    uint32_t rows, colsSrc, colsDst;
+    int qmax;
+};
+
+// ---------------------------------------------------------------------------------
+// scalar kernel: any shape, one thread per output byte (odd K, unaligned rows)
+// ---------------------------------------------------------------------------------
+template <int KIND>
+__global__ __launch_bounds__(256) void quant_scalar_kernel(QuantParams p)
+{
+    const uint64_t total = (uint64_t)p.rows * p.colsDst;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (uint64_t)gridDim.x * blockDim.x) {
+        const uint32_t row = (uint32_t)(i / p.colsDst);
+        const uint32_t cd = (uint32_t)(i % p.colsDst);
+        uint32_t byte = 0;
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const uint32_t c = cd * 2 + e;
+            if (c >= p.colsSrc) continue;
+            const f16 xv = bits_to_f16(p.x[(uint64_t)row * p.colsSrc + c]);
+            const bool first = c < (uint32_t)kQuantColK;
+            uint32_t code;
+            if (KIND == kSym) {
+                code = sym_code(xv, row_rcp(bits_to_f16(p.s1[row])), p.qmax);
+            } else if (KIND == kSymDual) {
+                code = sym_code(xv, row_rcp(bits_to_f16(first ? p.s1[row] : p.s2[row])), p.qmax);
+            } else if (KIND == kAsym) {
+                code = asym_code(xv, row_rcp(bits_to_f16(p.s1[row])), rint_i32((float)bits_to_f16(p.z1[row])));
+            } else {
+                code = asym_pre_code(xv, row_rcp(bits_to_f16(first ? p.s1[row] : p.s2[row])),
+                                     bits_to_f16(first ? p.z1[row] : p.z2[row]));
+            }
+            byte |= code << (4 * e);
+        }
+        p.q[i] = (uint8_t)byte;
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// vector kernel: colsSrc % 8 == 0, x 16-byte aligned, q 4-byte aligned.
+// One lane step = 8 elements in, one 32-bit word out; consecutive lanes take
+// consecutive words, so loads are 1 KiB and stores 256 B contiguous per wavefront.
+// ---------------------------------------------------------------------------------
+template <int KIND>
+__device__ __forceinline__ uint32_t quant8(const v4u raw, uint32_t col0, float r1, float r2, int qmax, int zi,
+                                           f16 z1, f16 z2)
+{
+    uint32_t word = 0;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const uint32_t w = raw[e >> 1];
+        const f16 xv = bits_to_f16((uint16_t)((e & 1) ? (w >> 16) : (w & 0xFFFFu)));
+        uint32_t code;
+        if (KIND == kSym) {
+            code = sym_code(xv, r1, qmax);
+        } else if (KIND == kSymDual) {
+            code = sym_code(xv, (col0 + e) < (uint32_t)kQuantColK ? r1 : r2, qmax);
+        } else if (KIND == kAsym) {
+            code = asym_code(xv, r1, zi);
+        } else {
+            const bool first = (col0 + e) < (uint32_t)kQuantColK;
+            code = asym_pre_code(xv, first ? r1 : r2, first ? z1 : z2);
+        }
+        word |= code << (4 * e);
+    }
+    return word;
+}
+
+template <int KIND>
+__global__ __launch_bounds__(256) void quant_vec_kernel(QuantParams p)
+{
+    const uint32_t vecPerRow = p.colsSrc >> 3;
+    const uint64_t total = (uint64_t)p.rows * vecPerRow;
+    const v4u *x4 = reinterpret_cast<const v4u *>(p.x);
+    uint32_t *q32 = reinterpret_cast<uint32_t *>(p.q);
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (uint64_t)gridDim.x * blockDim.x) {
+        const uint32_t row = (uint32_t)(i / vecPerRow);
+        const uint32_t vec = (uint32_t)(i % vecPerRow);
+        const v4u raw = __builtin_nontemporal_load(&x4[i]);
+        const float r1 = row_rcp(bits_to_f16(p.s1[row]));
+        float r2 = 0.f;
+        int zi = 0;
+        f16 z1 = (f16)0, z2 = (f16)0;
+        if (KIND == kSymDual || KIND == kAsymDual) r2 = row_rcp(bits_to_f16(p.s2[row]));
+        if (KIND == kAsym) zi = rint_i32((float)bits_to_f16(p.z1[row]));
+        if (KIND == kAsymDual) {
+            z1 = bits_to_f16(p.z1[row]);
+            z2 = bits_to_f16(p.z2[row]);
+        }
+        q32[i] = quant8<KIND>(raw, vec * 8, r1, r2, p.qmax, zi, z1, z2);
+    }
+}
+
+template <int KIND>
+static int launch_quant(const QuantParams &p, hipStream_t stream)
+{
+    if (p.rows == 0 || p.colsSrc == 0) return 0;
+    const bool vec_ok = (p.colsSrc % 8 == 0) && (reinterpret_cast<uintptr_t>(p.x) % 16 == 0) &&
+                        (reinterpret_cast<uintptr_t>(p.q) % 4 == 0);
+    if (vec_ok) {
+        const uint64_t total = (uint64_t)p.rows * (p.colsSrc / 8);
+        const uint32_t blocks = (uint32_t)std::min<uint64_t>((total + 255) / 256, 1u << 20);
+        hipLaunchKernelGGL(quant_vec_kernel<KIND>, dim3(blocks), dim3(256), 0, stream, p);
+    } else {
+        const uint64_t total = (uint64_t)p.rows * p.colsDst;
+        const uint32_t blocks = (uint32_t)std::min<uint64_t>((total + 255) / 256, 1u << 20);
+        hipLaunchKernelGGL(quant_scalar_kernel<KIND>, dim3(blocks), dim3(256), 0, stream, p);
+    }
+    return (int)hipGetLastError();
+}
+
+int launch_sym_quant(const uint16_t *x, const uint16_t *scale, uint32_t rows, uint32_t colsSrc, uint32_t colsDst,
+                     int qmax, uint8_t *q, hipStream_t stream)
+{
+    QuantParams p{x, scale, nullptr, nullptr, nullptr, q, rows, colsSrc, colsDst, qmax};
+    return launch_quant<kSym>(p, stream);
+}
+int launch_sym_dual_quant(const uint16_t *x, const uint16_t *s1, const uint16_t *s2, uint32_t rows,
+                          uint32_t colsSrc, uint32_t colsDst, int qmax, uint8_t *q, hipStream_t stream)
+{
+    QuantParams p{x, s1, nullptr, s2, nullptr, q, rows, colsSrc, colsDst, qmax};
+    return launch_quant<kSymDual>(p, stream);
+}
+int launch_asym_quant(const uint16_t *x, const uint16_t *scale, const uint16_t *zeros, uint32_t rows,
+                      uint32_t colsSrc, uint32_t colsDst, uint8_t *q, hipStream_t stream)
+{
+    QuantParams p{x, scale, zeros, nullptr, nullptr, q, rows, colsSrc, colsDst, 15};
+    return launch_quant<kAsym>(p, stream);
+}
+int launch_asym_dual_quant(const uint16_t *x, const uint16_t *s1, const uint16_t *z1, const uint16_t *s2,
+                           const uint16_t *z2, uint32_t rows, uint32_t colsSrc, uint32_t colsDst, uint8_t *q,
+                           hipStream_t stream)
+{
+    QuantParams p{x, s1, z1, s2, z2, q, rows, colsSrc, colsDst, 15};
+    return launch_quant<kAsymDual>(p, stream);
+}
+
+// ---------------------------------------------------------------------------------
+// fused row kernels: scale (and zero) + quantize in one pass over x
+// ---------------------------------------------------------------------------------
+// A row of `cols` elements is split into groups of 32 (four 128-bit loads, one 128-bit
+// store).  WAVES wavefronts share one row; lane t owns groups t, t+T, t+2T, ... (T =
+// 64*WAVES) and keeps up to MAXG of them in registers between the reduction and the
+// quantization, so x is read from HBM exactly once.  Rows longer than 32*MAXG*T elements
+// run the same code with CACHED = false: the groups are read a second time (from L2).
+constexpr int kMaxGroups = 2;  // 2 groups = 64 elements = 32 VGPRs of row data per lane
+
+struct RowParams {
+    const uint16_t *x;
+    uint8_t *q;
+    uint16_t *scale;
+    uint16_t *zeros;
+    uint32_t rows, cols;
+    float clip;
+    int qmax;
+};
+
+__device__ __forceinline__ uint32_t pk_absmax_u16(uint32_t acc, uint32_t w)
+{
+    const v2us a = __builtin_bit_cast(v2us, acc);
+    const v2us b = __builtin_bit_cast(v2us, w & 0x7FFF7FFFu);
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(a, b));
+}
+
+template <int WAVES, bool ASYM, bool CACHED>
+__global__ __launch_bounds__(WAVES * 64) void quantize_rows_kernel(RowParams p)
+{
+    constexpr int T = WAVES * 64;
+    __shared__ float red[2][WAVES];
+    const uint32_t row = blockIdx.x;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t ngroups = p.cols >> 5;  // groups of 32 elements
+    const v4u *xrow = reinterpret_cast<const v4u *>(p.x + (uint64_t)row * p.cols);
+    v4u *qrow = reinterpret_cast<v4u *>(p.q + (uint64_t)row * (p.cols >> 1));
+
+    v4u regs[kMaxGroups][4];
+    uint32_t amax = 0;        // sym: packed max of |x| bit patterns (NaN patterns win, as in torch.max)
+    float fmin_ = INFINITY;   // asym
+    float fmax_ = -INFINITY;
+
+    auto reduce_group = [&](const v4u(&g)[4]) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                if (!ASYM) {
+                    amax = pk_absmax_u16(amax, g[v][w]);
+                } else {
+                    const float lo = (float)bits_to_f16((uint16_t)(g[v][w] & 0xFFFFu));
+                    const float hi = (float)bits_to_f16((uint16_t)(g[v][w] >> 16));
+                    fmin_ = fminf(fmin_, fminf(lo, hi));
+                    fmax_ = fmaxf(fmax_, fmaxf(lo, hi));
+                }
+            }
+    };
+
+    if (CACHED) {
+#pragma unroll
+        for (int i = 0; i < kMaxGroups; ++i) {
+            const uint32_t g = tid + i * T;
+            if (g < ngroups) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v) regs[i][v] = __builtin_nontemporal_load(&xrow[g * 4 + v]);
+            } else {
+#pragma unroll
+                for (int v = 0; v < 4; ++v) regs[i][v] = v4u{0u, 0u, 0u, 0u};
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kMaxGroups; ++i)
+            if (tid + i * T < ngroups) reduce_group(regs[i]);
+    } else {
+        for (uint32_t g = tid; g < ngroups; g += T) {
+            v4u tmp[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) tmp[v] = xrow[g * 4 + v];
+            reduce_group(tmp);
+        }
+    }
+
+    // ---- row reduction: shuffles inside a wavefront, one LDS hop across wavefronts ----
+    float a, b = 0.f;
+    if (!ASYM) {
+        const uint32_t m16 = max(amax & 0xFFFFu, amax >> 16);
+        a = __builtin_bit_cast(float, wave_max_u32(m16));  // carried as raw bits
+    } else {
+        a = wave_min_f32(fmin_);
+        b = wave_max_f32(fmax_);
+    }
+    if (WAVES > 1) {
+        const uint32_t wave = tid >> 6;
+        if ((tid & 63u) == 0) {
+            red[0][wave] = a;
+            red[1][wave] = b;
+        }
+        __syncthreads();
+        if (!ASYM) {
+            uint32_t m = 0;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) m = max(m, __builtin_bit_cast(uint32_t, red[0][w]));
+            a = __builtin_bit_cast(float, m);
+        } else {
+            a = red[0][0];
+            b = red[1][0];
+#pragma unroll
+            for (int w = 1; w < WAVES; ++w) {
+                a = fminf(a, red[0][w]);
+                b = fmaxf(b, red[1][w]);
+            }
+        }
+    }
+
+    // ---- per-token scale / zero (qlinear4bit/nn/quantizer.py:13, 27-31) ----
+    f16 s;
+    f16 z = (f16)0;
+    if (!ASYM) {
+        const f16 am = bits_to_f16((uint16_t)__builtin_bit_cast(uint32_t, a));
+        const f16 s0 = (f16)((float)am / 7.0f);
+        s = (f16)((float)s0 * p.clip);
+    } else {
+        const f16 mn = (f16)a, mx = (f16)b;  // exact: both are binary16 values
+        const f16 d = mx - mn;
+        s = (f16)((float)d / 15.0f);
+        const f16 neg = -mn;
+        const f16 qz = (f16)((float)neg / (float)s);
+        z = (f16)__builtin_rintf((float)qz);
+    }
+    if (tid == 0) {
+        p.scale[row] = f16_to_bits(s);
+        if (ASYM) p.zeros[row] = f16_to_bits(z);
+    }
+    const float rcp = row_rcp(s);
+    const int zi = ASYM ? rint_i32((float)z) : 0;
+
+    // ---- quantize + pack: 32 elements -> one 128-bit store ----
+    auto quant_group = [&](const v4u(&g)[4]) {
+        v4u out;
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+            out[v] = ASYM ? quant8<kAsym>(g[v], 0, rcp, 0.f, 15, zi, (f16)0, (f16)0)
+                          : quant8<kSym>(g[v], 0, rcp, 0.f, p.qmax, 0, (f16)0, (f16)0);
+        return out;
+    };
+    if (CACHED) {
+#pragma unroll
+        for (int i = 0; i < kMaxGroups; ++i) {
+            const uint32_t g = tid + i * T;
+            if (g < ngroups) qrow[g] = quant_group(regs[i]);
+        }
+    } else {
+        for (uint32_t g = tid; g < ngroups; g += T) {
+            v4u tmp[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) tmp[v] = xrow[g * 4 + v];
+            qrow[g] = quant_group(tmp);
+        }
+    }
+}
+
+template <bool ASYM>
+static int launch_rows(const RowParams &p, hipStream_t stream)
+{
+    if (p.rows == 0 || p.cols == 0) return 0;
+    const uint32_t ngroups = p.cols / 32;
+    const dim3 grid(p.rows);
+    // fewest wavefronts per row that still keep the whole row in registers; short rows use
+    // one wavefront, and few-row (decode) calls spread one row over more lanes for latency.
+    int waves = 1;
+    while (waves < 16 && (uint32_t)(waves * 64 * kMaxGroups) < ngroups) waves *= 2;
+    if (p.rows <= 64)
+        while (waves < 4 && (uint32_t)(waves * 64) < ngroups) waves *= 2;
+    const bool cached = (uint32_t)(waves * 64 * kMaxGroups) >= ngroups;
+#define DUQ_ROWS_CASE(W)                                                                                     \
+    case W:                                                                                                  \
+        if (cached)                                                                                          \
+            hipLaunchKernelGGL((quantize_rows_kernel<W, ASYM, true>), grid, dim3(W * 64), 0, stream, p);     \
+        else                                                                                                 \
+            hipLaunchKernelGGL((quantize_rows_kernel<W, ASYM, false>), grid, dim3(W * 64), 0, stream, p);    \
+        break;
+    switch (waves) {
+        DUQ_ROWS_CASE(1)
+        DUQ_ROWS_CASE(2)
+        DUQ_ROWS_CASE(4)
+        DUQ_ROWS_CASE(8)
+        DUQ_ROWS_CASE(16)
+    }
+#undef DUQ_ROWS_CASE
+    return (int)hipGetLastError();
+}
+
+int launch_quantize_rows_sym(const uint16_t *x, uint32_t rows, uint32_t cols, float clip, int qmax, uint8_t *q,
+                             uint16_t *scale, hipStream_t stream)
+{
+    RowParams p{x, q, scale, nullptr, rows, cols, clip, qmax};
+    return launch_rows<false>(p, stream);
+}
+int launch_quantize_rows_asym(const uint16_t *x, uint32_t rows, uint32_t cols, uint8_t *q, uint16_t *scale,
+                              uint16_t *zeros, hipStream_t stream)
+{
+    RowParams p{x, q, scale, zeros, rows, cols, 1.0f, 15};
+    return launch_rows<true>(p, stream);
+}
+
+}  // namespace duq

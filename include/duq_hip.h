@@ -1,0 +1,174 @@
+/*
+ * duq_hip.h - C ABI of libduq_hip.so, the MI355X (gfx950) implementation of the
+ * Linear4bit forward path: per-token int4 quantize -> s4 x s4 GEMM (int32) -> fp16
+ * dequant.
+ *
+ * Every entry point replaces one raw-pointer host launcher of the reference (cited per
+ * function, paths relative to the reference checkout) and keeps its argument order and
+ * meaning, with three changes that hold throughout:
+ *   - binary16 values travel as `duq_half` (uint16_t bit patterns) so the header needs
+ *     no GPU toolkit;
+ *   - a trailing `duq_stream_t` (a hipStream_t, NULL = the null stream) is added: the
+ *     reference always launches on the legacy default stream;
+ *   - the functions return a status instead of void: 0 on success, a negative DUQ_E_*
+ *     code for a rejected argument, or a positive hipError_t from the launch.  They
+ *     never exit, abort or throw.
+ *
+ * All pointers are DEVICE pointers on the current HIP device; inputs are borrowed,
+ * outputs are caller-allocated, the library owns no memory and keeps no global state
+ * (re-entrant).  No call synchronises the host.
+ *
+ * Packed int4 layout everywhere: element i of a row is in byte i/2, low nibble first
+ * (include/int4.h:86-98).
+ */
+#ifndef DUQ_HIP_H
+#define DUQ_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef uint16_t duq_half;   /* IEEE binary16 bit pattern */
+typedef void *duq_stream_t;  /* hipStream_t */
+
+/* status codes (negative = argument rejected before any launch) */
+#define DUQ_OK 0
+#define DUQ_E_NULL (-1)      /* a required pointer is NULL */
+#define DUQ_E_SHAPE (-2)     /* a dimension is inconsistent (e.g. colsDst != ceil(colsSrc/2)) */
+#define DUQ_E_KALIGN (-3)    /* GEMM K is not a multiple of 64 (qlinear4bit/tools/tensor_utils.py:52) */
+#define DUQ_E_MODE (-4)      /* unknown epilogue mode / unsupported qmax */
+#define DUQ_E_ALIGN (-5)     /* a pointer misses the alignment the entry point documents */
+#define DUQ_E_TOO_LARGE (-6) /* a dimension exceeds what the kernels index with 32 bits */
+
+/* symmetric clamp used by the device quantizer of the reference: qmax_sym evaluates to 6
+ * (include/common.h:53-54).  7 is the bound of the Python fake-quant path
+ * (qlinear4bit/tools/quantization.py:29-32). */
+#define DUQ_QMAX_SYM_DEVICE 6
+#define DUQ_QMAX_SYM_FAKEQUANT 7
+#define DUQ_QUANT_COL_K 10   /* include/quant.h:5 */
+
+/* epilogue selectors for duq_linear4bit_forward */
+#define DUQ_EPI_SYM 0        /* src/kernels/quant.cu:64-81   */
+#define DUQ_EPI_ASYM 1       /* src/kernels/quant.cu:149-169 */
+#define DUQ_EPI_SYM_DUAL 2   /* src/kernels/quant2.cu:62-83  */
+#define DUQ_EPI_ASYM_DUAL 3  /* src/kernels/quant2.cu:158-186 */
+
+/* ---- library info ------------------------------------------------------------------ */
+
+/* ABI version of this header (bumped on incompatible change). */
+int duq_abi_version(void);
+/* Text for a status code returned by any function below (static storage). */
+const char *duq_status_string(int status);
+/* QUANT_COL_K; replaces get_dual_quant_col_k (src/export/bindings.cpp:471-473). */
+int duq_get_dual_quant_col_k(void);
+
+/* ---- per-token quantizers with caller-supplied scales ------------------------------- */
+
+/* Replaces sym_quant_host (include/quant.h:9-16, src/kernels/quant.cu:48-61).
+ * q[r, j] packs clamp(rint(x[r,2j]/scale[r]), -8, 6) and the same for 2j+1; the division
+ * is the binary16 quotient, rounding is to nearest even.  colsDst must be
+ * ceil(colsSrc/2); an odd colsSrc leaves the last high nibble 0. */
+int duq_sym_quant_host(const duq_half *x, const duq_half *scale, uint32_t rows, uint32_t colsSrc,
+                       uint32_t colsDst, uint8_t *q, duq_stream_t stream);
+/* Same with an explicit upper clamp (6 or 7). */
+int duq_sym_quant_host_qmax(const duq_half *x, const duq_half *scale, uint32_t rows, uint32_t colsSrc,
+                            uint32_t colsDst, int32_t qmax, uint8_t *q, duq_stream_t stream);
+
+/* Replaces sym_dual_quant_host (include/quant.h:29-37, src/kernels/quant2.cu:47-60):
+ * columns < 10 use scale_1[r], the others scale_2[r]. */
+int duq_sym_dual_quant_host(const duq_half *x, const duq_half *scale_1, const duq_half *scale_2,
+                            uint32_t rows, uint32_t colsSrc, uint32_t colsDst, uint8_t *q,
+                            duq_stream_t stream);
+
+/* Replaces asym_quant_host (include/quant.h:50-58, src/kernels/quant.cu:134-147):
+ * unsigned nibble clamp(rint(x/scale[r]) + rint(zeros[r]), 0, 15). */
+int duq_asym_quant_host(const duq_half *x, const duq_half *scale, const duq_half *zeros, uint32_t rows,
+                        uint32_t colsSrc, uint32_t colsDst, uint8_t *q, duq_stream_t stream);
+
+/* Replaces asym_dual_quant_host.  Argument order follows the DEFINITION
+ * (src/kernels/quant2.cu:141-151: scale_1, zeros_1, scale_2, zeros_2) and its only caller
+ * (src/export/bindings.cpp:417-420), not the differing declaration in
+ * include/quant.h:92-102.  The zero is added in binary16 before rounding
+ * (quant2.cu:133). */
+int duq_asym_dual_quant_host(const duq_half *x, const duq_half *scale_1, const duq_half *zeros_1,
+                             const duq_half *scale_2, const duq_half *zeros_2, uint32_t rows,
+                             uint32_t colsSrc, uint32_t colsDst, uint8_t *q, duq_stream_t stream);
+
+/* ---- fused per-token quantizers (scale computed in the same pass) -------------------- */
+
+/* One pass over x replacing SymQuantizer.forward (qlinear4bit/nn/quantizer.py:10-16;
+ * C++ Quantizer4bit::forward, src/module/quant_tensor.cu:151-161), i.e. the ~5 torch ops
+ * for the scale plus sym_quant_host:
+ *   scale[r] = h(h(max_k|x[r,k]| / 7) * clip),  q as duq_sym_quant_host_qmax.
+ * x rows must be 16-byte aligned (cols % 8 == 0 and x 16-byte aligned); cols even. */
+int duq_quantize_rows_sym(const duq_half *x, uint32_t rows, uint32_t cols, float clip, int32_t qmax,
+                          uint8_t *q, duq_half *scale, duq_stream_t stream);
+
+/* One pass replacing AsymQuantizer.forward (qlinear4bit/nn/quantizer.py:24-35):
+ *   scale[r] = h(h(max-min)/15), zeros[r] = h(rint(h(h(-min)/scale[r]))), q as
+ * duq_asym_quant_host.  Same alignment rules as duq_quantize_rows_sym. */
+int duq_quantize_rows_asym(const duq_half *x, uint32_t rows, uint32_t cols, uint8_t *q, duq_half *scale,
+                           duq_half *zeros, duq_stream_t stream);
+
+/* ---- GEMM ---------------------------------------------------------------------------- */
+
+/* Replaces matmul_host_4bit (include/gemm.h:5-12, src/kernels/gemm.cu:8-43):
+ * C[m,n] = sum_k s4(A[m,k]) * s4(B[n,k]), A [M,K/2] and B [N,K/2] row-major packed,
+ * C [M,N] row-major int32, both operands read as SIGNED nibbles.  K % 64 == 0
+ * (qlinear4bit/tools/tensor_utils.py:52); A, B rows 16-byte aligned follows from that
+ * when A and B are 16-byte aligned, which is required.  Exact for K <= 131008. */
+int duq_matmul_host_4bit(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N, uint32_t K,
+                         int32_t *C, duq_stream_t stream);
+
+/* ---- stand-alone dequant epilogues (int32 accumulators in HBM -> fp16) ---------------- */
+
+/* Replaces sym_dequant_host (include/quant.h:19-26, src/kernels/quant.cu:83-97):
+ * x[r,c] = h(h(scale_row[r]*scale_col[c]) * h_rn(q[r,c])). */
+int duq_sym_dequant_host(const int32_t *q, const duq_half *scale_row, const duq_half *scale_col,
+                         uint32_t rows, uint32_t cols, duq_half *x, duq_stream_t stream);
+
+/* Replaces sym_dual_dequant_host (include/quant.h:40-48, src/kernels/quant2.cu:85-98):
+ * column scale = c < 10 ? scale_col_1[c] : scale_col_2[c]. */
+int duq_sym_dual_dequant_host(const int32_t *q, const duq_half *scale_row, const duq_half *scale_col_1,
+                              const duq_half *scale_col_2, uint32_t rows, uint32_t cols, duq_half *x,
+                              duq_stream_t stream);
+
+/* Replaces asym_dequant_host (include/quant.h:60-69, src/kernels/quant.cu:171-188):
+ * x = h(h(s_r*s_c) * h(h(h_rn(q) - z_r) - z_c)). */
+int duq_asym_dequant_host(const int32_t *q, const duq_half *scale_row, const duq_half *zeros_row,
+                          const duq_half *scale_col, const duq_half *zeros_col, uint32_t rows,
+                          uint32_t cols, duq_half *x, duq_stream_t stream);
+
+/* Replaces asym_dual_dequant_host (include/quant.h:105-116, src/kernels/quant2.cu:188-208):
+ * the column selector of the reference kernel is non-zero for column 0 only
+ * (quant2.cu:182-183), so column 0 uses (scale_col_1, zeros_col_1) and every other
+ * column (scale_col_2, zeros_col_2). */
+int duq_asym_dual_dequant_host(const int32_t *q, const duq_half *scale_row, const duq_half *zeros_row,
+                               const duq_half *scale_col_1, const duq_half *zeros_col_1,
+                               const duq_half *scale_col_2, const duq_half *zeros_col_2, uint32_t rows,
+                               uint32_t cols, duq_half *x, duq_stream_t stream);
+
+/* ---- fused GEMM + dequant (+ bias) ---------------------------------------------------- */
+
+/* One launch replacing matmul_host_4bit + {sym,asym,sym_dual,asym_dual}_dequant_host and
+ * the trailing torch `+ bias` of the module forwards (qlinear4bit/nn/linear.py:42-56,
+ * 104-115,167-176,239-250; C++ Linear4bit::forward, src/module/linear.cu:108-153):
+ * the int32 accumulators never go to HBM.  Results are bit-identical to the unfused
+ * sequence.
+ *   mode       DUQ_EPI_*
+ *   xq         [M,K/2] packed activations, scale_x [M], zeros_x [M] (asym modes, else NULL)
+ *   w          [N,K/2] packed weights
+ *   w_scale_1  [N]; w_zeros_1 [N] (asym modes); w_scale_2 / w_zeros_2 [N] (dual modes)
+ *   bias       [N] or NULL;  y [M,N] fp16 row-major
+ * K % 64 == 0; xq, w 16-byte aligned. */
+int duq_linear4bit_forward(int32_t mode, const uint8_t *xq, const duq_half *scale_x, const duq_half *zeros_x,
+                           const uint8_t *w, const duq_half *w_scale_1, const duq_half *w_zeros_1,
+                           const duq_half *w_scale_2, const duq_half *w_zeros_2, const duq_half *bias,
+                           uint32_t M, uint32_t N, uint32_t K, duq_half *y, duq_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DUQ_HIP_H */

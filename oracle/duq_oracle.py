@@ -1,0 +1,416 @@
+"""CPU oracle for the Linear4bit forward path (quantize -> s4 x s4 GEMM -> dequant).
+
+TEST INFRASTRUCTURE ONLY.  This module is the checker the HIP kernels are compared
+against.  Nothing in the product package may import it; only tests, the smoke entry
+and the benchmark's cpu_baseline leg do.
+
+Every function restates, in NumPy, what one piece of the reference computes, and
+cites the reference lines it follows (paths relative to the reference checkout).
+
+Conventions
+-----------
+* ``h(v)``: round-to-nearest-even to IEEE binary16.  Every fp16 operator of the
+  reference rounds after each operation; here each operation is computed in float32
+  and rounded to float16, which is identical for +, -, *, / on binary16 operands
+  (float32 carries 24 >= 2*11+2 significand bits).
+* Packed int4: element ``i`` of a row lives in byte ``i // 2``, low nibble first
+  (include/int4.h:86-98, qlinear4bit/tools/quantization.py:45-46).
+* ``QMAX_SYM_DEVICE = 6``: the device quantizer clamps to [-8, 6] because
+  ``constexpr int qmax_sym = (7 - 1e-8)`` truncates (include/common.h:53-54).
+  The Python fake-quant path clamps to [-8, 7]
+  (qlinear4bit/tools/quantization.py:29-32).
+
+Pinning status (which independent check fixes each function) is listed next to each
+function; the checks themselves live in tests/test_oracle_*.py.
+
+Behaviour that only the reference's own hardware could settle, and that this oracle
+fixes by definition instead ("parity unpinned" for exactly these corners):
+  * ``__hdiv`` is taken to be the IEEE binary16 quotient (CUDA's is a reciprocal
+    based approximation with a fix-up and may differ in the last bit in rare cases).
+  * the undefined shift in src/kernels/quant2.cu:182-183 for column >= 128 is taken
+    as "false" (the second scale/zero set), the same value it has for 1 <= col < 128.
+  * float->int conversion of +-inf / NaN follows the PTX ``cvt.rni.s32.f16`` rule
+    (saturate, NaN -> 0) and the following int add wraps modulo 2**32.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+QMIN_SYM = -8
+QMAX_SYM_DEVICE = 6      # include/common.h:53-54
+QMAX_SYM_FAKEQUANT = 7   # qlinear4bit/tools/quantization.py:7-8,29-32
+QMIN_ASYM = 0
+QMAX_ASYM = 15           # include/common.h:56-57
+QUANT_COL_K = 10         # include/quant.h:5
+
+_F32 = np.float32
+_F16 = np.float16
+
+
+# ----------------------------------------------------------------------------------
+# fp16 helpers
+# ----------------------------------------------------------------------------------
+def h(v):
+    """Round to binary16 (nearest-even)."""
+    with np.errstate(over="ignore", invalid="ignore"):
+        return np.asarray(v, dtype=_F32).astype(_F16)
+
+
+def _f32(v):
+    return np.asarray(v).astype(_F32)
+
+
+def hmul(a, b):
+    with np.errstate(over="ignore", invalid="ignore"):
+        return h(_f32(a) * _f32(b))
+
+
+def hsub(a, b):
+    with np.errstate(over="ignore", invalid="ignore"):
+        return h(_f32(a) - _f32(b))
+
+
+def hadd(a, b):
+    with np.errstate(over="ignore", invalid="ignore"):
+        return h(_f32(a) + _f32(b))
+
+
+def hdiv(a, b):
+    with np.errstate(over="ignore", invalid="ignore", divide="ignore"):
+        return h(_f32(a) / _f32(b))
+
+
+def int_to_half(acc):
+    """``__int2half_rn`` (src/kernels/quant.cu:4-8): one rounding int32 -> binary16,
+    overflow to +-inf from |v| >= 65520."""
+    with np.errstate(over="ignore"):
+        return np.asarray(acc, dtype=np.int64).astype(np.float64).astype(_F16)
+
+
+def half_to_int_rn(v):
+    """``__half2int_rn``: nearest-even to int32, saturating, NaN -> 0."""
+    x = np.asarray(v, dtype=_F16).astype(np.float64)
+    with np.errstate(invalid="ignore"):
+        r = np.rint(x)
+    r = np.where(np.isnan(r), 0.0, r)
+    r = np.clip(r, -2147483648.0, 2147483647.0)
+    return r.astype(np.int64).astype(np.int32)
+
+
+# ----------------------------------------------------------------------------------
+# A10  pack / unpack  (qlinear4bit/tools/quantization.py:4-15,40-72; int4.h:86-98)
+# pinned by: exhaustive enumeration of all 256 byte values + hand-written bytes.
+# ----------------------------------------------------------------------------------
+def pack_i4(q, sym: bool = True):
+    """[rows, K] integer array -> [rows, ceil(K/2)] uint8.  Range is asserted like the
+    reference (quantization.py:41-43).  Odd K leaves the last high nibble 0, as the
+    device kernels do (src/kernels/quant.cu:27-35)."""
+    q = np.asarray(q)
+    assert q.ndim == 2
+    lo, hi = (-8, 7) if sym else (0, 15)
+    assert q.size == 0 or (q.min() >= lo and q.max() <= hi), "value out of int4 range"
+    nib = (q.astype(np.int64) & 0xF).astype(np.uint8)
+    rows, k = nib.shape
+    if k % 2:
+        nib = np.concatenate([nib, np.zeros((rows, 1), np.uint8)], axis=1)
+    return (nib[:, 0::2] | (nib[:, 1::2] << 4)).astype(np.uint8)
+
+
+def unpack_i4(b, signed: bool = True):
+    """uint8 [..., Kb] -> int32 [..., 2*Kb]; sign-extends when ``signed``
+    (quantization.py:49-72)."""
+    b = np.asarray(b, dtype=np.uint8)
+    lo = (b & 0x0F).astype(np.int32)
+    hi = (b >> 4).astype(np.int32)
+    if signed:
+        lo = np.where(lo >= 8, lo - 16, lo)
+        hi = np.where(hi >= 8, hi - 16, hi)
+    out = np.empty(b.shape[:-1] + (b.shape[-1] * 2,), np.int32)
+    out[..., 0::2] = lo
+    out[..., 1::2] = hi
+    return out
+
+
+# ----------------------------------------------------------------------------------
+# A1  symmetric per-token scale  (qlinear4bit/nn/quantizer.py:13;
+#     src/module/quant_tensor.cu:151-156)
+# pinned by: exact rational model over all non-negative binary16 maxima; torch-CPU.
+# ----------------------------------------------------------------------------------
+def sym_scales(x, clip: float = 1.0):
+    """scale[m] = h( h(max_k|x[m,k]| / 7) * clip ), shape [M, 1] float16.
+
+    torch evaluates fp16-tensor <op> python-scalar in float32 and rounds once.  On a
+    GPU torch multiplies by float32(1/7) instead of dividing; both give the same
+    binary16 for every binary16 maximum (checked exhaustively in the tests)."""
+    x = np.asarray(x, dtype=_F16)
+    amax = np.max(np.abs(x), axis=-1, keepdims=True)
+    with np.errstate(invalid="ignore"):
+        s = h(_f32(amax) / _F32(7.0))
+        s = h(_f32(s) * _F32(clip))
+    return s
+
+
+# ----------------------------------------------------------------------------------
+# A2  symmetric quantize  (src/kernels/quant.cu:11-45)
+# pinned by: hand-computed tie cases; exact rational model on a brute-force grid;
+#            invariants (range, monotone, odd symmetry away from the clamp).
+# ----------------------------------------------------------------------------------
+def sym_quant_values(x, scale, qmax: int = QMAX_SYM_DEVICE):
+    """Unpacked integer codes, int32 [M, K]."""
+    x = np.asarray(x, dtype=_F16)
+    s = np.asarray(scale, dtype=_F16).reshape(-1, 1)
+    q = half_to_int_rn(hdiv(x, s))
+    return np.clip(q, QMIN_SYM, qmax).astype(np.int32)
+
+
+def sym_quant(x, scale, qmax: int = QMAX_SYM_DEVICE):
+    """Packed uint8 [M, ceil(K/2)]."""
+    return pack_i4(sym_quant_values(x, scale, qmax), sym=True)
+
+
+def sym_dual_quant_values(x, scale_1, scale_2, qmax: int = QMAX_SYM_DEVICE):
+    """src/kernels/quant2.cu:9-45: column < 10 uses scale_1[row], else scale_2[row]."""
+    x = np.asarray(x, dtype=_F16)
+    s1 = np.asarray(scale_1, dtype=_F16).reshape(-1, 1)
+    s2 = np.asarray(scale_2, dtype=_F16).reshape(-1, 1)
+    col = np.arange(x.shape[1])[None, :]
+    s = np.where(col < QUANT_COL_K, s1, s2)
+    q = half_to_int_rn(hdiv(x, s))
+    return np.clip(q, QMIN_SYM, qmax).astype(np.int32)
+
+
+def sym_dual_quant(x, scale_1, scale_2, qmax: int = QMAX_SYM_DEVICE):
+    return pack_i4(sym_dual_quant_values(x, scale_1, scale_2, qmax), sym=True)
+
+
+# ----------------------------------------------------------------------------------
+# A3  asymmetric per-token scale/zero + quantize
+#     (qlinear4bit/nn/quantizer.py:24-35; src/kernels/quant.cu:99-132)
+# ----------------------------------------------------------------------------------
+def asym_scales_zeros(x):
+    """scale = h(h(max-min)/15); zero = h(rint(h(h(-min)/scale))); both [M,1] fp16."""
+    x = np.asarray(x, dtype=_F16)
+    mn = np.min(x, axis=-1, keepdims=True)
+    mx = np.max(x, axis=-1, keepdims=True)
+    with np.errstate(invalid="ignore", divide="ignore", over="ignore"):
+        scale = h(_f32(hsub(mx, mn)) / _F32(15.0))
+        neg = h(-_f32(mn))
+        zero = h(np.rint(_f32(hdiv(neg, scale))))
+    return scale, zero
+
+
+def _wrap_i32(v):
+    return ((np.asarray(v, dtype=np.int64) + 2**31) % 2**32 - 2**31).astype(np.int64)
+
+
+def asym_quant_values(x, scale, zero):
+    """u = clamp( rint(h(x/s)) + rint(z), 0, 15 ) (src/kernels/quant.cu:125-126)."""
+    x = np.asarray(x, dtype=_F16)
+    s = np.asarray(scale, dtype=_F16).reshape(-1, 1)
+    z = np.asarray(zero, dtype=_F16).reshape(-1, 1)
+    q = half_to_int_rn(hdiv(x, s)).astype(np.int64)
+    zi = half_to_int_rn(z).astype(np.int64)
+    return np.clip(_wrap_i32(q + zi), QMIN_ASYM, QMAX_ASYM).astype(np.int32)
+
+
+def asym_quant(x, scale, zero):
+    return pack_i4(asym_quant_values(x, scale, zero), sym=False)
+
+
+def asym_dual_quant_values(x, scale_1, zeros_1, scale_2, zeros_2):
+    """src/kernels/quant2.cu:101-139: the zero is added in binary16 BEFORE rounding
+    (``__half2int_rn(data + zero_val)``), unlike quant.cu:126."""
+    x = np.asarray(x, dtype=_F16)
+    col = np.arange(x.shape[1])[None, :]
+    pick = col < QUANT_COL_K
+    s = np.where(pick, np.asarray(scale_1, _F16).reshape(-1, 1), np.asarray(scale_2, _F16).reshape(-1, 1))
+    z = np.where(pick, np.asarray(zeros_1, _F16).reshape(-1, 1), np.asarray(zeros_2, _F16).reshape(-1, 1))
+    q = half_to_int_rn(hadd(hdiv(x, s), z))
+    return np.clip(q, QMIN_ASYM, QMAX_ASYM).astype(np.int32)
+
+
+def asym_dual_quant(x, scale_1, zeros_1, scale_2, zeros_2):
+    return pack_i4(asym_dual_quant_values(x, scale_1, zeros_1, scale_2, zeros_2), sym=False)
+
+
+# ----------------------------------------------------------------------------------
+# A4  s4 x s4 -> s32 GEMM  (src/kernels/gemm.cu:8-43)
+# pinned by: closed form (exact integers), brute-force Python loops on tiny shapes,
+#            special cases (all -8, one-hot rows).
+# ----------------------------------------------------------------------------------
+def matmul_s4(a_packed, b_packed):
+    """C[m,n] = sum_k s4(A[m,k]) * s4(B[n,k]); both operands are read as SIGNED nibbles
+    whatever produced them (src/kernels/gemm.cu:18-20).  int32 [M, N]."""
+    a = unpack_i4(a_packed, signed=True)
+    b = unpack_i4(b_packed, signed=True)
+    assert a.shape[1] == b.shape[1]
+    # float32 GEMM of small integers is exact while |acc| < 2**24 (64*K); use it for
+    # speed when that holds, int64 otherwise.
+    k = a.shape[1]
+    if 64 * k < (1 << 24):
+        c = a.astype(np.float32) @ b.astype(np.float32).T
+        return c.astype(np.int32)
+    return (a.astype(np.int64) @ b.astype(np.int64).T).astype(np.int32)
+
+
+# ----------------------------------------------------------------------------------
+# A5/A6/A7  dequant epilogues  (src/kernels/quant.cu:64-81,149-169;
+#                               src/kernels/quant2.cu:62-83,158-186)
+# pinned by: exact rational model of each rounding on a grid incl. the 65504/65520
+#            boundary; selector enumeration for the dual variants.
+# ----------------------------------------------------------------------------------
+def sym_dequant(acc, scale_row, scale_col):
+    """y = h( h(s_row*s_col) * h_rn(acc) ), float16 [M, N]."""
+    sr = np.asarray(scale_row, _F16).reshape(-1, 1)
+    sc = np.asarray(scale_col, _F16).reshape(1, -1)
+    return hmul(hmul(sr, sc), int_to_half(acc))
+
+
+def asym_dequant(acc, scale_row, zeros_row, scale_col, zeros_col):
+    """y = h( h(s_r*s_c) * h( h( h_rn(acc) - z_r ) - z_c ) )  (quant.cu:167-168)."""
+    sr = np.asarray(scale_row, _F16).reshape(-1, 1)
+    zr = np.asarray(zeros_row, _F16).reshape(-1, 1)
+    sc = np.asarray(scale_col, _F16).reshape(1, -1)
+    zc = np.asarray(zeros_col, _F16).reshape(1, -1)
+    inner = hsub(hsub(int_to_half(acc), zr), zc)
+    return hmul(hmul(sr, sc), inner)
+
+
+def sym_dual_col_scale(scale_col_1, scale_col_2):
+    """col < 10 ? s1[col] : s2[col]  (quant2.cu:81)."""
+    s1 = np.asarray(scale_col_1, _F16).reshape(-1)
+    s2 = np.asarray(scale_col_2, _F16).reshape(-1)
+    col = np.arange(s1.shape[0])
+    return np.where(col < QUANT_COL_K, s1, s2)
+
+
+def sym_dual_dequant(acc, scale_row, scale_col_1, scale_col_2):
+    return sym_dequant(acc, scale_row, sym_dual_col_scale(scale_col_1, scale_col_2))
+
+
+def asym_dual_col_select(v1, v2):
+    """``(QUANT_COL_ST << col & 1)`` parses as ``(ST << col) & 1`` and is non-zero only
+    for col == 0 (quant2.cu:182-183; bit 0 of ST is set, include/quant.h:7)."""
+    v1 = np.asarray(v1, _F16).reshape(-1)
+    v2 = np.asarray(v2, _F16).reshape(-1)
+    col = np.arange(v1.shape[0])
+    return np.where(col == 0, v1, v2)
+
+
+def asym_dual_dequant(acc, scale_row, zeros_row, scale_col_1, zeros_col_1, scale_col_2, zeros_col_2):
+    sc = asym_dual_col_select(scale_col_1, scale_col_2)
+    zc = asym_dual_col_select(zeros_col_1, zeros_col_2)
+    return asym_dequant(acc, scale_row, zeros_row, sc, zc)
+
+
+def add_bias(y, bias):
+    """y + bias as one fp16 torch op (qlinear4bit/nn/linear.py:53-54)."""
+    return hadd(y, np.asarray(bias, _F16).reshape(1, -1))
+
+
+# ----------------------------------------------------------------------------------
+# A8  module forwards as compositions (qlinear4bit/nn/linear.py:42-56,104-115,
+#     167-176,239-250)
+# ----------------------------------------------------------------------------------
+def linear4bit_sq_forward(x, w_packed, w_scales, bias=None, clip=1.0, qmax=QMAX_SYM_DEVICE):
+    """Sequential(SymQuantizer, Linear4bitSQ)(x).  Returns (y, acc, q_x, s_x)."""
+    x = np.asarray(x, _F16)
+    s_x = sym_scales(x, clip)
+    q_x = sym_quant(x, s_x, qmax)
+    acc = matmul_s4(q_x, w_packed)
+    y = sym_dequant(acc, s_x, w_scales)
+    if bias is not None:
+        y = add_bias(y, bias)
+    return y, acc, q_x, s_x
+
+
+def linear4bit_asq_forward(x, w_packed, w_scales, w_zeros, bias=None):
+    """Linear4bitASQ(x) with its own AsymQuantizer.  Returns (y, acc, q_x, s_x, z_x)."""
+    x = np.asarray(x, _F16)
+    s_x, z_x = asym_scales_zeros(x)
+    q_x = asym_quant(x, s_x, z_x)
+    acc = matmul_s4(q_x, w_packed)
+    y = asym_dequant(acc, s_x, z_x, w_scales, w_zeros)
+    if bias is not None:
+        y = add_bias(y, bias)
+    return y, acc, q_x, s_x, z_x
+
+
+def linear4bit_dusq_forward(x, w_packed, w_scales_1, w_scales_2, bias=None, clip=1.0, qmax=QMAX_SYM_DEVICE):
+    x = np.asarray(x, _F16)
+    s_x = sym_scales(x, clip)
+    q_x = sym_quant(x, s_x, qmax)
+    acc = matmul_s4(q_x, w_packed)
+    y = sym_dual_dequant(acc, s_x, w_scales_1, w_scales_2)
+    if bias is not None:
+        y = add_bias(y, bias)
+    return y, acc, q_x, s_x
+
+
+def linear4bit_duasq_forward(x, w_packed, ws1, wz1, ws2, wz2, bias=None):
+    x = np.asarray(x, _F16)
+    s_x, z_x = asym_scales_zeros(x)
+    q_x = asym_quant(x, s_x, z_x)
+    acc = matmul_s4(q_x, w_packed)
+    y = asym_dual_dequant(acc, s_x, z_x, ws1, wz1, ws2, wz2)
+    if bias is not None:
+        y = add_bias(y, bias)
+    return y, acc, q_x, s_x, z_x
+
+
+# ----------------------------------------------------------------------------------
+# A11  CPU fake-quant primitives (qlinear4bit/tools/quantization.py:17-37), for fp16
+#      inputs (torch-CPU computes each op in float32 and stores binary16).
+# pinned by: the torch-CPU ops themselves (the library routine the reference calls).
+# ----------------------------------------------------------------------------------
+def fq_sym_quant(x, scale, maxq=QMAX_SYM_FAKEQUANT):
+    """q = clamp(round(x / scale), -(maxq+1), maxq), as float16 values."""
+    x = np.asarray(x, _F16)
+    s = np.asarray(scale, _F16)
+    with np.errstate(invalid="ignore"):
+        q = h(np.rint(_f32(hdiv(x, s))))
+        return h(np.clip(_f32(q), -(maxq + 1), maxq))
+
+
+def fq_sym_dequant(q, scale):
+    return hmul(scale, q)
+
+
+def fq_asym_quant(x, scale, zero, maxq=QMAX_ASYM):
+    x = np.asarray(x, _F16)
+    with np.errstate(invalid="ignore"):
+        r = h(np.rint(_f32(hdiv(x, scale))))
+        return h(np.clip(_f32(hadd(r, zero)), 0, maxq))
+
+
+def fq_asym_dequant(q, scale, zero):
+    return hmul(scale, hsub(q, zero))
+
+
+# ----------------------------------------------------------------------------------
+# Weight preparation (qlinear4bit/nn/linear.py:58-78,117-145) - used to build the
+# benchmark / parity inputs the way the reference builds its buffers.
+# ----------------------------------------------------------------------------------
+def weight_sym_from_float(w, w_scales):
+    """int_w = round(W / s_w) in fp16, no clamp; pack_i4 asserts the range
+    (linear.py:72-73)."""
+    w = np.asarray(w, _F16)
+    s = np.asarray(w_scales, _F16).reshape(-1, 1)
+    q = np.rint(_f32(hdiv(w, s))).astype(np.int32)
+    return pack_i4(q, sym=True)
+
+
+def weight_asym_from_linear(w):
+    """Linear4bitASQ.from_linear (linear.py:126-140): max|W| and min|W| (abs on both),
+    scale = (max-min)/15, zero = round(-min/scale), q = clamp(round(W/scale)+zero,0,15).
+    Returns (packed u8 [N,K/2], scale fp16 [N,1], zero fp16 [N,1])."""
+    w = np.asarray(w, _F16)
+    aw = np.abs(w)
+    mx = np.max(aw, axis=-1, keepdims=True)
+    mn = np.min(aw, axis=-1, keepdims=True)
+    with np.errstate(invalid="ignore", divide="ignore", over="ignore"):
+        scale = h(_f32(hsub(mx, mn)) / _F32(15.0))
+        zero = h(np.rint(_f32(hdiv(h(-_f32(mn)), scale))))
+        r = h(np.rint(_f32(hdiv(w, scale))))
+        q = np.clip(_f32(hadd(r, zero)), 0, 15)
+    return pack_i4(q.astype(np.int32), sym=False), scale, zero
