@@ -24,7 +24,7 @@ __device__ __forceinline__ uint16_t f16_to_bits(f16 v) { return __builtin_bit_ca
 __device__ __forceinline__ int cvt_i32_sat(float v)
 {
     int r;
-    asm volatile("v_cvt_i32_f32 %0, %1" : "=v"(r) : "v"(v));
+    asm("v_cvt_i32_f32 %0, %1" : "=v"(r) : "v"(v));
     return r;
 }
 

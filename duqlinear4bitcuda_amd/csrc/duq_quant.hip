@@ -287,7 +287,11 @@ __global__ __launch_bounds__(WAVES * 64) void quantize_rows_kernel(RowParams p)
     if (!ASYM) {
         const f16 am = bits_to_f16((uint16_t)__builtin_bit_cast(uint32_t, a));
         const f16 s0 = (f16)((float)am / 7.0f);
-        s = (f16)((float)s0 * p.clip);
+        // torch multiplies in float32, rounds to float32, then to binary16: keep the two
+        // roundings apart (a mixed-precision FMA would round the exact product once).
+        float sc = (float)s0 * p.clip;
+        asm volatile("" : "+v"(sc));
+        s = (f16)sc;
     } else {
         const f16 mn = (f16)a, mx = (f16)b;  // exact: both are binary16 values
         const f16 d = mx - mn;
