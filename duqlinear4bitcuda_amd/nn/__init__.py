@@ -1,0 +1,2 @@
+from .linear import Linear4bitSQ, Linear4bitASQ, Linear4bitDUSQ, LinearQuant4bitDUASQ
+from .quantizer import SymQuantizer, AsymQuantizer

@@ -1,0 +1,224 @@
+"""4-bit linear layers with the class names, buffer names/shapes and forward semantics
+of the reference's ``qlinear4bit/nn/linear.py``.  The forward is one fused launch
+(GEMM + dequant + bias) instead of matmul + dequant + a torch add; ``fused = False`` on
+a module switches back to the reference's three-step sequence (same bits).
+
+Buffers (the state_dict contract): ``weight`` uint8 [N, K/2]; ``weight_scales`` [N, 1]
+(``weight_scales_1/_2`` for the dual layers); ``weight_zeros*`` fp16 [N, 1] for the
+asymmetric layers; optional ``bias`` [N].
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import _HIP as _ops
+from ..tools import quantization as quant_utils
+from ..tools import tensor_utils
+from .quantizer import AsymQuantizer, SymQuantizer  # noqa: F401  (re-exported like the reference)
+
+_INT4_LEVELS = 2 ** 4
+
+
+def _placeholder_weight(out_features, in_features):
+    return torch.randint(1, 7, (out_features, in_features // 2), dtype=torch.uint8, requires_grad=False)
+
+
+def _asym_params(w: torch.Tensor):
+    """Per-row scale / zero / codes the way the reference's ``from_linear`` computes them:
+    max and min are taken over |W| (linear.py:129-136)."""
+    aw = w.abs()
+    w_max = aw.amax(dim=-1, keepdim=True)
+    w_min = aw.amin(dim=-1, keepdim=True)
+    scale = (w_max - w_min) / (_INT4_LEVELS - 1)
+    zeros = (-w_min / scale).round().to(torch.float16)
+    codes = torch.clamp(torch.round(w / scale) + zeros, 0, _INT4_LEVELS - 1)
+    return scale, zeros, codes
+
+
+class _Linear4bitBase(torch.nn.Module):
+    fused = True
+
+    def _finish(self, y):
+        return y if self.bias is None else y + self.bias
+
+
+class Linear4bitSQ(_Linear4bitBase):
+    """Symmetric 4-bit linear layer; takes a PackedQuantizedTensor (linear.py:24-78)."""
+
+    def __init__(self, in_features, out_features, bias=False, dtype=torch.float16):
+        super().__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+        self.register_buffer("weight_scales", torch.zeros((out_features, 1), requires_grad=False))
+        self.register_buffer("weight", _placeholder_weight(out_features, in_features))
+        if bias:
+            self.register_buffer("bias", torch.zeros((out_features), dtype=dtype))
+        else:
+            self.bias = None
+
+    def forward(self, x):
+        assert type(x) == tensor_utils.PackedQuantizedTensor  # quantized input is required
+        xq, scales_x = x.quantized_x, x.scales_x
+        if self.fused:
+            return tensor_utils.linear_forward(_ops.EPI_SYM, xq, scales_x, None, self.weight, self.weight_scales,
+                                               bias=self.bias)
+        acc = tensor_utils.matmul(xq, self.weight)
+        return self._finish(tensor_utils.sym_dequant(acc, scales_x, self.weight_scales))
+
+    @staticmethod
+    def from_float(module: torch.nn.Linear, weight_scales=None):
+        """Quantize ``module.weight`` with the given per-row scales: round(W / s), no clamp
+        (pack_i4 rejects values outside [-8, 7]) (linear.py:58-78)."""
+        w = module.weight.data
+        new = Linear4bitSQ(module.in_features, module.out_features, bias=module.bias is not None,
+                           dtype=w.dtype).to(w.dtype)
+        if weight_scales is not None:
+            assert weight_scales.shape == (module.out_features, 1), "weight_scales should have shape (out_features, 1)"
+            new.weight_scales.copy_(weight_scales.to(w.dtype))
+            codes = (w / weight_scales.to(w.device)).round()
+            new.weight.copy_(quant_utils.pack_i4(codes.to(torch.int8)))
+            if module.bias is not None:
+                new.bias.copy_(module.bias)
+        return new
+
+
+class Linear4bitASQ(_Linear4bitBase):
+    """Asymmetric 4-bit linear layer with its own AsymQuantizer (linear.py:80-145)."""
+
+    def __init__(self, in_features, out_features, bias=False, require_quantizer=True):
+        super().__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+        self.require_quantizer = require_quantizer
+        self.register_buffer("weight_scales", torch.zeros((out_features, 1), requires_grad=False, dtype=torch.float16))
+        self.register_buffer("weight_zeros", torch.zeros((out_features, 1), requires_grad=False, dtype=torch.float16))
+        self.register_buffer("weight", _placeholder_weight(out_features, in_features))
+        if bias:
+            self.register_buffer("bias", torch.zeros((out_features), dtype=torch.float16))
+        else:
+            self.bias = None
+        if require_quantizer:
+            self.quantizer = AsymQuantizer()
+
+    def forward(self, x):
+        if self.require_quantizer:
+            x = self.quantizer(x)
+        assert type(x) == tensor_utils.PackedQuantizedTensor, \
+            "Input should be quantized tensor, or require_quantizer should be passed as initial argument"
+        xq, scales_x, zeros_x = x.quantized_x, x.scales_x, x.zeros_x
+        if self.fused:
+            return tensor_utils.linear_forward(_ops.EPI_ASYM, xq, scales_x, zeros_x, self.weight, self.weight_scales,
+                                               self.weight_zeros, bias=self.bias)
+        acc = tensor_utils.matmul(xq, self.weight)
+        return self._finish(tensor_utils.asym_dequant(acc, scales_x, zeros_x, self.weight_scales, self.weight_zeros))
+
+    @classmethod
+    def from_linear(cls, module: torch.nn.Linear, require_quantizer: bool = True):
+        new = cls(module.in_features, module.out_features, bias=module.bias is not None,
+                  require_quantizer=require_quantizer)
+        scale, zeros, codes = _asym_params(module.weight.data)
+        new.weight.copy_(quant_utils.pack_i4(codes.to(torch.int8), sym=False))
+        new.weight_scales.copy_(scale.to(torch.float16))
+        new.weight_zeros.copy_(zeros.to(torch.float16))
+        if module.bias is not None:
+            new.bias.copy_(module.bias)
+        return new
+
+
+class Linear4bitDUSQ(_Linear4bitBase):
+    """Symmetric layer with two per-row weight scales: input columns < 10 were quantized
+    with scale 1, the rest with scale 2; the epilogue picks per OUTPUT column < 10
+    (linear.py:147-206, quant2.cu:81)."""
+
+    def __init__(self, in_features, out_features, bias=False, dtype=torch.float16):
+        super().__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+        self.register_buffer("weight_scales_1", torch.zeros((out_features, 1), requires_grad=False))
+        self.register_buffer("weight_scales_2", torch.zeros((out_features, 1), requires_grad=False))
+        self.register_buffer("weight", _placeholder_weight(out_features, in_features))
+        if bias:
+            self.register_buffer("bias", torch.zeros((out_features), dtype=dtype))
+        else:
+            self.bias = None
+
+    def forward(self, x):
+        assert type(x) == tensor_utils.PackedQuantizedTensor
+        xq, scales_x = x.quantized_x, x.scales_x
+        if self.fused:
+            return tensor_utils.linear_forward(_ops.EPI_SYM_DUAL, xq, scales_x, None, self.weight,
+                                               self.weight_scales_1, None, self.weight_scales_2, bias=self.bias)
+        acc = tensor_utils.matmul(xq, self.weight)
+        return self._finish(tensor_utils.sym_dual_dequant(acc, scales_x, self.weight_scales_1, self.weight_scales_2))
+
+    @staticmethod
+    def from_float(module: torch.nn.Linear, weight_scales_1=None, weight_scales_2=None):
+        w = module.weight.data
+        new = Linear4bitDUSQ(module.in_features, module.out_features, bias=module.bias is not None,
+                             dtype=w.dtype).to(w.dtype)
+        if weight_scales_1 is not None and weight_scales_2 is not None:
+            shape = (module.out_features, 1)
+            assert weight_scales_1.shape == shape, "weight_scales_1 should have shape (out_features, 1)"
+            assert weight_scales_2.shape == shape, "weight_scales_2 should have shape (out_features, 1)"
+            new.weight_scales_1.copy_(weight_scales_1.to(w.dtype))
+            new.weight_scales_2.copy_(weight_scales_2.to(w.dtype))
+            split = tensor_utils.get_dual_quant_col()
+            left = (w[:, :split] / weight_scales_1.to(w.device)).round()
+            right = (w[:, split:] / weight_scales_2.to(w.device)).round()
+            codes = torch.cat([left, right], dim=-1)
+            new.weight.copy_(quant_utils.pack_i4(codes.to(torch.int8)))
+            if module.bias is not None:
+                new.bias.copy_(module.bias)
+        return new
+
+
+class LinearQuant4bitDUASQ(_Linear4bitBase):
+    """Asymmetric dual-uniform layer (linear.py:209-297)."""
+
+    def __init__(self, in_features, out_features, bias=False, require_quantizer=True):
+        super().__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+        self.require_quantizer = require_quantizer
+        for name in ("weight_scales_1", "weight_zeros_1", "weight_scales_2", "weight_zeros_2"):
+            self.register_buffer(name, torch.zeros((out_features, 1), requires_grad=False, dtype=torch.float16))
+        self.register_buffer("weight", _placeholder_weight(out_features, in_features))
+        if bias:
+            self.register_buffer("bias", torch.zeros((out_features), dtype=torch.float16))
+        else:
+            self.bias = None
+        if self.require_quantizer:
+            self.quantizer = AsymQuantizer()
+
+    def forward(self, x):
+        if self.require_quantizer:
+            x = self.quantizer(x)
+        assert type(x) == tensor_utils.PackedQuantizedTensor, \
+            "Input should be quantized tensor, or require_quantizer should be passed as initial argument"
+        xq, scales_x, zeros_x = x.quantized_x, x.scales_x, x.zeros_x
+        if self.fused:
+            return tensor_utils.linear_forward(_ops.EPI_ASYM_DUAL, xq, scales_x, zeros_x, self.weight,
+                                               self.weight_scales_1, self.weight_zeros_1, self.weight_scales_2,
+                                               self.weight_zeros_2, bias=self.bias)
+        acc = tensor_utils.matmul(xq, self.weight)
+        return self._finish(tensor_utils.asym_dual_dequant(acc, scales_x, zeros_x, self.weight_scales_1,
+                                                           self.weight_zeros_1, self.weight_scales_2,
+                                                           self.weight_zeros_2))
+
+    @classmethod
+    def from_linear(cls, module: torch.nn.Linear, require_quantizer=True):
+        new = cls(module.in_features, module.out_features, bias=module.bias is not None,
+                  require_quantizer=require_quantizer)
+        w = module.weight.data
+        split = tensor_utils.get_dual_quant_col()
+        s1, z1, c1 = _asym_params(w[:, :split])
+        s2, z2, c2 = _asym_params(w[:, split:])
+        codes = torch.cat([c1, c2], dim=-1)
+        new.weight.copy_(quant_utils.pack_i4(codes.to(torch.int8), sym=False))
+        new.weight_scales_1.copy_(s1.to(torch.float16))
+        new.weight_zeros_1.copy_(z1.to(torch.float16))
+        new.weight_scales_2.copy_(s2.to(torch.float16))
+        new.weight_zeros_2.copy_(z2.to(torch.float16))
+        if module.bias is not None:
+            new.bias.copy_(module.bias)
+        return new

@@ -1,0 +1,144 @@
+"""Shape-handling wrappers over the device ops, with the names, argument order and
+asserts of the reference's ``qlinear4bit/tools/tensor_utils.py`` (which calls
+``qlinear4bit._CUDA``; this one calls ``duqlinear4bitcuda_amd._HIP``).
+
+Leading dimensions are flattened for the kernels and restored on the result.
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import _HIP as _ops
+
+
+class PackedQuantizedTensor:
+    """A quantized activation: packed nibbles plus per-token scale (and zero point)
+    (tensor_utils.py:20-38)."""
+
+    def __init__(self, quantized_x: torch.Tensor, scales_x: torch.Tensor, zeros_x: torch.Tensor = None):
+        self.quantized_x = quantized_x
+        self.scales_x = scales_x
+        self.zeros_x = zeros_x
+
+    def size(self):
+        return self.quantized_x.size()
+
+    @property
+    def device(self):
+        return self.quantized_x.device
+
+    @property
+    def dtype(self):
+        return self.quantized_x.dtype
+
+
+def flatten_last_dim_and_return_shape(x: torch.Tensor):
+    lead = x.shape[:-1]
+    return x.view(-1, x.shape[-1]), lead
+
+
+def _flat(x):
+    return x.view(-1, x.shape[-1]), tuple(x.shape[:-1])
+
+
+def matmul(A, B):
+    """Packed s4 x packed s4 -> int32; the packed last dim must be a multiple of 32 bytes
+    (tensor_utils.py:51-55)."""
+    assert A.shape[-1] % 32 == 0, "A.shape[-1]: {} must be multiplication of 32".format(A.shape[-1])
+    A2, a_lead = _flat(A)
+    B2, b_lead = _flat(B)
+    return _ops.matmul(A2, B2).view(*a_lead, *b_lead)
+
+
+def sym_quant(x, scale, qmax: int = 6):
+    assert x.dtype == scale.dtype == torch.float16
+    x2, lead = _flat(x)
+    return _ops.sym_quant(x2, scale.view(-1), qmax).view(*lead, -1)
+
+
+def sym_dual_quant(x, scale_1, scale_2):
+    assert x.dtype == scale_1.dtype == scale_2.dtype == torch.float16
+    x2, lead = _flat(x)
+    return _ops.sym_dual_quant(x2, scale_1.view(-1), scale_2.view(-1)).view(*lead, -1)
+
+
+def sym_dequant(q, scale_row, scale_col, bits=32):
+    assert q.dtype == torch.int32
+    assert scale_row.dtype == scale_col.dtype == torch.float16
+    q2, lead = _flat(q)
+    return _ops.sym_dequant(q2, scale_row.view(-1), scale_col, bits).view(*lead, -1)
+
+
+def sym_dual_dequant(q, scale_row, scale_col_1, scale_col_2, bits=32):
+    assert q.dtype == torch.int32
+    assert scale_row.dtype == scale_col_1.dtype == scale_col_2.dtype == torch.float16
+    q2, lead = _flat(q)
+    return _ops.sym_dual_dequant(q2, scale_row.view(-1), scale_col_1, scale_col_2, bits).view(*lead, -1)
+
+
+def asym_quant(q, scale, zero):
+    assert q.dtype == torch.float16
+    assert scale.dtype == zero.dtype == torch.float16
+    x2, lead = _flat(q)
+    return _ops.asym_quant(x2, scale.view(-1), zero.view(-1)).view(*lead, -1)
+
+
+def asym_dequant(q, scale_row, zeros_row, scale_col, zeros_col, bits=32):
+    assert q.dtype == torch.int32
+    assert scale_row.dtype == zeros_row.dtype == scale_col.dtype == zeros_col.dtype == torch.float16
+    q2, lead = _flat(q)
+    return _ops.asym_dequant(q2, scale_row.view(-1), zeros_row.view(-1), scale_col.view(-1), zeros_col.view(-1),
+                             bits).view(*lead, -1)
+
+
+def asym_dual_quant(q, scale_1, zeros1, scale_2, zeros2):
+    """The reference wrapper asserts ``q.dtype == int32`` here (tensor_utils.py:126), which
+    can never hold for the fp16 input the kernel takes; fp16 is what is checked."""
+    assert q.dtype == torch.float16
+    assert scale_1.dtype == scale_2.dtype == torch.float16
+    assert zeros1.dtype == zeros2.dtype == torch.float16
+    x2, lead = _flat(q)
+    return _ops.asym_dual_quant(x2, scale_1.view(-1), zeros1.view(-1), scale_2.view(-1),
+                                zeros2.view(-1)).view(*lead, -1)
+
+
+def asym_dual_dequant(q, scale_row, zeros_row, scale_col_1, zeros_col_1, scale_col_2, zeros_col_2, bits=32):
+    assert q.dtype == torch.int32
+    assert scale_row.dtype == scale_col_1.dtype == scale_col_2.dtype == torch.float16
+    assert zeros_row.dtype == zeros_col_1.dtype == zeros_col_2.dtype == torch.float16
+    q2, lead = _flat(q)
+    return _ops.asym_dual_dequant(q2, scale_row.view(-1), zeros_row.view(-1), scale_col_1.view(-1),
+                                  zeros_col_1.view(-1), scale_col_2.view(-1), zeros_col_2.view(-1),
+                                  bits).view(*lead, -1)
+
+
+def get_dual_quant_col():
+    return _ops.get_dual_quant_col_k()
+
+
+# ---- fused additions (no counterpart in the reference wrappers) ------------------------
+
+def quantize_sym(x, clip: float = 1.0, qmax: int = 6):
+    """One launch for scale + quantize; returns (q [..., K/2], scales [..., 1])."""
+    assert x.dtype == torch.float16
+    x2, lead = _flat(x)
+    q, s = _ops.quantize_rows_sym(x2, clip, qmax)
+    return q.view(*lead, -1), s.view(*lead, 1)
+
+
+def quantize_asym(x):
+    assert x.dtype == torch.float16
+    x2, lead = _flat(x)
+    q, s, z = _ops.quantize_rows_asym(x2)
+    return q.view(*lead, -1), s.view(*lead, 1), z.view(*lead, 1)
+
+
+def linear_forward(mode, xq, scales_x, zeros_x, weight, w_scale_1, w_zeros_1=None, w_scale_2=None, w_zeros_2=None,
+                   bias=None):
+    """GEMM + dequant (+ bias) in one launch; result has xq's leading dims and N columns."""
+    assert xq.shape[-1] % 32 == 0, "A.shape[-1]: {} must be multiplication of 32".format(xq.shape[-1])
+    x2, lead = _flat(xq)
+    v = lambda t: None if t is None else t.view(-1)
+    y = _ops.linear4bit_forward(mode, x2, v(scales_x), v(zeros_x), weight, v(w_scale_1), v(w_zeros_1), v(w_scale_2),
+                                v(w_zeros_2), v(bias))
+    return y.view(*lead, -1)
