@@ -23,6 +23,8 @@
 //    (no LDS for operands), partial sums meet in LDS once at the end.
 #include "duq_epilogue.h"
 #include "duq_launch.h"
+#include <cstdlib>
+#include <type_traits>
 
 namespace duq {
 
@@ -236,6 +238,208 @@ __global__ __launch_bounds__(256) void gemm_s4_tile_kernel(GemmParams p)
 }
 
 // ---------------------------------------------------------------------------------
+// stream kernel (prefill): weights global -> registers, activations through LDS
+// ---------------------------------------------------------------------------------
+// Workgroup = 4 wavefronts side by side along N: every wavefront owns 16*TN weight rows
+// that no other wavefront of the workgroup needs, so weight fragments never go through
+// LDS: lane (l16, g) loads bytes [g*32, g*32+32) of the 128-byte row segment of a 256-k
+// chunk straight into registers (two 128-bit loads = one full cache line per row and
+// chunk), one chunk ahead of the MFMAs that consume them.  The 16*TM activation rows are
+// shared by the four wavefronts: they are expanded to bytes once on the way into LDS
+// (double buffered, rows padded to 272 B) and read back as 128-bit fragments.
+// LDS traffic per 256-k chunk drops to BM*256 B written + 4*BM*256 B read.
+//
+// All global reads are raw buffer loads on per-workgroup descriptors that cover exactly
+// the rows of this tile: rows past M or N read as zero without a branch, and the chunk
+// offset rides in the scalar offset.  Only a ragged last chunk (K % 256 != 0) uses
+// per-piece guarded offsets.
+constexpr int kCK = 256;         // k elements per chunk (128 packed bytes per row)
+constexpr int kXStride = 272;    // LDS bytes per activation row: 256 expanded + 16 pad
+constexpr uint32_t kOobOffset = 0xFFFFFF00u;  // beyond any descriptor: the load returns 0
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, uint32_t bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ v4u buf_load16(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff)
+{
+    return __builtin_bit_cast(v4u, __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)soff, 0));
+}
+
+template <int TM, int TN, int EPI, bool BIAS>
+__global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
+{
+    constexpr int BM = 16 * TM;
+    constexpr int WN = 16 * TN;
+    constexpr int BN = 4 * WN;
+    constexpr int NXP = BM / 32;  // 16-byte activation pieces per thread and chunk
+    static_assert(BM % 32 == 0, "BM");
+
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2][BM * kXStride];
+
+    uint32_t tile_m, tile_n;
+    tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+    const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u, wave = tid >> 6;
+    const uint32_t l16 = lane & 15u, g = lane >> 4;
+    const uint32_t kbytes = p.K >> 1;
+    const uint32_t nfull = p.K / kCK;
+    const uint32_t nchunks = (p.K + kCK - 1) / kCK;
+
+    const __amdgpu_buffer_rsrc_t rW = make_rsrc(p.B + (uint64_t)n0 * kbytes, min(p.N - n0, (uint32_t)BN) * kbytes);
+    const __amdgpu_buffer_rsrc_t rX = make_rsrc(p.A + (uint64_t)m0 * kbytes, min(p.M - m0, (uint32_t)BM) * kbytes);
+
+    uint32_t woff[TN];
+#pragma unroll
+    for (int a = 0; a < TN; ++a) woff[a] = (wave * WN + a * 16 + l16) * kbytes + g * 32;
+    uint32_t xoff[NXP], xlds[NXP];
+    const uint32_t xq = tid & 7u;  // which 16-byte piece of the 128-byte row segment
+#pragma unroll
+    for (int i = 0; i < NXP; ++i) {
+        const uint32_t row = (tid >> 3) + i * 32;
+        xoff[i] = row * kbytes + xq * 16;
+        xlds[i] = row * kXStride + xq * 32;
+    }
+
+    v4u wreg[TN][2];
+    v4u xreg[NXP];
+
+    // PF selects how the NEXT chunk is fetched: 0 none, 1 full chunk (no guards), 2 ragged
+    // last chunk (pieces past the row end are redirected out of bounds and read as zero).
+    auto load_w = [&](auto pf, int j, uint32_t c) {
+        constexpr int PF = decltype(pf)::value;
+        const uint32_t koff = c * (kCK / 2);
+        if (PF == 1) {
+#pragma unroll
+            for (int a = 0; a < TN; ++a) wreg[a][j] = buf_load16(rW, woff[a] + j * 16, koff);
+        } else if (PF == 2) {
+            const bool ok = koff + g * 32 + j * 16 < kbytes;  // K % 64 == 0: all in or all out
+#pragma unroll
+            for (int a = 0; a < TN; ++a) wreg[a][j] = buf_load16(rW, ok ? woff[a] + j * 16 : kOobOffset, koff);
+        }
+    };
+    auto load_x = [&](auto pf, uint32_t c) {
+        constexpr int PF = decltype(pf)::value;
+        const uint32_t koff = c * (kCK / 2);
+        if (PF == 1) {
+#pragma unroll
+            for (int i = 0; i < NXP; ++i) xreg[i] = buf_load16(rX, xoff[i], koff);
+        } else if (PF == 2) {
+            const bool okx = koff + xq * 16 < kbytes;
+#pragma unroll
+            for (int i = 0; i < NXP; ++i) xreg[i] = buf_load16(rX, okx ? xoff[i] : kOobOffset, koff);
+        }
+    };
+    auto store_x = [&](uint32_t buf) {
+        uint8_t *base = lds[buf];
+#pragma unroll
+        for (int i = 0; i < NXP; ++i) {
+            v4u ev, od;
+            expand_nibbles(xreg[i], ev, od);
+            *reinterpret_cast<v4u *>(base + xlds[i]) = ev;
+            *reinterpret_cast<v4u *>(base + xlds[i] + 16) = od;
+        }
+    };
+
+    v4i acc[TN][TM];
+#pragma unroll
+    for (int a = 0; a < TN; ++a)
+#pragma unroll
+        for (int b = 0; b < TM; ++b) acc[a][b] = v4i{0, 0, 0, 0};
+
+    const uint32_t fragX = l16 * kXStride + g * 64;  // fragment step*16 with step = j*2+par
+
+    // One chunk = 4 MFMA steps (j, par), each TM groups of TN MFMAs.  The instruction order
+    // is fixed by hand (scheduling fences around every MFMA group): while the TN MFMAs of a
+    // group run, the next step's activation fragment for the same group index is read from
+    // LDS, the weight registers of half j are refilled for the next chunk right after they
+    // were expanded, and the next chunk's activations are expanded and written to the other
+    // LDS buffer inside the last step.  MFMAs are issued through inline assembly with the
+    // accumulators tied to the accumulation register file, so they never move.
+    auto body = [&](auto pf, uint32_t c) {
+        constexpr int PF = decltype(pf)::value;
+        const uint32_t cur = c & 1u;
+        const uint8_t *base = lds[cur] + fragX;
+        uint8_t *nbase = lds[cur ^ 1u];
+        load_x(pf, c + 1);
+        v4i fx[2][TM];
+#pragma unroll
+        for (int b = 0; b < TM; ++b) fx[0][b] = *reinterpret_cast<const v4i *>(base + b * 16 * kXStride);
+        v4u we[TN], wo[TN];
+#pragma unroll
+        for (int step = 0; step < 4; ++step) {
+            const int j = step >> 1, par = step & 1;
+            if (par == 0) {
+#pragma unroll
+                for (int a = 0; a < TN; ++a) expand_nibbles(wreg[a][j], we[a], wo[a]);
+                load_w(pf, j, c + 1);
+            }
+#pragma unroll
+            for (int b = 0; b < TM; ++b) {
+                if (step < 3)
+                    fx[(step + 1) & 1][b] =
+                        *reinterpret_cast<const v4i *>(base + b * 16 * kXStride + (step + 1) * 16);
+                if (PF != 0 && step == 3 && b < NXP) {  // next chunk's activations -> LDS
+                    v4u ev, od;
+                    expand_nibbles(xreg[b], ev, od);
+                    *reinterpret_cast<v4u *>(nbase + xlds[b]) = ev;
+                    *reinterpret_cast<v4u *>(nbase + xlds[b] + 16) = od;
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int a = 0; a < TN; ++a)
+                    asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0"
+                                 : "+a"(acc[a][b])
+                                 : "v"(par ? wo[a] : we[a]), "v"(fx[step & 1][b]));
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        __syncthreads();
+    };
+
+    using PF0 = std::integral_constant<int, 0>;
+    using PF1 = std::integral_constant<int, 1>;
+    using PF2 = std::integral_constant<int, 2>;
+    const bool ragged = nchunks != nfull;
+    // prologue: chunk 0 into registers / LDS
+    if (nfull > 0) {
+        load_w(PF1{}, 0, 0);
+        load_w(PF1{}, 1, 0);
+        load_x(PF1{}, 0);
+    } else {
+        load_w(PF2{}, 0, 0);
+        load_w(PF2{}, 1, 0);
+        load_x(PF2{}, 0);
+    }
+    store_x(0);
+    __syncthreads();
+    uint32_t c = 0;
+    for (; c + 1 < nfull; ++c) body(PF1{}, c);       // next chunk is a full one
+    if (c + 1 < nchunks) {                           // next (last) chunk is ragged
+        body(PF2{}, c);
+        ++c;
+    }
+    if (c < nchunks) body(PF0{}, c);                 // last chunk: nothing to fetch
+    (void)ragged;
+    // the MFMAs above are opaque to the compiler's hazard tracking: let the last ones retire
+    // before the accumulators are read
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+
+    const bool vec_ok = (EPI < 0) ? (p.N % 4 == 0 && reinterpret_cast<uintptr_t>(p.C) % 16 == 0)
+                                  : (p.N % 4 == 0 && reinterpret_cast<uintptr_t>(p.y) % 8 == 0);
+#pragma unroll
+    for (int b = 0; b < TM; ++b)
+#pragma unroll
+        for (int a = 0; a < TN; ++a) {
+            v4i v = acc[a][b];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) v[r] >>= 8;
+            store_quad<EPI, BIAS>(p, m0 + b * 16 + l16, n0 + wave * WN + a * 16 + g * 4, v, vec_ok);
+        }
+}
+
+// ---------------------------------------------------------------------------------
 // skinny kernel (M <= 16)
 // ---------------------------------------------------------------------------------
 // Workgroup = WAVES wavefronts, 16 output columns.  Wavefront w owns the k range
@@ -324,7 +528,13 @@ static void launch_epi(GemmParams &p, hipStream_t stream)
     // largest tile that still yields at least one workgroup per CU (256 CUs); small
     // problems take the small tile to spread over the chip.
     auto tiles = [&](uint32_t bm, uint32_t bn) { return ((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn); };
-    if (tiles(128, 256) >= 256 && p.M > 64) {
+    static const int variant = getenv("DUQ_GEMM_VARIANT") ? atoi(getenv("DUQ_GEMM_VARIANT")) : 1;
+    if (variant == 1 && tiles(128, 256) >= 128 && p.M > 64) {
+        p.tiles_m = (p.M + 127) / 128;
+        p.tiles_n = (p.N + 255) / 256;
+        hipLaunchKernelGGL((gemm_s4_stream_kernel<8, 4, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0,
+                           stream, p);
+    } else if (tiles(128, 256) >= 256 && p.M > 64) {
         p.tiles_m = (p.M + 127) / 128;
         p.tiles_n = (p.N + 255) / 256;
         hipLaunchKernelGGL((gemm_s4_tile_kernel<128, 256, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0,
