@@ -55,4 +55,57 @@ __device__ __forceinline__ uint16_t dequant_one(int acc, f16 s_row, f16 z_row, c
     return f16_to_bits(y);
 }
 
+// Column parameters of four consecutive output columns n0 .. n0+3, fetched with 64-bit
+// loads when the arrays allow it (`vec`: 8-byte aligned bases and n0 + 3 < cols).
+template <int MODE, bool BIAS>
+struct QuadCols {
+    ColParams c[4];
+};
+
+__device__ __forceinline__ void load4_f16(const uint16_t *ptr, uint32_t n0, uint32_t cols, bool vec, uint16_t (&out)[4])
+{
+    if (vec && n0 + 3 < cols) {
+        const v2u v = *reinterpret_cast<const v2u *>(ptr + n0);
+        out[0] = (uint16_t)(v[0] & 0xFFFFu);
+        out[1] = (uint16_t)(v[0] >> 16);
+        out[2] = (uint16_t)(v[1] & 0xFFFFu);
+        out[3] = (uint16_t)(v[1] >> 16);
+    } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) out[r] = ptr[min(n0 + r, cols - 1)];
+    }
+}
+
+template <int MODE, bool BIAS>
+__device__ __forceinline__ QuadCols<MODE, BIAS> load_quad_cols(const uint16_t *s1, const uint16_t *z1,
+                                                               const uint16_t *s2, const uint16_t *z2,
+                                                               const uint16_t *bias, uint32_t n0, uint32_t cols,
+                                                               bool vec)
+{
+    QuadCols<MODE, BIAS> q;
+    uint16_t a[4], b[4];
+    load4_f16(s1, n0, cols, vec, a);
+    if (MODE == 2 || MODE == 3) load4_f16(s2, n0, cols, vec, b);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const uint32_t col = n0 + r;
+        const bool first = MODE == 2 ? col < (uint32_t)kQuantColK : col == 0;  // see load_col
+        q.c[r].s = bits_to_f16((MODE == 2 || MODE == 3) ? (first ? a[r] : b[r]) : a[r]);
+        q.c[r].z = (f16)0;
+        q.c[r].bias = (f16)0;
+    }
+    if (MODE == 1 || MODE == 3) {
+        load4_f16(z1, n0, cols, vec, a);
+        if (MODE == 3) load4_f16(z2, n0, cols, vec, b);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) q.c[r].z = bits_to_f16(MODE == 3 ? ((n0 + r) == 0 ? a[r] : b[r]) : a[r]);
+    }
+    if (BIAS) {
+        load4_f16(bias, n0, cols, vec, a);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) q.c[r].bias = bits_to_f16(a[r]);
+    }
+    return q;
+}
+
 }  // namespace duq

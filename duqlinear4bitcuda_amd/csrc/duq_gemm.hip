@@ -238,24 +238,40 @@ __global__ __launch_bounds__(256) void gemm_s4_tile_kernel(GemmParams p)
 }
 
 // ---------------------------------------------------------------------------------
-// stream kernel (prefill): weights global -> registers, activations through LDS
+// stream kernel (prefill): weights global -> registers, activations through LDS,
+// v_mfma_i32_32x32x32_i8
 // ---------------------------------------------------------------------------------
-// Workgroup = 4 wavefronts side by side along N: every wavefront owns 16*TN weight rows
-// that no other wavefront of the workgroup needs, so weight fragments never go through
-// LDS: lane (l16, g) loads bytes [g*32, g*32+32) of the 128-byte row segment of a 256-k
-// chunk straight into registers (two 128-bit loads = one full cache line per row and
-// chunk), one chunk ahead of the MFMAs that consume them.  The 16*TM activation rows are
-// shared by the four wavefronts: they are expanded to bytes once on the way into LDS
-// (double buffered, rows padded to 272 B) and read back as 128-bit fragments.
-// LDS traffic per 256-k chunk drops to BM*256 B written + 4*BM*256 B read.
+// Tile 128 (M) x 256 (N), 4 wavefronts side by side along N: every wavefront owns 64 weight
+// rows that no other wavefront of the workgroup needs, so weight fragments never go through
+// LDS: lane (l32, h) loads 16-byte piece i (0..3) = bytes [i*32 + h*16, +16) of the 128-byte
+// row segment of a 256-k chunk straight into registers.  The 128 activation rows are shared
+// by the four wavefronts: they are expanded to bytes once on the way into LDS (three
+// buffers, rows padded to 272 B) and read back as 128-bit fragments.  LDS traffic per chunk
+// is 32 KB written + 128 KB read.
+//
+// The 32x32x32 MFMA keeps the matrix pipe full from a single wavefront per SIMD (32 cycles
+// per instruction, 16 per 32768 operations); the 16x16x64 form needs 18 and loses more to
+// interleaved vector work.  A chunk is 8 k-steps (piece i, nibble parity) of 8 MFMAs (2
+// weight tiles x 4 activation tiles).  The order is fixed by hand, a scheduling fence after
+// every MFMA, and everything else rides in the MFMA shadows, a few instructions per slot:
+//   every step    : the next step's four activation fragments (step 7: the next chunk's);
+//   step 2i       : refetch weight piece i for the next chunk (its registers were just
+//                   expanded), expand piece i+1 of weight tile 0;  step 2i+1: of tile 1;
+//   step 1        : fetch the activations two chunks ahead;
+//   steps 4..7    : expand + store those activations into the third LDS buffer;
+//   steps 6, 7    : expand the next chunk's weight piece 0.
+// MFMAs are issued through inline assembly with the accumulators tied to the accumulation
+// register file, so they never move.
 //
 // All global reads are raw buffer loads on per-workgroup descriptors that cover exactly
 // the rows of this tile: rows past M or N read as zero without a branch, and the chunk
-// offset rides in the scalar offset.  Only a ragged last chunk (K % 256 != 0) uses
-// per-piece guarded offsets.
+// offset rides in the scalar offset.  The last chunks use per-piece guarded offsets (a
+// piece at or past the row end is redirected out of bounds and reads as zero).
 constexpr int kCK = 256;         // k elements per chunk (128 packed bytes per row)
 constexpr int kXStride = 272;    // LDS bytes per activation row: 256 expanded + 16 pad
 constexpr uint32_t kOobOffset = 0xFFFFFF00u;  // beyond any descriptor: the load returns 0
+
+typedef int v16i __attribute__((ext_vector_type(16)));
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, uint32_t bytes)
 {
@@ -266,23 +282,22 @@ __device__ __forceinline__ v4u buf_load16(__amdgpu_buffer_rsrc_t r, uint32_t vof
     return __builtin_bit_cast(v4u, __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)soff, 0));
 }
 
-template <int TM, int TN, int EPI, bool BIAS>
+template <int EPI, bool BIAS>
 __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
 {
-    constexpr int BM = 16 * TM;
-    constexpr int WN = 16 * TN;
-    constexpr int BN = 4 * WN;
-    constexpr int NXP = BM / 32;  // 16-byte activation pieces per thread and chunk
-    static_assert(BM % 32 == 0, "BM");
+    constexpr int BM = 128, BN = 256;
+    constexpr int TM = 4, TN = 2;      // 32x32 tiles per wavefront: 128 x 64
+    constexpr int NXP = 4;             // 16-byte activation pieces per thread and chunk
+    constexpr uint32_t kBuf = BM * kXStride;
 
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2][BM * kXStride];
+    __shared__ __attribute__((aligned(16))) uint8_t lds[3 * kBuf];
 
     uint32_t tile_m, tile_n;
     tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63u, wave = tid >> 6;
-    const uint32_t l16 = lane & 15u, g = lane >> 4;
+    const uint32_t l32 = lane & 31u, h = lane >> 5;
     const uint32_t kbytes = p.K >> 1;
     const uint32_t nfull = p.K / kCK;
     const uint32_t nchunks = (p.K + kCK - 1) / kCK;
@@ -292,7 +307,7 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
 
     uint32_t woff[TN];
 #pragma unroll
-    for (int a = 0; a < TN; ++a) woff[a] = (wave * WN + a * 16 + l16) * kbytes + g * 32;
+    for (int t = 0; t < TN; ++t) woff[t] = (wave * 64 + t * 32 + l32) * kbytes + h * 16;
     uint32_t xoff[NXP], xlds[NXP];
     const uint32_t xq = tid & 7u;  // which 16-byte piece of the 128-byte row segment
 #pragma unroll
@@ -302,141 +317,204 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
         xlds[i] = row * kXStride + xq * 32;
     }
 
-    v4u wreg[TN][2];
-    v4u xreg[NXP];
+    v4u wreg[TN][4];      // raw weight pieces [tile][piece]
+    v4u xreg[NXP];        // raw activation pieces
+    v4u wexp[2][2][TN];   // expanded weights [piece & 1][parity][tile]
+    v4i fx[2][TM];        // activation fragments [step & 1][tile]
+    v16i acc[TN][TM];
+#pragma unroll
+    for (int t = 0; t < TN; ++t)
+#pragma unroll
+        for (int b = 0; b < TM; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[t][b][r] = 0;
 
-    // PF selects how the NEXT chunk is fetched: 0 none, 1 full chunk (no guards), 2 ragged
-    // last chunk (pieces past the row end are redirected out of bounds and read as zero).
-    auto load_w = [&](auto pf, int j, uint32_t c) {
-        constexpr int PF = decltype(pf)::value;
-        const uint32_t koff = c * (kCK / 2);
-        if (PF == 1) {
-#pragma unroll
-            for (int a = 0; a < TN; ++a) wreg[a][j] = buf_load16(rW, woff[a] + j * 16, koff);
-        } else if (PF == 2) {
-            const bool ok = koff + g * 32 + j * 16 < kbytes;  // K % 64 == 0: all in or all out
-#pragma unroll
-            for (int a = 0; a < TN; ++a) wreg[a][j] = buf_load16(rW, ok ? woff[a] + j * 16 : kOobOffset, koff);
-        }
-    };
-    auto load_x = [&](auto pf, uint32_t c) {
-        constexpr int PF = decltype(pf)::value;
-        const uint32_t koff = c * (kCK / 2);
-        if (PF == 1) {
-#pragma unroll
-            for (int i = 0; i < NXP; ++i) xreg[i] = buf_load16(rX, xoff[i], koff);
-        } else if (PF == 2) {
-            const bool okx = koff + xq * 16 < kbytes;
-#pragma unroll
-            for (int i = 0; i < NXP; ++i) xreg[i] = buf_load16(rX, okx ? xoff[i] : kOobOffset, koff);
-        }
-    };
-    auto store_x = [&](uint32_t buf) {
-        uint8_t *base = lds[buf];
-#pragma unroll
-        for (int i = 0; i < NXP; ++i) {
-            v4u ev, od;
-            expand_nibbles(xreg[i], ev, od);
-            *reinterpret_cast<v4u *>(base + xlds[i]) = ev;
-            *reinterpret_cast<v4u *>(base + xlds[i] + 16) = od;
-        }
+    // fragment of step (i, par) for activation tile b: + b*32*kXStride + i*64 + par*16
+    const uint32_t fragX = l32 * kXStride + h * 32;
+
+    auto expand_word = [&](const v4u &raw, v4u &even, v4u &odd, int w) {
+        even[w] = (raw[w] << 4) & kNibbleMask;
+        odd[w] = raw[w] & kNibbleMask;
     };
 
-    v4i acc[TN][TM];
+    // GUARD = false: every chunk fetched is complete, plain offsets.
+    auto body = [&](auto guard, uint32_t c, uint32_t cur, uint32_t nxt, uint32_t nx2) {
+        constexpr bool G = decltype(guard)::value;
+        const uint32_t koff1 = (c + 1) * (kCK / 2), koff2 = (c + 2) * (kCK / 2);
+        const bool okx = !G || (koff2 + xq * 16 < kbytes);  // K % 64 == 0: a piece is all in or all out
+        v4u xe, xo;
 #pragma unroll
-    for (int a = 0; a < TN; ++a)
+        for (int step = 0; step < 8; ++step) {
+            const int i = step >> 1, par = step & 1;
+            const bool okw = !G || (koff1 + i * 32 + h * 16 < kbytes);
 #pragma unroll
-        for (int b = 0; b < TM; ++b) acc[a][b] = v4i{0, 0, 0, 0};
-
-    const uint32_t fragX = l16 * kXStride + g * 64;  // fragment step*16 with step = j*2+par
-
-    // One chunk = 4 MFMA steps (j, par), each TM groups of TN MFMAs.  The instruction order
-    // is fixed by hand (scheduling fences around every MFMA group): while the TN MFMAs of a
-    // group run, the next step's activation fragment for the same group index is read from
-    // LDS, the weight registers of half j are refilled for the next chunk right after they
-    // were expanded, and the next chunk's activations are expanded and written to the other
-    // LDS buffer inside the last step.  MFMAs are issued through inline assembly with the
-    // accumulators tied to the accumulation register file, so they never move.
-    auto body = [&](auto pf, uint32_t c) {
-        constexpr int PF = decltype(pf)::value;
-        const uint32_t cur = c & 1u;
-        const uint8_t *base = lds[cur] + fragX;
-        uint8_t *nbase = lds[cur ^ 1u];
-        load_x(pf, c + 1);
-        v4i fx[2][TM];
-#pragma unroll
-        for (int b = 0; b < TM; ++b) fx[0][b] = *reinterpret_cast<const v4i *>(base + b * 16 * kXStride);
-        v4u we[TN], wo[TN];
-#pragma unroll
-        for (int step = 0; step < 4; ++step) {
-            const int j = step >> 1, par = step & 1;
-            if (par == 0) {
-#pragma unroll
-                for (int a = 0; a < TN; ++a) expand_nibbles(wreg[a][j], we[a], wo[a]);
-                load_w(pf, j, c + 1);
-            }
-#pragma unroll
-            for (int b = 0; b < TM; ++b) {
-                if (step < 3)
-                    fx[(step + 1) & 1][b] =
-                        *reinterpret_cast<const v4i *>(base + b * 16 * kXStride + (step + 1) * 16);
-                if (PF != 0 && step == 3 && b < NXP) {  // next chunk's activations -> LDS
-                    v4u ev, od;
-                    expand_nibbles(xreg[b], ev, od);
-                    *reinterpret_cast<v4u *>(nbase + xlds[b]) = ev;
-                    *reinterpret_cast<v4u *>(nbase + xlds[b] + 16) = od;
-                }
+            for (int slot = 0; slot < 8; ++slot) {
+                const int b = slot >> 1, t = slot & 1;
+                asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0"
+                             : "+a"(acc[t][b])
+                             : "v"(wexp[i & 1][par][t]), "v"(fx[step & 1][b]));
                 __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int a = 0; a < TN; ++a)
-                    asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0"
-                                 : "+a"(acc[a][b])
-                                 : "v"(par ? wo[a] : we[a]), "v"(fx[step & 1][b]));
+                // ---- side work in the shadow of this MFMA
+                if (slot < 4) {  // next step's activation fragment for tile `slot`
+                    const uint8_t *src = step < 7 ? lds + cur + fragX + ((step + 1) >> 1) * 64 + ((step + 1) & 1) * 16
+                                                  : lds + nxt + fragX;
+                    fx[(step + 1) & 1][slot] = *reinterpret_cast<const v4i *>(src + slot * 32 * kXStride);
+                }
+                if (par == 0 && slot < TN)  // piece i was expanded earlier: refetch it for the next chunk
+                    wreg[slot][i] = buf_load16(rW, okw ? woff[slot] + i * 32 : kOobOffset, koff1);
+                if (step == 1 && slot < NXP)  // activations two chunks ahead
+                    xreg[slot] = buf_load16(rX, okx ? xoff[slot] : kOobOffset, koff2);
+                if (slot >= 4) {  // expand the next weight piece of tile `par`, one word per slot
+                    const int np = (i + 1) & 3;  // pieces 1, 2, 3 of this chunk, then piece 0 of the next
+                    expand_word(wreg[par][np], wexp[(i + 1) & 1][0][par], wexp[(i + 1) & 1][1][par], slot - 4);
+                }
+                if (step >= 4 && slot < 4) {  // activations two chunks ahead -> third LDS buffer
+                    expand_word(xreg[step - 4], xe, xo, slot);
+                    if (slot == 3) {
+                        *reinterpret_cast<v4u *>(lds + nx2 + xlds[step - 4]) = xe;
+                        *reinterpret_cast<v4u *>(lds + nx2 + xlds[step - 4] + 16) = xo;
+                    }
+                }
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
         __syncthreads();
     };
 
-    using PF0 = std::integral_constant<int, 0>;
-    using PF1 = std::integral_constant<int, 1>;
-    using PF2 = std::integral_constant<int, 2>;
-    const bool ragged = nchunks != nfull;
-    // prologue: chunk 0 into registers / LDS
-    if (nfull > 0) {
-        load_w(PF1{}, 0, 0);
-        load_w(PF1{}, 1, 0);
-        load_x(PF1{}, 0);
-    } else {
-        load_w(PF2{}, 0, 0);
-        load_w(PF2{}, 1, 0);
-        load_x(PF2{}, 0);
+    using Plain = std::false_type;
+    using Guarded = std::true_type;
+
+    // ---- prologue: chunks 0 and 1 activations -> LDS, chunk 0 weights -> registers
+    {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const bool okw = i * 32 + h * 16 < kbytes;
+#pragma unroll
+            for (int t = 0; t < TN; ++t) wreg[t][i] = buf_load16(rW, okw ? woff[t] + i * 32 : kOobOffset, 0);
+        }
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const bool okx = q * (kCK / 2) + xq * 16 < kbytes;
+#pragma unroll
+            for (int i = 0; i < NXP; ++i) xreg[i] = buf_load16(rX, okx ? xoff[i] : kOobOffset, q * (kCK / 2));
+#pragma unroll
+            for (int i = 0; i < NXP; ++i) {
+                v4u ev, od;
+                expand_nibbles(xreg[i], ev, od);
+                *reinterpret_cast<v4u *>(lds + q * kBuf + xlds[i]) = ev;
+                *reinterpret_cast<v4u *>(lds + q * kBuf + xlds[i] + 16) = od;
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < TN; ++t) expand_nibbles(wreg[t][0], wexp[0][0][t], wexp[0][1][t]);
+        __syncthreads();
+#pragma unroll
+        for (int b = 0; b < TM; ++b) fx[0][b] = *reinterpret_cast<const v4i *>(lds + fragX + b * 32 * kXStride);
     }
-    store_x(0);
-    __syncthreads();
+
+    uint32_t cur = 0, nxt = kBuf, nx2 = 2 * kBuf;
+    auto rotate = [&]() {
+        const uint32_t t = cur;
+        cur = nxt;
+        nxt = nx2;
+        nx2 = t;
+    };
     uint32_t c = 0;
-    for (; c + 1 < nfull; ++c) body(PF1{}, c);       // next chunk is a full one
-    if (c + 1 < nchunks) {                           // next (last) chunk is ragged
-        body(PF2{}, c);
-        ++c;
+    for (; c + 2 < nfull; ++c) {  // steady state: chunks c+1 and c+2 are complete ones
+        body(Plain{}, c, cur, nxt, nx2);
+        rotate();
     }
-    if (c < nchunks) body(PF0{}, c);                 // last chunk: nothing to fetch
-    (void)ragged;
+    for (; c < nchunks; ++c) {  // last chunks: guarded fetches (a fetch past K reads zeros, unused)
+        body(Guarded{}, c, cur, nxt, nx2);
+        rotate();
+    }
     // the MFMAs above are opaque to the compiler's hazard tracking: let the last ones retire
     // before the accumulators are read
-    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 
-    const bool vec_ok = (EPI < 0) ? (p.N % 4 == 0 && reinterpret_cast<uintptr_t>(p.C) % 16 == 0)
-                                  : (p.N % 4 == 0 && reinterpret_cast<uintptr_t>(p.y) % 8 == 0);
+    // lane holds, for activation row m = l32 of tile b and weight tile t: registers r = 4*q..4*q+3
+    // are the four consecutive output columns n = 8*q + 4*h + (0..3), q = 0..3
+    if (EPI < 0) {
+        const bool vec_ok = p.N % 4 == 0 && reinterpret_cast<uintptr_t>(p.C) % 16 == 0;
 #pragma unroll
-    for (int b = 0; b < TM; ++b)
+        for (int b = 0; b < TM; ++b)
 #pragma unroll
-        for (int a = 0; a < TN; ++a) {
-            v4i v = acc[a][b];
+            for (int t = 0; t < TN; ++t)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) v[r] >>= 8;
-            store_quad<EPI, BIAS>(p, m0 + b * 16 + l16, n0 + wave * WN + a * 16 + g * 4, v, vec_ok);
+                for (int q = 0; q < 4; ++q) {
+                    v4i v;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) v[r] = acc[t][b][q * 4 + r] >> 8;
+                    store_quad<EPI, BIAS>(p, m0 + b * 32 + l32, n0 + wave * 64 + t * 32 + q * 8 + h * 4, v, vec_ok);
+                }
+    } else {
+        constexpr int MODE = EPI < 0 ? 0 : EPI;
+        const Epilogue &e = p.epi;
+        const bool vec_st = p.N % 4 == 0 && reinterpret_cast<uintptr_t>(p.y) % 8 == 0;
+        const bool vec_ld = p.N % 4 == 0 && reinterpret_cast<uintptr_t>(e.s_col_1) % 8 == 0 &&
+                            (MODE == 0 || MODE == 2 || reinterpret_cast<uintptr_t>(e.z_col_1) % 8 == 0) &&
+                            (MODE < 2 || reinterpret_cast<uintptr_t>(e.s_col_2) % 8 == 0) &&
+                            (MODE != 3 || reinterpret_cast<uintptr_t>(e.z_col_2) % 8 == 0) &&
+                            (!BIAS || reinterpret_cast<uintptr_t>(e.bias) % 8 == 0);
+        f16 s_row[TM], z_row[TM];
+#pragma unroll
+        for (int b = 0; b < TM; ++b) {
+            const uint32_t m = min(m0 + b * 32 + l32, p.M - 1);
+            s_row[b] = bits_to_f16(e.s_row[m]);
+            z_row[b] = (MODE == 1 || MODE == 3) ? bits_to_f16(e.z_row[m]) : (f16)0;
         }
+        // When rows of y are 16-byte aligned, the 128 x 64 fp16 tile of this wavefront goes
+        // through LDS (free now) so that the global stores are whole 128-byte lines: the MFMA
+        // layout itself only offers 16 contiguous bytes per row and store instruction.
+        constexpr uint32_t kYStride = 144;  // bytes per staged row: 128 + pad
+        const bool staged = p.N % 8 == 0 && reinterpret_cast<uintptr_t>(p.y) % 16 == 0;
+        uint8_t *stage = lds + wave * (BM * kYStride);
+        if (staged) __syncthreads();  // every wavefront is done reading the activation buffers
+#pragma unroll
+        for (int t = 0; t < TN; ++t)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t ncol = t * 32 + q * 8 + h * 4;  // column inside the wavefront's tile
+                const uint32_t nq = n0 + wave * 64 + ncol;
+                if (!staged && nq >= p.N) continue;
+                const QuadCols<MODE, BIAS> cols = load_quad_cols<MODE, BIAS>(e.s_col_1, e.z_col_1, e.s_col_2, e.z_col_2,
+                                                                             e.bias, min(nq, p.N - 1), p.N, vec_ld);
+#pragma unroll
+                for (int b = 0; b < TM; ++b) {
+                    const uint32_t m = m0 + b * 32 + l32;
+                    uint16_t out[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        out[r] = dequant_one<MODE, BIAS>(acc[t][b][q * 4 + r] >> 8, s_row[b], z_row[b], cols.c[r]);
+                    const v2u packed = v2u{(uint32_t)out[0] | ((uint32_t)out[1] << 16),
+                                           (uint32_t)out[2] | ((uint32_t)out[3] << 16)};
+                    if (staged) {
+                        *reinterpret_cast<v2u *>(stage + (b * 32 + l32) * kYStride + ncol * 2) = packed;
+                    } else if (m < p.M) {
+                        uint16_t *dst = p.y + (uint64_t)m * p.N + nq;
+                        if (vec_st && nq + 3 < p.N) {
+                            *reinterpret_cast<v2u *>(dst) = packed;
+                        } else {
+#pragma unroll
+                            for (int r = 0; r < 4; ++r)
+                                if (nq + r < p.N) dst[r] = out[r];
+                        }
+                    }
+                }
+            }
+        if (staged) {
+            // same wavefront wrote and reads its stage: LDS operations complete in order
+            const uint32_t piece = lane & 7u, rsub = lane >> 3;
+            const uint32_t ncol0 = n0 + wave * 64 + piece * 8;
+#pragma unroll
+            for (int it = 0; it < BM / 8; ++it) {
+                const uint32_t row = it * 8 + rsub;
+                const v4u v = *reinterpret_cast<const v4u *>(stage + row * kYStride + piece * 16);
+                if (m0 + row < p.M && ncol0 < p.N)
+                    *reinterpret_cast<v4u *>(p.y + (uint64_t)(m0 + row) * p.N + ncol0) = v;
+            }
+        }
+    }
 }
 
 // ---------------------------------------------------------------------------------
@@ -532,8 +610,7 @@ static void launch_epi(GemmParams &p, hipStream_t stream)
     if (variant == 1 && tiles(128, 256) >= 128 && p.M > 64) {
         p.tiles_m = (p.M + 127) / 128;
         p.tiles_n = (p.N + 255) / 256;
-        hipLaunchKernelGGL((gemm_s4_stream_kernel<8, 4, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0,
-                           stream, p);
+        hipLaunchKernelGGL((gemm_s4_stream_kernel<EPI, BIAS>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, stream, p);
     } else if (tiles(128, 256) >= 256 && p.M > 64) {
         p.tiles_m = (p.M + 127) / 128;
         p.tiles_n = (p.N + 255) / 256;
