@@ -1,0 +1,61 @@
+"""Writes tests/golden/linear4bit_small.npz: seeded inputs and the expected packed codes,
+scales, int32 accumulators and fp16 outputs of the four Linear4bit forwards.
+
+The reference ships no golden vectors for this path (its tests only print), so these come
+from the pinned CPU oracle; the file freezes them so that a later change of the oracle or
+of a kernel shows up as a diff against data, not against code.
+
+    python tests/golden/make_golden.py
+"""
+import os
+import sys
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, ROOT)
+from oracle import duq_oracle as orc  # noqa: E402
+
+
+def main():
+    g = torch.Generator().manual_seed(20240)
+    M, K, N = 24, 256, 48
+    out = {}
+    # symmetric: N(0,1) activations with two x20 outlier channels, one all-zero token
+    x = torch.randn(M, K, generator=g)
+    x[:, [5, 77]] *= 20
+    x[3] = 0
+    x = x.half().numpy()
+    w = (torch.randn(N, K, generator=g) * 0.02).half().numpy()
+    s_w = orc.sym_scales(w)
+    wq = orc.weight_sym_from_float(w, s_w)
+    bias = torch.randn(N, generator=g).half().numpy()
+    out.update(sym_x=x, sym_w=wq, sym_sw=s_w, bias=bias)
+    for qmax in (6, 7):
+        y, acc, qx, sx = orc.linear4bit_sq_forward(x, wq, s_w, bias, qmax=qmax)
+        out.update({f"sym_q{qmax}_y": y, f"sym_q{qmax}_acc": acc, f"sym_q{qmax}_qx": qx, f"sym_q{qmax}_sx": sx})
+    s_w2 = (s_w.astype(np.float32) * 1.5).astype(np.float16)
+    y, acc, qx, sx = orc.linear4bit_dusq_forward(x, wq, s_w, s_w2, bias)
+    out.update(dusq_sw2=s_w2, dusq_y=y)
+    # asymmetric: U[0,6) activations plus one signed and one constant token
+    xa = (torch.rand(M, K, generator=g) * 6)
+    xa[1] = torch.randn(K, generator=g)
+    xa[2] = 1.5
+    xa = xa.half().numpy()
+    wa, sa, za = orc.weight_asym_from_linear(w)
+    y, acc, qx, sx, zx = orc.linear4bit_asq_forward(xa, wa, sa, za, bias)
+    out.update(asym_x=xa, asym_w=wa, asym_sw=sa, asym_zw=za, asym_y=y, asym_acc=acc, asym_qx=qx, asym_sx=sx, asym_zx=zx)
+    wa1, sa1, za1 = orc.weight_asym_from_linear(w[:, :10])
+    wa2, sa2, za2 = orc.weight_asym_from_linear(w[:, 10:])
+    codes = np.concatenate([orc.unpack_i4(wa1, signed=False), orc.unpack_i4(wa2, signed=False)], axis=1)
+    wd = orc.pack_i4(codes, sym=False)
+    y, *_ = orc.linear4bit_duasq_forward(xa, wd, sa1, za1, sa2, za2, bias)
+    out.update(duasq_w=wd, duasq_s1=sa1, duasq_z1=za1, duasq_s2=sa2, duasq_z2=za2, duasq_y=y)
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "linear4bit_small.npz")
+    np.savez_compressed(path, **out)
+    print(path, os.path.getsize(path), "bytes")
+
+
+if __name__ == "__main__":
+    main()

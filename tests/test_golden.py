@@ -1,0 +1,79 @@
+"""The committed fixture tests/golden/linear4bit_small.npz against the oracle (CPU) and
+against the HIP path through the module interface (GPU)."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import duq_oracle as orc
+from tests import cases
+
+G = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "linear4bit_small.npz"))
+
+
+def same16(a, b):
+    a = np.asarray(a, np.float16)
+    b = np.asarray(b, np.float16)
+    return bool(((a.view(np.uint16) == b.view(np.uint16)) | (np.isnan(a) & np.isnan(b))).all())
+
+
+def test_oracle_reproduces_the_fixture():
+    for qmax in (6, 7):
+        y, acc, qx, sx = orc.linear4bit_sq_forward(G["sym_x"], G["sym_w"], G["sym_sw"], G["bias"], qmax=qmax)
+        assert np.array_equal(qx, G[f"sym_q{qmax}_qx"]) and np.array_equal(acc, G[f"sym_q{qmax}_acc"])
+        assert same16(sx, G[f"sym_q{qmax}_sx"]) and same16(y, G[f"sym_q{qmax}_y"])
+    y, *_ = orc.linear4bit_dusq_forward(G["sym_x"], G["sym_w"], G["sym_sw"], G["dusq_sw2"], G["bias"])
+    assert same16(y, G["dusq_y"])
+    y, acc, qx, sx, zx = orc.linear4bit_asq_forward(G["asym_x"], G["asym_w"], G["asym_sw"], G["asym_zw"], G["bias"])
+    assert np.array_equal(qx, G["asym_qx"]) and np.array_equal(acc, G["asym_acc"])
+    assert same16(sx, G["asym_sx"]) and same16(zx, G["asym_zx"]) and same16(y, G["asym_y"])
+    y, *_ = orc.linear4bit_duasq_forward(G["asym_x"], G["duasq_w"], G["duasq_s1"], G["duasq_z1"], G["duasq_s2"],
+                                        G["duasq_z2"], G["bias"])
+    assert same16(y, G["duasq_y"])
+
+
+def test_fixture_sanity():
+    # accumulators of the fixture equal the plain integer product of its own codes
+    a = orc.unpack_i4(G["sym_q6_qx"]).astype(np.int64)
+    b = orc.unpack_i4(G["sym_w"]).astype(np.int64)
+    assert np.array_equal(a @ b.T, G["sym_q6_acc"])
+    assert (G["sym_q6_qx"][3] == 0).all() and float(G["sym_q6_sx"][3, 0]) == 0.0   # the all-zero token
+    assert orc.unpack_i4(G["sym_q6_qx"]).max() == 6 and orc.unpack_i4(G["sym_q7_qx"]).max() == 7
+
+
+@pytest.mark.gpu
+def test_modules_reproduce_the_fixture(dev):
+    from duqlinear4bitcuda_amd import nn as qnn
+
+    T = lambda k: cases.t(G[k], dev)
+    K, N = G["sym_x"].shape[1], G["sym_w"].shape[0]
+    for qmax in (6, 7):
+        lin = qnn.Linear4bitSQ(K, N, bias=True).half().to(dev)
+        lin.load_state_dict({"weight": T("sym_w"), "weight_scales": T("sym_sw"), "bias": T("bias")})
+        p = qnn.SymQuantizer(1.0, qmax=qmax)(T("sym_x"))
+        assert np.array_equal(p.quantized_x.cpu().numpy(), G[f"sym_q{qmax}_qx"])
+        assert same16(p.scales_x.cpu().numpy(), G[f"sym_q{qmax}_sx"])
+        for fused in (True, False):
+            lin.fused = fused
+            assert same16(lin(p).cpu().numpy(), G[f"sym_q{qmax}_y"])
+    du = qnn.Linear4bitDUSQ(K, N, bias=True).half().to(dev)
+    du.load_state_dict({"weight": T("sym_w"), "weight_scales_1": T("sym_sw"), "weight_scales_2": T("dusq_sw2"), "bias": T("bias")})
+    p = qnn.SymQuantizer(1.0)(T("sym_x"))
+    for fused in (True, False):
+        du.fused = fused
+        assert same16(du(p).cpu().numpy(), G["dusq_y"])
+    a = qnn.Linear4bitASQ(K, N, bias=True).to(dev)
+    a.load_state_dict({"weight": T("asym_w"), "weight_scales": T("asym_sw"), "weight_zeros": T("asym_zw"), "bias": T("bias")})
+    for fused in (True, False):
+        a.fused = fused
+        assert same16(a(T("asym_x")).cpu().numpy(), G["asym_y"])
+    p = a.quantizer(T("asym_x"))
+    assert np.array_equal(p.quantized_x.cpu().numpy(), G["asym_qx"])
+    assert same16(p.scales_x.cpu().numpy(), G["asym_sx"]) and same16(p.zeros_x.cpu().numpy(), G["asym_zx"])
+    d = qnn.LinearQuant4bitDUASQ(K, N, bias=True).to(dev)
+    d.load_state_dict({"weight": T("duasq_w"), "weight_scales_1": T("duasq_s1"), "weight_zeros_1": T("duasq_z1"),
+                       "weight_scales_2": T("duasq_s2"), "weight_zeros_2": T("duasq_z2"), "bias": T("bias")})
+    for fused in (True, False):
+        d.fused = fused
+        assert same16(d(T("asym_x")).cpu().numpy(), G["duasq_y"])

@@ -1,0 +1,254 @@
+"""GPU tests of the module layer and of the benchmark configurations: module forward ==
+oracle composition, leading dimensions, error paths, and size-independent properties at
+the full benchmark sizes where the oracle would be too slow."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import duq_oracle as orc
+from oracle import duq_oracle_c as orc_c
+from tests import cases
+
+pytestmark = pytest.mark.gpu
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+@pytest.fixture(scope="module")
+def qnn(dev):
+    from duqlinear4bitcuda_amd import nn
+
+    return nn
+
+
+def _sq_module(qnn, dev, wq, sw, bias=None):
+    N, K = wq.shape[0], wq.shape[1] * 2
+    lin = qnn.Linear4bitSQ(K, N, bias=bias is not None).half().to(dev)
+    sd = {"weight": cases.t(wq, dev), "weight_scales": cases.t(sw, dev)}
+    if bias is not None:
+        sd["bias"] = cases.t(bias, dev)
+    lin.load_state_dict(sd)
+    return lin
+
+
+def test_config1_cpu_fakequant_parity(qnn, dev):
+    """Config 1: M16, K = N = 4096, N(0,1) activations with 0.5 % channels x20, W ~ N(0,0.02)
+    quantized per output channel; both clamp conventions; packed codes and accumulators
+    bit-exact, fp16 outputs equal."""
+    _say("config 1")
+    M, K, N = 16, 4096, 4096
+    x = cases.acts_outliers(M, K, seed=1)
+    wq, sw = cases.weights_from_float_sym(N, K, seed=11)
+    lin = _sq_module(qnn, dev, wq, sw)
+    from duqlinear4bitcuda_amd.tools import tensor_utils as tu
+
+    for qmax in (6, 7):
+        y_want, acc_want, q_want, s_want = orc.linear4bit_sq_forward(x, wq, sw, qmax=qmax)
+        p = qnn.SymQuantizer(1.0, qmax=qmax)(cases.t(x, dev))
+        assert np.array_equal(p.quantized_x.cpu().numpy(), q_want)
+        assert cases.bits_equal(p.scales_x.cpu().numpy(), s_want)
+        acc = tu.matmul(p.quantized_x, lin.weight)
+        assert np.array_equal(acc.cpu().numpy(), acc_want)
+        y = lin(p).cpu().numpy()
+        assert cases.bits_equal(y, y_want)
+        rel = np.abs(y.astype(np.float32) - y_want.astype(np.float32)) / np.maximum(np.abs(y_want.astype(np.float32)), 1e-3)
+        assert rel.max() <= 1e-3  # the stated bar; bit equality above is stronger
+
+
+@pytest.mark.parametrize("M,N", [(1, 4096), (4, 11008), (16, 4096)])
+def test_config2_decode(qnn, dev, M, N):
+    _say("config 2", M, N)
+    K = 4096
+    x = cases.acts_normal(M, K, seed=2)
+    wq, sw = cases.weights_random_nibbles(N, K, seed=22)
+    y_want, acc_want, q_want, s_want = orc.linear4bit_sq_forward(x, wq, sw)
+    lin = _sq_module(qnn, dev, wq, sw)
+    y = torch.nn.Sequential(qnn.SymQuantizer(1.0), lin)(cases.t(x, dev)).cpu().numpy()
+    assert cases.bits_equal(y, y_want)
+
+
+def test_config3_prefill_against_c_oracle(qnn, dev):
+    """Config 3 at full size for K = N = 4096 (the C oracle does the 34 G multiply-adds on
+    the host cores), heavy-tailed activations."""
+    _say("config 3 full")
+    M, K, N = 2048, 4096, 4096
+    x = cases.acts_heavy_tail(M, K, seed=3)
+    wq, sw = cases.weights_random_nibbles(N, K, seed=33)
+    s_want = orc.sym_scales(x)
+    q_want = orc.sym_quant(x, s_want)
+    lin = _sq_module(qnn, dev, wq, sw)
+    p = qnn.SymQuantizer(1.0)(cases.t(x, dev))
+    assert np.array_equal(p.quantized_x.cpu().numpy(), q_want)
+    assert cases.bits_equal(p.scales_x.cpu().numpy(), s_want)
+    from duqlinear4bitcuda_amd.tools import tensor_utils as tu
+
+    acc_want = orc_c.matmul_s4(q_want, wq)
+    acc = tu.matmul(p.quantized_x, lin.weight).cpu().numpy()
+    assert np.array_equal(acc, acc_want)
+    y = lin(p).cpu().numpy()
+    assert cases.bits_equal(y, orc.sym_dequant(acc_want, s_want, sw))
+
+
+@pytest.mark.parametrize("K,N", [(4096, 11008), (11008, 4096)])
+def test_config3_other_shapes_by_properties(qnn, dev, K, N):
+    """Full-size prefill shapes checked through properties that need no CPU GEMM:
+    (1) a sampled set of rows/columns against the oracle, (2) linearity in the weights:
+    acc(A, B1) + acc(A, B2) == acc(A, B1 + B2) when the nibble sums stay in range,
+    (3) the fused fp16 output equals the stand-alone dequant of the int32 output."""
+    _say("config 3 properties", K, N)
+    M = 2048
+    from duqlinear4bitcuda_amd import _HIP as hip
+
+    rng = np.random.default_rng(K + N)
+    x = cases.acts_heavy_tail(M, K, seed=3)
+    q, s = hip.quantize_rows_sym(cases.t(x, dev))
+    b1 = rng.integers(-4, 4, (N, K)).astype(np.int8)
+    b2 = rng.integers(-4, 4, (N, K)).astype(np.int8)
+    B1, B2, B12 = (cases.t(orc.pack_i4(b), dev) for b in (b1, b2, b1 + b2))
+    c1, c2, c12 = hip.matmul(q, B1), hip.matmul(q, B2), hip.matmul(q, B12)
+    assert torch.equal(c1 + c2, c12)
+    rows = rng.choice(M, 24, replace=False)
+    cols = rng.choice(N, 40, replace=False)
+    a_cpu = orc.unpack_i4(q.cpu().numpy()[rows]).astype(np.int64)
+    want = a_cpu @ b1[cols].astype(np.int64).T
+    assert np.array_equal(c1.cpu().numpy()[np.ix_(rows, cols)], want)
+    sw = cases.t(rng.uniform(0.001, 0.01, (N, 1)).astype(np.float16), dev)
+    y_fused = hip.linear4bit_forward(hip.EPI_SYM, q, s, None, B1, sw)
+    y_unfused = hip.sym_dequant(c1, s.view(-1), sw, 32)
+    assert torch.equal(y_fused.view(torch.int16), y_unfused.view(torch.int16))
+
+
+def test_config4_asym_dual_uniform(qnn, dev):
+    _say("config 4")
+    M, K, N = 512, 4096, 4096
+    x = cases.acts_uniform(M, K, seed=4)
+    wq, sw, zw = cases.weights_from_linear_asym(N, K, seed=44)
+    y_want, acc_want, q_want, s_want, z_want = orc.linear4bit_asq_forward(x, wq, sw, zw)
+    m = qnn.Linear4bitASQ(K, N).to(dev)
+    m.load_state_dict({"weight": cases.t(wq, dev), "weight_scales": cases.t(sw, dev), "weight_zeros": cases.t(zw, dev)})
+    p = m.quantizer(cases.t(x, dev))
+    assert np.array_equal(p.quantized_x.cpu().numpy(), q_want)
+    assert cases.bits_equal(p.scales_x.cpu().numpy(), s_want) and cases.bits_equal(p.zeros_x.cpu().numpy(), z_want)
+    from duqlinear4bitcuda_amd.tools import tensor_utils as tu
+
+    assert np.array_equal(tu.matmul(p.quantized_x, m.weight).cpu().numpy(), acc_want)
+    assert cases.bits_equal(m(cases.t(x, dev)).cpu().numpy(), y_want)
+    # the dual-uniform layer on the same input (from_linear on the device)
+    lin = torch.nn.Linear(K, N, bias=False).half()
+    with torch.no_grad():
+        lin.weight.copy_((torch.randn(N, K, generator=torch.Generator().manual_seed(45)) * 0.02).half())
+    du = qnn.LinearQuant4bitDUASQ.from_linear(lin).to(dev)
+    sd = {k: v.cpu().numpy() for k, v in du.state_dict().items()}
+    y_want, *_ = orc.linear4bit_duasq_forward(x, sd["weight"], sd["weight_scales_1"], sd["weight_zeros_1"],
+                                             sd["weight_scales_2"], sd["weight_zeros_2"])
+    assert cases.bits_equal(du(cases.t(x, dev)).cpu().numpy(), y_want)
+
+
+@pytest.mark.parametrize("M,K,N", [(1, 8192, 28672), (1, 28672, 8192)])
+def test_config5_decode_70b_shapes(qnn, dev, M, K, N):
+    _say("config 5 decode", K, N)
+    x = cases.acts_outliers(M, K, seed=5)
+    wq, sw = cases.weights_random_nibbles(N, K, seed=55)
+    y_want, *_ = orc.linear4bit_sq_forward(x, wq, sw)
+    lin = _sq_module(qnn, dev, wq, sw)
+    y = lin(qnn.SymQuantizer(1.0)(cases.t(x, dev))).cpu().numpy()
+    assert cases.bits_equal(y, y_want)
+
+
+def test_config5_prefill_70b_shape_by_properties(qnn, dev):
+    """M 4096, K 8192, N 28672 (1.9 T multiply-adds): sampled entries against the oracle and
+    fused == unfused."""
+    _say("config 5 prefill")
+    from duqlinear4bitcuda_amd import _HIP as hip
+
+    M, K, N = 4096, 8192, 28672
+    rng = np.random.default_rng(5)
+    x = cases.acts_outliers(M, K, seed=5)
+    q, s = hip.quantize_rows_sym(cases.t(x, dev))
+    assert np.array_equal(q.cpu().numpy()[::97], orc.sym_quant(x[::97], orc.sym_scales(x[::97])))
+    wq, sw = cases.weights_random_nibbles(N, K, seed=56)
+    W, SW = cases.t(wq, dev), cases.t(sw, dev)
+    c = hip.matmul(q, W)
+    rows = rng.choice(M, 16, replace=False)
+    cols = rng.choice(N, 32, replace=False)
+    want = orc.unpack_i4(q.cpu().numpy()[rows]).astype(np.int64) @ orc.unpack_i4(wq[cols]).astype(np.int64).T
+    assert np.array_equal(c.cpu().numpy()[np.ix_(rows, cols)], want)
+    y_fused = hip.linear4bit_forward(hip.EPI_SYM, q, s, None, W, SW)
+    y_unfused = hip.sym_dequant(c, s.view(-1), SW, 32)
+    assert torch.equal(y_fused.view(torch.int16), y_unfused.view(torch.int16))
+
+
+def test_leading_dims_and_odd_widths(qnn, dev):
+    """[B, S, K] inputs keep their leading dims; a width that is not a multiple of 32 takes
+    the torch-scale + given-scale kernel route and gives the same bits."""
+    _say("leading dims")
+    B, S, K, N = 2, 5, 128, 64
+    x = cases.acts_normal(B * S, K, seed=6).reshape(B, S, K)
+    wq, sw = cases.weights_random_nibbles(N, K, seed=66)
+    lin = _sq_module(qnn, dev, wq, sw)
+    p = qnn.SymQuantizer(1.0)(cases.t(x, dev))
+    assert tuple(p.quantized_x.shape) == (B, S, K // 2) and tuple(p.scales_x.shape) == (B, S, 1)
+    y = lin(p)
+    assert tuple(y.shape) == (B, S, N)
+    y_want, *_ = orc.linear4bit_sq_forward(x.reshape(-1, K), wq, sw)
+    assert cases.bits_equal(y.cpu().numpy().reshape(-1, N), y_want)
+    lin.fused = False
+    assert cases.bits_equal(lin(p).cpu().numpy().reshape(-1, N), y_want)
+    # odd width for the quantizers only (the GEMM needs K % 64 == 0)
+    xo = cases.acts_normal(7, 50, seed=7)
+    po = qnn.SymQuantizer(1.0)(cases.t(xo, dev))
+    so = orc.sym_scales(xo)
+    assert cases.bits_equal(po.scales_x.cpu().numpy(), so)
+    assert np.array_equal(po.quantized_x.cpu().numpy(), orc.sym_quant(xo, so))
+    pa = qnn.AsymQuantizer()(cases.t(xo, dev))
+    sa, za = orc.asym_scales_zeros(xo)
+    assert cases.bits_equal(pa.scales_x.cpu().numpy(), sa) and cases.bits_equal(pa.zeros_x.cpu().numpy(), za)
+    assert np.array_equal(pa.quantized_x.cpu().numpy(), orc.asym_quant(xo, sa, za))
+    # a non-contiguous input is made contiguous first (quantizer.py:11-12)
+    xt = cases.t(cases.acts_normal(64, 8, seed=8), dev).t()
+    pt = qnn.SymQuantizer(1.0)(xt)
+    assert np.array_equal(pt.quantized_x.cpu().numpy(), orc.sym_quant(xt.cpu().numpy(), orc.sym_scales(xt.cpu().numpy())))
+
+
+def test_error_paths_on_device(dev):
+    from duqlinear4bitcuda_amd import _HIP as hip
+    from duqlinear4bitcuda_amd.tools import tensor_utils as tu
+
+    a = torch.zeros(4, 32, dtype=torch.uint8, device=dev)
+    q = torch.zeros(4, 4, dtype=torch.int32, device=dev)
+    s4 = torch.ones(4, dtype=torch.float16, device=dev)
+    with pytest.raises(RuntimeError, match="Unsupported data type"):
+        hip.sym_dequant(q, s4, s4, 16)                                   # bindings.cpp:159-167
+    with pytest.raises(RuntimeError, match="contiguous"):
+        hip.matmul(a.t(), a)
+    with pytest.raises(RuntimeError, match="size"):
+        hip.sym_dequant(q, s4[:3], s4, 32)
+    with pytest.raises(RuntimeError, match="size"):
+        hip.sym_quant(torch.zeros(4, 64, dtype=torch.float16, device=dev), s4[:2])
+    with pytest.raises(RuntimeError):
+        hip.matmul(a, torch.zeros(4, 32, dtype=torch.uint8))             # other device
+    with pytest.raises(RuntimeError, match="multiple of 64"):
+        hip.matmul(torch.zeros(4, 48, dtype=torch.uint8, device=dev), torch.zeros(4, 48, dtype=torch.uint8, device=dev))
+    with pytest.raises(AssertionError):
+        tu.matmul(torch.zeros(4, 48, dtype=torch.uint8, device=dev), torch.zeros(4, 48, dtype=torch.uint8, device=dev))
+    # empty problems are no-ops
+    assert tuple(hip.matmul(a[:0], a).shape) == (0, 4)
+    assert tuple(hip.sym_quant(torch.zeros(0, 64, dtype=torch.float16, device=dev), s4[:0]).shape) == (0, 32)
+
+
+def test_runs_on_a_side_stream(qnn, dev):
+    """The ops launch on torch's current stream."""
+    M, K, N = 64, 256, 128
+    x = cases.acts_normal(M, K, seed=9)
+    wq, sw = cases.weights_random_nibbles(N, K, seed=99)
+    lin = _sq_module(qnn, dev, wq, sw)
+    want, *_ = orc.linear4bit_sq_forward(x, wq, sw)
+    side = torch.cuda.Stream()
+    xt = cases.t(x, dev)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        y = lin(qnn.SymQuantizer(1.0)(xt))
+    side.synchronize()
+    assert cases.bits_equal(y.cpu().numpy(), want)

@@ -1,0 +1,174 @@
+"""CPU-side checks: the C ABI library loads and exports what include/duq_hip.h declares,
+argument validation returns the documented codes before anything is launched, and the
+Python host layer keeps the reference's interface (names, buffers, asserts, errors)."""
+import ctypes
+import os
+import re
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _header_functions():
+    text = open(os.path.join(ROOT, "include", "duq_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(duq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from duqlinear4bitcuda_amd import _lib
+
+    lib = _lib.load()
+    names = _header_functions()
+    assert len(names) >= 16
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in include/duq_hip.h but not exported"
+    # and the binding table covers the header
+    assert set(_lib.PROTOTYPES) | {"duq_status_string"} == set(names)
+    assert lib.duq_abi_version() == 1
+    assert lib.duq_get_dual_quant_col_k() == 10
+
+
+def test_status_strings():
+    from duqlinear4bitcuda_amd import _lib
+
+    lib = _lib.load()
+    assert lib.duq_status_string(0) == b"ok"
+    for code in (-1, -2, -3, -4, -5, -6):
+        assert len(lib.duq_status_string(code)) > 3
+    assert b"64" in lib.duq_status_string(-3)
+
+
+def test_argument_validation_without_launch():
+    """Rejected calls return before touching the device (fake non-null pointers are never
+    dereferenced on the host)."""
+    from duqlinear4bitcuda_amd import _lib
+
+    lib = _lib.load()
+    P = 0x1000  # aligned, never dereferenced
+    assert lib.duq_matmul_host_4bit(P, P, 4, 4, 100, P, None) == -3          # K % 64
+    assert lib.duq_matmul_host_4bit(P, P, 4, 4, 131072, P, None) == -6       # K too large for the scaled accumulators
+    assert lib.duq_matmul_host_4bit(None, P, 4, 4, 64, P, None) == -1
+    assert lib.duq_matmul_host_4bit(P + 4, P, 4, 4, 64, P, None) == -5       # alignment
+    assert lib.duq_matmul_host_4bit(P, P, 4, 4, 64, None, None) == -1
+    assert lib.duq_matmul_host_4bit(None, None, 0, 4, 64, None, None) == 0   # empty problem is a no-op
+    assert lib.duq_sym_quant_host(P, P, 2, 10, 4, P, None) == -2             # colsDst != ceil(colsSrc/2)
+    assert lib.duq_sym_quant_host_qmax(P, P, 2, 10, 5, 9, P, None) == -4     # qmax
+    assert lib.duq_sym_quant_host(None, P, 2, 10, 5, P, None) == -1
+    assert lib.duq_sym_quant_host(None, None, 0, 10, 5, None, None) == 0
+    assert lib.duq_asym_quant_host(P, P, None, 2, 10, 5, P, None) == -1
+    assert lib.duq_quantize_rows_sym(P, 2, 48, 1.0, 6, P, P, None) == -2     # cols % 32
+    assert lib.duq_quantize_rows_sym(P + 2, 2, 64, 1.0, 6, P, P, None) == -5
+    assert lib.duq_quantize_rows_asym(P, 2, 64, P, P, None, None) == -1
+    assert lib.duq_sym_dequant_host(P, None, P, 2, 2, P, None) == -1
+    assert lib.duq_linear4bit_forward(7, P, P, None, P, P, None, None, None, None, 4, 4, 64, P, None) == -4
+    assert lib.duq_linear4bit_forward(1, P, P, None, P, P, None, None, None, None, 4, 4, 64, P, None) == -1  # asym needs zeros
+    assert lib.duq_linear4bit_forward(2, P, P, None, P, P, None, None, None, None, 4, 4, 64, P, None) == -1  # dual needs scale 2
+    assert lib.duq_linear4bit_forward(0, P, P, None, P, P, None, None, None, None, 4, 4, 96, P, None) == -3
+
+
+def test_check_raises_runtime_error():
+    from duqlinear4bitcuda_amd import _lib
+
+    with pytest.raises(RuntimeError, match="multiple of 64"):
+        _lib.check(-3, "matmul")
+    _lib.check(0, "ok")
+
+
+def test_ops_reject_cpu_tensors_like_the_reference_binding():
+    from duqlinear4bitcuda_amd import _HIP as hip
+
+    a = torch.zeros(4, 32, dtype=torch.uint8)
+    with pytest.raises(RuntimeError, match="GPU"):
+        hip.matmul(a, a)
+    x = torch.zeros(4, 64, dtype=torch.float16)
+    with pytest.raises(RuntimeError):
+        hip.sym_quant(x, torch.ones(4, dtype=torch.float16))
+    with pytest.raises(RuntimeError, match="contiguous"):
+        hip.matmul(a.t(), a)
+    assert hip.get_dual_quant_col_k() == 10
+
+
+def test_tensor_utils_asserts():
+    from duqlinear4bitcuda_amd.tools import tensor_utils as tu
+
+    with pytest.raises(AssertionError, match="multiplication of 32"):
+        tu.matmul(torch.zeros(2, 48, dtype=torch.uint8), torch.zeros(2, 48, dtype=torch.uint8))
+    with pytest.raises(AssertionError):
+        tu.sym_quant(torch.zeros(2, 64), torch.ones(2, 1, dtype=torch.float16))      # fp32 input
+    with pytest.raises(AssertionError):
+        tu.sym_dequant(torch.zeros(2, 2, dtype=torch.int64), torch.ones(2, dtype=torch.float16), torch.ones(2, dtype=torch.float16))
+    p = tu.PackedQuantizedTensor(torch.zeros(3, 8, dtype=torch.uint8), torch.ones(3, 1))
+    assert tuple(p.size()) == (3, 8) and p.dtype == torch.uint8 and p.device.type == "cpu" and p.zeros_x is None
+    assert tu.get_dual_quant_col() == 10
+
+
+def test_module_buffers_and_weight_prep_contract():
+    from duqlinear4bitcuda_amd import nn as qnn
+    from duqlinear4bitcuda_amd.tools import unpack_i4
+    from oracle import duq_oracle as orc
+
+    torch.manual_seed(0)
+    lin = torch.nn.Linear(64, 24, bias=True).half()
+    w = lin.weight.detach()
+    s = (w.abs().amax(-1, keepdim=True) / 7).half()
+
+    m = qnn.Linear4bitSQ.from_float(lin, s)
+    sd = m.state_dict()
+    assert list(sd) == ["weight_scales", "weight", "bias"]
+    assert sd["weight"].dtype == torch.uint8 and tuple(sd["weight"].shape) == (24, 32)
+    assert sd["weight_scales"].dtype == torch.float16 and tuple(sd["weight_scales"].shape) == (24, 1)
+    assert sd["bias"].dtype == torch.float16 and tuple(sd["bias"].shape) == (24,)
+    assert np.array_equal(sd["weight"].numpy(), orc.weight_sym_from_float(w.numpy(), s.numpy()))
+    assert torch.equal(unpack_i4(sd["weight"]), (w / s).round().to(torch.int32))
+    # a freshly constructed module has fp32 scales until it is cast, like the reference (linear.py:32-33)
+    assert qnn.Linear4bitSQ(64, 24).weight_scales.dtype == torch.float32
+    assert qnn.Linear4bitSQ(64, 24, bias=False).bias is None
+    with pytest.raises(AssertionError, match="out_features"):
+        qnn.Linear4bitSQ.from_float(lin, s.view(-1))
+    # round trip through state_dict
+    m2 = qnn.Linear4bitSQ(64, 24, bias=True).half()
+    m2.load_state_dict(sd)
+    assert all(torch.equal(a, b) for a, b in zip(m2.state_dict().values(), sd.values()))
+
+    a = qnn.Linear4bitASQ.from_linear(lin)
+    assert list(a.state_dict()) == ["weight_scales", "weight_zeros", "weight", "bias"]
+    pk, sc, z = orc.weight_asym_from_linear(w.numpy())
+    assert np.array_equal(a.weight.numpy(), pk)
+    assert np.array_equal(a.weight_scales.numpy().view(np.uint16), sc.view(np.uint16))
+    assert np.array_equal(a.weight_zeros.numpy().view(np.uint16), z.view(np.uint16))
+    assert isinstance(a.quantizer, qnn.AsymQuantizer)
+    assert not hasattr(qnn.Linear4bitASQ.from_linear(lin, require_quantizer=False), "quantizer")
+
+    d = qnn.Linear4bitDUSQ.from_float(lin, s, s * 2)
+    assert list(d.state_dict()) == ["weight_scales_1", "weight_scales_2", "weight", "bias"]
+    codes = unpack_i4(d.weight)
+    assert torch.equal(codes[:, :10], (w[:, :10] / s).round().to(torch.int32))
+    assert torch.equal(codes[:, 10:], (w[:, 10:] / (s * 2)).round().to(torch.int32))
+
+    u = qnn.LinearQuant4bitDUASQ.from_linear(lin)
+    assert list(u.state_dict()) == ["weight_scales_1", "weight_zeros_1", "weight_scales_2", "weight_zeros_2", "weight", "bias"]
+    assert all(v.dtype == torch.float16 and tuple(v.shape) == (24, 1) for k, v in u.state_dict().items() if "scales" in k or "zeros" in k)
+
+    with pytest.raises(AssertionError):
+        m(torch.zeros(2, 64).half())  # Linear4bitSQ wants a PackedQuantizedTensor (linear.py:46)
+
+
+def test_quantizer_attributes():
+    from duqlinear4bitcuda_amd import nn as qnn
+
+    q = qnn.SymQuantizer(0.9)
+    assert q.input_clip_ratio == 0.9 and q.qmax == 6
+    a = qnn.AsymQuantizer()
+    assert a.n_levels == 16 and a.input_clip_ratio == 1.0
+
+
+def test_bench_refuses_more_than_one_gpu():
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0
+    assert "ONE GPU" in r.stderr
