@@ -109,9 +109,9 @@ def decode_section(dev, quick):
     from duqlinear4bitcuda_amd import _HIP as hip
 
     out = []
-    shapes = [(1, 4096, 4096), (16, 4096, 4096), (1, 11008, 4096), (16, 11008, 4096)]
+    shapes = [(1, 4096, 4096), (4, 4096, 4096), (16, 4096, 4096), (1, 11008, 4096), (16, 11008, 4096)]
     if not quick:
-        shapes += [(4, 4096, 4096), (4, 11008, 4096), (1, 28672, 8192), (1, 8192, 28672)]
+        shapes += [(4, 11008, 4096), (1, 28672, 8192), (1, 8192, 28672), (16, 28672, 8192)]
     for (M, N, K) in shapes:
         wbytes = N * K // 2
         nbuf = min(96, max(3, int(600e6 // wbytes) + 1))
@@ -220,14 +220,14 @@ def main():
                             args.warmup)
     quant_us = event_time_us(lambda: hip.quantize_rows_sym(x), args.steps, args.warmup)
     achieved = ops / gemm_us / 1e6
-    roofline = {"bound": "mfma", "kernel": "gemm_s4_tile_kernel (fused GEMM + dequant)", "achieved": round(achieved, 1),
+    roofline = {"bound": "mfma", "kernel": "gemm_s4_stream_kernel<0,false> (fused GEMM + dequant)", "achieved": round(achieved, 1),
                 "peak": PEAK_INT8_TOPS, "unit": "TOP/s", "frac": round(achieved / PEAK_INT8_TOPS, 4),
                 "avg_kernel_us": round(gemm_us, 2), "traffic": None}
 
     decode = decode_section(dev, args.quick)
     quantizer = quantizer_section(dev)
     best_decode = max(decode, key=lambda d: d["GBps"])
-    roofline_decode = {"bound": "hbm", "kernel": "gemm_s4_skinny_kernel", "achieved": best_decode["GBps"],
+    roofline_decode = {"bound": "hbm", "kernel": "gemv_s4_dot_kernel (M<=4) / gemm_s4_skinny_kernel (M<=16)", "achieved": best_decode["GBps"],
                        "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": best_decode["frac_hbm"],
                        "shape": {k: best_decode[k] for k in ("M", "N", "K")}, "traffic": None}
 
@@ -235,6 +235,13 @@ def main():
     if not args.no_cpu:
         wq_cpu = unpack_i4(w.cpu()).float()
         cpu = cpu_baseline(x_cpu, wq_cpu, sw.cpu(), ops, budget_s=5.0 if args.quick else 15.0)
+
+    # a device copy of known size: the reference point for scaling hardware byte counters
+    # (FETCH_SIZE / WRITE_SIZE) when this script runs under rocprofv3 --pmc
+    ref_src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+    ref_dst = torch.empty_like(ref_src)
+    ref_dst.copy_(ref_src)
+    torch.cuda.synchronize()
 
     props = torch.cuda.get_device_properties(0)
     line = {

@@ -10,20 +10,19 @@
 // 256*|C| stays below 2^31 for K <= 131008.  Integer accumulation is order-free, so the
 // k order inside a tile only has to be the same for A and B.
 //
-// Two kernels:
-//  * tile kernel (prefill, M > 16): BM x BN x 128 tiles, 4 wavefronts (2 x 2), packed
-//    nibbles are expanded to bytes on the way from global memory into LDS, LDS rows are
-//    padded to 144 B so that the 128-bit fragment reads are bank-conflict free, LDS is
-//    double buffered and the next tile's global loads are in flight during the MFMAs.
-//    The weight operand goes to the MFMA "A" side, so each lane ends up with four
-//    consecutive output columns of one row and stores them as one vector.
-//  * skinny kernel (decode, M <= 16): HBM-bound weight streaming.  One workgroup owns 16
-//    output columns, its wavefronts split K, every lane issues all of its 128-bit weight
-//    loads before the first MFMA, fragments go from global memory straight to registers
-//    (no LDS for operands), partial sums meet in LDS once at the end.
+// Four kernels, picked by shape in launch_epi():
+//  * stream kernel (prefill, M > 64 and at least 128 tiles of 128 x 256): weights go from
+//    global memory straight to registers, activations are expanded once into LDS,
+//    v_mfma_i32_32x32x32_i8 with a hand-ordered schedule (see the kernel);
+//  * tile kernel (everything else above 16 rows): BM x BN x 128 tiles, 4 wavefronts (2 x 2),
+//    both operands expanded on the way into double-buffered LDS, v_mfma_i32_16x16x64_i8;
+//  * skinny kernel (decode, 5 <= M <= 16): one workgroup owns 16 output columns, its
+//    wavefronts split K, fragments go from global memory straight to registers;
+//  * dot kernel (decode, M <= 4): v_dot8_i32_i4 on the packed nibbles, a pure HBM stream.
+// In the MFMA kernels the weight operand goes to the MFMA "A" side, so each lane ends up
+// with four consecutive output columns of one row.
 #include "duq_epilogue.h"
 #include "duq_launch.h"
-#include <cstdlib>
 #include <type_traits>
 
 namespace duq {
@@ -552,7 +551,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_s4_skinny_kernel(GemmParams p
         for (int u = 0; u < kSkinnyUnroll; ++u) {
             const uint32_t off = (s0 + u) * 64;
             const bool ok = (s0 + u) < seg_end && off + g * 16 < kbytes;
-            w[u] = ok ? __builtin_nontemporal_load(reinterpret_cast<const v4u *>(wsrc + off)) : v4u{0u, 0u, 0u, 0u};
+            w[u] = ok ? *reinterpret_cast<const v4u *>(wsrc + off) : v4u{0u, 0u, 0u, 0u};
             x[u] = (ok && xrow_ok) ? *reinterpret_cast<const v4u *>(xsrc + off) : v4u{0u, 0u, 0u, 0u};
         }
 #pragma unroll
@@ -586,11 +585,125 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_s4_skinny_kernel(GemmParams p
 }
 
 // ---------------------------------------------------------------------------------
+// dot kernel (decode, M <= 4): weight streaming on v_dot8_i32_i4
+// ---------------------------------------------------------------------------------
+// The signed 4-bit dot product instruction consumes packed nibbles as they lie in memory,
+// so nothing is expanded and no MFMA is needed: the kernel is a pure HBM stream.
+// Workgroup = 4 wavefronts = 8 weight rows, K split four ways.  Lane (r8, j) walks its
+// quarter of row r8 in 128-byte steps, loading bytes [step*128 + j*16, +16): one wavefront
+// load is eight full cache lines.  Eight loads per lane are kept in flight (a register
+// ring), and with ~40 VGPRs eight wavefronts fit on a SIMD, so a CU keeps > 100 KB of
+// weights in flight.  The M activation rows sit in LDS (lanes of different rows read the
+// same address: a broadcast).  Partial sums meet through three lane shuffles and one LDS hop.
+constexpr int kDotRing = 8;
+
+template <int MROWS, int EPI, bool BIAS>
+__global__ __launch_bounds__(256) void gemv_s4_dot_kernel(GemmParams p)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [MROWS][xstride] packed activations
+    __shared__ int part[4][8][MROWS];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u, wave = tid >> 6;
+    const uint32_t r8 = lane >> 3, j = lane & 7u;
+    const uint32_t kbytes = p.K >> 1;
+    const uint32_t nsteps_all = (kbytes + 127) / 128;
+    const uint32_t xstride = nsteps_all * 128;
+    const uint32_t per = (nsteps_all + 3) / 4;
+    const uint32_t step0 = wave * per;
+    const uint32_t nsteps = step0 < nsteps_all ? min(per, nsteps_all - step0) : 0;
+    const uint32_t n = blockIdx.x * 8 + r8;
+
+    const __amdgpu_buffer_rsrc_t rW = make_rsrc(p.B, p.N * kbytes);  // rows past N read as zero
+    const uint32_t wbase = n * kbytes + j * 16;
+
+    auto w_off = [&](uint32_t s) -> uint32_t {  // step s of this wavefront's slice
+        const uint32_t off = (step0 + s) * 128 + j * 16;
+        return (s < nsteps && off < kbytes && n < p.N) ? wbase + (step0 + s) * 128 : kOobOffset;
+    };
+
+    v4u ring[kDotRing];
+#pragma unroll
+    for (int u = 0; u < kDotRing; ++u) ring[u] = buf_load16(rW, w_off(u), 0);
+
+    // activations -> LDS (all rows, whole K), zero beyond the row end
+    for (uint32_t i = tid; i < MROWS * (xstride / 16); i += 256) {
+        const uint32_t m = i / (xstride / 16), o = (i % (xstride / 16)) * 16;
+        v4u v = v4u{0u, 0u, 0u, 0u};
+        if (m < p.M && o < kbytes) v = *reinterpret_cast<const v4u *>(p.A + (uint64_t)m * kbytes + o);
+        *reinterpret_cast<v4u *>(xs + m * xstride + o) = v;
+    }
+    __syncthreads();
+
+    int acc[MROWS];
+#pragma unroll
+    for (int m = 0; m < MROWS; ++m) acc[m] = 0;
+
+    for (uint32_t s = 0; s < nsteps; s += kDotRing) {
+#pragma unroll
+        for (int u = 0; u < kDotRing; ++u) {
+            const v4u w = ring[u];
+            ring[u] = buf_load16(rW, w_off(s + u + kDotRing), 0);
+            const uint32_t xo = (step0 + s + u) * 128 + j * 16;
+            if (s + u < nsteps) {
+#pragma unroll
+                for (int m = 0; m < MROWS; ++m) {
+                    const v4u x = *reinterpret_cast<const v4u *>(xs + m * xstride + xo);
+#pragma unroll
+                    for (int d = 0; d < 4; ++d) acc[m] = __builtin_amdgcn_sdot8((int)w[d], (int)x[d], acc[m], false);
+                }
+            }
+        }
+    }
+
+    // the 8 lanes of a row, then the 4 wavefronts
+#pragma unroll
+    for (int m = 0; m < MROWS; ++m) {
+        acc[m] += __shfl_xor(acc[m], 1, kWave);
+        acc[m] += __shfl_xor(acc[m], 2, kWave);
+        acc[m] += __shfl_xor(acc[m], 4, kWave);
+    }
+    if (j == 0) {
+#pragma unroll
+        for (int m = 0; m < MROWS; ++m) part[wave][r8][m] = acc[m];
+    }
+    __syncthreads();
+    if (tid < 8 * MROWS) {
+        const uint32_t rr = tid / MROWS, m = tid % MROWS;
+        const uint32_t nn = blockIdx.x * 8 + rr;
+        if (nn < p.N && m < p.M) {
+            const int v = part[0][rr][m] + part[1][rr][m] + part[2][rr][m] + part[3][rr][m];
+            if (EPI < 0) {
+                p.C[(uint64_t)m * p.N + nn] = v;
+            } else {
+                constexpr int MODE = EPI < 0 ? 0 : EPI;
+                const ColParams c = load_col<MODE, BIAS>(p.epi.s_col_1, p.epi.z_col_1, p.epi.s_col_2, p.epi.z_col_2,
+                                                         p.epi.bias, nn);
+                const f16 s_row = bits_to_f16(p.epi.s_row[m]);
+                const f16 z_row = (MODE == 1 || MODE == 3) ? bits_to_f16(p.epi.z_row[m]) : (f16)0;
+                p.y[(uint64_t)m * p.N + nn] = dequant_one<MODE, BIAS>(v, s_row, z_row, c);
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------
 // dispatch
 // ---------------------------------------------------------------------------------
 template <int EPI, bool BIAS>
 static void launch_epi(GemmParams &p, hipStream_t stream)
 {
+    const uint64_t wbytes = (uint64_t)p.N * (p.K / 2);
+    const uint32_t xstride = ((p.K / 2 + 127) / 128) * 128;
+    if (p.M <= 4 && wbytes < 0xFFFFFF00ull && 4 * xstride <= 60 * 1024 && p.K > 0) {
+        const dim3 grid((p.N + 7) / 8);
+        if (p.M == 1)
+            hipLaunchKernelGGL((gemv_s4_dot_kernel<1, EPI, BIAS>), grid, dim3(256), 1 * xstride, stream, p);
+        else if (p.M == 2)
+            hipLaunchKernelGGL((gemv_s4_dot_kernel<2, EPI, BIAS>), grid, dim3(256), 2 * xstride, stream, p);
+        else
+            hipLaunchKernelGGL((gemv_s4_dot_kernel<4, EPI, BIAS>), grid, dim3(256), 4 * xstride, stream, p);
+        return;
+    }
     if (p.M <= 16) {
         const dim3 grid((p.N + 15) / 16);
         const uint32_t segs = (p.K / 2 + 63) / 64;
@@ -606,8 +719,7 @@ static void launch_epi(GemmParams &p, hipStream_t stream)
     // largest tile that still yields at least one workgroup per CU (256 CUs); small
     // problems take the small tile to spread over the chip.
     auto tiles = [&](uint32_t bm, uint32_t bn) { return ((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn); };
-    static const int variant = getenv("DUQ_GEMM_VARIANT") ? atoi(getenv("DUQ_GEMM_VARIANT")) : 1;
-    if (variant == 1 && tiles(128, 256) >= 128 && p.M > 64) {
+    if (tiles(128, 256) >= 128 && p.M > 64) {
         p.tiles_m = (p.M + 127) / 128;
         p.tiles_n = (p.N + 255) / 256;
         hipLaunchKernelGGL((gemm_s4_stream_kernel<EPI, BIAS>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, stream, p);

@@ -88,6 +88,12 @@ def test_quantize_rows_sym(hip, dev, M, K):
     x = cases.acts_outliers(M, K, seed=30 + M + K)
     if M > 2:
         x[1, :] = 0  # an all-zero token: scale 0, codes 0
+    if M > 8:
+        x[2, 5] = np.nan          # NaN statistic: every code of the row becomes 0
+        x[3, 7] = np.inf          # inf statistic: scale inf, codes 0
+        x[4, :] = 0
+        x[4, 9] = 6e-8            # max/7 underflows to a zero scale on a non-zero row
+        x[5, :] *= 1e-4           # a subnormal-range row
     for qmax, clip in ((6, 1.0), (7, 1.0), (6, 0.9)):
         s_want = orc.sym_scales(x, clip)
         q_want = orc.sym_quant(x, s_want, qmax)
@@ -104,6 +110,10 @@ def test_quantize_rows_asym(hip, dev, M, K):
         x[1, :] = cases.acts_normal(1, K, seed=5)[0]  # a signed row
     if M > 3:
         x[2, :] = 1.5  # max == min: scale 0
+    if M > 8:
+        x[3, :] = x[3, :] * 0.01 + 900.0   # large offset: zero point far above 480
+        x[4, 3] = np.inf
+        x[5, :] = -x[5, :]                 # all negative
     s_want, z_want = orc.asym_scales_zeros(x)
     q_want = orc.asym_quant(x, s_want, z_want)
     q, s, z = hip.quantize_rows_asym(cases.t(x, dev))
