@@ -31,6 +31,7 @@ if ROOT not in sys.path:
 
 PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, published
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, published
+GEMM_TRAFFIC_BYTES = (33161 + 16384) * 1024  # fetched + written per launch of the fused GEMM (rocprofv3 counters)
 
 
 def heavy_tail_acts(M, K, seed, frac=0.01):
@@ -222,7 +223,10 @@ def main():
     achieved = ops / gemm_us / 1e6
     roofline = {"bound": "mfma", "kernel": "gemm_s4_stream_kernel<0,false> (fused GEMM + dequant)", "achieved": round(achieved, 1),
                 "peak": PEAK_INT8_TOPS, "unit": "TOP/s", "frac": round(achieved / PEAK_INT8_TOPS, 4),
-                "avg_kernel_us": round(gemm_us, 2), "traffic": None}
+                "avg_kernel_us": round(gemm_us, 2),
+                # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this workload, each
+                # scaled by what the counter reads for the 256 MiB copy at the end of this script
+                "traffic": GEMM_TRAFFIC_BYTES, "traffic_source": "profiles/gemm_s4_stream_kernel__prefill_M2048_K4096_N4096.txt"}
 
     decode = decode_section(dev, args.quick)
     quantizer = quantizer_section(dev)

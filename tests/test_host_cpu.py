@@ -172,3 +172,17 @@ def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert r.returncode != 0
     assert "ONE GPU" in r.stderr
+
+
+def test_reference_package_name_is_importable():
+    import qlinear4bit._CUDA as ops
+    import qlinear4bit.nn as rnn
+    import qlinear4bit.tools.tensor_utils as tu
+    from duqlinear4bitcuda_amd import nn as impl
+    from qlinear4bit.tools.quantization import pack_i4, unpack_i4  # noqa: F401
+
+    assert rnn.Linear4bitSQ is impl.Linear4bitSQ and rnn.SymQuantizer is impl.SymQuantizer
+    assert tu.get_dual_quant_col() == ops.get_dual_quant_col_k() == 10
+    for name in ("matmul", "sym_quant", "sym_dual_quant", "sym_dequant", "sym_dual_dequant", "asym_quant",
+                 "asym_dequant", "asym_dual_quant", "asym_dual_dequant", "get_dual_quant_col_k"):
+        assert callable(getattr(ops, name)), name       # the op names of src/export/bindings.cpp:772-923
