@@ -108,4 +108,23 @@ __device__ __forceinline__ QuadCols<MODE, BIAS> load_quad_cols(const uint16_t *s
     return q;
 }
 
+// Same selection as load_quad_cols, from raw 64-bit words fetched earlier (four binary16
+// values per word, column n0 first).
+template <int MODE, bool BIAS>
+__device__ __forceinline__ QuadCols<MODE, BIAS> quad_cols_from_raw(v2u s1, v2u z1, v2u s2, v2u z2, v2u bias, uint32_t n0)
+{
+    auto pick = [](v2u v, int r) -> uint16_t { return (uint16_t)((r & 1) ? (v[r >> 1] >> 16) : (v[r >> 1] & 0xFFFFu)); };
+    QuadCols<MODE, BIAS> q;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const uint32_t col = n0 + r;
+        const bool first = MODE == 2 ? col < (uint32_t)kQuantColK : col == 0;
+        q.c[r].s = bits_to_f16((MODE == 2 || MODE == 3) ? (first ? pick(s1, r) : pick(s2, r)) : pick(s1, r));
+        q.c[r].z = (MODE == 1) ? bits_to_f16(pick(z1, r))
+                               : (MODE == 3 ? bits_to_f16(col == 0 ? pick(z1, r) : pick(z2, r)) : (f16)0);
+        q.c[r].bias = BIAS ? bits_to_f16(pick(bias, r)) : (f16)0;
+    }
+    return q;
+}
+
 }  // namespace duq

@@ -411,6 +411,38 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
         for (int b = 0; b < TM; ++b) fx[0][b] = *reinterpret_cast<const v4i *>(lds + fragX + b * 32 * kXStride);
     }
 
+    // ---- epilogue parameters: fetched now so that their latency hides behind the main loop
+    constexpr int MODE = EPI < 0 ? 0 : EPI;
+    const Epilogue &e = p.epi;
+    bool staged = false;
+    v2u raw_s1[TN * 4], raw_z1[TN * 4], raw_s2[TN * 4], raw_z2[TN * 4], raw_bias[TN * 4];
+    f16 s_row[TM], z_row[TM];
+    if (EPI >= 0) {
+        const bool vec_ld = p.N % 4 == 0 && reinterpret_cast<uintptr_t>(e.s_col_1) % 8 == 0 &&
+                            (MODE == 0 || MODE == 2 || reinterpret_cast<uintptr_t>(e.z_col_1) % 8 == 0) &&
+                            (MODE < 2 || reinterpret_cast<uintptr_t>(e.s_col_2) % 8 == 0) &&
+                            (MODE != 3 || reinterpret_cast<uintptr_t>(e.z_col_2) % 8 == 0) &&
+                            (!BIAS || reinterpret_cast<uintptr_t>(e.bias) % 8 == 0);
+        staged = p.N % 8 == 0 && reinterpret_cast<uintptr_t>(p.y) % 16 == 0 && vec_ld;
+#pragma unroll
+        for (int b = 0; b < TM; ++b) {
+            const uint32_t m = min(m0 + b * 32 + l32, p.M - 1);
+            s_row[b] = bits_to_f16(e.s_row[m]);
+            z_row[b] = (MODE == 1 || MODE == 3) ? bits_to_f16(e.z_row[m]) : (f16)0;
+        }
+        if (staged) {
+#pragma unroll
+            for (int tq = 0; tq < TN * 4; ++tq) {
+                const uint32_t nq = min(n0 + wave * 64 + (tq >> 2) * 32 + (tq & 3) * 8 + h * 4, p.N - 4);
+                raw_s1[tq] = *reinterpret_cast<const v2u *>(e.s_col_1 + nq);
+                if (MODE == 1 || MODE == 3) raw_z1[tq] = *reinterpret_cast<const v2u *>(e.z_col_1 + nq);
+                if (MODE >= 2) raw_s2[tq] = *reinterpret_cast<const v2u *>(e.s_col_2 + nq);
+                if (MODE == 3) raw_z2[tq] = *reinterpret_cast<const v2u *>(e.z_col_2 + nq);
+                if (BIAS) raw_bias[tq] = *reinterpret_cast<const v2u *>(e.bias + nq);
+            }
+        }
+    }
+
     uint32_t cur = 0, nxt = kBuf, nx2 = 2 * kBuf;
     auto rotate = [&]() {
         const uint32_t t = cur;
@@ -447,70 +479,74 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
                     store_quad<EPI, BIAS>(p, m0 + b * 32 + l32, n0 + wave * 64 + t * 32 + q * 8 + h * 4, v, vec_ok);
                 }
     } else {
-        constexpr int MODE = EPI < 0 ? 0 : EPI;
-        const Epilogue &e = p.epi;
-        const bool vec_st = p.N % 4 == 0 && reinterpret_cast<uintptr_t>(p.y) % 8 == 0;
-        const bool vec_ld = p.N % 4 == 0 && reinterpret_cast<uintptr_t>(e.s_col_1) % 8 == 0 &&
-                            (MODE == 0 || MODE == 2 || reinterpret_cast<uintptr_t>(e.z_col_1) % 8 == 0) &&
-                            (MODE < 2 || reinterpret_cast<uintptr_t>(e.s_col_2) % 8 == 0) &&
-                            (MODE != 3 || reinterpret_cast<uintptr_t>(e.z_col_2) % 8 == 0) &&
-                            (!BIAS || reinterpret_cast<uintptr_t>(e.bias) % 8 == 0);
-        f16 s_row[TM], z_row[TM];
-#pragma unroll
-        for (int b = 0; b < TM; ++b) {
-            const uint32_t m = min(m0 + b * 32 + l32, p.M - 1);
-            s_row[b] = bits_to_f16(e.s_row[m]);
-            z_row[b] = (MODE == 1 || MODE == 3) ? bits_to_f16(e.z_row[m]) : (f16)0;
-        }
-        // When rows of y are 16-byte aligned, the 128 x 64 fp16 tile of this wavefront goes
-        // through LDS (free now) so that the global stores are whole 128-byte lines: the MFMA
-        // layout itself only offers 16 contiguous bytes per row and store instruction.
+        // Fast path (uniform condition): rows of y are 16-byte aligned and the column
+        // parameter arrays 8-byte aligned.  The 128 x 64 fp16 tile of this wavefront goes
+        // through LDS (free now) so that global stores are whole 128-byte lines (the MFMA
+        // layout only offers 16 contiguous bytes per row and instruction), and the code is
+        // branch-free: parameter loads are clamped, stores are buffer stores whose offset
+        // is redirected out of range for rows past M or columns past N.
         constexpr uint32_t kYStride = 144;  // bytes per staged row: 128 + pad
-        const bool staged = p.N % 8 == 0 && reinterpret_cast<uintptr_t>(p.y) % 16 == 0;
-        uint8_t *stage = lds + wave * (BM * kYStride);
-        if (staged) __syncthreads();  // every wavefront is done reading the activation buffers
+        if (staged) {
+            uint8_t *stage = lds + wave * (BM * kYStride);
+            __syncthreads();  // every wavefront is done reading the activation buffers
 #pragma unroll
-        for (int t = 0; t < TN; ++t)
+            for (int t = 0; t < TN; ++t)
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const uint32_t ncol = t * 32 + q * 8 + h * 4;  // column inside the wavefront's tile
-                const uint32_t nq = n0 + wave * 64 + ncol;
-                if (!staged && nq >= p.N) continue;
-                const QuadCols<MODE, BIAS> cols = load_quad_cols<MODE, BIAS>(e.s_col_1, e.z_col_1, e.s_col_2, e.z_col_2,
-                                                                             e.bias, min(nq, p.N - 1), p.N, vec_ld);
+                for (int q = 0; q < 4; ++q) {
+                    const uint32_t ncol = t * 32 + q * 8 + h * 4;  // column inside the wavefront's tile
+                    const uint32_t nq = min(n0 + wave * 64 + ncol, p.N - 4);
+                    const QuadCols<MODE, BIAS> cols = quad_cols_from_raw<MODE, BIAS>(
+                        raw_s1[t * 4 + q], raw_z1[t * 4 + q], raw_s2[t * 4 + q], raw_z2[t * 4 + q], raw_bias[t * 4 + q], nq);
 #pragma unroll
-                for (int b = 0; b < TM; ++b) {
-                    const uint32_t m = m0 + b * 32 + l32;
-                    uint16_t out[4];
+                    for (int b = 0; b < TM; ++b) {
+                        uint16_t out[4];
 #pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        out[r] = dequant_one<MODE, BIAS>(acc[t][b][q * 4 + r] >> 8, s_row[b], z_row[b], cols.c[r]);
-                    const v2u packed = v2u{(uint32_t)out[0] | ((uint32_t)out[1] << 16),
-                                           (uint32_t)out[2] | ((uint32_t)out[3] << 16)};
-                    if (staged) {
-                        *reinterpret_cast<v2u *>(stage + (b * 32 + l32) * kYStride + ncol * 2) = packed;
-                    } else if (m < p.M) {
-                        uint16_t *dst = p.y + (uint64_t)m * p.N + nq;
-                        if (vec_st && nq + 3 < p.N) {
-                            *reinterpret_cast<v2u *>(dst) = packed;
-                        } else {
-#pragma unroll
-                            for (int r = 0; r < 4; ++r)
-                                if (nq + r < p.N) dst[r] = out[r];
-                        }
+                        for (int r = 0; r < 4; ++r)
+                            out[r] = dequant_one<MODE, BIAS>(acc[t][b][q * 4 + r] >> 8, s_row[b], z_row[b], cols.c[r]);
+                        *reinterpret_cast<v2u *>(stage + (b * 32 + l32) * kYStride + ncol * 2) =
+                            v2u{(uint32_t)out[0] | ((uint32_t)out[1] << 16), (uint32_t)out[2] | ((uint32_t)out[3] << 16)};
                     }
                 }
-            }
-        if (staged) {
-            // same wavefront wrote and reads its stage: LDS operations complete in order
+            // the same wavefront wrote and reads its stage: LDS operations complete in order
+            const uint32_t rows_here = min(p.M - m0, (uint32_t)BM);
+            const __amdgpu_buffer_rsrc_t rY = make_rsrc(p.y + (uint64_t)m0 * p.N, rows_here * p.N * 2);
             const uint32_t piece = lane & 7u, rsub = lane >> 3;
             const uint32_t ncol0 = n0 + wave * 64 + piece * 8;
 #pragma unroll
             for (int it = 0; it < BM / 8; ++it) {
                 const uint32_t row = it * 8 + rsub;
                 const v4u v = *reinterpret_cast<const v4u *>(stage + row * kYStride + piece * 16);
-                if (m0 + row < p.M && ncol0 < p.N)
-                    *reinterpret_cast<v4u *>(p.y + (uint64_t)(m0 + row) * p.N + ncol0) = v;
+                const uint32_t off = (row < rows_here && ncol0 < p.N) ? (row * p.N + ncol0) * 2 : kOobOffset;
+                __builtin_amdgcn_raw_buffer_store_b128(v, rY, (int)off, 0, 0);
+            }
+        } else {
+#pragma unroll 1
+            for (int tq = 0; tq < TN * 4; ++tq) {
+                // generic path (odd N / unaligned pointers): per-element guards; the accumulator
+                // registers are picked with a switch because they cannot be indexed at run time
+                const int t = tq >> 2, q = tq & 3;
+                const uint32_t nq = n0 + wave * 64 + t * 32 + q * 8 + h * 4;
+                if (nq >= p.N) continue;
+                const QuadCols<MODE, BIAS> cols = load_quad_cols<MODE, BIAS>(e.s_col_1, e.z_col_1, e.s_col_2, e.z_col_2,
+                                                                             e.bias, nq, p.N, false);
+#pragma unroll
+                for (int b = 0; b < TM; ++b) {
+                    const uint32_t m = m0 + b * 32 + l32;
+                    v4i v;
+#pragma unroll
+                    for (int tt = 0; tt < TN; ++tt)
+#pragma unroll
+                        for (int qq = 0; qq < 4; ++qq)
+                            if (tt == t && qq == q) {
+#pragma unroll
+                                for (int r = 0; r < 4; ++r) v[r] = acc[tt][b][qq * 4 + r] >> 8;
+                            }
+                    if (m >= p.M) continue;
+                    uint16_t *dst = p.y + (uint64_t)m * p.N + nq;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (nq + r < p.N) dst[r] = dequant_one<MODE, BIAS>(v[r], s_row[b], z_row[b], cols.c[r]);
+                }
             }
         }
     }
