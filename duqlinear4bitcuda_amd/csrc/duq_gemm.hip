@@ -553,71 +553,112 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
 }
 
 // ---------------------------------------------------------------------------------
-// skinny kernel (M <= 16)
+// skinny kernel (5 <= M <= 16; also M <= 4 when the dot kernel's limits do not hold)
 // ---------------------------------------------------------------------------------
-// Workgroup = WAVES wavefronts, 16 output columns.  Wavefront w owns the k range
-// [w*kw, (w+1)*kw) with kw = ceil(K/64/WAVES)*64 elements, walked in steps of 128 k (64 B
-// per row): lane (l16, g) loads bytes [g*16, g*16+16) of the 64-byte segment of weight
-// row n0+l16 and of activation row l16, expands both and issues two MFMAs (even k, odd k).
-constexpr int kSkinnyUnroll = 8;  // 128-bit loads in flight per operand per lane
+// Workgroup = WAVES wavefronts that split K; it walks `tiles_per_wg` consecutive 16-column
+// tiles.  Wavefront w owns 64-byte row segments [w*S, (w+1)*S), S <= 8: lane (l16, g) holds
+// bytes [g*16, +16) of each.  The activation fragments of that k range do not depend on the
+// column tile, so they are loaded and expanded ONCE per workgroup and stay in registers;
+// per tile only the weights stream in (the next tile's loads are issued before the current
+// tile's MFMAs), two MFMAs per 16-byte weight piece (even k, odd k).  Partial sums of the
+// wavefronts meet in LDS (double buffered: one barrier per tile).
+constexpr int kSkinnySegs = 8;  // 64-byte segments per wavefront = 128-bit weight loads in flight per lane
 
 template <int WAVES, int EPI, bool BIAS>
 __global__ __launch_bounds__(WAVES * 64) void gemm_s4_skinny_kernel(GemmParams p)
 {
-    __shared__ v4i part[WAVES][64];
+    __shared__ v4i part[2][WAVES][64];
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63u, wave = tid >> 6;
     const uint32_t l16 = lane & 15u, g = lane >> 4;
-    const uint32_t n0 = blockIdx.x * 16;
     const uint32_t kbytes = p.K >> 1;
-    const uint32_t segs = kbytes / 64 + ((kbytes % 64) ? 1 : 0);  // 64-byte segments per row
-    const uint32_t per_wave = (segs + WAVES - 1) / WAVES;
-    const uint32_t seg_begin = wave * per_wave;
-    const uint32_t seg_end = min(seg_begin + per_wave, segs);
+    const uint32_t segs = (kbytes + 63) / 64;
+    const uint32_t seg0 = wave * kSkinnySegs;  // the launcher guarantees WAVES * kSkinnySegs >= segs
+    const uint32_t tiles_per_wg = p.tiles_m;   // (field reused: column tiles per workgroup)
+    const uint32_t ntiles = (p.N + 15) / 16;
+    const uint32_t tile0 = blockIdx.x * tiles_per_wg;
+    const uint32_t tile_end = min(tile0 + tiles_per_wg, ntiles);
 
-    const uint32_t wrow = min(n0 + l16, p.N - 1);
-    const bool xrow_ok = l16 < p.M;
-    const uint8_t *wsrc = p.B + (uint64_t)wrow * kbytes + g * 16;
-    const uint8_t *xsrc = p.A + (uint64_t)(xrow_ok ? l16 : 0) * kbytes + g * 16;
+    const __amdgpu_buffer_rsrc_t rW = make_rsrc(p.B, p.N * kbytes);  // rows past N read as zero
+    const __amdgpu_buffer_rsrc_t rX = make_rsrc(p.A, p.M * kbytes);  // rows past M read as zero
 
-    v4i acc = v4i{0, 0, 0, 0};
-    for (uint32_t s0 = seg_begin; s0 < seg_end; s0 += kSkinnyUnroll) {
-        v4u w[kSkinnyUnroll], x[kSkinnyUnroll];
+    uint32_t koff[kSkinnySegs];  // byte offset inside a row, or out of range for pieces past K
 #pragma unroll
-        for (int u = 0; u < kSkinnyUnroll; ++u) {
-            const uint32_t off = (s0 + u) * 64;
-            const bool ok = (s0 + u) < seg_end && off + g * 16 < kbytes;
-            w[u] = ok ? *reinterpret_cast<const v4u *>(wsrc + off) : v4u{0u, 0u, 0u, 0u};
-            x[u] = (ok && xrow_ok) ? *reinterpret_cast<const v4u *>(xsrc + off) : v4u{0u, 0u, 0u, 0u};
-        }
+    for (int u = 0; u < kSkinnySegs; ++u) {
+        const uint32_t off = (seg0 + u) * 64 + g * 16;
+        koff[u] = (seg0 + u < segs && off < kbytes) ? off : kOobOffset;
+    }
+
+    // activations of this wavefront's k range: once per workgroup
+    v4u xe[kSkinnySegs], xo[kSkinnySegs];
 #pragma unroll
-        for (int u = 0; u < kSkinnyUnroll; ++u) {
-            v4u we, wo, xe, xo;
+    for (int u = 0; u < kSkinnySegs; ++u) {
+        const v4u x = buf_load16(rX, koff[u] == kOobOffset ? kOobOffset : l16 * kbytes + koff[u], 0);
+        expand_nibbles(x, xe[u], xo[u]);
+    }
+
+    auto load_tile = [&](uint32_t tile, v4u(&w)[kSkinnySegs]) {
+        const uint32_t row = tile * 16 + l16;
+        const bool rok = tile < tile_end && row < p.N;
+#pragma unroll
+        for (int u = 0; u < kSkinnySegs; ++u)
+            w[u] = buf_load16(rW, (rok && koff[u] != kOobOffset) ? row * kbytes + koff[u] : kOobOffset, 0);
+    };
+    auto compute_tile = [&](uint32_t tile, const v4u(&w)[kSkinnySegs], uint32_t buf) {
+        v4i acc = v4i{0, 0, 0, 0};
+#pragma unroll
+        for (int u = 0; u < kSkinnySegs; ++u) {
+            v4u we, wo;
             expand_nibbles(w[u], we, wo);
-            expand_nibbles(x[u], xe, xo);
-            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i, we), __builtin_bit_cast(v4i, xe),
-                                                        acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i, wo), __builtin_bit_cast(v4i, xo),
-                                                        acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i, we), __builtin_bit_cast(v4i, xe[u]), acc,
+                                                        0, 0, 0);
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i, wo), __builtin_bit_cast(v4i, xo[u]), acc,
+                                                        0, 0, 0);
         }
-    }
+        if (WAVES > 1) {
+            // every wavefront parks its 16 x 16 partial tile, then the first 256 threads each
+            // finish one output element (sum over wavefronts, epilogue, store): no wavefront
+            // is a serial bottleneck
+            part[buf][wave][lane] = acc;
+            __syncthreads();
+            if (tid < 256) {
+                const uint32_t src_lane = tid >> 2, r = tid & 3u;
+                int sum = 0;
+#pragma unroll
+                for (int w2 = 0; w2 < WAVES; ++w2) sum += part[buf][w2][src_lane][r];
+                sum >>= 8;
+                const uint32_t m = src_lane & 15u, n = tile * 16 + (src_lane >> 4) * 4 + r;
+                if (m < p.M && n < p.N) {
+                    if (EPI < 0) {
+                        p.C[(uint64_t)m * p.N + n] = sum;
+                    } else {
+                        constexpr int MODE = EPI < 0 ? 0 : EPI;
+                        const ColParams c = load_col<MODE, BIAS>(p.epi.s_col_1, p.epi.z_col_1, p.epi.s_col_2,
+                                                                 p.epi.z_col_2, p.epi.bias, n);
+                        const f16 s_row = bits_to_f16(p.epi.s_row[m]);
+                        const f16 z_row = (MODE == 1 || MODE == 3) ? bits_to_f16(p.epi.z_row[m]) : (f16)0;
+                        p.y[(uint64_t)m * p.N + n] = dequant_one<MODE, BIAS>(sum, s_row, z_row, c);
+                    }
+                }
+            }
+            return;
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[r] >>= 8;
+        const bool vec_ok = (EPI < 0) ? (p.N % 4 == 0 && reinterpret_cast<uintptr_t>(p.C) % 16 == 0)
+                                      : (p.N % 4 == 0 && reinterpret_cast<uintptr_t>(p.y) % 8 == 0);
+        store_quad<EPI, BIAS>(p, l16, tile * 16 + g * 4, acc, vec_ok);
+    };
 
-    if (WAVES > 1) {
-        part[wave][lane] = acc;
-        __syncthreads();
-        if (wave != 0) return;
-#pragma unroll
-        for (int w = 1; w < WAVES; ++w) {
-            const v4i o = part[w][lane];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) acc[r] += o[r];
-        }
+    // two register sets alternate so that one tile's loads are in flight during the other's MFMAs
+    v4u w0[kSkinnySegs], w1[kSkinnySegs];
+    load_tile(tile0, w0);
+    for (uint32_t t = tile0; t < tile_end; t += 2) {
+        load_tile(t + 1, w1);
+        compute_tile(t, w0, 0);
+        load_tile(t + 2, w0);
+        if (t + 1 < tile_end) compute_tile(t + 1, w1, 1);
     }
-#pragma unroll
-    for (int r = 0; r < 4; ++r) acc[r] >>= 8;
-    const bool vec_ok = (EPI < 0) ? (p.N % 4 == 0 && reinterpret_cast<uintptr_t>(p.C) % 16 == 0)
-                                  : (p.N % 4 == 0 && reinterpret_cast<uintptr_t>(p.y) % 8 == 0);
-    store_quad<EPI, BIAS>(p, l16, n0 + g * 4, acc, vec_ok);
 }
 
 // ---------------------------------------------------------------------------------
@@ -741,17 +782,24 @@ static void launch_epi(GemmParams &p, hipStream_t stream)
         return;
     }
     if (p.M <= 16) {
-        const dim3 grid((p.N + 15) / 16);
+        const uint32_t ntiles = (p.N + 15) / 16;
         const uint32_t segs = (p.K / 2 + 63) / 64;
-        // enough wavefronts per workgroup that each walks about one unrolled step of K
-        if (segs <= 4 * kSkinnyUnroll)
+        // several column tiles per workgroup once there are plenty of them (activations are
+        // fetched and expanded once per workgroup); at least ~2 workgroups per CU stay
+        const uint32_t tpw = ntiles >= 1536 ? 4 : (ntiles >= 640 ? 2 : 1);
+        p.tiles_m = tpw;
+        const dim3 grid((ntiles + tpw - 1) / tpw);
+        if (segs <= 4 * kSkinnySegs)
             hipLaunchKernelGGL((gemm_s4_skinny_kernel<4, EPI, BIAS>), grid, dim3(256), 0, stream, p);
-        else if (segs <= 8 * kSkinnyUnroll)
+        else if (segs <= 8 * kSkinnySegs)
             hipLaunchKernelGGL((gemm_s4_skinny_kernel<8, EPI, BIAS>), grid, dim3(512), 0, stream, p);
-        else
+        else if (segs <= 16 * kSkinnySegs)
             hipLaunchKernelGGL((gemm_s4_skinny_kernel<16, EPI, BIAS>), grid, dim3(1024), 0, stream, p);
+        else
+            goto tiles_path;  // K above 16384: the tile kernels take it
         return;
     }
+tiles_path:
     // largest tile that still yields at least one workgroup per CU (256 CUs); small
     // problems take the small tile to spread over the chip.
     auto tiles = [&](uint32_t bm, uint32_t bn) { return ((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn); };

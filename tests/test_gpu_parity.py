@@ -130,7 +130,8 @@ def _rand_packed(rng, rows, K):
 @pytest.mark.parametrize("M,N,K", [
     (1, 16, 64), (1, 4096, 4096), (4, 4096, 4096), (16, 11008, 4096), (16, 40, 128), (7, 33, 192),
     (17, 64, 64), (64, 64, 128), (65, 130, 192), (100, 257, 320), (128, 256, 4096), (300, 520, 1024),
-    (2048, 4096, 256), (256, 4096, 11008), (130, 1000, 64), (16, 16, 8192), (2, 48, 28672),
+    (2048, 4096, 256), (256, 4096, 11008), (130, 1000, 64), (16, 16, 8192), (2, 48, 28672), (7, 48, 28672),
+    (9, 40000, 64), (16, 33000, 192), (12, 17000, 8192), (5, 100, 16384),
 ])
 def test_matmul_bit_exact(hip, dev, M, N, K):
     _say("matmul", M, N, K)
