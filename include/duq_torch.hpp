@@ -1,0 +1,266 @@
+// duq_torch.hpp - header-only libtorch (C++) twin of the Linear4bit path over the C ABI in
+// duq_hip.h, with the class and function names of the reference's C++ API:
+//   PackedQuantizedTensor, Quantizer4bit, DeQuantizer4bit, sym_quant, sym_dequant,
+//   sym_dual_dequant, pack_i4          include/quant_tensor.h:11-90, src/module/quant_tensor.cu
+//   Linear4bit, Linear4bitDUQ          include/linear.h:31-60,    src/module/linear.cu:83-281
+// Tensors live on a ROCm device ("cuda" device type in PyTorch-ROCm); every call launches on
+// torch's current HIP stream.  Argument errors raise c10::Error through TORCH_CHECK like the
+// reference's torch::check* calls; a non-zero status of the C ABI raises too.
+//
+// Build: hipcc / g++ with the libtorch include paths, -DUSE_ROCM -D__HIP_PLATFORM_AMD__, link
+// libduq_hip.so, libtorch, libc10, libc10_hip.
+#pragma once
+
+#include <torch/torch.h>
+
+#include <c10/hip/HIPStream.h>
+
+#include <tuple>
+#include <utility>
+#include <vector>
+
+#include "duq_hip.h"
+
+namespace duq {
+
+inline duq_stream_t current_stream(const torch::Tensor &t)
+{
+    return static_cast<duq_stream_t>(c10::hip::getCurrentHIPStream(t.device().index()).stream());
+}
+
+inline void check_status(int status, const char *what) { TORCH_CHECK(status == DUQ_OK, what, ": ", duq_status_string(status)); }
+
+inline void check_device_tensor(const torch::Tensor &t, const char *what, const char *name)
+{
+    TORCH_CHECK(t.is_contiguous(), what, ": expected ", name, " to be contiguous");
+    TORCH_CHECK(t.is_cuda(), what, ": expected ", name, " to be on a GPU device");
+}
+
+inline const duq_half *half_ptr(const torch::Tensor &t)
+{
+    TORCH_CHECK(t.scalar_type() == torch::kFloat16, "expected a float16 tensor");  // bf16 storage is rejected
+    return reinterpret_cast<const duq_half *>(t.data_ptr());
+}
+
+// [..., K] -> ([rows, K], leading sizes)
+inline std::pair<torch::Tensor, std::vector<int64_t>> flatten_last_dim_and_return_shape(const torch::Tensor &x)
+{
+    std::vector<int64_t> lead(x.sizes().begin(), x.sizes().end() - 1);
+    return {x.view({-1, x.size(-1)}), lead};
+}
+
+// ---- quantized activation (include/quant_tensor.h:11-27)
+class PackedQuantizedTensor {
+public:
+    torch::Tensor quantized_x;
+    torch::Tensor scale;
+    PackedQuantizedTensor(torch::Tensor quantized_x, torch::Tensor scale)
+        : quantized_x(std::move(quantized_x)), scale(std::move(scale)) {}
+    torch::IntArrayRef sizes() const { return quantized_x.sizes(); }
+    torch::Device device() const { return quantized_x.device(); }
+};
+
+// ---- tensor-level ops (src/module/quant_tensor.cu:11-148)
+inline torch::Tensor sym_quant(const torch::Tensor &x, const torch::Tensor &scale, int qmax = DUQ_QMAX_SYM_DEVICE)
+{
+    check_device_tensor(x, "sym_quant", "x");
+    check_device_tensor(scale, "sym_quant", "scale");
+    TORCH_CHECK(x.dim() == 2 && scale.size(0) == x.size(0), "sym_quant: expected scale to have size ", x.size(0), " at dimension 0");
+    const uint32_t rows = x.size(0), cols = x.size(1), cd = (cols + 1) / 2;
+    auto q = torch::empty({rows, cd}, torch::dtype(torch::kUInt8).device(x.device()));
+    check_status(duq_sym_quant_host_qmax(half_ptr(x), half_ptr(scale), rows, cols, cd, qmax, q.data_ptr<uint8_t>(),
+                                         current_stream(x)),
+                 "sym_quant");
+    return q;
+}
+
+inline torch::Tensor sym_dequant(const torch::Tensor &q, const torch::Tensor &scale_row, const torch::Tensor &scale_col, int bits)
+{
+    check_device_tensor(q, "sym_dequant", "q");
+    check_device_tensor(scale_row, "sym_dequant", "scale_row");
+    check_device_tensor(scale_col, "sym_dequant", "scale_col");
+    TORCH_CHECK(bits == 32, "Unsupported data type");  // src/module/quant_tensor.cu:93-96
+    TORCH_CHECK(q.scalar_type() == torch::kInt32 && q.dim() == 2, "sym_dequant: q must be int32 [rows, cols]");
+    const uint32_t rows = q.size(0), cols = q.size(1);
+    TORCH_CHECK(scale_row.size(0) == rows && scale_col.size(0) == cols, "sym_dequant: scale sizes do not match q");
+    auto x = torch::empty(q.sizes(), torch::dtype(torch::kHalf).device(q.device()));
+    check_status(duq_sym_dequant_host(q.data_ptr<int32_t>(), half_ptr(scale_row), half_ptr(scale_col), rows, cols,
+                                      reinterpret_cast<duq_half *>(x.data_ptr()), current_stream(q)),
+                 "sym_dequant");
+    return x;
+}
+
+inline torch::Tensor sym_dual_dequant(const torch::Tensor &q, const torch::Tensor &scale_row, const torch::Tensor &scale_col_1,
+                                      const torch::Tensor &scale_col_2, int bits)
+{
+    check_device_tensor(q, "sym_dual_dequant", "q");
+    TORCH_CHECK(bits == 32, "Unsupported data type");
+    TORCH_CHECK(q.scalar_type() == torch::kInt32 && q.dim() == 2, "sym_dual_dequant: q must be int32 [rows, cols]");
+    const uint32_t rows = q.size(0), cols = q.size(1);
+    TORCH_CHECK(scale_row.size(0) == rows && scale_col_1.size(0) == cols && scale_col_2.size(0) == cols,
+                "sym_dual_dequant: scale sizes do not match q");
+    auto x = torch::empty(q.sizes(), torch::dtype(torch::kHalf).device(q.device()));
+    check_status(duq_sym_dual_dequant_host(q.data_ptr<int32_t>(), half_ptr(scale_row), half_ptr(scale_col_1),
+                                           half_ptr(scale_col_2), rows, cols, reinterpret_cast<duq_half *>(x.data_ptr()),
+                                           current_stream(q)),
+                 "sym_dual_dequant");
+    return x;
+}
+
+// int4Unpack(A) @ int4Unpack(B)^T -> int32 (src/export/bindings.cpp:10-26)
+inline torch::Tensor matmul(const torch::Tensor &A, const torch::Tensor &B)
+{
+    check_device_tensor(A, "matmul", "A");
+    check_device_tensor(B, "matmul", "B");
+    TORCH_CHECK(A.dim() == 2 && B.dim() == 2 && A.size(1) == B.size(1), "matmul: packed K differs");
+    const uint32_t M = A.size(0), N = B.size(0), K = A.size(1) * 2;
+    auto C = torch::empty({M, N}, torch::dtype(torch::kInt32).device(A.device()));
+    check_status(duq_matmul_host_4bit(A.data_ptr<uint8_t>(), B.data_ptr<uint8_t>(), M, N, K, C.data_ptr<int32_t>(), current_stream(A)),
+                 "matmul");
+    return C;
+}
+
+// signed integer tensor [rows, K] with values in [-8, 7] -> uint8 [rows, K/2] (quant_tensor.cu:197-206)
+inline torch::Tensor pack_i4(const torch::Tensor &q)
+{
+    TORCH_CHECK(q.dim() == 2 && q.size(1) % 2 == 0, "pack_i4: expected [rows, even K]");
+    TORCH_CHECK(torch::all(q.ge(-8).logical_and(q.le(7))).item<bool>(), "pack_i4: value outside the int4 range");
+    auto codes = torch::where(q < 0, q + 16, q).to(torch::kUInt8);
+    using torch::indexing::Slice;
+    return codes.index({Slice(), Slice(0, torch::indexing::None, 2)}) |
+           (codes.index({Slice(), Slice(1, torch::indexing::None, 2)}) * 16);
+}
+
+// ---- modules
+// Per-token symmetric quantizer, one fused kernel (src/module/quant_tensor.cu:151-161)
+class Quantizer4bit : public torch::nn::Module {
+public:
+    float input_clip_ratio;
+    int qmax;
+    explicit Quantizer4bit(float input_clip_ratio, int qmax = DUQ_QMAX_SYM_DEVICE) : input_clip_ratio(input_clip_ratio), qmax(qmax) {}
+    PackedQuantizedTensor forward(torch::Tensor x)
+    {
+        x = x.contiguous();
+        check_device_tensor(x, "Quantizer4bit::forward", "x");
+        auto [x2, lead] = flatten_last_dim_and_return_shape(x);
+        const uint32_t rows = x2.size(0), cols = x2.size(1);
+        TORCH_CHECK(cols % 32 == 0, "Quantizer4bit::forward: the last dimension must be a multiple of 32");
+        auto q = torch::empty({rows, cols / 2}, torch::dtype(torch::kUInt8).device(x.device()));
+        auto s = torch::empty({rows, 1}, torch::dtype(torch::kHalf).device(x.device()));
+        check_status(duq_quantize_rows_sym(half_ptr(x2), rows, cols, input_clip_ratio, qmax, q.data_ptr<uint8_t>(),
+                                           reinterpret_cast<duq_half *>(s.data_ptr()), current_stream(x)),
+                     "Quantizer4bit::forward");
+        auto qshape = lead;
+        qshape.push_back(cols / 2);
+        auto sshape = lead;
+        sshape.push_back(1);
+        return PackedQuantizedTensor(q.view(qshape), s.view(sshape));
+    }
+};
+
+class DeQuantizer4bit : public torch::nn::Module {
+public:
+    uint32_t bits = 32;
+    DeQuantizer4bit() {}
+    explicit DeQuantizer4bit(uint32_t bits) : bits(bits) {}
+    torch::Tensor forward(torch::Tensor &x, torch::Tensor &scale_x, torch::Tensor &weight_scale)
+    {
+        return sym_dequant(x, scale_x.view(-1), weight_scale, static_cast<int>(bits));
+    }
+};
+
+namespace detail {
+inline torch::Tensor fused_forward(int mode, const PackedQuantizedTensor &input, const torch::Tensor &weight,
+                                   const torch::Tensor &s1, const torch::Tensor &s2, const torch::Tensor &bias)
+{
+    const torch::Tensor &x = input.quantized_x;
+    TORCH_CHECK(x.size(-1) % 32 == 0, "packed activation width must be a multiple of 32 bytes");  // linear.cu:115
+    auto [A, lead] = flatten_last_dim_and_return_shape(x);
+    check_device_tensor(A, "Linear4bit::forward", "A");
+    check_device_tensor(weight, "Linear4bit::forward", "B");
+    TORCH_CHECK(A.device() == weight.device(), "Linear4bit::forward: operands on different devices");
+    const uint32_t M = A.size(0), N = weight.size(0), K = A.size(1) * 2;
+    TORCH_CHECK(weight.size(1) == A.size(1), "Linear4bit::forward: packed K differs");
+    auto scale_row = input.scale.contiguous().view(-1);
+    TORCH_CHECK(scale_row.size(0) == M, "Linear4bit::forward: one activation scale per token expected");
+    auto y = torch::empty({M, N}, torch::dtype(torch::kHalf).device(A.device()));
+    check_status(duq_linear4bit_forward(mode, A.data_ptr<uint8_t>(), half_ptr(scale_row), nullptr, weight.data_ptr<uint8_t>(),
+                                        half_ptr(s1), nullptr, s2.defined() ? half_ptr(s2) : nullptr, nullptr,
+                                        bias.defined() ? half_ptr(bias) : nullptr, M, N, K,
+                                        reinterpret_cast<duq_half *>(y.data_ptr()), current_stream(A)),
+                 "Linear4bit::forward");
+    lead.push_back(N);
+    return y.view(lead);
+}
+}  // namespace detail
+
+// Symmetric 4-bit linear layer (include/linear.h:31-45, src/module/linear.cu:83-176)
+class Linear4bit : public torch::nn::Module {
+public:
+    torch::Tensor weight;        // uint8 [out, in/2]
+    torch::Tensor weight_scale;  // fp16 [out, 1]
+    torch::Tensor bias;          // fp16 [out] or undefined
+
+    Linear4bit(uint32_t input_dim, uint32_t output_dim, bool use_bias, torch::Dtype dtype = torch::kFloat16)
+    {
+        weight = torch::zeros({output_dim, input_dim / 2}, torch::dtype(torch::kUInt8).device(torch::kCUDA));
+        weight_scale = torch::zeros({output_dim, 1}, torch::dtype(dtype).device(torch::kCUDA));
+        if (use_bias) bias = torch::zeros({output_dim}, torch::dtype(dtype).device(torch::kCUDA));
+    }
+
+    torch::Tensor forward(PackedQuantizedTensor input)
+    {
+        return detail::fused_forward(DUQ_EPI_SYM, input, weight, weight_scale.view(-1), torch::Tensor(), bias);
+    }
+
+    // round(W / weight_scales) packed to nibbles (src/module/linear.cu:161-176)
+    static Linear4bit from_float(torch::nn::Linear &linear, torch::Tensor weight_scales)
+    {
+        auto w = linear->weight.detach().to(torch::kCUDA);
+        Linear4bit out(w.size(1), w.size(0), linear->bias.defined(), w.scalar_type());
+        TORCH_CHECK(weight_scales.dim() == 2 && weight_scales.size(0) == w.size(0) && weight_scales.size(1) == 1,
+                    "weight_scales should have shape (out_features, 1)");
+        out.weight_scale.copy_(weight_scales.to(w.scalar_type()));
+        out.weight.copy_(pack_i4((w / weight_scales.to(w.device())).round().to(torch::kInt8)));
+        if (linear->bias.defined()) out.bias.copy_(linear->bias.detach());
+        return out;
+    }
+};
+
+// Dual-uniform variant: output columns < 10 use weight_scale_1 (include/linear.h:48-60, linear.cu:178-281)
+class Linear4bitDUQ : public torch::nn::Module {
+public:
+    torch::Tensor weight;
+    torch::Tensor weight_scale_1;
+    torch::Tensor weight_scale_2;
+    torch::Tensor bias;
+
+    Linear4bitDUQ(uint32_t input_dim, uint32_t output_dim, bool use_bias, torch::Dtype dtype = torch::kFloat16)
+    {
+        weight = torch::zeros({output_dim, input_dim / 2}, torch::dtype(torch::kUInt8).device(torch::kCUDA));
+        weight_scale_1 = torch::zeros({output_dim, 1}, torch::dtype(dtype).device(torch::kCUDA));
+        weight_scale_2 = torch::zeros({output_dim, 1}, torch::dtype(dtype).device(torch::kCUDA));
+        if (use_bias) bias = torch::zeros({output_dim}, torch::dtype(dtype).device(torch::kCUDA));
+    }
+
+    torch::Tensor forward(PackedQuantizedTensor input)
+    {
+        return detail::fused_forward(DUQ_EPI_SYM_DUAL, input, weight, weight_scale_1.view(-1), weight_scale_2.view(-1), bias);
+    }
+
+    static Linear4bitDUQ from_float(torch::nn::Linear &linear, torch::Tensor weight_scales_1, torch::Tensor weight_scales_2)
+    {
+        auto w = linear->weight.detach().to(torch::kCUDA);
+        Linear4bitDUQ out(w.size(1), w.size(0), linear->bias.defined(), w.scalar_type());
+        out.weight_scale_1.copy_(weight_scales_1.to(w.scalar_type()));
+        out.weight_scale_2.copy_(weight_scales_2.to(w.scalar_type()));
+        const int64_t split = duq_get_dual_quant_col_k();
+        auto left = (w.slice(1, 0, split) / weight_scales_1.to(w.device())).round();
+        auto right = (w.slice(1, split) / weight_scales_2.to(w.device())).round();
+        out.weight.copy_(pack_i4(torch::cat({left, right}, 1).to(torch::kInt8)));
+        if (linear->bias.defined()) out.bias.copy_(linear->bias.detach());
+        return out;
+    }
+};
+
+}  // namespace duq

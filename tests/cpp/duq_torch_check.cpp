@@ -1,0 +1,66 @@
+// Runs the libtorch classes of include/duq_torch.hpp on the current GPU and checks the fused
+// Linear4bit / Linear4bitDUQ forwards against the three-step path (matmul, dequant, bias add)
+// built from the same header, bit for bit.  Prints "OK <checksum>" and exits 0 on success.
+#include <cstdio>
+#include <cstdlib>
+
+#include "duq_torch.hpp"
+
+static bool same_bits(const torch::Tensor &a, const torch::Tensor &b)
+{
+    return a.sizes() == b.sizes() && torch::equal(a.contiguous().view(torch::kInt16), b.contiguous().view(torch::kInt16));
+}
+
+int main(int argc, char **argv)
+{
+    const int64_t M = argc > 1 ? atoll(argv[1]) : 48, K = argc > 2 ? atoll(argv[2]) : 256, N = argc > 3 ? atoll(argv[3]) : 192;
+    torch::manual_seed(1234);
+    auto dev = torch::Device(torch::kCUDA, 0);
+    auto x = (torch::randn({3, M / 3, K}, torch::dtype(torch::kFloat32).device(dev)) * 1.5).to(torch::kHalf);
+
+    torch::nn::Linear lin(torch::nn::LinearOptions(K, N).bias(true));
+    lin->to(dev, torch::kHalf);
+    auto w = lin->weight.detach();
+    auto ws = (w.abs().amax(1, true).to(torch::kFloat32) / 7.0).to(torch::kHalf);
+
+    duq::Quantizer4bit quant(1.0f);
+    auto p = quant.forward(x);
+    if (p.quantized_x.size(-1) != K / 2 || p.scale.size(-1) != 1 || p.scale.dim() != 3) { std::puts("FAIL quantizer shapes"); return 1; }
+
+    // scale = h(h(max|x| / 7) * clip) with clip = 1, exact in float then rounded once
+    auto want_scale = (x.abs().amax(-1, true).to(torch::kFloat32) / 7.0).to(torch::kHalf);
+    if (!same_bits(p.scale, want_scale)) { std::puts("FAIL quantizer scale"); return 1; }
+    // the packed codes must be what sym_quant gives for that scale
+    auto q2 = duq::sym_quant(x.view({-1, K}), p.scale.view(-1));
+    if (!torch::equal(q2, p.quantized_x.view({-1, K / 2}))) { std::puts("FAIL quantizer codes"); return 1; }
+
+    auto l = duq::Linear4bit::from_float(lin, ws);
+    auto y = l.forward(p);
+    auto acc = duq::matmul(p.quantized_x.view({-1, K / 2}), l.weight);
+    auto y3 = (duq::sym_dequant(acc, p.scale.view(-1), l.weight_scale.view(-1), 32) + l.bias).view({3, M / 3, N});
+    if (!same_bits(y, y3)) { std::puts("FAIL Linear4bit fused vs three-step"); return 1; }
+
+    // close to the fp16 layer it replaces (4-bit error, loose bound) - guards against a transposed operand
+    auto yref = lin->forward(x).to(torch::kFloat32);
+    auto rel = ((y.to(torch::kFloat32) - yref).norm() / yref.norm()).item<float>();
+    if (!(rel < 0.35f)) { std::printf("FAIL Linear4bit vs fp16 layer: rel %.3f\n", rel); return 1; }
+
+    auto ws1 = (w.slice(1, 0, 10).abs().amax(1, true).to(torch::kFloat32) / 7.0).to(torch::kHalf);
+    auto d = duq::Linear4bitDUQ::from_float(lin, ws1, ws);
+    auto yd = d.forward(p);
+    auto yd3 = (duq::sym_dual_dequant(acc.copy_(duq::matmul(p.quantized_x.view({-1, K / 2}), d.weight)), p.scale.view(-1),
+                                      d.weight_scale_1.view(-1), d.weight_scale_2.view(-1), 32) +
+                d.bias).view({3, M / 3, N});
+    if (!same_bits(yd, yd3)) { std::puts("FAIL Linear4bitDUQ fused vs three-step"); return 1; }
+
+    bool threw = false;
+    try { duq::sym_dequant(acc, p.scale.view(-1), l.weight_scale.view(-1), 16); } catch (const c10::Error &) { threw = true; }
+    if (!threw) { std::puts("FAIL bits != 32 accepted"); return 1; }
+    threw = false;
+    try { quant.forward(x.to(torch::kBFloat16)); } catch (const c10::Error &) { threw = true; }
+    if (!threw) { std::puts("FAIL bf16 accepted"); return 1; }
+
+    torch::cuda::synchronize();
+    std::printf("OK %.6f rel %.4f\n", y.to(torch::kFloat32).abs().sum().item<float>(), rel);
+    return 0;
+}

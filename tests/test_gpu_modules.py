@@ -252,3 +252,17 @@ def test_runs_on_a_side_stream(qnn, dev):
         y = lin(qnn.SymQuantizer(1.0)(xt))
     side.synchronize()
     assert cases.bits_equal(y.cpu().numpy(), want)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(48, 256, 192), (6, 4096, 512), (384, 1024, 1024)])
+def test_libtorch_classes_fused_equals_three_step(shape):
+    """The C++ classes of include/duq_torch.hpp (twin of the reference's include/linear.h and
+    include/quant_tensor.h) run in a stand-alone libtorch program: fused forward == matmul +
+    dequant + bias bit for bit, quantizer scale/codes as specified, error paths raise."""
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpp", "duq_torch_check")
+    assert os.path.exists(exe), "tests/cpp/duq_torch_check is not built (run build())"
+    r = subprocess.run([exe] + [str(v) for v in shape], capture_output=True, text=True, timeout=100)
+    assert r.returncode == 0 and r.stdout.startswith("OK"), (r.returncode, r.stdout[-2000:], r.stderr[-2000:])

@@ -186,3 +186,29 @@ def test_reference_package_name_is_importable():
     for name in ("matmul", "sym_quant", "sym_dual_quant", "sym_dequant", "sym_dual_dequant", "asym_quant",
                  "asym_dequant", "asym_dual_quant", "asym_dual_dequant", "get_dual_quant_col_k"):
         assert callable(getattr(ops, name)), name       # the op names of src/export/bindings.cpp:772-923
+
+
+def test_libtorch_header_compiles_against_the_c_abi(tmp_path):
+    """include/duq_torch.hpp (the C++ twin of include/linear.h / include/quant_tensor.h of the
+    reference) must parse and type-check against libtorch's headers and duq_hip.h."""
+    import shutil
+    if shutil.which("g++") is None:
+        pytest.skip("no host C++ compiler")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    tinc = os.path.join(os.path.dirname(torch.__file__), "include")
+    if not os.path.exists(os.path.join(tinc, "c10", "hip", "HIPStream.h")):
+        pytest.skip("libtorch was built without ROCm headers")
+    src = tmp_path / "use_duq_torch.cpp"
+    src.write_text(
+        '#include "duq_torch.hpp"\n'
+        "torch::Tensor run(torch::Tensor x, duq::Linear4bit &l, duq::Linear4bitDUQ &d) {\n"
+        "    duq::Quantizer4bit q(1.0f);\n"
+        "    auto p = q.forward(x);\n"
+        "    return l.forward(p) + d.forward(p) + duq::sym_dequant(duq::matmul(p.quantized_x, l.weight),\n"
+        "        p.scale.view(-1), l.weight_scale.view(-1), 32);\n"
+        "}\n")
+    cmd = ["g++", "-std=c++17", "-fsyntax-only", "-DUSE_ROCM", "-D__HIP_PLATFORM_AMD__",
+           "-I", os.path.join(root, "include"), "-I", tinc,
+           "-I", os.path.join(tinc, "torch", "csrc", "api", "include"), "-I", "/opt/rocm/include", str(src)]
+    r = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-3000:]
