@@ -169,12 +169,13 @@ int launch_asym_dual_quant(const uint16_t *x, const uint16_t *s1, const uint16_t
 // ---------------------------------------------------------------------------------
 // fused row kernels: scale (and zero) + quantize in one pass over x
 // ---------------------------------------------------------------------------------
-// A row of `cols` elements is split into groups of 32 (four 128-bit loads, one 128-bit
-// store).  WAVES wavefronts share one row; lane t owns groups t, t+T, t+2T, ... (T =
-// 64*WAVES) and keeps up to MAXG of them in registers between the reduction and the
-// quantization, so x is read from HBM exactly once.  Rows longer than 32*MAXG*T elements
-// run the same code with CACHED = false: the groups are read a second time (from L2).
-constexpr int kMaxGroups = 2;  // 2 groups = 64 elements = 32 VGPRs of row data per lane
+// A row of `cols` elements is split into units of 8 (one 128-bit load, one 32-bit store).
+// WAVES wavefronts share one row; lane t owns units t, t+T, t+2T, ... (T = 64*WAVES), so
+// every load and store instruction of a wavefront covers one contiguous 1 KB / 256 B span,
+// and keeps up to kMaxUnits of them in registers between the reduction and the
+// quantization: x is read from HBM exactly once.  Rows longer than 8*kMaxUnits*T elements
+// run the same code with CACHED = false: the units are read a second time (from L2).
+constexpr int kMaxUnits = 8;  // 64 elements = 32 VGPRs of row data per lane
 
 struct RowParams {
     const uint16_t *x;
@@ -200,53 +201,40 @@ __global__ __launch_bounds__(WAVES * 64) void quantize_rows_kernel(RowParams p)
     __shared__ float red[2][WAVES];
     const uint32_t row = blockIdx.x;
     const uint32_t tid = threadIdx.x;
-    const uint32_t ngroups = p.cols >> 5;  // groups of 32 elements
+    const uint32_t nunits = p.cols >> 3;  // units of 8 elements
     const v4u *xrow = reinterpret_cast<const v4u *>(p.x + (uint64_t)row * p.cols);
-    v4u *qrow = reinterpret_cast<v4u *>(p.q + (uint64_t)row * (p.cols >> 1));
+    uint32_t *qrow = reinterpret_cast<uint32_t *>(p.q + (uint64_t)row * (p.cols >> 1));
 
-    v4u regs[kMaxGroups][4];
+    v4u regs[kMaxUnits];
     uint32_t amax = 0;        // sym: packed max of |x| bit patterns (NaN patterns win, as in torch.max)
     float fmin_ = INFINITY;   // asym
     float fmax_ = -INFINITY;
 
-    auto reduce_group = [&](const v4u(&g)[4]) {
+    auto reduce_unit = [&](const v4u &g) {
 #pragma unroll
-        for (int v = 0; v < 4; ++v)
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                if (!ASYM) {
-                    amax = pk_absmax_u16(amax, g[v][w]);
-                } else {
-                    const float lo = (float)bits_to_f16((uint16_t)(g[v][w] & 0xFFFFu));
-                    const float hi = (float)bits_to_f16((uint16_t)(g[v][w] >> 16));
-                    fmin_ = fminf(fmin_, fminf(lo, hi));
-                    fmax_ = fmaxf(fmax_, fmaxf(lo, hi));
-                }
+        for (int w = 0; w < 4; ++w) {
+            if (!ASYM) {
+                amax = pk_absmax_u16(amax, g[w]);
+            } else {
+                const float lo = (float)bits_to_f16((uint16_t)(g[w] & 0xFFFFu));
+                const float hi = (float)bits_to_f16((uint16_t)(g[w] >> 16));
+                fmin_ = fminf(fmin_, fminf(lo, hi));
+                fmax_ = fmaxf(fmax_, fmaxf(lo, hi));
             }
+        }
     };
 
     if (CACHED) {
 #pragma unroll
-        for (int i = 0; i < kMaxGroups; ++i) {
-            const uint32_t g = tid + i * T;
-            if (g < ngroups) {
-#pragma unroll
-                for (int v = 0; v < 4; ++v) regs[i][v] = __builtin_nontemporal_load(&xrow[g * 4 + v]);
-            } else {
-#pragma unroll
-                for (int v = 0; v < 4; ++v) regs[i][v] = v4u{0u, 0u, 0u, 0u};
-            }
+        for (int i = 0; i < kMaxUnits; ++i) {
+            const uint32_t u = tid + i * T;
+            regs[i] = u < nunits ? __builtin_nontemporal_load(&xrow[u]) : v4u{0u, 0u, 0u, 0u};
         }
 #pragma unroll
-        for (int i = 0; i < kMaxGroups; ++i)
-            if (tid + i * T < ngroups) reduce_group(regs[i]);
+        for (int i = 0; i < kMaxUnits; ++i)
+            if (tid + i * T < nunits) reduce_unit(regs[i]);
     } else {
-        for (uint32_t g = tid; g < ngroups; g += T) {
-            v4u tmp[4];
-#pragma unroll
-            for (int v = 0; v < 4; ++v) tmp[v] = xrow[g * 4 + v];
-            reduce_group(tmp);
-        }
+        for (uint32_t u = tid; u < nunits; u += T) reduce_unit(xrow[u]);
     }
 
     // ---- row reduction: shuffles inside a wavefront, one LDS hop across wavefronts ----
@@ -350,33 +338,20 @@ __global__ __launch_bounds__(WAVES * 64) void quantize_rows_kernel(RowParams p)
         return __builtin_amdgcn_perm(t1, t0, 0x06040200u);
     };
 
-    // ---- quantize + pack: 32 elements -> one 128-bit store ----
-    auto quant_group = [&](const v4u(&g)[4]) {
-        v4u out;
-        if (fast) {
-#pragma unroll
-            for (int v = 0; v < 4; ++v) out[v] = quant8_fast(g[v]);
-        } else {
-#pragma unroll
-            for (int v = 0; v < 4; ++v)
-                out[v] = ASYM ? quant8<kAsym>(g[v], 0, rcp, 0.f, 15, zi, (f16)0, (f16)0)
-                              : quant8<kSym>(g[v], 0, rcp, 0.f, p.qmax, 0, (f16)0, (f16)0);
-        }
-        return out;
+    // ---- quantize + pack: 8 elements -> one 32-bit store ----
+    auto quant_unit = [&](const v4u &g) -> uint32_t {
+        if (fast) return quant8_fast(g);
+        return ASYM ? quant8<kAsym>(g, 0, rcp, 0.f, 15, zi, (f16)0, (f16)0)
+                    : quant8<kSym>(g, 0, rcp, 0.f, p.qmax, 0, (f16)0, (f16)0);
     };
     if (CACHED) {
 #pragma unroll
-        for (int i = 0; i < kMaxGroups; ++i) {
-            const uint32_t g = tid + i * T;
-            if (g < ngroups) qrow[g] = quant_group(regs[i]);
+        for (int i = 0; i < kMaxUnits; ++i) {
+            const uint32_t u = tid + i * T;
+            if (u < nunits) qrow[u] = quant_unit(regs[i]);
         }
     } else {
-        for (uint32_t g = tid; g < ngroups; g += T) {
-            v4u tmp[4];
-#pragma unroll
-            for (int v = 0; v < 4; ++v) tmp[v] = xrow[g * 4 + v];
-            qrow[g] = quant_group(tmp);
-        }
+        for (uint32_t u = tid; u < nunits; u += T) qrow[u] = quant_unit(xrow[u]);
     }
 }
 
@@ -384,15 +359,20 @@ template <bool ASYM>
 static int launch_rows(const RowParams &p, hipStream_t stream)
 {
     if (p.rows == 0 || p.cols == 0) return 0;
-    const uint32_t ngroups = p.cols / 32;
+    const uint32_t nunits = p.cols / 8;
     const dim3 grid(p.rows);
-    // fewest wavefronts per row that still keep the whole row in registers; short rows use
-    // one wavefront, and few-row (decode) calls spread one row over more lanes for latency.
-    int waves = 1;
-    while (waves < 16 && (uint32_t)(waves * 64 * kMaxGroups) < ngroups) waves *= 2;
-    if (p.rows <= 64)
-        while (waves < 4 && (uint32_t)(waves * 64) < ngroups) waves *= 2;
-    const bool cached = (uint32_t)(waves * 64 * kMaxGroups) >= ngroups;
+    // Wavefronts per row: enough that a lane holds at most `per_lane` units.  Four units per
+    // lane stream best when the grid is large; smaller grids are latency-bound and spread a
+    // row over more lanes (2, then 1 unit each) to shorten every lane's serial work.
+    auto waves_for = [&](uint32_t per_lane) {
+        uint32_t w = 1;
+        while (w < 16 && w * 64 * per_lane < nunits) w *= 2;
+        return w;
+    };
+    uint32_t waves = waves_for(4);
+    if ((uint64_t)p.rows * waves < 2048) waves = waves_for(2);
+    if ((uint64_t)p.rows * waves < 512) waves = waves_for(1);
+    const bool cached = waves * 64 * kMaxUnits >= nunits;
 #define DUQ_ROWS_CASE(W)                                                                                     \
     case W:                                                                                                  \
         if (cached)                                                                                          \
