@@ -785,8 +785,14 @@ static void launch_epi(GemmParams &p, hipStream_t stream)
         const uint32_t ntiles = (p.N + 15) / 16;
         const uint32_t segs = (p.K / 2 + 63) / 64;
         // several column tiles per workgroup once there are plenty of them (activations are
-        // fetched and expanded once per workgroup); at least ~2 workgroups per CU stay
-        const uint32_t tpw = ntiles >= 1536 ? 4 : (ntiles >= 640 ? 2 : 1);
+        // fetched and expanded once per workgroup); at least ~2 workgroups per CU stay.
+        // Long rows (8+ wavefronts per workgroup, one workgroup per CU): size the grid to
+        // whole rounds of 256 workgroups, at most 8 tiles each.
+        uint32_t tpw = ntiles >= 6144 ? 8 : (ntiles >= 1536 ? 4 : (ntiles >= 640 ? 2 : 1));
+        if (segs > 4 * kSkinnySegs && ntiles >= 512) {
+            const uint32_t rounds = (ntiles + 2047) / 2048;
+            tpw = (ntiles + 256 * rounds - 1) / (256 * rounds);
+        }
         p.tiles_m = tpw;
         const dim3 grid((ntiles + tpw - 1) / tpw);
         if (segs <= 4 * kSkinnySegs)
