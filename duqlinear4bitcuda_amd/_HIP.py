@@ -19,6 +19,28 @@ def _stream(t: torch.Tensor):
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
+_raw_stream = torch._C._cuda_getCurrentRawStream  # (device index) -> hipStream_t as int; no Stream object built
+_F16, _U8 = torch.float16, torch.uint8
+
+
+def _launch(dev: torch.device, fn, *args):
+    """Call ``fn(*args, stream)`` with ``dev`` current, on its current torch stream.  The
+    device guard is only entered when another device is current."""
+    idx = dev.index
+    if idx == torch._C._cuda_getDevice():
+        return fn(*args, _raw_stream(idx))
+    with torch.cuda.device(idx):
+        return fn(*args, _raw_stream(idx))
+
+
+def _fast_check(name, what, t, dtype, dev):
+    """Contiguity / device / dtype check of one tensor of a fused op."""
+    if t.dtype is not dtype or not t.is_cuda or not t.is_contiguous() or (dev is not None and t.device != dev):
+        _check(name, t)
+        _check_dtype(name, t, what, dtype)
+        raise RuntimeError(f"{name}: expected all tensors on {dev}, {what} is on {t.device}")
+
+
 def _check(name, *tensors):
     dev = None
     for i, t in enumerate(tensors):
@@ -226,31 +248,44 @@ def get_dual_quant_col_k() -> int:
 # ---- additions over the reference module: fused ops -----------------------------------
 
 def quantize_rows_sym(x: torch.Tensor, clip: float = 1.0, qmax: int = 6):
-    """One-pass SymQuantizer (qlinear4bit/nn/quantizer.py:10-16): returns (q uint8 [M,K/2],
-    scales fp16 [M,1]).  Requires K % 32 == 0."""
-    _check("quantize_rows_sym", x)
-    _check_dtype("quantize_rows_sym", x, "x", torch.float16)
-    rows, cols = x.size(0), x.size(1)
-    q = torch.empty((rows, cols // 2), dtype=torch.uint8, device=x.device)
-    s = torch.empty((rows, 1), dtype=torch.float16, device=x.device)
-    with torch.cuda.device(x.device):
-        st = _lib.load().duq_quantize_rows_sym(_ptr(x), rows, cols, float(clip), qmax, _ptr(q), _ptr(s), _stream(x))
-    _lib.check(st, "quantize_rows_sym")
+    """One-pass SymQuantizer (qlinear4bit/nn/quantizer.py:10-16) over the last dimension of a
+    contiguous fp16 tensor [..., K]: returns (q uint8 [..., K/2], scales fp16 [..., 1]).
+    Requires K % 32 == 0."""
+    if not isinstance(x, torch.Tensor):
+        raise RuntimeError("quantize_rows_sym: argument #0 is not a tensor")
+    _fast_check("quantize_rows_sym", "x", x, _F16, None)
+    shape = x.shape
+    cols = shape[-1]
+    rows = x.numel() // cols if cols else 0
+    lead = shape[:-1]
+    dev = x.device
+    q = torch.empty(lead + (cols // 2,), dtype=_U8, device=dev)
+    s = torch.empty(lead + (1,), dtype=_F16, device=dev)
+    st = _launch(dev, _lib.load().duq_quantize_rows_sym, x.data_ptr(), rows, cols, float(clip), qmax, q.data_ptr(),
+                 s.data_ptr())
+    if st:
+        _lib.check(st, "quantize_rows_sym")
     return q, s
 
 
 def quantize_rows_asym(x: torch.Tensor):
-    """One-pass AsymQuantizer (qlinear4bit/nn/quantizer.py:24-35): returns (q, scale [M,1],
-    zeros [M,1]).  Requires K % 32 == 0."""
-    _check("quantize_rows_asym", x)
-    _check_dtype("quantize_rows_asym", x, "x", torch.float16)
-    rows, cols = x.size(0), x.size(1)
-    q = torch.empty((rows, cols // 2), dtype=torch.uint8, device=x.device)
-    s = torch.empty((rows, 1), dtype=torch.float16, device=x.device)
-    z = torch.empty((rows, 1), dtype=torch.float16, device=x.device)
-    with torch.cuda.device(x.device):
-        st = _lib.load().duq_quantize_rows_asym(_ptr(x), rows, cols, _ptr(q), _ptr(s), _ptr(z), _stream(x))
-    _lib.check(st, "quantize_rows_asym")
+    """One-pass AsymQuantizer (qlinear4bit/nn/quantizer.py:24-35) over the last dimension:
+    returns (q, scale [..., 1], zeros [..., 1]).  Requires K % 32 == 0."""
+    if not isinstance(x, torch.Tensor):
+        raise RuntimeError("quantize_rows_asym: argument #0 is not a tensor")
+    _fast_check("quantize_rows_asym", "x", x, _F16, None)
+    shape = x.shape
+    cols = shape[-1]
+    rows = x.numel() // cols if cols else 0
+    lead = shape[:-1]
+    dev = x.device
+    q = torch.empty(lead + (cols // 2,), dtype=_U8, device=dev)
+    s = torch.empty(lead + (1,), dtype=_F16, device=dev)
+    z = torch.empty(lead + (1,), dtype=_F16, device=dev)
+    st = _launch(dev, _lib.load().duq_quantize_rows_asym, x.data_ptr(), rows, cols, q.data_ptr(), s.data_ptr(),
+                 z.data_ptr())
+    if st:
+        _lib.check(st, "quantize_rows_asym")
     return q, s, z
 
 
@@ -260,28 +295,45 @@ EPI_SYM, EPI_ASYM, EPI_SYM_DUAL, EPI_ASYM_DUAL = 0, 1, 2, 3
 def linear4bit_forward(mode, xq, scale_x, zeros_x, w, w_scale_1, w_zeros_1=None, w_scale_2=None, w_zeros_2=None,
                        bias=None):
     """matmul + dequant (+ bias) in one launch; bit-identical to the separate ops.
-    All tensors 2-D / 1-D-viewable and contiguous; returns fp16 [M, N]."""
-    present = [t for t in (xq, scale_x, zeros_x, w, w_scale_1, w_zeros_1, w_scale_2, w_zeros_2, bias) if t is not None]
-    _check("linear4bit_forward", *present)
-    _check_dtype("linear4bit_forward", xq, "xq", torch.uint8)
-    _check_dtype("linear4bit_forward", w, "w", torch.uint8)
-    for t in present:
-        if t is not xq and t is not w:
-            _check_dtype("linear4bit_forward", t, "scale/zero/bias", torch.float16)
-    M, N, K = xq.size(0), w.size(0), xq.size(1) * 2
-    if w.size(1) != xq.size(1):
-        raise RuntimeError(f"linear4bit_forward: packed K differs: x {tuple(xq.shape)} vs w {tuple(w.shape)}")
-    _check_size0("linear4bit_forward", scale_x.view(-1), "scale_x", M)
-    for t, n in ((w_scale_1, "w_scale_1"), (w_zeros_1, "w_zeros_1"), (w_scale_2, "w_scale_2"),
-                 (w_zeros_2, "w_zeros_2"), (bias, "bias")):
-        if t is not None:
-            _check_size0("linear4bit_forward", t.view(-1), n, N)
+    ``xq`` is uint8 [..., K/2] (leading dimensions are flattened to M rows), ``w`` uint8
+    [N, K/2]; per-row tensors hold M, per-column tensors N fp16 values in any contiguous
+    shape.  Returns fp16 [..., N]."""
+    name = "linear4bit_forward"
+    if not isinstance(xq, torch.Tensor) or not isinstance(w, torch.Tensor):
+        raise RuntimeError(f"{name}: xq and w must be tensors")
+    dev = xq.device
+    _fast_check(name, "xq", xq, _U8, None)
+    _fast_check(name, "w", w, _U8, dev)
+    kb = xq.shape[-1]
+    if w.dim() != 2 or w.shape[1] != kb:
+        raise RuntimeError(f"{name}: packed K differs: x {tuple(xq.shape)} vs w {tuple(w.shape)}")
+    M = xq.numel() // kb if kb else 0
+    N = w.shape[0]
+    _fast_check(name, "scale_x", scale_x, _F16, dev)
+    if scale_x.numel() != M:
+        _check_size0(name, scale_x.reshape(-1), "scale_x", M)
+    pz = 0
     if zeros_x is not None:
-        _check_size0("linear4bit_forward", zeros_x.view(-1), "zeros_x", M)
-    y = torch.empty((M, N), dtype=torch.float16, device=xq.device)
-    with torch.cuda.device(xq.device):
-        st = _lib.load().duq_linear4bit_forward(mode, _ptr(xq), _ptr(scale_x), _ptr(zeros_x), _ptr(w), _ptr(w_scale_1),
-                                                _ptr(w_zeros_1), _ptr(w_scale_2), _ptr(w_zeros_2), _ptr(bias), M, N, K,
-                                                _ptr(y), _stream(xq))
-    _lib.check(st, "linear4bit_forward")
+        _fast_check(name, "zeros_x", zeros_x, _F16, dev)
+        if zeros_x.numel() != M:
+            _check_size0(name, zeros_x.reshape(-1), "zeros_x", M)
+        pz = zeros_x.data_ptr()
+    _fast_check(name, "w_scale_1", w_scale_1, _F16, dev)
+    if w_scale_1.numel() != N:
+        _check_size0(name, w_scale_1.reshape(-1), "w_scale_1", N)
+    ptrs = [0, 0, 0, 0]
+    if w_zeros_1 is not None or w_scale_2 is not None or w_zeros_2 is not None or bias is not None:
+        for k, (t, what) in enumerate(((w_zeros_1, "w_zeros_1"), (w_scale_2, "w_scale_2"), (w_zeros_2, "w_zeros_2"),
+                                       (bias, "bias"))):
+            if t is not None:
+                _fast_check(name, what, t, _F16, dev)
+                if t.numel() != N:
+                    _check_size0(name, t.reshape(-1), what, N)
+                ptrs[k] = t.data_ptr()
+    y = torch.empty(xq.shape[:-1] + (N,), dtype=_F16, device=dev)
+    st = _launch(dev, _lib.load().duq_linear4bit_forward, mode, xq.data_ptr(), scale_x.data_ptr(), pz or None,
+                 w.data_ptr(), w_scale_1.data_ptr(), ptrs[0] or None, ptrs[1] or None, ptrs[2] or None,
+                 ptrs[3] or None, M, N, kb * 2, y.data_ptr())
+    if st:
+        _lib.check(st, name)
     return y

@@ -121,24 +121,16 @@ def get_dual_quant_col():
 def quantize_sym(x, clip: float = 1.0, qmax: int = 6):
     """One launch for scale + quantize; returns (q [..., K/2], scales [..., 1])."""
     assert x.dtype == torch.float16
-    x2, lead = _flat(x)
-    q, s = _ops.quantize_rows_sym(x2, clip, qmax)
-    return q.view(*lead, -1), s.view(*lead, 1)
+    return _ops.quantize_rows_sym(x, clip, qmax)
 
 
 def quantize_asym(x):
     assert x.dtype == torch.float16
-    x2, lead = _flat(x)
-    q, s, z = _ops.quantize_rows_asym(x2)
-    return q.view(*lead, -1), s.view(*lead, 1), z.view(*lead, 1)
+    return _ops.quantize_rows_asym(x)
 
 
 def linear_forward(mode, xq, scales_x, zeros_x, weight, w_scale_1, w_zeros_1=None, w_scale_2=None, w_zeros_2=None,
                    bias=None):
     """GEMM + dequant (+ bias) in one launch; result has xq's leading dims and N columns."""
     assert xq.shape[-1] % 32 == 0, "A.shape[-1]: {} must be multiplication of 32".format(xq.shape[-1])
-    x2, lead = _flat(xq)
-    v = lambda t: None if t is None else t.view(-1)
-    y = _ops.linear4bit_forward(mode, x2, v(scales_x), v(zeros_x), weight, v(w_scale_1), v(w_zeros_1), v(w_scale_2),
-                                v(w_zeros_2), v(bias))
-    return y.view(*lead, -1)
+    return _ops.linear4bit_forward(mode, xq, scales_x, zeros_x, weight, w_scale_1, w_zeros_1, w_scale_2, w_zeros_2, bias)
