@@ -337,3 +337,91 @@ def linear4bit_forward(mode, xq, scale_x, zeros_x, w, w_scale_1, w_zeros_1=None,
     if st:
         _lib.check(st, name)
     return y
+
+
+# ---- asymmetric path with exact zero-point correction (row sums); not in the reference ----
+
+_I32 = torch.int32
+
+
+def quantize_rows_asym_shifted(x: torch.Tensor):
+    """AsymQuantizer with signed-shifted storage: the codes of ``quantize_rows_asym`` minus 8
+    (signed nibbles), zero points minus 8, and the per-row sums of the shifted codes.
+    Returns (q uint8 [..., K/2], scale [..., 1], zeros [..., 1], rowsum int32 [...])."""
+    if not isinstance(x, torch.Tensor):
+        raise RuntimeError("quantize_rows_asym_shifted: argument #0 is not a tensor")
+    _fast_check("quantize_rows_asym_shifted", "x", x, _F16, None)
+    shape = x.shape
+    cols = shape[-1]
+    rows = x.numel() // cols if cols else 0
+    lead = shape[:-1]
+    dev = x.device
+    q = torch.empty(lead + (cols // 2,), dtype=_U8, device=dev)
+    s = torch.empty(lead + (1,), dtype=_F16, device=dev)
+    z = torch.empty(lead + (1,), dtype=_F16, device=dev)
+    r = torch.empty(lead, dtype=_I32, device=dev)
+    st = _launch(dev, _lib.load().duq_quantize_rows_asym_shifted, x.data_ptr(), rows, cols, q.data_ptr(), s.data_ptr(),
+                 z.data_ptr(), r.data_ptr())
+    if st:
+        _lib.check(st, "quantize_rows_asym_shifted")
+    return q, s, z, r
+
+
+def _rowsum_args(name, M, N, dev, scale_x, zeros_x, rowsum_x, w_scale, w_zeros, w_rowsum_adj, bias):
+    for t, what, dt, n in ((scale_x, "scale_x", _F16, M), (zeros_x, "zeros_x", _F16, M), (rowsum_x, "rowsum_x", _I32, M),
+                           (w_scale, "w_scale", _F16, N), (w_zeros, "w_zeros", _F16, N),
+                           (w_rowsum_adj, "w_rowsum_adj", _I32, N)):
+        if not isinstance(t, torch.Tensor):
+            raise RuntimeError(f"{name}: {what} must be a tensor")
+        _fast_check(name, what, t, dt, dev)
+        if t.numel() != n:
+            _check_size0(name, t.reshape(-1), what, n)
+    pb = None
+    if bias is not None:
+        _fast_check(name, "bias", bias, _F16, dev)
+        if bias.numel() != N:
+            _check_size0(name, bias.reshape(-1), "bias", N)
+        pb = bias.data_ptr()
+    return pb
+
+
+def linear4bit_forward_rowsum(xq, scale_x, zeros_x, rowsum_x, w, w_scale, w_zeros, w_rowsum_adj, bias=None):
+    """GEMM + exact asymmetric dequant (+ bias) in one launch on signed-shifted operands:
+    y = s_x*s_w * (acc - z_x*w_rowsum_adj - z_w*rowsum_x), w_rowsum_adj = sum_k c_w - K*z_w.
+    ``xq`` uint8 [..., K/2]; returns fp16 [..., N]."""
+    name = "linear4bit_forward_rowsum"
+    if not isinstance(xq, torch.Tensor) or not isinstance(w, torch.Tensor):
+        raise RuntimeError(f"{name}: xq and w must be tensors")
+    dev = xq.device
+    _fast_check(name, "xq", xq, _U8, None)
+    _fast_check(name, "w", w, _U8, dev)
+    kb = xq.shape[-1]
+    if w.dim() != 2 or w.shape[1] != kb:
+        raise RuntimeError(f"{name}: packed K differs: x {tuple(xq.shape)} vs w {tuple(w.shape)}")
+    M = xq.numel() // kb if kb else 0
+    N = w.shape[0]
+    pb = _rowsum_args(name, M, N, dev, scale_x, zeros_x, rowsum_x, w_scale, w_zeros, w_rowsum_adj, bias)
+    y = torch.empty(xq.shape[:-1] + (N,), dtype=_F16, device=dev)
+    st = _launch(dev, _lib.load().duq_linear4bit_forward_rowsum, xq.data_ptr(), scale_x.data_ptr(), zeros_x.data_ptr(),
+                 rowsum_x.data_ptr(), w.data_ptr(), w_scale.data_ptr(), w_zeros.data_ptr(), w_rowsum_adj.data_ptr(), pb,
+                 M, N, kb * 2, y.data_ptr())
+    if st:
+        _lib.check(st, name)
+    return y
+
+
+def asym_rowsum_dequant(q, scale_row, zeros_row, rowsum_row, scale_col, zeros_col, rowsum_adj_col, bias=None):
+    """The row-sum epilogue on int32 accumulators [rows, cols] already in memory."""
+    name = "asym_rowsum_dequant"
+    _check(name, q)
+    _check_dtype(name, q, "q", _I32)
+    rows, cols = q.size(0), q.size(1)
+    pb = _rowsum_args(name, rows, cols, q.device, scale_row, zeros_row, rowsum_row, scale_col, zeros_col,
+                      rowsum_adj_col, bias)
+    x = torch.empty((rows, cols), dtype=_F16, device=q.device)
+    st = _launch(q.device, _lib.load().duq_asym_rowsum_dequant_host, q.data_ptr(), scale_row.data_ptr(),
+                 zeros_row.data_ptr(), rowsum_row.data_ptr(), scale_col.data_ptr(), zeros_col.data_ptr(),
+                 rowsum_adj_col.data_ptr(), pb, rows, cols, x.data_ptr())
+    if st:
+        _lib.check(st, name)
+    return x

@@ -34,6 +34,10 @@ PROTOTYPES = {
     "duq_asym_dual_dequant_host": [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_u32, _c_u32, _c_p, _c_p],
     "duq_linear4bit_forward": [_c_i32, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_u32, _c_u32,
                                _c_u32, _c_p, _c_p],
+    "duq_quantize_rows_asym_shifted": [_c_p, _c_u32, _c_u32, _c_p, _c_p, _c_p, _c_p, _c_p],
+    "duq_linear4bit_forward_rowsum": [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_u32, _c_u32, _c_u32,
+                                      _c_p, _c_p],
+    "duq_asym_rowsum_dequant_host": [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_u32, _c_u32, _c_p, _c_p],
 }
 
 _lib = None

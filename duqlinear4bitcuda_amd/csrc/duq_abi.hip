@@ -115,7 +115,17 @@ int duq_quantize_rows_asym(const duq_half *x, uint32_t rows, uint32_t cols, uint
     if (!x || !q || !scale || !zeros) return DUQ_E_NULL;
     if (cols % 32 != 0) return DUQ_E_SHAPE;
     if (!aligned(x, 16) || !aligned(q, 16)) return DUQ_E_ALIGN;
-    return duq::launch_quantize_rows_asym(x, rows, cols, q, scale, zeros, as_stream(stream));
+    return duq::launch_quantize_rows_asym(x, rows, cols, q, scale, zeros, nullptr, as_stream(stream));
+}
+
+int duq_quantize_rows_asym_shifted(const duq_half *x, uint32_t rows, uint32_t cols, uint8_t *q, duq_half *scale,
+                                   duq_half *zeros, int32_t *rowsum, duq_stream_t stream)
+{
+    if (rows == 0 || cols == 0) return DUQ_OK;
+    if (!x || !q || !scale || !zeros || !rowsum) return DUQ_E_NULL;
+    if (cols % 32 != 0) return DUQ_E_SHAPE;
+    if (!aligned(x, 16) || !aligned(q, 16)) return DUQ_E_ALIGN;
+    return duq::launch_quantize_rows_asym(x, rows, cols, q, scale, zeros, rowsum, as_stream(stream));
 }
 
 int duq_matmul_host_4bit(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N, uint32_t K, int32_t *C,
@@ -132,7 +142,7 @@ int duq_sym_dequant_host(const int32_t *q, const duq_half *scale_row, const duq_
 {
     if (rows == 0 || cols == 0) return DUQ_OK;
     if (!q || !scale_row || !scale_col || !x) return DUQ_E_NULL;
-    duq::Epilogue e{DUQ_EPI_SYM, scale_row, nullptr, scale_col, nullptr, nullptr, nullptr, nullptr};
+    duq::Epilogue e{DUQ_EPI_SYM, scale_row, nullptr, scale_col, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
     return duq::launch_dequant(q, e, rows, cols, x, as_stream(stream));
 }
 
@@ -152,7 +162,7 @@ int duq_asym_dequant_host(const int32_t *q, const duq_half *scale_row, const duq
 {
     if (rows == 0 || cols == 0) return DUQ_OK;
     if (!q || !scale_row || !zeros_row || !scale_col || !zeros_col || !x) return DUQ_E_NULL;
-    duq::Epilogue e{DUQ_EPI_ASYM, scale_row, zeros_row, scale_col, zeros_col, nullptr, nullptr, nullptr};
+    duq::Epilogue e{DUQ_EPI_ASYM, scale_row, zeros_row, scale_col, zeros_col, nullptr, nullptr, nullptr, nullptr, nullptr};
     return duq::launch_dequant(q, e, rows, cols, x, as_stream(stream));
 }
 
@@ -165,7 +175,7 @@ int duq_asym_dual_dequant_host(const int32_t *q, const duq_half *scale_row, cons
     if (!q || !scale_row || !zeros_row || !scale_col_1 || !zeros_col_1 || !scale_col_2 || !zeros_col_2 || !x)
         return DUQ_E_NULL;
     duq::Epilogue e{DUQ_EPI_ASYM_DUAL, scale_row, zeros_row, scale_col_1, zeros_col_1, scale_col_2, zeros_col_2,
-                    nullptr};
+                    nullptr, nullptr, nullptr};
     return duq::launch_dequant(q, e, rows, cols, x, as_stream(stream));
 }
 
@@ -183,7 +193,33 @@ int duq_linear4bit_forward(int32_t mode, const uint8_t *xq, const duq_half *scal
     if (asym && (!zeros_x || !w_zeros_1)) return DUQ_E_NULL;
     if (dual && !w_scale_2) return DUQ_E_NULL;
     if (asym && dual && !w_zeros_2) return DUQ_E_NULL;
-    duq::Epilogue e{mode, scale_x, zeros_x, w_scale_1, w_zeros_1, w_scale_2, w_zeros_2, bias};
+    duq::Epilogue e{mode, scale_x, zeros_x, w_scale_1, w_zeros_1, w_scale_2, w_zeros_2, bias, nullptr, nullptr};
+    return duq::launch_gemm_s4(xq, w, M, N, K, nullptr, &e, y, as_stream(stream));
+}
+
+int duq_asym_rowsum_dequant_host(const int32_t *q, const duq_half *scale_row, const duq_half *zeros_row,
+                                 const int32_t *rowsum_row, const duq_half *scale_col, const duq_half *zeros_col,
+                                 const int32_t *rowsum_adj_col, const duq_half *bias, uint32_t rows, uint32_t cols,
+                                 duq_half *x, duq_stream_t stream)
+{
+    if (rows == 0 || cols == 0) return DUQ_OK;
+    if (!q || !scale_row || !zeros_row || !rowsum_row || !scale_col || !zeros_col || !rowsum_adj_col || !x)
+        return DUQ_E_NULL;
+    duq::Epilogue e{DUQ_EPI_ASYM_ROWSUM, scale_row, zeros_row, scale_col, zeros_col, nullptr, nullptr, bias,
+                    rowsum_row, rowsum_adj_col};
+    return duq::launch_dequant(q, e, rows, cols, x, as_stream(stream));
+}
+
+int duq_linear4bit_forward_rowsum(const uint8_t *xq, const duq_half *scale_x, const duq_half *zeros_x,
+                                  const int32_t *rowsum_x, const uint8_t *w, const duq_half *w_scale,
+                                  const duq_half *w_zeros, const int32_t *w_rowsum_adj, const duq_half *bias,
+                                  uint32_t M, uint32_t N, uint32_t K, duq_half *y, duq_stream_t stream)
+{
+    if (int e = check_gemm(xq, w, M, N, K)) return e;
+    if (M == 0 || N == 0) return DUQ_OK;
+    if (!scale_x || !zeros_x || !rowsum_x || !w_scale || !w_zeros || !w_rowsum_adj || !y) return DUQ_E_NULL;
+    duq::Epilogue e{DUQ_EPI_ASYM_ROWSUM, scale_x, zeros_x, w_scale, w_zeros, nullptr, nullptr, bias, rowsum_x,
+                    w_rowsum_adj};
     return duq::launch_gemm_s4(xq, w, M, N, K, nullptr, &e, y, as_stream(stream));
 }
 

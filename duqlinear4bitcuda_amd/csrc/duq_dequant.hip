@@ -17,8 +17,7 @@ __global__ __launch_bounds__(256) void dequant_kernel(const int32_t *__restrict_
          i += (uint64_t)gridDim.x * blockDim.x) {
         const uint32_t row = (uint32_t)(i / perRow);
         const uint32_t col0 = (uint32_t)(i % perRow) * E;
-        const f16 s_row = bits_to_f16(epi.s_row[row]);
-        const f16 z_row = (MODE == 1 || MODE == 3) ? bits_to_f16(epi.z_row[row]) : (f16)0;
+        const RowEpi rp = load_row<MODE>(epi, row);
         if (VEC) {
             const v4i a0 = __builtin_nontemporal_load(reinterpret_cast<const v4i *>(acc + (uint64_t)row * cols + col0));
             const v4i a1 =
@@ -27,8 +26,8 @@ __global__ __launch_bounds__(256) void dequant_kernel(const int32_t *__restrict_
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const ColParams c =
-                    load_col<MODE, BIAS>(epi.s_col_1, epi.z_col_1, epi.s_col_2, epi.z_col_2, epi.bias, col0 + e);
-                const uint32_t bits = dequant_one<MODE, BIAS>(e < 4 ? a0[e & 3] : a1[e & 3], s_row, z_row, c);
+                    load_col<MODE, BIAS>(epi.s_col_1, epi.z_col_1, epi.s_col_2, epi.z_col_2, epi.bias, col0 + e, epi.rs_col);
+                const uint32_t bits = dequant_one<MODE, BIAS>(e < 4 ? a0[e & 3] : a1[e & 3], rp, c);
                 if (e & 1)
                     out[e >> 1] |= bits << 16;
                 else
@@ -37,8 +36,8 @@ __global__ __launch_bounds__(256) void dequant_kernel(const int32_t *__restrict_
             *reinterpret_cast<v4u *>(y + (uint64_t)row * cols + col0) = v4u{out[0], out[1], out[2], out[3]};
         } else {
             const ColParams c =
-                load_col<MODE, BIAS>(epi.s_col_1, epi.z_col_1, epi.s_col_2, epi.z_col_2, epi.bias, col0);
-            y[(uint64_t)row * cols + col0] = dequant_one<MODE, BIAS>(acc[(uint64_t)row * cols + col0], s_row, z_row, c);
+                load_col<MODE, BIAS>(epi.s_col_1, epi.z_col_1, epi.s_col_2, epi.z_col_2, epi.bias, col0, epi.rs_col);
+            y[(uint64_t)row * cols + col0] = dequant_one<MODE, BIAS>(acc[(uint64_t)row * cols + col0], rp, c);
         }
     }
 }
@@ -74,6 +73,7 @@ int launch_dequant(const int32_t *acc, const Epilogue &epi, uint32_t rows, uint3
         DUQ_DQ(1)
         DUQ_DQ(2)
         DUQ_DQ(3)
+        DUQ_DQ(4)
     default:
         return (int)hipErrorInvalidValue;
     }

@@ -2,8 +2,14 @@
 // dequant kernels and the fused GEMM so that both give identical bits.
 //   sym       : src/kernels/quant.cu:64-81      asym      : src/kernels/quant.cu:149-169
 //   sym dual  : src/kernels/quant2.cu:62-83     asym dual : src/kernels/quant2.cu:158-186
+// Mode 4 has no counterpart in the reference: operands hold signed-shifted codes c = u - 8 with
+// shifted zero points z (x ~ s * (c - z)), and the epilogue applies the exact correction
+//   corr = acc - z_row * (R_col - K * z_col) - z_col * R_row,   y = h(f32(corr) * (f32(s_row) * f32(s_col)))
+// in 32-bit integers (R = per-row / per-column sums of the shifted codes; the column term is
+// precomputed with the weights).
 #pragma once
 #include "duq_device.h"
+#include "duq_launch.h"
 
 namespace duq {
 
@@ -13,17 +19,41 @@ struct ColParams {
     f16 s;
     f16 z;
     f16 bias;
+    int rs;  // mode 4
 };
+
+// Row-side parameters of one output row.
+struct RowEpi {
+    f16 s;
+    f16 z;
+    int rs;  // mode 4
+};
+
+template <int MODE>
+__device__ __forceinline__ RowEpi load_row(const Epilogue &e, uint32_t row)
+{
+    RowEpi r;
+    r.s = bits_to_f16(e.s_row[row]);
+    r.z = (MODE == 1 || MODE == 3 || MODE == 4) ? bits_to_f16(e.z_row[row]) : (f16)0;
+    r.rs = MODE == 4 ? e.rs_row[row] : 0;
+    return r;
+}
 
 template <int MODE, bool BIAS>
 __device__ __forceinline__ ColParams load_col(const uint16_t *s1, const uint16_t *z1, const uint16_t *s2,
-                                              const uint16_t *z2, const uint16_t *bias, uint32_t col)
+                                              const uint16_t *z2, const uint16_t *bias, uint32_t col,
+                                              const int32_t *rs = nullptr)
 {
     ColParams c;
     c.z = (f16)0;
     c.bias = (f16)0;
+    c.rs = 0;
     if (MODE == 0) {
         c.s = bits_to_f16(s1[col]);
+    } else if (MODE == 4) {
+        c.s = bits_to_f16(s1[col]);
+        c.z = bits_to_f16(z1[col]);
+        c.rs = rs[col];
     } else if (MODE == 1) {
         c.s = bits_to_f16(s1[col]);
         c.z = bits_to_f16(z1[col]);
@@ -40,16 +70,26 @@ __device__ __forceinline__ ColParams load_col(const uint16_t *s1, const uint16_t
 }
 
 template <int MODE, bool BIAS>
-__device__ __forceinline__ uint16_t dequant_one(int acc, f16 s_row, f16 z_row, const ColParams &c)
+__device__ __forceinline__ uint16_t dequant_one(int acc, const RowEpi &r, const ColParams &c)
 {
-    const f16 e = acc_to_f16(acc);
-    const f16 ss = s_row * c.s;  // h(s_row * s_col)
     f16 y;
-    if (MODE == 0 || MODE == 2) {
-        y = ss * e;
+    if (MODE == 4) {
+        // 32-bit wrapping integer arithmetic; zero points are integer-valued binary16 numbers
+        const uint32_t zr = (uint32_t)rint_i32((float)r.z), zc = (uint32_t)rint_i32((float)c.z);
+        const int corr = (int)((uint32_t)acc - zr * (uint32_t)c.rs - zc * (uint32_t)r.rs);
+        const float ss = (float)r.s * (float)c.s;  // exact: 11-bit x 11-bit significands
+        float prod = (float)corr * ss;
+        asm volatile("" : "+v"(prod));  // round to float32 here, then to binary16 (no single-rounding mixed FMA)
+        y = (f16)prod;
     } else {
-        const f16 t = (e - z_row) - c.z;
-        y = ss * t;
+        const f16 e = acc_to_f16(acc);
+        const f16 ss = r.s * c.s;  // h(s_row * s_col)
+        if (MODE == 0 || MODE == 2) {
+            y = ss * e;
+        } else {
+            const f16 t = (e - r.z) - c.z;
+            y = ss * t;
+        }
     }
     if (BIAS) y = y + c.bias;
     return f16_to_bits(y);
@@ -80,7 +120,7 @@ template <int MODE, bool BIAS>
 __device__ __forceinline__ QuadCols<MODE, BIAS> load_quad_cols(const uint16_t *s1, const uint16_t *z1,
                                                                const uint16_t *s2, const uint16_t *z2,
                                                                const uint16_t *bias, uint32_t n0, uint32_t cols,
-                                                               bool vec)
+                                                               bool vec, const int32_t *rs = nullptr)
 {
     QuadCols<MODE, BIAS> q;
     uint16_t a[4], b[4];
@@ -93,8 +133,9 @@ __device__ __forceinline__ QuadCols<MODE, BIAS> load_quad_cols(const uint16_t *s
         q.c[r].s = bits_to_f16((MODE == 2 || MODE == 3) ? (first ? a[r] : b[r]) : a[r]);
         q.c[r].z = (f16)0;
         q.c[r].bias = (f16)0;
+        q.c[r].rs = MODE == 4 ? rs[min(col, cols - 1)] : 0;
     }
-    if (MODE == 1 || MODE == 3) {
+    if (MODE == 1 || MODE == 3 || MODE == 4) {
         load4_f16(z1, n0, cols, vec, a);
         if (MODE == 3) load4_f16(z2, n0, cols, vec, b);
 #pragma unroll
@@ -111,7 +152,8 @@ __device__ __forceinline__ QuadCols<MODE, BIAS> load_quad_cols(const uint16_t *s
 // Same selection as load_quad_cols, from raw 64-bit words fetched earlier (four binary16
 // values per word, column n0 first).
 template <int MODE, bool BIAS>
-__device__ __forceinline__ QuadCols<MODE, BIAS> quad_cols_from_raw(v2u s1, v2u z1, v2u s2, v2u z2, v2u bias, uint32_t n0)
+__device__ __forceinline__ QuadCols<MODE, BIAS> quad_cols_from_raw(v2u s1, v2u z1, v2u s2, v2u z2, v2u bias, uint32_t n0,
+                                                                   v4i rs = v4i{0, 0, 0, 0})
 {
     auto pick = [](v2u v, int r) -> uint16_t { return (uint16_t)((r & 1) ? (v[r >> 1] >> 16) : (v[r >> 1] & 0xFFFFu)); };
     QuadCols<MODE, BIAS> q;
@@ -120,7 +162,8 @@ __device__ __forceinline__ QuadCols<MODE, BIAS> quad_cols_from_raw(v2u s1, v2u z
         const uint32_t col = n0 + r;
         const bool first = MODE == 2 ? col < (uint32_t)kQuantColK : col == 0;
         q.c[r].s = bits_to_f16((MODE == 2 || MODE == 3) ? (first ? pick(s1, r) : pick(s2, r)) : pick(s1, r));
-        q.c[r].z = (MODE == 1) ? bits_to_f16(pick(z1, r))
+        q.c[r].rs = MODE == 4 ? rs[r] : 0;
+        q.c[r].z = (MODE == 1 || MODE == 4) ? bits_to_f16(pick(z1, r))
                                : (MODE == 3 ? bits_to_f16(col == 0 ? pick(z1, r) : pick(z2, r)) : (f16)0);
         q.c[r].bias = BIAS ? bits_to_f16(pick(bias, r)) : (f16)0;
     }

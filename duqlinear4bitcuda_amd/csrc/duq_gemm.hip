@@ -85,15 +85,14 @@ __device__ __forceinline__ void store_quad(const GemmParams &p, uint32_t m, uint
         }
     } else {
         constexpr int MODE = EPI < 0 ? 0 : EPI;
-        const f16 s_row = bits_to_f16(p.epi.s_row[m]);
-        const f16 z_row = (MODE == 1 || MODE == 3) ? bits_to_f16(p.epi.z_row[m]) : (f16)0;
+        const RowEpi rp = load_row<MODE>(p.epi, m);
         uint16_t out[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const uint32_t n = min(n0 + r, p.N - 1);
             const ColParams c = load_col<MODE, BIAS>(p.epi.s_col_1, p.epi.z_col_1, p.epi.s_col_2, p.epi.z_col_2,
-                                                     p.epi.bias, n);
-            out[r] = dequant_one<MODE, BIAS>(acc[r], s_row, z_row, c);
+                                                     p.epi.bias, n, p.epi.rs_col);
+            out[r] = dequant_one<MODE, BIAS>(acc[r], rp, c);
         }
         uint16_t *dst = p.y + (uint64_t)m * p.N + n0;
         if (vec_ok && n0 + 3 < p.N) {
@@ -416,10 +415,12 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
     const Epilogue &e = p.epi;
     bool staged = false;
     v2u raw_s1[TN * 4], raw_z1[TN * 4], raw_s2[TN * 4], raw_z2[TN * 4], raw_bias[TN * 4];
-    f16 s_row[TM], z_row[TM];
+    v4i raw_rs[TN * 4];
+    RowEpi rowp[TM];
     if (EPI >= 0) {
         const bool vec_ld = p.N % 4 == 0 && reinterpret_cast<uintptr_t>(e.s_col_1) % 8 == 0 &&
                             (MODE == 0 || MODE == 2 || reinterpret_cast<uintptr_t>(e.z_col_1) % 8 == 0) &&
+                            (MODE != 4 || reinterpret_cast<uintptr_t>(e.rs_col) % 16 == 0) &&
                             (MODE < 2 || reinterpret_cast<uintptr_t>(e.s_col_2) % 8 == 0) &&
                             (MODE != 3 || reinterpret_cast<uintptr_t>(e.z_col_2) % 8 == 0) &&
                             (!BIAS || reinterpret_cast<uintptr_t>(e.bias) % 8 == 0);
@@ -427,15 +428,15 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
 #pragma unroll
         for (int b = 0; b < TM; ++b) {
             const uint32_t m = min(m0 + b * 32 + l32, p.M - 1);
-            s_row[b] = bits_to_f16(e.s_row[m]);
-            z_row[b] = (MODE == 1 || MODE == 3) ? bits_to_f16(e.z_row[m]) : (f16)0;
+            rowp[b] = load_row<MODE>(e, m);
         }
         if (staged) {
 #pragma unroll
             for (int tq = 0; tq < TN * 4; ++tq) {
                 const uint32_t nq = min(n0 + wave * 64 + (tq >> 2) * 32 + (tq & 3) * 8 + h * 4, p.N - 4);
                 raw_s1[tq] = *reinterpret_cast<const v2u *>(e.s_col_1 + nq);
-                if (MODE == 1 || MODE == 3) raw_z1[tq] = *reinterpret_cast<const v2u *>(e.z_col_1 + nq);
+                if (MODE == 1 || MODE == 3 || MODE == 4) raw_z1[tq] = *reinterpret_cast<const v2u *>(e.z_col_1 + nq);
+                if (MODE == 4) raw_rs[tq] = *reinterpret_cast<const v4i *>(e.rs_col + nq);
                 if (MODE >= 2) raw_s2[tq] = *reinterpret_cast<const v2u *>(e.s_col_2 + nq);
                 if (MODE == 3) raw_z2[tq] = *reinterpret_cast<const v2u *>(e.z_col_2 + nq);
                 if (BIAS) raw_bias[tq] = *reinterpret_cast<const v2u *>(e.bias + nq);
@@ -496,13 +497,14 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
                     const uint32_t ncol = t * 32 + q * 8 + h * 4;  // column inside the wavefront's tile
                     const uint32_t nq = min(n0 + wave * 64 + ncol, p.N - 4);
                     const QuadCols<MODE, BIAS> cols = quad_cols_from_raw<MODE, BIAS>(
-                        raw_s1[t * 4 + q], raw_z1[t * 4 + q], raw_s2[t * 4 + q], raw_z2[t * 4 + q], raw_bias[t * 4 + q], nq);
+                        raw_s1[t * 4 + q], raw_z1[t * 4 + q], raw_s2[t * 4 + q], raw_z2[t * 4 + q], raw_bias[t * 4 + q], nq,
+                        raw_rs[t * 4 + q]);
 #pragma unroll
                     for (int b = 0; b < TM; ++b) {
                         uint16_t out[4];
 #pragma unroll
                         for (int r = 0; r < 4; ++r)
-                            out[r] = dequant_one<MODE, BIAS>(acc[t][b][q * 4 + r] >> 8, s_row[b], z_row[b], cols.c[r]);
+                            out[r] = dequant_one<MODE, BIAS>(acc[t][b][q * 4 + r] >> 8, rowp[b], cols.c[r]);
                         *reinterpret_cast<v2u *>(stage + (b * 32 + l32) * kYStride + ncol * 2) =
                             v2u{(uint32_t)out[0] | ((uint32_t)out[1] << 16), (uint32_t)out[2] | ((uint32_t)out[3] << 16)};
                     }
@@ -528,7 +530,7 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
                 const uint32_t nq = n0 + wave * 64 + t * 32 + q * 8 + h * 4;
                 if (nq >= p.N) continue;
                 const QuadCols<MODE, BIAS> cols = load_quad_cols<MODE, BIAS>(e.s_col_1, e.z_col_1, e.s_col_2, e.z_col_2,
-                                                                             e.bias, nq, p.N, false);
+                                                                             e.bias, nq, p.N, false, e.rs_col);
 #pragma unroll
                 for (int b = 0; b < TM; ++b) {
                     const uint32_t m = m0 + b * 32 + l32;
@@ -545,7 +547,7 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
                     uint16_t *dst = p.y + (uint64_t)m * p.N + nq;
 #pragma unroll
                     for (int r = 0; r < 4; ++r)
-                        if (nq + r < p.N) dst[r] = dequant_one<MODE, BIAS>(v[r], s_row[b], z_row[b], cols.c[r]);
+                        if (nq + r < p.N) dst[r] = dequant_one<MODE, BIAS>(v[r], rowp[b], cols.c[r]);
                 }
             }
         }
@@ -634,10 +636,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_s4_skinny_kernel(GemmParams p
                     } else {
                         constexpr int MODE = EPI < 0 ? 0 : EPI;
                         const ColParams c = load_col<MODE, BIAS>(p.epi.s_col_1, p.epi.z_col_1, p.epi.s_col_2,
-                                                                 p.epi.z_col_2, p.epi.bias, n);
-                        const f16 s_row = bits_to_f16(p.epi.s_row[m]);
-                        const f16 z_row = (MODE == 1 || MODE == 3) ? bits_to_f16(p.epi.z_row[m]) : (f16)0;
-                        p.y[(uint64_t)m * p.N + n] = dequant_one<MODE, BIAS>(sum, s_row, z_row, c);
+                                                                 p.epi.z_col_2, p.epi.bias, n, p.epi.rs_col);
+                        p.y[(uint64_t)m * p.N + n] = dequant_one<MODE, BIAS>(sum, load_row<MODE>(p.epi, m), c);
                     }
                 }
             }
@@ -754,10 +754,8 @@ __global__ __launch_bounds__(256) void gemv_s4_dot_kernel(GemmParams p)
             } else {
                 constexpr int MODE = EPI < 0 ? 0 : EPI;
                 const ColParams c = load_col<MODE, BIAS>(p.epi.s_col_1, p.epi.z_col_1, p.epi.s_col_2, p.epi.z_col_2,
-                                                         p.epi.bias, nn);
-                const f16 s_row = bits_to_f16(p.epi.s_row[m]);
-                const f16 z_row = (MODE == 1 || MODE == 3) ? bits_to_f16(p.epi.z_row[m]) : (f16)0;
-                p.y[(uint64_t)m * p.N + nn] = dequant_one<MODE, BIAS>(v, s_row, z_row, c);
+                                                         p.epi.bias, nn, p.epi.rs_col);
+                p.y[(uint64_t)m * p.N + nn] = dequant_one<MODE, BIAS>(v, load_row<MODE>(p.epi, m), c);
             }
         }
     }
@@ -860,6 +858,7 @@ int launch_gemm_s4(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N, u
             DUQ_GEMM(1)
             DUQ_GEMM(2)
             DUQ_GEMM(3)
+            DUQ_GEMM(4)
         default:
             return (int)hipErrorInvalidValue;
         }

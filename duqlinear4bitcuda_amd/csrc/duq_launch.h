@@ -18,11 +18,14 @@ int launch_asym_dual_quant(const uint16_t *x, const uint16_t *s1, const uint16_t
                            hipStream_t stream);
 int launch_quantize_rows_sym(const uint16_t *x, uint32_t rows, uint32_t cols, float clip, int qmax, uint8_t *q,
                              uint16_t *scale, hipStream_t stream);
+// rowsum == nullptr: unsigned codes and zero points as the reference stores them; otherwise the
+// signed-shifted form (code - 8, zero - 8) plus the per-row sum of the shifted codes.
 int launch_quantize_rows_asym(const uint16_t *x, uint32_t rows, uint32_t cols, uint8_t *q, uint16_t *scale,
-                              uint16_t *zeros, hipStream_t stream);
+                              uint16_t *zeros, int32_t *rowsum, hipStream_t stream);
 
 // Epilogue description shared by the stand-alone dequant kernels and the fused GEMM.
-// mode: 0 sym, 1 asym, 2 sym-dual, 3 asym-dual (DUQ_EPI_* of the public header).
+// mode: 0 sym, 1 asym, 2 sym-dual, 3 asym-dual, 4 asym with row-sum zero-point correction
+// (DUQ_EPI_* of the public header).
 struct Epilogue {
     int mode;
     const uint16_t *s_row;   // [rows]
@@ -32,6 +35,8 @@ struct Epilogue {
     const uint16_t *s_col_2; // [cols]  dual modes
     const uint16_t *z_col_2; // [cols]  asym-dual
     const uint16_t *bias;    // [cols] or nullptr
+    const int32_t *rs_row;   // [rows]  mode 4: sum over k of the row's shifted codes
+    const int32_t *rs_col;   // [cols]  mode 4: sum over k of the column's shifted codes minus K * zero
 };
 
 int launch_dequant(const int32_t *acc, const Epilogue &epi, uint32_t rows, uint32_t cols, uint16_t *y,

@@ -185,6 +185,7 @@ struct RowParams {
     uint32_t rows, cols;
     float clip;
     int qmax;
+    int32_t *rowsum;  // asym only: non-null selects the signed-shifted form (code - 8, zero - 8, sum of codes)
 };
 
 __device__ __forceinline__ uint32_t pk_absmax_u16(uint32_t acc, uint32_t w)
@@ -199,6 +200,9 @@ __global__ __launch_bounds__(WAVES * 64) void quantize_rows_kernel(RowParams p)
 {
     constexpr int T = WAVES * 64;
     __shared__ float red[2][WAVES];
+    __shared__ int red_sum[WAVES];
+    const bool shifted = ASYM && p.rowsum != nullptr;
+    int code_sum = 0;  // sum of this lane's unsigned codes (shifted form only)
     const uint32_t row = blockIdx.x;
     const uint32_t tid = threadIdx.x;
     const uint32_t nunits = p.cols >> 3;  // units of 8 elements
@@ -290,7 +294,7 @@ __global__ __launch_bounds__(WAVES * 64) void quantize_rows_kernel(RowParams p)
     }
     if (tid == 0) {
         p.scale[row] = f16_to_bits(s);
-        if (ASYM) p.zeros[row] = f16_to_bits(z);
+        if (ASYM) p.zeros[row] = f16_to_bits(shifted ? z - (f16)8.0f : z);
     }
     const float rcp = row_rcp(s);
     const int zi = ASYM ? rint_i32((float)z) : 0;
@@ -340,9 +344,16 @@ __global__ __launch_bounds__(WAVES * 64) void quantize_rows_kernel(RowParams p)
 
     // ---- quantize + pack: 8 elements -> one 32-bit store ----
     auto quant_unit = [&](const v4u &g) -> uint32_t {
-        if (fast) return quant8_fast(g);
-        return ASYM ? quant8<kAsym>(g, 0, rcp, 0.f, 15, zi, (f16)0, (f16)0)
-                    : quant8<kSym>(g, 0, rcp, 0.f, p.qmax, 0, (f16)0, (f16)0);
+        uint32_t w = fast ? quant8_fast(g)
+                          : (ASYM ? quant8<kAsym>(g, 0, rcp, 0.f, 15, zi, (f16)0, (f16)0)
+                                  : quant8<kSym>(g, 0, rcp, 0.f, p.qmax, 0, (f16)0, (f16)0));
+        if (shifted) {
+            // eight unsigned codes: sum them, then u - 8 as a signed nibble is u with bit 3 flipped
+            const uint32_t pairs = (w & 0x0F0F0F0Fu) + ((w >> 4) & 0x0F0F0F0Fu);
+            code_sum = (int)__builtin_amdgcn_udot4(pairs, 0x01010101u, (uint32_t)code_sum, false);
+            w ^= 0x88888888u;
+        }
+        return w;
     };
     if (CACHED) {
 #pragma unroll
@@ -352,6 +363,18 @@ __global__ __launch_bounds__(WAVES * 64) void quantize_rows_kernel(RowParams p)
         }
     } else {
         for (uint32_t u = tid; u < nunits; u += T) qrow[u] = quant_unit(xrow[u]);
+    }
+    if (shifted) {  // uniform branch: sum of (u - 8) over the row
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) code_sum += __shfl_xor(code_sum, off, kWave);
+        if (WAVES > 1) {
+            if ((tid & 63u) == 0) red_sum[tid >> 6] = code_sum;
+            __syncthreads();
+            code_sum = 0;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) code_sum += red_sum[w];
+        }
+        if (tid == 0) p.rowsum[row] = code_sum - 8 * (int)p.cols;
     }
 }
 
@@ -394,13 +417,13 @@ static int launch_rows(const RowParams &p, hipStream_t stream)
 int launch_quantize_rows_sym(const uint16_t *x, uint32_t rows, uint32_t cols, float clip, int qmax, uint8_t *q,
                              uint16_t *scale, hipStream_t stream)
 {
-    RowParams p{x, q, scale, nullptr, rows, cols, clip, qmax};
+    RowParams p{x, q, scale, nullptr, rows, cols, clip, qmax, nullptr};
     return launch_rows<false>(p, stream);
 }
 int launch_quantize_rows_asym(const uint16_t *x, uint32_t rows, uint32_t cols, uint8_t *q, uint16_t *scale,
-                              uint16_t *zeros, hipStream_t stream)
+                              uint16_t *zeros, int32_t *rowsum, hipStream_t stream)
 {
-    RowParams p{x, q, scale, zeros, rows, cols, 1.0f, 15};
+    RowParams p{x, q, scale, zeros, rows, cols, 1.0f, 15, rowsum};
     return launch_rows<true>(p, stream);
 }
 

@@ -125,6 +125,65 @@ class Linear4bitASQ(_Linear4bitBase):
         return new
 
 
+class Linear4bitASQRowSum(_Linear4bitBase):
+    """Asymmetric 4-bit linear layer with the exact zero-point correction.  Not in the
+    reference: its Linear4bitASQ stores unsigned codes that the signed GEMM misreads
+    (README.md:31-32) and its epilogue subtracts the zero points from the accumulator
+    (src/kernels/quant.cu:167-168).  Here codes and zero points are stored minus 8, the signed
+    GEMM is exact for them, and the epilogue applies
+        y = s_x * s_w * (acc - z_x * (R_w - K * z_w) - z_w * R_x)
+    with R_w - K * z_w precomputed per output channel (``weight_rowsum``) and R_x delivered by
+    the activation quantizer."""
+
+    def __init__(self, in_features, out_features, bias=False, require_quantizer=True):
+        super().__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+        self.require_quantizer = require_quantizer
+        self.register_buffer("weight_scales", torch.zeros((out_features, 1), requires_grad=False, dtype=torch.float16))
+        self.register_buffer("weight_zeros", torch.zeros((out_features, 1), requires_grad=False, dtype=torch.float16))
+        self.register_buffer("weight_rowsum", torch.zeros((out_features,), requires_grad=False, dtype=torch.int32))
+        self.register_buffer("weight", _placeholder_weight(out_features, in_features))
+        if bias:
+            self.register_buffer("bias", torch.zeros((out_features), dtype=torch.float16))
+        else:
+            self.bias = None
+        if require_quantizer:
+            self.quantizer = AsymQuantizer(shifted=True)
+
+    def forward(self, x):
+        if self.require_quantizer:
+            x = self.quantizer(x)
+        assert type(x) == tensor_utils.PackedQuantizedTensor and x.rowsum_x is not None, \
+            "Input should come from AsymQuantizer(shifted=True), or require_quantizer should be set"
+        if self.fused:
+            return tensor_utils.linear_forward_rowsum(x.quantized_x, x.scales_x, x.zeros_x, x.rowsum_x, self.weight,
+                                                      self.weight_scales, self.weight_zeros, self.weight_rowsum,
+                                                      bias=self.bias)
+        acc = tensor_utils.matmul(x.quantized_x, self.weight)
+        lead = acc.shape[:-1]
+        y = _ops.asym_rowsum_dequant(acc.view(-1, acc.shape[-1]), x.scales_x, x.zeros_x, x.rowsum_x, self.weight_scales,
+                                     self.weight_zeros, self.weight_rowsum, self.bias)
+        return y.view(*lead, -1)
+
+    @classmethod
+    def from_linear(cls, module: torch.nn.Linear, require_quantizer: bool = True):
+        """Per-output-channel min/max quantization of ``module.weight`` on the device it lives on
+        (the activation quantizer kernel, applied to the weight rows)."""
+        w = module.weight.data
+        assert w.is_cuda, "weight preparation runs on the GPU: move the layer there first"
+        new = cls(module.in_features, module.out_features, bias=module.bias is not None,
+                  require_quantizer=require_quantizer).to(w.device)
+        q, scale, zeros, rowsum = tensor_utils.quantize_asym_shifted(w.to(torch.float16).contiguous())
+        new.weight.copy_(q)
+        new.weight_scales.copy_(scale)
+        new.weight_zeros.copy_(zeros)
+        new.weight_rowsum.copy_(rowsum - module.in_features * zeros.view(-1).to(torch.int32))
+        if module.bias is not None:
+            new.bias.copy_(module.bias)
+        return new
+
+
 class Linear4bitDUSQ(_Linear4bitBase):
     """Symmetric layer with two per-row weight scales: input columns < 10 were quantized
     with scale 1, the rest with scale 2; the epilogue picks per OUTPUT column < 10

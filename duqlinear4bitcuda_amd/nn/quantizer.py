@@ -36,14 +36,20 @@ class AsymQuantizer(torch.nn.Module):
     (quantizer.py:24-35).  ``input_clip_ratio`` is accepted and unused, as in the
     reference."""
 
-    def __init__(self, input_clip_ratio: float = 1.0):
+    def __init__(self, input_clip_ratio: float = 1.0, shifted: bool = False):
         super().__init__()
         self.n_levels = 2 ** 4
         self.input_clip_ratio = input_clip_ratio
+        # shifted=True (not in the reference): codes and zero points are stored minus 8, so that the signed
+        # GEMM reads them exactly, and the per-token sums of the codes come along for the row-sum epilogue
+        self.shifted = shifted
 
     def forward(self, x) -> tensor_utils.PackedQuantizedTensor:
         if not x.is_contiguous():
             x = x.contiguous()
+        if self.shifted:
+            assert x.shape[-1] % 32 == 0 and x.data_ptr() % 16 == 0, "shifted quantization needs K % 32 == 0"
+            return tensor_utils.PackedQuantizedTensor(*tensor_utils.quantize_asym_shifted(x))
         if x.shape[-1] % 32 == 0 and x.data_ptr() % 16 == 0:
             q, scale, zeros = tensor_utils.quantize_asym(x)
         else:

@@ -15,10 +15,13 @@ class PackedQuantizedTensor:
     """A quantized activation: packed nibbles plus per-token scale (and zero point)
     (tensor_utils.py:20-38)."""
 
-    def __init__(self, quantized_x: torch.Tensor, scales_x: torch.Tensor, zeros_x: torch.Tensor = None):
+    def __init__(self, quantized_x: torch.Tensor, scales_x: torch.Tensor, zeros_x: torch.Tensor = None,
+                 rowsum_x: torch.Tensor = None):
         self.quantized_x = quantized_x
         self.scales_x = scales_x
         self.zeros_x = zeros_x
+        # set only by the signed-shifted asymmetric quantizer (codes - 8, zeros - 8): per-token sums of the codes
+        self.rowsum_x = rowsum_x
 
     def size(self):
         return self.quantized_x.size()
@@ -127,6 +130,19 @@ def quantize_sym(x, clip: float = 1.0, qmax: int = 6):
 def quantize_asym(x):
     assert x.dtype == torch.float16
     return _ops.quantize_rows_asym(x)
+
+
+def quantize_asym_shifted(x):
+    """Signed-shifted asymmetric quantization for the row-sum epilogue:
+    (q [..., K/2], scales [..., 1], zeros - 8 [..., 1], rowsum int32 [...])."""
+    assert x.dtype == torch.float16
+    return _ops.quantize_rows_asym_shifted(x)
+
+
+def linear_forward_rowsum(xq, scales_x, zeros_x, rowsum_x, weight, w_scale, w_zeros, w_rowsum_adj, bias=None):
+    """GEMM + exact zero-point correction (+ bias) in one launch on signed-shifted operands."""
+    assert xq.shape[-1] % 32 == 0, "A.shape[-1]: {} must be multiplication of 32".format(xq.shape[-1])
+    return _ops.linear4bit_forward_rowsum(xq, scales_x, zeros_x, rowsum_x, weight, w_scale, w_zeros, w_rowsum_adj, bias)
 
 
 def linear_forward(mode, xq, scales_x, zeros_x, weight, w_scale_1, w_zeros_1=None, w_scale_2=None, w_zeros_2=None,

@@ -54,6 +54,7 @@ typedef void *duq_stream_t;  /* hipStream_t */
 #define DUQ_EPI_ASYM 1       /* src/kernels/quant.cu:149-169 */
 #define DUQ_EPI_SYM_DUAL 2   /* src/kernels/quant2.cu:62-83  */
 #define DUQ_EPI_ASYM_DUAL 3  /* src/kernels/quant2.cu:158-186 */
+#define DUQ_EPI_ASYM_ROWSUM 4 /* exact zero-point correction with row sums; not in the reference */
 
 /* ---- library info ------------------------------------------------------------------ */
 
@@ -112,6 +113,14 @@ int duq_quantize_rows_sym(const duq_half *x, uint32_t rows, uint32_t cols, float
 int duq_quantize_rows_asym(const duq_half *x, uint32_t rows, uint32_t cols, uint8_t *q, duq_half *scale,
                            duq_half *zeros, duq_stream_t stream);
 
+/* Signed-shifted form of duq_quantize_rows_asym for the row-sum epilogue (no counterpart in
+ * the reference, whose unsigned codes are misread by its signed GEMM, README.md:31-32):
+ * same scale and the same codes u as duq_quantize_rows_asym, stored as the signed nibble
+ * u - 8; zeros[r] = h(zero - 8); rowsum[r] = sum_k (u[r,k] - 8).  Then
+ * x[r,k] ~ scale[r] * (s4(q[r,k]) - zeros[r]) and the signed GEMM is exact for it. */
+int duq_quantize_rows_asym_shifted(const duq_half *x, uint32_t rows, uint32_t cols, uint8_t *q,
+                                   duq_half *scale, duq_half *zeros, int32_t *rowsum, duq_stream_t stream);
+
 /* ---- GEMM ---------------------------------------------------------------------------- */
 
 /* Replaces matmul_host_4bit (include/gemm.h:5-12, src/kernels/gemm.cu:8-43):
@@ -167,6 +176,31 @@ int duq_linear4bit_forward(int32_t mode, const uint8_t *xq, const duq_half *scal
                            const uint8_t *w, const duq_half *w_scale_1, const duq_half *w_zeros_1,
                            const duq_half *w_scale_2, const duq_half *w_zeros_2, const duq_half *bias,
                            uint32_t M, uint32_t N, uint32_t K, duq_half *y, duq_stream_t stream);
+
+/* ---- asymmetric forward with exact zero-point correction (row sums) -------------------- */
+
+/* No counterpart in the reference (its asymmetric epilogue, src/kernels/quant.cu:167-168,
+ * subtracts the zero points from the accumulator, which is not the correction).  Operands
+ * hold signed-shifted codes c with shifted zero points z, x[m,k] ~ s_x[m]*(c_x[m,k] - z_x[m])
+ * and w[n,k] ~ s_w[n]*(c_w[n,k] - z_w[n]), so that
+ *   sum_k x*w = s_x*s_w * (acc - z_x*(R_w[n] - K*z_w[n]) - z_w[n]*R_x[m]),  R = sum_k c.
+ *   rowsum_x      [M] int32  R_x, as written by duq_quantize_rows_asym_shifted
+ *   w_rowsum_adj  [N] int32  R_w[n] - K*z_w[n], computed once with the weights
+ * The correction is evaluated in wrapping 32-bit integers (zero points are integer-valued
+ * binary16 numbers, converted with round-to-nearest), then
+ *   y = h(f32(f32(corr) * (f32(s_x)*f32(s_w))));  with bias: y = h(y + bias[n]).
+ * Same shape and alignment rules as duq_linear4bit_forward. */
+int duq_linear4bit_forward_rowsum(const uint8_t *xq, const duq_half *scale_x, const duq_half *zeros_x,
+                                  const int32_t *rowsum_x, const uint8_t *w, const duq_half *w_scale,
+                                  const duq_half *w_zeros, const int32_t *w_rowsum_adj, const duq_half *bias,
+                                  uint32_t M, uint32_t N, uint32_t K, duq_half *y, duq_stream_t stream);
+
+/* The same epilogue on int32 accumulators already in HBM (q [rows, cols] from
+ * duq_matmul_host_4bit); bit-identical to duq_linear4bit_forward_rowsum. */
+int duq_asym_rowsum_dequant_host(const int32_t *q, const duq_half *scale_row, const duq_half *zeros_row,
+                                 const int32_t *rowsum_row, const duq_half *scale_col, const duq_half *zeros_col,
+                                 const int32_t *rowsum_adj_col, const duq_half *bias, uint32_t rows, uint32_t cols,
+                                 duq_half *x, duq_stream_t stream);
 
 #ifdef __cplusplus
 }

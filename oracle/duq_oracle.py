@@ -309,6 +309,64 @@ def add_bias(y, bias):
 
 
 # ----------------------------------------------------------------------------------
+# Row-sum mode: asymmetric forward with the exact zero-point correction.  The reference has
+# no such path (its epilogue, src/kernels/quant.cu:167-168, subtracts the zero points from
+# the accumulator; README.md:31-32 notes the signed/unsigned mismatch); this restates the
+# definition the library documents in include/duq_hip.h.  Pinned by the integer identity
+# corr == sum_k (c_x - z_x)(c_w - z_w) (brute force) and by dequantize-then-matmul in float64.
+# ----------------------------------------------------------------------------------
+def asym_quant_shifted(x):
+    """Codes of asym_quant stored as u - 8 (signed nibble), zeros as h(z - 8), and the row sums
+    of the shifted codes.  Returns (packed u8, scale [M,1], zeros_shifted [M,1], rowsum int32 [M])."""
+    x = np.asarray(x, _F16)
+    s, z = asym_scales_zeros(x)
+    c = asym_quant_values(x, s, z).astype(np.int32) - 8
+    zs = hsub(z, _F16(8.0))
+    return pack_i4(c, sym=True), s, zs, c.sum(axis=-1, dtype=np.int64).astype(np.int32)
+
+
+def weight_rowsum_adj(w_packed_shifted, zeros_shifted):
+    """R_w[n] - K * z_w[n] in wrapping int32, from shifted weight codes and shifted zero points."""
+    c = unpack_i4(w_packed_shifted, signed=True).astype(np.int64)
+    K = c.shape[1]
+    z = half_to_int_rn(np.asarray(zeros_shifted, _F16).reshape(-1)).astype(np.int64)
+    return _wrap_i32(c.sum(axis=1) - K * z).astype(np.int32)
+
+
+def asym_rowsum_dequant(acc, scale_row, zeros_row, rowsum_row, scale_col, zeros_col, rowsum_adj_col, bias=None):
+    """corr = acc - z_row * adj_col - z_col * rowsum_row (wrapping int32);
+    y = h(f32(f32(corr) * (f32(s_row) * f32(s_col)))); with bias y = h(y + bias)."""
+    acc = np.asarray(acc, np.int64)
+    zr = half_to_int_rn(np.asarray(zeros_row, _F16).reshape(-1)).astype(np.int64)[:, None]
+    zc = half_to_int_rn(np.asarray(zeros_col, _F16).reshape(-1)).astype(np.int64)[None, :]
+    rr = np.asarray(rowsum_row, np.int64).reshape(-1, 1)
+    ac = np.asarray(rowsum_adj_col, np.int64).reshape(1, -1)
+    corr = _wrap_i32(_wrap_i32(acc - _wrap_i32(zr * ac)) - _wrap_i32(zc * rr)).astype(np.int32)
+    ss = _f32(np.asarray(scale_row, _F16).reshape(-1, 1)) * _f32(np.asarray(scale_col, _F16).reshape(1, -1))
+    with np.errstate(invalid="ignore", over="ignore"):
+        y = (corr.astype(_F32) * ss).astype(_F16)
+    if bias is not None:
+        y = add_bias(y, bias)
+    return y
+
+
+def weight_asym_shifted_from_linear(w):
+    """Weight preparation for the row-sum mode: per-row true min/max quantization
+    scale = h(h(max-min)/15), zero = h(rint(h(h(-min)/scale))), u = clamp(rint(h(w/scale)) + zero, 0, 15),
+    stored shifted.  Returns (packed u8, scale [N,1], zeros_shifted [N,1], rowsum_adj int32 [N])."""
+    q, s, zs, _ = asym_quant_shifted(w)
+    return q, s, zs, weight_rowsum_adj(q, zs)
+
+
+def linear4bit_asq_rowsum_forward(x, w_packed_shifted, w_scales, w_zeros_shifted, w_rowsum_adj, bias=None):
+    """AsymQuantizer(shifted) + row-sum epilogue.  Returns (y, acc, q_x, s_x, z_x, rowsum_x)."""
+    q_x, s_x, z_x, r_x = asym_quant_shifted(x)
+    acc = matmul_s4(q_x, w_packed_shifted)
+    y = asym_rowsum_dequant(acc, s_x, z_x, r_x, w_scales, w_zeros_shifted, w_rowsum_adj, bias)
+    return y, acc, q_x, s_x, z_x, r_x
+
+
+# ----------------------------------------------------------------------------------
 # A8  module forwards as compositions (qlinear4bit/nn/linear.py:42-56,104-115,
 #     167-176,239-250)
 # ----------------------------------------------------------------------------------

@@ -1,0 +1,163 @@
+"""Asymmetric forward with exact zero-point correction (row sums).  The reference has no such
+path, so parity is against the definition in include/duq_hip.h restated by the oracle; the
+oracle itself is pinned here by the integer identity and by dequantize-then-matmul in float64
+(a dropped term, a wrong sign or a transposed operand fails both)."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import duq_oracle as orc
+from tests import cases
+
+
+def _ints(z):
+    return np.rint(np.asarray(z, np.float64)).astype(np.int64)
+
+
+# ------------------------------------------------------------------ oracle pins (CPU)
+@pytest.mark.parametrize("M,N,K,seed", [(5, 7, 64, 0), (3, 4, 192, 1), (8, 2, 64, 2)])
+def test_oracle_rowsum_identity_and_closed_form(M, N, K, seed):
+    rng = np.random.default_rng(seed)
+    x = (rng.random((M, K)) * 6 - (seed == 1) * 2).astype(np.float16)   # nonnegative skew; one case crosses zero
+    w = (rng.standard_normal((N, K)) * 0.05).astype(np.float16)
+    wq, ws, wz, adj = orc.weight_asym_shifted_from_linear(w)
+    y, acc, qx, sx, zx, rx = orc.linear4bit_asq_rowsum_forward(x, wq, ws, wz, adj)
+
+    # shifted storage == unshifted codes / zeros minus 8
+    s0, z0 = orc.asym_scales_zeros(x)
+    u = orc.asym_quant_values(x, s0, z0)
+    cx = orc.unpack_i4(qx, signed=True).astype(np.int64)
+    assert np.array_equal(cx, u.astype(np.int64) - 8)
+    assert np.array_equal(orc.asym_quant(x, s0, z0) ^ 0x88, qx)
+    assert np.array_equal(_ints(zx), _ints(z0) - 8) and np.array_equal(sx, s0)
+    assert np.array_equal(rx, cx.sum(axis=1))
+
+    # integer identity, term by term from a brute-force triple loop
+    cw = orc.unpack_i4(wq, signed=True).astype(np.int64)
+    zxi, zwi = _ints(zx).reshape(-1), _ints(wz).reshape(-1)
+    want_corr = np.zeros((M, N), np.int64)
+    for m in range(M):
+        for n in range(N):
+            want_corr[m, n] = sum(int(cx[m, k] - zxi[m]) * int(cw[n, k] - zwi[n]) for k in range(K))
+    corr = acc.astype(np.int64) - zxi[:, None] * adj.astype(np.int64)[None, :] - zwi[None, :] * rx.astype(np.int64)[:, None]
+    assert np.array_equal(corr, want_corr)
+
+    # y is s_x * s_w * corr rounded: within one binary16 + one float32 rounding of the exact product
+    exact = sx.astype(np.float64) * ws.astype(np.float64).reshape(1, -1) * want_corr
+    assert np.all(np.abs(y.astype(np.float64) - exact) <= np.abs(exact) * (2.0 ** -11 + 2.0 ** -23) + 6e-8)
+    # and it is the product of the dequantized operands
+    ref = (sx.astype(np.float64) * (cx - zxi[:, None])) @ (ws.astype(np.float64) * (cw - zwi[:, None])).T
+    assert np.allclose(exact, ref, rtol=1e-12, atol=0)
+
+    # the point of the mode: close to the real product, where the reference-faithful path is not
+    true = x.astype(np.float64) @ w.astype(np.float64).T
+    err = np.abs(y.astype(np.float64) - true).max() / np.abs(true).max()
+    y_ref_mode, *_ = orc.linear4bit_asq_forward(x, *orc.weight_asym_from_linear(w))
+    err_ref_mode = np.abs(y_ref_mode.astype(np.float64) - true).max() / np.abs(true).max()
+    assert err < 0.25 and err < err_ref_mode
+
+
+def test_oracle_rowsum_bias_and_wrapping():
+    acc = np.array([[2 ** 31 - 5, -7]], np.int32)
+    sr = np.array([[0.5]], np.float16); zr = np.array([[-3.0]], np.float16); rr = np.array([10], np.int32)
+    sc = np.array([0.25, 2.0], np.float16); zc = np.array([1.0, -2.0], np.float16); ac = np.array([4, -6], np.int32)
+    y = orc.asym_rowsum_dequant(acc, sr, zr, rr, sc, zc, ac, bias=np.array([1.0, 0.5], np.float16))
+    # column 0: 2^31-5 + 12 - 10 wraps to -2^31 - 3 + ... ; computed by hand in Python integers
+    c0 = ((2 ** 31 - 5) - (-3) * 4 - 1 * 10 + 2 ** 31) % 2 ** 32 - 2 ** 31
+    c1 = -7 - (-3) * (-6) - (-2) * 10
+    want0 = np.float16(np.float32(c0) * np.float32(0.125)) + np.float16(1.0)
+    want1 = np.float16(np.float16(np.float32(c1) * np.float32(1.0)) + np.float16(0.5))
+    assert y[0, 1] == want1 and (y[0, 0] == want0 or (np.isinf(y[0, 0]) and np.isinf(want0)))
+    assert c1 == -5
+
+
+def test_abi_validation_rowsum_entries():
+    from duqlinear4bitcuda_amd import _lib
+    lib = _lib.load()
+    buf = (ctypes.c_char * 4096)()
+    P = (ctypes.addressof(buf) + 15) & ~15
+    assert lib.duq_quantize_rows_asym_shifted(P, 2, 64, P, P, P, None, None) == -1
+    assert lib.duq_quantize_rows_asym_shifted(P, 2, 48, P, P, P, P, None) == -2
+    assert lib.duq_quantize_rows_asym_shifted(P, 0, 64, None, None, None, None, None) == 0
+    assert lib.duq_linear4bit_forward_rowsum(P, P, P, None, P, P, P, P, None, 4, 4, 64, P, None) == -1
+    assert lib.duq_linear4bit_forward_rowsum(P, P, P, P, P, P, P, P, None, 4, 4, 96, P, None) == -3
+    assert lib.duq_asym_rowsum_dequant_host(P, P, P, P, P, P, None, None, 4, 4, P, None) == -1
+
+
+# ------------------------------------------------------------------ GPU parity
+@pytest.fixture(scope="module")
+def hip(dev):
+    from duqlinear4bitcuda_amd import _HIP
+    return _HIP
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,K", [(1, 64), (16, 4096), (300, 1024), (2048, 4096), (3, 11008), (2, 66048), (40, 32)])
+def test_gpu_quantize_rows_asym_shifted(hip, dev, M, K):
+    print("asym_shifted", M, K, flush=True)
+    x = cases.acts_uniform(M, K, seed=M + K) if K % 3 else cases.acts_outliers(M, K, seed=M + K)
+    wq, ws, wz, wr = orc.asym_quant_shifted(x)
+    q, s, z, r = hip.quantize_rows_asym_shifted(cases.t(x, dev))
+    assert np.array_equal(q.cpu().numpy(), wq)
+    assert cases.bits_equal(s.cpu().numpy(), ws) and cases.bits_equal(z.cpu().numpy(), wz)
+    assert np.array_equal(r.cpu().numpy(), wr)
+    # the unshifted kernel still gives the unshifted form
+    q0, s0, z0 = hip.quantize_rows_asym(cases.t(x, dev))
+    assert np.array_equal(q0.cpu().numpy() ^ 0x88, wq)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (4, 1000, 512), (16, 4096, 4096), (9, 300, 8192), (48, 96, 256),
+                                   (100, 257, 320), (512, 4096, 4096), (300, 1000, 4160), (2048, 4096, 1024)])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_gpu_rowsum_forward(hip, dev, M, N, K, with_bias):
+    """Every GEMM kernel family (dot, skinny, tile, stream; aligned and ragged epilogues) in row-sum mode:
+    fused == unfused == oracle, bit for bit."""
+    print("rowsum forward", M, N, K, with_bias, flush=True)
+    rng = np.random.default_rng(M + 3 * N + 7 * K)
+    x = cases.acts_uniform(M, K, seed=M + N + K)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float16)
+    wq, ws, wz, adj = orc.weight_asym_shifted_from_linear(w)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float16) if with_bias else None
+    want, acc, qx, sx, zx, rx = orc.linear4bit_asq_rowsum_forward(x, wq, ws, wz, adj, bias)
+    T = lambda v: cases.t(v, dev)
+    q, s, z, r = hip.quantize_rows_asym_shifted(T(x))
+    got = hip.linear4bit_forward_rowsum(q, s, z, r, T(wq), T(ws), T(wz), T(adj), None if bias is None else T(bias))
+    assert cases.bits_equal(got.cpu().numpy(), want)
+    acc_gpu = hip.matmul(q, T(wq))
+    assert np.array_equal(acc_gpu.cpu().numpy(), acc)
+    unfused = hip.asym_rowsum_dequant(acc_gpu, s, z, r, T(ws), T(wz), T(adj), None if bias is None else T(bias))
+    assert cases.bits_equal(unfused.cpu().numpy(), want)
+
+
+@pytest.mark.gpu
+def test_gpu_rowsum_module_config4(dev):
+    """Config 4 (M=512, K=N=4096, activations ~U[0,6]) through the module: weights prepared on the
+    device, forward equals the oracle, and the result is close to the fp16 layer it replaces."""
+    from duqlinear4bitcuda_amd.nn import Linear4bitASQRowSum
+    M, K, N = 512, 4096, 4096
+    x = cases.acts_uniform(M, K, seed=4)
+    g = torch.Generator().manual_seed(44)
+    lin = torch.nn.Linear(K, N, bias=True).half()
+    with torch.no_grad():
+        lin.weight.copy_((torch.randn(N, K, generator=g) * 0.02).half())
+        lin.bias.copy_(torch.randn(N, generator=g).half())
+    mod = Linear4bitASQRowSum.from_linear(lin.to(dev))
+    w = lin.weight.detach().cpu().numpy()
+    wq, ws, wz, adj = orc.weight_asym_shifted_from_linear(w)
+    assert np.array_equal(mod.weight.cpu().numpy(), wq)
+    assert cases.bits_equal(mod.weight_scales.cpu().numpy(), ws) and cases.bits_equal(mod.weight_zeros.cpu().numpy(), wz)
+    assert np.array_equal(mod.weight_rowsum.cpu().numpy(), adj)
+    y = mod(cases.t(x, dev).view(2, 256, K))
+    assert y.shape == (2, 256, N)
+    want, *_ = orc.linear4bit_asq_rowsum_forward(x, wq, ws, wz, adj, lin.bias.detach().cpu().numpy())
+    assert cases.bits_equal(y.view(M, N).cpu().numpy(), want)
+    mod.fused = False
+    assert cases.bits_equal(mod(cases.t(x, dev)).cpu().numpy(), want)
+    true = x.astype(np.float64) @ w.astype(np.float64).T + lin.bias.detach().cpu().numpy().astype(np.float64)
+    rel = np.linalg.norm(want.astype(np.float64) - true) / np.linalg.norm(true)
+    y_ref_mode, *_ = orc.linear4bit_asq_forward(x, *orc.weight_asym_from_linear(w), bias=lin.bias.detach().cpu().numpy())
+    rel_ref_mode = np.linalg.norm(y_ref_mode.astype(np.float64) - true) / np.linalg.norm(true)
+    assert rel < 0.25 and rel < 0.5 * rel_ref_mode, (rel, rel_ref_mode)  # 4-bit x 4-bit noise, not a broken correction
