@@ -146,6 +146,31 @@ def quantizer_section(dev):
     return out
 
 
+def asym_section(dev):
+    """Dual-uniform / asymmetric configuration (M=512, K=N=4096, activations ~U[0,6]): one module step
+    (quantize + GEMM + dequant, two launches) in the reference-faithful mode and in the row-sum mode."""
+    import torch
+
+    from duqlinear4bitcuda_amd.nn import Linear4bitASQ, Linear4bitASQRowSum
+
+    M, K, N = 512, 4096, 4096
+    g = torch.Generator().manual_seed(4)
+    x = (torch.rand(M, K, generator=g) * 6).half().to(dev)
+    lin = torch.nn.Linear(K, N, bias=False).half()
+    with torch.no_grad():
+        lin.weight.copy_((torch.randn(N, K, generator=g) * 0.02).half())
+    ref_mode = Linear4bitASQ.from_linear(lin).to(dev)
+    rowsum_mode = Linear4bitASQRowSum.from_linear(lin.to(dev))
+    true = x.float() @ lin.weight.float().t()
+    out = {"M": M, "N": N, "K": K}
+    for name, mod in (("reference_mode", ref_mode), ("rowsum_mode", rowsum_mode)):
+        us = graph_time_us([lambda: mod(x)] * 20)
+        y = mod(x).float()
+        out[name] = {"step_us": round(us, 2), "TOPS": round(2.0 * M * N * K / us / 1e6, 1),
+                     "rel_error_vs_fp32_matmul": round(float((y.detach() - true).norm() / true.norm()), 4)}
+    return out
+
+
 def cpu_baseline(x_cpu, wq_cpu, sw_cpu, ops, budget_s=15.0):
     """The reference's CPU fake-quant path (torch-CPU) on the same workload, host cores."""
     import torch
@@ -252,6 +277,7 @@ def main():
 
     decode = decode_section(dev, args.quick)
     quantizer = quantizer_section(dev)
+    asym = None if args.quick else asym_section(dev)
     best_decode = max(decode, key=lambda d: d["GBps"])
     roofline_decode = {"bound": "hbm", "kernel": "gemv_s4_dot_kernel (M<=4) / gemm_s4_skinny_kernel (M<=16)", "achieved": best_decode["GBps"],
                        "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": best_decode["frac_hbm"],
@@ -286,6 +312,7 @@ def main():
         "roofline_decode": roofline_decode,
         "decode": decode,
         "quantizer": quantizer,
+        "asym": asym,
         "cpu_baseline": cpu,
         "device": {"name": props.name, "arch": props.gcnArchName, "cus": props.multi_processor_count},
     }

@@ -31,6 +31,9 @@ fixes by definition instead ("parity unpinned" for exactly these corners):
     as "false" (the second scale/zero set), the same value it has for 1 <= col < 128.
   * float->int conversion of +-inf / NaN follows the PTX ``cvt.rni.s32.f16`` rule
     (saturate, NaN -> 0) and the following int add wraps modulo 2**32.
+The row-sum functions (``asym_quant_shifted`` ... ``linear4bit_asq_rowsum_forward``) restate a
+mode the reference does not have; there is nothing of the reference to be in parity with, and
+they are pinned by the integer identity and the float64 product of the dequantized operands.
 """
 from __future__ import annotations
 

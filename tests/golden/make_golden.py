@@ -1,5 +1,6 @@
 """Writes tests/golden/linear4bit_small.npz: seeded inputs and the expected packed codes,
-scales, int32 accumulators and fp16 outputs of the four Linear4bit forwards.
+scales, int32 accumulators and fp16 outputs of the four Linear4bit forwards and of the row-sum
+(exact zero-point correction) forward.
 
 The reference ships no golden vectors for this path (its tests only print), so these come
 from the pinned CPU oracle; the file freezes them so that a later change of the oracle or
@@ -52,6 +53,10 @@ def main():
     wd = orc.pack_i4(codes, sym=False)
     y, *_ = orc.linear4bit_duasq_forward(xa, wd, sa1, za1, sa2, za2, bias)
     out.update(duasq_w=wd, duasq_s1=sa1, duasq_z1=za1, duasq_s2=sa2, duasq_z2=za2, duasq_y=y)
+    # asymmetric with exact zero-point correction (row sums): signed-shifted codes, same activations
+    wr, sr, zr, adj = orc.weight_asym_shifted_from_linear(w)
+    y, acc, qx, sx, zx, rx = orc.linear4bit_asq_rowsum_forward(xa, wr, sr, zr, adj, bias)
+    out.update(rs_w=wr, rs_sw=sr, rs_zw=zr, rs_adj=adj, rs_y=y, rs_acc=acc, rs_qx=qx, rs_sx=sx, rs_zx=zx, rs_rx=rx)
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "linear4bit_small.npz")
     np.savez_compressed(path, **out)
     print(path, os.path.getsize(path), "bytes")

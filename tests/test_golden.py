@@ -31,6 +31,10 @@ def test_oracle_reproduces_the_fixture():
     y, *_ = orc.linear4bit_duasq_forward(G["asym_x"], G["duasq_w"], G["duasq_s1"], G["duasq_z1"], G["duasq_s2"],
                                         G["duasq_z2"], G["bias"])
     assert same16(y, G["duasq_y"])
+    y, acc, qx, sx, zx, rx = orc.linear4bit_asq_rowsum_forward(G["asym_x"], G["rs_w"], G["rs_sw"], G["rs_zw"], G["rs_adj"],
+                                                             G["bias"])
+    assert np.array_equal(qx, G["rs_qx"]) and np.array_equal(acc, G["rs_acc"]) and np.array_equal(rx, G["rs_rx"])
+    assert same16(sx, G["rs_sx"]) and same16(zx, G["rs_zx"]) and same16(y, G["rs_y"])
 
 
 def test_fixture_sanity():
@@ -40,6 +44,13 @@ def test_fixture_sanity():
     assert np.array_equal(a @ b.T, G["sym_q6_acc"])
     assert (G["sym_q6_qx"][3] == 0).all() and float(G["sym_q6_sx"][3, 0]) == 0.0   # the all-zero token
     assert orc.unpack_i4(G["sym_q6_qx"]).max() == 6 and orc.unpack_i4(G["sym_q7_qx"]).max() == 7
+    # row-sum vectors: shifted codes are the unshifted ones minus 8; sums and accumulators follow from the codes
+    assert np.array_equal(G["rs_qx"], G["asym_qx"] ^ 0x88)
+    cx = orc.unpack_i4(G["rs_qx"]).astype(np.int64)
+    cw = orc.unpack_i4(G["rs_w"]).astype(np.int64)
+    assert np.array_equal(cx.sum(1), G["rs_rx"]) and np.array_equal(cx @ cw.T, G["rs_acc"])
+    zw = np.rint(G["rs_zw"].astype(np.float64)).astype(np.int64).reshape(-1)
+    assert np.array_equal(cw.sum(1) - cw.shape[1] * zw, G["rs_adj"])
 
 
 @pytest.mark.gpu
@@ -77,3 +88,12 @@ def test_modules_reproduce_the_fixture(dev):
     for fused in (True, False):
         d.fused = fused
         assert same16(d(T("asym_x")).cpu().numpy(), G["duasq_y"])
+    r = qnn.Linear4bitASQRowSum(K, N, bias=True).to(dev)
+    r.load_state_dict({"weight": T("rs_w"), "weight_scales": T("rs_sw"), "weight_zeros": T("rs_zw"),
+                       "weight_rowsum": T("rs_adj"), "bias": T("bias")})
+    for fused in (True, False):
+        r.fused = fused
+        assert same16(r(T("asym_x")).cpu().numpy(), G["rs_y"])
+    p = r.quantizer(T("asym_x"))
+    assert np.array_equal(p.quantized_x.cpu().numpy(), G["rs_qx"]) and np.array_equal(p.rowsum_x.cpu().numpy(), G["rs_rx"])
+    assert same16(p.zeros_x.cpu().numpy(), G["rs_zx"])
