@@ -11,9 +11,9 @@
 // k order inside a tile only has to be the same for A and B.
 //
 // Four kernels, picked by shape in launch_epi():
-//  * stream kernel (prefill, M > 64 and at least 128 tiles of 128 x 256): weights go from
-//    global memory straight to registers, activations are expanded once into LDS,
-//    v_mfma_i32_32x32x32_i8 with a hand-ordered schedule (see the kernel);
+//  * stream kernel (prefill, M >= 128; tiles of 128, 64 or 32 rows x 256 columns, the height
+//    picked per shape): weights go from global memory straight to registers, activations are
+//    expanded once into LDS, v_mfma_i32_32x32x32_i8 with a hand-ordered schedule (see the kernel);
 //  * tile kernel (everything else above 16 rows): BM x BN x 128 tiles, 4 wavefronts (2 x 2),
 //    both operands expanded on the way into double-buffered LDS, v_mfma_i32_16x16x64_i8;
 //  * skinny kernel (decode, 5 <= M <= 16): one workgroup owns 16 output columns, its
@@ -239,7 +239,9 @@ __global__ __launch_bounds__(256) void gemm_s4_tile_kernel(GemmParams p)
 // stream kernel (prefill): weights global -> registers, activations through LDS,
 // v_mfma_i32_32x32x32_i8
 // ---------------------------------------------------------------------------------
-// Tile 128 (M) x 256 (N), 4 wavefronts side by side along N: every wavefront owns 64 weight
+// Tile 32*TM (M) x 256 (N), TM = 4 for large problems (described below; TM = 2 and 1 run the same
+// schedule with 4 and 2 MFMA slots per step and exist to give mid-size M one workgroup per
+// CU), 4 wavefronts side by side along N: every wavefront owns 64 weight
 // rows that no other wavefront of the workgroup needs, so weight fragments never go through
 // LDS: lane (l32, h) loads 16-byte piece i (0..3) = bytes [i*32 + h*16, +16) of the 128-byte
 // row segment of a 256-k chunk straight into registers.  The 128 activation rows are shared
@@ -280,12 +282,14 @@ __device__ __forceinline__ v4u buf_load16(__amdgpu_buffer_rsrc_t r, uint32_t vof
     return __builtin_bit_cast(v4u, __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)soff, 0));
 }
 
-template <int EPI, bool BIAS>
+template <int TM, int EPI, bool BIAS>
 __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
 {
-    constexpr int BM = 128, BN = 256;
-    constexpr int TM = 4, TN = 2;      // 32x32 tiles per wavefront: 128 x 64
-    constexpr int NXP = 4;             // 16-byte activation pieces per thread and chunk
+    static_assert(TM == 4 || TM == 2 || TM == 1, "32-row activation tiles per wavefront");
+    constexpr int BM = 32 * TM, BN = 256;
+    constexpr int TN = 2;              // 32x32 tiles per wavefront: BM x 64
+    constexpr int S = TM * TN;         // MFMA slots per step
+    constexpr int NXP = TM;            // 16-byte activation pieces per thread and chunk
     constexpr uint32_t kBuf = BM * kXStride;
 
     __shared__ __attribute__((aligned(16))) uint8_t lds[3 * kBuf];
@@ -346,14 +350,14 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
             const int i = step >> 1, par = step & 1;
             const bool okw = !G || (koff1 + i * 32 + h * 16 < kbytes);
 #pragma unroll
-            for (int slot = 0; slot < 8; ++slot) {
+            for (int slot = 0; slot < S; ++slot) {
                 const int b = slot >> 1, t = slot & 1;
                 asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0"
                              : "+a"(acc[t][b])
                              : "v"(wexp[i & 1][par][t]), "v"(fx[step & 1][b]));
                 __builtin_amdgcn_sched_barrier(0);
                 // ---- side work in the shadow of this MFMA
-                if (slot < 4) {  // next step's activation fragment for tile `slot`
+                if (slot < TM) {  // next step's activation fragment for tile `slot`
                     const uint8_t *src = step < 7 ? lds + cur + fragX + ((step + 1) >> 1) * 64 + ((step + 1) & 1) * 16
                                                   : lds + nxt + fragX;
                     fx[(step + 1) & 1][slot] = *reinterpret_cast<const v4i *>(src + slot * 32 * kXStride);
@@ -362,16 +366,25 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
                     wreg[slot][i] = buf_load16(rW, okw ? woff[slot] + i * 32 : kOobOffset, koff1);
                 if (step == 1 && slot < NXP)  // activations two chunks ahead
                     xreg[slot] = buf_load16(rX, okx ? xoff[slot] : kOobOffset, koff2);
-                if (slot >= 4) {  // expand the next weight piece of tile `par`, one word per slot
+                // expand the next weight piece of tile `par`: its four words over the last four slots (or
+                // two / one per slot when a step has fewer than four slots)
+                {
                     const int np = (i + 1) & 3;  // pieces 1, 2, 3 of this chunk, then piece 0 of the next
-                    expand_word(wreg[par][np], wexp[(i + 1) & 1][0][par], wexp[(i + 1) & 1][1][par], slot - 4);
+#pragma unroll
+                    for (int w = 0; w < 4; ++w)
+                        if ((S >= 4 ? S - 4 + w : w * S / 4) == slot)
+                            expand_word(wreg[par][np], wexp[(i + 1) & 1][0][par], wexp[(i + 1) & 1][1][par], w);
                 }
-                if (step >= 4 && slot < 4) {  // activations two chunks ahead -> third LDS buffer
-                    expand_word(xreg[step - 4], xe, xo, slot);
-                    if (slot == 3) {
-                        *reinterpret_cast<v4u *>(lds + nx2 + xlds[step - 4]) = xe;
-                        *reinterpret_cast<v4u *>(lds + nx2 + xlds[step - 4] + 16) = xo;
-                    }
+                if (step >= 8 - NXP) {  // activations two chunks ahead -> third LDS buffer, one piece per step
+#pragma unroll
+                    for (int w = 0; w < 4; ++w)
+                        if ((S >= 4 ? w : w * S / 4) == slot) {
+                            expand_word(xreg[step - (8 - NXP)], xe, xo, w);
+                            if (w == 3) {
+                                *reinterpret_cast<v4u *>(lds + nx2 + xlds[step - (8 - NXP)]) = xe;
+                                *reinterpret_cast<v4u *>(lds + nx2 + xlds[step - (8 - NXP)] + 16) = xo;
+                            }
+                        }
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -804,13 +817,34 @@ static void launch_epi(GemmParams &p, hipStream_t stream)
         return;
     }
 tiles_path:
-    // largest tile that still yields at least one workgroup per CU (256 CUs); small
-    // problems take the small tile to spread over the chip.
+    // Stream kernel with 128, 64 or 32 activation rows per workgroup: whole rounds of 256 workgroups
+    // (one per CU) cost about nchunks * c + f microseconds each, c and f measured per tile height;
+    // the cheapest wins.  Small problems (few column tiles) stay on the tile kernels.
     auto tiles = [&](uint32_t bm, uint32_t bn) { return ((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn); };
-    if (tiles(128, 256) >= 128 && p.M > 64) {
-        p.tiles_m = (p.M + 127) / 128;
+    int best_tm = 0;
+    if (p.M >= 128 && tiles(32, 256) >= 32) {
+        const float nch = (float)((p.K + kCK - 1) / kCK);
+        const float c_us[3] = {1.5f, 1.0f, 0.8f}, f_us[3] = {9.f, 7.f, 6.f};
+        float best = 0.f;
+        for (int k = 0; k < 3; ++k) {
+            const uint32_t t = tiles(128u >> k, 256);
+            const float cost = (float)((t + 255) / 256) * (nch * c_us[k] + f_us[k]);
+            if (best_tm == 0 || cost < best) {
+                best = cost;
+                best_tm = 4 >> k;
+            }
+        }
+    }
+    if (best_tm) {
+        p.tiles_m = (p.M + 32 * best_tm - 1) / (32 * best_tm);
         p.tiles_n = (p.N + 255) / 256;
-        hipLaunchKernelGGL((gemm_s4_stream_kernel<EPI, BIAS>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, stream, p);
+        const dim3 grid(p.tiles_m * p.tiles_n);
+        if (best_tm == 4)
+            hipLaunchKernelGGL((gemm_s4_stream_kernel<4, EPI, BIAS>), grid, dim3(256), 0, stream, p);
+        else if (best_tm == 2)
+            hipLaunchKernelGGL((gemm_s4_stream_kernel<2, EPI, BIAS>), grid, dim3(256), 0, stream, p);
+        else
+            hipLaunchKernelGGL((gemm_s4_stream_kernel<1, EPI, BIAS>), grid, dim3(256), 0, stream, p);
     } else if (tiles(128, 256) >= 256 && p.M > 64) {
         p.tiles_m = (p.M + 127) / 128;
         p.tiles_n = (p.N + 255) / 256;

@@ -198,7 +198,10 @@ def test_dequant_kernels(hip, dev, M, N):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (16, 4096, 4096), (16, 50, 128), (100, 257, 320), (512, 4096, 4096),
-                                   (130, 1000, 64)])
+                                   (130, 1000, 64),
+                                   # the stream kernel at its three tile heights, aligned and ragged epilogues:
+                                   # 64 rows (1024 x 4096, 900 x 4100), 32 rows (200 x 2051), 128 rows (1100 x 8200)
+                                   (1024, 4096, 512), (900, 4100, 128), (200, 2051, 192), (1100, 8200, 320)])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_fused_forward_equals_unfused_and_oracle(hip, dev, M, N, K, with_bias):
     _say("fused", M, N, K, with_bias)
