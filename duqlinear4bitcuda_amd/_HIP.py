@@ -217,6 +217,33 @@ def asym_dequant(q, scale_row, zeros_row, scale_col, zeros_col, bits: int = 32):
     return x
 
 
+def asym_batch_dequant(q, scale_row, zeros_row, scale_col, zeros_col, bits: int = 32):
+    """bindings.cpp:351-391 (kernel src/kernels/quant.cu:190-239): the asymmetric epilogue on a batch
+    of accumulator matrices q [batches, rows, cols], every batch with its own row / column
+    parameters (scale_row, zeros_row [batches, rows(,1)]; scale_col, zeros_col [batches, cols(,1)])."""
+    ts = (q, scale_row, zeros_row, scale_col, zeros_col)
+    _check("asym_batch_dequant", *ts)
+    _check_dtype("asym_batch_dequant", q, "q", torch.int32)
+    if q.dim() != 3:
+        raise RuntimeError(f"asym_batch_dequant: expected q [batches, rows, cols], got {tuple(q.shape)}")
+    batches, rows, cols = q.shape
+    for t, n, want in zip(ts[1:], ("scale_row", "zeros_row", "scale_col", "zeros_col"), (rows, rows, cols, cols)):
+        _check_dtype("asym_batch_dequant", t, n, torch.float16)
+        if t.dim() < 2 or t.size(1) != want or t.numel() != batches * want:
+            raise RuntimeError(f"asym_batch_dequant: expected {n} to have size {want} at dimension 1, got {tuple(t.shape)}")
+    _check_bits("asym_batch_dequant", bits)
+    x = torch.empty(q.shape, dtype=torch.float16, device=q.device)
+    fn = _lib.load().duq_asym_dequant_host
+    esz = 2
+    for b in range(batches):
+        st = _launch(q.device, fn, q.data_ptr() + b * rows * cols * 4, scale_row.data_ptr() + b * rows * esz,
+                     zeros_row.data_ptr() + b * rows * esz, scale_col.data_ptr() + b * cols * esz,
+                     zeros_col.data_ptr() + b * cols * esz, rows, cols, x.data_ptr() + b * rows * cols * esz)
+        if st:
+            _lib.check(st, "asym_batch_dequant")
+    return x
+
+
 def asym_dual_dequant(q, scale_row, zeros_row, scale_col_1, zeros_col_1, scale_col_2, zeros_col_2, bits: int = 32):
     """bindings.cpp:423-467."""
     ts = (q, scale_row, zeros_row, scale_col_1, zeros_col_1, scale_col_2, zeros_col_2)

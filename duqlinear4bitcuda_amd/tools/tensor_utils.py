@@ -94,6 +94,18 @@ def asym_dequant(q, scale_row, zeros_row, scale_col, zeros_col, bits=32):
                              bits).view(*lead, -1)
 
 
+def flatten_last_two_dim_and_return_shape(x: torch.Tensor):
+    return x.reshape(-1, x.shape[-2], x.shape[-1]), x.shape[:-2], x.shape[-2:]
+
+
+def asym_batch_dequant(q, scale_row, zeros_row, scale_col, zeros_col, bits=32):
+    """tensor_utils.py:116-123."""
+    assert q.dtype == torch.int32
+    assert scale_row.dtype == zeros_row.dtype == scale_col.dtype == zeros_col.dtype == torch.float16
+    q3, lead, last2 = flatten_last_two_dim_and_return_shape(q)
+    return _ops.asym_batch_dequant(q3, scale_row, zeros_row, scale_col, zeros_col, bits).view(*lead, last2[0], last2[1])
+
+
 def asym_dual_quant(q, scale_1, zeros1, scale_2, zeros2):
     """The reference wrapper asserts ``q.dtype == int32`` here (tensor_utils.py:126), which
     can never hold for the fp16 input the kernel takes; fp16 is what is checked."""

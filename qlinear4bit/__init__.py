@@ -9,6 +9,7 @@ _ALIASES = {
     "nn": "nn",
     "nn.linear": "nn.linear",
     "nn.quantizer": "nn.quantizer",
+    "nn.matmul": "nn.matmul",
     "tools": "tools",
     "tools.tensor_utils": "tools.tensor_utils",
     "tools.quantization": "tools.quantization",

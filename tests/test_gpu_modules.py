@@ -266,3 +266,54 @@ def test_libtorch_classes_fused_equals_three_step(shape):
     assert os.path.exists(exe), "tests/cpp/duq_torch_check is not built (run build())"
     r = subprocess.run([exe] + [str(v) for v in shape], capture_output=True, text=True, timeout=100)
     assert r.returncode == 0 and r.stdout.startswith("OK"), (r.returncode, r.stdout[-2000:], r.stderr[-2000:])
+
+
+@pytest.mark.gpu
+def test_sym_quant_matmul_module(dev):
+    """SymQuantMatMul (qlinear4bit/nn/matmul.py:69-84): both operands quantized per row, A @ B^T."""
+    from duqlinear4bitcuda_amd.nn import SymQuantMatMul
+    a = cases.acts_outliers(48, 256, seed=71)
+    b = cases.acts_normal(96, 256, seed=72)
+    sa, sb = orc.sym_scales(a), orc.sym_scales(b)
+    want = orc.sym_dequant(orc.matmul_s4(orc.sym_quant(a, sa), orc.sym_quant(b, sb)), sa, sb)
+    mod = SymQuantMatMul()
+    for fused in (True, False):
+        mod.fused = fused
+        got = mod(cases.t(a, dev), cases.t(b, dev)).cpu().numpy()
+        assert cases.bits_equal(got, want)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("transpose_b", [False, True])
+def test_asym_quant_matmul_module(dev, transpose_b):
+    """AsymQuantMatMul (qlinear4bit/nn/matmul.py:19-66): batched, per-batch-entry scales and zero
+    points, a B height that is not a multiple of 32 (the reference pads and unpads it)."""
+    from duqlinear4bitcuda_amd.nn import AsymQuantMatMul
+    from duqlinear4bitcuda_amd.tools import tensor_utils
+    lead, HA, HB, W = (2, 3), 40, 33, 128
+    a = cases.acts_uniform(6 * HA, W, seed=81).reshape(*lead, HA, W)
+    b = cases.acts_normal(6 * HB, W, seed=82).reshape(*lead, HB, W)
+    want = np.empty((*lead, HA, HB), np.float16)
+    accs = np.empty((6, HA, HB), np.int32)
+    params = []
+    for i in range(2):
+        for j in range(3):
+            sa, za = orc.asym_scales_zeros(a[i, j])
+            sb, zb = orc.asym_scales_zeros(b[i, j])
+            acc = orc.matmul_s4(orc.asym_quant(a[i, j], sa, za), orc.asym_quant(b[i, j], sb, zb))
+            want[i, j] = orc.asym_dequant(acc, sa, za, sb, zb)
+            accs[i * 3 + j] = acc
+            params.append((sa, za, sb, zb))
+    mod = AsymQuantMatMul(transpose_B=transpose_b)
+    tb = cases.t(b, dev)
+    if transpose_b:
+        tb = tb.transpose(-1, -2).contiguous()
+    for fused in (True, False):
+        mod.fused = fused
+        got = mod(cases.t(a, dev), tb)
+        assert got.shape == (*lead, HA, HB)
+        assert cases.bits_equal(got.cpu().numpy(), want)
+    # the batched dequant op on its own, 4-D accumulators as the reference wrapper accepts them
+    st = lambda k: cases.t(np.stack([p[k] for p in params]), dev)
+    got = tensor_utils.asym_batch_dequant(cases.t(accs.reshape(*lead, HA, HB), dev), st(0), st(1), st(2), st(3))
+    assert cases.bits_equal(got.cpu().numpy(), want)
