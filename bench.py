@@ -279,7 +279,7 @@ def main():
     quantizer = quantizer_section(dev)
     asym = None if args.quick else asym_section(dev)
     best_decode = max(decode, key=lambda d: d["GBps"])
-    roofline_decode = {"bound": "hbm", "kernel": "gemv_s4_dot_kernel (M<=4) / gemm_s4_skinny_kernel (M<=16)", "achieved": best_decode["GBps"],
+    roofline_decode = {"bound": "hbm", "kernel": "gemv_s4_dot_kernel (M=1) / gemm_s4_skinny_kernel (2<=M<=16)", "achieved": best_decode["GBps"],
                        "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": best_decode["frac_hbm"],
                        "shape": {k: best_decode[k] for k in ("M", "N", "K")}, "traffic": None}
 

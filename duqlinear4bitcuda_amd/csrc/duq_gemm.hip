@@ -16,9 +16,10 @@
 //    expanded once into LDS, v_mfma_i32_32x32x32_i8 with a hand-ordered schedule (see the kernel);
 //  * tile kernel (everything else above 16 rows): BM x BN x 128 tiles, 4 wavefronts (2 x 2),
 //    both operands expanded on the way into double-buffered LDS, v_mfma_i32_16x16x64_i8;
-//  * skinny kernel (decode, 5 <= M <= 16): one workgroup owns 16 output columns, its
+//  * skinny kernel (decode, 2 <= M <= 16): one workgroup owns 16 output columns, its
 //    wavefronts split K, fragments go from global memory straight to registers;
-//  * dot kernel (decode, M <= 4): v_dot8_i32_i4 on the packed nibbles, a pure HBM stream.
+//  * dot kernel (decode, M = 1; M <= 4 for long rows): v_dot8_i32_i4 on the packed nibbles, a pure HBM
+//    stream.
 // In the MFMA kernels the weight operand goes to the MFMA "A" side, so each lane ends up
 // with four consecutive output columns of one row.
 #include "duq_epilogue.h"
@@ -568,7 +569,7 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
 }
 
 // ---------------------------------------------------------------------------------
-// skinny kernel (5 <= M <= 16; also M <= 4 when the dot kernel's limits do not hold)
+// skinny kernel (2 <= M <= 16; also one row when the dot kernel's limits do not hold)
 // ---------------------------------------------------------------------------------
 // Workgroup = WAVES wavefronts that split K; it walks `tiles_per_wg` consecutive 16-column
 // tiles.  Wavefront w owns 64-byte row segments [w*S, (w+1)*S), S <= 8: lane (l16, g) holds
@@ -675,7 +676,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_s4_skinny_kernel(GemmParams p
 }
 
 // ---------------------------------------------------------------------------------
-// dot kernel (decode, M <= 4): weight streaming on v_dot8_i32_i4
+// dot kernel (decode, M = 1, and M <= 4 when K > 16384 or M = 2 with K > 4096): weight streaming on v_dot8_i32_i4
 // ---------------------------------------------------------------------------------
 // The signed 4-bit dot product instruction consumes packed nibbles as they lie in memory,
 // so nothing is expanded and no MFMA is needed: the kernel is a pure HBM stream.
@@ -782,7 +783,10 @@ static void launch_epi(GemmParams &p, hipStream_t stream)
 {
     const uint64_t wbytes = (uint64_t)p.N * (p.K / 2);
     const uint32_t xstride = ((p.K / 2 + 127) / 128) * 128;
-    if (p.M <= 4 && wbytes < 0xFFFFFF00ull && 4 * xstride <= 60 * 1024 && p.K > 0) {
+    // dot kernel: always for one row and for rows too long for the skinny kernel; two rows when K > 4096
+    // (measured: the MFMA skinny kernel is level or ahead for 2-4 rows otherwise)
+    const bool dot_shape = p.M == 1 || p.K > 16384 || (p.M == 2 && p.K > 4096);
+    if (p.M <= 4 && dot_shape && wbytes < 0xFFFFFF00ull && 4 * xstride <= 60 * 1024 && p.K > 0) {
         const dim3 grid((p.N + 7) / 8);
         if (p.M == 1)
             hipLaunchKernelGGL((gemv_s4_dot_kernel<1, EPI, BIAS>), grid, dim3(256), 1 * xstride, stream, p);

@@ -132,6 +132,8 @@ def _rand_packed(rng, rows, K):
     (17, 64, 64), (64, 64, 128), (65, 130, 192), (100, 257, 320), (128, 256, 4096), (300, 520, 1024),
     (2048, 4096, 256), (256, 4096, 11008), (130, 1000, 64), (16, 16, 8192), (2, 48, 28672), (7, 48, 28672),
     (9, 40000, 64), (16, 33000, 192), (12, 17000, 8192), (5, 100, 16384),
+    # one to four rows: dot kernel (one row; two rows with K > 4096; up to four with K > 16384), skinny otherwise
+    (2, 512, 8192), (2, 300, 4096), (3, 300, 20480), (4, 64, 28672), (3, 1000, 2048), (4, 520, 8192), (1, 77, 20480),
 ])
 def test_matmul_bit_exact(hip, dev, M, N, K):
     _say("matmul", M, N, K)
@@ -201,7 +203,9 @@ def test_dequant_kernels(hip, dev, M, N):
                                    (130, 1000, 64),
                                    # the stream kernel at its three tile heights, aligned and ragged epilogues:
                                    # 64 rows (1024 x 4096, 900 x 4100), 32 rows (200 x 2051), 128 rows (1100 x 8200)
-                                   (1024, 4096, 512), (900, 4100, 128), (200, 2051, 192), (1100, 8200, 320)])
+                                   (1024, 4096, 512), (900, 4100, 128), (200, 2051, 192), (1100, 8200, 320),
+                                   # two to four rows on either decode kernel
+                                   (2, 512, 8192), (3, 300, 20480), (4, 1000, 4096), (2, 300, 4096)])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_fused_forward_equals_unfused_and_oracle(hip, dev, M, N, K, with_bias):
     _say("fused", M, N, K, with_bias)
