@@ -1,7 +1,7 @@
 // duq_torch.hpp - header-only libtorch (C++) twin of the Linear4bit path over the C ABI in
 // duq_hip.h, with the class and function names of the reference's C++ API:
-//   PackedQuantizedTensor, Quantizer4bit, DeQuantizer4bit, sym_quant, sym_dequant,
-//   sym_dual_dequant, pack_i4          include/quant_tensor.h:11-90, src/module/quant_tensor.cu
+//   PackedQuantizedTensor, PackedDoubleQuantizedTensor, Quantizer4bit, DeQuantizer4bit, sym_quant,
+//   sym_dual_quant, sym_dequant, sym_dual_dequant, pack_i4          include/quant_tensor.h:11-90, src/module/quant_tensor.cu
 //   Linear4bit, Linear4bitDUQ          include/linear.h:31-60,    src/module/linear.cu:83-281
 // Tensors live on a ROCm device ("cuda" device type in PyTorch-ROCm); every call launches on
 // torch's current HIP stream.  Argument errors raise c10::Error through TORCH_CHECK like the
@@ -60,6 +60,18 @@ public:
     torch::Device device() const { return quantized_x.device(); }
 };
 
+// quantized activation with two scales: columns < 10 and the rest (include/quant_tensor.h:29-45)
+class PackedDoubleQuantizedTensor {
+public:
+    torch::Tensor quantized_x;
+    torch::Tensor scale_1;
+    torch::Tensor scale_2;
+    PackedDoubleQuantizedTensor(torch::Tensor quantized_x, torch::Tensor scale_1, torch::Tensor scale_2)
+        : quantized_x(std::move(quantized_x)), scale_1(std::move(scale_1)), scale_2(std::move(scale_2)) {}
+    torch::IntArrayRef sizes() const { return quantized_x.sizes(); }
+    torch::Device device() const { return quantized_x.device(); }
+};
+
 // ---- tensor-level ops (src/module/quant_tensor.cu:11-148)
 inline torch::Tensor sym_quant(const torch::Tensor &x, const torch::Tensor &scale, int qmax = DUQ_QMAX_SYM_DEVICE)
 {
@@ -71,6 +83,22 @@ inline torch::Tensor sym_quant(const torch::Tensor &x, const torch::Tensor &scal
     check_status(duq_sym_quant_host_qmax(half_ptr(x), half_ptr(scale), rows, cols, cd, qmax, q.data_ptr<uint8_t>(),
                                          current_stream(x)),
                  "sym_quant");
+    return q;
+}
+
+// columns < 10 of every row use scale_1, the others scale_2 (src/module/quant_tensor.cu:31-57)
+inline torch::Tensor sym_dual_quant(const torch::Tensor &x, const torch::Tensor &scale_1, const torch::Tensor &scale_2)
+{
+    check_device_tensor(x, "sym_dual_quant", "x");
+    check_device_tensor(scale_1, "sym_dual_quant", "scale_1");
+    check_device_tensor(scale_2, "sym_dual_quant", "scale_2");
+    TORCH_CHECK(x.dim() == 2 && scale_1.size(0) == x.size(0) && scale_2.size(0) == x.size(0),
+                "sym_dual_quant: expected both scales to have size ", x.size(0), " at dimension 0");
+    const uint32_t rows = x.size(0), cols = x.size(1), cd = (cols + 1) / 2;
+    auto q = torch::empty({rows, cd}, torch::dtype(torch::kUInt8).device(x.device()));
+    check_status(duq_sym_dual_quant_host(half_ptr(x), half_ptr(scale_1), half_ptr(scale_2), rows, cols, cd,
+                                         q.data_ptr<uint8_t>(), current_stream(x)),
+                 "sym_dual_quant");
     return q;
 }
 

@@ -34,6 +34,17 @@ int main(int argc, char **argv)
     auto q2 = duq::sym_quant(x.view({-1, K}), p.scale.view(-1));
     if (!torch::equal(q2, p.quantized_x.view({-1, K / 2}))) { std::puts("FAIL quantizer codes"); return 1; }
 
+    // dual quantizer op: with equal scales it is the plain one; with different scales columns >= 10 follow scale_2
+    auto sx1 = p.scale.view(-1);
+    if (!torch::equal(duq::sym_dual_quant(x.view({-1, K}), sx1, sx1), q2)) { std::puts("FAIL sym_dual_quant equal scales"); return 1; }
+    auto qd = duq::sym_dual_quant(x.view({-1, K}), sx1, sx1 * 2);
+    auto qhalf = duq::sym_quant(x.view({-1, K}), sx1 * 2);
+    if (!torch::equal(qd.slice(1, 0, 5), q2.slice(1, 0, 5)) || !torch::equal(qd.slice(1, 5), qhalf.slice(1, 5))) {
+        std::puts("FAIL sym_dual_quant split"); return 1;
+    }
+    duq::PackedDoubleQuantizedTensor pd(qd, p.scale, p.scale * 2);
+    if (pd.sizes() != qd.sizes()) { std::puts("FAIL PackedDoubleQuantizedTensor"); return 1; }
+
     auto l = duq::Linear4bit::from_float(lin, ws);
     auto y = l.forward(p);
     auto acc = duq::matmul(p.quantized_x.view({-1, K / 2}), l.weight);
