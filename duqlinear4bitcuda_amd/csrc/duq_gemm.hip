@@ -10,12 +10,14 @@
 // 256*|C| stays below 2^31 for K <= 131008.  Integer accumulation is order-free, so the
 // k order inside a tile only has to be the same for A and B.
 //
-// Four kernels, picked by shape in launch_epi():
+// Five kernels, picked by shape in launch_epi():
 //  * stream kernel (prefill, M >= 128; tiles of 128, 64 or 32 rows x 256 columns, the height
 //    picked per shape): weights go from global memory straight to registers, activations are
 //    expanded once into LDS, v_mfma_i32_32x32x32_i8 with a hand-ordered schedule (see the kernel);
 //  * tile kernel (everything else above 16 rows): BM x BN x 128 tiles, 4 wavefronts (2 x 2),
 //    both operands expanded on the way into double-buffered LDS, v_mfma_i32_16x16x64_i8;
+//  * ring kernel (17 <= M <= 64, and up to 16 rows longer than 8192 elements): packed activations of all
+//    rows in LDS, every wavefront streams whole weight rows through a ring of loads;
 //  * skinny kernel (decode, 2 <= M <= 16): one workgroup owns 16 output columns, its
 //    wavefronts split K, fragments go from global memory straight to registers;
 //  * dot kernel (decode, M = 1; M <= 4 for long rows): v_dot8_i32_i4 on the packed nibbles, a pure HBM
@@ -676,6 +678,126 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_s4_skinny_kernel(GemmParams p
 }
 
 // ---------------------------------------------------------------------------------
+// ring kernel (17 <= M <= 64, and M <= 16 with rows too long for the skinny kernel)
+// ---------------------------------------------------------------------------------
+// The packed activations of all 16*RB rows sit in LDS for the whole K range (rows padded so that
+// 16 rows x 16 bytes cover every bank once); a wavefront owns a 16-column tile and a K slice
+// and streams the weights of that slice through a ring of kRing 128-bit loads per lane that is
+// refilled slot by slot, across tile boundaries too, so the loads in flight never drain.  Every
+// weight fragment is expanded once and multiplied with the RB activation fragments read from
+// LDS (one expansion each).  No barrier inside the K loop; when several wavefronts split K for
+// a tile their partial sums meet in LDS once per tile.  More rows than 16*RB are covered by
+// blockIdx.y (groups of 16*RB rows, each streaming the weights again).
+constexpr int kRing = 8;  // 128-bit weight loads in flight per lane
+
+template <int XBYTES, int RB, int EPI, bool BIAS>
+__global__ __launch_bounds__(256) void gemm_s4_ring_kernel(GemmParams p)
+{
+    constexpr uint32_t WAVES = 4, T = WAVES * 64;
+    constexpr uint32_t XS = XBYTES + 16;  // LDS row stride = 16 (mod 256)
+    __shared__ __attribute__((aligned(16))) uint8_t xs[16 * RB * XS];
+    __shared__ v4i part[WAVES][RB][64];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u, wave = tid >> 6;
+    const uint32_t l16 = lane & 15u, g = lane >> 4;
+    const uint32_t kbytes = p.K >> 1;
+    const uint32_t segs = (kbytes + 63) / 64;
+    const uint32_t kslices = p.tiles_m;  // (fields reused) wavefronts that split K for one tile: 1, 2 or 4
+    const uint32_t items = p.tiles_n;    // tiles each wavefront walks through
+    const uint32_t tiles_per_wg = WAVES / kslices;
+    const uint32_t slice = wave % kslices, tsub = wave / kslices;
+    const uint32_t sps = (segs + kslices - 1) / kslices;  // 64-byte segments per slice
+    const uint32_t seg_lo = slice * sps;
+    const uint32_t nblk = (sps + kRing - 1) / kRing;
+    const uint32_t m_base = blockIdx.y * (16 * RB);
+
+    const __amdgpu_buffer_rsrc_t rW = make_rsrc(p.B, p.N * kbytes);  // rows past N read as zero
+    const __amdgpu_buffer_rsrc_t rX = make_rsrc(p.A, p.M * kbytes);  // rows past M read as zero
+
+    v4u ring[kRing];
+    auto tile_of = [&](uint32_t it) { return (blockIdx.x * items + it) * tiles_per_wg + tsub; };
+    auto issue = [&](uint32_t it, uint32_t blk, int j) {
+        const uint32_t row = tile_of(it) * 16 + l16;
+        const uint32_t sg = blk * kRing + j;
+        const uint32_t off = (seg_lo + sg) * 64 + g * 16;
+        const bool ok = it < items && row < p.N && sg < sps && off < kbytes;
+        ring[j] = buf_load16(rW, ok ? row * kbytes + off : kOobOffset, 0);
+    };
+#pragma unroll
+    for (int j = 0; j < kRing; ++j) issue(0, 0, j);  // the first weights are under way before the activations
+
+    {
+        const uint32_t ppr = kbytes >> 4;  // 16-byte pieces per row
+        for (uint32_t c = tid; c < ppr; c += T) {
+#pragma unroll
+            for (int r0 = 0; r0 < 16 * RB; r0 += 16) {
+                v4u v[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) v[r] = buf_load16(rX, (m_base + r0 + r) * kbytes + c * 16, 0);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) *reinterpret_cast<v4u *>(xs + (r0 + r) * XS + c * 16) = v[r];
+            }
+        }
+    }
+    __syncthreads();
+
+    const bool vec_ok = (EPI < 0) ? (p.N % 4 == 0 && reinterpret_cast<uintptr_t>(p.C) % 16 == 0)
+                                  : (p.N % 4 == 0 && reinterpret_cast<uintptr_t>(p.y) % 8 == 0);
+    const uint32_t xbase = l16 * XS + g * 16;
+    for (uint32_t it = 0; it < items; ++it) {
+        v4i acc[RB];
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) acc[rb] = v4i{0, 0, 0, 0};
+        for (uint32_t blk = 0; blk < nblk; ++blk) {
+            const bool last = blk + 1 == nblk;
+            const uint32_t nit = last ? it + 1 : it, nb = last ? 0 : blk + 1;
+#pragma unroll
+            for (int j = 0; j < kRing; ++j) {
+                const v4u w = ring[j];
+                issue(nit, nb, j);
+                // segments past the slice carry zero weights; their activation read only has to stay inside the row
+                const uint32_t xoff = min((seg_lo + blk * kRing + j) * 64, (uint32_t)XBYTES - 64);
+                v4u we, wo;
+                expand_nibbles(w, we, wo);
+#pragma unroll
+                for (int rb = 0; rb < RB; ++rb) {
+                    const v4u x = *reinterpret_cast<const v4u *>(xs + rb * 16 * XS + xbase + xoff);
+                    v4u xe, xo;
+                    expand_nibbles(x, xe, xo);
+                    acc[rb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i, we),
+                                                                   __builtin_bit_cast(v4i, xe), acc[rb], 0, 0, 0);
+                    acc[rb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i, wo),
+                                                                   __builtin_bit_cast(v4i, xo), acc[rb], 0, 0, 0);
+                }
+            }
+        }
+        const uint32_t tile = tile_of(it);
+        if (kslices > 1) {
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) part[wave][rb][lane] = acc[rb];
+            __syncthreads();
+            if (slice == 0)
+                for (uint32_t s2 = 1; s2 < kslices; ++s2)
+#pragma unroll
+                    for (int rb = 0; rb < RB; ++rb) {
+                        const v4i o = part[wave + s2][rb][lane];
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) acc[rb][r] += o[r];
+                    }
+            __syncthreads();  // the partial sums are consumed before the next tile overwrites them
+        }
+        if (slice == 0) {
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[rb][r] >>= 8;
+                store_quad<EPI, BIAS>(p, m_base + rb * 16 + l16, tile * 16 + g * 4, acc[rb], vec_ok);
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------
 // dot kernel (decode, M = 1, and M <= 4 when K > 16384 or M = 2 with K > 4096): weight streaming on v_dot8_i32_i4
 // ---------------------------------------------------------------------------------
 // The signed 4-bit dot product instruction consumes packed nibbles as they lie in memory,
@@ -796,6 +918,42 @@ static void launch_epi(GemmParams &p, hipStream_t stream)
             hipLaunchKernelGGL((gemv_s4_dot_kernel<4, EPI, BIAS>), grid, dim3(256), 4 * xstride, stream, p);
         return;
     }
+    {
+        // ring kernel: 17..64 rows whose packed activations fit in LDS, and up to 16 rows that are too long
+        // for the skinny kernel's registers
+        const uint32_t rb_all = (p.M + 15) / 16;
+        const uint32_t rb_max = p.K <= 4096 ? 4 : (p.K <= 8192 ? 2 : 1);  // 16-row blocks whose activations fit in LDS
+        const uint32_t rb = std::min(rb_all, rb_max);
+        const uint32_t row_groups = (rb_all + rb - 1) / rb;
+        const bool long_rows = p.M <= 16 && p.K > 8192;
+        // (several row groups re-stream the weights: with enough column tiles to fill the chip the stream
+        // kernel's 32-row tiles are cheaper then)
+        const uint32_t tiles32 = ((p.M + 31) / 32) * ((p.N + 255) / 256);
+        const bool mid_rows = p.M > 16 && p.M <= 64 && !(row_groups > 1 && tiles32 >= 128);
+        if ((long_rows || mid_rows) && p.K <= 16384 && wbytes < 0xFFFFFF00ull && p.K > 0) {
+            const uint32_t ntiles = (p.N + 15) / 16;
+            const uint32_t segs = (p.K / 2 + 63) / 64;
+            // wavefronts splitting K for one tile: as few as give the chip ~2048 wavefronts, slices of at
+            // least 512 bytes per row
+            uint32_t kslices = 1;
+            while (ntiles * kslices < 2048 && kslices < 4 && segs / (kslices * 2) >= (uint32_t)kRing) kslices *= 2;
+            const uint32_t groups = (ntiles + 4 / kslices - 1) / (4 / kslices);
+            const uint32_t xbytes = p.K <= 4096 ? 2048 : (p.K <= 8192 ? 4096 : 8192);
+            const uint32_t lds = 16 * rb * (xbytes + 16) + 4 * rb * 1024;
+            const uint32_t slots = 256 * std::max(1u, std::min(8u, (160u * 1024) / lds));
+            p.tiles_m = kslices;
+            p.tiles_n = (groups + slots - 1) / slots;
+            const dim3 grid((groups + p.tiles_n - 1) / p.tiles_n, row_groups);
+#define DUQ_RING(X, R) hipLaunchKernelGGL((gemm_s4_ring_kernel<X, R, EPI, BIAS>), grid, dim3(256), 0, stream, p)
+            if (xbytes == 8192) DUQ_RING(8192, 1);
+            else if (xbytes == 4096) DUQ_RING(4096, 2);
+            else if (rb == 2) DUQ_RING(2048, 2);
+            else if (rb == 3) DUQ_RING(2048, 3);
+            else DUQ_RING(2048, 4);
+#undef DUQ_RING
+            return;
+        }
+    }
     if (p.M <= 16) {
         const uint32_t ntiles = (p.N + 15) / 16;
         const uint32_t segs = (p.K / 2 + 63) / 64;
@@ -826,7 +984,7 @@ tiles_path:
     // the cheapest wins.  Small problems (few column tiles) stay on the tile kernels.
     auto tiles = [&](uint32_t bm, uint32_t bn) { return ((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn); };
     int best_tm = 0;
-    if (p.M >= 128 && tiles(32, 256) >= 32) {
+    if (p.M > 32 && tiles(32, 256) >= 32) {
         const float nch = (float)((p.K + kCK - 1) / kCK);
         const float c_us[3] = {1.5f, 1.0f, 0.8f}, f_us[3] = {9.f, 7.f, 6.f};
         float best = 0.f;

@@ -134,6 +134,9 @@ def _rand_packed(rng, rows, K):
     (9, 40000, 64), (16, 33000, 192), (12, 17000, 8192), (5, 100, 16384),
     # one to four rows: dot kernel (one row; two rows with K > 4096; up to four with K > 16384), skinny otherwise
     (2, 512, 8192), (2, 300, 4096), (3, 300, 20480), (4, 64, 28672), (3, 1000, 2048), (4, 520, 8192), (1, 77, 20480),
+    # ring kernel: 17..64 rows (2, 3, 4 row blocks; several row groups when K is long) and long rows up to 16
+    (17, 4096, 4096), (33, 300, 8192), (64, 520, 11008), (48, 4099, 1024), (40, 64, 16384), (16, 300, 11008),
+    (9, 4096, 16384), (64, 11008, 4096), (50, 1000, 4160),
 ])
 def test_matmul_bit_exact(hip, dev, M, N, K):
     _say("matmul", M, N, K)
@@ -205,7 +208,9 @@ def test_dequant_kernels(hip, dev, M, N):
                                    # 64 rows (1024 x 4096, 900 x 4100), 32 rows (200 x 2051), 128 rows (1100 x 8200)
                                    (1024, 4096, 512), (900, 4100, 128), (200, 2051, 192), (1100, 8200, 320),
                                    # two to four rows on either decode kernel
-                                   (2, 512, 8192), (3, 300, 20480), (4, 1000, 4096), (2, 300, 4096)])
+                                   (2, 512, 8192), (3, 300, 20480), (4, 1000, 4096), (2, 300, 4096),
+                                   # ring kernel
+                                   (33, 300, 8192), (64, 520, 11008), (48, 4099, 1024), (16, 300, 11008), (20, 4096, 4096)])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_fused_forward_equals_unfused_and_oracle(hip, dev, M, N, K, with_bias):
     _say("fused", M, N, K, with_bias)
