@@ -112,7 +112,8 @@ def decode_section(dev, quick):
     out = []
     shapes = [(1, 4096, 4096), (4, 4096, 4096), (16, 4096, 4096), (1, 11008, 4096), (16, 11008, 4096)]
     if not quick:
-        shapes += [(4, 11008, 4096), (1, 28672, 8192), (1, 8192, 28672), (16, 28672, 8192)]
+        shapes += [(4, 11008, 4096), (32, 4096, 4096), (64, 11008, 4096), (16, 4096, 11008), (1, 28672, 8192), (1, 8192, 28672),
+                   (16, 28672, 8192)]
     for (M, N, K) in shapes:
         wbytes = N * K // 2
         nbuf = min(96, max(3, int(600e6 // wbytes) + 1))
@@ -279,7 +280,7 @@ def main():
     quantizer = quantizer_section(dev)
     asym = None if args.quick else asym_section(dev)
     best_decode = max(decode, key=lambda d: d["GBps"])
-    roofline_decode = {"bound": "hbm", "kernel": "gemv_s4_dot_kernel (M=1) / gemm_s4_skinny_kernel (2<=M<=16)", "achieved": best_decode["GBps"],
+    roofline_decode = {"bound": "hbm", "kernel": "gemv_s4_dot_kernel (M=1) / gemm_s4_skinny_kernel (2<=M<=16) / gemm_s4_ring_kernel (17<=M<=64, long rows)", "achieved": best_decode["GBps"],
                        "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": best_decode["frac_hbm"],
                        "shape": {k: best_decode[k] for k in ("M", "N", "K")}, "traffic": None}
 
