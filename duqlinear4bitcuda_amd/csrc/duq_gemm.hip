@@ -919,7 +919,8 @@ static void launch_epi(GemmParams &p, hipStream_t stream)
         return;
     }
     {
-        // ring kernel: 17..64 rows whose packed activations fit in LDS, and up to 16 rows that are too long
+        // ring kernel: 17..256 rows in groups whose packed activations fit in LDS (a few groups only, or a
+        // problem too narrow to fill the chip with stream-kernel tiles), and up to 16 rows that are too long
         // for the skinny kernel's registers
         const uint32_t rb_all = (p.M + 15) / 16;
         const uint32_t rb_max = p.K <= 4096 ? 4 : (p.K <= 8192 ? 2 : 1);  // 16-row blocks whose activations fit in LDS
@@ -929,7 +930,8 @@ static void launch_epi(GemmParams &p, hipStream_t stream)
         // (several row groups re-stream the weights: with enough column tiles to fill the chip the stream
         // kernel's 32-row tiles are cheaper then)
         const uint32_t tiles32 = ((p.M + 31) / 32) * ((p.N + 255) / 256);
-        const bool mid_rows = p.M > 16 && p.M <= 64 && !(row_groups > 1 && tiles32 >= 128);
+        const bool few_groups = row_groups <= 2 || (row_groups <= 6 && tiles32 < 64) || tiles32 < 48;
+        const bool mid_rows = p.M > 16 && p.M <= 256 && few_groups && !(row_groups > 1 && tiles32 >= 128);
         if ((long_rows || mid_rows) && p.K <= 16384 && wbytes < 0xFFFFFF00ull && p.K > 0) {
             const uint32_t ntiles = (p.N + 15) / 16;
             const uint32_t segs = (p.K / 2 + 63) / 64;

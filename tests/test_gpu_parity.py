@@ -137,6 +137,8 @@ def _rand_packed(rng, rows, K):
     # ring kernel: 17..64 rows (2, 3, 4 row blocks; several row groups when K is long) and long rows up to 16
     (17, 4096, 4096), (33, 300, 8192), (64, 520, 11008), (48, 4099, 1024), (40, 64, 16384), (16, 300, 11008),
     (9, 4096, 16384), (64, 11008, 4096), (50, 1000, 4160),
+    # ring kernel with several row groups: 65..256 rows of a narrow or short problem
+    (100, 1000, 4096), (128, 4096, 4096), (200, 520, 8192), (90, 300, 11008), (256, 1024, 8192),
 ])
 def test_matmul_bit_exact(hip, dev, M, N, K):
     _say("matmul", M, N, K)
@@ -210,7 +212,8 @@ def test_dequant_kernels(hip, dev, M, N):
                                    # two to four rows on either decode kernel
                                    (2, 512, 8192), (3, 300, 20480), (4, 1000, 4096), (2, 300, 4096),
                                    # ring kernel
-                                   (33, 300, 8192), (64, 520, 11008), (48, 4099, 1024), (16, 300, 11008), (20, 4096, 4096)])
+                                   (33, 300, 8192), (64, 520, 11008), (48, 4099, 1024), (16, 300, 11008), (20, 4096, 4096),
+                                   (100, 1000, 4096), (200, 520, 8192)])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_fused_forward_equals_unfused_and_oracle(hip, dev, M, N, K, with_bias):
     _say("fused", M, N, K, with_bias)
