@@ -452,3 +452,125 @@ def asym_rowsum_dequant(q, scale_row, zeros_row, rowsum_row, scale_col, zeros_co
     if st:
         _lib.check(st, name)
     return x
+
+
+# ---- the forward on the 6-bit float matrix path (exact; not in the reference) --------------
+
+EPI_ASYM_ROWSUM = 4
+
+
+def weight_shadow_bf6(w: torch.Tensor) -> torch.Tensor:
+    """E3M2 shadow of packed-int4 weights ``w`` uint8 [N, K/2]: uint8 [N, 3K/4] in the
+    library's tile order.  Made once per weight tensor.  N % 16 == 0, K % 128 == 0."""
+    name = "weight_shadow_bf6"
+    if not isinstance(w, torch.Tensor):
+        raise RuntimeError(f"{name}: argument #0 is not a tensor")
+    _fast_check(name, "w", w, _U8, None)
+    if w.dim() != 2:
+        raise RuntimeError(f"{name}: expected a 2-D tensor, got {tuple(w.shape)}")
+    N, kb = w.shape
+    out = torch.empty((N, kb * 3 // 2), dtype=_U8, device=w.device)
+    st = _launch(w.device, _lib.load().duq_weight_shadow_bf6, w.data_ptr(), N, kb * 2, out.data_ptr())
+    if st:
+        _lib.check(st, name)
+    return out
+
+
+def activation_shadow_bf6(xq: torch.Tensor) -> torch.Tensor:
+    """E3M2 shadow of packed-int4 activations uint8 [..., K/2]: uint8 [..., 3K/4] (per row:
+    the 16-byte parts of its K/32 blocks, then the 8-byte parts).  K % 128 == 0."""
+    name = "activation_shadow_bf6"
+    if not isinstance(xq, torch.Tensor):
+        raise RuntimeError(f"{name}: argument #0 is not a tensor")
+    _fast_check(name, "xq", xq, _U8, None)
+    kb = xq.shape[-1]
+    M = xq.numel() // kb if kb else 0
+    out = torch.empty(xq.shape[:-1] + (kb * 3 // 2,), dtype=_U8, device=xq.device)
+    st = _launch(xq.device, _lib.load().duq_activation_shadow_bf6, xq.data_ptr(), M, kb * 2, out.data_ptr())
+    if st:
+        _lib.check(st, name)
+    return out
+
+
+def linear4bit_forward_bf6(mode, x_bf6, scale_x, zeros_x, w_bf6, w_scale_1, w_zeros_1=None, w_scale_2=None,
+                           w_zeros_2=None, bias=None, rowsum_x=None, w_rowsum_adj=None):
+    """``linear4bit_forward`` (modes 0-3) or ``linear4bit_forward_rowsum`` (mode 4) on E3M2
+    shadows: ``x_bf6`` uint8 [..., 3K/4], ``w_bf6`` uint8 [N, 3K/4].  Bit-identical results."""
+    name = "linear4bit_forward_bf6"
+    if not isinstance(x_bf6, torch.Tensor) or not isinstance(w_bf6, torch.Tensor):
+        raise RuntimeError(f"{name}: x_bf6 and w_bf6 must be tensors")
+    dev = x_bf6.device
+    _fast_check(name, "x_bf6", x_bf6, _U8, None)
+    _fast_check(name, "w_bf6", w_bf6, _U8, dev)
+    kb = x_bf6.shape[-1]
+    if w_bf6.dim() != 2 or w_bf6.shape[1] != kb:
+        raise RuntimeError(f"{name}: shadow row length differs: x {tuple(x_bf6.shape)} vs w {tuple(w_bf6.shape)}")
+    if kb % 96:
+        raise RuntimeError(f"{name}: shadow rows must hold a multiple of 128 elements (96 bytes), got {kb} bytes")
+    M = x_bf6.numel() // kb if kb else 0
+    N = w_bf6.shape[0]
+    ptrs = []
+    for t, what, dt, n in ((scale_x, "scale_x", _F16, M), (zeros_x, "zeros_x", _F16, M), (rowsum_x, "rowsum_x", _I32, M),
+                           (w_scale_1, "w_scale_1", _F16, N), (w_zeros_1, "w_zeros_1", _F16, N),
+                           (w_scale_2, "w_scale_2", _F16, N), (w_zeros_2, "w_zeros_2", _F16, N),
+                           (w_rowsum_adj, "w_rowsum_adj", _I32, N), (bias, "bias", _F16, N)):
+        if t is None:
+            ptrs.append(None)
+            continue
+        _fast_check(name, what, t, dt, dev)
+        if t.numel() != n:
+            _check_size0(name, t.reshape(-1), what, n)
+        ptrs.append(t.data_ptr())
+    y = torch.empty(x_bf6.shape[:-1] + (N,), dtype=_F16, device=dev)
+    st = _launch(dev, _lib.load().duq_linear4bit_forward_bf6, mode, x_bf6.data_ptr(), ptrs[0], ptrs[1], ptrs[2],
+                 w_bf6.data_ptr(), ptrs[3], ptrs[4], ptrs[5], ptrs[6], ptrs[7], ptrs[8], M, N, kb * 4 // 3, y.data_ptr())
+    if st:
+        _lib.check(st, name)
+    return y
+
+
+def quantize_rows_sym_bf6(x: torch.Tensor, clip: float = 1.0, qmax: int = 6, with_q: bool = True):
+    """``quantize_rows_sym`` that also writes the E3M2 shadow of the codes: returns
+    (q or None, x_bf6 uint8 [..., 3K/4], scales).  K % 128 == 0."""
+    name = "quantize_rows_sym_bf6"
+    if not isinstance(x, torch.Tensor):
+        raise RuntimeError(f"{name}: argument #0 is not a tensor")
+    _fast_check(name, "x", x, _F16, None)
+    shape = x.shape
+    cols = shape[-1]
+    rows = x.numel() // cols if cols else 0
+    lead = shape[:-1]
+    dev = x.device
+    q = torch.empty(lead + (cols // 2,), dtype=_U8, device=dev) if with_q else None
+    b = torch.empty(lead + (cols * 3 // 4,), dtype=_U8, device=dev)
+    s = torch.empty(lead + (1,), dtype=_F16, device=dev)
+    st = _launch(dev, _lib.load().duq_quantize_rows_sym_bf6, x.data_ptr(), rows, cols, float(clip), qmax,
+                 q.data_ptr() if with_q else None, b.data_ptr(), s.data_ptr())
+    if st:
+        _lib.check(st, name)
+    return q, b, s
+
+
+def quantize_rows_asym_bf6(x: torch.Tensor, shifted: bool = False, with_q: bool = True):
+    """``quantize_rows_asym`` (or ``quantize_rows_asym_shifted``) that also writes the E3M2
+    shadow: returns (q or None, x_bf6, scale, zeros[, rowsum])."""
+    name = "quantize_rows_asym_bf6"
+    if not isinstance(x, torch.Tensor):
+        raise RuntimeError(f"{name}: argument #0 is not a tensor")
+    _fast_check(name, "x", x, _F16, None)
+    shape = x.shape
+    cols = shape[-1]
+    rows = x.numel() // cols if cols else 0
+    lead = shape[:-1]
+    dev = x.device
+    q = torch.empty(lead + (cols // 2,), dtype=_U8, device=dev) if with_q else None
+    b = torch.empty(lead + (cols * 3 // 4,), dtype=_U8, device=dev)
+    s = torch.empty(lead + (1,), dtype=_F16, device=dev)
+    z = torch.empty(lead + (1,), dtype=_F16, device=dev)
+    r = torch.empty(lead, dtype=_I32, device=dev) if shifted else None
+    st = _launch(dev, _lib.load().duq_quantize_rows_asym_bf6, x.data_ptr(), rows, cols,
+                 q.data_ptr() if with_q else None, b.data_ptr(), s.data_ptr(), z.data_ptr(),
+                 r.data_ptr() if shifted else None)
+    if st:
+        _lib.check(st, name)
+    return (q, b, s, z, r) if shifted else (q, b, s, z)

@@ -105,7 +105,7 @@ int duq_quantize_rows_sym(const duq_half *x, uint32_t rows, uint32_t cols, float
     if (!x || !q || !scale) return DUQ_E_NULL;
     if (cols % 32 != 0) return DUQ_E_SHAPE;
     if (!aligned(x, 16) || !aligned(q, 16)) return DUQ_E_ALIGN;
-    return duq::launch_quantize_rows_sym(x, rows, cols, clip, qmax, q, scale, as_stream(stream));
+    return duq::launch_quantize_rows_sym(x, rows, cols, clip, qmax, q, scale, nullptr, as_stream(stream));
 }
 
 int duq_quantize_rows_asym(const duq_half *x, uint32_t rows, uint32_t cols, uint8_t *q, duq_half *scale,
@@ -115,7 +115,7 @@ int duq_quantize_rows_asym(const duq_half *x, uint32_t rows, uint32_t cols, uint
     if (!x || !q || !scale || !zeros) return DUQ_E_NULL;
     if (cols % 32 != 0) return DUQ_E_SHAPE;
     if (!aligned(x, 16) || !aligned(q, 16)) return DUQ_E_ALIGN;
-    return duq::launch_quantize_rows_asym(x, rows, cols, q, scale, zeros, nullptr, as_stream(stream));
+    return duq::launch_quantize_rows_asym(x, rows, cols, q, scale, zeros, nullptr, nullptr, as_stream(stream));
 }
 
 int duq_quantize_rows_asym_shifted(const duq_half *x, uint32_t rows, uint32_t cols, uint8_t *q, duq_half *scale,
@@ -125,7 +125,7 @@ int duq_quantize_rows_asym_shifted(const duq_half *x, uint32_t rows, uint32_t co
     if (!x || !q || !scale || !zeros || !rowsum) return DUQ_E_NULL;
     if (cols % 32 != 0) return DUQ_E_SHAPE;
     if (!aligned(x, 16) || !aligned(q, 16)) return DUQ_E_ALIGN;
-    return duq::launch_quantize_rows_asym(x, rows, cols, q, scale, zeros, rowsum, as_stream(stream));
+    return duq::launch_quantize_rows_asym(x, rows, cols, q, scale, zeros, rowsum, nullptr, as_stream(stream));
 }
 
 int duq_matmul_host_4bit(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N, uint32_t K, int32_t *C,
@@ -221,6 +221,75 @@ int duq_linear4bit_forward_rowsum(const uint8_t *xq, const duq_half *scale_x, co
     duq::Epilogue e{DUQ_EPI_ASYM_ROWSUM, scale_x, zeros_x, w_scale, w_zeros, nullptr, nullptr, bias, rowsum_x,
                     w_rowsum_adj};
     return duq::launch_gemm_s4(xq, w, M, N, K, nullptr, &e, y, as_stream(stream));
+}
+
+int duq_quantize_rows_sym_bf6(const duq_half *x, uint32_t rows, uint32_t cols, float clip, int32_t qmax, uint8_t *q,
+                              uint8_t *x_bf6, duq_half *scale, duq_stream_t stream)
+{
+    if (int e = check_qmax(qmax)) return e;
+    if (rows == 0 || cols == 0) return DUQ_OK;
+    if (!x || !x_bf6 || !scale) return DUQ_E_NULL;
+    if (cols % 128 != 0) return DUQ_E_SHAPE;
+    if (!aligned(x, 16) || !aligned(q, 16) || !aligned(x_bf6, 16)) return DUQ_E_ALIGN;
+    return duq::launch_quantize_rows_sym(x, rows, cols, clip, qmax, q, scale, x_bf6, as_stream(stream));
+}
+
+int duq_quantize_rows_asym_bf6(const duq_half *x, uint32_t rows, uint32_t cols, uint8_t *q, uint8_t *x_bf6,
+                               duq_half *scale, duq_half *zeros, int32_t *rowsum, duq_stream_t stream)
+{
+    if (rows == 0 || cols == 0) return DUQ_OK;
+    if (!x || !x_bf6 || !scale || !zeros) return DUQ_E_NULL;
+    if (cols % 128 != 0) return DUQ_E_SHAPE;
+    if (!aligned(x, 16) || !aligned(q, 16) || !aligned(x_bf6, 16)) return DUQ_E_ALIGN;
+    return duq::launch_quantize_rows_asym(x, rows, cols, q, scale, zeros, rowsum, x_bf6, as_stream(stream));
+}
+
+int duq_weight_shadow_bf6(const uint8_t *w, uint32_t N, uint32_t K, uint8_t *w_bf6, duq_stream_t stream)
+{
+    if (N == 0 || K == 0) return DUQ_OK;
+    if (!w || !w_bf6) return DUQ_E_NULL;
+    if (K % 128 != 0) return DUQ_E_KALIGN;
+    if (N % 16 != 0) return DUQ_E_SHAPE;
+    if (K > 131008u) return DUQ_E_TOO_LARGE;
+    if (!aligned(w, 16) || !aligned(w_bf6, 16)) return DUQ_E_ALIGN;
+    return duq::launch_weight_shadow_bf6(w, N, K, w_bf6, as_stream(stream));
+}
+
+int duq_activation_shadow_bf6(const uint8_t *xq, uint32_t M, uint32_t K, uint8_t *x_bf6, duq_stream_t stream)
+{
+    if (M == 0 || K == 0) return DUQ_OK;
+    if (!xq || !x_bf6) return DUQ_E_NULL;
+    if (K % 128 != 0) return DUQ_E_KALIGN;
+    if (K > 131008u) return DUQ_E_TOO_LARGE;
+    if (!aligned(xq, 16) || !aligned(x_bf6, 16)) return DUQ_E_ALIGN;
+    return duq::launch_activation_shadow_bf6(xq, M, K, x_bf6, as_stream(stream));
+}
+
+int duq_linear4bit_forward_bf6(int32_t mode, const uint8_t *x_bf6, const duq_half *scale_x, const duq_half *zeros_x,
+                               const int32_t *rowsum_x, const uint8_t *w_bf6, const duq_half *w_scale_1,
+                               const duq_half *w_zeros_1, const duq_half *w_scale_2, const duq_half *w_zeros_2,
+                               const int32_t *w_rowsum_adj, const duq_half *bias, uint32_t M, uint32_t N, uint32_t K,
+                               duq_half *y, duq_stream_t stream)
+{
+    if (mode < DUQ_EPI_SYM || mode > DUQ_EPI_ASYM_ROWSUM) return DUQ_E_MODE;
+    if (M == 0 || N == 0) return DUQ_OK;
+    if (!x_bf6 || !w_bf6 || !scale_x || !w_scale_1 || !y) return DUQ_E_NULL;
+    if (K == 0 || K % 128 != 0) return DUQ_E_KALIGN;
+    if (N % 16 != 0) return DUQ_E_SHAPE;
+    if (K > 131008u) return DUQ_E_TOO_LARGE;
+    const bool asym = mode == DUQ_EPI_ASYM || mode == DUQ_EPI_ASYM_DUAL || mode == DUQ_EPI_ASYM_ROWSUM;
+    const bool dual = mode == DUQ_EPI_SYM_DUAL || mode == DUQ_EPI_ASYM_DUAL;
+    if (asym && (!zeros_x || !w_zeros_1)) return DUQ_E_NULL;
+    if (dual && !w_scale_2) return DUQ_E_NULL;
+    if (asym && dual && !w_zeros_2) return DUQ_E_NULL;
+    if (mode == DUQ_EPI_ASYM_ROWSUM && (!rowsum_x || !w_rowsum_adj)) return DUQ_E_NULL;
+    // the kernel fetches column parameters four at a time and stores whole 16-byte pieces
+    if (!aligned(x_bf6, 16) || !aligned(w_bf6, 16) || !aligned(y, 16) || !aligned(w_scale_1, 8) ||
+        !aligned(w_zeros_1, 8) || !aligned(w_scale_2, 8) || !aligned(w_zeros_2, 8) || !aligned(bias, 8) ||
+        !aligned(w_rowsum_adj, 16))
+        return DUQ_E_ALIGN;
+    duq::Epilogue e{mode, scale_x, zeros_x, w_scale_1, w_zeros_1, w_scale_2, w_zeros_2, bias, rowsum_x, w_rowsum_adj};
+    return duq::launch_gemm_bf6(x_bf6, w_bf6, M, N, K, e, y, as_stream(stream));
 }
 
 }  // extern "C"

@@ -1,0 +1,383 @@
+// The same int4 x int4 GEMM on the 6-bit floating point matrix path of gfx950.
+//
+// Every int4 value -8..7 is exactly an E3M2 ("bf6") number, every product of two of them is
+// an integer of at most 7 bits, and the float32 accumulator of v_mfma_f32_16x16x128_f8f6f4
+// holds every integer below 2^24 exactly.  |C| <= 64*K < 2^24 for K <= 131008 (the bound of
+// the integer kernels), all partial sums are integers below 2^24 whatever the order, so the
+// float32 result converted back to int32 is the integer result bit for bit.  The instruction
+// runs at twice the rate of the i8 MFMA and the operands need no expansion in the loop.
+//
+// Operands are "shadows" of the packed-int4 tensors, made once (weights) or by the quantizer
+// (activations).  A block is 32 consecutive k of one row: 32 codes x 6 bits = 24 bytes, as
+// v_cvt_scalef32_pk32_bf6_f16 writes them; it is kept as a 16-byte part and an 8-byte part
+// so that every load is naturally aligned.
+//   activation shadow  [M][K/32 x 16 B | K/32 x 8 B]      (row-major, two planes per row)
+//   weight shadow      [N/16][K/128][64 lanes x 16 B | 64 lanes x 8 B]
+//                      lane l of a (16-row tile, 128-k step) holds the block of row l % 16,
+//                      k-block l / 16: the fragment order of the MFMA, so a wavefront load is
+//                      one contiguous 1 KB (512 B) span.
+// K % 128 == 0 and N % 16 == 0: no padding anywhere.
+//
+// Kernel: tile 128 (M) x 256 (N) per workgroup, 4 wavefronts side by side along N (128 x 64
+// each: 8 x 4 MFMA tiles, 128 accumulator registers).  Weights go global -> registers (a ring
+// of four 128-k steps), activations global -> registers -> LDS (three buffers of 256 k, one
+// barrier per buffer) -> fragments read two MFMA groups ahead.  The weight operand is the
+// MFMA "A" side, so a lane ends up with four consecutive output columns of one row.
+#include "duq_epilogue.h"
+#include "duq_launch.h"
+#include "duq_tiles.h"
+#include <type_traits>
+
+namespace duq {
+
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef int v6i __attribute__((ext_vector_type(6)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef _Float16 v32h __attribute__((ext_vector_type(32)));
+
+// ---------------------------------------------------------------------------------
+// weight shadow
+// ---------------------------------------------------------------------------------
+// 32 signed nibbles (16 bytes, element 2j in the low nibble of byte j) -> one bf6 block.
+// Position 8d + 2i + h of the block holds nibble i + 4h of word d (the order the quantizer
+// kernels produce cheaply); both operands use it, and the sum over k does not care.
+__device__ __forceinline__ v6i bf6_block_from_nibbles(const v4u w)
+{
+    v32h f;
+#pragma unroll
+    for (int pos = 0; pos < 32; ++pos) {
+        const int d = pos >> 3, e = ((pos & 7) >> 1) + 4 * (pos & 1);
+        const int v = ((int)(w[d] << (28 - 4 * e))) >> 28;
+        f[pos] = (f16)(float)v;
+    }
+    return __builtin_bit_cast(v6i, __builtin_amdgcn_cvt_scalef32_pk32_bf6_f16(f, 1.0f));
+}
+
+__global__ __launch_bounds__(256) void weight_shadow_kernel(const uint8_t *w, uint32_t N, uint32_t K, uint8_t *out)
+{
+    const uint32_t ksteps = K / 128;
+    const uint64_t total = (uint64_t)(N / 16) * ksteps * 64;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (uint64_t)gridDim.x * blockDim.x) {
+        const uint32_t lane = (uint32_t)(i & 63u);
+        const uint64_t ts = i >> 6;  // tile * ksteps + step
+        const uint32_t step = (uint32_t)(ts % ksteps), tile = (uint32_t)(ts / ksteps);
+        const uint32_t n = tile * 16 + (lane & 15u), kb = step * 4 + (lane >> 4);
+        const v4u raw = *reinterpret_cast<const v4u *>(w + (uint64_t)n * (K / 2) + kb * 16);
+        const v6i b = bf6_block_from_nibbles(raw);
+        uint8_t *dst = out + ts * 1536;
+        *reinterpret_cast<v4i *>(dst + lane * 16) = v4i{b[0], b[1], b[2], b[3]};
+        *reinterpret_cast<v2i *>(dst + 1024 + lane * 8) = v2i{b[4], b[5]};
+    }
+}
+
+int launch_weight_shadow_bf6(const uint8_t *w, uint32_t N, uint32_t K, uint8_t *out, hipStream_t stream)
+{
+    const uint64_t total = (uint64_t)(N / 16) * (K / 128) * 64;
+    if (total == 0) return 0;
+    const uint32_t blocks = (uint32_t)std::min<uint64_t>((total + 255) / 256, 1u << 16);
+    hipLaunchKernelGGL(weight_shadow_kernel, dim3(blocks), dim3(256), 0, stream, w, N, K, out);
+    return (int)hipGetLastError();
+}
+
+// activation shadow from packed nibbles (the quantizers write it directly; this is the
+// stand-alone conversion for tensors quantized elsewhere)
+__global__ __launch_bounds__(256) void activation_shadow_kernel(const uint8_t *q, uint32_t M, uint32_t K, uint8_t *out)
+{
+    const uint32_t nblk = K / 32;
+    const uint64_t total = (uint64_t)M * nblk;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (uint64_t)gridDim.x * blockDim.x) {
+        const uint32_t b = (uint32_t)(i % nblk);
+        const uint64_t m = i / nblk;
+        const v4u raw = *reinterpret_cast<const v4u *>(q + m * (K / 2) + b * 16);
+        const v6i f = bf6_block_from_nibbles(raw);
+        uint8_t *row = out + m * (uint64_t)nblk * 24;
+        *reinterpret_cast<v4i *>(row + b * 16) = v4i{f[0], f[1], f[2], f[3]};
+        *reinterpret_cast<v2i *>(row + (uint64_t)nblk * 16 + b * 8) = v2i{f[4], f[5]};
+    }
+}
+
+int launch_activation_shadow_bf6(const uint8_t *q, uint32_t M, uint32_t K, uint8_t *out, hipStream_t stream)
+{
+    const uint64_t total = (uint64_t)M * (K / 32);
+    if (total == 0) return 0;
+    const uint32_t blocks = (uint32_t)std::min<uint64_t>((total + 255) / 256, 1u << 16);
+    hipLaunchKernelGGL(activation_shadow_kernel, dim3(blocks), dim3(256), 0, stream, q, M, K, out);
+    return (int)hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------------
+// GEMM
+// ---------------------------------------------------------------------------------
+// Workgroup barrier that waits for this wavefront's LDS traffic only.  __syncthreads() also
+// drains the vector memory counter, which here would wait for the weight and activation
+// prefetches issued just before it (a full memory latency per chunk).
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+struct Bf6Params {
+    const uint8_t *X;  // activation shadow
+    const uint8_t *W;  // weight shadow
+    uint32_t M, N, K;
+    uint16_t *y;
+    Epilogue epi;
+    uint32_t tiles_m, tiles_n;
+};
+
+constexpr uint32_t kP0Stride = 144;  // LDS bytes per row, 16-byte parts of the 8 blocks of a chunk + pad
+constexpr uint32_t kP1Stride = 80;   // LDS bytes per row, 8-byte parts + pad
+
+template <int EPI, bool BIAS>
+__global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
+{
+    constexpr int BM = 128, BN = 256;
+    constexpr int TMI = 8, TNI = 4;  // 16 x 16 MFMA tiles per wavefront: 128 rows x 64 columns
+    constexpr uint32_t kP1Base = BM * kP0Stride;
+    constexpr uint32_t kBuf = BM * (kP0Stride + kP1Stride);
+    constexpr int MODE = EPI;
+
+    __shared__ __attribute__((aligned(16))) uint8_t lds[3 * kBuf];
+
+    uint32_t tile_m, tile_n;
+    tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+    const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u, wave = tid >> 6;
+    const uint32_t l16 = lane & 15u, kb = lane >> 4;
+    const uint32_t nblk = p.K / 32;
+    const uint32_t row_bytes = nblk * 24, p1off = nblk * 16;
+    const uint32_t ksteps = p.K / 128;
+    const uint32_t nchunks = (ksteps + 1) / 2;
+
+    const uint32_t wtiles = min(p.N - n0, (uint32_t)BN) / 16;
+    const __amdgpu_buffer_rsrc_t rW =
+        make_rsrc(p.W + (uint64_t)(n0 / 16) * ksteps * 1536, wtiles * ksteps * 1536);
+    const __amdgpu_buffer_rsrc_t rX =
+        make_rsrc(p.X + (uint64_t)m0 * row_bytes, min(p.M - m0, (uint32_t)BM) * row_bytes);
+
+    // weight fragment (ni, step g): 1536 bytes at ((wave*4 + ni) * ksteps + g) * 1536
+    const uint32_t wv0 = wave * 4 * ksteps * 1536 + lane * 16, wv1 = wave * 4 * ksteps * 1536 + 1024 + lane * 8;
+    // (the scalar offset is not part of the hardware range check: tiles past N and steps past K are
+    // redirected explicitly)
+    auto load_w = [&](v6i &dst, int ni, uint32_t g) {
+        const uint32_t soff = (ni * ksteps + g) * 1536;
+        const bool ok = g < ksteps && wave * 4 + ni < wtiles;
+        const v4i a = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rW, (int)(ok ? wv0 : kOobOffset), (int)soff, 0));
+        const v2i b = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(rW, (int)(ok ? wv1 : kOobOffset), (int)soff, 0));
+        dst = v6i{a[0], a[1], a[2], a[3], b[0], b[1]};
+    };
+    auto load_w0 = [&](v6i &dst, int ni, uint32_t g) {
+        const uint32_t soff = (ni * ksteps + g) * 1536;
+        const v4i a = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rW, (int)(g < ksteps && wave * 4 + ni < wtiles ? wv0 : kOobOffset), (int)soff, 0));
+        dst[0] = a[0], dst[1] = a[1], dst[2] = a[2], dst[3] = a[3];
+    };
+    auto load_w1 = [&](v6i &dst, int ni, uint32_t g) {
+        const uint32_t soff = (ni * ksteps + g) * 1536;
+        const v2i b = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(rW, (int)(g < ksteps && wave * 4 + ni < wtiles ? wv1 : kOobOffset), (int)soff, 0));
+        dst[4] = b[0], dst[5] = b[1];
+    };
+
+    // activation pieces of a chunk (256 k = 8 blocks): 4 of plane 0 and 2 of plane 1 per thread
+    uint32_t xoff[6], xlds[6];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t row = (tid >> 3) + j * 32, piece = tid & 7u;
+        xoff[j] = row * row_bytes + piece * 16;
+        xlds[j] = row * kP0Stride + piece * 16;
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const uint32_t row = (tid >> 2) + j * 64, piece = tid & 3u;
+        xoff[4 + j] = row * row_bytes + p1off + piece * 16;
+        xlds[4 + j] = kP1Base + row * kP1Stride + piece * 16;
+    }
+    auto load_x = [&](v4u &dst, int j, uint32_t c) {  // piece j of chunk c; pieces of a step past K read as zero
+        const uint32_t blk = c * 8 + (j < 4 ? (tid & 7u) : (tid & 3u) * 2);
+        dst = buf_load16(rX, blk < nblk ? xoff[j] : kOobOffset, j < 4 ? c * 128 : c * 64);
+    };
+
+    // fragment of rows mi*16 + l16, k-step s of a chunk: plane 0 + mi*16*kP0Stride + s*64, plane 1 + ... + s*32
+    const uint32_t frag0 = l16 * kP0Stride + kb * 16, frag1 = kP1Base + l16 * kP1Stride + kb * 8;
+
+    v6i wf[4][TNI];   // weight fragments [ring slot][column tile]
+    v6i xf[4];        // activation fragments, ring over mi
+    v4u xreg[6];
+    v4f acc[TMI][TNI];
+#pragma unroll
+    for (int a = 0; a < TMI; ++a)
+#pragma unroll
+        for (int b = 0; b < TNI; ++b) acc[a][b] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    auto read_x0 = [&](v6i &dst, uint32_t buf, int mi, int s) {
+        const v4i a = *reinterpret_cast<const v4i *>(lds + buf + frag0 + mi * 16 * kP0Stride + s * 64);
+        dst[0] = a[0], dst[1] = a[1], dst[2] = a[2], dst[3] = a[3];
+    };
+    auto read_x1 = [&](v6i &dst, uint32_t buf, int mi, int s) {
+        const v2i b = *reinterpret_cast<const v2i *>(lds + buf + frag1 + mi * 16 * kP1Stride + s * 32);
+        dst[4] = b[0], dst[5] = b[1];
+    };
+
+    // ---- prologue: weights of steps 0..3, activations of chunks 0 and 1 -> LDS, chunk 2 -> registers
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+#pragma unroll
+        for (int ni = 0; ni < TNI; ++ni) load_w(wf[g][ni], ni, g);
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+#pragma unroll
+        for (int j = 0; j < 6; ++j) load_x(xreg[j], j, q);
+#pragma unroll
+        for (int j = 0; j < 6; ++j) *reinterpret_cast<v4u *>(lds + q * kBuf + xlds[j]) = xreg[j];
+    }
+#pragma unroll
+    for (int j = 0; j < 6; ++j) load_x(xreg[j], j, 2);
+    lds_barrier();
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi) {
+        read_x0(xf[mi], 0, mi, 0);
+        read_x1(xf[mi], 0, mi, 0);
+    }
+
+    // ---- epilogue parameters: fetched now so that their latency hides behind the main loop
+    const Epilogue &e = p.epi;
+    v2u raw_s1[TNI], raw_z1[TNI], raw_s2[TNI], raw_z2[TNI], raw_bias[TNI];
+    v4i raw_rs[TNI];
+    RowEpi rowp[TMI];
+#pragma unroll
+    for (int mi = 0; mi < TMI; ++mi) rowp[mi] = load_row<MODE>(e, min(m0 + mi * 16 + l16, p.M - 1));
+#pragma unroll
+    for (int ni = 0; ni < TNI; ++ni) {
+        const uint32_t nq = min(n0 + wave * 64 + ni * 16 + kb * 4, p.N - 4);
+        raw_s1[ni] = *reinterpret_cast<const v2u *>(e.s_col_1 + nq);
+        if (MODE == 1 || MODE == 3 || MODE == 4) raw_z1[ni] = *reinterpret_cast<const v2u *>(e.z_col_1 + nq);
+        if (MODE == 4) raw_rs[ni] = *reinterpret_cast<const v4i *>(e.rs_col + nq);
+        if (MODE >= 2 && MODE != 4) raw_s2[ni] = *reinterpret_cast<const v2u *>(e.s_col_2 + nq);
+        if (MODE == 3) raw_z2[ni] = *reinterpret_cast<const v2u *>(e.z_col_2 + nq);
+        if (BIAS) raw_bias[ni] = *reinterpret_cast<const v2u *>(e.bias + nq);
+    }
+
+    // One chunk = two 128-k steps.  PAR = chunk parity: the weight ring slots of this chunk
+    // are 2*PAR and 2*PAR + 1; a slot is refilled (with the step four ahead) during the step
+    // after its use.
+    auto chunk = [&](auto par, uint32_t c, uint32_t cur, uint32_t nxt, uint32_t nx2) {
+        constexpr int PAR = decltype(par)::value;
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            const int slot = 2 * PAR + s;
+            const int prev = (slot + 3) & 3;          // slot of the step before this one
+            const uint32_t gprev = 2 * c + s - 1 + 4;  // the step that slot receives now
+#pragma unroll
+            for (int mi = 0; mi < TMI; ++mi) {
+#pragma unroll
+                for (int ni = 0; ni < TNI; ++ni) {
+                    asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 cbsz:3 blgp:3"
+                                 : "+a"(acc[mi][ni])
+                                 : "v"(wf[slot][ni]), "v"(xf[mi & 3]));
+                    __builtin_amdgcn_sched_barrier(0);
+                    // ---- side work in the shadow of this MFMA
+                    if (ni < 2) {  // activation fragment two groups ahead
+                        const int nm = (mi + 2) & 7, ns = mi + 2 < 8 ? s : s + 1;
+                        const uint32_t buf = ns < 2 ? cur : nxt;
+                        if (ni == 0)
+                            read_x0(xf[nm & 3], buf, nm, ns & 1);
+                        else
+                            read_x1(xf[nm & 3], buf, nm, ns & 1);
+                    }
+                    if (ni == 2) {  // refill the previous step's slot, one load per group (step 0 fetches step 3 again)
+                        if (mi & 1)
+                            load_w1(wf[prev][mi >> 1], mi >> 1, gprev);
+                        else
+                            load_w0(wf[prev][mi >> 1], mi >> 1, gprev);
+                    }
+                    if (ni == 3 && s == 1 && mi < 6) {  // chunk c+2 -> its LDS buffer, then fetch chunk c+3
+                        *reinterpret_cast<v4u *>(lds + nx2 + xlds[mi]) = xreg[mi];
+                        load_x(xreg[mi], mi, c + 3);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+        // the MFMAs are opaque to the compiler's hazard tracking: any accumulator copy it places
+        // at a control-flow join must find them retired
+        asm volatile("s_nop 15" ::: "memory");
+        lds_barrier();
+    };
+
+    uint32_t cur = 0, nxt = kBuf, nx2 = 2 * kBuf;
+    auto rotate = [&]() {
+        const uint32_t t = cur;
+        cur = nxt;
+        nxt = nx2;
+        nx2 = t;
+    };
+    using Even = std::integral_constant<int, 0>;
+    using Odd = std::integral_constant<int, 1>;
+    uint32_t c = 0;
+    for (; c < nchunks; c += 2) {
+        chunk(Even{}, c, cur, nxt, nx2);
+        rotate();
+        if (c + 1 < nchunks) {
+            chunk(Odd{}, c + 1, cur, nxt, nx2);
+            rotate();
+        }
+    }
+    // the MFMAs above are opaque to the compiler's hazard tracking: let the last ones retire
+    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+
+    // ---- epilogue: lane holds acc[mi][ni][r] = C[m = mi*16 + l16][n = ni*16 + 4*kb + r].  The
+    // 128 x 64 fp16 tile of the wavefront goes through LDS so that global stores are whole
+    // 128-byte lines.
+    constexpr uint32_t kYStride = 144;
+    uint8_t *stage = lds + wave * (BM * kYStride);
+#pragma unroll
+    for (int ni = 0; ni < TNI; ++ni) {
+        const uint32_t ncol = ni * 16 + kb * 4;
+        const uint32_t nq = min(n0 + wave * 64 + ncol, p.N - 4);
+        const QuadCols<MODE, BIAS> cols =
+            quad_cols_from_raw<MODE, BIAS>(raw_s1[ni], raw_z1[ni], raw_s2[ni], raw_z2[ni], raw_bias[ni], nq, raw_rs[ni]);
+#pragma unroll
+        for (int mi = 0; mi < TMI; ++mi) {
+            uint16_t out[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) out[r] = dequant_one<MODE, BIAS>((int)acc[mi][ni][r], rowp[mi], cols.c[r]);
+            *reinterpret_cast<v2u *>(stage + (mi * 16 + l16) * kYStride + ncol * 2) =
+                v2u{(uint32_t)out[0] | ((uint32_t)out[1] << 16), (uint32_t)out[2] | ((uint32_t)out[3] << 16)};
+        }
+    }
+    const uint32_t rows_here = min(p.M - m0, (uint32_t)BM);
+    const __amdgpu_buffer_rsrc_t rY = make_rsrc(p.y + (uint64_t)m0 * p.N, rows_here * p.N * 2);
+    const uint32_t piece = lane & 7u, rsub = lane >> 3;
+    const uint32_t ncol0 = n0 + wave * 64 + piece * 8;
+#pragma unroll
+    for (int it = 0; it < BM / 8; ++it) {
+        const uint32_t row = it * 8 + rsub;
+        const v4u v = *reinterpret_cast<const v4u *>(stage + row * kYStride + piece * 16);
+        const uint32_t off = (row < rows_here && ncol0 < p.N) ? (row * p.N + ncol0) * 2 : kOobOffset;
+        __builtin_amdgcn_raw_buffer_store_b128(v, rY, (int)off, 0, 0);
+    }
+}
+
+template <int EPI>
+static void launch_mode(const Bf6Params &p, hipStream_t stream)
+{
+    const dim3 grid(p.tiles_m * p.tiles_n);
+    if (p.epi.bias)
+        hipLaunchKernelGGL((gemm_bf6_kernel<EPI, true>), grid, dim3(256), 0, stream, p);
+    else
+        hipLaunchKernelGGL((gemm_bf6_kernel<EPI, false>), grid, dim3(256), 0, stream, p);
+}
+
+int launch_gemm_bf6(const uint8_t *X, const uint8_t *W, uint32_t M, uint32_t N, uint32_t K, const Epilogue &epi,
+                    uint16_t *y, hipStream_t stream)
+{
+    if (M == 0 || N == 0) return 0;
+    Bf6Params p{X, W, M, N, K, y, epi, (M + 127) / 128, (N + 255) / 256};
+    switch (epi.mode) {
+    case 0: launch_mode<0>(p, stream); break;
+    case 1: launch_mode<1>(p, stream); break;
+    case 2: launch_mode<2>(p, stream); break;
+    case 3: launch_mode<3>(p, stream); break;
+    default: launch_mode<4>(p, stream); break;
+    }
+    return (int)hipGetLastError();
+}
+
+}  // namespace duq

@@ -26,6 +26,7 @@
 // with four consecutive output columns of one row.
 #include "duq_epilogue.h"
 #include "duq_launch.h"
+#include "duq_tiles.h"
 #include <type_traits>
 
 namespace duq {
@@ -51,26 +52,6 @@ __device__ __forceinline__ void expand_nibbles(const v4u w, v4u &even, v4u &odd)
     }
 }
 
-// Workgroup id -> tile id.  Consecutive workgroup ids land on consecutive XCDs (8 of them,
-// each with its own L2), so ids are regrouped to give every XCD one contiguous range of
-// tiles; tiles inside a range walk down a band of 8 tile-rows first, which keeps the A and
-// B panels an XCD touches compact.
-__device__ __forceinline__ void tile_of_block(uint32_t bid, uint32_t tiles_m, uint32_t tiles_n, uint32_t &tm,
-                                              uint32_t &tn)
-{
-    const uint32_t ntiles = tiles_m * tiles_n;
-    const uint32_t per = ntiles / 8, rem = ntiles % 8;
-    const uint32_t xcd = bid % 8, local = bid / 8;
-    const uint32_t logical = xcd < rem ? xcd * (per + 1) + local : rem * (per + 1) + (xcd - rem) * per + local;
-    constexpr uint32_t GM = 8;
-    const uint32_t per_band = GM * tiles_n;
-    const uint32_t band = logical / per_band;
-    const uint32_t first_m = band * GM;
-    const uint32_t band_h = min(tiles_m - first_m, GM);
-    const uint32_t in_band = logical % per_band;
-    tm = first_m + in_band % band_h;
-    tn = in_band / band_h;
-}
 
 // Store four consecutive output columns of one row.
 template <int EPI, bool BIAS>
@@ -272,18 +253,9 @@ __global__ __launch_bounds__(256) void gemm_s4_tile_kernel(GemmParams p)
 // piece at or past the row end is redirected out of bounds and reads as zero).
 constexpr int kCK = 256;         // k elements per chunk (128 packed bytes per row)
 constexpr int kXStride = 272;    // LDS bytes per activation row: 256 expanded + 16 pad
-constexpr uint32_t kOobOffset = 0xFFFFFF00u;  // beyond any descriptor: the load returns 0
 
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, uint32_t bytes)
-{
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
-}
-__device__ __forceinline__ v4u buf_load16(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff)
-{
-    return __builtin_bit_cast(v4u, __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)soff, 0));
-}
 
 template <int TM, int EPI, bool BIAS>
 __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
@@ -453,7 +425,7 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
                 raw_s1[tq] = *reinterpret_cast<const v2u *>(e.s_col_1 + nq);
                 if (MODE == 1 || MODE == 3 || MODE == 4) raw_z1[tq] = *reinterpret_cast<const v2u *>(e.z_col_1 + nq);
                 if (MODE == 4) raw_rs[tq] = *reinterpret_cast<const v4i *>(e.rs_col + nq);
-                if (MODE >= 2) raw_s2[tq] = *reinterpret_cast<const v2u *>(e.s_col_2 + nq);
+                if (MODE == 2 || MODE == 3) raw_s2[tq] = *reinterpret_cast<const v2u *>(e.s_col_2 + nq);
                 if (MODE == 3) raw_z2[tq] = *reinterpret_cast<const v2u *>(e.z_col_2 + nq);
                 if (BIAS) raw_bias[tq] = *reinterpret_cast<const v2u *>(e.bias + nq);
             }

@@ -16,12 +16,13 @@ int launch_asym_quant(const uint16_t *x, const uint16_t *scale, const uint16_t *
 int launch_asym_dual_quant(const uint16_t *x, const uint16_t *s1, const uint16_t *z1, const uint16_t *s2,
                            const uint16_t *z2, uint32_t rows, uint32_t colsSrc, uint32_t colsDst, uint8_t *q,
                            hipStream_t stream);
+// bf6 != nullptr (cols % 128 == 0): also write the E3M2 shadow of the codes; q may then be nullptr.
 int launch_quantize_rows_sym(const uint16_t *x, uint32_t rows, uint32_t cols, float clip, int qmax, uint8_t *q,
-                             uint16_t *scale, hipStream_t stream);
+                             uint16_t *scale, uint8_t *bf6, hipStream_t stream);
 // rowsum == nullptr: unsigned codes and zero points as the reference stores them; otherwise the
 // signed-shifted form (code - 8, zero - 8) plus the per-row sum of the shifted codes.
 int launch_quantize_rows_asym(const uint16_t *x, uint32_t rows, uint32_t cols, uint8_t *q, uint16_t *scale,
-                              uint16_t *zeros, int32_t *rowsum, hipStream_t stream);
+                              uint16_t *zeros, int32_t *rowsum, uint8_t *bf6, hipStream_t stream);
 
 // Epilogue description shared by the stand-alone dequant kernels and the fused GEMM.
 // mode: 0 sym, 1 asym, 2 sym-dual, 3 asym-dual, 4 asym with row-sum zero-point correction
@@ -45,5 +46,13 @@ int launch_dequant(const int32_t *acc, const Epilogue &epi, uint32_t rows, uint3
 // GEMM: out_acc != nullptr -> int32 accumulators [M,N]; else fused epilogue into y.
 int launch_gemm_s4(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N, uint32_t K, int32_t *out_acc,
                    const Epilogue *epi, uint16_t *y, hipStream_t stream);
+
+
+// 6-bit float (E3M2) shadows of packed-int4 tensors and the GEMM that multiplies them
+// (duq_bf6.hip).  K % 128 == 0, N % 16 == 0.
+int launch_weight_shadow_bf6(const uint8_t *w, uint32_t N, uint32_t K, uint8_t *out, hipStream_t stream);
+int launch_activation_shadow_bf6(const uint8_t *q, uint32_t M, uint32_t K, uint8_t *out, hipStream_t stream);
+int launch_gemm_bf6(const uint8_t *X, const uint8_t *W, uint32_t M, uint32_t N, uint32_t K, const Epilogue &epi,
+                    uint16_t *y, hipStream_t stream);
 
 }  // namespace duq

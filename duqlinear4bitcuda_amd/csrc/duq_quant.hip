@@ -186,7 +186,33 @@ struct RowParams {
     float clip;
     int qmax;
     int32_t *rowsum;  // asym only: non-null selects the signed-shifted form (code - 8, zero - 8, sum of codes)
+    uint8_t *bf6;     // BF6 kernels: E3M2 shadow of the codes, [rows][cols/32 x 16 B | cols/32 x 8 B]; q may be null
 };
+
+typedef _Float16 v32h __attribute__((ext_vector_type(32)));
+typedef unsigned int v6u __attribute__((ext_vector_type(6)));
+
+// 32 codes (four packed words, read as signed nibbles like the GEMM reads them) -> one E3M2
+// block.  Position 8d + 2i + h of the block holds nibble i + 4h of word d: the pairing that
+// costs one shift and one mask per two elements; the weight shadow uses the same order and
+// the sum over k does not care.  0x6400 | u is the binary16 number 1024 + u, and the signed
+// value of nibble n is (n ^ 8) - 8.
+__device__ __forceinline__ v6u bf6_block(const uint32_t (&w)[4])
+{
+    typedef uint32_t v16u_t __attribute__((ext_vector_type(16)));
+    v16u_t pairs;
+    const v2h off = v2h{(f16)1032.0f, (f16)1032.0f};
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+        const uint32_t u = w[d] ^ 0x88888888u;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t bits = ((u >> (4 * i)) & 0x000F000Fu) | 0x64006400u;
+            pairs[d * 4 + i] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(v2h, bits) - off);
+        }
+    }
+    return __builtin_amdgcn_cvt_scalef32_pk32_bf6_f16(__builtin_bit_cast(v32h, pairs), 1.0f);
+}
 
 __device__ __forceinline__ uint32_t pk_absmax_u16(uint32_t acc, uint32_t w)
 {
@@ -195,7 +221,9 @@ __device__ __forceinline__ uint32_t pk_absmax_u16(uint32_t acc, uint32_t w)
     return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(a, b));
 }
 
-template <int WAVES, bool ASYM, bool CACHED>
+// BF6: a lane owns whole blocks of 32 elements (four consecutive units) and also writes their
+// E3M2 shadow; the packed nibbles are written only when p.q is given.
+template <int WAVES, bool ASYM, bool CACHED, bool BF6 = false>
 __global__ __launch_bounds__(WAVES * 64) void quantize_rows_kernel(RowParams p)
 {
     constexpr int T = WAVES * 64;
@@ -208,6 +236,8 @@ __global__ __launch_bounds__(WAVES * 64) void quantize_rows_kernel(RowParams p)
     const uint32_t nunits = p.cols >> 3;  // units of 8 elements
     const v4u *xrow = reinterpret_cast<const v4u *>(p.x + (uint64_t)row * p.cols);
     uint32_t *qrow = reinterpret_cast<uint32_t *>(p.q + (uint64_t)row * (p.cols >> 1));
+    // unit held in register slot i
+    auto unit_of = [&](int i) -> uint32_t { return BF6 ? 4 * (tid + (i >> 2) * T) + (i & 3) : tid + i * T; };
 
     v4u regs[kMaxUnits];
     uint32_t amax = 0;        // sym: packed max of |x| bit patterns (NaN patterns win, as in torch.max)
@@ -231,12 +261,12 @@ __global__ __launch_bounds__(WAVES * 64) void quantize_rows_kernel(RowParams p)
     if (CACHED) {
 #pragma unroll
         for (int i = 0; i < kMaxUnits; ++i) {
-            const uint32_t u = tid + i * T;
+            const uint32_t u = unit_of(i);
             regs[i] = u < nunits ? __builtin_nontemporal_load(&xrow[u]) : v4u{0u, 0u, 0u, 0u};
         }
 #pragma unroll
         for (int i = 0; i < kMaxUnits; ++i)
-            if (tid + i * T < nunits) reduce_unit(regs[i]);
+            if (unit_of(i) < nunits) reduce_unit(regs[i]);
     } else {
         for (uint32_t u = tid; u < nunits; u += T) reduce_unit(xrow[u]);
     }
@@ -355,7 +385,36 @@ __global__ __launch_bounds__(WAVES * 64) void quantize_rows_kernel(RowParams p)
         }
         return w;
     };
-    if (CACHED) {
+    if (BF6) {
+        // cols % 32 == 0: a block is all inside the row or all outside
+        const uint32_t nblk = p.cols >> 5;
+        uint8_t *srow = p.bf6 + (uint64_t)row * nblk * 24;
+        auto put_block = [&](uint32_t b, const uint32_t (&w)[4]) {
+            if (p.q) *reinterpret_cast<v4u *>(qrow + 4 * b) = v4u{w[0], w[1], w[2], w[3]};
+            const v6u f = bf6_block(w);
+            *reinterpret_cast<v4u *>(srow + b * 16) = v4u{f[0], f[1], f[2], f[3]};
+            *reinterpret_cast<v2u *>(srow + nblk * 16 + b * 8) = v2u{f[4], f[5]};
+        };
+        if (CACHED) {
+#pragma unroll
+            for (int g = 0; g < kMaxUnits / 4; ++g) {
+                const uint32_t b = tid + g * T;
+                if (b < nblk) {
+                    uint32_t w[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) w[j] = quant_unit(regs[4 * g + j]);
+                    put_block(b, w);
+                }
+            }
+        } else {
+            for (uint32_t b = tid; b < nblk; b += T) {
+                uint32_t w[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) w[j] = quant_unit(xrow[4 * b + j]);
+                put_block(b, w);
+            }
+        }
+    } else if (CACHED) {
 #pragma unroll
         for (int i = 0; i < kMaxUnits; ++i) {
             const uint32_t u = tid + i * T;
@@ -393,15 +452,23 @@ static int launch_rows(const RowParams &p, hipStream_t stream)
         return w;
     };
     uint32_t waves = waves_for(4);
-    if ((uint64_t)p.rows * waves < 2048) waves = waves_for(2);
-    if ((uint64_t)p.rows * waves < 512) waves = waves_for(1);
+    if (!p.bf6) {  // (a lane of the shadow-writing kernel holds whole blocks: four units at least)
+        if ((uint64_t)p.rows * waves < 2048) waves = waves_for(2);
+        if ((uint64_t)p.rows * waves < 512) waves = waves_for(1);
+    }
     const bool cached = waves * 64 * kMaxUnits >= nunits;
+#define DUQ_ROWS_LAUNCH(W, C)                                                                                \
+    if (p.bf6)                                                                                               \
+        hipLaunchKernelGGL((quantize_rows_kernel<W, ASYM, C, true>), grid, dim3(W * 64), 0, stream, p);      \
+    else                                                                                                     \
+        hipLaunchKernelGGL((quantize_rows_kernel<W, ASYM, C, false>), grid, dim3(W * 64), 0, stream, p);
 #define DUQ_ROWS_CASE(W)                                                                                     \
     case W:                                                                                                  \
-        if (cached)                                                                                          \
-            hipLaunchKernelGGL((quantize_rows_kernel<W, ASYM, true>), grid, dim3(W * 64), 0, stream, p);     \
-        else                                                                                                 \
-            hipLaunchKernelGGL((quantize_rows_kernel<W, ASYM, false>), grid, dim3(W * 64), 0, stream, p);    \
+        if (cached) {                                                                                        \
+            DUQ_ROWS_LAUNCH(W, true)                                                                         \
+        } else {                                                                                             \
+            DUQ_ROWS_LAUNCH(W, false)                                                                        \
+        }                                                                                                    \
         break;
     switch (waves) {
         DUQ_ROWS_CASE(1)
@@ -411,19 +478,20 @@ static int launch_rows(const RowParams &p, hipStream_t stream)
         DUQ_ROWS_CASE(16)
     }
 #undef DUQ_ROWS_CASE
+#undef DUQ_ROWS_LAUNCH
     return (int)hipGetLastError();
 }
 
 int launch_quantize_rows_sym(const uint16_t *x, uint32_t rows, uint32_t cols, float clip, int qmax, uint8_t *q,
-                             uint16_t *scale, hipStream_t stream)
+                             uint16_t *scale, uint8_t *bf6, hipStream_t stream)
 {
-    RowParams p{x, q, scale, nullptr, rows, cols, clip, qmax, nullptr};
+    RowParams p{x, q, scale, nullptr, rows, cols, clip, qmax, nullptr, bf6};
     return launch_rows<false>(p, stream);
 }
 int launch_quantize_rows_asym(const uint16_t *x, uint32_t rows, uint32_t cols, uint8_t *q, uint16_t *scale,
-                              uint16_t *zeros, int32_t *rowsum, hipStream_t stream)
+                              uint16_t *zeros, int32_t *rowsum, uint8_t *bf6, hipStream_t stream)
 {
-    RowParams p{x, q, scale, zeros, rows, cols, 1.0f, 15, rowsum};
+    RowParams p{x, q, scale, zeros, rows, cols, 1.0f, 15, rowsum, bf6};
     return launch_rows<true>(p, stream);
 }
 

@@ -202,6 +202,37 @@ int duq_asym_rowsum_dequant_host(const int32_t *q, const duq_half *scale_row, co
                                  const int32_t *rowsum_adj_col, const duq_half *bias, uint32_t rows, uint32_t cols,
                                  duq_half *x, duq_stream_t stream);
 
+/* ---- the same forward on the 6-bit float matrix path ---------------------------------- */
+
+/* No counterpart in the reference.  Every int4 value is exactly an E3M2 ("bf6") number and
+ * the float32 accumulation of their products is exact below 2^24 (|C| <= 64*K), so the
+ * MFMA for 6-bit floats, which runs at twice the rate of the 8-bit integer one, returns the
+ * integer GEMM bit for bit.  The operands are shadows of the packed-int4 tensors, 3/4 byte per
+ * element, in a layout private to the library:
+ *   duq_weight_shadow_bf6      w    [N,K/2] -> w_bf6 [N*K*3/4 bytes], once per weight tensor
+ *   duq_activation_shadow_bf6  xq   [M,K/2] -> x_bf6 [M*K*3/4 bytes] (the *_bf6 quantizers
+ *                              below write it directly)
+ * duq_linear4bit_forward_bf6 takes the shadows in place of xq and w, and otherwise the
+ * arguments of duq_linear4bit_forward (modes DUQ_EPI_SYM .. DUQ_EPI_ASYM_DUAL) or of
+ * duq_linear4bit_forward_rowsum (mode DUQ_EPI_ASYM_ROWSUM: rowsum_x, w_rowsum_adj; NULL in
+ * the other modes); y is bit-identical to theirs.
+ * K % 128 == 0, N % 16 == 0; shadows and y 16-byte aligned, per-column arrays 8-byte
+ * aligned (w_rowsum_adj 16). */
+int duq_weight_shadow_bf6(const uint8_t *w, uint32_t N, uint32_t K, uint8_t *w_bf6, duq_stream_t stream);
+/* duq_quantize_rows_sym / duq_quantize_rows_asym (rowsum NULL) / duq_quantize_rows_asym_shifted
+ * (rowsum given) that also write the shadow of the codes; q may be NULL when only the shadow is
+ * wanted.  cols % 128 == 0. */
+int duq_quantize_rows_sym_bf6(const duq_half *x, uint32_t rows, uint32_t cols, float clip, int32_t qmax, uint8_t *q,
+                              uint8_t *x_bf6, duq_half *scale, duq_stream_t stream);
+int duq_quantize_rows_asym_bf6(const duq_half *x, uint32_t rows, uint32_t cols, uint8_t *q, uint8_t *x_bf6,
+                               duq_half *scale, duq_half *zeros, int32_t *rowsum, duq_stream_t stream);
+int duq_activation_shadow_bf6(const uint8_t *xq, uint32_t M, uint32_t K, uint8_t *x_bf6, duq_stream_t stream);
+int duq_linear4bit_forward_bf6(int32_t mode, const uint8_t *x_bf6, const duq_half *scale_x, const duq_half *zeros_x,
+                               const int32_t *rowsum_x, const uint8_t *w_bf6, const duq_half *w_scale_1,
+                               const duq_half *w_zeros_1, const duq_half *w_scale_2, const duq_half *w_zeros_2,
+                               const int32_t *w_rowsum_adj, const duq_half *bias, uint32_t M, uint32_t N, uint32_t K,
+                               duq_half *y, duq_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
