@@ -227,7 +227,7 @@ template <int WAVES, bool ASYM, bool CACHED, bool BF6 = false>
 __global__ __launch_bounds__(WAVES * 64) void quantize_rows_kernel(RowParams p)
 {
     constexpr int T = WAVES * 64;
-    __shared__ float red[2][WAVES];
+    __shared__ float red[3][WAVES];
     __shared__ int red_sum[WAVES];
     const bool shifted = ASYM && p.rowsum != nullptr;
     int code_sum = 0;  // sum of this lane's unsigned codes (shifted form only)
@@ -247,9 +247,8 @@ __global__ __launch_bounds__(WAVES * 64) void quantize_rows_kernel(RowParams p)
     auto reduce_unit = [&](const v4u &g) {
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
-            if (!ASYM) {
-                amax = pk_absmax_u16(amax, g[w]);
-            } else {
+            amax = pk_absmax_u16(amax, g[w]);  // asym: only to see NaNs, which fminf / fmaxf drop
+            if (ASYM) {
                 const float lo = (float)bits_to_f16((uint16_t)(g[w] & 0xFFFFu));
                 const float hi = (float)bits_to_f16((uint16_t)(g[w] >> 16));
                 fmin_ = fminf(fmin_, fminf(lo, hi));
@@ -273,9 +272,9 @@ __global__ __launch_bounds__(WAVES * 64) void quantize_rows_kernel(RowParams p)
 
     // ---- row reduction: shuffles inside a wavefront, one LDS hop across wavefronts ----
     float a, b = 0.f;
+    uint32_t m16 = wave_max_u32(max(amax & 0xFFFFu, amax >> 16));  // largest |x| bit pattern; above 0x7C00: a NaN
     if (!ASYM) {
-        const uint32_t m16 = max(amax & 0xFFFFu, amax >> 16);
-        a = __builtin_bit_cast(float, wave_max_u32(m16));  // carried as raw bits
+        a = __builtin_bit_cast(float, m16);  // carried as raw bits
     } else {
         a = wave_min_f32(fmin_);
         b = wave_max_f32(fmax_);
@@ -285,6 +284,7 @@ __global__ __launch_bounds__(WAVES * 64) void quantize_rows_kernel(RowParams p)
         if ((tid & 63u) == 0) {
             red[0][wave] = a;
             red[1][wave] = b;
+            red[2][wave] = __builtin_bit_cast(float, m16);
         }
         __syncthreads();
         if (!ASYM) {
@@ -295,13 +295,16 @@ __global__ __launch_bounds__(WAVES * 64) void quantize_rows_kernel(RowParams p)
         } else {
             a = red[0][0];
             b = red[1][0];
+            m16 = __builtin_bit_cast(uint32_t, red[2][0]);
 #pragma unroll
             for (int w = 1; w < WAVES; ++w) {
                 a = fminf(a, red[0][w]);
                 b = fmaxf(b, red[1][w]);
+                m16 = max(m16, __builtin_bit_cast(uint32_t, red[2][w]));
             }
         }
     }
+    if (ASYM && m16 > 0x7C00u) a = b = __builtin_nanf("");  // torch's min / max return NaN for a row that holds one
 
     // ---- per-token scale / zero (qlinear4bit/nn/quantizer.py:13, 27-31) ----
     f16 s;

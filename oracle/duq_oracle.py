@@ -34,6 +34,10 @@ fixes by definition instead ("parity unpinned" for exactly these corners):
 The row-sum functions (``asym_quant_shifted`` ... ``linear4bit_asq_rowsum_forward``) restate a
 mode the reference does not have; there is nothing of the reference to be in parity with, and
 they are pinned by the integer identity and the float64 product of the dequantized operands.
+The E3M2 shadow functions (``e3m2_decode`` ... ``weight_shadow_bf6``) describe a storage format
+of the library, not of the reference: they are pinned by the published OCP Microscaling
+formula for E3M2 (decode), by decode(encode(v)) == v for every int4 value, and by the round
+trip through ``shadow_block_unpack``; what the GEMM computes from them stays ``matmul_s4``.
 """
 from __future__ import annotations
 
@@ -475,3 +479,91 @@ def weight_asym_from_linear(w):
         r = h(np.rint(_f32(hdiv(w, scale))))
         q = np.clip(_f32(hadd(r, zero)), 0, 15)
     return pack_i4(q.astype(np.int32), sym=False), scale, zero
+
+
+# ----------------------------------------------------------------------------------
+# E3M2 ("bf6") shadows of packed-int4 tensors: the operand format of the library's 6-bit
+# float matrix path (no counterpart in the reference; results stay those of matmul_s4)
+# ----------------------------------------------------------------------------------
+def e3m2_decode(code):
+    """Value of a 6-bit E3M2 code (OCP Microscaling Formats v1.0, FP6 E3M2: 1 sign, 3 exponent
+    bits with bias 3, 2 mantissa bits, subnormals at exponent 0, no inf / NaN)."""
+    code = np.asarray(code, dtype=np.int64)
+    sign = np.where((code >> 5) & 1, -1.0, 1.0)
+    e = (code >> 2) & 7
+    m = code & 3
+    mag = np.where(e == 0, (m / 4.0) * 2.0 ** (1 - 3), (1.0 + m / 4.0) * 2.0 ** (e.astype(np.float64) - 3))
+    return sign * mag
+
+
+def e3m2_encode_int4(v):
+    """The E3M2 code of an integer in [-8, 7] (exact: every such integer has at most three
+    significant bits).  Zero is +0."""
+    v = np.asarray(v, dtype=np.int64)
+    table = np.zeros(16, dtype=np.uint8)
+    values = e3m2_decode(np.arange(64))
+    for x in range(-8, 8):
+        hits = [c for c in range(64) if values[c] == x and not (x == 0 and c >= 32)]
+        assert len(hits) == 1
+        table[x & 15] = hits[0]
+    return table[v & 15]
+
+
+def _shadow_positions():
+    """Element index (inside a block of 32 consecutive k) stored at each of the 32 positions:
+    position 8d + 2i + hh holds element 8d + i + 4hh (the pairing the quantizer kernels get
+    with one shift and one mask per two nibbles)."""
+    pos = np.arange(32)
+    d, i, hh = pos >> 3, (pos & 7) >> 1, pos & 1
+    return 8 * d + i + 4 * hh
+
+
+def shadow_block_pack(values):
+    """values int [..., 32] in [-8, 7] -> uint8 [..., 24]: 32 six-bit codes, position p in bits
+    6p .. 6p+5 of the 192-bit little-endian block."""
+    values = np.asarray(values)
+    codes = e3m2_encode_int4(values[..., _shadow_positions()]).astype(np.uint64)
+    bits = np.zeros(values.shape[:-1] + (192,), dtype=np.uint8)
+    for b in range(6):
+        bits[..., b::6] = ((codes >> np.uint64(b)) & np.uint64(1)).astype(np.uint8)
+    out = np.packbits(bits, axis=-1, bitorder="little")
+    return out
+
+
+def shadow_block_unpack(block):
+    """Inverse of shadow_block_pack: uint8 [..., 24] -> int [..., 32]."""
+    bits = np.unpackbits(np.asarray(block, dtype=np.uint8), axis=-1, bitorder="little")
+    codes = np.zeros(bits.shape[:-1] + (32,), dtype=np.int64)
+    for b in range(6):
+        codes |= bits[..., b::6].astype(np.int64) << b
+    vals = e3m2_decode(codes).astype(np.int64)
+    out = np.zeros_like(vals)
+    out[..., _shadow_positions()] = vals
+    return out
+
+
+def activation_shadow_bf6(q_packed):
+    """uint8 [M, K/2] packed nibbles (read as signed, like the GEMM reads them) -> uint8
+    [M, 3K/4]: per row the first 16 bytes of each of its K/32 blocks, then the last 8 bytes of
+    each.  K % 32 == 0."""
+    v = unpack_i4(q_packed, signed=True)
+    M, K = v.shape
+    blocks = shadow_block_pack(v.reshape(M, K // 32, 32))  # [M, K/32, 24]
+    return np.concatenate([blocks[..., :16].reshape(M, -1), blocks[..., 16:].reshape(M, -1)], axis=1)
+
+
+def weight_shadow_bf6(w_packed):
+    """uint8 [N, K/2] -> uint8 [N, 3K/4] in tile order.  For every pair of 16-row tiles and every
+    128-k step, lane l = (row l % 16, k-block l // 16) owns one block of each tile; the 3072
+    bytes of the (pair, step) are three arrays of 64 lanes x 16 bytes: bytes 0-15 of the first
+    tile's blocks | bytes 16-23 of the first and 0-7 of the second | bytes 8-23 of the second.
+    N % 32 == 0, K % 128 == 0."""
+    v = unpack_i4(w_packed, signed=True)
+    N, K = v.shape
+    blocks = shadow_block_pack(v.reshape(N, K // 32, 32))  # [N, K/32, 24]
+    b = blocks.reshape(N // 32, 2, 16, K // 128, 4, 24)    # pair, tile, row, step, kb, byte
+    b = b.transpose(0, 3, 1, 4, 2, 5)                      # pair, step, tile, kb, row, byte  (lane = kb*16 + row)
+    first, second = b[:, :, 0].reshape(N // 32, K // 128, 64, 24), b[:, :, 1].reshape(N // 32, K // 128, 64, 24)
+    parts = np.stack([first[..., :16], np.concatenate([first[..., 16:], second[..., :8]], axis=-1), second[..., 8:]],
+                     axis=2)                               # pair, step, part, lane, 16
+    return np.ascontiguousarray(parts).reshape(N, K * 3 // 4)
