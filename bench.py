@@ -5,8 +5,11 @@
 
 One "step" is one pass of the hot path over one batch of synthetic input, everything
 resident in HBM: per-token symmetric int4 quantization of the fp16 activations, the
-packed int4 x int4 GEMM on the i8 MFMA units and the fused fp16 dequant epilogue
-(``Sequential(SymQuantizer, Linear4bitSQ)``).  The workload is the prefill configuration
+int4 x int4 GEMM and the fused fp16 dequant epilogue (``Sequential(SymQuantizer,
+Linear4bitSQ)``).  The GEMM runs on the matrix path for 6-bit floats (every int4 value is
+exactly an E3M2 number and the float32 accumulation of their products is exact, so the result
+is the integer GEMM bit for bit at twice the i8 MFMA rate); the same step on the i8 MFMA
+kernels is timed beside it (``integer_path``).  The workload is the prefill configuration
 the metric is quoted on: M = 2048 tokens, K = N = 4096 (a Llama-2-7B attention
 projection), activations ~N(0,1) with 1 % heavy-tailed channels, weights uniform random
 nibbles with per-channel scales.
@@ -14,7 +17,7 @@ nibbles with per-channel scales.
 Prints ONE JSON line.  ``value`` is 2*M*N*K / (time per step) in TOPS for the whole step.
 ``roofline`` describes the dominant kernel (the fused GEMM): achieved = 2*M*N*K / its own
 average duration, measured with HIP events around ``steps`` back-to-back launches on the
-launch stream.  ``decode`` and ``quantizer`` report the HBM-bound parts of the metric
+launch stream, against the published dense peak of the matrix instruction it uses.  ``decode`` and ``quantizer`` report the HBM-bound parts of the metric
 (GB/s with algorithmic bytes), ``cpu_baseline`` the CPU fake-quant path on the host.
 """
 from __future__ import annotations
@@ -30,8 +33,10 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, published
+PEAK_FP6_TOPS = 10100.0   # MI355X dense fp6 / fp4 MFMA, published
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, published
-GEMM_TRAFFIC_BYTES = (33047 + 16384) * 1024  # fetched + written per launch of the fused GEMM (rocprofv3 counters)
+GEMM_TRAFFIC_BYTES = None  # fetched + written per launch of the fused GEMM (rocprofv3 counters)
+GEMM_I8_TRAFFIC_BYTES = (33047 + 16384) * 1024
 
 
 def heavy_tail_acts(M, K, seed, frac=0.01):
@@ -141,7 +146,11 @@ def quantizer_section(dev):
         xs = [torch.randn(M, K, device=dev).half() for _ in range(nbuf)]
         us = graph_time_us([(lambda x=x: hip.quantize_rows_sym(x)) for x in xs] * 2)
         byts = 2 * M * K + M * K // 2 + 2 * M
-        out.append({"M": M, "K": K, "us": round(us, 3), "GBps": round(byts / us / 1e3, 1),
+        out.append({"M": M, "K": K, "out": "int4", "us": round(us, 3), "GBps": round(byts / us / 1e3, 1),
+                    "frac_hbm": round(byts / us / 1e3 / PEAK_HBM_GBS, 4)})
+        us = graph_time_us([(lambda x=x: hip.quantize_rows_sym_bf6(x, with_q=False)) for x in xs] * 2)
+        byts = 2 * M * K + M * K * 3 // 4 + 2 * M
+        out.append({"M": M, "K": K, "out": "e3m2 shadow", "us": round(us, 3), "GBps": round(byts / us / 1e3, 1),
                     "frac_hbm": round(byts / us / 1e3 / PEAK_HBM_GBS, 4)})
         del xs
     return out
@@ -224,10 +233,21 @@ def main():
     lin = Linear4bitSQ(K, N, bias=False).to(dev)
     lin.weight.copy_(w)
     lin.weight_scales = sw
-    quant = SymQuantizer(1.0)
+    lin.enable_fp6()
+    quant = SymQuantizer(1.0, shadow="only", shadow_min_rows=1)
+    lin_i8 = Linear4bitSQ(K, N, bias=False).to(dev)   # the same layer on the i8 MFMA kernels
+    lin_i8.weight.copy_(w)
+    lin_i8.weight_scales = sw
+    quant_i8 = SymQuantizer(1.0)
 
     def step():
         return lin(quant(x))
+
+    def step_i8():
+        return lin_i8(quant_i8(x))
+
+    if not torch.equal(step().view(torch.int16), step_i8().view(torch.int16)):
+        raise SystemExit("bench.py: the 6-bit float path and the integer path disagree")
 
     # ---- whole-step throughput: W warm-up steps, then exactly K timed steps ----
     for _ in range(args.warmup):
@@ -262,19 +282,42 @@ def main():
     except RuntimeError as exc:  # capture unsupported: keep the eager figure only
         print(f"graph capture skipped: {exc}", file=sys.stderr)
 
+    # ---- the same steps on the integer kernels ----
+    for _ in range(args.warmup):
+        step_i8()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step_i8()
+    torch.cuda.synchronize()
+    i8_ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
     # ---- dominant kernel (fused GEMM + dequant) alone, HIP events on the launch stream ----
     pq = quant(x)
-    xq, sx = pq.quantized_x, pq.scales_x
-    gemm_us = event_time_us(lambda: hip.linear4bit_forward(hip.EPI_SYM, xq, sx, None, lin.weight, sw), args.steps,
-                            args.warmup)
-    quant_us = event_time_us(lambda: hip.quantize_rows_sym(x), args.steps, args.warmup)
+    xs, sx = pq.shadow_x, pq.scales_x
+    gemm_us = event_time_us(lambda: hip.linear4bit_forward_bf6(hip.EPI_SYM, xs, sx, None, lin.weight_shadow, sw),
+                            args.steps, args.warmup)
+    quant_us = event_time_us(lambda: hip.quantize_rows_sym_bf6(x, with_q=False), args.steps, args.warmup)
     achieved = ops / gemm_us / 1e6
-    roofline = {"bound": "mfma", "kernel": "gemm_s4_stream_kernel<0,false> (fused GEMM + dequant)", "achieved": round(achieved, 1),
-                "peak": PEAK_INT8_TOPS, "unit": "TOP/s", "frac": round(achieved / PEAK_INT8_TOPS, 4),
-                "avg_kernel_us": round(gemm_us, 2),
+    roofline = {"bound": "mfma", "kernel": "gemm_bf6_kernel<0,false> (fused GEMM + dequant on v_mfma_f32_16x16x128_f8f6f4)",
+                "achieved": round(achieved, 1), "peak": PEAK_FP6_TOPS, "unit": "TOP/s",
+                "frac": round(achieved / PEAK_FP6_TOPS, 4), "avg_kernel_us": round(gemm_us, 2),
+                "peak_note": "published dense fp6 peak; the same achieved rate is %.3f of the int8 peak (5.0 POP/s) the "
+                             "integer kernel is priced against" % (achieved / PEAK_INT8_TOPS),
                 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this workload, each
                 # scaled by what the counter reads for the 256 MiB copy at the end of this script
-                "traffic": GEMM_TRAFFIC_BYTES, "traffic_source": "profiles/gemm_s4_stream_kernel__prefill_M2048_K4096_N4096.txt"}
+                "traffic": GEMM_TRAFFIC_BYTES, "traffic_source": "profiles/gemm_bf6_kernel__prefill_M2048_K4096_N4096.txt"}
+    xq = quant_i8(x).quantized_x
+    i8_gemm_us = event_time_us(lambda: hip.linear4bit_forward(hip.EPI_SYM, xq, sx, None, lin_i8.weight, sw), args.steps,
+                               args.warmup)
+    i8_quant_us = event_time_us(lambda: hip.quantize_rows_sym(x), args.steps, args.warmup)
+    integer_path = {"ms_per_step": round(i8_ms_per_step, 5), "TOPS": round(ops / (i8_ms_per_step * 1e-3) / 1e12, 2),
+                    "kernel": "gemm_s4_stream_kernel<4,0,false> (v_mfma_i32_32x32x32_i8)", "gemm_fused_us": round(i8_gemm_us, 2),
+                    "quantize_rows_sym_us": round(i8_quant_us, 2),
+                    "roofline": {"bound": "mfma", "achieved": round(ops / i8_gemm_us / 1e6, 1), "peak": PEAK_INT8_TOPS,
+                                 "unit": "TOP/s", "frac": round(ops / i8_gemm_us / 1e6 / PEAK_INT8_TOPS, 4),
+                                 "traffic": GEMM_I8_TRAFFIC_BYTES,
+                                 "traffic_source": "profiles/gemm_s4_stream_kernel__prefill_M2048_K4096_N4096.txt"}}
 
     decode = decode_section(dev, args.quick)
     quantizer = quantizer_section(dev)
@@ -303,13 +346,15 @@ def main():
         "ms_per_step": round(ms_per_step, 5),
         "graph_ms_per_step": None if graph_ms_per_step is None else round(graph_ms_per_step, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int8", "dtype_detail": "int4 x int4 codes widened to int8 for v_mfma_i32_32x32x32_i8, int32 accumulate, fp16 epilogue",
+        "dtype": "fp6", "dtype_detail": "int4 x int4 codes held as E3M2 6-bit floats for v_mfma_f32_16x16x128_f8f6f4, float32 "
+                                        "accumulate (exact: integers below 2^24), fp16 epilogue; bit-identical to the int8 path",
         "data": "synthetic",
         "config": {"workload": "prefill Linear4bit forward (quantize + GEMM + dequant), M=2048 K=4096 N=4096, "
                                "symmetric int4 both operands, activations ~N(0,1) with 1% Student-t(3) channels",
                    "M": M, "N": N, "K": K, "step_kernels": {"quantize_rows_sym_us": round(quant_us, 2),
                                                              "gemm_fused_us": round(gemm_us, 2)}},
         "roofline": roofline,
+        "integer_path": integer_path,
         "roofline_decode": roofline_decode,
         "decode": decode,
         "quantizer": quantizer,

@@ -221,8 +221,10 @@ __device__ __forceinline__ uint32_t pk_absmax_u16(uint32_t acc, uint32_t w)
     return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(a, b));
 }
 
-// BF6: a lane owns whole blocks of 32 elements (four consecutive units) and also writes their
-// E3M2 shadow; the packed nibbles are written only when p.q is given.
+// BF6: the kernel also writes the E3M2 shadow of the codes (blocks of 32 elements = four
+// consecutive units); the packed words of a row meet in LDS so that the loads keep the
+// coalesced unit-per-lane pattern and a lane still converts whole blocks.  The packed nibbles
+// are written only when p.q is given.
 template <int WAVES, bool ASYM, bool CACHED, bool BF6 = false>
 __global__ __launch_bounds__(WAVES * 64) void quantize_rows_kernel(RowParams p)
 {
@@ -236,8 +238,9 @@ __global__ __launch_bounds__(WAVES * 64) void quantize_rows_kernel(RowParams p)
     const uint32_t nunits = p.cols >> 3;  // units of 8 elements
     const v4u *xrow = reinterpret_cast<const v4u *>(p.x + (uint64_t)row * p.cols);
     uint32_t *qrow = reinterpret_cast<uint32_t *>(p.q + (uint64_t)row * (p.cols >> 1));
+    __shared__ __attribute__((aligned(16))) uint32_t words[BF6 && CACHED ? T * kMaxUnits : 4];
     // unit held in register slot i
-    auto unit_of = [&](int i) -> uint32_t { return BF6 ? 4 * (tid + (i >> 2) * T) + (i & 3) : tid + i * T; };
+    auto unit_of = [&](int i) -> uint32_t { return tid + i * T; };
 
     v4u regs[kMaxUnits];
     uint32_t amax = 0;        // sym: packed max of |x| bit patterns (NaN patterns win, as in torch.max)
@@ -400,13 +403,24 @@ __global__ __launch_bounds__(WAVES * 64) void quantize_rows_kernel(RowParams p)
         };
         if (CACHED) {
 #pragma unroll
+            for (int i = 0; i < kMaxUnits; ++i) {
+                const uint32_t u = tid + i * T;
+                if (u < nunits) {
+                    const uint32_t w = quant_unit(regs[i]);
+                    words[u] = w;
+                    if (p.q) qrow[u] = w;
+                }
+            }
+            __syncthreads();
+#pragma unroll
             for (int g = 0; g < kMaxUnits / 4; ++g) {
                 const uint32_t b = tid + g * T;
                 if (b < nblk) {
-                    uint32_t w[4];
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) w[j] = quant_unit(regs[4 * g + j]);
-                    put_block(b, w);
+                    const v4u w4 = *reinterpret_cast<const v4u *>(&words[4 * b]);
+                    const uint32_t w[4] = {w4[0], w4[1], w4[2], w4[3]};
+                    const v6u f = bf6_block(w);
+                    *reinterpret_cast<v4u *>(srow + b * 16) = v4u{f[0], f[1], f[2], f[3]};
+                    *reinterpret_cast<v2u *>(srow + nblk * 16 + b * 8) = v2u{f[4], f[5]};
                 }
             }
         } else {
@@ -455,10 +469,8 @@ static int launch_rows(const RowParams &p, hipStream_t stream)
         return w;
     };
     uint32_t waves = waves_for(4);
-    if (!p.bf6) {  // (a lane of the shadow-writing kernel holds whole blocks: four units at least)
-        if ((uint64_t)p.rows * waves < 2048) waves = waves_for(2);
-        if ((uint64_t)p.rows * waves < 512) waves = waves_for(1);
-    }
+    if ((uint64_t)p.rows * waves < 2048) waves = waves_for(2);
+    if ((uint64_t)p.rows * waves < 512) waves = waves_for(1);
     const bool cached = waves * 64 * kMaxUnits >= nunits;
 #define DUQ_ROWS_LAUNCH(W, C)                                                                                \
     if (p.bf6)                                                                                               \

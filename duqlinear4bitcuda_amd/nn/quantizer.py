@@ -8,6 +8,18 @@ import torch
 from ..tools import tensor_utils
 
 
+def _shadow_choice(quantizer, x, override):
+    """False, True or "only": the per-call override if given, else the module's setting when the input is
+    large enough; never for widths the matrix path does not take."""
+    if x.shape[-1] % 128 or x.data_ptr() % 16 or not x.is_cuda:
+        return False
+    if override is not None:
+        return override
+    if quantizer.shadow and x.numel() // x.shape[-1] >= quantizer.shadow_min_rows:
+        return quantizer.shadow
+    return False
+
+
 class SymQuantizer(torch.nn.Module):
     """x fp16 [..., K] -> PackedQuantizedTensor(q u8 [..., K/2], scales fp16 [..., 1]).
 
@@ -15,14 +27,23 @@ class SymQuantizer(torch.nn.Module):
     clamp of the codes: 6 is what the reference's device kernel applies
     (include/common.h:53-54), 7 what its Python fake-quant path applies."""
 
-    def __init__(self, input_clip_ratio=1.0, qmax: int = 6):
+    def __init__(self, input_clip_ratio=1.0, qmax: int = 6, shadow=False, shadow_min_rows: int = 1024):
         super().__init__()
         self.input_clip_ratio = input_clip_ratio
         self.qmax = qmax
+        # shadow (not in the reference): True also writes the codes as 6-bit floats for the 6-bit float
+        # matrix path of the linear layers, "only" writes nothing else (quantized_x is None); applies to
+        # inputs of at least shadow_min_rows tokens whose width is a multiple of 128
+        self.shadow = shadow
+        self.shadow_min_rows = shadow_min_rows
 
-    def forward(self, x) -> tensor_utils.PackedQuantizedTensor:
+    def forward(self, x, shadow=None) -> tensor_utils.PackedQuantizedTensor:
         if not x.is_contiguous():
             x = x.contiguous()
+        shadow = _shadow_choice(self, x, shadow)
+        if shadow:
+            q, sh, scales = tensor_utils.quantize_sym_shadow(x, self.input_clip_ratio, self.qmax, shadow != "only")
+            return tensor_utils.PackedQuantizedTensor(q, scales, shadow_x=sh)
         if x.shape[-1] % 32 == 0 and x.data_ptr() % 16 == 0:
             q, scales = tensor_utils.quantize_sym(x, self.input_clip_ratio, self.qmax)
         else:  # odd widths: scale with torch ops, quantize with the given-scale kernel
@@ -36,17 +57,23 @@ class AsymQuantizer(torch.nn.Module):
     (quantizer.py:24-35).  ``input_clip_ratio`` is accepted and unused, as in the
     reference."""
 
-    def __init__(self, input_clip_ratio: float = 1.0, shifted: bool = False):
+    def __init__(self, input_clip_ratio: float = 1.0, shifted: bool = False, shadow=False, shadow_min_rows: int = 1024):
         super().__init__()
+        self.shadow = shadow                  # see SymQuantizer
+        self.shadow_min_rows = shadow_min_rows
         self.n_levels = 2 ** 4
         self.input_clip_ratio = input_clip_ratio
         # shifted=True (not in the reference): codes and zero points are stored minus 8, so that the signed
         # GEMM reads them exactly, and the per-token sums of the codes come along for the row-sum epilogue
         self.shifted = shifted
 
-    def forward(self, x) -> tensor_utils.PackedQuantizedTensor:
+    def forward(self, x, shadow=None) -> tensor_utils.PackedQuantizedTensor:
         if not x.is_contiguous():
             x = x.contiguous()
+        shadow = _shadow_choice(self, x, shadow)
+        if shadow:
+            out = tensor_utils.quantize_asym_shadow(x, self.shifted, shadow != "only")
+            return tensor_utils.PackedQuantizedTensor(out[0], out[2], out[3], out[4] if self.shifted else None, shadow_x=out[1])
         if self.shifted:
             assert x.shape[-1] % 32 == 0 and x.data_ptr() % 16 == 0, "shifted quantization needs K % 32 == 0"
             return tensor_utils.PackedQuantizedTensor(*tensor_utils.quantize_asym_shifted(x))

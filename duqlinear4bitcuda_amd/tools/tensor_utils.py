@@ -16,23 +16,28 @@ class PackedQuantizedTensor:
     (tensor_utils.py:20-38)."""
 
     def __init__(self, quantized_x: torch.Tensor, scales_x: torch.Tensor, zeros_x: torch.Tensor = None,
-                 rowsum_x: torch.Tensor = None):
+                 rowsum_x: torch.Tensor = None, shadow_x: torch.Tensor = None):
         self.quantized_x = quantized_x
         self.scales_x = scales_x
         self.zeros_x = zeros_x
         # set only by the signed-shifted asymmetric quantizer (codes - 8, zeros - 8): per-token sums of the codes
         self.rowsum_x = rowsum_x
+        # set by a quantizer with shadow=True / "only": the same codes as 6-bit floats [..., 3K/4] for the
+        # 6-bit float matrix path; with "only", quantized_x is None
+        self.shadow_x = shadow_x
 
     def size(self):
-        return self.quantized_x.size()
+        if self.quantized_x is not None:
+            return self.quantized_x.size()
+        return torch.Size(self.shadow_x.shape[:-1] + (self.shadow_x.shape[-1] * 2 // 3,))
 
     @property
     def device(self):
-        return self.quantized_x.device
+        return self.scales_x.device
 
     @property
     def dtype(self):
-        return self.quantized_x.dtype
+        return torch.uint8
 
 
 def flatten_last_dim_and_return_shape(x: torch.Tensor):
@@ -162,3 +167,28 @@ def linear_forward(mode, xq, scales_x, zeros_x, weight, w_scale_1, w_zeros_1=Non
     """GEMM + dequant (+ bias) in one launch; result has xq's leading dims and N columns."""
     assert xq.shape[-1] % 32 == 0, "A.shape[-1]: {} must be multiplication of 32".format(xq.shape[-1])
     return _ops.linear4bit_forward(mode, xq, scales_x, zeros_x, weight, w_scale_1, w_zeros_1, w_scale_2, w_zeros_2, bias)
+
+
+# ---- 6-bit float matrix path (no counterpart in the reference) ---------------------------
+
+def quantize_sym_shadow(x, clip: float = 1.0, qmax: int = 6, with_q: bool = True):
+    """(q or None, shadow [..., 3K/4], scales): quantize_sym that also (or only) writes the E3M2 shadow."""
+    assert x.dtype == torch.float16
+    return _ops.quantize_rows_sym_bf6(x, clip, qmax, with_q)
+
+
+def quantize_asym_shadow(x, shifted: bool = False, with_q: bool = True):
+    """(q or None, shadow, scales, zeros[, rowsum])."""
+    assert x.dtype == torch.float16
+    return _ops.quantize_rows_asym_bf6(x, shifted, with_q)
+
+
+def weight_shadow(weight):
+    return _ops.weight_shadow_bf6(weight)
+
+
+def linear_forward_shadow(mode, x_shadow, scales_x, zeros_x, weight_shadow, w_scale_1, w_zeros_1=None, w_scale_2=None,
+                          w_zeros_2=None, bias=None, rowsum_x=None, w_rowsum_adj=None):
+    """linear_forward / linear_forward_rowsum on shadows; bit-identical results."""
+    return _ops.linear4bit_forward_bf6(mode, x_shadow, scales_x, zeros_x, weight_shadow, w_scale_1, w_zeros_1, w_scale_2,
+                                       w_zeros_2, bias, rowsum_x, w_rowsum_adj)

@@ -317,3 +317,62 @@ def test_asym_quant_matmul_module(dev, transpose_b):
     st = lambda k: cases.t(np.stack([p[k] for p in params]), dev)
     got = tensor_utils.asym_batch_dequant(cases.t(accs.reshape(*lead, HA, HB), dev), st(0), st(1), st(2), st(3))
     assert cases.bits_equal(got.cpu().numpy(), want)
+
+
+def _bits(t):
+    return t.view(torch.int16)
+
+
+@pytest.mark.gpu
+def test_fp6_matrix_path_in_the_layers(qnn, dev):
+    """enable_fp6(): every layer class gives the same bits through the 6-bit float matrix path as through the
+    integer kernels; the shadow stays out of the state_dict and follows the weights."""
+    _say("fp6 modules")
+    M, K, N = 300, 512, 352
+    torch.manual_seed(5)
+    x = torch.randn(2, M // 2, K, device=dev).half()
+    lin = torch.nn.Linear(K, N, bias=True).half().to(dev)
+    sw = (lin.weight.abs().amax(dim=1, keepdim=True) / 7).half()
+    split = 10
+    s1 = (lin.weight[:, :split].abs().amax(dim=1, keepdim=True) / 7).half()
+    s2 = (lin.weight[:, split:].abs().amax(dim=1, keepdim=True) / 7).half()
+    layers = [
+        (qnn.Linear4bitSQ.from_float(lin, sw).to(dev), qnn.SymQuantizer),
+        (qnn.Linear4bitDUSQ.from_float(lin, s1, s2).to(dev), qnn.SymQuantizer),
+        (qnn.Linear4bitASQ.from_linear(lin).to(dev), None),
+        (qnn.LinearQuant4bitDUASQ.from_linear(lin).to(dev), None),
+        (qnn.Linear4bitASQRowSum.from_linear(lin), None),
+    ]
+    for layer, quantizer in layers:
+        name = type(layer).__name__
+        _say("  ", name)
+        feed = (lambda q: q(x)) if quantizer else (lambda q: x)
+        want = layer(feed(quantizer() if quantizer else None))
+        layer.enable_fp6()
+        layer.fp6_min_tiles = 1
+        assert "weight_shadow" not in layer.state_dict() and layer.weight_shadow.shape == (N, K * 3 // 4)
+        if quantizer:
+            for shadow in (True, "only"):
+                p = quantizer(shadow=shadow, shadow_min_rows=1)(x)
+                assert p.shadow_x is not None and (p.quantized_x is None) == (shadow == "only")
+                assert p.size() == torch.Size((2, M // 2, K // 2))
+                assert torch.equal(_bits(layer(p)), _bits(want)), name
+            # a small input keeps the nibbles only
+            assert quantizer(shadow="only")(x).shadow_x is None
+        else:
+            got = layer(x)
+            assert got.shape == want.shape and torch.equal(_bits(got), _bits(want)), name
+            layer.fp6_min_tiles = 10 ** 6          # too small for the path: integer kernels, same bits
+            assert torch.equal(_bits(layer(x)), _bits(want)), name
+            layer.fp6_min_tiles = 1
+        # new weights: the shadow is rebuilt
+        sd = {k: v.clone() for k, v in layer.state_dict().items()}
+        sd["weight"] = sd["weight"].flip(0).contiguous()
+        layer.load_state_dict(sd)
+        old_shadow = layer.weight_shadow
+        layer.fp6_min_tiles = 10 ** 6
+        want2 = layer(feed(quantizer() if quantizer else None))
+        layer.fp6_min_tiles = 1
+        got2 = layer(quantizer(shadow=True, shadow_min_rows=1)(x)) if quantizer else layer(x)
+        assert torch.equal(_bits(got2), _bits(want2)) and not torch.equal(_bits(got2), _bits(want)), name
+        assert layer.weight_shadow is not old_shadow
