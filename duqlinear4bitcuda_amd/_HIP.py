@@ -461,7 +461,7 @@ EPI_ASYM_ROWSUM = 4
 
 def weight_shadow_bf6(w: torch.Tensor) -> torch.Tensor:
     """E3M2 shadow of packed-int4 weights ``w`` uint8 [N, K/2]: uint8 [N, 3K/4] in the
-    library's tile order.  Made once per weight tensor.  N % 32 == 0, K % 128 == 0."""
+    library's tile order.  Made once per weight tensor.  N % 16 == 0, K % 128 == 0."""
     name = "weight_shadow_bf6"
     if not isinstance(w, torch.Tensor):
         raise RuntimeError(f"{name}: argument #0 is not a tensor")

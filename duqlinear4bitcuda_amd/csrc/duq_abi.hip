@@ -249,7 +249,7 @@ int duq_weight_shadow_bf6(const uint8_t *w, uint32_t N, uint32_t K, uint8_t *w_b
     if (N == 0 || K == 0) return DUQ_OK;
     if (!w || !w_bf6) return DUQ_E_NULL;
     if (K % 128 != 0) return DUQ_E_KALIGN;
-    if (N % 32 != 0) return DUQ_E_SHAPE;
+    if (N % 16 != 0) return DUQ_E_SHAPE;
     if (K > 131008u) return DUQ_E_TOO_LARGE;
     if (!aligned(w, 16) || !aligned(w_bf6, 16)) return DUQ_E_ALIGN;
     return duq::launch_weight_shadow_bf6(w, N, K, w_bf6, as_stream(stream));
@@ -275,7 +275,7 @@ int duq_linear4bit_forward_bf6(int32_t mode, const uint8_t *x_bf6, const duq_hal
     if (M == 0 || N == 0) return DUQ_OK;
     if (!x_bf6 || !w_bf6 || !scale_x || !w_scale_1 || !y) return DUQ_E_NULL;
     if (K == 0 || K % 128 != 0) return DUQ_E_KALIGN;
-    if (N % 32 != 0) return DUQ_E_SHAPE;
+    if (N % 16 != 0) return DUQ_E_SHAPE;
     if (K > 131008u) return DUQ_E_TOO_LARGE;
     const bool asym = mode == DUQ_EPI_ASYM || mode == DUQ_EPI_ASYM_DUAL || mode == DUQ_EPI_ASYM_ROWSUM;
     const bool dual = mode == DUQ_EPI_SYM_DUAL || mode == DUQ_EPI_ASYM_DUAL;

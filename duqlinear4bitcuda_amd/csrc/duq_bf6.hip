@@ -12,15 +12,15 @@
 // v_cvt_scalef32_pk32_bf6_f16 writes them; it is kept as a 16-byte part and an 8-byte part
 // so that every load is naturally aligned.
 //   activation shadow  [M][K/32 x 16 B | K/32 x 8 B]      (row-major, two planes per row)
-//   weight shadow      [N/32][K/128][3 x 64 lanes x 16 B]
+//   weight shadow      [N/16][K/128][64 lanes x 16 B | 64 lanes x 8 B]
 //                      lane l of a (16-row tile, 128-k step) holds the block of row l % 16,
-//                      k-block l / 16: the fragment order of the MFMA.  Two tiles (32 rows) share
-//                      three 1 KB parts: words 0-3 of the first tile's blocks | words 4-5 of the
-//                      first and 0-1 of the second | words 2-5 of the second.  Three 128-bit loads
-//                      per lane fill twelve consecutive registers = the two fragments, and every
-//                      vector memory instruction moves a full 1 KB (the memory pipeline of a CU
-//                      takes one wavefront instruction per 16 cycles whatever its width).
-// K % 128 == 0 and N % 32 == 0: no padding anywhere.
+//                      k-block l / 16: the fragment order of the MFMA, so a wavefront load is
+//                      one contiguous 1 KB (512 B) span and lands in the six registers of the
+//                      fragment without a move.  (A variant with three 128-bit loads per two
+//                      fragments moved fewer instructions through the memory pipeline but cost
+//                      two register moves per fragment and ran no faster: the loop is bound by
+//                      the issue rate of its one wavefront per SIMD.)
+// K % 128 == 0 and N % 16 == 0: no padding anywhere.
 //
 // Kernel: tile 128 (M) x 256 (N) per workgroup, 4 wavefronts side by side along N (128 x 64
 // each: 8 x 4 MFMA tiles, 128 accumulator registers).  Weights go global -> registers (a ring
@@ -36,7 +36,6 @@ namespace duq {
 
 typedef int v2i __attribute__((ext_vector_type(2)));
 typedef int v6i __attribute__((ext_vector_type(6)));
-typedef int v12i __attribute__((ext_vector_type(12)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef _Float16 v32h __attribute__((ext_vector_type(32)));
 
@@ -61,24 +60,22 @@ __device__ __forceinline__ v6i bf6_block_from_nibbles(const v4u w)
 __global__ __launch_bounds__(256) void weight_shadow_kernel(const uint8_t *w, uint32_t N, uint32_t K, uint8_t *out)
 {
     const uint32_t ksteps = K / 128;
-    const uint64_t total = (uint64_t)(N / 32) * ksteps * 64;
+    const uint64_t total = (uint64_t)(N / 16) * ksteps * 64;
     for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (uint64_t)gridDim.x * blockDim.x) {
         const uint32_t lane = (uint32_t)(i & 63u);
-        const uint64_t ps = i >> 6;  // pair * ksteps + step
-        const uint32_t step = (uint32_t)(ps % ksteps), pair = (uint32_t)(ps / ksteps);
-        const uint32_t n = pair * 32 + (lane & 15u), kb = step * 4 + (lane >> 4);
-        const v6i a = bf6_block_from_nibbles(*reinterpret_cast<const v4u *>(w + (uint64_t)n * (K / 2) + kb * 16));
-        const v6i b = bf6_block_from_nibbles(*reinterpret_cast<const v4u *>(w + (uint64_t)(n + 16) * (K / 2) + kb * 16));
-        uint8_t *dst = out + ps * 3072 + lane * 16;
-        *reinterpret_cast<v4i *>(dst) = v4i{a[0], a[1], a[2], a[3]};
-        *reinterpret_cast<v4i *>(dst + 1024) = v4i{a[4], a[5], b[0], b[1]};
-        *reinterpret_cast<v4i *>(dst + 2048) = v4i{b[2], b[3], b[4], b[5]};
+        const uint64_t ts = i >> 6;  // tile * ksteps + step
+        const uint32_t step = (uint32_t)(ts % ksteps), tile = (uint32_t)(ts / ksteps);
+        const uint32_t n = tile * 16 + (lane & 15u), kb = step * 4 + (lane >> 4);
+        const v6i b = bf6_block_from_nibbles(*reinterpret_cast<const v4u *>(w + (uint64_t)n * (K / 2) + kb * 16));
+        uint8_t *dst = out + ts * 1536;
+        *reinterpret_cast<v4i *>(dst + lane * 16) = v4i{b[0], b[1], b[2], b[3]};
+        *reinterpret_cast<v2i *>(dst + 1024 + lane * 8) = v2i{b[4], b[5]};
     }
 }
 
 int launch_weight_shadow_bf6(const uint8_t *w, uint32_t N, uint32_t K, uint8_t *out, hipStream_t stream)
 {
-    const uint64_t total = (uint64_t)(N / 32) * (K / 128) * 64;
+    const uint64_t total = (uint64_t)(N / 16) * (K / 128) * 64;
     if (total == 0) return 0;
     const uint32_t blocks = (uint32_t)std::min<uint64_t>((total + 255) / 256, 1u << 16);
     hipLaunchKernelGGL(weight_shadow_kernel, dim3(blocks), dim3(256), 0, stream, w, N, K, out);
@@ -153,26 +150,30 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
     const uint32_t ksteps = p.K / 128;
     const uint32_t nchunks = (ksteps + 1) / 2;
 
-    const uint32_t wpairs = min(p.N - n0, (uint32_t)BN) / 32;
+    const uint32_t wtiles = min(p.N - n0, (uint32_t)BN) / 16;
     const __amdgpu_buffer_rsrc_t rW =
-        make_rsrc(p.W + (uint64_t)(n0 / 32) * ksteps * 3072, wpairs * ksteps * 3072);
+        make_rsrc(p.W + (uint64_t)(n0 / 16) * ksteps * 1536, wtiles * ksteps * 1536);
     const __amdgpu_buffer_rsrc_t rX =
         make_rsrc(p.X + (uint64_t)m0 * row_bytes, min(p.M - m0, (uint32_t)BM) * row_bytes);
     const __amdgpu_buffer_rsrc_t rNone = make_rsrc(p.X, 0);  // every read returns zero
 
-    // part `part` of weight pair pr (tiles 2*pr, 2*pr + 1 of this wavefront) at step g: 1 KB at
-    // ((wave*2 + pr) * ksteps + g) * 3072 + part * 1024.  The scalar offset is not part of the hardware
-    // range check: pairs past N sit in the vector offset, steps past K switch to the empty descriptor.
-    uint32_t wv[2];
+    // weight fragment (ni, step g): 1536 bytes at ((wave*4 + ni) * ksteps + g) * 1536, a 16-byte and an 8-byte
+    // part per lane.  The scalar offset is not part of the hardware range check: tiles past N sit in the
+    // vector offset, steps past K switch to the empty descriptor.
+    uint32_t wv0[TNI], wv1[TNI];
 #pragma unroll
-    for (int pr = 0; pr < 2; ++pr)
-        wv[pr] = wave * 2 + pr < wpairs ? (wave * 2 + pr) * ksteps * 3072 + lane * 16 : kOobOffset;
-    auto load_w = [&](v12i &dst, int pr, uint32_t g) {
-        const __amdgpu_buffer_rsrc_t r = g < ksteps ? rW : rNone;
-        const v4i a = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(r, (int)wv[pr], (int)(g * 3072), 0));
-        const v4i b = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(r, (int)wv[pr] + 1024, (int)(g * 3072), 0));
-        const v4i c = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(r, (int)wv[pr] + 2048, (int)(g * 3072), 0));
-        dst = v12i{a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3], c[0], c[1], c[2], c[3]};
+    for (int ni = 0; ni < TNI; ++ni) {
+        const bool ok = wave * 4 + ni < wtiles;
+        wv0[ni] = ok ? (wave * 4 + ni) * ksteps * 1536 + lane * 16 : kOobOffset;
+        wv1[ni] = ok ? (wave * 4 + ni) * ksteps * 1536 + 1024 + lane * 8 : kOobOffset;
+    }
+    auto load_w0 = [&](v6i &dst, int ni, uint32_t g, __amdgpu_buffer_rsrc_t r) {
+        const v4i a = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(r, (int)wv0[ni], (int)(g * 1536), 0));
+        dst[0] = a[0], dst[1] = a[1], dst[2] = a[2], dst[3] = a[3];
+    };
+    auto load_w1 = [&](v6i &dst, int ni, uint32_t g, __amdgpu_buffer_rsrc_t r) {
+        const v2i b = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(r, (int)wv1[ni], (int)(g * 1536), 0));
+        dst[4] = b[0], dst[5] = b[1];
     };
 
     // activation pieces of a chunk (256 k = 8 blocks): 4 of plane 0 and 2 of plane 1 per thread
@@ -192,14 +193,14 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
     // piece j of chunk c.  The chunk offset rides in the vector offset so that the range check sees it: when
     // K is an odd number of steps the last chunk's second half reads the next row (unused) or, in the last
     // row, past the descriptor (zero).
-    auto load_x = [&](v4u &dst, int j, uint32_t c) {
-        dst = buf_load16(c < nchunks ? rX : rNone, xoff[j] + (j < 4 ? c * 128 : c * 64), 0);
+    auto load_x = [&](v4u &dst, int j, uint32_t c, __amdgpu_buffer_rsrc_t r) {
+        dst = buf_load16(r, xoff[j] + (j < 4 ? c * 128 : c * 64), 0);
     };
 
     // fragment of rows mi*16 + l16, k-step s of a chunk: plane 0 + mi*16*kP0Stride + s*64, plane 1 + ... + s*32
     const uint32_t frag0 = l16 * kP0Stride + kb * 16, frag1 = kP1Base + l16 * kP1Stride + kb * 8;
 
-    v12i wf[4][2];    // weight fragments [ring slot][pair of column tiles]
+    v6i wf[4][TNI];   // weight fragments [ring slot][column tile]
     v6i xf[4];        // activation fragments, ring over mi
     v4u xreg[6];
     v4f acc[TMI][TNI];
@@ -217,20 +218,33 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
         dst[4] = b[0], dst[5] = b[1];
     };
 
-    // ---- prologue: weights of steps 0..3, activations of chunks 0 and 1 -> LDS, chunk 2 -> registers
+    // ---- prologue: weights of steps 0..3, activations of chunks 0 and 1 -> LDS, chunk 2 -> registers.  Issued
+    // in the order of first use, so that the wait for the two activation chunks (vector memory waits are in
+    // order) leaves the weights of steps 1..3 in flight: all 256 workgroups start together and their first
+    // ~170 KB each are bound by the L2 -> CU rate, not by latency.
+    v4u x1[6];
 #pragma unroll
-    for (int g = 0; g < 4; ++g)
+    for (int j = 0; j < 6; ++j) load_x(xreg[j], j, 0, rX);
 #pragma unroll
-        for (int pr = 0; pr < 2; ++pr) load_w(wf[g][pr], pr, g);
-#pragma unroll
-    for (int q = 0; q < 2; ++q) {
-#pragma unroll
-        for (int j = 0; j < 6; ++j) load_x(xreg[j], j, q);
-#pragma unroll
-        for (int j = 0; j < 6; ++j) *reinterpret_cast<v4u *>(lds + q * kBuf + xlds[j]) = xreg[j];
+    for (int ni = 0; ni < TNI; ++ni) {
+        load_w0(wf[0][ni], ni, 0, rW);
+        load_w1(wf[0][ni], ni, 0, rW);
     }
 #pragma unroll
-    for (int j = 0; j < 6; ++j) load_x(xreg[j], j, 2);
+    for (int j = 0; j < 6; ++j) load_x(x1[j], j, 1, 1 < nchunks ? rX : rNone);
+#pragma unroll
+    for (int g = 1; g < 4; ++g)
+#pragma unroll
+        for (int ni = 0; ni < TNI; ++ni) {
+            load_w0(wf[g][ni], ni, g, (uint32_t)g < ksteps ? rW : rNone);
+            load_w1(wf[g][ni], ni, g, (uint32_t)g < ksteps ? rW : rNone);
+        }
+#pragma unroll
+    for (int j = 0; j < 6; ++j) *reinterpret_cast<v4u *>(lds + xlds[j]) = xreg[j];
+#pragma unroll
+    for (int j = 0; j < 6; ++j) *reinterpret_cast<v4u *>(lds + kBuf + xlds[j]) = x1[j];
+#pragma unroll
+    for (int j = 0; j < 6; ++j) load_x(xreg[j], j, 2, 2 < nchunks ? rX : rNone);
     lds_barrier();
 #pragma unroll
     for (int mi = 0; mi < 2; ++mi) {
@@ -261,23 +275,25 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
     // after its use.
     auto chunk = [&](auto par, uint32_t c, uint32_t cur, uint32_t nxt, uint32_t nx2) {
         constexpr int PAR = decltype(par)::value;
+        // Side work is spread one instruction per MFMA: the loop is bound by the issue rate of its single
+        // wavefront per SIMD, and a slot that holds more than about 12 cycles of other work stalls the matrix pipe.
+        const __amdgpu_buffer_rsrc_t rXc = c + 3 < nchunks ? rX : rNone;
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
             const int slot = 2 * PAR + s;
             const int prev = (slot + 3) & 3;          // slot of the step before this one
             const uint32_t gprev = 2 * c + s - 1 + 4;  // the step that slot receives now
+            const __amdgpu_buffer_rsrc_t rG = gprev < ksteps ? rW : rNone;
 #pragma unroll
             for (int mi = 0; mi < TMI; ++mi) {
 #pragma unroll
                 for (int ni = 0; ni < TNI; ++ni) {
-                    const v12i &wp = wf[slot][ni >> 1];
-                    const v6i wfrag = (ni & 1) ? __builtin_shufflevector(wp, wp, 6, 7, 8, 9, 10, 11)
-                                               : __builtin_shufflevector(wp, wp, 0, 1, 2, 3, 4, 5);
-                    // (s_nop: a register move the compiler places in front of this opaque statement would
-                    // otherwise be too close to the read of the matrix instruction)
-                    asm volatile("s_nop 1\n\tv_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 cbsz:3 blgp:3"
+                    // The operands are written by loads only (the compiler waits for those).  A register move
+                    // placed right in front of this opaque statement would need wait states the compiler
+                    // cannot know of; the generated loop has none, and the bit-exact parity tests would show one.
+                    asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 cbsz:3 blgp:3"
                                  : "+a"(acc[mi][ni])
-                                 : "v"(wfrag), "v"(xf[mi & 3]));
+                                 : "v"(wf[slot][ni]), "v"(xf[mi & 3]));
                     __builtin_amdgcn_sched_barrier(0);
                     // ---- side work in the shadow of this MFMA
                     if (ni < 2) {  // activation fragment two groups ahead
@@ -288,12 +304,16 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
                         else
                             read_x1(xf[nm & 3], buf, nm, ns & 1);
                     }
-                    if (ni == 2 && (mi == 0 || mi == 3))  // refill the previous step's slot (step 0 fetches step 3 again)
-                        load_w(wf[prev][mi / 3], mi / 3, gprev);
-                    if (ni == 3 && s == 1 && mi < 6) {  // chunk c+2 -> its LDS buffer, then fetch chunk c+3
-                        *reinterpret_cast<v4u *>(lds + nx2 + xlds[mi]) = xreg[mi];
-                        load_x(xreg[mi], mi, c + 3);
+                    if (ni == 2) {  // refill the previous step's slot, one load per group (step 0 fetches step 3 again)
+                        if (mi & 1)
+                            load_w1(wf[prev][mi >> 1], mi >> 1, gprev, rG);
+                        else
+                            load_w0(wf[prev][mi >> 1], mi >> 1, gprev, rG);
                     }
+                    if (ni == 3 && s == 1 && mi < 6)  // chunk c+2 -> its LDS buffer
+                        *reinterpret_cast<v4u *>(lds + nx2 + xlds[mi]) = xreg[mi];
+                    if (ni == 1 && s == 1 && mi >= 1 && mi < 7)  // ... and, one group later, fetch chunk c+3 into the register
+                        load_x(xreg[mi - 1], mi - 1, c + 3, rXc);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
@@ -314,14 +334,15 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
     using Even = std::integral_constant<int, 0>;
     using Odd = std::integral_constant<int, 1>;
     uint32_t c = 0;
-    for (; c < nchunks; c += 2) {
+    // (no branch inside the loop: a path that skips a chunk would make the compiler count only that
+    // path's loads when it waits for a fragment, and drain the prefetch ring every iteration)
+    for (; c + 1 < nchunks; c += 2) {
         chunk(Even{}, c, cur, nxt, nx2);
         rotate();
-        if (c + 1 < nchunks) {
-            chunk(Odd{}, c + 1, cur, nxt, nx2);
-            rotate();
-        }
+        chunk(Odd{}, c + 1, cur, nxt, nx2);
+        rotate();
     }
+    if (c < nchunks) chunk(Even{}, c, cur, nxt, nx2);
     // the MFMAs above are opaque to the compiler's hazard tracking: let the last ones retire
     asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 
@@ -338,11 +359,9 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
             quad_cols_from_raw<MODE, BIAS>(raw_s1[ni], raw_z1[ni], raw_s2[ni], raw_z2[ni], raw_bias[ni], nq, raw_rs[ni]);
 #pragma unroll
         for (int mi = 0; mi < TMI; ++mi) {
-            uint16_t out[4];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) out[r] = dequant_one<MODE, BIAS>((int)acc[mi][ni][r], rowp[mi], cols.c[r]);
             *reinterpret_cast<v2u *>(stage + (mi * 16 + l16) * kYStride + ncol * 2) =
-                v2u{(uint32_t)out[0] | ((uint32_t)out[1] << 16), (uint32_t)out[2] | ((uint32_t)out[3] << 16)};
+                v2u{dequant_pair<MODE, BIAS>(acc[mi][ni][0], acc[mi][ni][1], rowp[mi], cols.c[0], cols.c[1]),
+                    dequant_pair<MODE, BIAS>(acc[mi][ni][2], acc[mi][ni][3], rowp[mi], cols.c[2], cols.c[3])};
         }
     }
     const uint32_t rows_here = min(p.M - m0, (uint32_t)BM);

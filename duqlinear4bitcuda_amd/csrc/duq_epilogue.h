@@ -95,6 +95,46 @@ __device__ __forceinline__ uint16_t dequant_one(int acc, const RowEpi &r, const 
     return f16_to_bits(y);
 }
 
+// The same for an accumulator that arrives as an integer-valued float32 (|acc| < 2^24): the
+// binary16 rounding of the float is the rounding of the integer, so only mode 4 converts back.
+template <int MODE, bool BIAS>
+__device__ __forceinline__ uint16_t dequant_one(float acc, const RowEpi &r, const ColParams &c)
+{
+    if (MODE == 4) return dequant_one<MODE, BIAS>((int)acc, r, c);
+    const f16 e = (f16)acc;
+    const f16 ss = r.s * c.s;
+    f16 y;
+    if (MODE == 0 || MODE == 2) {
+        y = ss * e;
+    } else {
+        const f16 t = (e - r.z) - c.z;
+        y = ss * t;
+    }
+    if (BIAS) y = y + c.bias;
+    return f16_to_bits(y);
+}
+
+// Two neighbouring columns of one row at once, on the packed binary16 instructions (each lane of a
+// packed operation rounds like the scalar one): the low half of the result is column c0.
+template <int MODE, bool BIAS, typename ACC>
+__device__ __forceinline__ uint32_t dequant_pair(ACC acc0, ACC acc1, const RowEpi &r, const ColParams &c0,
+                                                 const ColParams &c1)
+{
+    if (MODE == 4)
+        return (uint32_t)dequant_one<MODE, BIAS>(acc0, r, c0) | ((uint32_t)dequant_one<MODE, BIAS>(acc1, r, c1) << 16);
+    const v2h e = v2h{(f16)(float)acc0, (f16)(float)acc1};  // int32 or integer-valued float32: one rounding
+    const v2h ss = v2h{r.s, r.s} * v2h{c0.s, c1.s};
+    v2h y;
+    if (MODE == 0 || MODE == 2) {
+        y = ss * e;
+    } else {
+        const v2h t = (e - v2h{r.z, r.z}) - v2h{c0.z, c1.z};
+        y = ss * t;
+    }
+    if (BIAS) y = y + v2h{c0.bias, c1.bias};
+    return __builtin_bit_cast(uint32_t, y);
+}
+
 // Column parameters of four consecutive output columns n0 .. n0+3, fetched with 64-bit
 // loads when the arrays allow it (`vec`: 8-byte aligned bases and n0 + 3 < cols).
 template <int MODE, bool BIAS>

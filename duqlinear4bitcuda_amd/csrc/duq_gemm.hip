@@ -489,12 +489,9 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
                         raw_rs[t * 4 + q]);
 #pragma unroll
                     for (int b = 0; b < TM; ++b) {
-                        uint16_t out[4];
-#pragma unroll
-                        for (int r = 0; r < 4; ++r)
-                            out[r] = dequant_one<MODE, BIAS>(acc[t][b][q * 4 + r] >> 8, rowp[b], cols.c[r]);
                         *reinterpret_cast<v2u *>(stage + (b * 32 + l32) * kYStride + ncol * 2) =
-                            v2u{(uint32_t)out[0] | ((uint32_t)out[1] << 16), (uint32_t)out[2] | ((uint32_t)out[3] << 16)};
+                            v2u{dequant_pair<MODE, BIAS>(acc[t][b][q * 4] >> 8, acc[t][b][q * 4 + 1] >> 8, rowp[b], cols.c[0], cols.c[1]),
+                                dequant_pair<MODE, BIAS>(acc[t][b][q * 4 + 2] >> 8, acc[t][b][q * 4 + 3] >> 8, rowp[b], cols.c[2], cols.c[3])};
                     }
                 }
             // the same wavefront wrote and reads its stage: LDS operations complete in order

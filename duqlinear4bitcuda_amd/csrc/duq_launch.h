@@ -49,7 +49,7 @@ int launch_gemm_s4(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N, u
 
 
 // 6-bit float (E3M2) shadows of packed-int4 tensors and the GEMM that multiplies them
-// (duq_bf6.hip).  K % 128 == 0, N % 32 == 0.
+// (duq_bf6.hip).  K % 128 == 0, N % 16 == 0.
 int launch_weight_shadow_bf6(const uint8_t *w, uint32_t N, uint32_t K, uint8_t *out, hipStream_t stream);
 int launch_activation_shadow_bf6(const uint8_t *q, uint32_t M, uint32_t K, uint8_t *out, hipStream_t stream);
 int launch_gemm_bf6(const uint8_t *X, const uint8_t *W, uint32_t M, uint32_t N, uint32_t K, const Epilogue &epi,

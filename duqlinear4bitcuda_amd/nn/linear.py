@@ -49,10 +49,10 @@ class _Linear4bitBase(torch.nn.Module):
     def enable_fp6(self):
         """Build the E3M2 shadow of ``weight`` (3/4 byte per element next to the 1/2 byte of the packed
         nibbles; not part of the state_dict; rebuilt when ``weight`` changes).  Results are bit-identical;
-        large inputs run ~20 % faster.  Needs out_features % 32 == 0 and in_features % 128 == 0."""
+        large inputs run ~20 % faster.  Needs out_features % 16 == 0 and in_features % 128 == 0."""
         assert self.weight.is_cuda, "the shadow is built on the GPU: move the layer there first"
-        assert self.out_features % 32 == 0 and self.in_features % 128 == 0, \
-            "the 6-bit float path needs out_features % 32 == 0 and in_features % 128 == 0"
+        assert self.out_features % 16 == 0 and self.in_features % 128 == 0, \
+            "the 6-bit float path needs out_features % 16 == 0 and in_features % 128 == 0"
         self.register_buffer("weight_shadow", tensor_utils.weight_shadow(self.weight), persistent=False)
         self._shadow_key = (self.weight._version, self.weight.data_ptr())
         return self

@@ -216,7 +216,7 @@ int duq_asym_rowsum_dequant_host(const int32_t *q, const duq_half *scale_row, co
  * arguments of duq_linear4bit_forward (modes DUQ_EPI_SYM .. DUQ_EPI_ASYM_DUAL) or of
  * duq_linear4bit_forward_rowsum (mode DUQ_EPI_ASYM_ROWSUM: rowsum_x, w_rowsum_adj; NULL in
  * the other modes); y is bit-identical to theirs.
- * K % 128 == 0, N % 32 == 0; shadows and y 16-byte aligned, per-column arrays 8-byte
+ * K % 128 == 0, N % 16 == 0; shadows and y 16-byte aligned, per-column arrays 8-byte
  * aligned (w_rowsum_adj 16). */
 int duq_weight_shadow_bf6(const uint8_t *w, uint32_t N, uint32_t K, uint8_t *w_bf6, duq_stream_t stream);
 /* duq_quantize_rows_sym / duq_quantize_rows_asym (rowsum NULL) / duq_quantize_rows_asym_shifted

@@ -553,17 +553,15 @@ def activation_shadow_bf6(q_packed):
 
 
 def weight_shadow_bf6(w_packed):
-    """uint8 [N, K/2] -> uint8 [N, 3K/4] in tile order.  For every pair of 16-row tiles and every
-    128-k step, lane l = (row l % 16, k-block l // 16) owns one block of each tile; the 3072
-    bytes of the (pair, step) are three arrays of 64 lanes x 16 bytes: bytes 0-15 of the first
-    tile's blocks | bytes 16-23 of the first and 0-7 of the second | bytes 8-23 of the second.
-    N % 32 == 0, K % 128 == 0."""
+    """uint8 [N, K/2] -> uint8 [N, 3K/4] in tile order.  For every 16-row tile and every 128-k
+    step, lane l = (row l % 16, k-block l // 16) owns one block; the 1536 bytes of the
+    (tile, step) are 64 lanes x bytes 0-15 of their blocks, then 64 lanes x bytes 16-23.
+    N % 16 == 0, K % 128 == 0."""
     v = unpack_i4(w_packed, signed=True)
     N, K = v.shape
     blocks = shadow_block_pack(v.reshape(N, K // 32, 32))  # [N, K/32, 24]
-    b = blocks.reshape(N // 32, 2, 16, K // 128, 4, 24)    # pair, tile, row, step, kb, byte
-    b = b.transpose(0, 3, 1, 4, 2, 5)                      # pair, step, tile, kb, row, byte  (lane = kb*16 + row)
-    first, second = b[:, :, 0].reshape(N // 32, K // 128, 64, 24), b[:, :, 1].reshape(N // 32, K // 128, 64, 24)
-    parts = np.stack([first[..., :16], np.concatenate([first[..., 16:], second[..., :8]], axis=-1), second[..., 8:]],
-                     axis=2)                               # pair, step, part, lane, 16
-    return np.ascontiguousarray(parts).reshape(N, K * 3 // 4)
+    b = blocks.reshape(N // 16, 16, K // 128, 4, 24)       # tile, row, step, kb, byte
+    b = b.transpose(0, 2, 3, 1, 4).reshape(N // 16, K // 128, 64, 24)  # tile, step, lane = kb*16 + row, byte
+    out = np.concatenate([b[..., :16].reshape(N // 16, K // 128, 1024), b[..., 16:].reshape(N // 16, K // 128, 512)],
+                         axis=-1)
+    return np.ascontiguousarray(out).reshape(N, K * 3 // 4)

@@ -88,17 +88,15 @@ def _loop_weight_shadow(q):
     N, K = v.shape
     out = np.zeros(N * K * 3 // 4, np.uint8)
     ksteps = K // 128
-    for pair in range(N // 32):
+    for tile in range(N // 16):
         for step in range(ksteps):
-            base = (pair * ksteps + step) * 3072
+            base = (tile * ksteps + step) * 1536
             for lane in range(64):
                 row, kb = lane % 16, lane // 16
                 k0 = step * 128 + kb * 32
-                a = orc.shadow_block_pack(v[pair * 32 + row, k0:k0 + 32])
-                b = orc.shadow_block_pack(v[pair * 32 + 16 + row, k0:k0 + 32])
-                out[base + lane * 16:base + lane * 16 + 16] = a[:16]
-                out[base + 1024 + lane * 16:base + 1024 + lane * 16 + 16] = np.concatenate([a[16:], b[:8]])
-                out[base + 2048 + lane * 16:base + 2048 + lane * 16 + 16] = b[8:]
+                blk = orc.shadow_block_pack(v[tile * 16 + row, k0:k0 + 32])
+                out[base + lane * 16:base + lane * 16 + 16] = blk[:16]
+                out[base + 1024 + lane * 8:base + 1024 + lane * 8 + 8] = blk[16:]
     return out.reshape(N, K * 3 // 4)
 
 
@@ -106,7 +104,7 @@ def test_shadow_layouts_against_plain_loops():
     rng = np.random.default_rng(2)
     q = rng.integers(0, 256, (5, 128), dtype=np.uint8)       # M = 5, K = 256
     assert np.array_equal(orc.activation_shadow_bf6(q), _loop_activation_shadow(q))
-    w = rng.integers(0, 256, (64, 192), dtype=np.uint8)      # N = 64, K = 384
+    w = rng.integers(0, 256, (48, 192), dtype=np.uint8)      # N = 48, K = 384
     assert np.array_equal(orc.weight_shadow_bf6(w), _loop_weight_shadow(w))
 
 
@@ -116,7 +114,7 @@ def test_abi_validation_bf6_entries():
     buf = (ctypes.c_char * 4096)()
     P = (ctypes.addressof(buf) + 15) & ~15
     assert lib.duq_weight_shadow_bf6(P, 32, 64, P, None) == -3          # K % 128
-    assert lib.duq_weight_shadow_bf6(P, 16, 128, P, None) == -2         # N % 32
+    assert lib.duq_weight_shadow_bf6(P, 24, 128, P, None) == -2         # N % 16
     assert lib.duq_weight_shadow_bf6(P, 32, 128, None, None) == -1
     assert lib.duq_weight_shadow_bf6(P, 0, 128, None, None) == 0
     assert lib.duq_activation_shadow_bf6(P, 4, 192, P, None) == -3
@@ -127,7 +125,7 @@ def test_abi_validation_bf6_entries():
     assert lib.duq_quantize_rows_asym_bf6(P, 2, 128, None, P, P, None, None, None) == -1
     fwd = lib.duq_linear4bit_forward_bf6
     assert fwd(0, P, P, None, None, P, P, None, None, None, None, None, 4, 32, 64, P, None) == -3
-    assert fwd(0, P, P, None, None, P, P, None, None, None, None, None, 4, 48, 128, P, None) == -2
+    assert fwd(0, P, P, None, None, P, P, None, None, None, None, None, 4, 40, 128, P, None) == -2
     assert fwd(5, P, P, None, None, P, P, None, None, None, None, None, 4, 32, 128, P, None) == -4
     assert fwd(1, P, P, None, None, P, P, None, None, None, None, None, 4, 32, 128, P, None) == -1   # zeros missing
     assert fwd(4, P, P, P, None, P, P, P, None, None, None, None, 4, 32, 128, P, None) == -1          # row sums missing
@@ -147,7 +145,7 @@ def _rand_packed(rng, rows, K):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("M,N,K", [(1, 32, 128), (5, 64, 256), (130, 96, 384), (64, 256, 4096), (33, 992, 1152)])
+@pytest.mark.parametrize("M,N,K", [(1, 16, 128), (5, 64, 256), (130, 80, 384), (64, 256, 4096), (33, 1008, 1152)])
 def test_gpu_shadow_kernels_match_the_format(hip, dev, M, N, K):
     print("bf6 shadows", M, N, K, flush=True)
     rng = np.random.default_rng(M + N + K)
@@ -197,12 +195,12 @@ def _epi_inputs(rng, M, N):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("M,N,K", [(1, 32, 128), (128, 256, 128), (128, 256, 256), (100, 224, 640), (257, 512, 1024),
-                                   (130, 96, 384), (300, 992, 1152), (512, 4096, 4096), (64, 1024, 11008)])
+@pytest.mark.parametrize("M,N,K", [(1, 16, 128), (128, 256, 128), (128, 256, 256), (100, 240, 640), (257, 512, 1024),
+                                   (130, 80, 384), (300, 1008, 1152), (512, 4096, 4096), (64, 1024, 11008)])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_gpu_forward_bf6_equals_oracle(hip, dev, M, N, K, with_bias):
     """One and several chunks, odd and even numbers of 128-k steps, ragged M, N that ends inside a
-    workgroup tile and inside a wavefront's pair of tiles; every epilogue."""
+    workgroup tile and inside a wavefront's four tiles; every epilogue."""
     print("bf6 forward", M, N, K, with_bias, flush=True)
     rng = np.random.default_rng(M * 11 + N * 5 + K)
     a, b = _rand_packed(rng, M, K), _rand_packed(rng, N, K)
