@@ -35,7 +35,7 @@ if ROOT not in sys.path:
 PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, published
 PEAK_FP6_TOPS = 10100.0   # MI355X dense fp6 / fp4 MFMA, published
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, published
-GEMM_TRAFFIC_BYTES = None  # fetched + written per launch of the fused GEMM (rocprofv3 counters)
+GEMM_TRAFFIC_BYTES = (49350 + 16384) * 1024  # fetched + written per launch of the fused GEMM (rocprofv3 counters)
 GEMM_I8_TRAFFIC_BYTES = (33047 + 16384) * 1024
 
 
