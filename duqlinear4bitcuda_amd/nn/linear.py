@@ -38,9 +38,10 @@ def _asym_params(w: torch.Tensor):
 class _Linear4bitBase(torch.nn.Module):
     fused = True
     # 6-bit float matrix path (not in the reference): taken when the layer holds a weight shadow
-    # (enable_fp6) and the input brings one, for problems of at least fp6_min_tiles 128 x 256 output tiles
-    # (below that the integer kernels' smaller tiles fill the chip better)
-    fp6_min_tiles = 96
+    # (enable_fp6) and the input brings one, for problems of at least fp6_min_tiles 128 x 256 output tiles,
+    # or more than 256 rows and 12 tiles (below that the integer kernels' smaller tiles fill the chip better;
+    # measured crossover on an MI355X)
+    fp6_min_tiles = 32
     _shadow_key = None
 
     def _finish(self, y):
@@ -49,7 +50,7 @@ class _Linear4bitBase(torch.nn.Module):
     def enable_fp6(self):
         """Build the E3M2 shadow of ``weight`` (3/4 byte per element next to the 1/2 byte of the packed
         nibbles; not part of the state_dict; rebuilt when ``weight`` changes).  Results are bit-identical;
-        large inputs run ~20 % faster.  Needs out_features % 16 == 0 and in_features % 128 == 0."""
+        large inputs run 20-25 % faster.  Needs out_features % 16 == 0 and in_features % 128 == 0."""
         assert self.weight.is_cuda, "the shadow is built on the GPU: move the layer there first"
         assert self.out_features % 16 == 0 and self.in_features % 128 == 0, \
             "the 6-bit float path needs out_features % 16 == 0 and in_features % 128 == 0"
@@ -66,7 +67,8 @@ class _Linear4bitBase(torch.nn.Module):
         return True
 
     def _fp6_wanted(self, rows):
-        return self._fp6_ready() and -(-rows // 128) * -(-self.out_features // 256) >= self.fp6_min_tiles
+        tiles = -(-rows // 128) * -(-self.out_features // 256)
+        return self._fp6_ready() and (tiles >= self.fp6_min_tiles or (rows > 256 and 8 * tiles >= 3 * self.fp6_min_tiles))
 
     def _use_shadow(self, x):
         """The input's shadow is used when the layer is ready for it and the problem is large enough, or
