@@ -128,11 +128,15 @@ struct Bf6Params {
 constexpr uint32_t kP0Stride = 144;  // LDS bytes per row, 16-byte parts of the 8 blocks of a chunk + pad
 constexpr uint32_t kP1Stride = 80;   // LDS bytes per row, 8-byte parts + pad
 
-template <int EPI, bool BIAS>
+// TMI = 8: 128-row tiles.  TMI = 4: 64-row tiles for problems that would leave most CUs without a 128-row tile
+// (half the MFMAs for the same weight traffic, but twice the workgroups).
+template <int TMI, int EPI, bool BIAS>
 __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
 {
-    constexpr int BM = 128, BN = 256;
-    constexpr int TMI = 8, TNI = 4;  // 16 x 16 MFMA tiles per wavefront: 128 rows x 64 columns
+    static_assert(TMI == 8 || TMI == 4, "16-row MFMA tiles per wavefront along M");
+    constexpr int BM = 16 * TMI, BN = 256;
+    constexpr int TNI = 4;           // 16 x 16 MFMA tiles per wavefront along N: BM rows x 64 columns
+    constexpr int NX0 = BM / 32, NX1 = BM / 64, NXP = NX0 + NX1;  // 16-byte activation pieces per thread and chunk
     constexpr uint32_t kP1Base = BM * kP0Stride;
     constexpr uint32_t kBuf = BM * (kP0Stride + kP1Stride);
     constexpr int MODE = EPI;
@@ -176,25 +180,25 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
         dst[4] = b[0], dst[5] = b[1];
     };
 
-    // activation pieces of a chunk (256 k = 8 blocks): 4 of plane 0 and 2 of plane 1 per thread
-    uint32_t xoff[6], xlds[6];
+    // activation pieces of a chunk (256 k = 8 blocks): NX0 of plane 0 and NX1 of plane 1 per thread
+    uint32_t xoff[NXP], xlds[NXP];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < NX0; ++j) {
         const uint32_t row = (tid >> 3) + j * 32, piece = tid & 7u;
         xoff[j] = row * row_bytes + piece * 16;
         xlds[j] = row * kP0Stride + piece * 16;
     }
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < NX1; ++j) {
         const uint32_t row = (tid >> 2) + j * 64, piece = tid & 3u;
-        xoff[4 + j] = row * row_bytes + p1off + piece * 16;
-        xlds[4 + j] = kP1Base + row * kP1Stride + piece * 16;
+        xoff[NX0 + j] = row * row_bytes + p1off + piece * 16;
+        xlds[NX0 + j] = kP1Base + row * kP1Stride + piece * 16;
     }
     // piece j of chunk c.  The chunk offset rides in the vector offset so that the range check sees it: when
     // K is an odd number of steps the last chunk's second half reads the next row (unused) or, in the last
     // row, past the descriptor (zero).
     auto load_x = [&](v4u &dst, int j, uint32_t c, __amdgpu_buffer_rsrc_t r) {
-        dst = buf_load16(r, xoff[j] + (j < 4 ? c * 128 : c * 64), 0);
+        dst = buf_load16(r, xoff[j] + (j < NX0 ? c * 128 : c * 64), 0);
     };
 
     // fragment of rows mi*16 + l16, k-step s of a chunk: plane 0 + mi*16*kP0Stride + s*64, plane 1 + ... + s*32
@@ -202,7 +206,7 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
 
     v6i wf[4][TNI];   // weight fragments [ring slot][column tile]
     v6i xf[4];        // activation fragments, ring over mi
-    v4u xreg[6];
+    v4u xreg[NXP];
     v4f acc[TMI][TNI];
 #pragma unroll
     for (int a = 0; a < TMI; ++a)
@@ -222,16 +226,16 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
     // in the order of first use, so that the wait for the two activation chunks (vector memory waits are in
     // order) leaves the weights of steps 1..3 in flight: all 256 workgroups start together and their first
     // ~170 KB each are bound by the L2 -> CU rate, not by latency.
-    v4u x1[6];
+    v4u x1[NXP];
 #pragma unroll
-    for (int j = 0; j < 6; ++j) load_x(xreg[j], j, 0, rX);
+    for (int j = 0; j < NXP; ++j) load_x(xreg[j], j, 0, rX);
 #pragma unroll
     for (int ni = 0; ni < TNI; ++ni) {
         load_w0(wf[0][ni], ni, 0, rW);
         load_w1(wf[0][ni], ni, 0, rW);
     }
 #pragma unroll
-    for (int j = 0; j < 6; ++j) load_x(x1[j], j, 1, 1 < nchunks ? rX : rNone);
+    for (int j = 0; j < NXP; ++j) load_x(x1[j], j, 1, 1 < nchunks ? rX : rNone);
 #pragma unroll
     for (int g = 1; g < 4; ++g)
 #pragma unroll
@@ -240,11 +244,11 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
             load_w1(wf[g][ni], ni, g, (uint32_t)g < ksteps ? rW : rNone);
         }
 #pragma unroll
-    for (int j = 0; j < 6; ++j) *reinterpret_cast<v4u *>(lds + xlds[j]) = xreg[j];
+    for (int j = 0; j < NXP; ++j) *reinterpret_cast<v4u *>(lds + xlds[j]) = xreg[j];
 #pragma unroll
-    for (int j = 0; j < 6; ++j) *reinterpret_cast<v4u *>(lds + kBuf + xlds[j]) = x1[j];
+    for (int j = 0; j < NXP; ++j) *reinterpret_cast<v4u *>(lds + kBuf + xlds[j]) = x1[j];
 #pragma unroll
-    for (int j = 0; j < 6; ++j) load_x(xreg[j], j, 2, 2 < nchunks ? rX : rNone);
+    for (int j = 0; j < NXP; ++j) load_x(xreg[j], j, 2, 2 < nchunks ? rX : rNone);
     lds_barrier();
 #pragma unroll
     for (int mi = 0; mi < 2; ++mi) {
@@ -297,23 +301,26 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
                     __builtin_amdgcn_sched_barrier(0);
                     // ---- side work in the shadow of this MFMA
                     if (ni < 2) {  // activation fragment two groups ahead
-                        const int nm = (mi + 2) & 7, ns = mi + 2 < 8 ? s : s + 1;
+                        const int nm = (mi + 2) & (TMI - 1), ns = mi + 2 < TMI ? s : s + 1;
                         const uint32_t buf = ns < 2 ? cur : nxt;
                         if (ni == 0)
                             read_x0(xf[nm & 3], buf, nm, ns & 1);
                         else
                             read_x1(xf[nm & 3], buf, nm, ns & 1);
                     }
-                    if (ni == 2) {  // refill the previous step's slot, one load per group (step 0 fetches step 3 again)
+                    // refill the previous step's slot: eight loads over the step (step 0 fetches step 3 again)
+                    if (TMI == 8 && ni == 2) {
                         if (mi & 1)
                             load_w1(wf[prev][mi >> 1], mi >> 1, gprev, rG);
                         else
                             load_w0(wf[prev][mi >> 1], mi >> 1, gprev, rG);
                     }
-                    if (ni == 3 && s == 1 && mi < 6)  // chunk c+2 -> its LDS buffer
+                    if (TMI == 4 && ni == 2) load_w0(wf[prev][mi], mi, gprev, rG);
+                    if (TMI == 4 && ni == 3) load_w1(wf[prev][mi], mi, gprev, rG);
+                    // chunk c+2 -> its LDS buffer and, one group later, chunk c+3 into the freed register
+                    if (s == 1 && mi < NXP && ni == (TMI == 8 ? 3 : 0))
                         *reinterpret_cast<v4u *>(lds + nx2 + xlds[mi]) = xreg[mi];
-                    if (ni == 1 && s == 1 && mi >= 1 && mi < 7)  // ... and, one group later, fetch chunk c+3 into the register
-                        load_x(xreg[mi - 1], mi - 1, c + 3, rXc);
+                    if (s == 1 && ni == 1 && mi >= 1 && mi <= NXP) load_x(xreg[mi - 1], mi - 1, c + 3, rXc);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
@@ -377,14 +384,31 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
     }
 }
 
-template <int EPI>
-static void launch_mode(const Bf6Params &p, hipStream_t stream)
+template <int TMI, int EPI>
+static void launch_tile(const Bf6Params &p, hipStream_t stream)
 {
     const dim3 grid(p.tiles_m * p.tiles_n);
     if (p.epi.bias)
-        hipLaunchKernelGGL((gemm_bf6_kernel<EPI, true>), grid, dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((gemm_bf6_kernel<TMI, EPI, true>), grid, dim3(256), 0, stream, p);
     else
-        hipLaunchKernelGGL((gemm_bf6_kernel<EPI, false>), grid, dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((gemm_bf6_kernel<TMI, EPI, false>), grid, dim3(256), 0, stream, p);
+}
+
+template <int EPI>
+static void launch_mode(Bf6Params &p, hipStream_t stream)
+{
+    // Tile height: whole rounds of 256 workgroups, a 64-row tile priced at kCost64 of a 128-row one (it does half
+    // the MFMAs for the same weight traffic; measured on an MI355X).
+    constexpr float kCost64 = 0.68f;
+    const uint32_t t128 = ((p.M + 127) / 128) * p.tiles_n, t64 = ((p.M + 63) / 64) * p.tiles_n;
+    const float c128 = (float)((t128 + 255) / 256), c64 = kCost64 * (float)((t64 + 255) / 256);
+    if (c64 < c128) {
+        p.tiles_m = (p.M + 63) / 64;
+        launch_tile<4, EPI>(p, stream);
+    } else {
+        p.tiles_m = (p.M + 127) / 128;
+        launch_tile<8, EPI>(p, stream);
+    }
 }
 
 int launch_gemm_bf6(const uint8_t *X, const uint8_t *W, uint32_t M, uint32_t N, uint32_t K, const Epilogue &epi,

@@ -196,7 +196,9 @@ def _epi_inputs(rng, M, N):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("M,N,K", [(1, 16, 128), (128, 256, 128), (128, 256, 256), (100, 240, 640), (257, 512, 1024),
-                                   (130, 80, 384), (300, 1008, 1152), (512, 4096, 4096), (64, 1024, 11008)])
+                                   (130, 80, 384), (300, 1008, 1152), (512, 4096, 4096), (64, 1024, 11008),
+                                   # enough tiles for the 128-row variant of the kernel (the ones above run 64-row tiles)
+                                   (2048 + 70, 4096 - 48, 384), (2048, 4096, 128)])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_gpu_forward_bf6_equals_oracle(hip, dev, M, N, K, with_bias):
     """One and several chunks, odd and even numbers of 128-k steps, ragged M, N that ends inside a
