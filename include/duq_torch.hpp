@@ -54,8 +54,11 @@ class PackedQuantizedTensor {
 public:
     torch::Tensor quantized_x;
     torch::Tensor scale;
-    PackedQuantizedTensor(torch::Tensor quantized_x, torch::Tensor scale)
-        : quantized_x(std::move(quantized_x)), scale(std::move(scale)) {}
+    // not in the reference: the same codes as 6-bit floats [..., 3K/4] for the 6-bit float matrix path
+    // (Quantizer4bit with shadow = true); undefined otherwise
+    torch::Tensor shadow_x;
+    PackedQuantizedTensor(torch::Tensor quantized_x, torch::Tensor scale, torch::Tensor shadow_x = torch::Tensor())
+        : quantized_x(std::move(quantized_x)), scale(std::move(scale)), shadow_x(std::move(shadow_x)) {}
     torch::IntArrayRef sizes() const { return quantized_x.sizes(); }
     torch::Device device() const { return quantized_x.device(); }
 };
@@ -165,7 +168,9 @@ class Quantizer4bit : public torch::nn::Module {
 public:
     float input_clip_ratio;
     int qmax;
-    explicit Quantizer4bit(float input_clip_ratio, int qmax = DUQ_QMAX_SYM_DEVICE) : input_clip_ratio(input_clip_ratio), qmax(qmax) {}
+    bool shadow;  // also write the 6-bit float shadow (inputs whose width is a multiple of 128)
+    explicit Quantizer4bit(float input_clip_ratio, int qmax = DUQ_QMAX_SYM_DEVICE, bool shadow = false)
+        : input_clip_ratio(input_clip_ratio), qmax(qmax), shadow(shadow) {}
     PackedQuantizedTensor forward(torch::Tensor x)
     {
         x = x.contiguous();
@@ -175,13 +180,23 @@ public:
         TORCH_CHECK(cols % 32 == 0, "Quantizer4bit::forward: the last dimension must be a multiple of 32");
         auto q = torch::empty({rows, cols / 2}, torch::dtype(torch::kUInt8).device(x.device()));
         auto s = torch::empty({rows, 1}, torch::dtype(torch::kHalf).device(x.device()));
-        check_status(duq_quantize_rows_sym(half_ptr(x2), rows, cols, input_clip_ratio, qmax, q.data_ptr<uint8_t>(),
-                                           reinterpret_cast<duq_half *>(s.data_ptr()), current_stream(x)),
-                     "Quantizer4bit::forward");
         auto qshape = lead;
         qshape.push_back(cols / 2);
         auto sshape = lead;
         sshape.push_back(1);
+        if (shadow && cols % 128 == 0) {
+            auto b = torch::empty({rows, cols * 3 / 4}, torch::dtype(torch::kUInt8).device(x.device()));
+            check_status(duq_quantize_rows_sym_bf6(half_ptr(x2), rows, cols, input_clip_ratio, qmax, q.data_ptr<uint8_t>(),
+                                                   b.data_ptr<uint8_t>(), reinterpret_cast<duq_half *>(s.data_ptr()),
+                                                   current_stream(x)),
+                         "Quantizer4bit::forward");
+            auto bshape = lead;
+            bshape.push_back(cols * 3 / 4);
+            return PackedQuantizedTensor(q.view(qshape), s.view(sshape), b.view(bshape));
+        }
+        check_status(duq_quantize_rows_sym(half_ptr(x2), rows, cols, input_clip_ratio, qmax, q.data_ptr<uint8_t>(),
+                                           reinterpret_cast<duq_half *>(s.data_ptr()), current_stream(x)),
+                     "Quantizer4bit::forward");
         return PackedQuantizedTensor(q.view(qshape), s.view(sshape));
     }
 };
@@ -198,6 +213,47 @@ public:
 };
 
 namespace detail {
+// E3M2 shadow of packed weights [N, K/2] -> [N, 3K/4] (N % 16 == 0, K % 128 == 0)
+inline torch::Tensor weight_shadow(const torch::Tensor &weight)
+{
+    check_device_tensor(weight, "weight_shadow", "weight");
+    const uint32_t N = weight.size(0), K = weight.size(1) * 2;
+    auto out = torch::empty({N, K * 3 / 4}, torch::dtype(torch::kUInt8).device(weight.device()));
+    check_status(duq_weight_shadow_bf6(weight.data_ptr<uint8_t>(), N, K, out.data_ptr<uint8_t>(), current_stream(weight)),
+                 "weight_shadow");
+    return out;
+}
+
+// The 6-bit float matrix path is taken when both shadows exist and the problem has at least 32 output tiles of
+// 64 x 256 (below, the integer kernels do better); same bits either way.
+inline bool use_shadow(const PackedQuantizedTensor &input, const torch::Tensor &w_shadow, int64_t N)
+{
+    if (!input.shadow_x.defined() || !w_shadow.defined()) return false;
+    const int64_t rows = input.shadow_x.numel() / input.shadow_x.size(-1);
+    return ((rows + 63) / 64) * ((N + 255) / 256) >= 32;
+}
+
+inline torch::Tensor fused_forward_shadow(int mode, const PackedQuantizedTensor &input, const torch::Tensor &w_shadow,
+                                          const torch::Tensor &s1, const torch::Tensor &s2, const torch::Tensor &bias)
+{
+    auto [A, lead] = flatten_last_dim_and_return_shape(input.shadow_x);
+    check_device_tensor(A, "Linear4bit::forward", "shadow_x");
+    TORCH_CHECK(A.device() == w_shadow.device(), "Linear4bit::forward: operands on different devices");
+    TORCH_CHECK(w_shadow.size(1) == A.size(1), "Linear4bit::forward: shadow row length differs");
+    const uint32_t M = A.size(0), N = w_shadow.size(0), K = A.size(1) * 4 / 3;
+    auto scale_row = input.scale.contiguous().view(-1);
+    TORCH_CHECK(scale_row.size(0) == M, "Linear4bit::forward: one activation scale per token expected");
+    auto y = torch::empty({M, N}, torch::dtype(torch::kHalf).device(A.device()));
+    check_status(duq_linear4bit_forward_bf6(mode, A.data_ptr<uint8_t>(), half_ptr(scale_row), nullptr, nullptr,
+                                            w_shadow.data_ptr<uint8_t>(), half_ptr(s1), nullptr,
+                                            s2.defined() ? half_ptr(s2) : nullptr, nullptr, nullptr,
+                                            bias.defined() ? half_ptr(bias) : nullptr, M, N, K,
+                                            reinterpret_cast<duq_half *>(y.data_ptr()), current_stream(A)),
+                 "Linear4bit::forward");
+    lead.push_back(N);
+    return y.view(lead);
+}
+
 inline torch::Tensor fused_forward(int mode, const PackedQuantizedTensor &input, const torch::Tensor &weight,
                                    const torch::Tensor &s1, const torch::Tensor &s2, const torch::Tensor &bias)
 {
@@ -236,8 +292,21 @@ public:
         if (use_bias) bias = torch::zeros({output_dim}, torch::dtype(dtype).device(torch::kCUDA));
     }
 
+    torch::Tensor weight_shadow;  // not in the reference: 6-bit float shadow of `weight`, see enable_fp6()
+
+    // Build the 6-bit float shadow of the weights (3/4 byte per element more): large inputs quantized with
+    // Quantizer4bit(..., shadow = true) then run on the 6-bit float matrix instruction, same bits, faster.
+    // Call again after changing `weight`.
+    Linear4bit &enable_fp6()
+    {
+        weight_shadow = detail::weight_shadow(weight);
+        return *this;
+    }
+
     torch::Tensor forward(PackedQuantizedTensor input)
     {
+        if (detail::use_shadow(input, weight_shadow, weight.size(0)))
+            return detail::fused_forward_shadow(DUQ_EPI_SYM, input, weight_shadow, weight_scale.view(-1), torch::Tensor(), bias);
         return detail::fused_forward(DUQ_EPI_SYM, input, weight, weight_scale.view(-1), torch::Tensor(), bias);
     }
 
@@ -271,8 +340,19 @@ public:
         if (use_bias) bias = torch::zeros({output_dim}, torch::dtype(dtype).device(torch::kCUDA));
     }
 
+    torch::Tensor weight_shadow;  // see Linear4bit::enable_fp6()
+
+    Linear4bitDUQ &enable_fp6()
+    {
+        weight_shadow = detail::weight_shadow(weight);
+        return *this;
+    }
+
     torch::Tensor forward(PackedQuantizedTensor input)
     {
+        if (detail::use_shadow(input, weight_shadow, weight.size(0)))
+            return detail::fused_forward_shadow(DUQ_EPI_SYM_DUAL, input, weight_shadow, weight_scale_1.view(-1),
+                                                weight_scale_2.view(-1), bias);
         return detail::fused_forward(DUQ_EPI_SYM_DUAL, input, weight, weight_scale_1.view(-1), weight_scale_2.view(-1), bias);
     }
 

@@ -64,6 +64,26 @@ int main(int argc, char **argv)
                 d.bias).view({3, M / 3, N});
     if (!same_bits(yd, yd3)) { std::puts("FAIL Linear4bitDUQ fused vs three-step"); return 1; }
 
+    // 6-bit float matrix path: large enough input (>= 32 tiles of 64 x 256), shadows on both sides, same bits
+    if (K % 128 == 0 && N % 16 == 0) {
+        const int64_t M2 = 64 * 32 * 256 / ((N + 255) / 256 * 256) + 64;
+        auto x2 = (torch::randn({M2, K}, torch::dtype(torch::kFloat32).device(dev)) * 1.5).to(torch::kHalf);
+        duq::Quantizer4bit quant6(1.0f, DUQ_QMAX_SYM_DEVICE, true);
+        auto p6 = quant6.forward(x2);
+        auto p4 = quant.forward(x2);
+        if (!p6.shadow_x.defined() || p6.shadow_x.size(-1) != K * 3 / 4 || !torch::equal(p6.quantized_x, p4.quantized_x)) {
+            std::puts("FAIL shadow quantizer"); return 1;
+        }
+        auto y4 = l.forward(p4);
+        auto yd4 = d.forward(p4);
+        l.enable_fp6();
+        d.enable_fp6();
+        if (!duq::detail::use_shadow(p6, l.weight_shadow, N)) { std::puts("FAIL 6-bit float path not taken"); return 1; }
+        if (!same_bits(l.forward(p6), y4)) { std::puts("FAIL Linear4bit 6-bit float path vs integer path"); return 1; }
+        if (!same_bits(d.forward(p6), yd4)) { std::puts("FAIL Linear4bitDUQ 6-bit float path vs integer path"); return 1; }
+        if (!same_bits(l.forward(p4), y4)) { std::puts("FAIL Linear4bit without an activation shadow"); return 1; }
+    }
+
     bool threw = false;
     try { duq::sym_dequant(acc, p.scale.view(-1), l.weight_scale.view(-1), 16); } catch (const c10::Error &) { threw = true; }
     if (!threw) { std::puts("FAIL bits != 32 accepted"); return 1; }
