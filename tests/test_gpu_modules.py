@@ -376,3 +376,39 @@ def test_fp6_matrix_path_in_the_layers(qnn, dev):
         got2 = layer(quantizer(shadow=True, shadow_min_rows=1)(x)) if quantizer else layer(x)
         assert torch.equal(_bits(got2), _bits(want2)) and not torch.equal(_bits(got2), _bits(want)), name
         assert layer.weight_shadow is not old_shadow
+
+
+@pytest.mark.gpu
+def test_step_replays_from_a_hip_graph(qnn, dev):
+    """A whole step (quantize + linear) on either matrix path, captured once and replayed several times with the
+    program's own eager work and synchronisations in between: every replay equals the eager result (the library
+    allocates nothing and records no memset; outputs come from torch's graph-private pool)."""
+    _say("graph replay")
+    M, K, N = 2304, 512, 512
+    torch.manual_seed(11)
+    lin = torch.nn.Linear(K, N, bias=True).half().to(dev)
+    sw = (lin.weight.abs().amax(dim=1, keepdim=True) / 7).half()
+    layer = qnn.Linear4bitSQ.from_float(lin, sw).to(dev)
+    for fp6 in (False, True):
+        if fp6:
+            layer.enable_fp6()
+        quant = qnn.SymQuantizer(1.0, shadow="only" if fp6 else False, shadow_min_rows=1)
+        x = torch.randn(M, K, device=dev).half()
+        want = layer(quant(x)).clone()
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            layer(quant(x))
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            y = layer(quant(x))
+        for rep in range(4):
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(_bits(y), _bits(want)), (fp6, rep)
+            # eager work between replays, and new input in the captured buffer for the next one
+            noise = layer(quant(torch.randn(M, K, device=dev).half()))
+            x.copy_(torch.randn(M, K, device=dev).half())
+            want = layer(quant(x)).clone()
+            torch.cuda.synchronize()
+            assert noise.shape == want.shape
