@@ -116,6 +116,10 @@ int launch_activation_shadow_bf6(const uint8_t *q, uint32_t M, uint32_t K, uint8
 // prefetches issued just before it (a full memory latency per chunk).
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+#ifndef DUQ_BF6_COST256
+#define DUQ_BF6_COST256 1.78f
+#endif
+
 struct Bf6Params {
     const uint8_t *X;  // activation shadow
     const uint8_t *W;  // weight shadow
@@ -125,23 +129,32 @@ struct Bf6Params {
     uint32_t tiles_m, tiles_n;
 };
 
-constexpr uint32_t kP0Stride = 144;  // LDS bytes per row, 16-byte parts of the 8 blocks of a chunk + pad
-constexpr uint32_t kP1Stride = 80;   // LDS bytes per row, 8-byte parts + pad
-
 // TMI = 8: 128-row tiles.  TMI = 4: 64-row tiles for problems that would leave most CUs without a 128-row tile
-// (half the MFMAs for the same weight traffic, but twice the workgroups).
+// (half the MFMAs for the same weight traffic, but twice the workgroups).  TMI = 16: 256-row tiles for problems
+// with at least one such tile per CU: the same weight traffic feeds twice the MFMAs, which takes the kernel off
+// the L2 -> CU limit that bounds the smaller tiles; all 256 AGPRs hold accumulators, an activation chunk is one
+// 128-k step (three buffers of two steps would not fit in LDS) and the epilogue parameters are fetched after the loop.
 template <int TMI, int EPI, bool BIAS>
 __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
 {
-    static_assert(TMI == 8 || TMI == 4, "16-row MFMA tiles per wavefront along M");
+    static_assert(TMI == 16 || TMI == 8 || TMI == 4, "16-row MFMA tiles per wavefront along M");
     constexpr int BM = 16 * TMI, BN = 256;
     constexpr int TNI = 4;           // 16 x 16 MFMA tiles per wavefront along N: BM rows x 64 columns
-    constexpr int NX0 = BM / 32, NX1 = BM / 64, NXP = NX0 + NX1;  // 16-byte activation pieces per thread and chunk
+    constexpr int CH = TMI == 16 ? 1 : 2;  // 128-k steps per activation chunk
+    constexpr int NPH = 4 / CH;            // chunk bodies per turn of the weight ring
+    // 16-byte activation pieces per thread and chunk: plane 0 (4*CH per row), plane 1 (2*CH per row)
+    constexpr int NX0 = BM * 4 * CH / 256, NX1 = BM * 2 * CH / 256, NXP = NX0 + NX1;
+    // LDS bytes per row: the 16-byte (8-byte) parts of the 4*CH blocks of a chunk + 16 bytes of padding, which
+    // makes the fragment reads of 16 rows conflict-free
+    constexpr uint32_t kP0Stride = 64 * CH + 16, kP1Stride = 32 * CH + 16;
     constexpr uint32_t kP1Base = BM * kP0Stride;
     constexpr uint32_t kBuf = BM * (kP0Stride + kP1Stride);
+    constexpr uint32_t kYStride = 144;  // bytes per staged output row: 128 + pad
+    constexpr uint32_t kLds = 3 * kBuf > 4 * BM * kYStride ? 3 * kBuf : 4 * BM * kYStride;
+    constexpr bool LATE_PARAMS = TMI == 16;
     constexpr int MODE = EPI;
 
-    __shared__ __attribute__((aligned(16))) uint8_t lds[3 * kBuf];
+    __shared__ __attribute__((aligned(16))) uint8_t lds[kLds];
 
     uint32_t tile_m, tile_n;
     tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
@@ -152,7 +165,7 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
     const uint32_t nblk = p.K / 32;
     const uint32_t row_bytes = nblk * 24, p1off = nblk * 16;
     const uint32_t ksteps = p.K / 128;
-    const uint32_t nchunks = (ksteps + 1) / 2;
+    const uint32_t nchunks = (ksteps + CH - 1) / CH;
 
     const uint32_t wtiles = min(p.N - n0, (uint32_t)BN) / 16;
     const __amdgpu_buffer_rsrc_t rW =
@@ -184,13 +197,13 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
     uint32_t xoff[NXP], xlds[NXP];
 #pragma unroll
     for (int j = 0; j < NX0; ++j) {
-        const uint32_t row = (tid >> 3) + j * 32, piece = tid & 7u;
+        const uint32_t row = tid / (4 * CH) + j * (256 / (4 * CH)), piece = tid % (4 * CH);
         xoff[j] = row * row_bytes + piece * 16;
         xlds[j] = row * kP0Stride + piece * 16;
     }
 #pragma unroll
     for (int j = 0; j < NX1; ++j) {
-        const uint32_t row = (tid >> 2) + j * 64, piece = tid & 3u;
+        const uint32_t row = tid / (2 * CH) + j * (256 / (2 * CH)), piece = tid % (2 * CH);
         xoff[NX0 + j] = row * row_bytes + p1off + piece * 16;
         xlds[NX0 + j] = kP1Base + row * kP1Stride + piece * 16;
     }
@@ -198,7 +211,7 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
     // K is an odd number of steps the last chunk's second half reads the next row (unused) or, in the last
     // row, past the descriptor (zero).
     auto load_x = [&](v4u &dst, int j, uint32_t c, __amdgpu_buffer_rsrc_t r) {
-        dst = buf_load16(r, xoff[j] + (j < NX0 ? c * 128 : c * 64), 0);
+        dst = buf_load16(r, xoff[j] + (j < NX0 ? c * (64 * CH) : c * (32 * CH)), 0);
     };
 
     // fragment of rows mi*16 + l16, k-step s of a chunk: plane 0 + mi*16*kP0Stride + s*64, plane 1 + ... + s*32
@@ -256,37 +269,40 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
         read_x1(xf[mi], 0, mi, 0);
     }
 
-    // ---- epilogue parameters: fetched now so that their latency hides behind the main loop
+    // ---- epilogue parameters: fetched now so that their latency hides behind the main loop (after the loop for
+    // the 256-row tile, whose loop has no registers to spare)
     const Epilogue &e = p.epi;
     v2u raw_s1[TNI], raw_z1[TNI], raw_s2[TNI], raw_z2[TNI], raw_bias[TNI];
     v4i raw_rs[TNI];
     RowEpi rowp[TMI];
+    auto load_params = [&]() {
 #pragma unroll
-    for (int mi = 0; mi < TMI; ++mi) rowp[mi] = load_row<MODE>(e, min(m0 + mi * 16 + l16, p.M - 1));
+        for (int mi = 0; mi < TMI; ++mi) rowp[mi] = load_row<MODE>(e, min(m0 + mi * 16 + l16, p.M - 1));
 #pragma unroll
-    for (int ni = 0; ni < TNI; ++ni) {
-        const uint32_t nq = min(n0 + wave * 64 + ni * 16 + kb * 4, p.N - 4);
-        raw_s1[ni] = *reinterpret_cast<const v2u *>(e.s_col_1 + nq);
-        if (MODE == 1 || MODE == 3 || MODE == 4) raw_z1[ni] = *reinterpret_cast<const v2u *>(e.z_col_1 + nq);
-        if (MODE == 4) raw_rs[ni] = *reinterpret_cast<const v4i *>(e.rs_col + nq);
-        if (MODE >= 2 && MODE != 4) raw_s2[ni] = *reinterpret_cast<const v2u *>(e.s_col_2 + nq);
-        if (MODE == 3) raw_z2[ni] = *reinterpret_cast<const v2u *>(e.z_col_2 + nq);
-        if (BIAS) raw_bias[ni] = *reinterpret_cast<const v2u *>(e.bias + nq);
-    }
+        for (int ni = 0; ni < TNI; ++ni) {
+            const uint32_t nq = min(n0 + wave * 64 + ni * 16 + kb * 4, p.N - 4);
+            raw_s1[ni] = *reinterpret_cast<const v2u *>(e.s_col_1 + nq);
+            if (MODE == 1 || MODE == 3 || MODE == 4) raw_z1[ni] = *reinterpret_cast<const v2u *>(e.z_col_1 + nq);
+            if (MODE == 4) raw_rs[ni] = *reinterpret_cast<const v4i *>(e.rs_col + nq);
+            if (MODE >= 2 && MODE != 4) raw_s2[ni] = *reinterpret_cast<const v2u *>(e.s_col_2 + nq);
+            if (MODE == 3) raw_z2[ni] = *reinterpret_cast<const v2u *>(e.z_col_2 + nq);
+            if (BIAS) raw_bias[ni] = *reinterpret_cast<const v2u *>(e.bias + nq);
+        }
+    };
+    if (!LATE_PARAMS) load_params();
 
-    // One chunk = two 128-k steps.  PAR = chunk parity: the weight ring slots of this chunk
-    // are 2*PAR and 2*PAR + 1; a slot is refilled (with the step four ahead) during the step
-    // after its use.
-    auto chunk = [&](auto par, uint32_t c, uint32_t cur, uint32_t nxt, uint32_t nx2) {
-        constexpr int PAR = decltype(par)::value;
+    // One chunk = CH 128-k steps.  PH = position of the chunk in a turn of the weight ring: its steps use ring
+    // slots CH*PH ..; a slot is refilled (with the step four ahead) during the step after its use.
+    auto chunk = [&](auto ph, uint32_t c, uint32_t cur, uint32_t nxt, uint32_t nx2) {
+        constexpr int PH = decltype(ph)::value;
         // Side work is spread one instruction per MFMA: the loop is bound by the issue rate of its single
         // wavefront per SIMD, and a slot that holds more than about 12 cycles of other work stalls the matrix pipe.
         const __amdgpu_buffer_rsrc_t rXc = c + 3 < nchunks ? rX : rNone;
 #pragma unroll
-        for (int s = 0; s < 2; ++s) {
-            const int slot = 2 * PAR + s;
+        for (int s = 0; s < CH; ++s) {
+            const int slot = CH * PH + s;
             const int prev = (slot + 3) & 3;          // slot of the step before this one
-            const uint32_t gprev = 2 * c + s - 1 + 4;  // the step that slot receives now
+            const uint32_t gprev = CH * c + s - 1 + 4;  // the step that slot receives now
             const __amdgpu_buffer_rsrc_t rG = gprev < ksteps ? rW : rNone;
 #pragma unroll
             for (int mi = 0; mi < TMI; ++mi) {
@@ -302,11 +318,11 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
                     // ---- side work in the shadow of this MFMA
                     if (ni < 2) {  // activation fragment two groups ahead
                         const int nm = (mi + 2) & (TMI - 1), ns = mi + 2 < TMI ? s : s + 1;
-                        const uint32_t buf = ns < 2 ? cur : nxt;
+                        const uint32_t buf = ns < CH ? cur : nxt;
                         if (ni == 0)
-                            read_x0(xf[nm & 3], buf, nm, ns & 1);
+                            read_x0(xf[nm & 3], buf, nm, ns % CH);
                         else
-                            read_x1(xf[nm & 3], buf, nm, ns & 1);
+                            read_x1(xf[nm & 3], buf, nm, ns % CH);
                     }
                     // refill the previous step's slot: eight loads over the step (step 0 fetches step 3 again)
                     if (TMI == 8 && ni == 2) {
@@ -317,10 +333,20 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
                     }
                     if (TMI == 4 && ni == 2) load_w0(wf[prev][mi], mi, gprev, rG);
                     if (TMI == 4 && ni == 3) load_w1(wf[prev][mi], mi, gprev, rG);
-                    // chunk c+2 -> its LDS buffer and, one group later, chunk c+3 into the freed register
-                    if (s == 1 && mi < NXP && ni == (TMI == 8 ? 3 : 0))
+                    if (TMI == 16 && ni == 2 && (mi & 1) == 0) {
+                        if (mi & 2)
+                            load_w1(wf[prev][mi >> 2], mi >> 2, gprev, rG);
+                        else
+                            load_w0(wf[prev][mi >> 2], mi >> 2, gprev, rG);
+                    }
+                    // chunk c+2 -> its LDS buffer and, one group (one slot) later, chunk c+3 into the freed register
+                    if (TMI <= 8 && s == 1 && mi < NXP && ni == (TMI == 8 ? 3 : 0))
                         *reinterpret_cast<v4u *>(lds + nx2 + xlds[mi]) = xreg[mi];
-                    if (s == 1 && ni == 1 && mi >= 1 && mi <= NXP) load_x(xreg[mi - 1], mi - 1, c + 3, rXc);
+                    if (TMI <= 8 && s == 1 && ni == 1 && mi >= 1 && mi <= NXP) load_x(xreg[mi - 1], mi - 1, c + 3, rXc);
+                    if (TMI == 16 && (mi & 1) == 1 && (mi >> 1) < NXP) {
+                        if (ni == 2) *reinterpret_cast<v4u *>(lds + nx2 + xlds[mi >> 1]) = xreg[mi >> 1];
+                        if (ni == 3) load_x(xreg[mi >> 1], mi >> 1, c + 3, rXc);
+                    }
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
@@ -338,25 +364,49 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
         nxt = nx2;
         nx2 = t;
     };
-    using Even = std::integral_constant<int, 0>;
-    using Odd = std::integral_constant<int, 1>;
+    using P0 = std::integral_constant<int, 0>;
+    using P1 = std::integral_constant<int, 1>;
+    using P2 = std::integral_constant<int, 2>;
+    using P3 = std::integral_constant<int, 3>;
     uint32_t c = 0;
     // (no branch inside the loop: a path that skips a chunk would make the compiler count only that
     // path's loads when it waits for a fragment, and drain the prefetch ring every iteration)
-    for (; c + 1 < nchunks; c += 2) {
-        chunk(Even{}, c, cur, nxt, nx2);
-        rotate();
-        chunk(Odd{}, c + 1, cur, nxt, nx2);
-        rotate();
+    if (NPH == 2) {
+        for (; c + 1 < nchunks; c += 2) {
+            chunk(P0{}, c, cur, nxt, nx2);
+            rotate();
+            chunk(P1{}, c + 1, cur, nxt, nx2);
+            rotate();
+        }
+        if (c < nchunks) chunk(P0{}, c, cur, nxt, nx2);
+    } else {
+        for (; c + 3 < nchunks; c += 4) {
+            chunk(P0{}, c, cur, nxt, nx2);
+            rotate();
+            chunk(P1{}, c + 1, cur, nxt, nx2);
+            rotate();
+            chunk(P2{}, c + 2, cur, nxt, nx2);
+            rotate();
+            chunk(P3{}, c + 3, cur, nxt, nx2);
+            rotate();
+        }
+        if (c < nchunks) {
+            chunk(P0{}, c, cur, nxt, nx2);
+            rotate();
+            if (c + 1 < nchunks) {
+                chunk(P1{}, c + 1, cur, nxt, nx2);
+                rotate();
+                if (c + 2 < nchunks) chunk(P2{}, c + 2, cur, nxt, nx2);
+            }
+        }
     }
-    if (c < nchunks) chunk(Even{}, c, cur, nxt, nx2);
+    if (LATE_PARAMS) load_params();
     // the MFMAs above are opaque to the compiler's hazard tracking: let the last ones retire
     asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 
     // ---- epilogue: lane holds acc[mi][ni][r] = C[m = mi*16 + l16][n = ni*16 + 4*kb + r].  The
     // 128 x 64 fp16 tile of the wavefront goes through LDS so that global stores are whole
     // 128-byte lines.
-    constexpr uint32_t kYStride = 144;
     uint8_t *stage = lds + wave * (BM * kYStride);
 #pragma unroll
     for (int ni = 0; ni < TNI; ++ni) {
@@ -397,12 +447,17 @@ static void launch_tile(const Bf6Params &p, hipStream_t stream)
 template <int EPI>
 static void launch_mode(Bf6Params &p, hipStream_t stream)
 {
-    // Tile height: whole rounds of 256 workgroups, a 64-row tile priced at kCost64 of a 128-row one (it does half
-    // the MFMAs for the same weight traffic; measured on an MI355X).
-    constexpr float kCost64 = 0.68f;
-    const uint32_t t128 = ((p.M + 127) / 128) * p.tiles_n, t64 = ((p.M + 63) / 64) * p.tiles_n;
-    const float c128 = (float)((t128 + 255) / 256), c64 = kCost64 * (float)((t64 + 255) / 256);
-    if (c64 < c128) {
+    // Tile height: whole rounds of 256 workgroups, with a 64-row / 256-row tile priced relative to a 128-row one
+    // (the weight traffic per tile is the same, the MFMAs are half / twice; measured on an MI355X).
+    constexpr float kCost64 = 0.68f, kCost256 = DUQ_BF6_COST256;
+    const uint32_t t256 = ((p.M + 255) / 256) * p.tiles_n, t128 = ((p.M + 127) / 128) * p.tiles_n,
+                   t64 = ((p.M + 63) / 64) * p.tiles_n;
+    const float c256 = kCost256 * (float)((t256 + 255) / 256), c128 = (float)((t128 + 255) / 256),
+                c64 = kCost64 * (float)((t64 + 255) / 256);
+    if (c256 < c128 && c256 <= c64) {
+        p.tiles_m = (p.M + 255) / 256;
+        launch_tile<16, EPI>(p, stream);
+    } else if (c64 < c128) {
         p.tiles_m = (p.M + 63) / 64;
         launch_tile<4, EPI>(p, stream);
     } else {

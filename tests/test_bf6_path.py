@@ -198,7 +198,9 @@ def _epi_inputs(rng, M, N):
 @pytest.mark.parametrize("M,N,K", [(1, 16, 128), (128, 256, 128), (128, 256, 256), (100, 240, 640), (257, 512, 1024),
                                    (130, 80, 384), (300, 1008, 1152), (512, 4096, 4096), (64, 1024, 11008),
                                    # enough tiles for the 128-row variant of the kernel (the ones above run 64-row tiles)
-                                   (2048 + 70, 4096 - 48, 384), (2048, 4096, 128)])
+                                   (2048 + 70, 4096 - 48, 384), (2048, 4096, 128),
+                                   # ... and for the 256-row variant: one to seven steps (its loop turns every four), ragged edges
+                                   (4096, 4096, 128), (4096 - 37, 4096 - 48, 384), (4096, 4096, 512), (4096, 4096 - 16, 896)])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_gpu_forward_bf6_equals_oracle(hip, dev, M, N, K, with_bias):
     """One and several chunks, odd and even numbers of 128-k steps, ragged M, N that ends inside a
@@ -263,7 +265,8 @@ def test_gpu_forward_bf6_extreme_accumulation(hip, dev):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("M,N,K", [(2048, 4096, 4096), (2048, 11008, 4096), (1000, 4096, 11008)])
+@pytest.mark.parametrize("M,N,K", [(2048, 4096, 4096), (2048, 11008, 4096), (1000, 4096, 11008), (4096, 4096, 4096),
+                                   (8192, 4096, 640)])
 def test_gpu_forward_bf6_full_size_equals_integer_kernels(hip, dev, M, N, K):
     """At the benchmark sizes the oracle is too slow: the integer kernels (pinned to the oracle at
     small sizes) are the comparison, on quantizer output, for the whole step."""
