@@ -299,7 +299,7 @@ def main():
                             args.steps, args.warmup)
     quant_us = event_time_us(lambda: hip.quantize_rows_sym_bf6(x, with_q=False), args.steps, args.warmup)
     achieved = ops / gemm_us / 1e6
-    roofline = {"bound": "mfma", "kernel": "gemm_bf6_kernel<0,false> (fused GEMM + dequant on v_mfma_f32_16x16x128_f8f6f4)",
+    roofline = {"bound": "mfma", "kernel": "gemm_bf6_kernel<8,0,false> (fused GEMM + dequant on v_mfma_f32_16x16x128_f8f6f4, 128 x 256 tiles)",
                 "achieved": round(achieved, 1), "peak": PEAK_FP6_TOPS, "unit": "TOP/s",
                 "frac": round(achieved / PEAK_FP6_TOPS, 4), "avg_kernel_us": round(gemm_us, 2),
                 "peak_note": "published dense fp6 peak; the same achieved rate is %.3f of the int8 peak (5.0 POP/s) the "
