@@ -22,7 +22,9 @@ int check_gemm(const void *A, const void *B, uint32_t M, uint32_t N, uint32_t K)
     if (M == 0 || N == 0) return DUQ_OK;
     if (!A || !B) return DUQ_E_NULL;
     if (K % 64 != 0) return DUQ_E_KALIGN;
-    if (K > 131008u) return DUQ_E_TOO_LARGE;
+    // K: accumulators are carried x256 in int32 (or as float32 integers below 2^24); M, N: the kernels index one
+    // output tile's rows with 32-bit byte offsets (256 rows x N x 4 bytes)
+    if (K > 131008u || N > (1u << 22) || M > (1u << 24)) return DUQ_E_TOO_LARGE;
     if (!aligned(A, 16) || !aligned(B, 16)) return DUQ_E_ALIGN;
     return DUQ_OK;
 }
@@ -276,7 +278,7 @@ int duq_linear4bit_forward_bf6(int32_t mode, const uint8_t *x_bf6, const duq_hal
     if (!x_bf6 || !w_bf6 || !scale_x || !w_scale_1 || !y) return DUQ_E_NULL;
     if (K == 0 || K % 128 != 0) return DUQ_E_KALIGN;
     if (N % 16 != 0) return DUQ_E_SHAPE;
-    if (K > 131008u) return DUQ_E_TOO_LARGE;
+    if (K > 131008u || N > (1u << 22) || M > (1u << 24)) return DUQ_E_TOO_LARGE;
     const bool asym = mode == DUQ_EPI_ASYM || mode == DUQ_EPI_ASYM_DUAL || mode == DUQ_EPI_ASYM_ROWSUM;
     const bool dual = mode == DUQ_EPI_SYM_DUAL || mode == DUQ_EPI_ASYM_DUAL;
     if (asym && (!zeros_x || !w_zeros_1)) return DUQ_E_NULL;

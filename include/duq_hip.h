@@ -40,7 +40,7 @@ typedef void *duq_stream_t;  /* hipStream_t */
 #define DUQ_E_KALIGN (-3)    /* GEMM K is not a multiple of 64 (qlinear4bit/tools/tensor_utils.py:52) */
 #define DUQ_E_MODE (-4)      /* unknown epilogue mode / unsupported qmax */
 #define DUQ_E_ALIGN (-5)     /* a pointer misses the alignment the entry point documents */
-#define DUQ_E_TOO_LARGE (-6) /* a dimension exceeds what the kernels index with 32 bits */
+#define DUQ_E_TOO_LARGE (-6) /* a dimension exceeds what the kernels index with 32 bits: K > 131008, N > 2^22, M > 2^24 */
 
 /* symmetric clamp used by the device quantizer of the reference: qmax_sym evaluates to 6
  * (include/common.h:53-54).  7 is the bound of the Python fake-quant path

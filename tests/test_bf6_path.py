@@ -131,6 +131,8 @@ def test_abi_validation_bf6_entries():
     assert fwd(4, P, P, P, None, P, P, P, None, None, None, None, 4, 32, 128, P, None) == -1          # row sums missing
     assert fwd(0, P, P, None, None, P, P + 2, None, None, None, None, None, 4, 32, 128, P, None) == -5
     assert fwd(0, None, None, None, None, None, None, None, None, None, None, None, 0, 32, 128, None, None) == 0
+    assert fwd(0, P, P, None, None, P, P, None, None, None, None, None, 4, (1 << 22) + 16, 128, P, None) == -6
+    assert lib.duq_matmul_host_4bit(P, P, 4, (1 << 22) + 1, 64, P, None) == -6
 
 
 # ------------------------------------------------------------------ GPU parity
