@@ -178,6 +178,13 @@ def asym_section(dev):
         y = mod(x).float()
         out[name] = {"step_us": round(us, 2), "TOPS": round(2.0 * M * N * K / us / 1e6, 1),
                      "rel_error_vs_fp32_matmul": round(float((y.detach() - true).norm() / true.norm()), 4)}
+        # the same layer on the 6-bit float matrix path (64-row tiles at this size): same bits
+        y_int = mod(x)
+        mod.enable_fp6()
+        same = bool(torch.equal(mod(x).view(torch.int16), y_int.view(torch.int16)))
+        us6 = graph_time_us([lambda: mod(x)] * 20)
+        out[name].update({"fp6_step_us": round(us6, 2), "fp6_TOPS": round(2.0 * M * N * K / us6 / 1e6, 1),
+                          "fp6_same_bits": same})
     return out
 
 
