@@ -171,7 +171,7 @@ def asym_section(dev):
         lin.weight.copy_((torch.randn(N, K, generator=g) * 0.02).half())
     ref_mode = Linear4bitASQ.from_linear(lin).to(dev)
     rowsum_mode = Linear4bitASQRowSum.from_linear(lin.to(dev))
-    true = x.float() @ lin.weight.float().t()
+    true = x.float() @ lin.weight.detach().float().t()
     out = {"M": M, "N": N, "K": K}
     for name, mod in (("reference_mode", ref_mode), ("rowsum_mode", rowsum_mode)):
         us = graph_time_us([lambda: mod(x)] * 20)
@@ -185,6 +185,35 @@ def asym_section(dev):
         us6 = graph_time_us([lambda: mod(x)] * 20)
         out[name].update({"fp6_step_us": round(us6, 2), "fp6_TOPS": round(2.0 * M * N * K / us6 / 1e6, 1),
                           "fp6_same_bits": same})
+    return out
+
+
+def other_shapes_section(dev):
+    """The other prefill shapes of the Llama-2-7B configuration and the Llama-2-70B MLP shapes at M = 4096 (a full
+    layer on one GPU): one module step (quantize + GEMM + dequant) on either matrix path, HIP-graph timed."""
+    import torch
+
+    from duqlinear4bitcuda_amd.nn import Linear4bitSQ, SymQuantizer
+
+    out = []
+    for (M, K, N) in [(2048, 4096, 11008), (2048, 11008, 4096), (4096, 8192, 28672), (4096, 28672, 8192)]:
+        x = heavy_tail_acts(M, K, seed=5).to(dev)
+        w, sw = random_weights(N, K, seed=55, dev=dev)
+        lin = Linear4bitSQ(K, N, bias=False).to(dev)
+        lin.weight.copy_(w)
+        lin.weight_scales = sw
+        q_i8 = SymQuantizer(1.0)
+        q_f6 = SymQuantizer(1.0, shadow="only", shadow_min_rows=1)
+        reps = 6 if M * N * K < 2e11 else 3
+        us_i8 = graph_time_us([lambda: lin(q_i8(x))] * reps)
+        y_i8 = lin(q_i8(x))
+        lin.enable_fp6()
+        same = bool(torch.equal(lin(q_f6(x)).view(torch.int16), y_i8.view(torch.int16)))
+        us_f6 = graph_time_us([lambda: lin(q_f6(x))] * reps)
+        ops = 2.0 * M * N * K
+        out.append({"M": M, "K": K, "N": N, "integer_step_us": round(us_i8, 1), "integer_TOPS": round(ops / us_i8 / 1e6, 1),
+                    "fp6_step_us": round(us_f6, 1), "fp6_TOPS": round(ops / us_f6 / 1e6, 1), "same_bits": same})
+        del lin, w, x
     return out
 
 
@@ -308,7 +337,8 @@ def main():
     achieved = ops / gemm_us / 1e6
     roofline = {"bound": "mfma", "kernel": "gemm_bf6_kernel<8,0,false> (fused GEMM + dequant on v_mfma_f32_16x16x128_f8f6f4, 128 x 256 tiles)",
                 "achieved": round(achieved, 1), "peak": PEAK_FP6_TOPS, "unit": "TOP/s",
-                "frac": round(achieved / PEAK_FP6_TOPS, 4), "avg_kernel_us": round(gemm_us, 2),
+                "frac": round(achieved / PEAK_FP6_TOPS, 4), "frac_of_int8_peak": round(achieved / PEAK_INT8_TOPS, 4),
+                "avg_kernel_us": round(gemm_us, 2),
                 "peak_note": "published dense fp6 peak; the same achieved rate is %.3f of the int8 peak (5.0 POP/s) the "
                              "integer kernel is priced against" % (achieved / PEAK_INT8_TOPS),
                 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this workload, each
@@ -329,6 +359,7 @@ def main():
     decode = decode_section(dev, args.quick)
     quantizer = quantizer_section(dev)
     asym = None if args.quick else asym_section(dev)
+    other = None if args.quick else other_shapes_section(dev)
     best_decode = max(decode, key=lambda d: d["GBps"])
     roofline_decode = {"bound": "hbm", "kernel": "gemv_s4_dot_kernel (M=1) / gemm_s4_skinny_kernel (2<=M<=16) / gemm_s4_ring_kernel (17<=M<=64, long rows)", "achieved": best_decode["GBps"],
                        "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": best_decode["frac_hbm"],
@@ -366,6 +397,7 @@ def main():
         "decode": decode,
         "quantizer": quantizer,
         "asym": asym,
+        "other_shapes": other,
         "cpu_baseline": cpu,
         "device": {"name": props.name, "arch": props.gcnArchName, "cus": props.multi_processor_count},
     }
