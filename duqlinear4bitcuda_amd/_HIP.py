@@ -574,3 +574,106 @@ def quantize_rows_asym_bf6(x: torch.Tensor, shifted: bool = False, with_q: bool 
     if st:
         _lib.check(st, name)
     return (q, b, s, z, r) if shifted else (q, b, s, z)
+
+
+# ---- 8-bit asymmetric layer (LinearQuant8bitASQ) --------------------------------------------
+
+_F32, _I8 = torch.float32, torch.int8
+
+
+def matmul_8bit(A: torch.Tensor, B: torch.Tensor) -> torch.Tensor:
+    """A [M, K] int8 @ B [N, K]^T int8 -> int32 [M, N] (bindings.cpp:28-45)."""
+    _check("matmul_8bit", A, B)
+    _check_dtype("matmul_8bit", A, "A", _I8)
+    _check_dtype("matmul_8bit", B, "B", _I8)
+    M, N, K = A.size(0), B.size(0), A.size(1)
+    if B.size(1) != K:
+        raise RuntimeError(f"matmul_8bit: K differs: A {tuple(A.shape)} vs B {tuple(B.shape)}")
+    C = torch.empty((M, N), dtype=torch.int32, device=A.device)
+    st = _launch(A.device, _lib.load().duq_matmul_host_8bit, _ptr(A), _ptr(B), M, N, K, _ptr(C))
+    _lib.check(st, "matmul_8bit")
+    return C
+
+
+def asym_quant_8bit(x, scale, zeros):
+    """float32 x [rows, cols], per-row float32 scale / zero -> int8 codes 0..126 (bindings.cpp:245-266)."""
+    _check("asym_quant_8bit", x, scale, zeros)
+    for t, n in ((x, "x"), (scale, "scale"), (zeros, "zeros")):
+        _check_dtype("asym_quant_8bit", t, n, _F32)
+    _check_size0("asym_quant_8bit", scale, "scale", x.size(0))
+    _check_size0("asym_quant_8bit", zeros, "zeros", x.size(0))
+    rows, cols = x.size(0), x.size(1)
+    q = torch.empty((rows, cols), dtype=_I8, device=x.device)
+    st = _launch(x.device, _lib.load().duq_asym_quant_host_8bit, _ptr(x), _ptr(scale), _ptr(zeros), rows, cols, _ptr(q))
+    _lib.check(st, "asym_quant_8bit")
+    return q
+
+
+def asym_dequant_hprec(q, scale_row, zeros_row, scale_col, zeros_col, bits: int = 32):
+    """(s_r * s_c) * (float(q) - (z_r + z_c)) in float32 (bindings.cpp:309-350)."""
+    _check("asym_dequant_hprec", q, scale_row, zeros_row, scale_col, zeros_col)
+    _check_bits("asym_dequant_hprec", bits)
+    _check_dtype("asym_dequant_hprec", q, "q", torch.int32)
+    for t, n in ((scale_row, "scale_row"), (zeros_row, "zeros_row"), (scale_col, "scale_col"), (zeros_col, "zeros_col")):
+        _check_dtype("asym_dequant_hprec", t, n, _F32)
+    rows, cols = q.size(0), q.size(1)
+    _check_size0("asym_dequant_hprec", scale_row, "scale_row", rows)
+    _check_size0("asym_dequant_hprec", zeros_row, "zeros_row", rows)
+    _check_size0("asym_dequant_hprec", scale_col, "scale_col", cols)
+    _check_size0("asym_dequant_hprec", zeros_col, "zeros_col", cols)
+    x = torch.empty((rows, cols), dtype=_F32, device=q.device)
+    st = _launch(q.device, _lib.load().duq_asym_dequant_host_hprec, _ptr(q), _ptr(scale_row), _ptr(zeros_row),
+                 _ptr(scale_col), _ptr(zeros_col), rows, cols, _ptr(x))
+    _lib.check(st, "asym_dequant_hprec")
+    return x
+
+
+def quantize_rows_asym_8bit(x: torch.Tensor):
+    """One-pass AsymQuantizer8bit (qlinear4bit/nn/quantizer.py:38-55) over the last dimension:
+    (q int8 [..., K], scale [..., 1], zeros [..., 1]) float32.  Requires K % 4 == 0."""
+    if not isinstance(x, torch.Tensor):
+        raise RuntimeError("quantize_rows_asym_8bit: argument #0 is not a tensor")
+    _fast_check("quantize_rows_asym_8bit", "x", x, _F32, None)
+    shape = x.shape
+    cols = shape[-1]
+    rows = x.numel() // cols if cols else 0
+    lead = shape[:-1]
+    dev = x.device
+    q = torch.empty(shape, dtype=_I8, device=dev)
+    s = torch.empty(lead + (1,), dtype=_F32, device=dev)
+    z = torch.empty(lead + (1,), dtype=_F32, device=dev)
+    st = _launch(dev, _lib.load().duq_quantize_rows_asym_8bit, x.data_ptr(), rows, cols, q.data_ptr(), s.data_ptr(),
+                 z.data_ptr())
+    if st:
+        _lib.check(st, "quantize_rows_asym_8bit")
+    return q, s, z
+
+
+def linear8bit_forward(xq, scale_x, zeros_x, w, w_scale, w_zeros, bias=None):
+    """matmul_8bit + asym_dequant_hprec (+ bias) in one launch; xq [..., K] int8 -> float32 [..., N]."""
+    name = "linear8bit_forward"
+    if not isinstance(xq, torch.Tensor):
+        raise RuntimeError(f"{name}: argument #0 is not a tensor")
+    dev = xq.device
+    _fast_check(name, "xq", xq, _I8, None)
+    _fast_check(name, "w", w, _I8, dev)
+    K = xq.shape[-1]
+    M = xq.numel() // K if K else 0
+    N = w.size(0)
+    if w.dim() != 2 or w.size(1) != K:
+        raise RuntimeError(f"{name}: K differs: xq {tuple(xq.shape)} vs w {tuple(w.shape)}")
+    for t, what, n in ((scale_x, "scale_x", M), (zeros_x, "zeros_x", M), (w_scale, "w_scale", N),
+                       (w_zeros, "w_zeros", N), (bias, "bias", N)):
+        if t is None and what == "bias":
+            continue
+        if not isinstance(t, torch.Tensor):
+            raise RuntimeError(f"{name}: {what} is not a tensor")
+        _fast_check(name, what, t, _F32, dev)
+        if t.numel() != n:
+            raise RuntimeError(f"{name}: expected {what} to have {n} elements, got {tuple(t.shape)}")
+    y = torch.empty(xq.shape[:-1] + (N,), dtype=_F32, device=dev)
+    st = _launch(dev, _lib.load().duq_linear8bit_forward, xq.data_ptr(), scale_x.data_ptr(), zeros_x.data_ptr(),
+                 w.data_ptr(), w_scale.data_ptr(), w_zeros.data_ptr(), _ptr(bias), M, N, K, y.data_ptr())
+    if st:
+        _lib.check(st, name)
+    return y

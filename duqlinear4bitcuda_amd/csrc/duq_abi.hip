@@ -41,7 +41,7 @@ const char *duq_status_string(int status)
     case DUQ_OK: return "ok";
     case DUQ_E_NULL: return "a required pointer is NULL";
     case DUQ_E_SHAPE: return "inconsistent dimensions";
-    case DUQ_E_KALIGN: return "K must be a multiple of 64 (packed row length a multiple of 32 bytes)";
+    case DUQ_E_KALIGN: return "K must be a multiple of 64 (packed row length a multiple of 32 bytes); 128 on the 6-bit float path, 32 on the 8-bit one";
     case DUQ_E_MODE: return "unknown epilogue mode or unsupported qmax";
     case DUQ_E_ALIGN: return "pointer alignment requirement not met";
     case DUQ_E_TOO_LARGE: return "dimension too large";
@@ -292,6 +292,68 @@ int duq_linear4bit_forward_bf6(int32_t mode, const uint8_t *x_bf6, const duq_hal
         return DUQ_E_ALIGN;
     duq::Epilogue e{mode, scale_x, zeros_x, w_scale_1, w_zeros_1, w_scale_2, w_zeros_2, bias, rowsum_x, w_rowsum_adj};
     return duq::launch_gemm_bf6(x_bf6, w_bf6, M, N, K, e, y, as_stream(stream));
+}
+
+// ---- 8-bit asymmetric layer ----------------------------------------------------------------
+
+static int check_gemm8(const void *A, const void *B, uint32_t M, uint32_t N, uint32_t K)
+{
+    if (M == 0 || N == 0) return DUQ_OK;
+    if (!A || !B) return DUQ_E_NULL;
+    if (K == 0 || K % 32 != 0) return DUQ_E_KALIGN;
+    // one tile's rows are indexed with 32-bit byte offsets: 256 rows x K bytes, 128 rows x N x 4 bytes
+    if (K > (1u << 23) || N > (1u << 22) || M > (1u << 24)) return DUQ_E_TOO_LARGE;
+    if (!aligned(A, 16) || !aligned(B, 16)) return DUQ_E_ALIGN;
+    return DUQ_OK;
+}
+
+int duq_asym_quant_host_8bit(const float *x, const float *scale, const float *zeros, uint32_t rows, uint32_t cols,
+                             int8_t *q, duq_stream_t stream)
+{
+    if (rows == 0 || cols == 0) return DUQ_OK;
+    if (!x || !scale || !zeros || !q) return DUQ_E_NULL;
+    return duq::launch_asym_quant8(x, scale, zeros, rows, cols, q, as_stream(stream));
+}
+
+int duq_quantize_rows_asym_8bit(const float *x, uint32_t rows, uint32_t cols, int8_t *q, float *scale, float *zeros,
+                                duq_stream_t stream)
+{
+    if (rows == 0 || cols == 0) return DUQ_OK;
+    if (!x || !q || !scale || !zeros) return DUQ_E_NULL;
+    if (cols % 4 != 0) return DUQ_E_SHAPE;
+    if (!aligned(x, 16) || !aligned(q, 4)) return DUQ_E_ALIGN;
+    return duq::launch_quantize_rows_asym8(x, rows, cols, q, scale, zeros, as_stream(stream));
+}
+
+int duq_matmul_host_8bit(const int8_t *A, const int8_t *B, uint32_t M, uint32_t N, uint32_t K, int32_t *C,
+                         duq_stream_t stream)
+{
+    if (int e = check_gemm8(A, B, M, N, K)) return e;
+    if (M == 0 || N == 0) return DUQ_OK;
+    if (!C) return DUQ_E_NULL;
+    if (!aligned(C, 4)) return DUQ_E_ALIGN;
+    return duq::launch_gemm_s8(A, B, M, N, K, C, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, as_stream(stream));
+}
+
+int duq_asym_dequant_host_hprec(const int32_t *q, const float *scale_row, const float *zeros_row,
+                                const float *scale_col, const float *zeros_col, uint32_t rows, uint32_t cols, float *x,
+                                duq_stream_t stream)
+{
+    if (rows == 0 || cols == 0) return DUQ_OK;
+    if (!q || !scale_row || !zeros_row || !scale_col || !zeros_col || !x) return DUQ_E_NULL;
+    return duq::launch_dequant_hprec(q, scale_row, zeros_row, scale_col, zeros_col, nullptr, rows, cols, x,
+                                     as_stream(stream));
+}
+
+int duq_linear8bit_forward(const int8_t *xq, const float *scale_x, const float *zeros_x, const int8_t *w,
+                           const float *w_scale, const float *w_zeros, const float *bias, uint32_t M, uint32_t N,
+                           uint32_t K, float *y, duq_stream_t stream)
+{
+    if (int e = check_gemm8(xq, w, M, N, K)) return e;
+    if (M == 0 || N == 0) return DUQ_OK;
+    if (!scale_x || !zeros_x || !w_scale || !w_zeros || !y) return DUQ_E_NULL;
+    if (!aligned(y, 4)) return DUQ_E_ALIGN;
+    return duq::launch_gemm_s8(xq, w, M, N, K, nullptr, scale_x, zeros_x, w_scale, w_zeros, bias, y, as_stream(stream));
 }
 
 }  // extern "C"

@@ -1,0 +1,450 @@
+// The 8-bit asymmetric layer of the reference (LinearQuant8bitASQ) for gfx950: per-token int8
+// quantizer (float32 in), int8 x int8 -> int32 GEMM on v_mfma_i32_32x32x32_i8, float32
+// dequant ("hprec") stand-alone or fused into the GEMM.
+//   quantize : src/kernels/quant.cu:241-279      scale/zero : qlinear4bit/nn/quantizer.py:38-55
+//   GEMM     : src/kernels/gemm.cu:46-81         dequant    : src/kernels/quant.cu:281-323
+// Arithmetic is float32 with one rounding per operator, as in the reference; the quantizer's
+// value goes through binary16 on its way to the integer (the reference passes a float to
+// __half2int_rn).
+#include "duq_device.h"
+#include "duq_launch.h"
+#include "duq_tiles.h"
+
+namespace duq {
+
+typedef float v4f32 __attribute__((ext_vector_type(4)));
+typedef int v16i32 __attribute__((ext_vector_type(16)));
+
+constexpr int kQmaxAsym8 = 126;  // src/kernels/quant.cu:242
+
+// clamp(rint(h(x / s)) + zi, 0, 126); the add wraps like the 32-bit add of the reference
+__device__ __forceinline__ uint32_t asym8_code(float x, float s, int zi)
+{
+    const f16 hq = (f16)(x / s);  // IEEE float32 quotient, then one rounding to binary16
+    const int qi = rint_i32((float)hq);
+    const int sum = (int)((uint32_t)qi + (uint32_t)zi);
+    return (uint32_t)clampi(sum, 0, kQmaxAsym8);
+}
+__device__ __forceinline__ int asym8_zero_int(float z) { return rint_i32((float)(f16)z); }
+
+// ---------------------------------------------------------------------------------
+// given-scale quantizer (asym_quant_host_8bit): 4 elements per lane step when the row
+// length allows, else one
+// ---------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void asym_quant8_kernel(const float *x, const float *scale, const float *zeros,
+                                                          uint32_t rows, uint32_t cols, int8_t *q, bool vec)
+{
+    if (vec) {
+        const uint32_t per_row = cols >> 2;
+        const uint64_t total = (uint64_t)rows * per_row;
+        for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (uint64_t)gridDim.x * blockDim.x) {
+            const uint32_t row = (uint32_t)(i / per_row);
+            const v4f32 v = __builtin_nontemporal_load(reinterpret_cast<const v4f32 *>(x) + i);
+            const float s = scale[row];
+            const int zi = asym8_zero_int(zeros[row]);
+            uint32_t w = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w |= asym8_code(v[e], s, zi) << (8 * e);
+            reinterpret_cast<uint32_t *>(q)[i] = w;
+        }
+    } else {
+        const uint64_t total = (uint64_t)rows * cols;
+        for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (uint64_t)gridDim.x * blockDim.x) {
+            const uint32_t row = (uint32_t)(i / cols);
+            q[i] = (int8_t)asym8_code(x[i], scale[row], asym8_zero_int(zeros[row]));
+        }
+    }
+}
+
+int launch_asym_quant8(const float *x, const float *scale, const float *zeros, uint32_t rows, uint32_t cols, int8_t *q,
+                       hipStream_t stream)
+{
+    if (rows == 0 || cols == 0) return 0;
+    const bool vec = cols % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(q) % 4 == 0;
+    const uint64_t total = (uint64_t)rows * (vec ? cols / 4 : cols);
+    const uint32_t blocks = (uint32_t)std::min<uint64_t>((total + 255) / 256, 1u << 20);
+    hipLaunchKernelGGL(asym_quant8_kernel, dim3(blocks), dim3(256), 0, stream, x, scale, zeros, rows, cols, q, vec);
+    return (int)hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------------
+// fused row quantizer (AsymQuantizer8bit.forward in one pass): one workgroup per row, the row
+// held in registers between the min / max reduction and the quantization (up to 8 x 4
+// elements per lane; longer rows are read a second time, from L2)
+// ---------------------------------------------------------------------------------
+constexpr int kMaxVec8 = 8;
+
+template <int WAVES, bool CACHED>
+__global__ __launch_bounds__(WAVES * 64) void quantize_rows_asym8_kernel(const float *x, uint32_t rows, uint32_t cols,
+                                                                         int8_t *q, float *scale, float *zeros)
+{
+    constexpr int T = WAVES * 64;
+    __shared__ float red[2][WAVES];
+    const uint32_t row = blockIdx.x, tid = threadIdx.x;
+    const uint32_t nvec = cols >> 2;
+    const v4f32 *xrow = reinterpret_cast<const v4f32 *>(x + (uint64_t)row * cols);
+    uint32_t *qrow = reinterpret_cast<uint32_t *>(q + (uint64_t)row * cols);
+    v4f32 regs[kMaxVec8];
+    float lo = INFINITY, hi = -INFINITY;
+    bool nan_seen = false;
+    auto reduce = [&](const v4f32 &g) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            lo = fminf(lo, g[e]);
+            hi = fmaxf(hi, g[e]);
+            nan_seen |= g[e] != g[e];
+        }
+    };
+    if (CACHED) {
+#pragma unroll
+        for (int i = 0; i < kMaxVec8; ++i) {
+            const uint32_t u = tid + i * T;
+            regs[i] = u < nvec ? __builtin_nontemporal_load(&xrow[u]) : v4f32{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int i = 0; i < kMaxVec8; ++i)
+            if (tid + i * T < nvec) reduce(regs[i]);
+    } else {
+        for (uint32_t u = tid; u < nvec; u += T) reduce(xrow[u]);
+    }
+    lo = wave_min_f32(lo);
+    hi = wave_max_f32(hi);
+    nan_seen = __builtin_amdgcn_ballot_w64(nan_seen) != 0;
+    if (WAVES > 1) {
+        if ((tid & 63u) == 0) {
+            red[0][tid >> 6] = nan_seen ? __builtin_nanf("") : lo;
+            red[1][tid >> 6] = hi;
+        }
+        __syncthreads();
+        lo = red[0][0];
+        hi = red[1][0];
+        nan_seen = lo != lo;
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) {
+            nan_seen |= red[0][w] != red[0][w];
+            lo = fminf(lo, red[0][w]);
+            hi = fmaxf(hi, red[1][w]);
+        }
+    }
+    if (nan_seen) lo = hi = __builtin_nanf("");  // torch's min / max return NaN for a row that holds one
+    // scale = (max - min) / 127, zeros = round(-min / scale)  (quantizer.py:50-51), float32.  torch evaluates
+    // tensor / scalar on a GPU as tensor * float32(1 / scalar), which is what the reference's scale is
+    const float d = hi - lo;
+    const float s = d * (1.0f / 127.0f);
+    const float z = __builtin_rintf((-lo) / s);
+    if (tid == 0) {
+        scale[row] = s;
+        zeros[row] = z;
+    }
+    const int zi = asym8_zero_int(z);
+    auto quant4 = [&](const v4f32 &g) -> uint32_t {
+        uint32_t w = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) w |= asym8_code(g[e], s, zi) << (8 * e);
+        return w;
+    };
+    if (CACHED) {
+#pragma unroll
+        for (int i = 0; i < kMaxVec8; ++i) {
+            const uint32_t u = tid + i * T;
+            if (u < nvec) qrow[u] = quant4(regs[i]);
+        }
+    } else {
+        for (uint32_t u = tid; u < nvec; u += T) qrow[u] = quant4(xrow[u]);
+    }
+}
+
+int launch_quantize_rows_asym8(const float *x, uint32_t rows, uint32_t cols, int8_t *q, float *scale, float *zeros,
+                               hipStream_t stream)
+{
+    if (rows == 0 || cols == 0) return 0;
+    const uint32_t nvec = cols / 4;
+    uint32_t waves = 1;
+    while (waves < 16 && waves * 64 * 4 < nvec) waves *= 2;  // four 128-bit loads per lane when the row allows
+    const bool cached = waves * 64 * kMaxVec8 >= nvec;
+    const dim3 grid(rows);
+#define DUQ_ROWS8(W)                                                                                              \
+    case W:                                                                                                       \
+        if (cached)                                                                                               \
+            hipLaunchKernelGGL((quantize_rows_asym8_kernel<W, true>), grid, dim3(W * 64), 0, stream, x, rows, cols, q, scale, zeros); \
+        else                                                                                                      \
+            hipLaunchKernelGGL((quantize_rows_asym8_kernel<W, false>), grid, dim3(W * 64), 0, stream, x, rows, cols, q, scale, zeros); \
+        break;
+    switch (waves) {
+        DUQ_ROWS8(1)
+        DUQ_ROWS8(2)
+        DUQ_ROWS8(4)
+        DUQ_ROWS8(8)
+        DUQ_ROWS8(16)
+    }
+#undef DUQ_ROWS8
+    return (int)hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------------
+// float32 dequant: x = (s_r * s_c) * (float(acc) - (z_r + z_c)) [+ bias]
+// ---------------------------------------------------------------------------------
+struct Epi8 {
+    const float *s_row, *z_row, *s_col, *z_col, *bias;
+};
+
+__device__ __forceinline__ float dequant_hprec_one(int acc, float sr, float zr, float sc, float zc)
+{
+    const float scales = sr * sc;
+    const float zeros = zr + zc;
+    const float t = (float)acc - zeros;
+    return scales * t;  // built with -ffp-contract=off: no fused multiply-add
+}
+
+__global__ __launch_bounds__(256) void dequant_hprec_kernel(const int32_t *acc, Epi8 e, uint32_t rows, uint32_t cols, float *x)
+{
+    const uint64_t total = (uint64_t)rows * cols;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (uint64_t)gridDim.x * blockDim.x) {
+        const uint32_t row = (uint32_t)(i / cols), col = (uint32_t)(i % cols);
+        float v = dequant_hprec_one(acc[i], e.s_row[row], e.z_row[row], e.s_col[col], e.z_col[col]);
+        if (e.bias) v = v + e.bias[col];
+        x[i] = v;
+    }
+}
+
+int launch_dequant_hprec(const int32_t *acc, const float *s_row, const float *z_row, const float *s_col,
+                         const float *z_col, const float *bias, uint32_t rows, uint32_t cols, float *x, hipStream_t stream)
+{
+    if (rows == 0 || cols == 0) return 0;
+    const uint64_t total = (uint64_t)rows * cols;
+    const uint32_t blocks = (uint32_t)std::min<uint64_t>((total + 255) / 256, 1u << 20);
+    hipLaunchKernelGGL(dequant_hprec_kernel, dim3(blocks), dim3(256), 0, stream, acc, Epi8{s_row, z_row, s_col, z_col, bias},
+                       rows, cols, x);
+    return (int)hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------------
+// GEMM  C[m,n] = sum_k A[m,k] * B[n,k]   (int8, int32 accumulation)
+// ---------------------------------------------------------------------------------
+// Tile 32*TM (M) x 256 (N), 4 wavefronts side by side along N (32*TM x 64 each, TM x 2 MFMA tiles of 32 x 32),
+// 128-k chunks.  Weights go global -> registers: lane (r = lane % 32, h = lane / 32) of a 32-row tile holds bytes
+// [h*64 + s*16, +16) of row r for step s of the chunk (four 128-bit loads of 64 contiguous bytes per lane; integer
+// accumulation is order-free, the activations use the same k order).  Activations go global -> registers -> LDS
+// (three buffers, rows padded to 144 bytes, one barrier per chunk) -> fragments read one step ahead.  The weight
+// operand is the MFMA "A" side, so a lane holds four consecutive output columns of one row.
+struct Gemm8Params {
+    const int8_t *A;  // [M, K]
+    const int8_t *B;  // [N, K]
+    uint32_t M, N, K;
+    int32_t *C;       // int32 out (not fused)
+    float *y;         // float32 out (fused)
+    Epi8 epi;
+    uint32_t tiles_m, tiles_n;
+};
+
+__device__ __forceinline__ void lds_barrier8() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+template <int TM, bool FUSED, bool BIAS>
+__global__ __launch_bounds__(256) void gemm_s8_kernel(Gemm8Params p)
+{
+    static_assert(TM == 4 || TM == 1, "32-row MFMA tiles per wavefront along M");
+    constexpr int BM = 32 * TM, BN = 256, TN = 2;
+    constexpr uint32_t kStride = 144;
+    constexpr uint32_t kBuf = BM * kStride;
+    constexpr int NXP = BM * 8 / 256;  // 16-byte activation pieces per thread and chunk
+
+    __shared__ __attribute__((aligned(16))) uint8_t lds[3 * kBuf];
+
+    uint32_t tile_m, tile_n;
+    tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+    const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u, wave = tid >> 6;
+    const uint32_t l32 = lane & 31u, h = lane >> 5;
+    const uint32_t nchunks = (p.K + 127) / 128;
+
+    const __amdgpu_buffer_rsrc_t rW = make_rsrc(p.B + (uint64_t)n0 * p.K, min(p.N - n0, (uint32_t)BN) * p.K);
+    const __amdgpu_buffer_rsrc_t rX = make_rsrc(p.A + (uint64_t)m0 * p.K, min(p.M - m0, (uint32_t)BM) * p.K);
+
+    // K % 32 == 0, so a 16-byte piece is all inside a row or all past its end; pieces past K (last chunk) and
+    // chunks past the last are redirected out of range and read as zero
+    auto load_w = [&](int t, int s, uint32_t c) -> v4i {
+        const uint32_t k = c * 128 + h * 64 + s * 16;
+        const uint32_t off = (wave * 64 + t * 32 + l32) * p.K + k;
+        return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rW, (int)(k < p.K ? off : kOobOffset), 0, 0));
+    };
+    uint32_t xrow[NXP], xlds[NXP];
+    const uint32_t xpiece = tid & 7u;
+#pragma unroll
+    for (int j = 0; j < NXP; ++j) {
+        xrow[j] = (tid >> 3) + j * 32;
+        xlds[j] = xrow[j] * kStride + xpiece * 16;
+    }
+    auto load_x = [&](int j, uint32_t c) -> v4u {
+        const uint32_t k = c * 128 + xpiece * 16;
+        return buf_load16(rX, k < p.K ? xrow[j] * p.K + k : kOobOffset, 0);
+    };
+    // fragment of rows b*32 + l32, step s: bytes [h*64 + s*16, +16) of the row's chunk
+    const uint32_t frag = l32 * kStride + h * 64;
+    auto read_x = [&](uint32_t buf, int b, int s) -> v4i {
+        return *reinterpret_cast<const v4i *>(lds + buf + frag + b * 32 * kStride + s * 16);
+    };
+
+    v4i wreg[2][TN][4];  // [chunk parity][column tile][step]
+    v4u xreg[NXP];
+    v4i fx[2][TM];
+    v16i32 acc[TN][TM];
+#pragma unroll
+    for (int t = 0; t < TN; ++t)
+#pragma unroll
+        for (int b = 0; b < TM; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[t][b][r] = 0;
+
+    // ---- prologue: activations of chunks 0 and 1 -> LDS, chunk 2 -> registers; weights of chunk 0
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+#pragma unroll
+        for (int j = 0; j < NXP; ++j) xreg[j] = load_x(j, q);
+#pragma unroll
+        for (int j = 0; j < NXP; ++j) *reinterpret_cast<v4u *>(lds + q * kBuf + xlds[j]) = xreg[j];
+    }
+#pragma unroll
+    for (int t = 0; t < TN; ++t)
+#pragma unroll
+        for (int s = 0; s < 4; ++s) wreg[0][t][s] = load_w(t, s, 0);
+#pragma unroll
+    for (int j = 0; j < NXP; ++j) xreg[j] = load_x(j, 2);
+    lds_barrier8();
+#pragma unroll
+    for (int b = 0; b < TM; ++b) fx[0][b] = read_x(0, b, 0);
+
+    auto chunk = [&](auto par, uint32_t c, uint32_t cur, uint32_t nxt, uint32_t nx2) {
+        constexpr int PAR = decltype(par)::value;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+#pragma unroll
+            for (int b = 0; b < TM; ++b) {
+#pragma unroll
+                for (int t = 0; t < TN; ++t) {
+                    asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0"
+                                 : "+a"(acc[t][b])
+                                 : "v"(wreg[PAR][t][s]), "v"(fx[s & 1][b]));
+                    __builtin_amdgcn_sched_barrier(0);
+                    // ---- side work in the shadow of this MFMA
+                    if (t == 0)  // next step's fragment of this row tile (the next chunk's first step comes from `nxt`)
+                        fx[(s + 1) & 1][b] = s < 3 ? read_x(cur, b, s + 1) : read_x(nxt, b, 0);
+                    if (t == 1 && b == 0) {  // weights of the next chunk: this step's two pieces
+                        wreg[PAR ^ 1][0][s] = load_w(0, s, c + 1);
+                        wreg[PAR ^ 1][1][s] = load_w(1, s, c + 1);
+                    }
+                    if (t == 1 && s == 3 && b < NXP) {  // chunk c+2 -> its LDS buffer, then fetch chunk c+3
+                        *reinterpret_cast<v4u *>(lds + nx2 + xlds[b]) = xreg[b];
+                        xreg[b] = load_x(b, c + 3);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+        // the MFMAs are opaque to the compiler's hazard tracking: accumulator copies at a join must find them retired
+        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+        lds_barrier8();
+    };
+
+    uint32_t cur = 0, nxt = kBuf, nx2 = 2 * kBuf;
+    auto rotate = [&]() {
+        const uint32_t t = cur;
+        cur = nxt;
+        nxt = nx2;
+        nx2 = t;
+    };
+    using Even = std::integral_constant<int, 0>;
+    using Odd = std::integral_constant<int, 1>;
+    uint32_t c = 0;
+    for (; c + 1 < nchunks; c += 2) {  // no branch inside the loop (the compiler's load counting stays exact)
+        chunk(Even{}, c, cur, nxt, nx2);
+        rotate();
+        chunk(Odd{}, c + 1, cur, nxt, nx2);
+        rotate();
+    }
+    if (c < nchunks) chunk(Even{}, c, cur, nxt, nx2);
+    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+
+    // ---- epilogue: for row tile b (row m = l32) and column tile t, registers 4*q..4*q+3 are the four consecutive
+    // output columns n = 8*q + 4*h + (0..3)
+    const bool vec_ok = p.N % 4 == 0 && reinterpret_cast<uintptr_t>(FUSED ? (const void *)p.y : (const void *)p.C) % 16 == 0;
+#pragma unroll
+    for (int t = 0; t < TN; ++t)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const uint32_t n = n0 + wave * 64 + t * 32 + q * 8 + h * 4;
+            float sc[4], zc[4], bs[4];
+            if (FUSED) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const uint32_t nn = min(n + r, p.N - 1);
+                    sc[r] = p.epi.s_col[nn];
+                    zc[r] = p.epi.z_col[nn];
+                    bs[r] = BIAS ? p.epi.bias[nn] : 0.f;
+                }
+            }
+#pragma unroll
+            for (int b = 0; b < TM; ++b) {
+                const uint32_t m = m0 + b * 32 + l32;
+                if (m >= p.M || n >= p.N) continue;
+                if (FUSED) {
+                    const float sr = p.epi.s_row[m], zr = p.epi.z_row[m];
+                    v4f32 v;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        float o = dequant_hprec_one(acc[t][b][q * 4 + r], sr, zr, sc[r], zc[r]);
+                        if (BIAS) o = o + bs[r];
+                        v[r] = o;
+                    }
+                    float *dst = p.y + (uint64_t)m * p.N + n;
+                    if (vec_ok && n + 3 < p.N) {
+                        *reinterpret_cast<v4f32 *>(dst) = v;
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            if (n + r < p.N) dst[r] = v[r];
+                    }
+                } else {
+                    int32_t *dst = p.C + (uint64_t)m * p.N + n;
+                    if (vec_ok && n + 3 < p.N) {
+                        *reinterpret_cast<v4i *>(dst) = v4i{acc[t][b][q * 4], acc[t][b][q * 4 + 1], acc[t][b][q * 4 + 2], acc[t][b][q * 4 + 3]};
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            if (n + r < p.N) dst[r] = acc[t][b][q * 4 + r];
+                    }
+                }
+            }
+        }
+}
+
+template <bool FUSED, bool BIAS>
+static void launch_gemm8_variant(Gemm8Params &p, hipStream_t stream)
+{
+    p.tiles_n = (p.N + 255) / 256;
+    // 128-row tiles unless the problem is too small to give most CUs one (then 32-row tiles)
+    if (p.M > 64 && ((p.M + 127) / 128) * p.tiles_n >= 96) {
+        p.tiles_m = (p.M + 127) / 128;
+        hipLaunchKernelGGL((gemm_s8_kernel<4, FUSED, BIAS>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, stream, p);
+    } else {
+        p.tiles_m = (p.M + 31) / 32;
+        hipLaunchKernelGGL((gemm_s8_kernel<1, FUSED, BIAS>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, stream, p);
+    }
+}
+
+int launch_gemm_s8(const int8_t *A, const int8_t *B, uint32_t M, uint32_t N, uint32_t K, int32_t *C, const float *s_row,
+                   const float *z_row, const float *s_col, const float *z_col, const float *bias, float *y,
+                   hipStream_t stream)
+{
+    if (M == 0 || N == 0) return 0;
+    Gemm8Params p{A, B, M, N, K, C, y, Epi8{s_row, z_row, s_col, z_col, bias}, 0, 0};
+    if (C)
+        launch_gemm8_variant<false, false>(p, stream);
+    else if (bias)
+        launch_gemm8_variant<true, true>(p, stream);
+    else
+        launch_gemm8_variant<true, false>(p, stream);
+    return (int)hipGetLastError();
+}
+
+}  // namespace duq

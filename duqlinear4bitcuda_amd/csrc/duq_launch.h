@@ -55,4 +55,17 @@ int launch_activation_shadow_bf6(const uint8_t *q, uint32_t M, uint32_t K, uint8
 int launch_gemm_bf6(const uint8_t *X, const uint8_t *W, uint32_t M, uint32_t N, uint32_t K, const Epilogue &epi,
                     uint16_t *y, hipStream_t stream);
 
+// 8-bit asymmetric layer (duq_int8.hip): float32 activations, int8 codes, int32 accumulators, float32 results.
+int launch_asym_quant8(const float *x, const float *scale, const float *zeros, uint32_t rows, uint32_t cols, int8_t *q,
+                       hipStream_t stream);
+int launch_quantize_rows_asym8(const float *x, uint32_t rows, uint32_t cols, int8_t *q, float *scale, float *zeros,
+                               hipStream_t stream);
+int launch_dequant_hprec(const int32_t *acc, const float *s_row, const float *z_row, const float *s_col,
+                         const float *z_col, const float *bias, uint32_t rows, uint32_t cols, float *x,
+                         hipStream_t stream);
+// C != nullptr -> int32 accumulators [M,N]; else the float32 dequant (+ bias) fused into y.
+int launch_gemm_s8(const int8_t *A, const int8_t *B, uint32_t M, uint32_t N, uint32_t K, int32_t *C, const float *s_row,
+                   const float *z_row, const float *s_col, const float *z_col, const float *bias, float *y,
+                   hipStream_t stream);
+
 }  // namespace duq

@@ -14,7 +14,7 @@ import torch
 from .. import _HIP as _ops
 from ..tools import quantization as quant_utils
 from ..tools import tensor_utils
-from .quantizer import AsymQuantizer, SymQuantizer  # noqa: F401  (re-exported like the reference)
+from .quantizer import AsymQuantizer, AsymQuantizer8bit, SymQuantizer  # noqa: F401  (re-exported like the reference)
 
 _INT4_LEVELS = 2 ** 4
 
@@ -339,6 +339,64 @@ class LinearQuant4bitDUASQ(_Linear4bitBase):
         new.weight_zeros_1.copy_(z1.to(torch.float16))
         new.weight_scales_2.copy_(s2.to(torch.float16))
         new.weight_zeros_2.copy_(z2.to(torch.float16))
+        if module.bias is not None:
+            new.bias.copy_(module.bias)
+        return new
+
+
+class LinearQuant8bitASQ(torch.nn.Module):
+    """Asymmetric 8-bit linear layer on float32 activations (linear.py:300-368): buffers ``weight`` int8
+    [N, K] (codes 0..127), ``weight_scales`` / ``weight_zeros`` float32 [N, 1], optional ``bias``
+    float32 [N]; float32 result.  ``fused = False`` runs the reference's three steps (same bits)."""
+
+    fused = True
+
+    def __init__(self, in_features, out_features, bias=False, require_quantizer=True):
+        super().__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+        self.require_quantizer = require_quantizer
+        self.register_buffer("weight_scales", torch.zeros((out_features, 1), requires_grad=False, dtype=torch.float32))
+        self.register_buffer("weight_zeros", torch.zeros((out_features, 1), requires_grad=False, dtype=torch.float32))
+        self.register_buffer("weight", torch.randint(1, 7, (out_features, in_features), dtype=torch.int8,
+                                                     requires_grad=False))
+        if bias:
+            self.register_buffer("bias", torch.zeros((out_features), dtype=torch.float32))
+        else:
+            self.bias = None
+        if require_quantizer:
+            self.quantizer = AsymQuantizer8bit()
+
+    def forward(self, x):
+        if self.require_quantizer:
+            x = self.quantizer(x)
+        assert type(x) == tensor_utils.PackedQuantizedTensor, \
+            "Input should be quantized tensor, or require_quantizer should be passed as initial argument"
+        xq, scales_x, zeros_x = x.quantized_x, x.scales_x, x.zeros_x
+        if self.fused:
+            return tensor_utils.linear8bit_forward(xq, scales_x, zeros_x, self.weight, self.weight_scales,
+                                                   self.weight_zeros, self.bias)
+        acc = tensor_utils.matmul_8bit(xq, self.weight)
+        y = tensor_utils.asym_dequant_hprec(acc, scales_x, zeros_x, self.weight_scales, self.weight_zeros)
+        return y if self.bias is None else y + self.bias
+
+    @classmethod
+    def from_linear(cls, module: torch.nn.Linear, require_quantizer: bool = True):
+        """Per-row scale / zero over |W| with 127 steps, codes clamp(round(W / s) + z, 0, 127)
+        (linear.py:338-368)."""
+        new = cls(module.in_features, module.out_features, bias=module.bias is not None,
+                  require_quantizer=require_quantizer)
+        w = module.weight.data
+        levels = 2 ** 7
+        aw = w.abs()
+        w_max = aw.amax(dim=-1, keepdim=True)
+        w_min = aw.amin(dim=-1, keepdim=True)
+        scale = (w_max - w_min) / (levels - 1)
+        zeros = (-w_min / scale).round().to(torch.float32)
+        codes = torch.clamp(torch.round(w / scale) + zeros, 0, levels - 1)
+        new.weight.copy_(codes.to(torch.int8))
+        new.weight_scales.copy_(scale.to(torch.float32))
+        new.weight_zeros.copy_(zeros.to(torch.float32))
         if module.bias is not None:
             new.bias.copy_(module.bias)
         return new

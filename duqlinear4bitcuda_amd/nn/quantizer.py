@@ -86,3 +86,27 @@ class AsymQuantizer(torch.nn.Module):
             zeros = (-lo / scale).round().to(torch.float16)
             q = tensor_utils.asym_quant(x, scale, zeros)
         return tensor_utils.PackedQuantizedTensor(q, scale, zeros)
+
+
+class AsymQuantizer8bit(torch.nn.Module):
+    """float32 activations -> int8 codes 0..126 with per-token float32 scale = (max - min) / 127 and
+    zero = round(-min / scale) (quantizer.py:38-55).  One launch when the row length is a multiple of 4;
+    otherwise torch computes scale and zero and the given-scale kernel quantizes, as in the reference."""
+
+    def __init__(self, input_clip_ratio: float = 1.0):
+        super().__init__()
+        self.n_levels = 2 ** 7
+        self.input_clip_ratio = input_clip_ratio
+        self.fused = True
+
+    def forward(self, x) -> tensor_utils.PackedQuantizedTensor:
+        if not x.is_contiguous():
+            x = x.contiguous()
+        if self.fused and x.shape[-1] % 4 == 0 and x.data_ptr() % 16 == 0 and x.dtype == torch.float32:
+            return tensor_utils.PackedQuantizedTensor(*tensor_utils.quantize_asym_8bit(x))
+        min_val, _ = x.min(dim=-1, keepdim=True)
+        max_val, _ = x.max(dim=-1, keepdim=True)
+        scale = (max_val - min_val) / (self.n_levels - 1)
+        zeros = (-min_val / scale).round().to(torch.float32)
+        q = tensor_utils.asym_quant_8bit(x, scale, zeros)
+        return tensor_utils.PackedQuantizedTensor(q, scale, zeros)

@@ -58,6 +58,14 @@ def matmul(A, B):
     return _ops.matmul(A2, B2).view(*a_lead, *b_lead)
 
 
+def matmul_8bit(A, B):
+    """int8 x int8 -> int32 (tensor_utils.py:57-61)."""
+    assert A.shape[-1] % 32 == 0, "A.shape[-1]: {} must be multiplication of 32".format(A.shape[-1])
+    A2, a_lead = _flat(A)
+    B2, b_lead = _flat(B)
+    return _ops.matmul_8bit(A2, B2).view(*a_lead, *b_lead)
+
+
 def sym_quant(x, scale, qmax: int = 6):
     assert x.dtype == scale.dtype == torch.float16
     x2, lead = _flat(x)
@@ -89,6 +97,23 @@ def asym_quant(q, scale, zero):
     assert scale.dtype == zero.dtype == torch.float16
     x2, lead = _flat(q)
     return _ops.asym_quant(x2, scale.view(-1), zero.view(-1)).view(*lead, -1)
+
+
+def asym_quant_8bit(q, scale, zero):
+    """tensor_utils.py:98-102."""
+    assert q.dtype == torch.float32
+    assert scale.dtype == zero.dtype == torch.float32
+    x2, lead = _flat(q)
+    return _ops.asym_quant_8bit(x2, scale.view(-1), zero.view(-1)).view(*lead, -1)
+
+
+def asym_dequant_hprec(q, scale_row, zeros_row, scale_col, zeros_col, bits=32):
+    """tensor_utils.py:110-114."""
+    assert q.dtype == torch.int32
+    assert scale_row.dtype == zeros_row.dtype == scale_col.dtype == zeros_col.dtype == torch.float32
+    q2, lead = _flat(q)
+    return _ops.asym_dequant_hprec(q2, scale_row.view(-1), zeros_row.view(-1), scale_col.view(-1), zeros_col.view(-1),
+                                   bits).view(*lead, -1)
 
 
 def asym_dequant(q, scale_row, zeros_row, scale_col, zeros_col, bits=32):
@@ -192,3 +217,17 @@ def linear_forward_shadow(mode, x_shadow, scales_x, zeros_x, weight_shadow, w_sc
     """linear_forward / linear_forward_rowsum on shadows; bit-identical results."""
     return _ops.linear4bit_forward_bf6(mode, x_shadow, scales_x, zeros_x, weight_shadow, w_scale_1, w_zeros_1, w_scale_2,
                                        w_zeros_2, bias, rowsum_x, w_rowsum_adj)
+
+
+# ---- 8-bit asymmetric layer, fused (no counterpart in the reference wrappers) --------------
+
+def quantize_asym_8bit(x):
+    """(q int8 [..., K], scales [..., 1], zeros [..., 1]) in one launch."""
+    assert x.dtype == torch.float32
+    return _ops.quantize_rows_asym_8bit(x)
+
+
+def linear8bit_forward(xq, scales_x, zeros_x, weight, w_scale, w_zeros, bias=None):
+    """int8 GEMM + float32 dequant (+ bias) in one launch."""
+    assert xq.shape[-1] % 32 == 0, "A.shape[-1]: {} must be multiplication of 32".format(xq.shape[-1])
+    return _ops.linear8bit_forward(xq, scales_x, zeros_x, weight, w_scale, w_zeros, bias)

@@ -233,6 +233,45 @@ int duq_linear4bit_forward_bf6(int32_t mode, const uint8_t *x_bf6, const duq_hal
                                const int32_t *w_rowsum_adj, const duq_half *bias, uint32_t M, uint32_t N, uint32_t K,
                                duq_half *y, duq_stream_t stream);
 
+/* ---- the 8-bit asymmetric layer (LinearQuant8bitASQ, qlinear4bit/nn/linear.py:300-368) ---- */
+
+/* float32 activations [rows, cols], per-row float32 scale and zero point ->
+ * int8 codes clamp(rint(half(x / scale)) + rint(half(zero)), 0, 126).
+ * Replaces asym_quant_host_8bit (include/quant.h:71, src/kernels/quant.cu:241-279;
+ * binding src/export/bindings.cpp:245-266). */
+int duq_asym_quant_host_8bit(const float *x, const float *scale, const float *zeros, uint32_t rows, uint32_t cols,
+                             int8_t *q, duq_stream_t stream);
+
+/* A [M,K] int8 times B [N,K] int8 (both row-major; B is the weight as stored) -> C [M,N]
+ * int32, K % 32 == 0, A and B 16-byte aligned.
+ * Replaces matmul_host_8bit (include/gemm.h:14, src/kernels/gemm.cu:46-81; binding
+ * src/export/bindings.cpp:28-45; the Python wrapper asserts K % 32 == 0,
+ * qlinear4bit/tools/tensor_utils.py:57-61). */
+int duq_matmul_host_8bit(const int8_t *A, const int8_t *B, uint32_t M, uint32_t N, uint32_t K, int32_t *C,
+                         duq_stream_t stream);
+
+/* x[r,c] = (scale_row[r] * scale_col[c]) * (float(q[r,c]) - (zeros_row[r] + zeros_col[c])), float32
+ * with one rounding per operator.
+ * Replaces asym_dequant_host_hprec (include/quant.h:118, src/kernels/quant.cu:281-323;
+ * binding src/export/bindings.cpp:309-350). */
+int duq_asym_dequant_host_hprec(const int32_t *q, const float *scale_row, const float *zeros_row,
+                                const float *scale_col, const float *zeros_col, uint32_t rows, uint32_t cols, float *x,
+                                duq_stream_t stream);
+
+/* No counterpart in the reference: AsymQuantizer8bit.forward (qlinear4bit/nn/quantizer.py:38-55)
+ * in one launch: per-row min / max, scale = (max - min) / 127, zero = rint(-min / scale), then
+ * the codes of duq_asym_quant_host_8bit.  cols % 4 == 0, x 16-byte aligned, q 4-byte aligned. */
+int duq_quantize_rows_asym_8bit(const float *x, uint32_t rows, uint32_t cols, int8_t *q, float *scale, float *zeros,
+                                duq_stream_t stream);
+
+/* No counterpart in the reference: duq_matmul_host_8bit + duq_asym_dequant_host_hprec (+ float32
+ * bias [N], may be NULL) in one launch, the accumulators never leaving the registers;
+ * y [M,N] float32 is bit-identical to the three steps (LinearQuant8bitASQ.forward,
+ * qlinear4bit/nn/linear.py:323-335). */
+int duq_linear8bit_forward(const int8_t *xq, const float *scale_x, const float *zeros_x, const int8_t *w,
+                           const float *w_scale, const float *w_zeros, const float *bias, uint32_t M, uint32_t N,
+                           uint32_t K, float *y, duq_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

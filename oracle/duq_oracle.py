@@ -34,6 +34,9 @@ fixes by definition instead ("parity unpinned" for exactly these corners):
 The row-sum functions (``asym_quant_shifted`` ... ``linear4bit_asq_rowsum_forward``) restate a
 mode the reference does not have; there is nothing of the reference to be in parity with, and
 they are pinned by the integer identity and the float64 product of the dequantized operands.
+The 8-bit functions (``asym8_scales_zeros`` ... ``linear8bit_asq_forward``) restate the reference's
+LinearQuant8bitASQ path (float32 arithmetic, one rounding per operator); pinned by hand-computed
+cases, float64 evaluation where float64 is exact, a brute-force GEMM and torch-CPU operators.
 The E3M2 shadow functions (``e3m2_decode`` ... ``weight_shadow_bf6``) describe a storage format
 of the library, not of the reference: they are pinned by the published OCP Microscaling
 formula for E3M2 (decode), by decode(encode(v)) == v for every int4 value, and by the round
@@ -565,3 +568,103 @@ def weight_shadow_bf6(w_packed):
     out = np.concatenate([b[..., :16].reshape(N // 16, K // 128, 1024), b[..., 16:].reshape(N // 16, K // 128, 512)],
                          axis=-1)
     return np.ascontiguousarray(out).reshape(N, K * 3 // 4)
+
+
+# ----------------------------------------------------------------------------------
+# 8-bit asymmetric path: AsymQuantizer8bit -> matmul_8bit -> asym_dequant_hprec
+# (qlinear4bit/nn/quantizer.py:38-55, src/kernels/quant.cu:241-323, src/kernels/gemm.cu:46-81,
+#  qlinear4bit/nn/linear.py:300-368).  Everything is float32 with one rounding per operator.
+# ----------------------------------------------------------------------------------
+QMAX_ASYM_8BIT = 126     # src/kernels/quant.cu:242
+LEVELS_8BIT = 2 ** 7     # quantizer.py:41, linear.py:350
+
+
+def asym8_scales_zeros(x, device_division: bool = True):
+    """AsymQuantizer8bit.forward (quantizer.py:47-51): scale = (max - min) / 127,
+    zeros = round(-min / scale), all float32 [rows, 1].
+
+    The reference runs these torch statements on its GPU, where torch evaluates
+    tensor / python-scalar as tensor * float32(1 / scalar) (one bit may differ from the
+    quotient); ``device_division=False`` gives the true quotient torch computes on a CPU.
+    tensor / tensor is the IEEE quotient on both."""
+    x = np.asarray(x, _F32)
+    lo = x.min(axis=-1, keepdims=True)
+    hi = x.max(axis=-1, keepdims=True)
+    with np.errstate(invalid="ignore", divide="ignore", over="ignore"):
+        d = (hi - lo).astype(_F32)
+        if device_division:
+            scale = (d * (_F32(1.0) / _F32(LEVELS_8BIT - 1))).astype(_F32)
+        else:
+            scale = (d / _F32(LEVELS_8BIT - 1)).astype(_F32)
+        zeros = np.rint(((-lo).astype(_F32) / scale).astype(_F32)).astype(_F32)
+    return scale, zeros
+
+
+def asym_quant_8bit(x, scale, zeros):
+    """asym_quantize_f16_i8_kernel (quant.cu:244-264): data = x / scale in float32; both
+    ``__half2int_rn`` calls take a float argument, which C++ converts to binary16 first
+    (round to nearest even, overflow to inf), then round to the nearest-even integer; the
+    int add wraps; clamp to [0, 126]; stored as int8."""
+    x = np.asarray(x, _F32)
+    s = np.asarray(scale, _F32).reshape(-1, 1)
+    z = np.asarray(zeros, _F32).reshape(-1, 1)
+    with np.errstate(invalid="ignore", divide="ignore", over="ignore"):
+        data = (x / s).astype(_F32)
+        qi = half_to_int_rn(data.astype(_F16))
+        zi = half_to_int_rn(z.astype(_F16))
+    total = _wrap_i32(qi.astype(np.int64) + zi.astype(np.int64))
+    return np.clip(total, 0, QMAX_ASYM_8BIT).astype(np.int8)
+
+
+def matmul_s8(a, b):
+    """matmul_host_8bit (gemm.cu:46-81): C[m,n] = sum_k A[m,k] * B[n,k], int8 operands,
+    int32 accumulation (wraps like the hardware accumulator; it cannot for K <= 133 152)."""
+    # float64 BLAS is exact here: |sum| <= 2^14 * K, far below 2^53
+    a = np.asarray(a, np.int8).astype(np.float64)
+    b = np.asarray(b, np.int8).astype(np.float64)
+    return _wrap_i32((a @ b.T).astype(np.int64))
+
+
+def asym_dequant_hprec(acc, scale_row, zeros_row, scale_col, zeros_col):
+    """asym_dequantize_i32_f16_hp_kernel (quant.cu:283-299), float32 throughout:
+    x = (s_r * s_c) * (float(acc) - (z_r + z_c))."""
+    acc = np.asarray(acc, np.int32)
+    sr = np.asarray(scale_row, _F32).reshape(-1, 1)
+    zr = np.asarray(zeros_row, _F32).reshape(-1, 1)
+    sc = np.asarray(scale_col, _F32).reshape(1, -1)
+    zc = np.asarray(zeros_col, _F32).reshape(1, -1)
+    with np.errstate(invalid="ignore", over="ignore"):
+        scales = (sr * sc).astype(_F32)
+        zeros = (zr + zc).astype(_F32)
+        return (scales * (acc.astype(_F32) - zeros).astype(_F32)).astype(_F32)
+
+
+def weight_asym8_from_linear(w):
+    """LinearQuant8bitASQ.from_linear (linear.py:346-360): max|W| and min|W| per row,
+    scale = (max - min) / 127, zero = round(-min / scale) as float32,
+    q = clamp(round(W / scale) + zero, 0, 127) as int8; the arithmetic runs in the dtype of
+    the layer's weight (binary16 in the reference's use).  The division by 127 is the true
+    quotient, as torch computes it for a module on the CPU (on a GPU see asym8_scales_zeros)."""
+    w = np.asarray(w)
+    dt = w.dtype.type
+    aw = np.abs(w)
+    mx = aw.max(axis=-1, keepdims=True)
+    mn = aw.min(axis=-1, keepdims=True)
+    with np.errstate(invalid="ignore", divide="ignore", over="ignore"):
+        scale = ((mx - mn).astype(dt) / dt(LEVELS_8BIT - 1)).astype(dt)
+        zero = np.rint(((-mn).astype(dt) / scale).astype(dt)).astype(_F32)
+        # the sum of the binary16 quotient and the float32 zero point is float32 (torch's type promotion)
+        q = np.clip(np.rint((w / scale).astype(dt)).astype(_F32) + zero, 0, LEVELS_8BIT - 1)
+    return q.astype(np.int8), scale.astype(_F32), zero
+
+
+def linear8bit_asq_forward(x, w_q, w_scales, w_zeros, bias=None):
+    """LinearQuant8bitASQ.forward (linear.py:326-337) for float32 x [M,K]:
+    returns (y float32, acc int32, q int8, scale, zeros)."""
+    s, z = asym8_scales_zeros(x)
+    q = asym_quant_8bit(x, s, z)
+    acc = matmul_s8(q, w_q)
+    y = asym_dequant_hprec(acc, s, z, w_scales, w_zeros)
+    if bias is not None:
+        y = (y + np.asarray(bias, _F32).reshape(1, -1)).astype(_F32)
+    return y, acc, q, s, z
