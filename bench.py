@@ -217,6 +217,49 @@ def other_shapes_section(dev):
     return out
 
 
+def int8_layer_section(dev):
+    """The 8-bit asymmetric layer (LinearQuant8bitASQ) at the headline shape: float32 activations, quantizer
+    launch + fused GEMM launch, float32 result; the GEMM alone against the dense int8 MFMA peak."""
+    import torch
+
+    from duqlinear4bitcuda_amd import _HIP
+    from duqlinear4bitcuda_amd.nn import LinearQuant8bitASQ
+
+    out = []
+    for (M, K, N) in [(2048, 4096, 4096), (2048, 4096, 11008), (16, 4096, 4096)]:
+        g = torch.Generator().manual_seed(6)
+        x = torch.randn(M, K, generator=g).to(dev)
+        layer = LinearQuant8bitASQ(K, N, bias=False).to(dev)
+        layer.weight.copy_(torch.randint(0, 128, (N, K), dtype=torch.int8, generator=g))
+        layer.weight_scales.copy_(torch.rand(N, 1, generator=g) * 0.009 + 0.001)
+        layer.weight_zeros.copy_(-torch.randint(0, 20, (N, 1), generator=g).float())
+        p = layer.quantizer(x)
+        y = layer(x)
+        layer.fused = False
+        same = bool(torch.equal(layer(x), y))     # the reference's three steps give the same bits
+        us3 = graph_time_us([lambda: layer(x)] * 10)
+        layer.fused = True
+        ops = 2.0 * M * N * K
+        us_step = graph_time_us([lambda: layer(x)] * 10)
+        wt = layer._tiled_weight()
+        us_gemm = graph_time_us([lambda: _HIP.linear8bit_forward(p.quantized_x, p.scales_x, p.zeros_x, wt,
+                                                                 layer.weight_scales, layer.weight_zeros,
+                                                                 tiled_rows=N)] * 10)
+        us_rowmajor = graph_time_us([lambda: _HIP.linear8bit_forward(p.quantized_x, p.scales_x, p.zeros_x, layer.weight,
+                                                                     layer.weight_scales, layer.weight_zeros)] * 10)
+        us_quant = graph_time_us([lambda: layer.quantizer(x)] * 10)
+        out.append({"M": M, "K": K, "N": N, "step_us": round(us_step, 2), "step_TOPS": round(ops / us_step / 1e6, 1),
+                    "three_step_us": round(us3, 2), "fused_equals_three_steps": same,
+                    "quantize_us": round(us_quant, 2),
+                    "quantize_GBps": round((M * K * 5 + M * 8) / us_quant / 1e3, 1),
+                    "gemm_rowmajor_weight_us": round(us_rowmajor, 2),
+                    "gemm_fused_us": round(us_gemm, 2), "gemm_TOPS": round(ops / us_gemm / 1e6, 1),
+                    "gemm_frac_of_int8_peak": round(ops / us_gemm / 1e6 / PEAK_INT8_TOPS, 4),
+                    "gemm_algorithmic_GBps": round((M * K + N * K + M * N * 4) / us_gemm / 1e3, 1)})
+        del layer, x
+    return out
+
+
 def cpu_baseline(x_cpu, wq_cpu, sw_cpu, ops, budget_s=15.0):
     """The reference's CPU fake-quant path (torch-CPU) on the same workload, host cores."""
     import torch
@@ -360,6 +403,7 @@ def main():
     quantizer = quantizer_section(dev)
     asym = None if args.quick else asym_section(dev)
     other = None if args.quick else other_shapes_section(dev)
+    int8_layer = None if args.quick else int8_layer_section(dev)
     best_decode = max(decode, key=lambda d: d["GBps"])
     roofline_decode = {"bound": "hbm", "kernel": "gemv_s4_dot_kernel (M=1) / gemm_s4_skinny_kernel (2<=M<=16) / gemm_s4_ring_kernel (17<=M<=64, long rows)", "achieved": best_decode["GBps"],
                        "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": best_decode["frac_hbm"],
@@ -398,6 +442,7 @@ def main():
         "quantizer": quantizer,
         "asym": asym,
         "other_shapes": other,
+        "int8_layer": int8_layer,
         "cpu_baseline": cpu,
         "device": {"name": props.name, "arch": props.gcnArchName, "cus": props.multi_processor_count},
     }

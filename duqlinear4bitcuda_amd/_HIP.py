@@ -649,8 +649,20 @@ def quantize_rows_asym_8bit(x: torch.Tensor):
     return q, s, z
 
 
-def linear8bit_forward(xq, scale_x, zeros_x, w, w_scale, w_zeros, bias=None):
-    """matmul_8bit + asym_dequant_hprec (+ bias) in one launch; xq [..., K] int8 -> float32 [..., N]."""
+def weight_tile_8bit(w: torch.Tensor) -> torch.Tensor:
+    """int8 weight [N, K] -> the tiled copy [ceil(N/32)*32*K] that linear8bit_forward(..., tiled_rows=N) takes."""
+    _check("weight_tile_8bit", w)
+    _check_dtype("weight_tile_8bit", w, "w", _I8)
+    N, K = w.size(0), w.size(1)
+    out = torch.empty(((N + 31) // 32 * 32 * K,), dtype=_I8, device=w.device)
+    st = _launch(w.device, _lib.load().duq_weight_tile_8bit, _ptr(w), N, K, _ptr(out))
+    _lib.check(st, "weight_tile_8bit")
+    return out
+
+
+def linear8bit_forward(xq, scale_x, zeros_x, w, w_scale, w_zeros, bias=None, tiled_rows=None):
+    """matmul_8bit + asym_dequant_hprec (+ bias) in one launch; xq [..., K] int8 -> float32 [..., N].
+    ``w`` is the weight [N, K], or with ``tiled_rows=N`` its tiled copy from weight_tile_8bit (same bits)."""
     name = "linear8bit_forward"
     if not isinstance(xq, torch.Tensor):
         raise RuntimeError(f"{name}: argument #0 is not a tensor")
@@ -659,9 +671,16 @@ def linear8bit_forward(xq, scale_x, zeros_x, w, w_scale, w_zeros, bias=None):
     _fast_check(name, "w", w, _I8, dev)
     K = xq.shape[-1]
     M = xq.numel() // K if K else 0
-    N = w.size(0)
-    if w.dim() != 2 or w.size(1) != K:
-        raise RuntimeError(f"{name}: K differs: xq {tuple(xq.shape)} vs w {tuple(w.shape)}")
+    if tiled_rows is not None:
+        N = int(tiled_rows)
+        if w.numel() != (N + 31) // 32 * 32 * K:
+            raise RuntimeError(f"{name}: the tiled weight has {w.numel()} bytes, expected {(N + 31) // 32 * 32 * K}")
+        entry = _lib.load().duq_linear8bit_forward_tiled
+    else:
+        N = w.size(0)
+        if w.dim() != 2 or w.size(1) != K:
+            raise RuntimeError(f"{name}: K differs: xq {tuple(xq.shape)} vs w {tuple(w.shape)}")
+        entry = _lib.load().duq_linear8bit_forward
     for t, what, n in ((scale_x, "scale_x", M), (zeros_x, "zeros_x", M), (w_scale, "w_scale", N),
                        (w_zeros, "w_zeros", N), (bias, "bias", N)):
         if t is None and what == "bias":
@@ -672,7 +691,7 @@ def linear8bit_forward(xq, scale_x, zeros_x, w, w_scale, w_zeros, bias=None):
         if t.numel() != n:
             raise RuntimeError(f"{name}: expected {what} to have {n} elements, got {tuple(t.shape)}")
     y = torch.empty(xq.shape[:-1] + (N,), dtype=_F32, device=dev)
-    st = _launch(dev, _lib.load().duq_linear8bit_forward, xq.data_ptr(), scale_x.data_ptr(), zeros_x.data_ptr(),
+    st = _launch(dev, entry, xq.data_ptr(), scale_x.data_ptr(), zeros_x.data_ptr(),
                  w.data_ptr(), w_scale.data_ptr(), w_zeros.data_ptr(), _ptr(bias), M, N, K, y.data_ptr())
     if st:
         _lib.check(st, name)

@@ -48,6 +48,8 @@ PROTOTYPES = {
     "duq_matmul_host_8bit": [_c_p, _c_p, _c_u32, _c_u32, _c_u32, _c_p, _c_p],
     "duq_asym_dequant_host_hprec": [_c_p, _c_p, _c_p, _c_p, _c_p, _c_u32, _c_u32, _c_p, _c_p],
     "duq_quantize_rows_asym_8bit": [_c_p, _c_u32, _c_u32, _c_p, _c_p, _c_p, _c_p],
+    "duq_weight_tile_8bit": [_c_p, _c_u32, _c_u32, _c_p, _c_p],
+    "duq_linear8bit_forward_tiled": [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_u32, _c_u32, _c_u32, _c_p, _c_p],
     "duq_linear8bit_forward": [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_u32, _c_u32, _c_u32, _c_p, _c_p],
 }
 

@@ -332,7 +332,7 @@ int duq_matmul_host_8bit(const int8_t *A, const int8_t *B, uint32_t M, uint32_t 
     if (M == 0 || N == 0) return DUQ_OK;
     if (!C) return DUQ_E_NULL;
     if (!aligned(C, 4)) return DUQ_E_ALIGN;
-    return duq::launch_gemm_s8(A, B, M, N, K, C, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, as_stream(stream));
+    return duq::launch_gemm_s8(A, B, false, M, N, K, C, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, as_stream(stream));
 }
 
 int duq_asym_dequant_host_hprec(const int32_t *q, const float *scale_row, const float *zeros_row,
@@ -353,7 +353,29 @@ int duq_linear8bit_forward(const int8_t *xq, const float *scale_x, const float *
     if (M == 0 || N == 0) return DUQ_OK;
     if (!scale_x || !zeros_x || !w_scale || !w_zeros || !y) return DUQ_E_NULL;
     if (!aligned(y, 4)) return DUQ_E_ALIGN;
-    return duq::launch_gemm_s8(xq, w, M, N, K, nullptr, scale_x, zeros_x, w_scale, w_zeros, bias, y, as_stream(stream));
+    return duq::launch_gemm_s8(xq, w, false, M, N, K, nullptr, scale_x, zeros_x, w_scale, w_zeros, bias, y, as_stream(stream));
+}
+
+int duq_weight_tile_8bit(const int8_t *w, uint32_t N, uint32_t K, int8_t *w_tiled, duq_stream_t stream)
+{
+    if (N == 0 || K == 0) return DUQ_OK;
+    if (!w || !w_tiled) return DUQ_E_NULL;
+    if (K % 32 != 0) return DUQ_E_KALIGN;
+    if (K > (1u << 23) || N > (1u << 22)) return DUQ_E_TOO_LARGE;
+    if (!aligned(w, 16) || !aligned(w_tiled, 16)) return DUQ_E_ALIGN;
+    return duq::launch_weight_tile8(w, N, K, w_tiled, as_stream(stream));
+}
+
+int duq_linear8bit_forward_tiled(const int8_t *xq, const float *scale_x, const float *zeros_x, const int8_t *w_tiled,
+                                 const float *w_scale, const float *w_zeros, const float *bias, uint32_t M, uint32_t N,
+                                 uint32_t K, float *y, duq_stream_t stream)
+{
+    if (int e = check_gemm8(xq, w_tiled, M, N, K)) return e;
+    if (M == 0 || N == 0) return DUQ_OK;
+    if (!scale_x || !zeros_x || !w_scale || !w_zeros || !y) return DUQ_E_NULL;
+    if (!aligned(y, 4)) return DUQ_E_ALIGN;
+    return duq::launch_gemm_s8(xq, w_tiled, true, M, N, K, nullptr, scale_x, zeros_x, w_scale, w_zeros, bias, y,
+                               as_stream(stream));
 }
 
 }  // extern "C"

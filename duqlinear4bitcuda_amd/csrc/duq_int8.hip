@@ -222,11 +222,14 @@ int launch_dequant_hprec(const int32_t *acc, const float *s_row, const float *z_
 // GEMM  C[m,n] = sum_k A[m,k] * B[n,k]   (int8, int32 accumulation)
 // ---------------------------------------------------------------------------------
 // Tile 32*TM (M) x 256 (N), 4 wavefronts side by side along N (32*TM x 64 each, TM x 2 MFMA tiles of 32 x 32),
-// 128-k chunks.  Weights go global -> registers: lane (r = lane % 32, h = lane / 32) of a 32-row tile holds bytes
-// [h*64 + s*16, +16) of row r for step s of the chunk (four 128-bit loads of 64 contiguous bytes per lane; integer
-// accumulation is order-free, the activations use the same k order).  Activations go global -> registers -> LDS
-// (three buffers, rows padded to 144 bytes, one barrier per chunk) -> fragments read one step ahead.  The weight
-// operand is the MFMA "A" side, so a lane holds four consecutive output columns of one row.
+// 256-k chunks of 8 steps.  A wavefront's 64 weight rows are needed by no other wavefront, so weights go
+// global -> registers: lane (r = lane % 32, h = lane / 32) holds bytes [32*s + 16*h, +16) of row r for step s, which
+// is the operand layout of v_mfma_i32_32x32x32_i8; the register of step s is refetched for the next chunk as soon
+// as the step's last MFMA has been issued, so every weight load has a whole chunk (64 MFMAs,
+// 2048 cycles) to arrive.  Activations are shared by the four wavefronts: global -> registers -> LDS (three buffers, rows padded
+// to 272 bytes, one barrier per chunk) -> fragments read one step ahead; the register of piece j is stored at step
+// j (for the chunk after next) and refetched at once (for the chunk after that), again a whole chunk ahead.
+// The weight operand is the MFMA "A" side, so a lane ends up with four consecutive output columns of one row.
 struct Gemm8Params {
     const int8_t *A;  // [M, K]
     const int8_t *B;  // [N, K]
@@ -239,16 +242,22 @@ struct Gemm8Params {
 
 __device__ __forceinline__ void lds_barrier8() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-template <int TM, bool FUSED, bool BIAS>
+template <int TM, bool FUSED, bool BIAS, bool TILED>
 __global__ __launch_bounds__(256) void gemm_s8_kernel(Gemm8Params p)
 {
-    static_assert(TM == 4 || TM == 1, "32-row MFMA tiles per wavefront along M");
+    static_assert(TM == 4 || TM == 2 || TM == 1, "32-row MFMA tiles per wavefront along M");
     constexpr int BM = 32 * TM, BN = 256, TN = 2;
-    constexpr uint32_t kStride = 144;
+    constexpr int NS = 8;                 // steps (of 32 k) per chunk
+    constexpr uint32_t kChunk = 32 * NS;  // 256
+    constexpr uint32_t kStride = kChunk + 16;
     constexpr uint32_t kBuf = BM * kStride;
-    constexpr int NXP = BM * 8 / 256;  // 16-byte activation pieces per thread and chunk
+    constexpr int NXP = BM / 16;          // 16-byte activation pieces per thread and chunk: 8, 4, 2
 
-    __shared__ __attribute__((aligned(16))) uint8_t lds[3 * kBuf];
+    constexpr uint32_t kEStride = 64 * 4 + 16;  // epilogue staging: 32 rows of 64 int32 per wavefront
+    constexpr uint32_t kLds = 3 * kBuf > 4 * 32 * kEStride ? 3 * kBuf : 4 * 32 * kEStride;
+
+    __shared__ __attribute__((aligned(16))) uint8_t lds[kLds];
+    __shared__ float row_par[2][BM];  // the tile's per-row scale and zero point, fetched before the loop
 
     uint32_t tile_m, tile_n;
     tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
@@ -256,36 +265,44 @@ __global__ __launch_bounds__(256) void gemm_s8_kernel(Gemm8Params p)
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63u, wave = tid >> 6;
     const uint32_t l32 = lane & 31u, h = lane >> 5;
-    const uint32_t nchunks = (p.K + 127) / 128;
+    const uint32_t nchunks = (p.K + kChunk - 1) / kChunk;
 
-    const __amdgpu_buffer_rsrc_t rW = make_rsrc(p.B + (uint64_t)n0 * p.K, min(p.N - n0, (uint32_t)BN) * p.K);
+    // tiled weights: whole 32-row tiles (the last one zero-padded), K * 32 bytes each
+    const uint32_t wrows = TILED ? min((p.N + 31u) / 32u * 32u - n0, (uint32_t)BN) : min(p.N - n0, (uint32_t)BN);
+    const __amdgpu_buffer_rsrc_t rW = make_rsrc(p.B + (uint64_t)n0 * p.K, wrows * p.K);
     const __amdgpu_buffer_rsrc_t rX = make_rsrc(p.A + (uint64_t)m0 * p.K, min(p.M - m0, (uint32_t)BM) * p.K);
 
-    // K % 32 == 0, so a 16-byte piece is all inside a row or all past its end; pieces past K (last chunk) and
-    // chunks past the last are redirected out of range and read as zero
+    // K % 32 == 0, so a 16-byte piece is all inside a row or all past its end; pieces past K (in the last chunk, or of
+    // chunks past the last) are redirected out of the descriptor's range and read as zero
+    uint32_t wrow[TN];
+#pragma unroll
+    for (int t = 0; t < TN; ++t)
+        wrow[t] = TILED ? (wave * 64 + t * 32) * p.K + lane * 16 : (wave * 64 + t * 32 + l32) * p.K + h * 16;
     auto load_w = [&](int t, int s, uint32_t c) -> v4i {
-        const uint32_t k = c * 128 + h * 64 + s * 16;
-        const uint32_t off = (wave * 64 + t * 32 + l32) * p.K + k;
-        return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rW, (int)(k < p.K ? off : kOobOffset), 0, 0));
+        const uint32_t k = c * kChunk + s * 32;  // + h*16 < K  <=>  k < K
+        // tiled: the fragment of (tile, step) is 1 KB in lane order, steps one after the other
+        return __builtin_bit_cast(v4i, buf_load16(rW, k < p.K ? wrow[t] + (TILED ? k * 32 : k) : kOobOffset, 0));
     };
     uint32_t xrow[NXP], xlds[NXP];
-    const uint32_t xpiece = tid & 7u;
+    const uint32_t xpiece = tid & 15u;
 #pragma unroll
     for (int j = 0; j < NXP; ++j) {
-        xrow[j] = (tid >> 3) + j * 32;
-        xlds[j] = xrow[j] * kStride + xpiece * 16;
+        const uint32_t row = (tid >> 4) + j * 16;
+        xrow[j] = row * p.K + xpiece * 16;
+        xlds[j] = row * kStride + xpiece * 16;
     }
     auto load_x = [&](int j, uint32_t c) -> v4u {
-        const uint32_t k = c * 128 + xpiece * 16;
-        return buf_load16(rX, k < p.K ? xrow[j] * p.K + k : kOobOffset, 0);
+        const uint32_t k = c * kChunk;
+        return buf_load16(rX, k + xpiece * 16 < p.K ? xrow[j] + k : kOobOffset, 0);
     };
-    // fragment of rows b*32 + l32, step s: bytes [h*64 + s*16, +16) of the row's chunk
-    const uint32_t frag = l32 * kStride + h * 64;
+    // fragment of rows b*32 + l32, step s: bytes [32*s + 16*h, +16) of the row's chunk
+    const uint32_t frag = l32 * kStride + h * 16;
     auto read_x = [&](uint32_t buf, int b, int s) -> v4i {
-        return *reinterpret_cast<const v4i *>(lds + buf + frag + b * 32 * kStride + s * 16);
+        return *reinterpret_cast<const v4i *>(lds + buf + frag + b * 32 * kStride + s * 32);
     };
 
-    v4i wreg[2][TN][4];  // [chunk parity][column tile][step]
+    constexpr int WR = 1;  // chunks of weights in flight (2 measured no faster: the loop is bound by bytes per cycle, not by latency)
+    v4i wreg[WR][TN][NS];
     v4u xreg[NXP];
     v4i fx[2][TM];
     v16i32 acc[TN][TM];
@@ -296,6 +313,25 @@ __global__ __launch_bounds__(256) void gemm_s8_kernel(Gemm8Params p)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[t][b][r] = 0;
 
+    // ---- epilogue parameters first: their latency disappears behind the loop
+    const uint32_t c16 = lane & 15u, r4 = lane >> 4;
+    const uint32_t n_out = n0 + wave * 64 + c16 * 4;  // first of the four output columns this lane stores
+    float sc[4], zc[4], bs[4];
+    if (FUSED) {
+        if (tid < BM) {
+            const uint32_t m = min(m0 + tid, p.M - 1);
+            row_par[0][tid] = p.epi.s_row[m];
+            row_par[1][tid] = p.epi.z_row[m];
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const uint32_t nn = min(n_out + r, p.N - 1);
+            sc[r] = p.epi.s_col[nn];
+            zc[r] = p.epi.z_col[nn];
+            bs[r] = BIAS ? p.epi.bias[nn] : 0.f;
+        }
+    }
+
     // ---- prologue: activations of chunks 0 and 1 -> LDS, chunk 2 -> registers; weights of chunk 0
 #pragma unroll
     for (int q = 0; q < 2; ++q) {
@@ -304,38 +340,56 @@ __global__ __launch_bounds__(256) void gemm_s8_kernel(Gemm8Params p)
 #pragma unroll
         for (int j = 0; j < NXP; ++j) *reinterpret_cast<v4u *>(lds + q * kBuf + xlds[j]) = xreg[j];
     }
+    // issued in the order of the main loop's chunks, so that the loop's wait counts are the same on entry and on
+    // the back edge (the compiler takes the stricter of the two)
 #pragma unroll
-    for (int t = 0; t < TN; ++t)
+    for (int w = 0; w < WR; ++w) {
 #pragma unroll
-        for (int s = 0; s < 4; ++s) wreg[0][t][s] = load_w(t, s, 0);
+        for (int s = 0; s < NS; ++s) {
+            if (TM == 1) {
+                wreg[w][0][s] = load_w(0, s, w);
+                wreg[w][1][s] = load_w(1, s, w);
+            }
+            if (w == WR - 1) {
 #pragma unroll
-    for (int j = 0; j < NXP; ++j) xreg[j] = load_x(j, 2);
+                for (int j = 0; j < NXP; ++j)
+                    if (j * NS / NXP == s) xreg[j] = load_x(j, 2);
+            }
+            if (TM != 1) {
+                wreg[w][0][s] = load_w(0, s, w);
+                wreg[w][1][s] = load_w(1, s, w);
+            }
+        }
+    }
     lds_barrier8();
 #pragma unroll
     for (int b = 0; b < TM; ++b) fx[0][b] = read_x(0, b, 0);
 
-    auto chunk = [&](auto par, uint32_t c, uint32_t cur, uint32_t nxt, uint32_t nx2) {
-        constexpr int PAR = decltype(par)::value;
+    uint32_t cur = 0, nxt = kBuf, nx2 = 2 * kBuf;
+    auto chunk = [&](auto par, uint32_t c) {
+        constexpr int W = decltype(par)::value % WR;
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
+        for (int s = 0; s < NS; ++s) {
 #pragma unroll
             for (int b = 0; b < TM; ++b) {
 #pragma unroll
                 for (int t = 0; t < TN; ++t) {
                     asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0"
                                  : "+a"(acc[t][b])
-                                 : "v"(wreg[PAR][t][s]), "v"(fx[s & 1][b]));
+                                 : "v"(wreg[W][t][s]), "v"(fx[s & 1][b]));
                     __builtin_amdgcn_sched_barrier(0);
                     // ---- side work in the shadow of this MFMA
                     if (t == 0)  // next step's fragment of this row tile (the next chunk's first step comes from `nxt`)
-                        fx[(s + 1) & 1][b] = s < 3 ? read_x(cur, b, s + 1) : read_x(nxt, b, 0);
-                    if (t == 1 && b == 0) {  // weights of the next chunk: this step's two pieces
-                        wreg[PAR ^ 1][0][s] = load_w(0, s, c + 1);
-                        wreg[PAR ^ 1][1][s] = load_w(1, s, c + 1);
-                    }
-                    if (t == 1 && s == 3 && b < NXP) {  // chunk c+2 -> its LDS buffer, then fetch chunk c+3
-                        *reinterpret_cast<v4u *>(lds + nx2 + xlds[b]) = xreg[b];
-                        xreg[b] = load_x(b, c + 3);
+                        fx[(s + 1) & 1][b] = s + 1 < NS ? read_x(cur, b, s + 1) : read_x(nxt, b, 0);
+                    if (b == TM - 1)  // last use of this step's weight register: refetch it for the next chunk
+                        wreg[W][t][s] = load_w(t, s, c + WR);
+                    if (t == 1 && b == 0) {  // activation pieces: chunk c+2 -> its LDS buffer, then fetch chunk c+3
+#pragma unroll
+                        for (int j = 0; j < NXP; ++j)
+                            if (j * NS / NXP == s) {
+                                *reinterpret_cast<v4u *>(lds + nx2 + xlds[j]) = xreg[j];
+                                xreg[j] = load_x(j, c + 3);
+                            }
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -344,10 +398,6 @@ __global__ __launch_bounds__(256) void gemm_s8_kernel(Gemm8Params p)
         // the MFMAs are opaque to the compiler's hazard tracking: accumulator copies at a join must find them retired
         asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
         lds_barrier8();
-    };
-
-    uint32_t cur = 0, nxt = kBuf, nx2 = 2 * kBuf;
-    auto rotate = [&]() {
         const uint32_t t = cur;
         cur = nxt;
         nxt = nx2;
@@ -357,93 +407,128 @@ __global__ __launch_bounds__(256) void gemm_s8_kernel(Gemm8Params p)
     using Odd = std::integral_constant<int, 1>;
     uint32_t c = 0;
     for (; c + 1 < nchunks; c += 2) {  // no branch inside the loop (the compiler's load counting stays exact)
-        chunk(Even{}, c, cur, nxt, nx2);
-        rotate();
-        chunk(Odd{}, c + 1, cur, nxt, nx2);
-        rotate();
+        chunk(Even{}, c);
+        chunk(Odd{}, c + 1);
     }
-    if (c < nchunks) chunk(Even{}, c, cur, nxt, nx2);
+    if (c < nchunks) chunk(Even{}, c);
     asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 
-    // ---- epilogue: for row tile b (row m = l32) and column tile t, registers 4*q..4*q+3 are the four consecutive
-    // output columns n = 8*q + 4*h + (0..3)
-    const bool vec_ok = p.N % 4 == 0 && reinterpret_cast<uintptr_t>(FUSED ? (const void *)p.y : (const void *)p.C) % 16 == 0;
+    // ---- epilogue.  In the accumulators a lane holds row l32 and, for column tile t and q = 0..3, the four
+    // consecutive columns 32*t + 8*q + 4*h + (0..3): stored from there, one instruction would touch 32 rows with 32
+    // bytes each.  Each wavefront turns its 32 x 64 block around in its own piece of LDS (the loop's buffers are free
+    // after the last barrier) so that a store instruction writes four rows of 256 contiguous bytes.
+    uint8_t *stage = lds + wave * (32 * kEStride);
+    const uint32_t n = n_out;
+    const void *outp = FUSED ? (const void *)p.y : (const void *)p.C;
+    const bool vec_ok = p.N % 4 == 0 && reinterpret_cast<uintptr_t>(outp) % 16 == 0;
 #pragma unroll
-    for (int t = 0; t < TN; ++t)
+    for (int b = 0; b < TM; ++b) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const uint32_t n = n0 + wave * 64 + t * 32 + q * 8 + h * 4;
-            float sc[4], zc[4], bs[4];
+        for (int t = 0; t < TN; ++t)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                *reinterpret_cast<v4i *>(stage + l32 * kEStride + (t * 32 + q * 8 + h * 4) * 4) =
+                    v4i{acc[t][b][q * 4], acc[t][b][q * 4 + 1], acc[t][b][q * 4 + 2], acc[t][b][q * 4 + 3]};
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+            const uint32_t row = it * 4 + r4;
+            const v4i a = *reinterpret_cast<const v4i *>(stage + row * kEStride + c16 * 16);
+            const uint32_t m = m0 + b * 32 + row;
+            if (m >= p.M || n >= p.N) continue;
             if (FUSED) {
+                const float sr = row_par[0][b * 32 + row], zr = row_par[1][b * 32 + row];
+                v4f32 v;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const uint32_t nn = min(n + r, p.N - 1);
-                    sc[r] = p.epi.s_col[nn];
-                    zc[r] = p.epi.z_col[nn];
-                    bs[r] = BIAS ? p.epi.bias[nn] : 0.f;
+                    float o = dequant_hprec_one(a[r], sr, zr, sc[r], zc[r]);
+                    if (BIAS) o = o + bs[r];
+                    v[r] = o;
                 }
-            }
-#pragma unroll
-            for (int b = 0; b < TM; ++b) {
-                const uint32_t m = m0 + b * 32 + l32;
-                if (m >= p.M || n >= p.N) continue;
-                if (FUSED) {
-                    const float sr = p.epi.s_row[m], zr = p.epi.z_row[m];
-                    v4f32 v;
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        float o = dequant_hprec_one(acc[t][b][q * 4 + r], sr, zr, sc[r], zc[r]);
-                        if (BIAS) o = o + bs[r];
-                        v[r] = o;
-                    }
-                    float *dst = p.y + (uint64_t)m * p.N + n;
-                    if (vec_ok && n + 3 < p.N) {
-                        *reinterpret_cast<v4f32 *>(dst) = v;
-                    } else {
-#pragma unroll
-                        for (int r = 0; r < 4; ++r)
-                            if (n + r < p.N) dst[r] = v[r];
-                    }
+                float *dst = p.y + (uint64_t)m * p.N + n;
+                if (vec_ok && n + 3 < p.N) {
+                    __builtin_nontemporal_store(v, reinterpret_cast<v4f32 *>(dst));
                 } else {
-                    int32_t *dst = p.C + (uint64_t)m * p.N + n;
-                    if (vec_ok && n + 3 < p.N) {
-                        *reinterpret_cast<v4i *>(dst) = v4i{acc[t][b][q * 4], acc[t][b][q * 4 + 1], acc[t][b][q * 4 + 2], acc[t][b][q * 4 + 3]};
-                    } else {
 #pragma unroll
-                        for (int r = 0; r < 4; ++r)
-                            if (n + r < p.N) dst[r] = acc[t][b][q * 4 + r];
-                    }
+                    for (int r = 0; r < 4; ++r)
+                        if (n + r < p.N) dst[r] = v[r];
+                }
+            } else {
+                int32_t *dst = p.C + (uint64_t)m * p.N + n;
+                if (vec_ok && n + 3 < p.N) {
+                    __builtin_nontemporal_store(a, reinterpret_cast<v4i *>(dst));
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (n + r < p.N) dst[r] = a[r];
                 }
             }
         }
-}
-
-template <bool FUSED, bool BIAS>
-static void launch_gemm8_variant(Gemm8Params &p, hipStream_t stream)
-{
-    p.tiles_n = (p.N + 255) / 256;
-    // 128-row tiles unless the problem is too small to give most CUs one (then 32-row tiles)
-    if (p.M > 64 && ((p.M + 127) / 128) * p.tiles_n >= 96) {
-        p.tiles_m = (p.M + 127) / 128;
-        hipLaunchKernelGGL((gemm_s8_kernel<4, FUSED, BIAS>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, stream, p);
-    } else {
-        p.tiles_m = (p.M + 31) / 32;
-        hipLaunchKernelGGL((gemm_s8_kernel<1, FUSED, BIAS>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, stream, p);
     }
 }
 
-int launch_gemm_s8(const int8_t *A, const int8_t *B, uint32_t M, uint32_t N, uint32_t K, int32_t *C, const float *s_row,
-                   const float *z_row, const float *s_col, const float *z_col, const float *bias, float *y,
-                   hipStream_t stream)
+template <bool FUSED, bool BIAS, bool TILED>
+static void launch_gemm8_variant(Gemm8Params &p, hipStream_t stream)
+{
+    p.tiles_n = (p.N + 255) / 256;
+    // the tallest tile that still gives most of the 256 CUs a workgroup
+    const uint32_t t128 = ((p.M + 127) / 128) * p.tiles_n, t64 = ((p.M + 63) / 64) * p.tiles_n;
+    if (p.M > 64 && t128 >= 160) {
+        p.tiles_m = (p.M + 127) / 128;
+        hipLaunchKernelGGL((gemm_s8_kernel<4, FUSED, BIAS, TILED>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, stream, p);
+    } else if (p.M > 32 && t64 >= 96) {
+        p.tiles_m = (p.M + 63) / 64;
+        hipLaunchKernelGGL((gemm_s8_kernel<2, FUSED, BIAS, TILED>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, stream, p);
+    } else {
+        p.tiles_m = (p.M + 31) / 32;
+        hipLaunchKernelGGL((gemm_s8_kernel<1, FUSED, BIAS, TILED>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, stream, p);
+    }
+}
+
+int launch_gemm_s8(const int8_t *A, const int8_t *B, bool b_tiled, uint32_t M, uint32_t N, uint32_t K, int32_t *C,
+                   const float *s_row, const float *z_row, const float *s_col, const float *z_col, const float *bias,
+                   float *y, hipStream_t stream)
 {
     if (M == 0 || N == 0) return 0;
     Gemm8Params p{A, B, M, N, K, C, y, Epi8{s_row, z_row, s_col, z_col, bias}, 0, 0};
     if (C)
-        launch_gemm8_variant<false, false>(p, stream);
+        launch_gemm8_variant<false, false, false>(p, stream);
+    else if (b_tiled && bias)
+        launch_gemm8_variant<true, true, true>(p, stream);
+    else if (b_tiled)
+        launch_gemm8_variant<true, false, true>(p, stream);
     else if (bias)
-        launch_gemm8_variant<true, true>(p, stream);
+        launch_gemm8_variant<true, true, false>(p, stream);
     else
-        launch_gemm8_variant<true, false>(p, stream);
+        launch_gemm8_variant<true, false, false>(p, stream);
+    return (int)hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------------
+// weight [N, K] row-major -> tiled: [ceil(N/32)][K/32][64 lanes][16 bytes], lane (r = lane % 32, h = lane / 32) of
+// tile (nt, ks) holding W[32*nt + r][32*ks + 16*h, +16) (zero past row N): each MFMA weight fragment is then one
+// contiguous kilobyte, eight cache lines per load instruction instead of thirty-two
+// ---------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void weight_tile8_kernel(const int8_t *w, uint32_t N, uint32_t K, int8_t *out)
+{
+    const uint32_t ksteps = K / 32;
+    const uint64_t pieces = (uint64_t)((N + 31) / 32) * ksteps * 64;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < pieces; i += (uint64_t)gridDim.x * blockDim.x) {
+        const uint32_t ln = (uint32_t)(i & 63u);
+        const uint64_t tile = i >> 6;
+        const uint32_t ks = (uint32_t)(tile % ksteps), nt = (uint32_t)(tile / ksteps);
+        const uint32_t row = nt * 32 + (ln & 31u), k = ks * 32 + (ln >> 5) * 16;
+        v4u v = {0u, 0u, 0u, 0u};
+        if (row < N) v = *reinterpret_cast<const v4u *>(w + (uint64_t)row * K + k);
+        reinterpret_cast<v4u *>(out)[i] = v;
+    }
+}
+
+int launch_weight_tile8(const int8_t *w, uint32_t N, uint32_t K, int8_t *out, hipStream_t stream)
+{
+    if (N == 0 || K == 0) return 0;
+    const uint64_t pieces = (uint64_t)((N + 31) / 32) * (K / 32) * 64;
+    const uint32_t blocks = (uint32_t)std::min<uint64_t>((pieces + 255) / 256, 1u << 20);
+    hipLaunchKernelGGL(weight_tile8_kernel, dim3(blocks), dim3(256), 0, stream, w, N, K, out);
     return (int)hipGetLastError();
 }
 

@@ -64,8 +64,10 @@ int launch_dequant_hprec(const int32_t *acc, const float *s_row, const float *z_
                          const float *z_col, const float *bias, uint32_t rows, uint32_t cols, float *x,
                          hipStream_t stream);
 // C != nullptr -> int32 accumulators [M,N]; else the float32 dequant (+ bias) fused into y.
-int launch_gemm_s8(const int8_t *A, const int8_t *B, uint32_t M, uint32_t N, uint32_t K, int32_t *C, const float *s_row,
-                   const float *z_row, const float *s_col, const float *z_col, const float *bias, float *y,
-                   hipStream_t stream);
+// b_tiled: B is the output of launch_weight_tile8 (fused form only).
+int launch_gemm_s8(const int8_t *A, const int8_t *B, bool b_tiled, uint32_t M, uint32_t N, uint32_t K, int32_t *C,
+                   const float *s_row, const float *z_row, const float *s_col, const float *z_col, const float *bias,
+                   float *y, hipStream_t stream);
+int launch_weight_tile8(const int8_t *w, uint32_t N, uint32_t K, int8_t *out, hipStream_t stream);
 
 }  // namespace duq

@@ -227,7 +227,11 @@ def quantize_asym_8bit(x):
     return _ops.quantize_rows_asym_8bit(x)
 
 
-def linear8bit_forward(xq, scales_x, zeros_x, weight, w_scale, w_zeros, bias=None):
-    """int8 GEMM + float32 dequant (+ bias) in one launch."""
+def weight_tile_8bit(weight):
+    return _ops.weight_tile_8bit(weight)
+
+
+def linear8bit_forward(xq, scales_x, zeros_x, weight, w_scale, w_zeros, bias=None, tiled_rows=None):
+    """int8 GEMM + float32 dequant (+ bias) in one launch; with ``tiled_rows`` = N, ``weight`` is the tiled copy."""
     assert xq.shape[-1] % 32 == 0, "A.shape[-1]: {} must be multiplication of 32".format(xq.shape[-1])
-    return _ops.linear8bit_forward(xq, scales_x, zeros_x, weight, w_scale, w_zeros, bias)
+    return _ops.linear8bit_forward(xq, scales_x, zeros_x, weight, w_scale, w_zeros, bias, tiled_rows)

@@ -272,6 +272,16 @@ int duq_linear8bit_forward(const int8_t *xq, const float *scale_x, const float *
                            const float *w_scale, const float *w_zeros, const float *bias, uint32_t M, uint32_t N,
                            uint32_t K, float *y, duq_stream_t stream);
 
+/* No counterpart in the reference: the same forward on a weight copy arranged for the MFMA operand layout.
+ * duq_weight_tile_8bit rewrites w [N,K] once into w_tiled, ceil(N/32)*32*K bytes (whole 32-row tiles, the
+ * last one zero-padded), in which the 64 x 16 bytes a wavefront loads for one MFMA are one contiguous
+ * kilobyte; duq_linear8bit_forward_tiled takes it in place of w and returns the same bits, faster (the
+ * row-major form touches four times as many cache lines per load).  K % 32 == 0; 16-byte alignment. */
+int duq_weight_tile_8bit(const int8_t *w, uint32_t N, uint32_t K, int8_t *w_tiled, duq_stream_t stream);
+int duq_linear8bit_forward_tiled(const int8_t *xq, const float *scale_x, const float *zeros_x, const int8_t *w_tiled,
+                                 const float *w_scale, const float *w_zeros, const float *bias, uint32_t M, uint32_t N,
+                                 uint32_t K, float *y, duq_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

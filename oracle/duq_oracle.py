@@ -658,6 +658,18 @@ def weight_asym8_from_linear(w):
     return q.astype(np.int8), scale.astype(_F32), zero
 
 
+def weight_tile_8bit(w):
+    """The library's tiled copy of an int8 weight [N, K] (K % 32 == 0; a storage format of the library, not of the
+    reference): [ceil(N/32)][K/32][h = 0..1][r = 0..31][16 bytes] holding W[32*nt + r][32*ks + 16*h + (0..15)],
+    rows past N zero; flat int8."""
+    w = np.asarray(w, np.int8)
+    n, k = w.shape
+    nt = -(-n // 32)
+    padded = np.zeros((nt * 32, k), np.int8)
+    padded[:n] = w
+    return padded.reshape(nt, 32, k // 32, 2, 16).transpose(0, 2, 3, 1, 4).reshape(-1).copy()
+
+
 def linear8bit_asq_forward(x, w_q, w_scales, w_zeros, bias=None):
     """LinearQuant8bitASQ.forward (linear.py:326-337) for float32 x [M,K]:
     returns (y float32, acc int32, q int8, scale, zeros)."""

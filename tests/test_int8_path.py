@@ -189,6 +189,23 @@ def test_linear8bit_forward_is_the_composition():
     assert y.dtype == F32 and y.shape == (9, 12)
 
 
+def test_weight_tile_layout_by_plain_loops():
+    rng = np.random.default_rng(8)
+    n, k = 40, 96
+    w = rng.integers(-128, 128, (n, k)).astype(np.int8)
+    got = orc.weight_tile_8bit(w)
+    assert got.dtype == np.int8 and got.size == 64 * k
+    want = np.zeros(64 * k, np.int8)
+    for nt in range(2):
+        for ks in range(k // 32):
+            for lane in range(64):
+                row, k0 = nt * 32 + lane % 32, ks * 32 + (lane // 32) * 16
+                if row < n:
+                    base = ((nt * (k // 32) + ks) * 64 + lane) * 16
+                    want[base:base + 16] = w[row, k0:k0 + 16]
+    assert np.array_equal(got, want)
+
+
 # ------------------------------------------------------------------ ABI (CPU, no compute)
 def test_abi_validation_8bit_entries():
     from duqlinear4bitcuda_amd import _lib
@@ -209,6 +226,13 @@ def test_abi_validation_8bit_entries():
     assert fwd(P, P, None, P, P, P, None, 4, 8, 32, P, None) == -1
     assert fwd(P, P, P, P, P, P, None, 4, 8, 32, None, None) == -1
     assert fwd(None, None, None, None, None, None, None, 4, 0, 32, None, None) == 0
+    tf = lib.duq_linear8bit_forward_tiled
+    assert tf(P, P, P, P, P, P, None, 4, 8, 40, P, None) == -3
+    assert tf(P, P, P, P + 4, P, P, None, 4, 8, 32, P, None) == -5
+    assert tf(P, P, P, P, None, P, None, 4, 8, 32, P, None) == -1
+    assert lib.duq_weight_tile_8bit(P, 8, 48, P, None) == -3
+    assert lib.duq_weight_tile_8bit(P, 8, 32, None, None) == -1
+    assert lib.duq_weight_tile_8bit(None, 0, 32, None, None) == 0
     assert lib.duq_asym_quant_host_8bit(P, P, None, 2, 8, P, None) == -1
     assert lib.duq_asym_quant_host_8bit(None, None, None, 0, 8, None, None) == 0
     assert lib.duq_asym_dequant_host_hprec(P, P, P, P, None, 2, 8, P, None) == -1
@@ -371,6 +395,12 @@ def test_gpu_linear8bit_forward(dev, hip, M, N, K, with_bias):
                                  None if bias is None else _t(bias, dev)).cpu().numpy()
     assert got.dtype == F32 and got.shape == (M, N)
     assert np.array_equal(got.view(np.uint32), y.view(np.uint32))
+    # the same launch on the tiled copy of the weight
+    wt = hip.weight_tile_8bit(_t(wq, dev))
+    assert np.array_equal(wt.cpu().numpy(), orc.weight_tile_8bit(wq))
+    got_t = hip.linear8bit_forward(gq, gs, gz, wt, _t(ws, dev), _t(wz, dev), None if bias is None else _t(bias, dev),
+                                   tiled_rows=N).cpu().numpy()
+    assert np.array_equal(got_t.view(np.uint32), y.view(np.uint32))
     # and the three separate steps of the reference give the same bits
     acc_g = hip.matmul_8bit(gq, _t(wq, dev))
     assert np.array_equal(acc_g.cpu().numpy(), acc)
@@ -407,7 +437,20 @@ def test_gpu_layer_8bit(dev):
     y = layer(xt)
     assert y.dtype == torch.float32 and tuple(y.shape) == (2, 37, N)
     assert np.array_equal(y.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    assert "weight_tiled" not in layer.state_dict() and layer._buffers["weight_tiled"].numel() == N * K
+    layer.tiled = False                       # the fused launch on the row-major weight
+    assert torch.equal(layer(xt), y)
     layer.fused = False                       # the reference's three steps
+    assert torch.equal(layer(xt), y)
+    layer.fused = layer.tiled = True
+    with torch.no_grad():                     # the tiled copy follows the weight
+        layer.weight[5, :] = 1
+    y_mod = layer(xt)
+    layer.tiled = False
+    assert torch.equal(layer(xt), y_mod) and not torch.equal(y_mod, y)
+    with torch.no_grad():
+        layer.weight.copy_(torch.from_numpy(wq))
+    layer.fused = False
     assert torch.equal(layer(xt), y)
     layer.quantizer.fused = False             # torch computes scale and zero, as in the reference
     assert torch.equal(layer(xt), y)
@@ -439,6 +482,7 @@ def test_gpu_8bit_full_size_properties(dev, hip):
     q, s, z = hip.quantize_rows_asym_8bit(x)
     assert int(q.min()) == 0 and int(q.max()) == 126
     y = hip.linear8bit_forward(q, s, z, wq, ws, wz, bias)
+    assert torch.equal(hip.linear8bit_forward(q, s, z, hip.weight_tile_8bit(wq), ws, wz, bias, tiled_rows=N), y)
     acc = hip.matmul_8bit(q, wq)
     y3 = hip.asym_dequant_hprec(acc, s.view(-1), z.view(-1), ws.view(-1), wz.view(-1)) + bias
     assert torch.equal(y, y3)
