@@ -217,7 +217,7 @@ def other_shapes_section(dev):
     return out
 
 
-def int8_layer_section(dev):
+def int8_layer_section(dev, quick=False):
     """The 8-bit asymmetric layer (LinearQuant8bitASQ) at the headline shape: float32 activations, quantizer
     launch + fused GEMM launch, float32 result; the GEMM alone against the dense int8 MFMA peak."""
     import torch
@@ -226,7 +226,7 @@ def int8_layer_section(dev):
     from duqlinear4bitcuda_amd.nn import LinearQuant8bitASQ
 
     out = []
-    for (M, K, N) in [(2048, 4096, 4096), (2048, 4096, 11008), (16, 4096, 4096)]:
+    for (M, K, N) in [(2048, 4096, 4096)] if quick else [(2048, 4096, 4096), (2048, 4096, 11008), (16, 4096, 4096)]:
         g = torch.Generator().manual_seed(6)
         x = torch.randn(M, K, generator=g).to(dev)
         layer = LinearQuant8bitASQ(K, N, bias=False).to(dev)
@@ -403,7 +403,7 @@ def main():
     quantizer = quantizer_section(dev)
     asym = None if args.quick else asym_section(dev)
     other = None if args.quick else other_shapes_section(dev)
-    int8_layer = None if args.quick else int8_layer_section(dev)
+    int8_layer = int8_layer_section(dev, args.quick)
     best_decode = max(decode, key=lambda d: d["GBps"])
     roofline_decode = {"bound": "hbm", "kernel": "gemv_s4_dot_kernel (M=1) / gemm_s4_skinny_kernel (2<=M<=16) / gemm_s4_ring_kernel (17<=M<=64, long rows)", "achieved": best_decode["GBps"],
                        "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": best_decode["frac_hbm"],
