@@ -257,6 +257,24 @@ def int8_layer_section(dev, quick=False):
                     "gemm_frac_of_int8_peak": round(ops / us_gemm / 1e6 / PEAK_INT8_TOPS, 4),
                     "gemm_algorithmic_GBps": round((M * K + N * K + M * N * 4) / us_gemm / 1e3, 1)})
         del layer, x
+    if quick:
+        return out
+    # decode: weights rotated over more than 512 MB of distinct buffers, as in decode_section
+    decode = []
+    for (M, K, N) in [(1, 4096, 4096), (16, 4096, 4096), (16, 4096, 11008), (32, 4096, 11008)]:
+        g = torch.Generator().manual_seed(7)
+        nbuf = int(600e6 // (N * K)) + 1
+        w0 = torch.randint(0, 128, (N, K), dtype=torch.int8, generator=g).to(dev)
+        tiled = [_HIP.weight_tile_8bit(torch.roll(w0, i, 0)) for i in range(nbuf)]
+        q = torch.randint(0, 127, (M, K), dtype=torch.int8, generator=g).to(dev)
+        sx, zx = torch.rand(M, 1, device=dev) + 0.1, torch.zeros(M, 1, device=dev)
+        sw, zw = torch.rand(N, 1, device=dev) * 0.01, torch.zeros(N, 1, device=dev)
+        us = graph_time_us([(lambda w=w: _HIP.linear8bit_forward(q, sx, zx, w, sw, zw, tiled_rows=N)) for w in tiled] * 2)
+        byts = M * K + N * K + 8 * N + 8 * M + 4 * M * N
+        decode.append({"M": M, "K": K, "N": N, "gemm_fused_us": round(us, 3), "GBps": round(byts / us / 1e3, 1),
+                       "frac_hbm": round(byts / us / 1e3 / PEAK_HBM_GBS, 4), "weight_buffers": nbuf})
+        del tiled, w0
+    out.append({"decode_rotated_weights": decode})
     return out
 
 

@@ -466,9 +466,129 @@ __global__ __launch_bounds__(256) void gemm_s8_kernel(Gemm8Params p)
     }
 }
 
+// ---------------------------------------------------------------------------------
+// skinny kernel (M <= 32): bound by reading the weight once from HBM
+// ---------------------------------------------------------------------------------
+// A workgroup owns 16 weight rows; its four wavefronts split K in contiguous quarters and meet in LDS at the end, so
+// N / 16 workgroups fill the chip at decode sizes.  v_mfma_i32_16x16x64_i8 with the weights on the "A" side: lane
+// (r = lane % 16, kb = lane / 16) holds 16 bytes of row r at k = 64*j + 16*kb for step j, from the row-major weight
+// (16 rows x 64 contiguous bytes per load) or from the tiled copy (four runs of 256 contiguous bytes per load).  The
+// activations (MT tiles of 16 rows) use the same layout on the "B" side, straight from global memory: they are
+// small and stay in L2.  A ring of kSkinnyRing steps per operand is in flight per lane and each register is
+// refetched right after its MFMA, so the whole K quarter of a 4096-long row is requested before the first MFMA.
+constexpr int kSkinnyRing = 16;
+
+template <int MT, bool FUSED, bool BIAS, bool TILED>
+__global__ __launch_bounds__(256) void gemm_s8_skinny_kernel(Gemm8Params p)
+{
+    __shared__ v4i part[4][MT][64];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u, wave = tid >> 6;
+    const uint32_t l16 = lane & 15u, kb = lane >> 4;
+    const uint32_t n0 = blockIdx.x * 16;
+    const uint32_t steps = (p.K + 63) / 64;
+    const uint32_t spw = (steps + 3) / 4;  // steps per wavefront
+    const uint32_t j0 = wave * spw;
+
+    // row-major: the descriptor covers this workgroup's rows (rows past N read as zero).  Tiled: it covers the 32-row
+    // tile (zero-padded past N) of which these 16 rows are the lower or upper half
+    const __amdgpu_buffer_rsrc_t rWt = TILED ? make_rsrc(p.B + (uint64_t)(n0 / 32) * 32 * p.K, 32u * p.K)
+                                             : make_rsrc(p.B + (uint64_t)n0 * p.K, min(p.N - n0, 16u) * p.K);
+    const __amdgpu_buffer_rsrc_t rX = make_rsrc(p.A, p.M * p.K);  // rows past M read as zero
+    const bool wrow_ok = n0 + l16 < p.N;
+    // byte offset of this lane's 16 bytes of step j: row-major  r*K + 64*j + 16*kb;
+    // tiled (step ks = 2*j + kb/2, half h = kb%2, row r + 16*(n0/16 % 2) of the tile)  ks*1024 + (h*32 + row)*16
+    const uint32_t wlane = TILED ? (kb >> 1) * 1024 + ((kb & 1u) * 32 + l16 + (n0 & 16u)) * 16 : l16 * p.K + kb * 16;
+    auto load_w = [&](uint32_t j) -> v4i {
+        const uint32_t k = j * 64 + kb * 16;
+        const bool ok = wrow_ok && j < j0 + spw && k < p.K;
+        return __builtin_bit_cast(v4i, buf_load16(rWt, ok ? wlane + (TILED ? j * 2048 : j * 64) : kOobOffset, 0));
+    };
+    auto load_x = [&](int mt, uint32_t j) -> v4i {
+        const uint32_t k = j * 64 + kb * 16;
+        const bool ok = j < j0 + spw && k < p.K;
+        return __builtin_bit_cast(v4i, buf_load16(rX, ok ? (mt * 16 + l16) * p.K + k : kOobOffset, 0));
+    };
+
+    v4i w[kSkinnyRing], x[MT][kSkinnyRing];
+#pragma unroll
+    for (int u = 0; u < kSkinnyRing; ++u) {
+        w[u] = load_w(j0 + u);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) x[mt][u] = load_x(mt, j0 + u);
+    }
+    v4i acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = v4i{0, 0, 0, 0};
+    for (uint32_t g = 0; g < spw; g += kSkinnyRing) {
+#pragma unroll
+        for (int u = 0; u < kSkinnyRing; ++u) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) acc[mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[u], x[mt][u], acc[mt], 0, 0, 0);
+            const uint32_t j = j0 + g + kSkinnyRing + u;  // past the wavefront's range: reads as zero
+            w[u] = load_w(j);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) x[mt][u] = load_x(mt, j);
+        }
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) part[wave][mt][lane] = acc[mt];
+    __syncthreads();
+    // lane (m = lane % 16, q = lane / 16) of tile mt holds C[mt*16 + m][n0 + 4*q + (0..3)]: MT * 64 threads finish
+    if (tid >= MT * 64) return;
+    const uint32_t mt = tid >> 6;
+    v4i sum = part[0][mt][lane];
+#pragma unroll
+    for (int w2 = 1; w2 < 4; ++w2) {
+        const v4i o = part[w2][mt][lane];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) sum[r] += o[r];
+    }
+    const uint32_t m = mt * 16 + l16, n = n0 + kb * 4;
+    if (m >= p.M || n >= p.N) return;
+    const void *outp = FUSED ? (const void *)p.y : (const void *)p.C;
+    const bool vec_ok = p.N % 4 == 0 && reinterpret_cast<uintptr_t>(outp) % 16 == 0 && n + 3 < p.N;
+    if (FUSED) {
+        const float sr = p.epi.s_row[m], zr = p.epi.z_row[m];
+        v4f32 v;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const uint32_t nn = min(n + r, p.N - 1);
+            float o = dequant_hprec_one(sum[r], sr, zr, p.epi.s_col[nn], p.epi.z_col[nn]);
+            if (BIAS) o = o + p.epi.bias[nn];
+            v[r] = o;
+        }
+        float *dst = p.y + (uint64_t)m * p.N + n;
+        if (vec_ok) {
+            *reinterpret_cast<v4f32 *>(dst) = v;
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (n + r < p.N) dst[r] = v[r];
+        }
+    } else {
+        int32_t *dst = p.C + (uint64_t)m * p.N + n;
+        if (vec_ok) {
+            *reinterpret_cast<v4i *>(dst) = sum;
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (n + r < p.N) dst[r] = sum[r];
+        }
+    }
+}
+
 template <bool FUSED, bool BIAS, bool TILED>
 static void launch_gemm8_variant(Gemm8Params &p, hipStream_t stream)
 {
+    if (p.M <= 32) {
+        const dim3 grid((p.N + 15) / 16);
+        if (p.M <= 16)
+            hipLaunchKernelGGL((gemm_s8_skinny_kernel<1, FUSED, BIAS, TILED>), grid, dim3(256), 0, stream, p);
+        else
+            hipLaunchKernelGGL((gemm_s8_skinny_kernel<2, FUSED, BIAS, TILED>), grid, dim3(256), 0, stream, p);
+        return;
+    }
     p.tiles_n = (p.N + 255) / 256;
     // the tallest tile that still gives most of the 256 CUs a workgroup
     const uint32_t t128 = ((p.M + 127) / 128) * p.tiles_n, t64 = ((p.M + 63) / 64) * p.tiles_n;

@@ -340,7 +340,9 @@ def test_gpu_fused_quantizer_8bit_matches_torch_ops(dev, hip):
     assert torch.equal(gq.view(300, 4096), hip.asym_quant_8bit(x, scale.view(-1), zeros.view(-1)))
 
 
-GEMM_SHAPES = [(1, 1, 32), (5, 7, 64), (32, 64, 96), (33, 250, 128), (100, 256, 160), (128, 260, 416),
+GEMM_SHAPES = [(1, 1, 32), (5, 7, 64), (32, 64, 96), (16, 16, 32), (9, 40, 96), (17, 250, 416), (32, 1030, 1056),
+               (3, 48, 8192), (16, 4096, 4096), (31, 300, 4128),   # skinny kernel: K split over four wavefronts
+ (33, 250, 128), (100, 256, 160), (128, 260, 416),
                (129, 512, 1024), (300, 100, 32), (64, 1024, 4096), (65, 300, 224),
                (1024, 3072, 256),   # 128-row tiles
                (1000, 3100, 288), (2048, 4096, 4096)]
@@ -375,7 +377,7 @@ def test_gpu_asym_dequant_hprec(dev, hip, rows, cols):
     assert got.dtype == F32 and np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
-FWD_SHAPES = [(1, 16, 32), (7, 33, 64), (40, 250, 160), (128, 512, 1024), (130, 1030, 416), (1024, 3072, 256),
+FWD_SHAPES = [(1, 16, 32), (7, 33, 64), (16, 48, 96), (17, 250, 416), (32, 1030, 1056), (4, 4096, 4096), (40, 250, 160), (128, 512, 1024), (130, 1030, 416), (1024, 3072, 256),
               (1000, 3102, 288)]
 
 
