@@ -1,6 +1,7 @@
 """Writes tests/golden/linear4bit_small.npz: seeded inputs and the expected packed codes,
 scales, int32 accumulators and fp16 outputs of the four Linear4bit forwards and of the row-sum
-(exact zero-point correction) forward.
+(exact zero-point correction) forward; and tests/golden/linear8bit_small.npz: the same for the
+8-bit asymmetric layer (float32 activations, int8 codes, float32 outputs).
 
 The reference ships no golden vectors for this path (its tests only print), so these come
 from the pinned CPU oracle; the file freezes them so that a later change of the oracle or
@@ -58,8 +59,27 @@ def main():
     y, acc, qx, sx, zx, rx = orc.linear4bit_asq_rowsum_forward(xa, wr, sr, zr, adj, bias)
     out.update(rs_w=wr, rs_sw=sr, rs_zw=zr, rs_adj=adj, rs_y=y, rs_acc=acc, rs_qx=qx, rs_sx=sx, rs_zx=zx, rs_rx=rx)
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "linear4bit_small.npz")
-    np.savez_compressed(path, **out)
-    print(path, os.path.getsize(path), "bytes")
+    if "--only-8bit" not in sys.argv:
+        np.savez_compressed(path, **out)
+        print(path, os.path.getsize(path), "bytes")
+
+    # 8-bit asymmetric layer: float32 activations with an offset, one constant and one all-positive token
+    g = torch.Generator().manual_seed(20248)
+    M, K, N = 20, 160, 40
+    x8 = torch.randn(M, K, generator=g) * 3 + 0.7
+    x8[2] = -2.25
+    x8[5] = x8[5].abs() + 1
+    x8 = x8.numpy()
+    w8 = (torch.randn(N, K, generator=g) * 0.05).numpy()
+    b8 = torch.randn(N, generator=g).numpy()
+    wq, ws, wz = orc.weight_asym8_from_linear(w8)
+    y, acc, q, sx, zx = orc.linear8bit_asq_forward(x8, wq, ws, wz, b8)
+    sx_cpu, zx_cpu = orc.asym8_scales_zeros(x8, device_division=False)
+    out8 = dict(x=x8, w_float=w8, bias=b8, w=wq, sw=ws, zw=wz, y=y, acc=acc.astype(np.int32), qx=q, sx=sx, zx=zx,
+                sx_quotient_form=sx_cpu, zx_quotient_form=zx_cpu, w_tiled=orc.weight_tile_8bit(wq))
+    path8 = os.path.join(os.path.dirname(os.path.abspath(__file__)), "linear8bit_small.npz")
+    np.savez_compressed(path8, **out8)
+    print(path8, os.path.getsize(path8), "bytes")
 
 
 if __name__ == "__main__":

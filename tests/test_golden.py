@@ -10,6 +10,7 @@ from oracle import duq_oracle as orc
 from tests import cases
 
 G = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "linear4bit_small.npz"))
+G8 = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "linear8bit_small.npz"))
 
 
 def same16(a, b):
@@ -97,3 +98,46 @@ def test_modules_reproduce_the_fixture(dev):
     p = r.quantizer(T("asym_x"))
     assert np.array_equal(p.quantized_x.cpu().numpy(), G["rs_qx"]) and np.array_equal(p.rowsum_x.cpu().numpy(), G["rs_rx"])
     assert same16(p.zeros_x.cpu().numpy(), G["rs_zx"])
+
+
+def same32(a, b):
+    a = np.asarray(a, np.float32)
+    b = np.asarray(b, np.float32)
+    return bool(((a.view(np.uint32) == b.view(np.uint32)) | (np.isnan(a) & np.isnan(b))).all())
+
+
+def test_oracle_reproduces_the_8bit_fixture():
+    wq, ws, wz = orc.weight_asym8_from_linear(G8["w_float"])
+    assert np.array_equal(wq, G8["w"]) and same32(ws, G8["sw"]) and same32(wz, G8["zw"])
+    y, acc, q, sx, zx = orc.linear8bit_asq_forward(G8["x"], G8["w"], G8["sw"], G8["zw"], G8["bias"])
+    assert np.array_equal(q, G8["qx"]) and np.array_equal(acc, G8["acc"])
+    assert same32(sx, G8["sx"]) and same32(zx, G8["zx"]) and same32(y, G8["y"])
+    assert np.array_equal(orc.weight_tile_8bit(G8["w"]), G8["w_tiled"])
+    # sanity of the data itself: accumulators are the plain integer product of the codes; code ranges; the constant
+    # token (-2.25) has scale 0, zero point 2.25 / 0 = +inf and codes INT_MIN + INT_MAX = -1 -> 0; the two forms of
+    # the scale differ somewhere
+    assert np.array_equal(G8["qx"].astype(np.int64) @ G8["w"].astype(np.int64).T, G8["acc"])
+    assert G8["qx"].min() == 0 and G8["qx"].max() == 126 and G8["w"].min() == 0 and G8["w"].max() == 127
+    assert float(G8["sx"][2, 0]) == 0.0 and np.isposinf(G8["zx"][2, 0]) and (G8["qx"][2] == 0).all()
+    assert float(G8["zx"][5, 0]) < 0                      # all-positive token: negative zero point
+    assert not same32(G8["sx"], G8["sx_quotient_form"])
+    assert np.allclose(G8["sx"], G8["sx_quotient_form"], rtol=2e-7, atol=0)
+
+
+@pytest.mark.gpu
+def test_8bit_layer_reproduces_the_fixture(dev):
+    from duqlinear4bitcuda_amd import _HIP
+    from duqlinear4bitcuda_amd import nn as qnn
+
+    T = lambda k: cases.t(G8[k], dev)
+    K, N = G8["x"].shape[1], G8["w"].shape[0]
+    layer = qnn.LinearQuant8bitASQ(K, N, bias=True).to(dev)
+    layer.load_state_dict({"weight": T("w"), "weight_scales": T("sw"), "weight_zeros": T("zw"), "bias": T("bias")})
+    p = layer.quantizer(T("x"))
+    assert np.array_equal(p.quantized_x.cpu().numpy(), G8["qx"])
+    assert same32(p.scales_x.cpu().numpy(), G8["sx"]) and same32(p.zeros_x.cpu().numpy(), G8["zx"])
+    assert np.array_equal(_HIP.matmul_8bit(p.quantized_x, layer.weight).cpu().numpy(), G8["acc"])
+    assert np.array_equal(_HIP.weight_tile_8bit(layer.weight).cpu().numpy(), G8["w_tiled"])
+    for fused, tiled in ((True, True), (True, False), (False, False)):
+        layer.fused, layer.tiled = fused, tiled
+        assert same32(layer(T("x")).cpu().numpy(), G8["y"])
