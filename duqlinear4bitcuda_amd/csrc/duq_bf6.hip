@@ -119,6 +119,9 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 #ifndef DUQ_BF6_COST256
 #define DUQ_BF6_COST256 1.78f
 #endif
+#ifndef DUQ_BF6_NARROW_MAX_TILES
+#define DUQ_BF6_NARROW_MAX_TILES 128
+#endif
 
 struct Bf6Params {
     const uint8_t *X;  // activation shadow
@@ -134,12 +137,14 @@ struct Bf6Params {
 // with at least one such tile per CU: the same weight traffic feeds twice the MFMAs, which takes the kernel off
 // the L2 -> CU limit that bounds the smaller tiles; all 256 AGPRs hold accumulators, an activation chunk is one
 // 128-k step (three buffers of two steps would not fit in LDS) and the epilogue parameters are fetched after the loop.
-template <int TMI, int EPI, bool BIAS>
+template <int TMI, int TNI, int EPI, bool BIAS>
 __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
 {
     static_assert(TMI == 16 || TMI == 8 || TMI == 4, "16-row MFMA tiles per wavefront along M");
-    constexpr int BM = 16 * TMI, BN = 256;
-    constexpr int TNI = 4;           // 16 x 16 MFMA tiles per wavefront along N: BM rows x 64 columns
+    // TNI = 16 x 16 MFMA tiles per wavefront along N: BM rows x 64 columns (TNI = 4), or BM x 32 (TNI = 2, with
+    // 64-row tiles only: twice the workgroups for problems that leave CUs without a 64 x 256 tile)
+    static_assert(TNI == 4 || (TNI == 2 && TMI == 4), "column tiles per wavefront");
+    constexpr int BM = 16 * TMI, BN = 64 * TNI;
     constexpr int CH = TMI == 16 ? 1 : 2;  // 128-k steps per activation chunk
     constexpr int NPH = 4 / CH;            // chunk bodies per turn of the weight ring
     // 16-byte activation pieces per thread and chunk: plane 0 (4*CH per row), plane 1 (2*CH per row)
@@ -149,7 +154,7 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
     constexpr uint32_t kP0Stride = 64 * CH + 16, kP1Stride = 32 * CH + 16;
     constexpr uint32_t kP1Base = BM * kP0Stride;
     constexpr uint32_t kBuf = BM * (kP0Stride + kP1Stride);
-    constexpr uint32_t kYStride = 144;  // bytes per staged output row: 128 + pad
+    constexpr uint32_t kYStride = 32 * TNI + 16;  // bytes per staged output row: 16*TNI binary16 + pad
     constexpr uint32_t kLds = 3 * kBuf > 4 * BM * kYStride ? 3 * kBuf : 4 * BM * kYStride;
     constexpr bool LATE_PARAMS = TMI == 16;
     constexpr int MODE = EPI;
@@ -180,9 +185,9 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
     uint32_t wv0[TNI], wv1[TNI];
 #pragma unroll
     for (int ni = 0; ni < TNI; ++ni) {
-        const bool ok = wave * 4 + ni < wtiles;
-        wv0[ni] = ok ? (wave * 4 + ni) * ksteps * 1536 + lane * 16 : kOobOffset;
-        wv1[ni] = ok ? (wave * 4 + ni) * ksteps * 1536 + 1024 + lane * 8 : kOobOffset;
+        const bool ok = wave * TNI + ni < wtiles;
+        wv0[ni] = ok ? (wave * TNI + ni) * ksteps * 1536 + lane * 16 : kOobOffset;
+        wv1[ni] = ok ? (wave * TNI + ni) * ksteps * 1536 + 1024 + lane * 8 : kOobOffset;
     }
     auto load_w0 = [&](v6i &dst, int ni, uint32_t g, __amdgpu_buffer_rsrc_t r) {
         const v4i a = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(r, (int)wv0[ni], (int)(g * 1536), 0));
@@ -280,7 +285,7 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
         for (int mi = 0; mi < TMI; ++mi) rowp[mi] = load_row<MODE>(e, min(m0 + mi * 16 + l16, p.M - 1));
 #pragma unroll
         for (int ni = 0; ni < TNI; ++ni) {
-            const uint32_t nq = min(n0 + wave * 64 + ni * 16 + kb * 4, p.N - 4);
+            const uint32_t nq = min(n0 + wave * (16 * TNI) + ni * 16 + kb * 4, p.N - 4);
             raw_s1[ni] = *reinterpret_cast<const v2u *>(e.s_col_1 + nq);
             if (MODE == 1 || MODE == 3 || MODE == 4) raw_z1[ni] = *reinterpret_cast<const v2u *>(e.z_col_1 + nq);
             if (MODE == 4) raw_rs[ni] = *reinterpret_cast<const v4i *>(e.rs_col + nq);
@@ -325,14 +330,25 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
                             read_x1(xf[nm & 3], buf, nm, ns % CH);
                     }
                     // refill the previous step's slot: eight loads over the step (step 0 fetches step 3 again)
-                    if (TMI == 8 && ni == 2) {
+                    if (TNI == 2 && mi < 2) {  // two fragments, four loads, with the first two row tiles
+                        if (ni == 0)
+                            load_w0(wf[prev][mi], mi, gprev, rG);
+                        else
+                            load_w1(wf[prev][mi], mi, gprev, rG);
+                    }
+                    if (TNI == 2 && s == 1 && mi >= 2) {  // three activation pieces per chunk: store, then refetch
+                        const int slot2 = (mi - 2) * 2 + ni;  // 0..3
+                        if (slot2 < NXP) *reinterpret_cast<v4u *>(lds + nx2 + xlds[slot2]) = xreg[slot2];
+                        if (slot2 >= 1 && slot2 <= NXP) load_x(xreg[slot2 - 1], slot2 - 1, c + 3, rXc);
+                    }
+                    if (TNI == 4 && TMI == 8 && ni == 2) {
                         if (mi & 1)
                             load_w1(wf[prev][mi >> 1], mi >> 1, gprev, rG);
                         else
                             load_w0(wf[prev][mi >> 1], mi >> 1, gprev, rG);
                     }
-                    if (TMI == 4 && ni == 2) load_w0(wf[prev][mi], mi, gprev, rG);
-                    if (TMI == 4 && ni == 3) load_w1(wf[prev][mi], mi, gprev, rG);
+                    if (TNI == 4 && TMI == 4 && ni == 2) load_w0(wf[prev][mi], mi, gprev, rG);
+                    if (TNI == 4 && TMI == 4 && ni == 3) load_w1(wf[prev][mi], mi, gprev, rG);
                     if (TMI == 16 && ni == 2 && (mi & 1) == 0) {
                         if (mi & 2)
                             load_w1(wf[prev][mi >> 2], mi >> 2, gprev, rG);
@@ -340,9 +356,10 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
                             load_w0(wf[prev][mi >> 2], mi >> 2, gprev, rG);
                     }
                     // chunk c+2 -> its LDS buffer and, one group (one slot) later, chunk c+3 into the freed register
-                    if (TMI <= 8 && s == 1 && mi < NXP && ni == (TMI == 8 ? 3 : 0))
+                    if (TNI == 4 && TMI <= 8 && s == 1 && mi < NXP && ni == (TMI == 8 ? 3 : 0))
                         *reinterpret_cast<v4u *>(lds + nx2 + xlds[mi]) = xreg[mi];
-                    if (TMI <= 8 && s == 1 && ni == 1 && mi >= 1 && mi <= NXP) load_x(xreg[mi - 1], mi - 1, c + 3, rXc);
+                    if (TNI == 4 && TMI <= 8 && s == 1 && ni == 1 && mi >= 1 && mi <= NXP)
+                        load_x(xreg[mi - 1], mi - 1, c + 3, rXc);
                     if (TMI == 16 && (mi & 1) == 1 && (mi >> 1) < NXP) {
                         if (ni == 2) *reinterpret_cast<v4u *>(lds + nx2 + xlds[mi >> 1]) = xreg[mi >> 1];
                         if (ni == 3) load_x(xreg[mi >> 1], mi >> 1, c + 3, rXc);
@@ -411,7 +428,7 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
 #pragma unroll
     for (int ni = 0; ni < TNI; ++ni) {
         const uint32_t ncol = ni * 16 + kb * 4;
-        const uint32_t nq = min(n0 + wave * 64 + ncol, p.N - 4);
+        const uint32_t nq = min(n0 + wave * (16 * TNI) + ncol, p.N - 4);
         const QuadCols<MODE, BIAS> cols =
             quad_cols_from_raw<MODE, BIAS>(raw_s1[ni], raw_z1[ni], raw_s2[ni], raw_z2[ni], raw_bias[ni], nq, raw_rs[ni]);
 #pragma unroll
@@ -423,25 +440,26 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
     }
     const uint32_t rows_here = min(p.M - m0, (uint32_t)BM);
     const __amdgpu_buffer_rsrc_t rY = make_rsrc(p.y + (uint64_t)m0 * p.N, rows_here * p.N * 2);
-    const uint32_t piece = lane & 7u, rsub = lane >> 3;
-    const uint32_t ncol0 = n0 + wave * 64 + piece * 8;
+    constexpr uint32_t PPR = 2 * TNI, RPI = 64 / PPR;  // 16-byte pieces per staged row, rows per store instruction
+    const uint32_t piece = lane % PPR, rsub = lane / PPR;
+    const uint32_t ncol0 = n0 + wave * (16 * TNI) + piece * 8;
 #pragma unroll
-    for (int it = 0; it < BM / 8; ++it) {
-        const uint32_t row = it * 8 + rsub;
+    for (int it = 0; it < BM / (int)RPI; ++it) {
+        const uint32_t row = it * RPI + rsub;
         const v4u v = *reinterpret_cast<const v4u *>(stage + row * kYStride + piece * 16);
         const uint32_t off = (row < rows_here && ncol0 < p.N) ? (row * p.N + ncol0) * 2 : kOobOffset;
         __builtin_amdgcn_raw_buffer_store_b128(v, rY, (int)off, 0, 0);
     }
 }
 
-template <int TMI, int EPI>
+template <int TMI, int TNI, int EPI>
 static void launch_tile(const Bf6Params &p, hipStream_t stream)
 {
     const dim3 grid(p.tiles_m * p.tiles_n);
     if (p.epi.bias)
-        hipLaunchKernelGGL((gemm_bf6_kernel<TMI, EPI, true>), grid, dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((gemm_bf6_kernel<TMI, TNI, EPI, true>), grid, dim3(256), 0, stream, p);
     else
-        hipLaunchKernelGGL((gemm_bf6_kernel<TMI, EPI, false>), grid, dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((gemm_bf6_kernel<TMI, TNI, EPI, false>), grid, dim3(256), 0, stream, p);
 }
 
 template <int EPI>
@@ -456,13 +474,20 @@ static void launch_mode(Bf6Params &p, hipStream_t stream)
                 c64 = kCost64 * (float)((t64 + 255) / 256);
     if (c256 < c128 && c256 <= c64) {
         p.tiles_m = (p.M + 255) / 256;
-        launch_tile<16, EPI>(p, stream);
+        launch_tile<16, 4, EPI>(p, stream);
     } else if (c64 < c128) {
         p.tiles_m = (p.M + 63) / 64;
-        launch_tile<4, EPI>(p, stream);
+        // CUs left without a 64 x 256 tile: 64 x 128 tiles, twice as many, as long as they still run in one round
+        // (measured: 23-35 % faster up to 128 tiles of 64 x 256, slower from 160 on)
+        if (t64 <= DUQ_BF6_NARROW_MAX_TILES) {
+            p.tiles_n = (p.N + 127) / 128;
+            launch_tile<4, 2, EPI>(p, stream);
+        } else {
+            launch_tile<4, 4, EPI>(p, stream);
+        }
     } else {
         p.tiles_m = (p.M + 127) / 128;
-        launch_tile<8, EPI>(p, stream);
+        launch_tile<8, 4, EPI>(p, stream);
     }
 }
 

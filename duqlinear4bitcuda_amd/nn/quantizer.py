@@ -27,7 +27,7 @@ class SymQuantizer(torch.nn.Module):
     clamp of the codes: 6 is what the reference's device kernel applies
     (include/common.h:53-54), 7 what its Python fake-quant path applies."""
 
-    def __init__(self, input_clip_ratio=1.0, qmax: int = 6, shadow=False, shadow_min_rows: int = 128):
+    def __init__(self, input_clip_ratio=1.0, qmax: int = 6, shadow=False, shadow_min_rows: int = 96):
         super().__init__()
         self.input_clip_ratio = input_clip_ratio
         self.qmax = qmax
@@ -57,7 +57,7 @@ class AsymQuantizer(torch.nn.Module):
     (quantizer.py:24-35).  ``input_clip_ratio`` is accepted and unused, as in the
     reference."""
 
-    def __init__(self, input_clip_ratio: float = 1.0, shifted: bool = False, shadow=False, shadow_min_rows: int = 128):
+    def __init__(self, input_clip_ratio: float = 1.0, shifted: bool = False, shadow=False, shadow_min_rows: int = 96):
         super().__init__()
         self.shadow = shadow                  # see SymQuantizer
         self.shadow_min_rows = shadow_min_rows

@@ -199,7 +199,9 @@ def _epi_inputs(rng, M, N):
 @pytest.mark.gpu
 @pytest.mark.parametrize("M,N,K", [(1, 16, 128), (128, 256, 128), (128, 256, 256), (100, 240, 640), (257, 512, 1024),
                                    (130, 80, 384), (300, 1008, 1152), (512, 4096, 4096), (64, 1024, 11008),
-                                   # enough tiles for the 128-row variant of the kernel (the ones above run 64-row tiles)
+                                   # more than 160 tiles of 64 x 256 (the ones above run 64 x 128 tiles): 64 x 256 tiles
+                                   (704, 4096, 512), (1000, 4096, 256), (900, 3000 - 8, 384),
+                                   # enough tiles for the 128-row variant of the kernel
                                    (2048 + 70, 4096 - 48, 384), (2048, 4096, 128),
                                    # ... and for the 256-row variant: one to seven steps (its loop turns every four), ragged edges
                                    (4096, 4096, 128), (4096 - 37, 4096 - 48, 384), (4096, 4096, 512), (4096, 4096 - 16, 896)])
