@@ -396,7 +396,7 @@ def main():
                             args.steps, args.warmup)
     quant_us = event_time_us(lambda: hip.quantize_rows_sym_bf6(x, with_q=False), args.steps, args.warmup)
     achieved = ops / gemm_us / 1e6
-    roofline = {"bound": "mfma", "kernel": "gemm_bf6_kernel<8,0,false> (fused GEMM + dequant on v_mfma_f32_16x16x128_f8f6f4, 128 x 256 tiles)",
+    roofline = {"bound": "mfma", "kernel": "gemm_bf6_kernel<8,4,0,false> (fused GEMM + dequant on v_mfma_f32_16x16x128_f8f6f4, 128 x 256 tiles)",
                 "achieved": round(achieved, 1), "peak": PEAK_FP6_TOPS, "unit": "TOP/s",
                 "frac": round(achieved / PEAK_FP6_TOPS, 4), "frac_of_int8_peak": round(achieved / PEAK_INT8_TOPS, 4),
                 "avg_kernel_us": round(gemm_us, 2),
