@@ -551,13 +551,22 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
 // wavefronts meet in LDS (double buffered: one barrier per tile).
 constexpr int kSkinnySegs = 8;  // 64-byte segments per wavefront = 128-bit weight loads in flight per lane
 
-template <int WAVES, int EPI, bool BIAS>
+
+template <int WAVES, bool LINES, int EPI, bool BIAS>
 __global__ __launch_bounds__(WAVES * 64) void gemm_s4_skinny_kernel(GemmParams p)
 {
     __shared__ v4i part[2][WAVES][64];
+    // Whole-line loads (LINES; 4-6 % faster from 512 column tiles on, slower on small problems, where the extra LDS
+    // hop is not hidden): a load instruction fetches 8 rows x 128 contiguous bytes instead of 16
+    // rows x 64 (half a cache line each); the wavefront turns the tile into the MFMA's lane layout through its own
+    // 8 KB of LDS (one 128-bit write and one 128-bit read per load; no barrier: the piece is private to the wavefront
+    // and a wavefront's LDS operations execute in order).  Slot s of a row's line holds its 16-byte piece
+    // s ^ ((row / 2) % 8), which makes the 16 rows x 16 bytes of a fragment read cover every bank once.
+    __shared__ __attribute__((aligned(16))) uint8_t turn[LINES ? WAVES * 8192 : 16];
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63u, wave = tid >> 6;
     const uint32_t l16 = lane & 15u, g = lane >> 4;
+    const uint32_t r8 = lane >> 3, j8 = lane & 7u;
     const uint32_t kbytes = p.K >> 1;
     const uint32_t segs = (kbytes + 63) / 64;
     const uint32_t seg0 = wave * kSkinnySegs;  // the launcher guarantees WAVES * kSkinnySegs >= segs
@@ -585,6 +594,17 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_s4_skinny_kernel(GemmParams p
     }
 
     auto load_tile = [&](uint32_t tile, v4u(&w)[kSkinnySegs]) {
+        if (LINES) {
+            // load u = 2 * line + half: rows 8 * half + r8 of the tile, slot j8 of line `line` of this wavefront's range
+#pragma unroll
+            for (int u = 0; u < kSkinnySegs; ++u) {
+                const uint32_t rt = (u & 1) * 8 + r8, row = tile * 16 + rt;
+                const uint32_t off = seg0 * 64 + (u >> 1) * 128 + ((j8 ^ ((rt >> 1) & 7u)) << 4);
+                const bool ok = tile < tile_end && row < p.N && off < kbytes;
+                w[u] = buf_load16(rW, ok ? row * kbytes + off : kOobOffset, 0);
+            }
+            return;
+        }
         const uint32_t row = tile * 16 + l16;
         const bool rok = tile < tile_end && row < p.N;
 #pragma unroll
@@ -593,10 +613,22 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_s4_skinny_kernel(GemmParams p
     };
     auto compute_tile = [&](uint32_t tile, const v4u(&w)[kSkinnySegs], uint32_t buf) {
         v4i acc = v4i{0, 0, 0, 0};
+        uint8_t *mine = turn + (LINES ? wave * 8192 : 0);
+        if (LINES) {
+#pragma unroll
+            for (int u = 0; u < kSkinnySegs; ++u) *reinterpret_cast<v4u *>(mine + u * 1024 + lane * 16) = w[u];
+        }
 #pragma unroll
         for (int u = 0; u < kSkinnySegs; ++u) {
             v4u we, wo;
-            expand_nibbles(w[u], we, wo);
+            v4u raw = w[u];
+            if (LINES) {
+                // segment u = 64 bytes: half (u % 2) of line u / 2; this lane's row l16 sits in load 2 * line + l16 / 8
+                const uint32_t piece = (u & 1) * 4 + g;
+                raw = *reinterpret_cast<const v4u *>(mine + ((u >> 1) * 2 + (l16 >> 3)) * 1024 + (l16 & 7u) * 128 +
+                                                     ((piece ^ ((l16 >> 1) & 7u)) << 4));
+            }
+            expand_nibbles(raw, we, wo);
             acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i, we), __builtin_bit_cast(v4i, xe[u]), acc,
                                                         0, 0, 0);
             acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i, wo), __builtin_bit_cast(v4i, xo[u]), acc,
@@ -939,14 +971,22 @@ static void launch_epi(GemmParams &p, hipStream_t stream)
         }
         p.tiles_m = tpw;
         const dim3 grid((ntiles + tpw - 1) / tpw);
-        if (segs <= 4 * kSkinnySegs)
-            hipLaunchKernelGGL((gemm_s4_skinny_kernel<4, EPI, BIAS>), grid, dim3(256), 0, stream, p);
-        else if (segs <= 8 * kSkinnySegs)
-            hipLaunchKernelGGL((gemm_s4_skinny_kernel<8, EPI, BIAS>), grid, dim3(512), 0, stream, p);
-        else if (segs <= 16 * kSkinnySegs)
-            hipLaunchKernelGGL((gemm_s4_skinny_kernel<16, EPI, BIAS>), grid, dim3(1024), 0, stream, p);
-        else
+        const bool lines = ntiles >= 512;  // whole-line weight loads turned through LDS
+        if (segs <= 4 * kSkinnySegs) {
+            if (lines)
+                hipLaunchKernelGGL((gemm_s4_skinny_kernel<4, true, EPI, BIAS>), grid, dim3(256), 0, stream, p);
+            else
+                hipLaunchKernelGGL((gemm_s4_skinny_kernel<4, false, EPI, BIAS>), grid, dim3(256), 0, stream, p);
+        } else if (segs <= 8 * kSkinnySegs) {
+            if (lines)
+                hipLaunchKernelGGL((gemm_s4_skinny_kernel<8, true, EPI, BIAS>), grid, dim3(512), 0, stream, p);
+            else
+                hipLaunchKernelGGL((gemm_s4_skinny_kernel<8, false, EPI, BIAS>), grid, dim3(512), 0, stream, p);
+        } else if (segs <= 16 * kSkinnySegs) {
+            hipLaunchKernelGGL((gemm_s4_skinny_kernel<16, false, EPI, BIAS>), grid, dim3(1024), 0, stream, p);
+        } else {
             goto tiles_path;  // K above 16384: the tile kernels take it
+        }
         return;
     }
 tiles_path:
