@@ -279,7 +279,8 @@ def int8_layer_section(dev, quick=False):
 
 
 def cpu_baseline(x_cpu, wq_cpu, sw_cpu, ops, budget_s=15.0):
-    """The reference's CPU fake-quant path (torch-CPU) on the same workload, host cores."""
+    """The reference's CPU fake-quant path (torch-CPU) on the same workload, host cores: whole forwards repeated for
+    about budget_s seconds."""
     import torch
 
     from oracle import fakequant_torch as fq
@@ -291,7 +292,7 @@ def cpu_baseline(x_cpu, wq_cpu, sw_cpu, ops, budget_s=15.0):
         fq.linear4bit_forward(x_cpu, wq_cpu, sw_cpu)
         reps += 1
         el = time.perf_counter() - t0
-        if el > budget_s or reps >= 50:
+        if el > budget_s or reps >= 400:
             break
     per = el / reps
     return {"value": round(ops / per / 1e12, 4), "unit": "TOPS", "cores": torch.get_num_threads(), "kind": "port",
