@@ -293,3 +293,70 @@ void duqo_add_bias(uint16_t *y, const uint16_t *bias, uint32_t rows, uint32_t co
     for (uint32_t r = 0; r < rows; ++r)
         for (uint32_t c = 0; c < cols; ++c) y[(size_t)r * cols + c] = hadd(y[(size_t)r * cols + c], bias[c]);
 }
+
+/* ---------------- 8-bit asymmetric layer (LinearQuant8bitASQ) ---------------- */
+
+/* qlinear4bit/nn/quantizer.py:47-51, float32.  device_division != 0: scale = (max - min) * float32(1/127), the form
+ * torch evaluates tensor / scalar in on a GPU; 0: the quotient (torch on a CPU). */
+void duqo_asym8_scales_zeros(const float *x, uint32_t rows, uint32_t cols, int device_division, float *scale, float *zero)
+{
+    const volatile float inv = 1.0f / 127.0f;
+    for (uint32_t r = 0; r < rows; ++r) {
+        float mn = INFINITY, mx = -INFINITY;
+        int nan = 0;
+        for (uint32_t c = 0; c < cols; ++c) {
+            float v = x[(size_t)r * cols + c];
+            if (v != v) nan = 1;
+            if (v < mn) mn = v;
+            if (v > mx) mx = v;
+        }
+        if (nan) mn = mx = NAN;
+        volatile float d = mx - mn;
+        volatile float s = device_division ? d * inv : d / 127.0f;
+        volatile float q = -mn / s;
+        scale[r] = s;
+        zero[r] = nearbyintf(q);
+    }
+}
+
+/* src/kernels/quant.cu:244-264: the float quotient and the float zero point are converted to binary16 on their way
+ * into __half2int_rn; the int add wraps; clamp to [0, 126] */
+void duqo_asym_quant_8bit(const float *x, const float *scale, const float *zeros, uint32_t rows, uint32_t cols, int8_t *q)
+{
+    for (uint32_t r = 0; r < rows; ++r) {
+        const int32_t zi = half_to_int_rn(duqo_f2h(zeros[r]));
+        for (uint32_t c = 0; c < cols; ++c) {
+            volatile float data = x[(size_t)r * cols + c] / scale[r];
+            const int32_t qi = half_to_int_rn(duqo_f2h(data));
+            const int32_t sum = (int32_t)((uint32_t)qi + (uint32_t)zi);
+            q[(size_t)r * cols + c] = (int8_t)clampi(sum, 0, 126);
+        }
+    }
+}
+
+/* src/kernels/gemm.cu:46-81: A [M,K] x B [N,K]^T, int32 accumulation (wrapping) */
+void duqo_matmul_s8(const int8_t *A, const int8_t *B, uint32_t M, uint32_t N, uint32_t K, int32_t *C)
+{
+#pragma omp parallel for
+    for (uint32_t m = 0; m < M; ++m)
+        for (uint32_t n = 0; n < N; ++n) {
+            uint32_t acc = 0;
+            for (uint32_t k = 0; k < K; ++k)
+                acc += (uint32_t)((int32_t)A[(size_t)m * K + k] * (int32_t)B[(size_t)n * K + k]);
+            C[(size_t)m * N + n] = (int32_t)acc;
+        }
+}
+
+/* src/kernels/quant.cu:283-299: float32, one rounding per operator */
+void duqo_asym_dequant_hprec(const int32_t *q, const float *scale_row, const float *zeros_row, const float *scale_col,
+                             const float *zeros_col, uint32_t rows, uint32_t cols, float *x)
+{
+    for (uint32_t r = 0; r < rows; ++r)
+        for (uint32_t c = 0; c < cols; ++c) {
+            volatile float e = (float)q[(size_t)r * cols + c];
+            volatile float scales = scale_row[r] * scale_col[c];
+            volatile float zeros = zeros_row[r] + zeros_col[c];
+            volatile float t = e - zeros;
+            x[(size_t)r * cols + c] = scales * t;
+        }
+}

@@ -163,3 +163,44 @@ def add_bias(y, bias):
     rows, cols = y.shape
     lib().duqo_add_bias(_p(y), _p(bias), _u32(rows), _u32(cols))
     return y
+
+
+# ---- 8-bit asymmetric layer ------------------------------------------------------------------
+
+def _f32(a):
+    return np.ascontiguousarray(np.asarray(a, dtype=np.float32))
+
+
+def asym8_scales_zeros(x, device_division=True):
+    x = _f32(x)
+    rows, cols = x.shape
+    s = np.empty((rows, 1), np.float32)
+    z = np.empty((rows, 1), np.float32)
+    lib().duqo_asym8_scales_zeros(_p(x), _u32(rows), _u32(cols), ctypes.c_int(1 if device_division else 0), _p(s), _p(z))
+    return s, z
+
+
+def asym_quant_8bit(x, scale, zeros):
+    x = _f32(x)
+    scale, zeros = _f32(scale).reshape(-1), _f32(zeros).reshape(-1)
+    rows, cols = x.shape
+    q = np.empty((rows, cols), np.int8)
+    lib().duqo_asym_quant_8bit(_p(x), _p(scale), _p(zeros), _u32(rows), _u32(cols), _p(q))
+    return q
+
+
+def matmul_s8(a, b):
+    a = np.ascontiguousarray(a, dtype=np.int8)
+    b = np.ascontiguousarray(b, dtype=np.int8)
+    c = np.empty((a.shape[0], b.shape[0]), np.int32)
+    lib().duqo_matmul_s8(_p(a), _p(b), _u32(a.shape[0]), _u32(b.shape[0]), _u32(a.shape[1]), _p(c))
+    return c
+
+
+def asym_dequant_hprec(acc, sr, zr, sc, zc):
+    acc = np.ascontiguousarray(acc, dtype=np.int32)
+    sr, zr, sc, zc = (_f32(v).reshape(-1) for v in (sr, zr, sc, zc))
+    rows, cols = acc.shape
+    y = np.empty((rows, cols), np.float32)
+    lib().duqo_asym_dequant_hprec(_p(acc), _p(sr), _p(zr), _p(sc), _p(zc), _u32(rows), _u32(cols), _p(y))
+    return y

@@ -206,6 +206,34 @@ def test_weight_tile_layout_by_plain_loops():
     assert np.array_equal(got, want)
 
 
+def test_c_oracle_agrees_with_numpy_oracle_8bit():
+    """The plain-C restatement (own binary16 conversion, scalar float arithmetic) against the NumPy one."""
+    from oracle import duq_oracle_c as orc_c
+    rng = np.random.default_rng(9)
+    x = (rng.standard_normal((40, 257)) * rng.uniform(0.01, 30, (40, 1))).astype(F32)
+    x[3, 5] = np.nan
+    x[4, :] = 2.5
+    x[5, 7] = np.inf
+    x[6, :] = np.abs(x[6, :]) + 1
+    for dev_div in (True, False):
+        s, z = orc.asym8_scales_zeros(x, device_division=dev_div)
+        sc, zc = orc_c.asym8_scales_zeros(x, dev_div)
+        assert np.array_equal(s, sc, equal_nan=True) and np.array_equal(z, zc, equal_nan=True)
+    s, z = orc.asym8_scales_zeros(x)
+    s[7, 0], z[8, 0], z[9, 0] = 3e-39, 2049.0, -70000.0
+    assert np.array_equal(orc_c.asym_quant_8bit(x, s, z), orc.asym_quant_8bit(x, s, z))
+    a = rng.integers(-128, 128, (17, 96)).astype(np.int8)
+    b = rng.integers(-128, 128, (23, 96)).astype(np.int8)
+    assert np.array_equal(orc_c.matmul_s8(a, b), orc.matmul_s8(a, b))
+    big = np.full((1, 1 << 17), -128, np.int8)
+    assert int(orc_c.matmul_s8(big, big)[0, 0]) == -(1 << 31)
+    acc = rng.integers(-2 ** 31, 2 ** 31, (17, 23)).astype(np.int32)
+    sr, zr = rng.uniform(1e-3, 1, 17).astype(F32), np.rint(rng.uniform(-100, 126, 17)).astype(F32)
+    scl, zcl = rng.uniform(1e-4, 0.1, 23).astype(F32), np.rint(rng.uniform(-100, 100, 23)).astype(F32)
+    got, want = orc_c.asym_dequant_hprec(acc, sr, zr, scl, zcl), orc.asym_dequant_hprec(acc, sr, zr, scl, zcl)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
 # ------------------------------------------------------------------ ABI (CPU, no compute)
 def test_abi_validation_8bit_entries():
     from duqlinear4bitcuda_amd import _lib
