@@ -372,6 +372,7 @@ GEMM_SHAPES = [(1, 1, 32), (5, 7, 64), (32, 64, 96), (16, 16, 32), (9, 40, 96), 
                (3, 48, 8192), (16, 4096, 4096), (31, 300, 4128),   # skinny kernel: K split over four wavefronts
  (33, 250, 128), (100, 256, 160), (128, 260, 416),
                (129, 512, 1024), (300, 100, 32), (64, 1024, 4096), (65, 300, 224),
+               (3, 40, 66560), (40, 300, 33280), (70, 260, 65600),   # long rows
                (1024, 3072, 256),   # 128-row tiles
                (1000, 3100, 288), (2048, 4096, 4096)]
 
