@@ -460,7 +460,7 @@ EPI_ASYM_ROWSUM = 4
 
 
 def weight_shadow_bf6(w: torch.Tensor) -> torch.Tensor:
-    """E3M2 shadow of packed-int4 weights ``w`` uint8 [N, K/2]: uint8 [N, 3K/4] in the
+    """E3M2 shadow of packed-int4 weights ``w`` uint8 [N, K/2]: uint8 [ceil(N/32)*32, 3K/4] in the
     library's tile order.  Made once per weight tensor.  N % 16 == 0, K % 128 == 0."""
     name = "weight_shadow_bf6"
     if not isinstance(w, torch.Tensor):
@@ -469,7 +469,7 @@ def weight_shadow_bf6(w: torch.Tensor) -> torch.Tensor:
     if w.dim() != 2:
         raise RuntimeError(f"{name}: expected a 2-D tensor, got {tuple(w.shape)}")
     N, kb = w.shape
-    out = torch.empty((N, kb * 3 // 2), dtype=_U8, device=w.device)
+    out = torch.empty(((N + 31) // 32 * 32, kb * 3 // 2), dtype=_U8, device=w.device)
     st = _launch(w.device, _lib.load().duq_weight_shadow_bf6, w.data_ptr(), N, kb * 2, out.data_ptr())
     if st:
         _lib.check(st, name)
@@ -495,7 +495,8 @@ def activation_shadow_bf6(xq: torch.Tensor) -> torch.Tensor:
 def linear4bit_forward_bf6(mode, x_bf6, scale_x, zeros_x, w_bf6, w_scale_1, w_zeros_1=None, w_scale_2=None,
                            w_zeros_2=None, bias=None, rowsum_x=None, w_rowsum_adj=None):
     """``linear4bit_forward`` (modes 0-3) or ``linear4bit_forward_rowsum`` (mode 4) on E3M2
-    shadows: ``x_bf6`` uint8 [..., 3K/4], ``w_bf6`` uint8 [N, 3K/4].  Bit-identical results."""
+    shadows: ``x_bf6`` uint8 [..., 3K/4], ``w_bf6`` uint8 [ceil(N/32)*32, 3K/4] from weight_shadow_bf6, N taken
+    from ``w_scale_1``.  Bit-identical results."""
     name = "linear4bit_forward_bf6"
     if not isinstance(x_bf6, torch.Tensor) or not isinstance(w_bf6, torch.Tensor):
         raise RuntimeError(f"{name}: x_bf6 and w_bf6 must be tensors")
@@ -508,7 +509,12 @@ def linear4bit_forward_bf6(mode, x_bf6, scale_x, zeros_x, w_bf6, w_scale_1, w_ze
     if kb % 96:
         raise RuntimeError(f"{name}: shadow rows must hold a multiple of 128 elements (96 bytes), got {kb} bytes")
     M = x_bf6.numel() // kb if kb else 0
-    N = w_bf6.shape[0]
+    if not isinstance(w_scale_1, torch.Tensor):
+        raise RuntimeError(f"{name}: w_scale_1 is not a tensor")
+    N = w_scale_1.numel()
+    if w_bf6.shape[0] != (N + 31) // 32 * 32:
+        raise RuntimeError(f"{name}: the weight shadow has {w_bf6.shape[0]} rows, expected {(N + 31) // 32 * 32} for "
+                           f"{N} output channels")
     ptrs = []
     for t, what, dt, n in ((scale_x, "scale_x", _F16, M), (zeros_x, "zeros_x", _F16, M), (rowsum_x, "rowsum_x", _I32, M),
                            (w_scale_1, "w_scale_1", _F16, N), (w_zeros_1, "w_zeros_1", _F16, N),

@@ -12,15 +12,15 @@
 // v_cvt_scalef32_pk32_bf6_f16 writes them; it is kept as a 16-byte part and an 8-byte part
 // so that every load is naturally aligned.
 //   activation shadow  [M][K/32 x 16 B | K/32 x 8 B]      (row-major, two planes per row)
-//   weight shadow      [N/16][K/128][64 lanes x 16 B | 64 lanes x 8 B]
-//                      lane l of a (16-row tile, 128-k step) holds the block of row l % 16,
-//                      k-block l / 16: the fragment order of the MFMA, so a wavefront load is
-//                      one contiguous 1 KB (512 B) span and lands in the six registers of the
-//                      fragment without a move.  (A variant with three 128-bit loads per two
-//                      fragments moved fewer instructions through the memory pipeline but cost
-//                      two register moves per fragment and ran no faster: the loop is bound by
-//                      the issue rate of its one wavefront per SIMD.)
-// K % 128 == 0 and N % 16 == 0: no padding anywhere.
+//   weight shadow      [ceil(N/32)][K/128][3][64 lanes x 16 B]
+//                      lane l of a (pair of 16-row tiles, 128-k step) holds the blocks of row l % 16,
+//                      k-block l / 16 of either tile: 12 dwords [tile 2p | tile 2p+1], cut into three
+//                      16-byte pieces; piece r of all lanes is one contiguous kilobyte.  Three 128-bit
+//                      loads bring the two MFMA operands into twelve consecutive registers, which the
+//                      kernel pins (mfma_pinned) so that the loads write them in place: three memory
+//                      instructions per two fragments instead of four (a 128-bit and a 64-bit load per
+//                      fragment), without a register move.  An odd last tile is paired with zeros.
+// K % 128 == 0 and N % 16 == 0.
 //
 // Kernel: tile 128 (M) x 256 (N) per workgroup, 4 wavefronts side by side along N (128 x 64
 // each: 8 x 4 MFMA tiles, 128 accumulator registers).  Weights go global -> registers (a ring
@@ -36,6 +36,7 @@ namespace duq {
 
 typedef int v2i __attribute__((ext_vector_type(2)));
 typedef int v6i __attribute__((ext_vector_type(6)));
+typedef int v12i __attribute__((ext_vector_type(12)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef _Float16 v32h __attribute__((ext_vector_type(32)));
 
@@ -57,25 +58,36 @@ __device__ __forceinline__ v6i bf6_block_from_nibbles(const v4u w)
     return __builtin_bit_cast(v6i, __builtin_amdgcn_cvt_scalef32_pk32_bf6_f16(f, 1.0f));
 }
 
+// Layout: for every pair of 16-row tiles and every 128-k step, 3072 bytes.  Lane l = (row l % 16, k-block l / 16) owns
+// one block (24 bytes = 6 dwords) of either tile; its 12 dwords [tile 2p | tile 2p+1] are cut into three 16-byte
+// pieces, and piece r of all 64 lanes forms run r (1 KB): three 128-bit loads bring two MFMA operands into twelve
+// consecutive registers.  An odd last tile is paired with zeros.
 __global__ __launch_bounds__(256) void weight_shadow_kernel(const uint8_t *w, uint32_t N, uint32_t K, uint8_t *out)
 {
-    const uint32_t ksteps = K / 128;
-    const uint64_t total = (uint64_t)(N / 16) * ksteps * 64;
+    const uint32_t ksteps = K / 128, tiles = N / 16;
+    const uint64_t total = (uint64_t)((tiles + 1) / 2) * ksteps * 64;
     for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (uint64_t)gridDim.x * blockDim.x) {
         const uint32_t lane = (uint32_t)(i & 63u);
-        const uint64_t ts = i >> 6;  // tile * ksteps + step
-        const uint32_t step = (uint32_t)(ts % ksteps), tile = (uint32_t)(ts / ksteps);
-        const uint32_t n = tile * 16 + (lane & 15u), kb = step * 4 + (lane >> 4);
-        const v6i b = bf6_block_from_nibbles(*reinterpret_cast<const v4u *>(w + (uint64_t)n * (K / 2) + kb * 16));
-        uint8_t *dst = out + ts * 1536;
-        *reinterpret_cast<v4i *>(dst + lane * 16) = v4i{b[0], b[1], b[2], b[3]};
-        *reinterpret_cast<v2i *>(dst + 1024 + lane * 8) = v2i{b[4], b[5]};
+        const uint64_t ps = i >> 6;  // pair * ksteps + step
+        const uint32_t step = (uint32_t)(ps % ksteps), pair = (uint32_t)(ps / ksteps);
+        const uint32_t kb = step * 4 + (lane >> 4);
+        v6i f[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const uint32_t tile = pair * 2 + h, n = tile * 16 + (lane & 15u);
+            f[h] = v6i{0, 0, 0, 0, 0, 0};
+            if (tile < tiles) f[h] = bf6_block_from_nibbles(*reinterpret_cast<const v4u *>(w + (uint64_t)n * (K / 2) + kb * 16));
+        }
+        uint8_t *dst = out + ps * 3072 + lane * 16;
+        *reinterpret_cast<v4i *>(dst) = v4i{f[0][0], f[0][1], f[0][2], f[0][3]};
+        *reinterpret_cast<v4i *>(dst + 1024) = v4i{f[0][4], f[0][5], f[1][0], f[1][1]};
+        *reinterpret_cast<v4i *>(dst + 2048) = v4i{f[1][2], f[1][3], f[1][4], f[1][5]};
     }
 }
 
 int launch_weight_shadow_bf6(const uint8_t *w, uint32_t N, uint32_t K, uint8_t *out, hipStream_t stream)
 {
-    const uint64_t total = (uint64_t)(N / 16) * (K / 128) * 64;
+    const uint64_t total = (uint64_t)((N / 16 + 1) / 2) * (K / 128) * 64;
     if (total == 0) return 0;
     const uint32_t blocks = (uint32_t)std::min<uint64_t>((total + 255) / 256, 1u << 16);
     hipLaunchKernelGGL(weight_shadow_kernel, dim3(blocks), dim3(256), 0, stream, w, N, K, out);
@@ -122,6 +134,76 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 #ifndef DUQ_BF6_NARROW_MAX_TILES
 #define DUQ_BF6_NARROW_MAX_TILES 128
 #endif
+
+// One MFMA on half h (0: registers 0..5, 1: registers 6..11) of weight pair tuple t, which lives in the twelve
+// registers v[128 + 12*t .. 139 + 12*t].  Naming the registers pins the tuple, so that the three 128-bit loads that
+// fill it write them in place and the two operands are its halves: no register moves, which an opaque MFMA would
+// need wait states behind (a "v" operand cannot name half of a tuple).  t and h are constants after unrolling; the
+// switch folds to one statement.
+#define DUQ_PIN(T, A0, A1, B0, B1)                                                                                     \
+    case 2 * T:                                                                                                       \
+        asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, v[" #A0 ":" #A1 "], %1, %0 cbsz:3 blgp:3"                        \
+                     : "+a"(acc)                                                                                       \
+                     : "v"(x), "{v[" #A0 ":" #B1 "]}"(w));                                                             \
+        break;                                                                                                        \
+    case 2 * T + 1:                                                                                                   \
+        asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, v[" #B0 ":" #B1 "], %1, %0 cbsz:3 blgp:3"                        \
+                     : "+a"(acc)                                                                                       \
+                     : "v"(x), "{v[" #A0 ":" #B1 "]}"(w));                                                             \
+        break;
+// BASE: first register of the ring (chosen per kernel variant so that the ring ends where the variant's register
+// count ends: the tuples are pinned, everything else is the compiler's).
+template <int BASE>
+__device__ __forceinline__ void mfma_pinned(int t, int h, v4f &acc, const v12i &w, const v6i &x)
+{
+    static_assert(BASE == 64 || BASE == 96 || BASE == 128 || BASE == 160, "ring base registers with a table below");
+    if (BASE == 64) {  // 4 tuples (64 x 128 tiles)
+        switch (2 * t + h) {
+        DUQ_PIN(0, 64, 69, 70, 75)
+        DUQ_PIN(1, 76, 81, 82, 87)
+        DUQ_PIN(2, 88, 93, 94, 99)
+        DUQ_PIN(3, 100, 105, 106, 111)
+        default: __builtin_unreachable();
+        }
+    } else if (BASE == 96) {
+        switch (2 * t + h) {
+        DUQ_PIN(0, 96, 101, 102, 107)
+        DUQ_PIN(1, 108, 113, 114, 119)
+        DUQ_PIN(2, 120, 125, 126, 131)
+        DUQ_PIN(3, 132, 137, 138, 143)
+        DUQ_PIN(4, 144, 149, 150, 155)
+        DUQ_PIN(5, 156, 161, 162, 167)
+        DUQ_PIN(6, 168, 173, 174, 179)
+        DUQ_PIN(7, 180, 185, 186, 191)
+        default: __builtin_unreachable();
+        }
+    } else if (BASE == 128) {
+        switch (2 * t + h) {
+        DUQ_PIN(0, 128, 133, 134, 139)
+        DUQ_PIN(1, 140, 145, 146, 151)
+        DUQ_PIN(2, 152, 157, 158, 163)
+        DUQ_PIN(3, 164, 169, 170, 175)
+        DUQ_PIN(4, 176, 181, 182, 187)
+        DUQ_PIN(5, 188, 193, 194, 199)
+        DUQ_PIN(6, 200, 205, 206, 211)
+        DUQ_PIN(7, 212, 217, 218, 223)
+        default: __builtin_unreachable();
+        }
+    } else {
+        switch (2 * t + h) {
+        DUQ_PIN(0, 160, 165, 166, 171)
+        DUQ_PIN(1, 172, 177, 178, 183)
+        DUQ_PIN(2, 184, 189, 190, 195)
+        DUQ_PIN(3, 196, 201, 202, 207)
+        DUQ_PIN(4, 208, 213, 214, 219)
+        DUQ_PIN(5, 220, 225, 226, 231)
+        DUQ_PIN(6, 232, 237, 238, 243)
+        DUQ_PIN(7, 244, 249, 250, 255)
+        default: __builtin_unreachable();
+        }
+    }
+}
+#undef DUQ_PIN
 
 struct Bf6Params {
     const uint8_t *X;  // activation shadow
@@ -172,30 +254,28 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
     const uint32_t ksteps = p.K / 128;
     const uint32_t nchunks = (ksteps + CH - 1) / CH;
 
-    const uint32_t wtiles = min(p.N - n0, (uint32_t)BN) / 16;
+    const uint32_t wpairs = (min(p.N - n0, (uint32_t)BN) / 16 + 1) / 2;  // pairs of 16-row weight tiles in this tile
     const __amdgpu_buffer_rsrc_t rW =
-        make_rsrc(p.W + (uint64_t)(n0 / 16) * ksteps * 1536, wtiles * ksteps * 1536);
+        make_rsrc(p.W + (uint64_t)(n0 / 32) * ksteps * 3072, wpairs * ksteps * 3072);
     const __amdgpu_buffer_rsrc_t rX =
         make_rsrc(p.X + (uint64_t)m0 * row_bytes, min(p.M - m0, (uint32_t)BM) * row_bytes);
     const __amdgpu_buffer_rsrc_t rNone = make_rsrc(p.X, 0);  // every read returns zero
 
-    // weight fragment (ni, step g): 1536 bytes at ((wave*4 + ni) * ksteps + g) * 1536, a 16-byte and an 8-byte
-    // part per lane.  The scalar offset is not part of the hardware range check: tiles past N sit in the
-    // vector offset, steps past K switch to the empty descriptor.
-    uint32_t wv0[TNI], wv1[TNI];
+    // weight fragments (2*pi, 2*pi + 1) of step g: 3072 bytes at ((wave*NP + pi) * ksteps + g) * 3072, three 16-byte
+    // parts per lane (12 consecutive registers: two MFMA operands).  The scalar offset is not part of the hardware
+    // range check: pairs past N sit in the vector offset, steps past K switch to the empty descriptor.
+    constexpr int NP = TNI / 2;
+    constexpr int kRingBase = TNI == 2 ? 64 : (TMI == 16 ? 160 : (TMI == 4 ? 96 : 128));
+    uint32_t wv[NP];
 #pragma unroll
-    for (int ni = 0; ni < TNI; ++ni) {
-        const bool ok = wave * TNI + ni < wtiles;
-        wv0[ni] = ok ? (wave * TNI + ni) * ksteps * 1536 + lane * 16 : kOobOffset;
-        wv1[ni] = ok ? (wave * TNI + ni) * ksteps * 1536 + 1024 + lane * 8 : kOobOffset;
-    }
-    auto load_w0 = [&](v6i &dst, int ni, uint32_t g, __amdgpu_buffer_rsrc_t r) {
-        const v4i a = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(r, (int)wv0[ni], (int)(g * 1536), 0));
-        dst[0] = a[0], dst[1] = a[1], dst[2] = a[2], dst[3] = a[3];
-    };
-    auto load_w1 = [&](v6i &dst, int ni, uint32_t g, __amdgpu_buffer_rsrc_t r) {
-        const v2i b = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(r, (int)wv1[ni], (int)(g * 1536), 0));
-        dst[4] = b[0], dst[5] = b[1];
+    for (int pi = 0; pi < NP; ++pi)
+        wv[pi] = wave * NP + pi < wpairs ? (wave * NP + pi) * ksteps * 3072 + lane * 16 : kOobOffset;
+    // part 0..2 of the pair's twelve registers
+    auto load_w = [&](v12i &dst, int pi, int part, uint32_t g, __amdgpu_buffer_rsrc_t r) {
+        const v4i a = __builtin_bit_cast(
+            v4i, __builtin_amdgcn_raw_buffer_load_b128(r, (int)(wv[pi] == kOobOffset ? kOobOffset : wv[pi] + part * 1024),
+                                                       (int)(g * 3072), 0));
+        dst[4 * part + 0] = a[0], dst[4 * part + 1] = a[1], dst[4 * part + 2] = a[2], dst[4 * part + 3] = a[3];
     };
 
     // activation pieces of a chunk (256 k = 8 blocks): NX0 of plane 0 and NX1 of plane 1 per thread
@@ -222,7 +302,7 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
     // fragment of rows mi*16 + l16, k-step s of a chunk: plane 0 + mi*16*kP0Stride + s*64, plane 1 + ... + s*32
     const uint32_t frag0 = l16 * kP0Stride + kb * 16, frag1 = kP1Base + l16 * kP1Stride + kb * 8;
 
-    v6i wf[4][TNI];   // weight fragments [ring slot][column tile]
+    v12i wf[4][NP];   // weight fragment pairs [ring slot][pair of column tiles], pinned to v[kRingBase + 12 * (slot * NP + pi) ..]
     v6i xf[4];        // activation fragments, ring over mi
     v4u xreg[NXP];
     v4f acc[TMI][TNI];
@@ -248,19 +328,17 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
 #pragma unroll
     for (int j = 0; j < NXP; ++j) load_x(xreg[j], j, 0, rX);
 #pragma unroll
-    for (int ni = 0; ni < TNI; ++ni) {
-        load_w0(wf[0][ni], ni, 0, rW);
-        load_w1(wf[0][ni], ni, 0, rW);
-    }
+    for (int pi = 0; pi < NP; ++pi)
+#pragma unroll
+        for (int part = 0; part < 3; ++part) load_w(wf[0][pi], pi, part, 0, rW);
 #pragma unroll
     for (int j = 0; j < NXP; ++j) load_x(x1[j], j, 1, 1 < nchunks ? rX : rNone);
 #pragma unroll
     for (int g = 1; g < 4; ++g)
 #pragma unroll
-        for (int ni = 0; ni < TNI; ++ni) {
-            load_w0(wf[g][ni], ni, g, (uint32_t)g < ksteps ? rW : rNone);
-            load_w1(wf[g][ni], ni, g, (uint32_t)g < ksteps ? rW : rNone);
-        }
+        for (int pi = 0; pi < NP; ++pi)
+#pragma unroll
+            for (int part = 0; part < 3; ++part) load_w(wf[g][pi], pi, part, g, (uint32_t)g < ksteps ? rW : rNone);
 #pragma unroll
     for (int j = 0; j < NXP; ++j) *reinterpret_cast<v4u *>(lds + xlds[j]) = xreg[j];
 #pragma unroll
@@ -316,9 +394,7 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
                     // The operands are written by loads only (the compiler waits for those).  A register move
                     // placed right in front of this opaque statement would need wait states the compiler
                     // cannot know of; the generated loop has none, and the bit-exact parity tests would show one.
-                    asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 cbsz:3 blgp:3"
-                                 : "+a"(acc[mi][ni])
-                                 : "v"(wf[slot][ni]), "v"(xf[mi & 3]));
+                    mfma_pinned<kRingBase>(slot * NP + ni / 2, ni & 1, acc[mi][ni], wf[slot][ni / 2], xf[mi & 3]);
                     __builtin_amdgcn_sched_barrier(0);
                     // ---- side work in the shadow of this MFMA
                     if (ni < 2) {  // activation fragment two groups ahead
@@ -329,31 +405,19 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
                         else
                             read_x1(xf[nm & 3], buf, nm, ns % CH);
                     }
-                    // refill the previous step's slot: eight loads over the step (step 0 fetches step 3 again)
-                    if (TNI == 2 && mi < 2) {  // two fragments, four loads, with the first two row tiles
-                        if (ni == 0)
-                            load_w0(wf[prev][mi], mi, gprev, rG);
-                        else
-                            load_w1(wf[prev][mi], mi, gprev, rG);
+                    // refill the previous step's slot: 3 * NP loads over the step (step 0 fetches step 3 again)
+                    {
+                        int widx = -1;  // which of the 3 * NP loads rides with this MFMA
+                        if (TNI == 2) widx = mi < 2 ? mi * 2 + ni : -1;
+                        if (TNI == 4 && TMI == 8) widx = ni == 2 ? mi : -1;
+                        if (TNI == 4 && TMI == 4) widx = ni >= 2 ? mi * 2 + (ni - 2) : -1;
+                        if (TNI == 4 && TMI == 16) widx = (ni == 2 && (mi & 1) == 0) ? mi / 2 : -1;
+                        if (widx >= 0 && widx < 3 * NP) load_w(wf[prev][widx / 3], widx / 3, widx % 3, gprev, rG);
                     }
                     if (TNI == 2 && s == 1 && mi >= 2) {  // three activation pieces per chunk: store, then refetch
                         const int slot2 = (mi - 2) * 2 + ni;  // 0..3
                         if (slot2 < NXP) *reinterpret_cast<v4u *>(lds + nx2 + xlds[slot2]) = xreg[slot2];
                         if (slot2 >= 1 && slot2 <= NXP) load_x(xreg[slot2 - 1], slot2 - 1, c + 3, rXc);
-                    }
-                    if (TNI == 4 && TMI == 8 && ni == 2) {
-                        if (mi & 1)
-                            load_w1(wf[prev][mi >> 1], mi >> 1, gprev, rG);
-                        else
-                            load_w0(wf[prev][mi >> 1], mi >> 1, gprev, rG);
-                    }
-                    if (TNI == 4 && TMI == 4 && ni == 2) load_w0(wf[prev][mi], mi, gprev, rG);
-                    if (TNI == 4 && TMI == 4 && ni == 3) load_w1(wf[prev][mi], mi, gprev, rG);
-                    if (TMI == 16 && ni == 2 && (mi & 1) == 0) {
-                        if (mi & 2)
-                            load_w1(wf[prev][mi >> 2], mi >> 2, gprev, rG);
-                        else
-                            load_w0(wf[prev][mi >> 2], mi >> 2, gprev, rG);
                     }
                     // chunk c+2 -> its LDS buffer and, one group (one slot) later, chunk c+3 into the freed register
                     if (TNI == 4 && TMI <= 8 && s == 1 && mi < NXP && ni == (TMI == 8 ? 3 : 0))

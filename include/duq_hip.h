@@ -209,7 +209,7 @@ int duq_asym_rowsum_dequant_host(const int32_t *q, const duq_half *scale_row, co
  * MFMA for 6-bit floats, which runs at twice the rate of the 8-bit integer one, returns the
  * integer GEMM bit for bit.  The operands are shadows of the packed-int4 tensors, 3/4 byte per
  * element, in a layout private to the library:
- *   duq_weight_shadow_bf6      w    [N,K/2] -> w_bf6 [N*K*3/4 bytes], once per weight tensor
+ *   duq_weight_shadow_bf6      w    [N,K/2] -> w_bf6 [ceil(N/32)*32*K*3/4 bytes], once per weight tensor
  *   duq_activation_shadow_bf6  xq   [M,K/2] -> x_bf6 [M*K*3/4 bytes] (the *_bf6 quantizers
  *                              below write it directly)
  * duq_linear4bit_forward_bf6 takes the shadows in place of xq and w, and otherwise the

@@ -213,12 +213,12 @@ public:
 };
 
 namespace detail {
-// E3M2 shadow of packed weights [N, K/2] -> [N, 3K/4] (N % 16 == 0, K % 128 == 0)
+// E3M2 shadow of packed weights [N, K/2] -> [ceil(N/32)*32, 3K/4] (N % 16 == 0, K % 128 == 0)
 inline torch::Tensor weight_shadow(const torch::Tensor &weight)
 {
     check_device_tensor(weight, "weight_shadow", "weight");
     const uint32_t N = weight.size(0), K = weight.size(1) * 2;
-    auto out = torch::empty({N, K * 3 / 4}, torch::dtype(torch::kUInt8).device(weight.device()));
+    auto out = torch::empty({(N + 31) / 32 * 32, K * 3 / 4}, torch::dtype(torch::kUInt8).device(weight.device()));
     check_status(duq_weight_shadow_bf6(weight.data_ptr<uint8_t>(), N, K, out.data_ptr<uint8_t>(), current_stream(weight)),
                  "weight_shadow");
     return out;
@@ -240,7 +240,8 @@ inline torch::Tensor fused_forward_shadow(int mode, const PackedQuantizedTensor 
     check_device_tensor(A, "Linear4bit::forward", "shadow_x");
     TORCH_CHECK(A.device() == w_shadow.device(), "Linear4bit::forward: operands on different devices");
     TORCH_CHECK(w_shadow.size(1) == A.size(1), "Linear4bit::forward: shadow row length differs");
-    const uint32_t M = A.size(0), N = w_shadow.size(0), K = A.size(1) * 4 / 3;
+    const uint32_t M = A.size(0), N = s1.numel(), K = A.size(1) * 4 / 3;
+    TORCH_CHECK(w_shadow.size(0) == (N + 31) / 32 * 32, "Linear4bit::forward: weight shadow rows do not match the scales");
     auto scale_row = input.scale.contiguous().view(-1);
     TORCH_CHECK(scale_row.size(0) == M, "Linear4bit::forward: one activation scale per token expected");
     auto y = torch::empty({M, N}, torch::dtype(torch::kHalf).device(A.device()));

@@ -556,18 +556,21 @@ def activation_shadow_bf6(q_packed):
 
 
 def weight_shadow_bf6(w_packed):
-    """uint8 [N, K/2] -> uint8 [N, 3K/4] in tile order.  For every 16-row tile and every 128-k
-    step, lane l = (row l % 16, k-block l // 16) owns one block; the 1536 bytes of the
-    (tile, step) are 64 lanes x bytes 0-15 of their blocks, then 64 lanes x bytes 16-23.
-    N % 16 == 0, K % 128 == 0."""
+    """uint8 [N, K/2] -> uint8 [ceil(N/32)*32, 3K/4] in tile-pair order.  For every pair of 16-row tiles and every
+    128-k step, lane l = (row l % 16, k-block l // 16) owns one 24-byte block of either tile; the lane's 48 bytes
+    [tile 2p | tile 2p+1] are cut into three 16-byte pieces and the 3072 bytes of the (pair, step) are piece 0 of
+    the 64 lanes, then piece 1, then piece 2.  An odd last tile is paired with zeros.  N % 16 == 0, K % 128 == 0."""
     v = unpack_i4(w_packed, signed=True)
     N, K = v.shape
+    tiles = N // 16
+    pairs = (tiles + 1) // 2
     blocks = shadow_block_pack(v.reshape(N, K // 32, 32))  # [N, K/32, 24]
-    b = blocks.reshape(N // 16, 16, K // 128, 4, 24)       # tile, row, step, kb, byte
-    b = b.transpose(0, 2, 3, 1, 4).reshape(N // 16, K // 128, 64, 24)  # tile, step, lane = kb*16 + row, byte
-    out = np.concatenate([b[..., :16].reshape(N // 16, K // 128, 1024), b[..., 16:].reshape(N // 16, K // 128, 512)],
-                         axis=-1)
-    return np.ascontiguousarray(out).reshape(N, K * 3 // 4)
+    padded = np.zeros((pairs * 32, K // 32, 24), np.uint8)
+    padded[:N] = blocks
+    b = padded.reshape(pairs, 2, 16, K // 128, 4, 24)       # pair, half, row, step, kb, byte
+    b = b.transpose(0, 3, 4, 2, 1, 5).reshape(pairs, K // 128, 64, 48)  # pair, step, lane = kb*16 + row, [half 0 | half 1]
+    out = b.reshape(pairs, K // 128, 64, 3, 16).transpose(0, 1, 3, 2, 4)  # pair, step, piece, lane, byte
+    return np.ascontiguousarray(out).reshape(pairs * 32, K * 3 // 4)
 
 
 # ----------------------------------------------------------------------------------

@@ -86,25 +86,34 @@ def _loop_activation_shadow(q):
 def _loop_weight_shadow(q):
     v = orc.unpack_i4(q, signed=True)
     N, K = v.shape
-    out = np.zeros(N * K * 3 // 4, np.uint8)
+    pairs = (N // 16 + 1) // 2
+    out = np.zeros(pairs * 32 * K * 3 // 4, np.uint8)
     ksteps = K // 128
-    for tile in range(N // 16):
+    for pair in range(pairs):
         for step in range(ksteps):
-            base = (tile * ksteps + step) * 1536
+            base = (pair * ksteps + step) * 3072
             for lane in range(64):
                 row, kb = lane % 16, lane // 16
                 k0 = step * 128 + kb * 32
-                blk = orc.shadow_block_pack(v[tile * 16 + row, k0:k0 + 32])
-                out[base + lane * 16:base + lane * 16 + 16] = blk[:16]
-                out[base + 1024 + lane * 8:base + 1024 + lane * 8 + 8] = blk[16:]
-    return out.reshape(N, K * 3 // 4)
+                both = np.zeros(48, np.uint8)      # the lane's twelve dwords: tile 2*pair, then tile 2*pair + 1
+                for half in range(2):
+                    n = (2 * pair + half) * 16 + row
+                    if n < N:
+                        both[24 * half:24 * half + 24] = orc.shadow_block_pack(v[n, k0:k0 + 32])
+                for piece in range(3):
+                    at = base + piece * 1024 + lane * 16
+                    out[at:at + 16] = both[16 * piece:16 * piece + 16]
+    return out.reshape(pairs * 32, K * 3 // 4)
 
 
 def test_shadow_layouts_against_plain_loops():
     rng = np.random.default_rng(2)
     q = rng.integers(0, 256, (5, 128), dtype=np.uint8)       # M = 5, K = 256
     assert np.array_equal(orc.activation_shadow_bf6(q), _loop_activation_shadow(q))
-    w = rng.integers(0, 256, (48, 192), dtype=np.uint8)      # N = 48, K = 384
+    w = rng.integers(0, 256, (48, 192), dtype=np.uint8)      # N = 48 (an odd number of 16-row tiles), K = 384
+    assert np.array_equal(orc.weight_shadow_bf6(w), _loop_weight_shadow(w))
+    assert orc.weight_shadow_bf6(w).shape == (64, 288)
+    w = rng.integers(0, 256, (64, 64), dtype=np.uint8)       # N = 64, K = 128
     assert np.array_equal(orc.weight_shadow_bf6(w), _loop_weight_shadow(w))
 
 
