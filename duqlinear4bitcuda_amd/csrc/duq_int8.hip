@@ -242,18 +242,21 @@ struct Gemm8Params {
 
 __device__ __forceinline__ void lds_barrier8() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-template <int TM, bool FUSED, bool BIAS, bool TILED>
+template <int TM, int TN, bool FUSED, bool BIAS, bool TILED>
 __global__ __launch_bounds__(256) void gemm_s8_kernel(Gemm8Params p)
 {
     static_assert(TM == 4 || TM == 2 || TM == 1, "32-row MFMA tiles per wavefront along M");
-    constexpr int BM = 32 * TM, BN = 256, TN = 2;
+    // TN = 32-column MFMA tiles per wavefront: tiles of 256 columns (TN = 2), or of 128 (TN = 1, with 64-row tiles:
+    // twice the workgroups for problems that leave CUs without a 64 x 256 tile)
+    static_assert(TN == 2 || (TN == 1 && TM == 2), "column tiles per wavefront");
+    constexpr int BM = 32 * TM, BN = 128 * TN;
     constexpr int NS = 8;                 // steps (of 32 k) per chunk
     constexpr uint32_t kChunk = 32 * NS;  // 256
     constexpr uint32_t kStride = kChunk + 16;
     constexpr uint32_t kBuf = BM * kStride;
     constexpr int NXP = BM / 16;          // 16-byte activation pieces per thread and chunk: 8, 4, 2
 
-    constexpr uint32_t kEStride = 64 * 4 + 16;  // epilogue staging: 32 rows of 64 int32 per wavefront
+    constexpr uint32_t kEStride = 32 * TN * 4 + 16;  // epilogue staging: 32 rows of 32*TN int32 per wavefront
     constexpr uint32_t kLds = 3 * kBuf > 4 * 32 * kEStride ? 3 * kBuf : 4 * 32 * kEStride;
 
     __shared__ __attribute__((aligned(16))) uint8_t lds[kLds];
@@ -277,7 +280,7 @@ __global__ __launch_bounds__(256) void gemm_s8_kernel(Gemm8Params p)
     uint32_t wrow[TN];
 #pragma unroll
     for (int t = 0; t < TN; ++t)
-        wrow[t] = TILED ? (wave * 64 + t * 32) * p.K + lane * 16 : (wave * 64 + t * 32 + l32) * p.K + h * 16;
+        wrow[t] = TILED ? (wave * (32 * TN) + t * 32) * p.K + lane * 16 : (wave * (32 * TN) + t * 32 + l32) * p.K + h * 16;
     auto load_w = [&](int t, int s, uint32_t c) -> v4i {
         const uint32_t k = c * kChunk + s * 32;  // + h*16 < K  <=>  k < K
         // tiled: the fragment of (tile, step) is 1 KB in lane order, steps one after the other
@@ -314,8 +317,9 @@ __global__ __launch_bounds__(256) void gemm_s8_kernel(Gemm8Params p)
             for (int r = 0; r < 16; ++r) acc[t][b][r] = 0;
 
     // ---- epilogue parameters first: their latency disappears behind the loop
-    const uint32_t c16 = lane & 15u, r4 = lane >> 4;
-    const uint32_t n_out = n0 + wave * 64 + c16 * 4;  // first of the four output columns this lane stores
+    constexpr uint32_t kLanesPerRow = 8 * TN, kRowsPerStore = 64 / kLanesPerRow;  // a staged row is 128 * TN bytes
+    const uint32_t c16 = lane % kLanesPerRow, r4 = lane / kLanesPerRow;
+    const uint32_t n_out = n0 + wave * (32 * TN) + c16 * 4;  // first of the four output columns this lane stores
     float sc[4], zc[4], bs[4];
     if (FUSED) {
         if (tid < BM) {
@@ -347,8 +351,8 @@ __global__ __launch_bounds__(256) void gemm_s8_kernel(Gemm8Params p)
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
             if (TM == 1) {
-                wreg[w][0][s] = load_w(0, s, w);
-                wreg[w][1][s] = load_w(1, s, w);
+#pragma unroll
+                for (int t = 0; t < TN; ++t) wreg[w][t][s] = load_w(t, s, w);
             }
             if (w == WR - 1) {
 #pragma unroll
@@ -356,8 +360,8 @@ __global__ __launch_bounds__(256) void gemm_s8_kernel(Gemm8Params p)
                     if (j * NS / NXP == s) xreg[j] = load_x(j, 2);
             }
             if (TM != 1) {
-                wreg[w][0][s] = load_w(0, s, w);
-                wreg[w][1][s] = load_w(1, s, w);
+#pragma unroll
+                for (int t = 0; t < TN; ++t) wreg[w][t][s] = load_w(t, s, w);
             }
         }
     }
@@ -383,7 +387,7 @@ __global__ __launch_bounds__(256) void gemm_s8_kernel(Gemm8Params p)
                         fx[(s + 1) & 1][b] = s + 1 < NS ? read_x(cur, b, s + 1) : read_x(nxt, b, 0);
                     if (b == TM - 1)  // last use of this step's weight register: refetch it for the next chunk
                         wreg[W][t][s] = load_w(t, s, c + WR);
-                    if (t == 1 && b == 0) {  // activation pieces: chunk c+2 -> its LDS buffer, then fetch chunk c+3
+                    if (t == TN - 1 && b == 0) {  // activation pieces: chunk c+2 -> its LDS buffer, then fetch chunk c+3
 #pragma unroll
                         for (int j = 0; j < NXP; ++j)
                             if (j * NS / NXP == s) {
@@ -416,7 +420,7 @@ __global__ __launch_bounds__(256) void gemm_s8_kernel(Gemm8Params p)
     // ---- epilogue.  In the accumulators a lane holds row l32 and, for column tile t and q = 0..3, the four
     // consecutive columns 32*t + 8*q + 4*h + (0..3): stored from there, one instruction would touch 32 rows with 32
     // bytes each.  Each wavefront turns its 32 x 64 block around in its own piece of LDS (the loop's buffers are free
-    // after the last barrier) so that a store instruction writes four rows of 256 contiguous bytes.
+    // after the last barrier) so that a store instruction writes whole rows of 256 (128) contiguous bytes.
     uint8_t *stage = lds + wave * (32 * kEStride);
     const uint32_t n = n_out;
     const void *outp = FUSED ? (const void *)p.y : (const void *)p.C;
@@ -430,8 +434,8 @@ __global__ __launch_bounds__(256) void gemm_s8_kernel(Gemm8Params p)
                 *reinterpret_cast<v4i *>(stage + l32 * kEStride + (t * 32 + q * 8 + h * 4) * 4) =
                     v4i{acc[t][b][q * 4], acc[t][b][q * 4 + 1], acc[t][b][q * 4 + 2], acc[t][b][q * 4 + 3]};
 #pragma unroll
-        for (int it = 0; it < 8; ++it) {
-            const uint32_t row = it * 4 + r4;
+        for (int it = 0; it < 32 / (int)kRowsPerStore; ++it) {
+            const uint32_t row = it * kRowsPerStore + r4;
             const v4i a = *reinterpret_cast<const v4i *>(stage + row * kEStride + c16 * 16);
             const uint32_t m = m0 + b * 32 + row;
             if (m >= p.M || n >= p.N) continue;
@@ -594,13 +598,20 @@ static void launch_gemm8_variant(Gemm8Params &p, hipStream_t stream)
     const uint32_t t128 = ((p.M + 127) / 128) * p.tiles_n, t64 = ((p.M + 63) / 64) * p.tiles_n;
     if (p.M > 64 && t128 >= 160) {
         p.tiles_m = (p.M + 127) / 128;
-        hipLaunchKernelGGL((gemm_s8_kernel<4, FUSED, BIAS, TILED>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, stream, p);
-    } else if (p.M > 32 && t64 >= 96) {
+        hipLaunchKernelGGL((gemm_s8_kernel<4, 2, FUSED, BIAS, TILED>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, stream, p);
+    } else if (p.M > 32 && t64 >= 48) {
         p.tiles_m = (p.M + 63) / 64;
-        hipLaunchKernelGGL((gemm_s8_kernel<2, FUSED, BIAS, TILED>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, stream, p);
+        // one round of 64 x 256 tiles would leave CUs idle: 64 x 128 tiles, twice as many (measured 21-24 % faster at
+        // 128 such tiles, 9 % at 64)
+        if (t64 <= 128) {
+            p.tiles_n = (p.N + 127) / 128;
+            hipLaunchKernelGGL((gemm_s8_kernel<2, 1, FUSED, BIAS, TILED>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, stream, p);
+        } else {
+            hipLaunchKernelGGL((gemm_s8_kernel<2, 2, FUSED, BIAS, TILED>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, stream, p);
+        }
     } else {
         p.tiles_m = (p.M + 31) / 32;
-        hipLaunchKernelGGL((gemm_s8_kernel<1, FUSED, BIAS, TILED>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((gemm_s8_kernel<1, 2, FUSED, BIAS, TILED>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, stream, p);
     }
 }
 

@@ -373,7 +373,8 @@ GEMM_SHAPES = [(1, 1, 32), (5, 7, 64), (32, 64, 96), (16, 16, 32), (9, 40, 96), 
  (33, 250, 128), (100, 256, 160), (128, 260, 416),
                (129, 512, 1024), (300, 100, 32), (64, 1024, 4096), (65, 300, 224),
                (3, 40, 66560), (40, 300, 33280), (70, 260, 65600),   # long rows
-               (1024, 3072, 256),   # 128-row tiles
+               (512, 4096, 256), (300, 3100, 288), (200, 3990, 96),   # 64 x 128 tiles (48..128 tiles of 64 x 256)
+               (1024, 3072, 256),   # 64 x 256 tiles
                (1000, 3100, 288), (2048, 4096, 4096)]
 
 
@@ -406,7 +407,7 @@ def test_gpu_asym_dequant_hprec(dev, hip, rows, cols):
     assert got.dtype == F32 and np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
-FWD_SHAPES = [(1, 16, 32), (7, 33, 64), (16, 48, 96), (17, 250, 416), (32, 1030, 1056), (4, 4096, 4096), (40, 250, 160), (128, 512, 1024), (130, 1030, 416), (1024, 3072, 256),
+FWD_SHAPES = [(512, 4096, 128), (300, 3102, 288), (1, 16, 32), (7, 33, 64), (16, 48, 96), (17, 250, 416), (32, 1030, 1056), (4, 4096, 4096), (40, 250, 160), (128, 512, 1024), (130, 1030, 416), (1024, 3072, 256),
               (1000, 3102, 288)]
 
 
