@@ -301,8 +301,10 @@ static int check_gemm8(const void *A, const void *B, uint32_t M, uint32_t N, uin
     if (M == 0 || N == 0) return DUQ_OK;
     if (!A || !B) return DUQ_E_NULL;
     if (K == 0 || K % 32 != 0) return DUQ_E_KALIGN;
-    // one tile's rows are indexed with 32-bit byte offsets: 256 rows x K bytes, 128 rows x N x 4 bytes
-    if (K > (1u << 23) || N > (1u << 22) || M > (1u << 24)) return DUQ_E_TOO_LARGE;
+    // K: no int32 accumulator can overflow (|sum| <= 2^14 * K < 2^31), so wrapping (this GEMM) and saturating (the
+    // reference's tensor-core GEMM) accumulation cannot differ; M, N: one tile's rows are indexed with 32-bit byte
+    // offsets (128 rows x N x 4 bytes)
+    if (K > 131040u || N > (1u << 22) || M > (1u << 24)) return DUQ_E_TOO_LARGE;
     if (!aligned(A, 16) || !aligned(B, 16)) return DUQ_E_ALIGN;
     return DUQ_OK;
 }
@@ -361,7 +363,7 @@ int duq_weight_tile_8bit(const int8_t *w, uint32_t N, uint32_t K, int8_t *w_tile
     if (N == 0 || K == 0) return DUQ_OK;
     if (!w || !w_tiled) return DUQ_E_NULL;
     if (K % 32 != 0) return DUQ_E_KALIGN;
-    if (K > (1u << 23) || N > (1u << 22)) return DUQ_E_TOO_LARGE;
+    if (K > 131040u || N > (1u << 22)) return DUQ_E_TOO_LARGE;
     if (!aligned(w, 16) || !aligned(w_tiled, 16)) return DUQ_E_ALIGN;
     return duq::launch_weight_tile8(w, N, K, w_tiled, as_stream(stream));
 }

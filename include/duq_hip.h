@@ -243,7 +243,8 @@ int duq_asym_quant_host_8bit(const float *x, const float *scale, const float *ze
                              int8_t *q, duq_stream_t stream);
 
 /* A [M,K] int8 times B [N,K] int8 (both row-major; B is the weight as stored) -> C [M,N]
- * int32, K % 32 == 0, A and B 16-byte aligned.
+ * int32, K % 32 == 0, K <= 131040 (no accumulator can overflow, so the result does not depend on whether the
+ * matrix unit wraps or saturates), A and B 16-byte aligned.
  * Replaces matmul_host_8bit (include/gemm.h:14, src/kernels/gemm.cu:46-81; binding
  * src/export/bindings.cpp:28-45; the Python wrapper asserts K % 32 == 0,
  * qlinear4bit/tools/tensor_utils.py:57-61). */

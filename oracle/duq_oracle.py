@@ -621,7 +621,8 @@ def asym_quant_8bit(x, scale, zeros):
 
 def matmul_s8(a, b):
     """matmul_host_8bit (gemm.cu:46-81): C[m,n] = sum_k A[m,k] * B[n,k], int8 operands,
-    int32 accumulation (wraps like the hardware accumulator; it cannot for K <= 133 152)."""
+    int32 accumulation.  The sum is taken modulo 2**32 here; the library accepts K <= 131040 only, where no
+    accumulator can overflow (|sum| <= 2**14 * K < 2**31) and wrapping and saturating units agree."""
     # float64 BLAS is exact here: |sum| <= 2^14 * K, far below 2^53
     a = np.asarray(a, np.int8).astype(np.float64)
     b = np.asarray(b, np.int8).astype(np.float64)

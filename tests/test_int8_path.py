@@ -247,7 +247,8 @@ def test_abi_validation_8bit_entries():
     assert mm(P, P, 4, 8, 32, None, None) == -1
     assert mm(P + 8, P, 4, 8, 32, P, None) == -5
     assert mm(P, P, 4, (1 << 22) + 1, 32, P, None) == -6
-    assert mm(P, P, 4, 8, (1 << 23) + 32, P, None) == -6
+    assert mm(P, P, 4, 8, 131072, P, None) == -6          # an accumulator could overflow
+    assert 16384 * 131040 < 2 ** 31
     assert mm(None, None, 0, 8, 32, None, None) == 0
     fwd = lib.duq_linear8bit_forward
     assert fwd(P, P, P, P, P, P, None, 4, 8, 40, P, None) == -3
