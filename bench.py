@@ -33,6 +33,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, published
+PREWARM_STEPS = 300       # untimed steps before the W warm-up steps of every timed loop (about 10 ms of GPU work)
 PEAK_FP6_TOPS = 10100.0   # MI355X dense fp6 / fp4 MFMA, published
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, published
 GEMM_TRAFFIC_BYTES = (49350 + 16384) * 1024  # fetched + written per launch of the fused GEMM (rocprofv3 counters)
@@ -355,7 +356,9 @@ def main():
         raise SystemExit("bench.py: the 6-bit float path and the integer path disagree")
 
     # ---- whole-step throughput: W warm-up steps, then exactly K timed steps ----
-    for _ in range(args.warmup):
+    # (before them, untimed, enough steps to bring the part to the clock it holds under this load: after an idle
+    # period that takes about a millisecond, and a short run would otherwise measure the ramp)
+    for _ in range(PREWARM_STEPS + args.warmup):
         step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -388,7 +391,7 @@ def main():
         print(f"graph capture skipped: {exc}", file=sys.stderr)
 
     # ---- the same steps on the integer kernels ----
-    for _ in range(args.warmup):
+    for _ in range(PREWARM_STEPS + args.warmup):
         step_i8()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -401,8 +404,8 @@ def main():
     pq = quant(x)
     xs, sx = pq.shadow_x, pq.scales_x
     gemm_us = event_time_us(lambda: hip.linear4bit_forward_bf6(hip.EPI_SYM, xs, sx, None, lin.weight_shadow, sw),
-                            args.steps, args.warmup)
-    quant_us = event_time_us(lambda: hip.quantize_rows_sym_bf6(x, with_q=False), args.steps, args.warmup)
+                            args.steps, PREWARM_STEPS + args.warmup)
+    quant_us = event_time_us(lambda: hip.quantize_rows_sym_bf6(x, with_q=False), args.steps, PREWARM_STEPS + args.warmup)
     achieved = ops / gemm_us / 1e6
     roofline = {"bound": "mfma", "kernel": "gemm_bf6_kernel<8,4,0,false> (fused GEMM + dequant on v_mfma_f32_16x16x128_f8f6f4, 128 x 256 tiles)",
                 "achieved": round(achieved, 1), "peak": PEAK_FP6_TOPS, "unit": "TOP/s",
@@ -415,8 +418,8 @@ def main():
                 "traffic": GEMM_TRAFFIC_BYTES, "traffic_source": "profiles/gemm_bf6_kernel__prefill_M2048_K4096_N4096.txt"}
     xq = quant_i8(x).quantized_x
     i8_gemm_us = event_time_us(lambda: hip.linear4bit_forward(hip.EPI_SYM, xq, sx, None, lin_i8.weight, sw), args.steps,
-                               args.warmup)
-    i8_quant_us = event_time_us(lambda: hip.quantize_rows_sym(x), args.steps, args.warmup)
+                               PREWARM_STEPS + args.warmup)
+    i8_quant_us = event_time_us(lambda: hip.quantize_rows_sym(x), args.steps, PREWARM_STEPS + args.warmup)
     integer_path = {"ms_per_step": round(i8_ms_per_step, 5), "TOPS": round(ops / (i8_ms_per_step * 1e-3) / 1e12, 2),
                     "kernel": "gemm_s4_stream_kernel<4,0,false> (v_mfma_i32_32x32x32_i8)", "gemm_fused_us": round(i8_gemm_us, 2),
                     "quantize_rows_sym_us": round(i8_quant_us, 2),
@@ -450,7 +453,7 @@ def main():
     props = torch.cuda.get_device_properties(0)
     line = {
         "metric": "int4 Linear TOPS (prefill) & HBM GB/s (decode) at Llama-7B shapes, 1 MI355X",
-        "value": round(tops, 2), "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "value": round(tops, 2), "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "prewarm_steps": PREWARM_STEPS,
         "ms_per_step": round(ms_per_step, 5),
         "graph_ms_per_step": None if graph_ms_per_step is None else round(graph_ms_per_step, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
