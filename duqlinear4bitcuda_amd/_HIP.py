@@ -366,6 +366,58 @@ def linear4bit_forward(mode, xq, scale_x, zeros_x, w, w_scale_1, w_zeros_1=None,
     return y
 
 
+def gemm_kernel_for(M: int, N: int, K: int) -> int:
+    """Which kernel family the int4 GEMM runs for a shape (host arithmetic, no GPU work): see
+    ``duq_gemm_kernel_for`` in include/duq_hip.h."""
+    return _lib.load().duq_gemm_kernel_for(M, N, K)
+
+
+def quantize_linear4bit_forward(x, w, w_scale_1, w_scale_2=None, bias=None, clip: float = 1.0, qmax: int = 6,
+                                return_quantized: bool = False):
+    """SymQuantizer + Linear4bitSQ / Linear4bitDUSQ forward (qlinear4bit/nn/quantizer.py:10-16,
+    qlinear4bit/nn/linear.py:42-56, 167-176) from binary16 activations ``x`` [..., K]: bit-identical to
+    ``quantize_rows_sym`` followed by ``linear4bit_forward``.  Up to four rows are ONE launch;
+    larger inputs run the two launches with the codes staged in a buffer allocated here.  With
+    ``return_quantized`` also returns (codes uint8 [..., K/2], scales [..., 1])."""
+    name = "quantize_linear4bit_forward"
+    if not isinstance(x, torch.Tensor) or not isinstance(w, torch.Tensor):
+        raise RuntimeError(f"{name}: x and w must be tensors")
+    dev = x.device
+    _fast_check(name, "x", x, _F16, None)
+    _fast_check(name, "w", w, _U8, dev)
+    K = x.shape[-1]
+    if w.dim() != 2 or w.shape[1] * 2 != K:
+        raise RuntimeError(f"{name}: K differs: x {tuple(x.shape)} vs packed w {tuple(w.shape)}")
+    M = x.numel() // K if K else 0
+    N = w.shape[0]
+    ptrs = [0, 0, 0]
+    for k, (t, what) in enumerate(((w_scale_1, "w_scale_1"), (w_scale_2, "w_scale_2"), (bias, "bias"))):
+        if t is None:
+            continue
+        _fast_check(name, what, t, _F16, dev)
+        if t.numel() != N:
+            _check_size0(name, t.reshape(-1), what, N)
+        ptrs[k] = t.data_ptr()
+    lead = x.shape[:-1]
+    y = torch.empty(lead + (N,), dtype=_F16, device=dev)
+    q = s = None
+    if return_quantized:
+        q = torch.empty(lead + (K // 2,), dtype=_U8, device=dev)
+        s = torch.empty(lead + (1,), dtype=_F16, device=dev)
+    lib = _lib.load()
+    ws, ws_bytes = None, 0
+    if not return_quantized:
+        ws_bytes = lib.duq_quantize_linear4bit_workspace_bytes(M, N, K)
+        if ws_bytes:
+            ws = torch.empty(ws_bytes, dtype=_U8, device=dev)
+    st = _launch(dev, lib.duq_quantize_linear4bit_forward, EPI_SYM if w_scale_2 is None else EPI_SYM_DUAL,
+                 x.data_ptr(), float(clip), qmax, w.data_ptr(), ptrs[0] or None, ptrs[1] or None, ptrs[2] or None, M, N, K,
+                 y.data_ptr(), _ptr(q), _ptr(s), _ptr(ws), ws_bytes)
+    if st:
+        _lib.check(st, name)
+    return (y, q, s) if return_quantized else y
+
+
 # ---- asymmetric path with exact zero-point correction (row sums); not in the reference ----
 
 _I32 = torch.int32

@@ -34,6 +34,10 @@ PROTOTYPES = {
     "duq_asym_dual_dequant_host": [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_u32, _c_u32, _c_p, _c_p],
     "duq_linear4bit_forward": [_c_i32, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_u32, _c_u32,
                                _c_u32, _c_p, _c_p],
+    "duq_gemm_kernel_for": [_c_u32, _c_u32, _c_u32],
+    "duq_quantize_linear4bit_workspace_bytes": [_c_u32, _c_u32, _c_u32],  # returns uint64_t (restype set in load())
+    "duq_quantize_linear4bit_forward": [_c_i32, _c_p, ctypes.c_float, _c_i32, _c_p, _c_p, _c_p, _c_p, _c_u32, _c_u32,
+                                        _c_u32, _c_p, _c_p, _c_p, _c_p, ctypes.c_uint64, _c_p],
     "duq_quantize_rows_asym_shifted": [_c_p, _c_u32, _c_u32, _c_p, _c_p, _c_p, _c_p, _c_p],
     "duq_linear4bit_forward_rowsum": [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_u32, _c_u32, _c_u32,
                                       _c_p, _c_p],
@@ -75,6 +79,7 @@ def load():
         fn = getattr(lib, name)
         fn.argtypes = argtypes
         fn.restype = ctypes.c_int
+    lib.duq_quantize_linear4bit_workspace_bytes.restype = ctypes.c_uint64
     lib.duq_status_string.argtypes = [ctypes.c_int]
     lib.duq_status_string.restype = ctypes.c_char_p
     _lib = lib

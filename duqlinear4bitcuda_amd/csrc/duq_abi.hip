@@ -29,6 +29,41 @@ int check_gemm(const void *A, const void *B, uint32_t M, uint32_t N, uint32_t K)
     return DUQ_OK;
 }
 
+// quantize + GEMM + dequant from binary16 activations: one launch for decode shapes, otherwise the quantizer
+// into `workspace` (codes, then scales) followed by the GEMM
+int quantize_linear_impl(int32_t mode, const duq_half *x, float clip, int32_t qmax, const uint8_t *w,
+                         const duq_half *w_scale_1, const duq_half *w_scale_2, const duq_half *bias, uint32_t M,
+                         uint32_t N, uint32_t K, duq_half *y, uint8_t *q_out, duq_half *scale_out, void *workspace,
+                         uint64_t workspace_bytes, duq_stream_t stream)
+{
+    if (mode != DUQ_EPI_SYM && mode != DUQ_EPI_SYM_DUAL) return DUQ_E_MODE;
+    if (int e = check_qmax(qmax)) return e;
+    if (M == 0 || N == 0) return DUQ_OK;
+    if (!x) return DUQ_E_NULL;
+    if (int e = check_gemm(x, w, M, N, K)) return e;
+    if (K == 0) return DUQ_E_KALIGN;
+    if (!w_scale_1 || !y) return DUQ_E_NULL;
+    if (mode == DUQ_EPI_SYM_DUAL && !w_scale_2) return DUQ_E_NULL;
+    if ((q_out && !aligned(q_out, 16))) return DUQ_E_ALIGN;
+    duq::Epilogue e{mode, nullptr, nullptr, w_scale_1, nullptr, w_scale_2, nullptr, bias, nullptr, nullptr};
+    if (duq::decode_fp16in_one_launch(M, N, K))
+        return duq::launch_decode_fp16in(x, clip, qmax, w, M, N, K, e, y, q_out, scale_out, as_stream(stream));
+    // two launches: the codes and scales go to the caller's outputs when given, else to the workspace
+    const uint64_t code_bytes = ((uint64_t)M * (K / 2) + 15) & ~(uint64_t)15;
+    uint8_t *q = q_out;
+    duq_half *s = scale_out;
+    if (!q || !s) {
+        if (!workspace) return DUQ_E_NULL;
+        if (!aligned(workspace, 16)) return DUQ_E_ALIGN;
+        if (workspace_bytes < code_bytes + (((uint64_t)M * 2 + 15) & ~(uint64_t)15)) return DUQ_E_SHAPE;
+        if (!q) q = static_cast<uint8_t *>(workspace);
+        if (!s) s = reinterpret_cast<duq_half *>(static_cast<uint8_t *>(workspace) + code_bytes);
+    }
+    if (int st = duq::launch_quantize_rows_sym(x, M, K, clip, qmax, q, s, nullptr, as_stream(stream))) return st;
+    e.s_row = s;
+    return duq::launch_gemm_s4(q, w, M, N, K, nullptr, &e, y, as_stream(stream));
+}
+
 }  // namespace
 
 extern "C" {
@@ -197,6 +232,26 @@ int duq_linear4bit_forward(int32_t mode, const uint8_t *xq, const duq_half *scal
     if (asym && dual && !w_zeros_2) return DUQ_E_NULL;
     duq::Epilogue e{mode, scale_x, zeros_x, w_scale_1, w_zeros_1, w_scale_2, w_zeros_2, bias, nullptr, nullptr};
     return duq::launch_gemm_s4(xq, w, M, N, K, nullptr, &e, y, as_stream(stream));
+}
+
+int duq_gemm_kernel_for(uint32_t M, uint32_t N, uint32_t K) { return duq::select_gemm_kernel(M, N, K); }
+
+uint64_t duq_quantize_linear4bit_workspace_bytes(uint32_t M, uint32_t N, uint32_t K)
+{
+    if (M == 0 || N == 0 || K == 0) return 0;
+    if (duq::decode_fp16in_one_launch(M, N, K)) return 0;  // nothing staged
+    // packed codes [M, K/2] (rounded up to 16 bytes so that the scales stay aligned), then the scales [M]
+    return (((uint64_t)M * (K / 2) + 15) & ~(uint64_t)15) + (((uint64_t)M * 2 + 15) & ~(uint64_t)15);
+}
+
+int duq_quantize_linear4bit_forward(int32_t mode, const duq_half *x, float clip, int32_t qmax, const uint8_t *w,
+                                    const duq_half *w_scale_1, const duq_half *w_scale_2, const duq_half *bias,
+                                    uint32_t M, uint32_t N, uint32_t K, duq_half *y, uint8_t *q_out,
+                                    duq_half *scale_out, void *workspace, uint64_t workspace_bytes,
+                                    duq_stream_t stream)
+{
+    return quantize_linear_impl(mode, x, clip, qmax, w, w_scale_1, w_scale_2, bias, M, N, K, y, q_out, scale_out,
+                                workspace, workspace_bytes, stream);
 }
 
 int duq_asym_rowsum_dequant_host(const int32_t *q, const duq_half *scale_row, const duq_half *zeros_row,

@@ -1,0 +1,472 @@
+// Decode kernels (M <= 16 activation rows, K <= 16384): weight streaming for problems of a few MB,
+// where a launch lives for two or three microseconds and what counts is that every byte is requested
+// in the kernel's first instructions and nothing else sits on the critical path.
+//
+//   C[m,n] = sum_k s4(A[m,k]) * s4(B[n,k])        (src/kernels/gemm.cu:8-43 of the reference, at M <= 16)
+//
+// Both kernels
+//  * issue every weight load of the workgroup before anything else (no ring: the whole share of a
+//    workgroup, 16-32 KB, is in flight at once),
+//  * fetch the epilogue parameters of the outputs a lane will store right behind them, so that no
+//    dependent memory round trip follows the arithmetic,
+//  * take the activations pre-quantized (packed nibbles, the reference's operator boundary); the rows kernel
+//    also takes them as binary16 (FUSEQ): the workgroup then computes the per-token scales and codes itself
+//    while its weights are in flight (SymQuantizer.forward, qlinear4bit/nn/quantizer.py:10-16, and
+//    src/kernels/quant.cu:11-45, through the same RowQuant code as the stand-alone quantizer), which makes
+//    quantize + GEMM + dequant one launch.  (Up to four rows only: every workgroup reads all the rows, and from
+//    eight rows on that is more bytes into a CU than its share of the weights.)
+//
+//  rows kernel (M <= 4): v_dot8_i32_i4 on the packed nibbles.  A wavefront owns four weight rows and the
+//    whole K range: lane l holds bytes [i*1024 + l*16, +16) of each row, so a load instruction covers 1 KB
+//    of one row and an activation register serves four rows.  The 4*M partial sums of a lane meet the other
+//    lanes' through the wavefront's own piece of LDS (no barrier) and a few DPP steps.
+//  MFMA kernel (M <= 16): v_mfma_i32_16x16x64_i8, eight wavefronts split K for one 16-column tile, the partial
+//    tiles meet in LDS, the first 256 threads finish one output each.
+#include "duq_epilogue.h"
+#include "duq_launch.h"
+#include "duq_rowquant.h"
+#include "duq_tiles.h"
+
+#ifndef DUQ_DEC_R
+#define DUQ_DEC_R 4
+#endif
+#ifndef DUQ_DEC_WAVES
+#define DUQ_DEC_WAVES 8
+#endif
+
+namespace duq {
+
+namespace {
+
+constexpr uint32_t kNibbleMaskD = 0xF0F0F0F0u;
+
+struct DecodeParams {
+    const uint8_t *A;    // packed activations [M, K/2] (pre-quantized input)
+    const uint16_t *X;   // binary16 activations [M, K] (FUSEQ)
+    const uint8_t *B;    // packed weights [N, K/2]
+    uint32_t M, N, K;
+    int32_t *C;          // int32 out (EPI < 0)
+    uint16_t *y;         // binary16 out (EPI >= 0)
+    Epilogue epi;        // FUSEQ: s_row is not read, the kernel computes it
+    float clip;          // FUSEQ
+    int qmax;            // FUSEQ
+    uint8_t *q_out;      // FUSEQ, optional: the packed codes [M, K/2] (written by workgroup 0)
+    uint16_t *s_out;     // FUSEQ, optional: the per-token scales [M]
+    uint32_t tiles_per_wg;
+};
+
+template <int CTRL>
+__device__ __forceinline__ int dpp_add(int v)
+{
+    return v + __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true);
+}
+// Sum over groups of G consecutive lanes (G = 2, 4, 8 or 16, inside one DPP row): every lane of a group
+// ends with the group's total.
+template <int G>
+__device__ __forceinline__ int group_sum(int v)
+{
+    v = dpp_add<0xB1>(v);               // quad_perm [1,0,3,2]
+    if (G >= 4) v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
+    if (G >= 8) v = dpp_add<0x141>(v);  // row_half_mirror: lane i <- lane 7 - i
+    if (G >= 16) v = dpp_add<0x140>(v); // row_mirror: lane i <- lane 15 - i
+    return v;
+}
+
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_max(uint32_t v)
+{
+    return max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true));
+}
+// maximum over the 64 lanes, the same value in every lane (four DPP steps inside the rows of 16, then the four
+// rows through scalar registers)
+__device__ __forceinline__ uint32_t wave_max_u32_dpp(uint32_t v)
+{
+    v = dpp_max<0xB1>(v);
+    v = dpp_max<0x4E>(v);
+    v = dpp_max<0x141>(v);
+    v = dpp_max<0x140>(v);
+    const uint32_t a = (uint32_t)__builtin_amdgcn_readlane((int)v, 0), b = (uint32_t)__builtin_amdgcn_readlane((int)v, 16);
+    const uint32_t c = (uint32_t)__builtin_amdgcn_readlane((int)v, 32), d = (uint32_t)__builtin_amdgcn_readlane((int)v, 48);
+    return max(max(a, b), max(c, d));
+}
+
+__device__ __forceinline__ v4u load16(const void *p) { return *reinterpret_cast<const v4u *>(p); }
+
+template <int MODE>
+__device__ __forceinline__ ColParams load_col_rt(const Epilogue &e, uint32_t col, bool bias)
+{
+    return bias ? load_col<MODE, true>(e.s_col_1, e.z_col_1, e.s_col_2, e.z_col_2, e.bias, col, e.rs_col)
+                : load_col<MODE, false>(e.s_col_1, e.z_col_1, e.s_col_2, e.z_col_2, e.bias, col, e.rs_col);
+}
+template <int MODE>
+__device__ __forceinline__ uint16_t dequant_rt(int acc, const RowEpi &r, const ColParams &c, bool bias)
+{
+    return bias ? dequant_one<MODE, true>(acc, r, c) : dequant_one<MODE, false>(acc, r, c);
+}
+
+// ---------------------------------------------------------------------------------
+// rows kernel: M <= MR <= 4, K <= XS * 2048
+// ---------------------------------------------------------------------------------
+template <int MR, int XS, bool FUSEQ, int EPI>
+__global__ __launch_bounds__(256) void gemv_s4_rows_kernel(DecodeParams p)
+{
+    constexpr int R = DUQ_DEC_R;     // weight rows per wavefront
+    constexpr int V = MR * R;        // partial sums per lane: 4, 8 or 16
+    constexpr int LPV = 64 / V;      // lanes that finish one sum: 16, 8 or 4
+    constexpr int MODE = EPI < 0 ? 0 : EPI;
+    constexpr uint32_t XSTRIDE = XS * 1024;
+    static_assert(MR == 1 || MR == 2 || MR == 4, "rows");
+    __shared__ __attribute__((aligned(16))) int red[4][V * 64];
+    __shared__ __attribute__((aligned(16))) uint8_t xs[FUSEQ ? MR * XSTRIDE : 16];
+    __shared__ uint32_t rmax[4];
+    __shared__ uint16_t srow[MR];
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t kbytes = p.K >> 1;
+    const uint32_t n0 = (blockIdx.x * 4 + wave) * R;
+
+
+    // ---- loads, in the order their data is needed (loads return in order: waiting for one waits for every
+    // earlier one): the activations first, then every weight byte of this wavefront, then the parameters of the
+    // output this lane will finish
+    // activations: lane l needs bytes [i*1024 + l*16, +16) of every row
+    v4u xr[MR][XS];
+    constexpr int WPR = 4 / MR;              // wavefronts that share a row in the quantize phase
+    constexpr int UPL = FUSEQ ? XS * MR : 1;  // 8-element units per lane in the quantize phase
+    const uint32_t qrow = wave / WPR, qpart = wave % WPR;
+    v4u raw[UPL];
+    const uint32_t nunits = p.K >> 3;
+    if (!FUSEQ) {
+        const __amdgpu_buffer_rsrc_t rX = make_rsrc(p.A, p.M * kbytes);  // rows past M read as zero
+#pragma unroll
+        for (int m = 0; m < MR; ++m)
+#pragma unroll
+            for (int i = 0; i < XS; ++i) {
+                const uint32_t off = i * 1024 + lane * 16;
+                xr[m][i] = buf_load16(rX, off < kbytes ? m * kbytes + off : kOobOffset, 0);
+            }
+    } else {
+        // the workgroup quantizes the MR rows into LDS: WPR = 4 / MR wavefronts share a row, wavefront `part` of
+        // a row owns its 8-element units part*64 + lane, + 64*WPR, ...
+        const __amdgpu_buffer_rsrc_t rX = make_rsrc(p.X, p.M * p.K * 2);  // rows past M read as zero
+#pragma unroll
+        for (int j = 0; j < UPL; ++j) {
+            const uint32_t c = qpart * 64 + lane + j * (64 * WPR);
+            raw[j] = buf_load16(rX, c < nunits ? (qrow * p.K + c * 8) * 2 : kOobOffset, 0);
+        }
+    }
+    const __amdgpu_buffer_rsrc_t rW = make_rsrc(p.B, p.N * kbytes);
+    v4u w[R][XS];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int i = 0; i < XS; ++i) {
+            const uint32_t off = i * 1024 + lane * 16;
+            const bool ok = off < kbytes && n0 + r < p.N;  // K % 64 == 0: a 16-byte piece is all in or all out
+            w[r][i] = buf_load16(rW, ok ? (n0 + r) * kbytes + off : kOobOffset, 0);
+        }
+    const uint32_t myv = lane / LPV, sub = lane % LPV;
+    const uint32_t my_m = myv / R, my_n = n0 + myv % R;
+    const bool bias = p.epi.bias != nullptr;
+    ColParams cp{};
+    RowEpi rp{};
+    if (EPI >= 0) {
+        cp = load_col_rt<MODE>(p.epi, min(my_n, p.N - 1), bias);
+        if (!FUSEQ) rp = load_row<MODE>(p.epi, min(my_m, p.M - 1));
+    }
+
+    if (FUSEQ) {
+        uint32_t am = 0;
+#pragma unroll
+        for (int j = 0; j < UPL; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) am = pk_absmax_u16(am, raw[j][q]);
+        uint32_t m16 = wave_max_u32_dpp(max(am & 0xFFFFu, am >> 16));
+        if (WPR > 1) {  // the row's maximum crosses its wavefronts through LDS
+            if (lane == 0) rmax[wave] = m16;
+            __syncthreads();
+            m16 = rmax[qrow * WPR];
+#pragma unroll
+            for (int i = 1; i < WPR; ++i) m16 = max(m16, rmax[qrow * WPR + i]);
+        }
+        {
+            RowQuant<false> rq;
+            rq.init(m16, 0.f, 0.f, p.clip, p.qmax);
+            const bool copy_out = blockIdx.x == 0 && qrow < p.M;
+#pragma unroll
+            for (int j = 0; j < UPL; ++j) {
+                const uint32_t c = qpart * 64 + lane + j * (64 * WPR);
+                if (c < nunits) {
+                    const uint32_t word = rq.quant8(raw[j]);
+                    *reinterpret_cast<uint32_t *>(xs + qrow * XSTRIDE + c * 4) = word;
+                    if (copy_out && p.q_out) reinterpret_cast<uint32_t *>(p.q_out + (uint64_t)qrow * kbytes)[c] = word;
+                }
+            }
+            if (qpart == 0 && lane == 0) {
+                srow[qrow] = f16_to_bits(rq.s);
+                if (copy_out && p.s_out) p.s_out[qrow] = f16_to_bits(rq.s);
+            }
+        }
+        __syncthreads();
+        // (bytes past the row end are never written: the weights read as zero there)
+#pragma unroll
+        for (int m = 0; m < MR; ++m)
+#pragma unroll
+            for (int i = 0; i < XS; ++i) xr[m][i] = load16(xs + m * XSTRIDE + i * 1024 + lane * 16);
+        rp.s = bits_to_f16(srow[min(my_m, (uint32_t)MR - 1)]);
+    }
+
+    // ---- dot products on the packed nibbles
+    int acc[MR][R];
+#pragma unroll
+    for (int m = 0; m < MR; ++m)
+#pragma unroll
+        for (int r = 0; r < R; ++r) acc[m][r] = 0;
+#pragma unroll
+    for (int i = 0; i < XS; ++i)
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int m = 0; m < MR; ++m)
+#pragma unroll
+                for (int d = 0; d < 4; ++d)
+                    acc[m][r] = __builtin_amdgcn_sdot8((int)w[r][i][d], (int)xr[m][i][d], acc[m][r], false);
+
+    // ---- the V sums of 64 lanes each: through this wavefront's piece of LDS (a wavefront's LDS operations
+    // execute in order: no barrier), V entries per lane back, then log2(LPV) DPP steps
+    int *mine = red[wave];
+#pragma unroll
+    for (int v = 0; v < V; ++v) mine[v * 64 + lane] = acc[v / R][v % R];
+    __builtin_amdgcn_wave_barrier();
+    int sum = 0;
+#pragma unroll
+    for (int e = 0; e < V / 4; ++e) {
+        const v4i t = *reinterpret_cast<const v4i *>(&mine[lane * V + e * 4]);  // = [myv * 64 + sub * V + e * 4]
+        sum += (t[0] + t[1]) + (t[2] + t[3]);
+    }
+    sum = group_sum<LPV>(sum);
+    if (sub == 0 && my_m < p.M && my_n < p.N) {
+        if (EPI < 0)
+            p.C[(uint64_t)my_m * p.N + my_n] = sum;
+        else
+            p.y[(uint64_t)my_m * p.N + my_n] = dequant_rt<MODE>(sum, rp, cp, bias);
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// MFMA kernel: M <= 16, K <= WAVES * SEGS * 128 <= 12288
+// ---------------------------------------------------------------------------------
+// WAVES wavefronts split K: wavefront v owns the 64-byte row segments [v*SEGS, (v+1)*SEGS); lane (l16, g)
+// holds bytes [g*16, +16) of each, of weight row l16 of the tile (MFMA "A" side) and of activation row l16
+// ("B" side), so it ends up with four consecutive output columns of row l16.  Nibble -> byte as in the
+// GEMM kernels: (w & 0xF0F0F0F0) is the four odd-k nibbles times 16, ((w << 4) & 0xF0F0F0F0) the even ones;
+// every product is 256 * a * b and one arithmetic shift recovers the sum.
+template <int WAVES, int SEGS, int EPI>
+__global__ __launch_bounds__(WAVES * 64) void gemm_s4_decode_kernel(DecodeParams p)
+{
+    constexpr int MODE = EPI < 0 ? 0 : EPI;
+    static_assert(WAVES == 4 || WAVES == 8, "wavefronts per workgroup");
+    __shared__ v4i part[2][WAVES][64];
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t l16 = lane & 15u, g = lane >> 4;
+    const uint32_t kbytes = p.K >> 1;
+    const uint32_t seg0 = wave * SEGS;
+    const uint32_t ntiles = (p.N + 15) / 16;
+    const uint32_t tile0 = blockIdx.x * p.tiles_per_wg;
+    const uint32_t tile_end = min(tile0 + p.tiles_per_wg, ntiles);
+
+    const __amdgpu_buffer_rsrc_t rW = make_rsrc(p.B, p.N * kbytes);  // rows past N read as zero
+    uint32_t koff[SEGS];  // byte offset inside a row, or out of range for pieces past K
+#pragma unroll
+    for (int u = 0; u < SEGS; ++u) {
+        const uint32_t off = (seg0 + u) * 64 + g * 16;
+        koff[u] = off < kbytes ? off : kOobOffset;
+    }
+    auto load_tile = [&](uint32_t tile, v4u(&w)[SEGS]) {
+        const uint32_t row = tile * 16 + l16;
+        const bool rok = tile < tile_end && row < p.N;
+#pragma unroll
+        for (int u = 0; u < SEGS; ++u)
+            w[u] = buf_load16(rW, (rok && koff[u] != kOobOffset) ? row * kbytes + koff[u] : kOobOffset, 0);
+    };
+
+    // ---- loads in the order their data is needed (loads return in order): the activation fragments of this
+    // wavefront's k range (packed; expanded when used), the first tile's weights, the parameters of the outputs
+    // this thread will finish
+    v4u xp[SEGS];
+    const __amdgpu_buffer_rsrc_t rX = make_rsrc(p.A, p.M * kbytes);  // rows past M read as zero
+#pragma unroll
+    for (int u = 0; u < SEGS; ++u)
+        xp[u] = buf_load16(rX, koff[u] != kOobOffset ? l16 * kbytes + koff[u] : kOobOffset, 0);
+    v4u w0[SEGS], w1[SEGS];
+    load_tile(tile0, w0);
+
+    // threads 0..255 finish one output each: element er of MFMA lane src_lane
+    const uint32_t src_lane = (tid >> 2) & 63u, er = tid & 3u;
+    const uint32_t my_m = src_lane & 15u, my_c = (src_lane >> 4) * 4 + er;
+    const bool bias = p.epi.bias != nullptr;
+    const bool finisher = tid < 256;
+    ColParams cp{};
+    RowEpi rp{};
+    auto load_cp = [&](uint32_t tile) {
+        ColParams c{};
+        if (EPI >= 0 && finisher) c = load_col_rt<MODE>(p.epi, min(tile * 16 + my_c, p.N - 1), bias);
+        return c;
+    };
+    cp = load_cp(tile0);
+    if (EPI >= 0 && finisher) rp = load_row<MODE>(p.epi, min(my_m, p.M - 1));
+
+    auto compute_tile = [&](uint32_t tile, const v4u(&w)[SEGS], uint32_t buf) {
+        const ColParams cpn = load_cp(tile + 1 < tile_end ? tile + 1 : tile);  // next tile's, under this tile's work
+        v4i acc = v4i{0, 0, 0, 0};
+#pragma unroll
+        for (int u = 0; u < SEGS; ++u) {
+            v4u we, wo, xe, xo;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                we[q] = (w[u][q] << 4) & kNibbleMaskD;
+                wo[q] = w[u][q] & kNibbleMaskD;
+                xe[q] = (xp[u][q] << 4) & kNibbleMaskD;
+                xo[q] = xp[u][q] & kNibbleMaskD;
+            }
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i, we), __builtin_bit_cast(v4i, xe), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i, wo), __builtin_bit_cast(v4i, xo), acc, 0, 0, 0);
+        }
+        part[buf][wave][lane] = acc;
+        __syncthreads();
+        if (finisher) {
+            int sum = 0;
+#pragma unroll
+            for (int w2 = 0; w2 < WAVES; ++w2) sum += part[buf][w2][src_lane][er];
+            sum >>= 8;
+            const uint32_t n = tile * 16 + my_c;
+            if (my_m < p.M && n < p.N) {
+                if (EPI < 0)
+                    p.C[(uint64_t)my_m * p.N + n] = sum;
+                else
+                    p.y[(uint64_t)my_m * p.N + n] = dequant_rt<MODE>(sum, rp, cp, bias);
+            }
+        }
+        cp = cpn;
+    };
+
+    // two register sets alternate so that one tile's loads are in flight during the other's MFMAs; the
+    // partial-sum buffers alternate too: one barrier per tile
+    for (uint32_t t = tile0; t < tile_end; t += 2) {
+        load_tile(t + 1, w1);
+        compute_tile(t, w0, 0);
+        load_tile(t + 2, w0);
+        if (t + 1 < tile_end) compute_tile(t + 1, w1, 1);
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// dispatch
+// ---------------------------------------------------------------------------------
+template <int MR, int XS, bool FUSEQ>
+void launch_rows_mode(const DecodeParams &p, int epi, hipStream_t stream)
+{
+    const dim3 grid((p.N + 4 * DUQ_DEC_R - 1) / (4 * DUQ_DEC_R));  // 4 wavefronts x R rows per workgroup
+#define DUQ_ROWS(E) hipLaunchKernelGGL((gemv_s4_rows_kernel<MR, XS, FUSEQ, E>), grid, dim3(256), 0, stream, p)
+    switch (epi) {
+    case 0: DUQ_ROWS(0); break;
+    case 2: DUQ_ROWS(2); break;
+    default:
+        if constexpr (!FUSEQ) {
+            switch (epi) {
+            case -1: DUQ_ROWS(-1); break;
+            case 1: DUQ_ROWS(1); break;
+            case 3: DUQ_ROWS(3); break;
+            case 4: DUQ_ROWS(4); break;
+            }
+        }
+    }
+#undef DUQ_ROWS
+}
+
+template <int MR, bool FUSEQ>
+void launch_rows_xs(const DecodeParams &p, int epi, hipStream_t stream)
+{
+    const uint32_t kbytes = p.K / 2;
+    if (kbytes <= 2048) launch_rows_mode<MR, 2, FUSEQ>(p, epi, stream);
+    else if (kbytes <= 4096) launch_rows_mode<MR, 4, FUSEQ>(p, epi, stream);
+    else if (kbytes <= 6144) launch_rows_mode<MR, 6, FUSEQ>(p, epi, stream);
+    else launch_rows_mode<MR, 8, FUSEQ>(p, epi, stream);
+}
+
+template <int WAVES, int SEGS>
+void launch_mfma_mode(const DecodeParams &p, int epi, hipStream_t stream)
+{
+    const uint32_t ntiles = (p.N + 15) / 16;
+    const dim3 grid((ntiles + p.tiles_per_wg - 1) / p.tiles_per_wg);
+#define DUQ_DEC(E) hipLaunchKernelGGL((gemm_s4_decode_kernel<WAVES, SEGS, E>), grid, dim3(WAVES * 64), 0, stream, p)
+    switch (epi) {
+    case -1: DUQ_DEC(-1); break;
+    case 0: DUQ_DEC(0); break;
+    case 1: DUQ_DEC(1); break;
+    case 2: DUQ_DEC(2); break;
+    case 3: DUQ_DEC(3); break;
+    case 4: DUQ_DEC(4); break;
+    }
+#undef DUQ_DEC
+}
+
+template <bool FUSEQ>
+void launch_decode_any(DecodeParams &p, int epi, hipStream_t stream)
+{
+    const uint32_t kbytes = p.K / 2;
+    if (decode_uses_rows_kernel(p.M)) {
+        if (p.M == 1) launch_rows_xs<1, FUSEQ>(p, epi, stream);
+        else if (p.M == 2) launch_rows_xs<2, FUSEQ>(p, epi, stream);
+        else launch_rows_xs<4, FUSEQ>(p, epi, stream);
+        return;
+    }
+    if constexpr (!FUSEQ) {
+        const uint32_t ntiles = (p.N + 15) / 16;
+        p.tiles_per_wg = decode_tiles_per_workgroup(ntiles);
+        constexpr int W = DUQ_DEC_WAVES, S = 32 / W;  // 64-byte segments per wavefront for 2 KB of a row
+        if (kbytes <= 2048) launch_mfma_mode<W, S>(p, epi, stream);
+        else if (kbytes <= 4096) launch_mfma_mode<W, 2 * S>(p, epi, stream);
+        else launch_mfma_mode<8, 12>(p, epi, stream);
+    }
+}
+
+}  // namespace
+
+int launch_decode_s4(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N, uint32_t K, int32_t *out_acc,
+                     const Epilogue *epi, uint16_t *y, hipStream_t stream)
+{
+    DecodeParams p{};
+    p.A = A;
+    p.B = B;
+    p.M = M;
+    p.N = N;
+    p.K = K;
+    p.C = out_acc;
+    p.y = y;
+    if (epi) p.epi = *epi;
+    launch_decode_any<false>(p, out_acc ? -1 : epi->mode, stream);
+    return (int)hipGetLastError();
+}
+
+int launch_decode_fp16in(const uint16_t *x, float clip, int qmax, const uint8_t *B, uint32_t M, uint32_t N, uint32_t K,
+                         const Epilogue &epi, uint16_t *y, uint8_t *q_out, uint16_t *s_out, hipStream_t stream)
+{
+    DecodeParams p{};
+    p.X = x;
+    p.B = B;
+    p.M = M;
+    p.N = N;
+    p.K = K;
+    p.y = y;
+    p.epi = epi;
+    p.clip = clip;
+    p.qmax = qmax;
+    p.q_out = q_out;
+    p.s_out = s_out;
+    launch_decode_any<true>(p, epi.mode, stream);
+    return (int)hipGetLastError();
+}
+
+}  // namespace duq

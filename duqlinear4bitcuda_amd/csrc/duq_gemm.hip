@@ -10,18 +10,19 @@
 // 256*|C| stays below 2^31 for K <= 131008.  Integer accumulation is order-free, so the
 // k order inside a tile only has to be the same for A and B.
 //
-// Five kernels, picked by shape in launch_epi():
+// Five kernels here, picked by shape in select_gemm_kernel() (decode shapes of a few MB run the two kernels of
+// duq_decode.hip):
 //  * stream kernel (prefill, M >= 128; tiles of 128, 64 or 32 rows x 256 columns, the height
 //    picked per shape): weights go from global memory straight to registers, activations are
 //    expanded once into LDS, v_mfma_i32_32x32x32_i8 with a hand-ordered schedule (see the kernel);
-//  * tile kernel (everything else above 16 rows): BM x BN x 128 tiles, 4 wavefronts (2 x 2),
-//    both operands expanded on the way into double-buffered LDS, v_mfma_i32_16x16x64_i8;
-//  * ring kernel (17 <= M <= 64, and up to 16 rows longer than 8192 elements): packed activations of all
-//    rows in LDS, every wavefront streams whole weight rows through a ring of loads;
-//  * skinny kernel (decode, 2 <= M <= 16): one workgroup owns 16 output columns, its
-//    wavefronts split K, fragments go from global memory straight to registers;
-//  * dot kernel (decode, M = 1; M <= 4 for long rows): v_dot8_i32_i4 on the packed nibbles, a pure HBM
-//    stream.
+//  * tile kernel (everything else above 16 rows, and any tensor of 4 GiB or more): BM x BN x 128 tiles,
+//    4 wavefronts (2 x 2), both operands expanded on the way into double-buffered LDS, v_mfma_i32_16x16x64_i8;
+//  * ring kernel (17 <= M <= 256 on narrow problems, and 5..16 rows of 12289..16384 elements): packed
+//    activations of all rows in LDS, every wavefront streams whole weight rows through a ring of loads;
+//  * skinny kernel (5 <= M <= 16 with 512 or more column tiles): one workgroup owns 16 output columns, its
+//    wavefronts split K, whole-line weight loads turned into fragments through LDS;
+//  * dot kernel (M <= 4 with rows longer than 16384 elements): v_dot8_i32_i4 on the packed nibbles, a
+//    pure HBM stream.
 // In the MFMA kernels the weight operand goes to the MFMA "A" side, so each lane ends up
 // with four consecutive output columns of one row.
 #include "duq_epilogue.h"
@@ -540,7 +541,7 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
 }
 
 // ---------------------------------------------------------------------------------
-// skinny kernel (2 <= M <= 16; also one row when the dot kernel's limits do not hold)
+// skinny kernel (5 <= M <= 16 on wide problems: 512 or more 16-column tiles, K <= 8192)
 // ---------------------------------------------------------------------------------
 // Workgroup = WAVES wavefronts that split K; it walks `tiles_per_wg` consecutive 16-column
 // tiles.  Wavefront w owns 64-byte row segments [w*S, (w+1)*S), S <= 8: lane (l16, g) holds
@@ -549,20 +550,21 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
 // per tile only the weights stream in (the next tile's loads are issued before the current
 // tile's MFMAs), two MFMAs per 16-byte weight piece (even k, odd k).  Partial sums of the
 // wavefronts meet in LDS (double buffered: one barrier per tile).
+// Weight loads fetch whole cache lines: an instruction covers 8 rows x 128 contiguous bytes instead of the
+// MFMA layout's 16 rows x 64 (half a line each); the wavefront turns the tile into the MFMA's lane layout
+// through its own 8 KB of LDS (one 128-bit write and one 128-bit read per load; no barrier: the piece is
+// private to the wavefront and a wavefront's LDS operations execute in order).  Slot s of a row's line holds
+// its 16-byte piece s ^ ((row / 2) % 8), which makes the 16 rows x 16 bytes of a fragment read cover every bank
+// once.  Measured 4-9 % faster than MFMA-layout loads from 512 column tiles on; smaller problems run the
+// decode kernels (duq_decode.hip), where the extra LDS hop is not hidden.
 constexpr int kSkinnySegs = 8;  // 64-byte segments per wavefront = 128-bit weight loads in flight per lane
 
 
-template <int WAVES, bool LINES, int EPI, bool BIAS>
+template <int WAVES, int EPI, bool BIAS>
 __global__ __launch_bounds__(WAVES * 64) void gemm_s4_skinny_kernel(GemmParams p)
 {
     __shared__ v4i part[2][WAVES][64];
-    // Whole-line loads (LINES; 4-6 % faster from 512 column tiles on, slower on small problems, where the extra LDS
-    // hop is not hidden): a load instruction fetches 8 rows x 128 contiguous bytes instead of 16
-    // rows x 64 (half a cache line each); the wavefront turns the tile into the MFMA's lane layout through its own
-    // 8 KB of LDS (one 128-bit write and one 128-bit read per load; no barrier: the piece is private to the wavefront
-    // and a wavefront's LDS operations execute in order).  Slot s of a row's line holds its 16-byte piece
-    // s ^ ((row / 2) % 8), which makes the 16 rows x 16 bytes of a fragment read cover every bank once.
-    __shared__ __attribute__((aligned(16))) uint8_t turn[LINES ? WAVES * 8192 : 16];
+    __shared__ __attribute__((aligned(16))) uint8_t turn[WAVES * 8192];
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63u, wave = tid >> 6;
     const uint32_t l16 = lane & 15u, g = lane >> 4;
@@ -575,96 +577,71 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_s4_skinny_kernel(GemmParams p
     const uint32_t tile0 = blockIdx.x * tiles_per_wg;
     const uint32_t tile_end = min(tile0 + tiles_per_wg, ntiles);
 
+    // 32-bit byte offsets over the whole tensors: the dispatcher only comes here while N * K / 2 < 2^32 - 256
     const __amdgpu_buffer_rsrc_t rW = make_rsrc(p.B, p.N * kbytes);  // rows past N read as zero
     const __amdgpu_buffer_rsrc_t rX = make_rsrc(p.A, p.M * kbytes);  // rows past M read as zero
-
-    uint32_t koff[kSkinnySegs];  // byte offset inside a row, or out of range for pieces past K
-#pragma unroll
-    for (int u = 0; u < kSkinnySegs; ++u) {
-        const uint32_t off = (seg0 + u) * 64 + g * 16;
-        koff[u] = (seg0 + u < segs && off < kbytes) ? off : kOobOffset;
-    }
 
     // activations of this wavefront's k range: once per workgroup
     v4u xe[kSkinnySegs], xo[kSkinnySegs];
 #pragma unroll
     for (int u = 0; u < kSkinnySegs; ++u) {
-        const v4u x = buf_load16(rX, koff[u] == kOobOffset ? kOobOffset : l16 * kbytes + koff[u], 0);
+        const uint32_t off = (seg0 + u) * 64 + g * 16;
+        const bool ok = seg0 + u < segs && off < kbytes;
+        const v4u x = buf_load16(rX, ok ? l16 * kbytes + off : kOobOffset, 0);
         expand_nibbles(x, xe[u], xo[u]);
     }
 
     auto load_tile = [&](uint32_t tile, v4u(&w)[kSkinnySegs]) {
-        if (LINES) {
-            // load u = 2 * line + half: rows 8 * half + r8 of the tile, slot j8 of line `line` of this wavefront's range
+        // load u = 2 * line + half: rows 8 * half + r8 of the tile, slot j8 of line `line` of this wavefront's range
 #pragma unroll
-            for (int u = 0; u < kSkinnySegs; ++u) {
-                const uint32_t rt = (u & 1) * 8 + r8, row = tile * 16 + rt;
-                const uint32_t off = seg0 * 64 + (u >> 1) * 128 + ((j8 ^ ((rt >> 1) & 7u)) << 4);
-                const bool ok = tile < tile_end && row < p.N && off < kbytes;
-                w[u] = buf_load16(rW, ok ? row * kbytes + off : kOobOffset, 0);
-            }
-            return;
+        for (int u = 0; u < kSkinnySegs; ++u) {
+            const uint32_t rt = (u & 1) * 8 + r8, row = tile * 16 + rt;
+            const uint32_t off = seg0 * 64 + (u >> 1) * 128 + ((j8 ^ ((rt >> 1) & 7u)) << 4);
+            const bool ok = tile < tile_end && row < p.N && off < kbytes;
+            w[u] = buf_load16(rW, ok ? row * kbytes + off : kOobOffset, 0);
         }
-        const uint32_t row = tile * 16 + l16;
-        const bool rok = tile < tile_end && row < p.N;
-#pragma unroll
-        for (int u = 0; u < kSkinnySegs; ++u)
-            w[u] = buf_load16(rW, (rok && koff[u] != kOobOffset) ? row * kbytes + koff[u] : kOobOffset, 0);
     };
     auto compute_tile = [&](uint32_t tile, const v4u(&w)[kSkinnySegs], uint32_t buf) {
         v4i acc = v4i{0, 0, 0, 0};
-        uint8_t *mine = turn + (LINES ? wave * 8192 : 0);
-        if (LINES) {
+        uint8_t *mine = turn + wave * 8192;
 #pragma unroll
-            for (int u = 0; u < kSkinnySegs; ++u) *reinterpret_cast<v4u *>(mine + u * 1024 + lane * 16) = w[u];
-        }
+        for (int u = 0; u < kSkinnySegs; ++u) *reinterpret_cast<v4u *>(mine + u * 1024 + lane * 16) = w[u];
 #pragma unroll
         for (int u = 0; u < kSkinnySegs; ++u) {
+            // segment u = 64 bytes: half (u % 2) of line u / 2; this lane's row l16 sits in load 2 * line + l16 / 8
+            const uint32_t piece = (u & 1) * 4 + g;
+            const v4u raw = *reinterpret_cast<const v4u *>(mine + ((u >> 1) * 2 + (l16 >> 3)) * 1024 + (l16 & 7u) * 128 +
+                                                           ((piece ^ ((l16 >> 1) & 7u)) << 4));
             v4u we, wo;
-            v4u raw = w[u];
-            if (LINES) {
-                // segment u = 64 bytes: half (u % 2) of line u / 2; this lane's row l16 sits in load 2 * line + l16 / 8
-                const uint32_t piece = (u & 1) * 4 + g;
-                raw = *reinterpret_cast<const v4u *>(mine + ((u >> 1) * 2 + (l16 >> 3)) * 1024 + (l16 & 7u) * 128 +
-                                                     ((piece ^ ((l16 >> 1) & 7u)) << 4));
-            }
             expand_nibbles(raw, we, wo);
             acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i, we), __builtin_bit_cast(v4i, xe[u]), acc,
                                                         0, 0, 0);
             acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i, wo), __builtin_bit_cast(v4i, xo[u]), acc,
                                                         0, 0, 0);
         }
-        if (WAVES > 1) {
-            // every wavefront parks its 16 x 16 partial tile, then the first 256 threads each
-            // finish one output element (sum over wavefronts, epilogue, store): no wavefront
-            // is a serial bottleneck
-            part[buf][wave][lane] = acc;
-            __syncthreads();
-            if (tid < 256) {
-                const uint32_t src_lane = tid >> 2, r = tid & 3u;
-                int sum = 0;
+        // every wavefront parks its 16 x 16 partial tile, then the first 256 threads each
+        // finish one output element (sum over wavefronts, epilogue, store): no wavefront
+        // is a serial bottleneck
+        part[buf][wave][lane] = acc;
+        __syncthreads();
+        if (tid < 256) {
+            const uint32_t src_lane = tid >> 2, r = tid & 3u;
+            int sum = 0;
 #pragma unroll
-                for (int w2 = 0; w2 < WAVES; ++w2) sum += part[buf][w2][src_lane][r];
-                sum >>= 8;
-                const uint32_t m = src_lane & 15u, n = tile * 16 + (src_lane >> 4) * 4 + r;
-                if (m < p.M && n < p.N) {
-                    if (EPI < 0) {
-                        p.C[(uint64_t)m * p.N + n] = sum;
-                    } else {
-                        constexpr int MODE = EPI < 0 ? 0 : EPI;
-                        const ColParams c = load_col<MODE, BIAS>(p.epi.s_col_1, p.epi.z_col_1, p.epi.s_col_2,
-                                                                 p.epi.z_col_2, p.epi.bias, n, p.epi.rs_col);
-                        p.y[(uint64_t)m * p.N + n] = dequant_one<MODE, BIAS>(sum, load_row<MODE>(p.epi, m), c);
-                    }
+            for (int w2 = 0; w2 < WAVES; ++w2) sum += part[buf][w2][src_lane][r];
+            sum >>= 8;
+            const uint32_t m = src_lane & 15u, n = tile * 16 + (src_lane >> 4) * 4 + r;
+            if (m < p.M && n < p.N) {
+                if (EPI < 0) {
+                    p.C[(uint64_t)m * p.N + n] = sum;
+                } else {
+                    constexpr int MODE = EPI < 0 ? 0 : EPI;
+                    const ColParams c = load_col<MODE, BIAS>(p.epi.s_col_1, p.epi.z_col_1, p.epi.s_col_2,
+                                                             p.epi.z_col_2, p.epi.bias, n, p.epi.rs_col);
+                    p.y[(uint64_t)m * p.N + n] = dequant_one<MODE, BIAS>(sum, load_row<MODE>(p.epi, m), c);
                 }
             }
-            return;
         }
-#pragma unroll
-        for (int r = 0; r < 4; ++r) acc[r] >>= 8;
-        const bool vec_ok = (EPI < 0) ? (p.N % 4 == 0 && reinterpret_cast<uintptr_t>(p.C) % 16 == 0)
-                                      : (p.N % 4 == 0 && reinterpret_cast<uintptr_t>(p.y) % 8 == 0);
-        store_quad<EPI, BIAS>(p, l16, tile * 16 + g * 4, acc, vec_ok);
     };
 
     // two register sets alternate so that one tile's loads are in flight during the other's MFMAs
@@ -679,7 +656,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_s4_skinny_kernel(GemmParams p
 }
 
 // ---------------------------------------------------------------------------------
-// ring kernel (17 <= M <= 64, and M <= 16 with rows too long for the skinny kernel)
+// ring kernel (17 <= M <= 256 on narrow problems, and M <= 16 with rows of 12289..16384 elements)
 // ---------------------------------------------------------------------------------
 // The packed activations of all 16*RB rows sit in LDS for the whole K range (rows padded so that
 // 16 rows x 16 bytes cover every bank once); a wavefront owns a 16-column tile and a K slice
@@ -799,7 +776,7 @@ __global__ __launch_bounds__(256) void gemm_s4_ring_kernel(GemmParams p)
 }
 
 // ---------------------------------------------------------------------------------
-// dot kernel (decode, M = 1, and M <= 4 when K > 16384 or M = 2 with K > 4096): weight streaming on v_dot8_i32_i4
+// dot kernel (M <= 4, rows longer than 16384 elements): weight streaming on v_dot8_i32_i4
 // ---------------------------------------------------------------------------------
 // The signed 4-bit dot product instruction consumes packed nibbles as they lie in memory,
 // so nothing is expanded and no MFMA is needed: the kernel is a pure HBM stream.
@@ -901,15 +878,52 @@ __global__ __launch_bounds__(256) void gemv_s4_dot_kernel(GemmParams p)
 // ---------------------------------------------------------------------------------
 // dispatch
 // ---------------------------------------------------------------------------------
+// Which kernel family takes a shape.  Host arithmetic only, so that the rule can be tested without a GPU:
+// every kernel whose weight offsets are 32-bit (decode, dot, ring: row * K/2 + offset, and a buffer descriptor
+// over the whole tensor) is reachable only while the packed weights stay below 4 GiB - 256 (the out-of-range
+// marker); larger tensors go to the stream / tile kernels, whose descriptors and pointers are per tile
+// (64-bit base, 32-bit offsets inside 256 rows).
+int select_gemm_kernel(uint32_t M, uint32_t N, uint32_t K)
+{
+    const uint64_t wbytes = (uint64_t)N * (K / 2);
+    const bool small_offsets = wbytes < 0xFFFFFF00ull && K > 0;
+    // decode: up to 16 rows.  Rows kernel for up to four rows (8 KB of every weight row per wavefront); above,
+    // the MFMA decode kernel (6 KB per row over eight wavefronts), or the skinny kernel once there are 512
+    // column tiles (its whole-line weight loads measure 7-9 % faster there)
+    if (M <= 4 && K <= 16384 && small_offsets) return kKernelDecodeRows;
+    if (M <= 16 && small_offsets) {
+        if ((N + 15) / 16 >= 512 && K <= 8192) return kKernelSkinny;
+        if (K <= 12288) return kKernelDecodeMfma;
+    }
+    const uint32_t xstride = ((K / 2 + 127) / 128) * 128;
+    // dot kernel: up to four rows too long for the decode kernels
+    if (M <= 4 && small_offsets && 4 * xstride <= 60 * 1024) return kKernelDot;
+    {
+        // ring kernel: 17..256 rows in groups whose packed activations fit in LDS (a few groups only, or a
+        // problem too narrow to fill the chip with stream-kernel tiles)
+        const uint32_t rb_all = (M + 15) / 16;
+        const uint32_t rb_max = K <= 4096 ? 4 : (K <= 8192 ? 2 : 1);  // 16-row blocks whose activations fit in LDS
+        const uint32_t rb = std::min(rb_all, rb_max);
+        const uint32_t row_groups = (rb_all + rb - 1) / rb;
+        // (several row groups re-stream the weights: with enough column tiles to fill the chip the stream
+        // kernel's 32-row tiles are cheaper then)
+        const uint32_t tiles32 = ((M + 31) / 32) * ((N + 255) / 256);
+        const bool few_groups = row_groups <= 2 || (row_groups <= 6 && tiles32 < 64) || tiles32 < 48;
+        const bool mid_rows = M > 16 && M <= 256 && few_groups && !(row_groups > 1 && tiles32 >= 128);
+        const bool long_rows = M <= 16 && K > 8192;  // 5..16 rows of 12289..16384 elements
+        if ((long_rows || mid_rows) && K <= 16384 && small_offsets) return kKernelRing;
+    }
+    auto tiles = [&](uint32_t bm, uint32_t bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+    if (M > 32 && tiles(32, 256) >= 32) return kKernelStream;
+    return kKernelTile;
+}
+
 template <int EPI, bool BIAS>
 static void launch_epi(GemmParams &p, hipStream_t stream)
 {
-    const uint64_t wbytes = (uint64_t)p.N * (p.K / 2);
-    const uint32_t xstride = ((p.K / 2 + 127) / 128) * 128;
-    // dot kernel: always for one row and for rows too long for the skinny kernel; two rows when K > 4096
-    // (measured: the MFMA skinny kernel is level or ahead for 2-4 rows otherwise)
-    const bool dot_shape = p.M == 1 || p.K > 16384 || (p.M == 2 && p.K > 4096);
-    if (p.M <= 4 && dot_shape && wbytes < 0xFFFFFF00ull && 4 * xstride <= 60 * 1024 && p.K > 0) {
+    const int kernel = select_gemm_kernel(p.M, p.N, p.K);
+    if (kernel == kKernelDot) {
+        const uint32_t xstride = ((p.K / 2 + 127) / 128) * 128;
         const dim3 grid((p.N + 7) / 8);
         if (p.M == 1)
             hipLaunchKernelGGL((gemv_s4_dot_kernel<1, EPI, BIAS>), grid, dim3(256), 1 * xstride, stream, p);
@@ -919,83 +933,58 @@ static void launch_epi(GemmParams &p, hipStream_t stream)
             hipLaunchKernelGGL((gemv_s4_dot_kernel<4, EPI, BIAS>), grid, dim3(256), 4 * xstride, stream, p);
         return;
     }
-    {
-        // ring kernel: 17..256 rows in groups whose packed activations fit in LDS (a few groups only, or a
-        // problem too narrow to fill the chip with stream-kernel tiles), and up to 16 rows that are too long
-        // for the skinny kernel's registers
-        const uint32_t rb_all = (p.M + 15) / 16;
-        const uint32_t rb_max = p.K <= 4096 ? 4 : (p.K <= 8192 ? 2 : 1);  // 16-row blocks whose activations fit in LDS
-        const uint32_t rb = std::min(rb_all, rb_max);
-        const uint32_t row_groups = (rb_all + rb - 1) / rb;
-        const bool long_rows = p.M <= 16 && p.K > 8192;
-        // (several row groups re-stream the weights: with enough column tiles to fill the chip the stream
-        // kernel's 32-row tiles are cheaper then)
-        const uint32_t tiles32 = ((p.M + 31) / 32) * ((p.N + 255) / 256);
-        const bool few_groups = row_groups <= 2 || (row_groups <= 6 && tiles32 < 64) || tiles32 < 48;
-        const bool mid_rows = p.M > 16 && p.M <= 256 && few_groups && !(row_groups > 1 && tiles32 >= 128);
-        if ((long_rows || mid_rows) && p.K <= 16384 && wbytes < 0xFFFFFF00ull && p.K > 0) {
-            const uint32_t ntiles = (p.N + 15) / 16;
-            const uint32_t segs = (p.K / 2 + 63) / 64;
-            // wavefronts splitting K for one tile: as few as give the chip ~2048 wavefronts, slices of at
-            // least 512 bytes per row
-            uint32_t kslices = 1;
-            while (ntiles * kslices < 2048 && kslices < 4 && segs / (kslices * 2) >= (uint32_t)kRing) kslices *= 2;
-            const uint32_t groups = (ntiles + 4 / kslices - 1) / (4 / kslices);
-            const uint32_t xbytes = p.K <= 4096 ? 2048 : (p.K <= 8192 ? 4096 : 8192);
-            const uint32_t lds = 16 * rb * (xbytes + 16) + 4 * rb * 1024;
-            const uint32_t slots = 256 * std::max(1u, std::min(8u, (160u * 1024) / lds));
-            p.tiles_m = kslices;
-            p.tiles_n = (groups + slots - 1) / slots;
-            const dim3 grid((groups + p.tiles_n - 1) / p.tiles_n, row_groups);
-#define DUQ_RING(X, R) hipLaunchKernelGGL((gemm_s4_ring_kernel<X, R, EPI, BIAS>), grid, dim3(256), 0, stream, p)
-            if (xbytes == 8192) DUQ_RING(8192, 1);
-            else if (xbytes == 4096) DUQ_RING(4096, 2);
-            else if (rb == 2) DUQ_RING(2048, 2);
-            else if (rb == 3) DUQ_RING(2048, 3);
-            else DUQ_RING(2048, 4);
-#undef DUQ_RING
-            return;
-        }
-    }
-    if (p.M <= 16) {
+    if (kernel == kKernelSkinny) {
         const uint32_t ntiles = (p.N + 15) / 16;
         const uint32_t segs = (p.K / 2 + 63) / 64;
-        // several column tiles per workgroup once there are plenty of them (activations are
-        // fetched and expanded once per workgroup); at least ~2 workgroups per CU stay.
-        // Long rows (8+ wavefronts per workgroup, one workgroup per CU): size the grid to
-        // whole rounds of 256 workgroups, at most 8 tiles each.
+        // several column tiles per workgroup (activations are fetched and expanded once per workgroup); at least
+        // ~2 workgroups per CU stay.  Long rows (8 wavefronts per workgroup, one workgroup per CU): whole rounds
+        // of 256 workgroups, at most 8 tiles each.
         uint32_t tpw = ntiles >= 6144 ? 8 : (ntiles >= 1536 ? 4 : (ntiles >= 640 ? 2 : 1));
-        if (segs > 4 * kSkinnySegs && ntiles >= 512) {
+        if (segs > 4 * kSkinnySegs) {
             const uint32_t rounds = (ntiles + 2047) / 2048;
             tpw = (ntiles + 256 * rounds - 1) / (256 * rounds);
         }
         p.tiles_m = tpw;
         const dim3 grid((ntiles + tpw - 1) / tpw);
-        const bool lines = ntiles >= 512;  // whole-line weight loads turned through LDS
-        if (segs <= 4 * kSkinnySegs) {
-            if (lines)
-                hipLaunchKernelGGL((gemm_s4_skinny_kernel<4, true, EPI, BIAS>), grid, dim3(256), 0, stream, p);
-            else
-                hipLaunchKernelGGL((gemm_s4_skinny_kernel<4, false, EPI, BIAS>), grid, dim3(256), 0, stream, p);
-        } else if (segs <= 8 * kSkinnySegs) {
-            if (lines)
-                hipLaunchKernelGGL((gemm_s4_skinny_kernel<8, true, EPI, BIAS>), grid, dim3(512), 0, stream, p);
-            else
-                hipLaunchKernelGGL((gemm_s4_skinny_kernel<8, false, EPI, BIAS>), grid, dim3(512), 0, stream, p);
-        } else if (segs <= 16 * kSkinnySegs) {
-            hipLaunchKernelGGL((gemm_s4_skinny_kernel<16, false, EPI, BIAS>), grid, dim3(1024), 0, stream, p);
-        } else {
-            goto tiles_path;  // K above 16384: the tile kernels take it
-        }
+        if (segs <= 4 * kSkinnySegs)
+            hipLaunchKernelGGL((gemm_s4_skinny_kernel<4, EPI, BIAS>), grid, dim3(256), 0, stream, p);
+        else
+            hipLaunchKernelGGL((gemm_s4_skinny_kernel<8, EPI, BIAS>), grid, dim3(512), 0, stream, p);
         return;
     }
-tiles_path:
+    if (kernel == kKernelRing) {
+        const uint32_t rb_all = (p.M + 15) / 16;
+        const uint32_t rb_max = p.K <= 4096 ? 4 : (p.K <= 8192 ? 2 : 1);
+        const uint32_t rb = std::min(rb_all, rb_max);
+        const uint32_t row_groups = (rb_all + rb - 1) / rb;
+        const uint32_t ntiles = (p.N + 15) / 16;
+        const uint32_t segs = (p.K / 2 + 63) / 64;
+        // wavefronts splitting K for one tile: as few as give the chip ~2048 wavefronts, slices of at
+        // least 512 bytes per row
+        uint32_t kslices = 1;
+        while (ntiles * kslices < 2048 && kslices < 4 && segs / (kslices * 2) >= (uint32_t)kRing) kslices *= 2;
+        const uint32_t groups = (ntiles + 4 / kslices - 1) / (4 / kslices);
+        const uint32_t xbytes = p.K <= 4096 ? 2048 : (p.K <= 8192 ? 4096 : 8192);
+        const uint32_t lds = 16 * rb * (xbytes + 16) + 4 * rb * 1024;
+        const uint32_t slots = 256 * std::max(1u, std::min(8u, (160u * 1024) / lds));
+        p.tiles_m = kslices;
+        p.tiles_n = (groups + slots - 1) / slots;
+        const dim3 grid((groups + p.tiles_n - 1) / p.tiles_n, row_groups);
+#define DUQ_RING(X, R) hipLaunchKernelGGL((gemm_s4_ring_kernel<X, R, EPI, BIAS>), grid, dim3(256), 0, stream, p)
+        if (xbytes == 8192) DUQ_RING(8192, 1);
+        else if (xbytes == 4096) DUQ_RING(4096, 2);
+        else if (rb == 2) DUQ_RING(2048, 2);
+        else if (rb == 3) DUQ_RING(2048, 3);
+        else DUQ_RING(2048, 4);
+#undef DUQ_RING
+        return;
+    }
     // Stream kernel with 128, 64 or 32 activation rows per workgroup: whole rounds of 256 workgroups
     // (one per CU) cost about nchunks * c + f microseconds each, c and f measured per tile height;
     // the cheapest wins.  Small problems (few column tiles) stay on the tile kernels.
     auto tiles = [&](uint32_t bm, uint32_t bn) { return ((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn); };
     int best_tm = 0;
-    if (p.M > 32 && tiles(32, 256) >= 32) {
+    if (kernel == kKernelStream) {
         const float nch = (float)((p.K + kCK - 1) / kCK);
         const float c_us[3] = {1.5f, 1.0f, 0.8f}, f_us[3] = {9.f, 7.f, 6.f};
         float best = 0.f;
@@ -1040,6 +1029,11 @@ int launch_gemm_s4(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N, u
                    const Epilogue *epi, uint16_t *y, hipStream_t stream)
 {
     if (M == 0 || N == 0) return 0;
+    {
+        const int kernel = select_gemm_kernel(M, N, K);
+        if (kernel == kKernelDecodeRows || kernel == kKernelDecodeMfma)
+            return launch_decode_s4(A, B, M, N, K, out_acc, epi, y, stream);
+    }
     GemmParams p{};
     p.A = A;
     p.B = B;

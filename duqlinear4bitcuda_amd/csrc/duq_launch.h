@@ -43,6 +43,37 @@ struct Epilogue {
 int launch_dequant(const int32_t *acc, const Epilogue &epi, uint32_t rows, uint32_t cols, uint16_t *y,
                    hipStream_t stream);
 
+// Kernel families of the int4 GEMM and the host-side rule that picks one (select_gemm_kernel: host arithmetic
+// only, exported as duq_gemm_kernel_for so that the rule can be tested without a GPU).
+enum GemmKernelId {
+    kKernelDecodeRows = 1,  // duq_decode.hip, v_dot8_i32_i4, M <= 4
+    kKernelDecodeMfma = 2,  // duq_decode.hip, MFMA, 5 <= M <= 16
+    kKernelDot = 3,         // duq_gemm.hip, M <= 4 with rows longer than 16384 elements
+    kKernelRing = 4,        // duq_gemm.hip, 17 <= M <= 256 on narrow problems
+    kKernelSkinny = 5,      // duq_gemm.hip, 5 <= M <= 16 with 512 or more column tiles
+    kKernelStream = 6,      // duq_gemm.hip, prefill
+    kKernelTile = 7,        // duq_gemm.hip, everything else (per-tile 64-bit bases: any tensor size)
+};
+int select_gemm_kernel(uint32_t M, uint32_t N, uint32_t K);
+inline bool decode_uses_rows_kernel(uint32_t M) { return M <= 4; }
+inline uint32_t decode_tiles_per_workgroup(uint32_t ntiles) { return (ntiles + 511) / 512; }
+// quantize + GEMM + dequant from binary16 activations in one launch: shapes of the rows kernel; from two rows on
+// only up to 16384 output columns (every workgroup quantizes the rows again: measured slower than two launches
+// beyond)
+inline bool decode_fp16in_one_launch(uint32_t M, uint32_t N, uint32_t K)
+{
+    return select_gemm_kernel(M, N, K) == kKernelDecodeRows && (M == 1 || N <= 16384);
+}
+// decode kernels (duq_decode.hip); the shape must be one select_gemm_kernel gives to them
+int launch_decode_s4(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N, uint32_t K, int32_t *out_acc,
+                     const Epilogue *epi, uint16_t *y, hipStream_t stream);
+// the same with binary16 activations in: per-token symmetric quantization (scale = h(h(max|x| / 7) * clip), codes
+// clamp(rint(h(x / scale)), -8, qmax)) happens inside the launch; epi.s_row is ignored; q_out / s_out (optional)
+// receive the codes and scales.  Modes DUQ_EPI_SYM and DUQ_EPI_SYM_DUAL; shapes of the rows kernel only
+// (select_gemm_kernel(M, N, K) == kKernelDecodeRows).
+int launch_decode_fp16in(const uint16_t *x, float clip, int qmax, const uint8_t *B, uint32_t M, uint32_t N, uint32_t K,
+                         const Epilogue &epi, uint16_t *y, uint8_t *q_out, uint16_t *s_out, hipStream_t stream);
+
 // GEMM: out_acc != nullptr -> int32 accumulators [M,N]; else fused epilogue into y.
 int launch_gemm_s4(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N, uint32_t K, int32_t *out_acc,
                    const Epilogue *epi, uint16_t *y, hipStream_t stream);

@@ -15,6 +15,7 @@
 //   scale: qlinear4bit/nn/quantizer.py:13, 27-31
 #include "duq_device.h"
 #include "duq_launch.h"
+#include "duq_rowquant.h"
 
 namespace duq {
 
@@ -214,13 +215,6 @@ __device__ __forceinline__ v6u bf6_block(const uint32_t (&w)[4])
     return __builtin_amdgcn_cvt_scalef32_pk32_bf6_f16(__builtin_bit_cast(v32h, pairs), 1.0f);
 }
 
-__device__ __forceinline__ uint32_t pk_absmax_u16(uint32_t acc, uint32_t w)
-{
-    const v2us a = __builtin_bit_cast(v2us, acc);
-    const v2us b = __builtin_bit_cast(v2us, w & 0x7FFF7FFFu);
-    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(a, b));
-}
-
 // BF6: the kernel also writes the E3M2 shadow of the codes (blocks of 32 elements = four
 // consecutive units); the packed words of a row meet in LDS so that the loads keep the
 // coalesced unit-per-lane pattern and a lane still converts whole blocks.  The packed nibbles
@@ -309,80 +303,17 @@ __global__ __launch_bounds__(WAVES * 64) void quantize_rows_kernel(RowParams p)
     }
     if (ASYM && m16 > 0x7C00u) a = b = __builtin_nanf("");  // torch's min / max return NaN for a row that holds one
 
-    // ---- per-token scale / zero (qlinear4bit/nn/quantizer.py:13, 27-31) ----
-    f16 s;
-    f16 z = (f16)0;
-    if (!ASYM) {
-        const f16 am = bits_to_f16((uint16_t)__builtin_bit_cast(uint32_t, a));
-        const f16 s0 = (f16)((float)am / 7.0f);
-        // torch multiplies in float32, rounds to float32, then to binary16: keep the two
-        // roundings apart (a mixed-precision FMA would round the exact product once).
-        float sc = (float)s0 * p.clip;
-        asm volatile("" : "+v"(sc));
-        s = (f16)sc;
-    } else {
-        const f16 mn = (f16)a, mx = (f16)b;  // exact: both are binary16 values
-        const f16 d = mx - mn;
-        s = (f16)((float)d / 15.0f);
-        const f16 neg = -mn;
-        const f16 qz = (f16)((float)neg / (float)s);
-        z = (f16)__builtin_rintf((float)qz);
-    }
+    // ---- per-token scale / zero and the quantization constants (duq_rowquant.h) ----
+    RowQuant<ASYM> rq;
+    rq.init(__builtin_bit_cast(uint32_t, a) & 0xFFFFu, a, b, p.clip, p.qmax);
     if (tid == 0) {
-        p.scale[row] = f16_to_bits(s);
-        if (ASYM) p.zeros[row] = f16_to_bits(shifted ? z - (f16)8.0f : z);
+        p.scale[row] = f16_to_bits(rq.s);
+        if (ASYM) p.zeros[row] = f16_to_bits(shifted ? rq.z - (f16)8.0f : rq.z);
     }
-    const float rcp = row_rcp(s);
-    const int zi = ASYM ? rint_i32((float)z) : 0;
-
-    // Rows whose statistics are finite (every realistic row) take the packed path: two
-    // elements per instruction in binary16, rounding by adding 1536 (its ulp is 1, so the
-    // sum is the nearest-even integer and its low nibble is the code).  That path cannot
-    // produce the NaN -> 0 conversions of the reference, which finite rows never need; any
-    // row with a NaN / inf statistic, a zero scale on a non-zero row, or a zero point too
-    // large for exact binary16 bounds runs the element-wise path.
-    bool fast;
-    float rcp_fast = rcp;
-    if (!ASYM) {
-        const uint32_t am_bits = __builtin_bit_cast(uint32_t, a) & 0xFFFFu;
-        const uint32_t s_bits = f16_to_bits(s) & 0x7FFFu;
-        fast = am_bits < 0x7C00u && s_bits < 0x7C00u && (s_bits != 0 || am_bits == 0);
-        if (s_bits == 0) rcp_fast = 0.f;
-    } else {
-        const uint32_t s_bits = f16_to_bits(s) & 0x7FFFu;
-        fast = fabsf(a) < 65520.f && fabsf(b) < 65520.f && s_bits != 0 && s_bits < 0x7C00u && zi >= -480 && zi <= 480;
-    }
-    const v2h lo2 = ASYM ? v2h{(f16)(float)(-zi), (f16)(float)(-zi)} : v2h{(f16)-8.0f, (f16)-8.0f};
-    const v2h hi2 = ASYM ? v2h{(f16)(float)(15 - zi), (f16)(float)(15 - zi)}
-                         : v2h{(f16)(float)p.qmax, (f16)(float)p.qmax};
-    const uint32_t zadd = ASYM ? (((uint32_t)zi & 0xFFFFu) * 0x00010001u) : 0u;
-
-    auto pair_code = [&](uint32_t w) -> uint32_t {  // two binary16 values -> codes in bits 0-3 and 16-19
-        const f16 x0 = bits_to_f16((uint16_t)(w & 0xFFFFu)), x1 = bits_to_f16((uint16_t)(w >> 16));
-        v2h q = v2h{(f16)((float)x0 * rcp_fast), (f16)((float)x1 * rcp_fast)};
-        q = __builtin_elementwise_min(__builtin_elementwise_max(q, lo2), hi2);
-        q = q + v2h{(f16)1536.0f, (f16)1536.0f};
-        uint32_t bits = __builtin_bit_cast(uint32_t, q);
-        if (ASYM) {
-            const v2us sum = __builtin_bit_cast(v2us, bits) + __builtin_bit_cast(v2us, zadd);
-            bits = __builtin_bit_cast(uint32_t, sum);
-        }
-        return bits & 0x000F000Fu;
-    };
-    auto quant8_fast = [&](const v4u raw) -> uint32_t {
-        const uint32_t b0 = pair_code(raw[0]), b1 = pair_code(raw[1]), b2 = pair_code(raw[2]), b3 = pair_code(raw[3]);
-        // gather the code bytes (bytes 0 and 2 of every pair), merge neighbours into one byte
-        const uint32_t p0 = __builtin_amdgcn_perm(b1, b0, 0x06040200u);
-        const uint32_t p1 = __builtin_amdgcn_perm(b3, b2, 0x06040200u);
-        const uint32_t t0 = p0 | (p0 >> 4), t1 = p1 | (p1 >> 4);
-        return __builtin_amdgcn_perm(t1, t0, 0x06040200u);
-    };
 
     // ---- quantize + pack: 8 elements -> one 32-bit store ----
     auto quant_unit = [&](const v4u &g) -> uint32_t {
-        uint32_t w = fast ? quant8_fast(g)
-                          : (ASYM ? quant8<kAsym>(g, 0, rcp, 0.f, 15, zi, (f16)0, (f16)0)
-                                  : quant8<kSym>(g, 0, rcp, 0.f, p.qmax, 0, (f16)0, (f16)0));
+        uint32_t w = rq.quant8(g);
         if (shifted) {
             // eight unsigned codes: sum them, then u - 8 as a signed nibble is u with bit 3 flipped
             const uint32_t pairs = (w & 0x0F0F0F0Fu) + ((w >> 4) & 0x0F0F0F0Fu);

@@ -177,6 +177,38 @@ int duq_linear4bit_forward(int32_t mode, const uint8_t *xq, const duq_half *scal
                            const duq_half *w_scale_2, const duq_half *w_zeros_2, const duq_half *bias,
                            uint32_t M, uint32_t N, uint32_t K, duq_half *y, duq_stream_t stream);
 
+/* Which kernel family duq_matmul_host_4bit / duq_linear4bit_forward run for a shape (no GPU work; for tests
+ * and tuning): 1 decode rows kernel (M <= 4), 2 decode MFMA kernel (M <= 16), 3 dot kernel (M <= 4, rows longer
+ * than 16384 elements), 4 ring kernel, 5 skinny kernel (M <= 16, wide problems), 6 stream kernel (prefill), 7 tile
+ * kernel.  Families 1-5 address the weight tensor with 32-bit byte offsets and are only picked while
+ * N * K / 2 < 2^32 - 256; larger tensors run the stream / tile kernels, whose bases are 64-bit per tile.  No
+ * counterpart in the reference (CUTLASS picks its own tile, src/kernels/gemm.cu:17-42). */
+int duq_gemm_kernel_for(uint32_t M, uint32_t N, uint32_t K);
+
+/* ---- quantize + GEMM + dequant (+ bias) from binary16 activations ---------------------- */
+
+/* No counterpart in the reference, where this is SymQuantizer.forward followed by Linear4bitSQ.forward /
+ * Linear4bitDUSQ.forward (qlinear4bit/nn/quantizer.py:10-16, qlinear4bit/nn/linear.py:42-56, 167-176: ~5 torch
+ * ops, sym_quant, matmul, sym_dequant, + bias).  y is bit-identical to duq_quantize_rows_sym followed by
+ * duq_linear4bit_forward:
+ *   x [M,K] binary16, 16-byte aligned;  clip, qmax as duq_quantize_rows_sym
+ *   mode DUQ_EPI_SYM (w_scale_2 NULL) or DUQ_EPI_SYM_DUAL;  w, w_scale_1, w_scale_2, bias, y as duq_linear4bit_forward
+ *   q_out [M,K/2] / scale_out [M]: optional (NULL): the packed codes and per-token scales, for callers that need
+ *   them as well
+ * Up to four rows (K <= 16384, N * K / 2 < 2^32 - 256; from two rows on N <= 16384) run as ONE launch: every
+ * workgroup quantizes the rows itself while its weights are in flight, and `workspace` is not touched.  Any
+ * other shape runs two launches
+ * (quantizer, then GEMM) and stages the codes and scales in `workspace`, device memory of at least
+ * duq_quantize_linear4bit_workspace_bytes(M, N, K) bytes (0 for the one-launch shapes), 16-byte aligned, that the
+ * caller provides and may reuse once the call's work has completed on the stream (DUQ_E_NULL / DUQ_E_SHAPE if it
+ * is missing or too small; codes and scales go to q_out / scale_out instead when both are given). */
+uint64_t duq_quantize_linear4bit_workspace_bytes(uint32_t M, uint32_t N, uint32_t K);
+int duq_quantize_linear4bit_forward(int32_t mode, const duq_half *x, float clip, int32_t qmax, const uint8_t *w,
+                                    const duq_half *w_scale_1, const duq_half *w_scale_2, const duq_half *bias,
+                                    uint32_t M, uint32_t N, uint32_t K, duq_half *y, uint8_t *q_out,
+                                    duq_half *scale_out, void *workspace, uint64_t workspace_bytes,
+                                    duq_stream_t stream);
+
 /* ---- asymmetric forward with exact zero-point correction (row sums) -------------------- */
 
 /* No counterpart in the reference (its asymmetric epilogue, src/kernels/quant.cu:167-168,

@@ -1,0 +1,155 @@
+"""GPU parity of the decode kernels (up to 16 activation rows) and of the quantize + GEMM + dequant entry point
+that takes binary16 activations, against the oracle, through the C ABI."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import duq_oracle as orc
+from tests import cases
+
+pytestmark = pytest.mark.gpu
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+@pytest.fixture(scope="module")
+def hip(dev):
+    from duqlinear4bitcuda_amd import _HIP
+
+    return _HIP
+
+
+# rows kernel (M <= 4: every K bucket, K and N tails), MFMA decode kernel (5..16 rows: K buckets of 4096 / 8192 /
+# 12288, tiles that end inside N), skinny kernel (512 or more column tiles), ring kernel for long rows
+SHAPES = [(1, 64, 64), (1, 20, 128), (2, 37, 4096), (3, 100, 2048), (4, 4096, 4096), (1, 4096, 4096), (1, 515, 11008),
+          (4, 130, 8192), (2, 64, 16384), (3, 33, 12352), (1, 11008, 4096),
+          (5, 64, 64), (16, 48, 128), (7, 100, 4096), (16, 4096, 4096), (16, 1000, 11008), (9, 257, 8192),
+          (13, 77, 12288), (8, 50, 2112), (16, 32, 6208),
+          (16, 11008, 4096), (6, 8200, 8192), (11, 8192, 2048),
+          (12, 40, 16384), (16, 24, 12352)]
+
+
+@pytest.mark.parametrize("M,N,K", SHAPES)
+def test_decode_kernels_against_the_oracle(hip, dev, M, N, K):
+    """int32 accumulators bit-exact, every fused epilogue bit-equal to the oracle's dequant of them, and the
+    binary16-input entry point equal to quantizer + forward (codes and scales included)."""
+    _say("decode", M, N, K, "kernel", hip.gemm_kernel_for(M, N, K))
+    rng = np.random.default_rng(M * 7 + N + K)
+    x = cases.acts_outliers(M, K, seed=M + K)
+    wq, sw = cases.weights_random_nibbles(N, K, seed=N + K)
+    sw2 = rng.uniform(0.001, 0.01, (N, 1)).astype(np.float16)
+    zw = rng.integers(0, 16, (N, 1)).astype(np.float16)
+    zw2 = rng.integers(0, 16, (N, 1)).astype(np.float16)
+    bias = rng.standard_normal(N).astype(np.float16)
+    sx = orc.sym_scales(x)
+    q = orc.sym_quant(x, sx)
+    zx = rng.integers(0, 16, (M, 1)).astype(np.float16)
+    acc = orc.matmul_s4(q, wq)
+    X, W, Q, SX, ZX = (cases.t(a, dev) for a in (x, wq, q, sx, zx))
+    SW, SW2, ZW, ZW2, B = (cases.t(a, dev) for a in (sw, sw2, zw, zw2, bias))
+    assert np.array_equal(hip.matmul(Q, W).cpu().numpy(), acc)
+    want = {
+        hip.EPI_SYM: orc.sym_dequant(acc, sx, sw),
+        hip.EPI_ASYM: orc.asym_dequant(acc, sx, zx, sw, zw),
+        hip.EPI_SYM_DUAL: orc.sym_dual_dequant(acc, sx, sw, sw2),
+        hip.EPI_ASYM_DUAL: orc.asym_dual_dequant(acc, sx, zx, sw, zw, sw2, zw2),
+    }
+    for mode, w in want.items():
+        asym, dual = mode in (hip.EPI_ASYM, hip.EPI_ASYM_DUAL), mode in (hip.EPI_SYM_DUAL, hip.EPI_ASYM_DUAL)
+        for b in (None, B):
+            y = hip.linear4bit_forward(mode, Q, SX, ZX if asym else None, W, SW, ZW if asym else None,
+                                       SW2 if dual else None, ZW2 if asym and dual else None, b)
+            assert cases.bits_equal(y.cpu().numpy(), w if b is None else orc.add_bias(w, bias)), (mode, b is not None)
+    for sw2_t, b, w in ((None, None, want[hip.EPI_SYM]), (SW2, B, orc.add_bias(want[hip.EPI_SYM_DUAL], bias))):
+        y, qf, sf = hip.quantize_linear4bit_forward(X, W, SW, sw2_t, b, return_quantized=True)
+        assert cases.bits_equal(y.cpu().numpy(), w)
+        assert np.array_equal(qf.cpu().numpy(), q) and cases.bits_equal(sf.cpu().numpy(), sx)
+        assert cases.bits_equal(hip.quantize_linear4bit_forward(X, W, SW, sw2_t, b).cpu().numpy(), w)
+
+
+def test_decode_rowsum_epilogue(hip, dev):
+    """The row-sum epilogue (mode 4) through both decode kernels."""
+    for M, N, K in ((3, 96, 512), (10, 80, 4096)):
+        _say("decode rowsum", M, N, K)
+        x = cases.acts_uniform(M, K, seed=31 + M)
+        w = (torch.randn(N, K, generator=torch.Generator().manual_seed(M)) * 0.02).to(torch.float16).numpy()
+        wq, sw, zw, adj = orc.weight_asym_shifted_from_linear(w)
+        want, *_ = orc.linear4bit_asq_rowsum_forward(x, wq, sw, zw, adj)
+        q, s, z, r = hip.quantize_rows_asym_shifted(cases.t(x, dev))
+        y = hip.linear4bit_forward_rowsum(q, s, z, r, cases.t(wq, dev), cases.t(sw, dev), cases.t(zw, dev), cases.t(adj, dev))
+        assert cases.bits_equal(y.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("M", [1, 2, 4])
+def test_fp16_input_special_rows_and_clamps(hip, dev, M):
+    """Rows of zeros, with an infinity, with a NaN, with subnormals only, clip 0.9 and both upper clamps: the
+    one-launch path gives the stand-alone quantizer's codes and scales and the oracle's outputs."""
+    _say("decode special rows", M)
+    N, K = 72, 1024
+    x = cases.acts_normal(4, K, seed=5)
+    x[0] = 0
+    x[1, 7] = np.inf
+    x[2, 100] = np.nan
+    x[3] = np.float16(3e-7)
+    x = np.ascontiguousarray(x[:M]) if M > 1 else np.ascontiguousarray(x[[1]])
+    wq, sw = cases.weights_random_nibbles(N, K, seed=9)
+    for clip, qmax in ((1.0, 6), (0.9, 7)):
+        sx = orc.sym_scales(x, clip)
+        q = orc.sym_quant(x, sx, qmax)
+        want = orc.sym_dequant(orc.matmul_s4(q, wq), sx, sw)
+        y, qf, sf = hip.quantize_linear4bit_forward(cases.t(x, dev), cases.t(wq, dev), cases.t(sw, dev), clip=clip,
+                                                    qmax=qmax, return_quantized=True)
+        assert np.array_equal(qf.cpu().numpy(), q) and cases.bits_equal(sf.cpu().numpy(), sx)
+        assert cases.bits_equal(y.cpu().numpy(), want)
+
+
+def test_fp16_input_entry_point_workspace_and_errors(dev):
+    """The C entry point itself: one-launch shapes take no workspace; others need it (too small / missing /
+    misaligned is rejected before any launch) and give the same bits; unknown modes are rejected."""
+    from duqlinear4bitcuda_amd import _lib
+
+    lib = _lib.load()
+    M, N, K = 24, 96, 256
+    x = cases.acts_normal(M, K, seed=3)
+    wq, sw = cases.weights_random_nibbles(N, K, seed=4)
+    want, *_ = orc.linear4bit_sq_forward(x, wq, sw)
+    X, W, SW = cases.t(x, dev), cases.t(wq, dev), cases.t(sw, dev)
+    y = torch.zeros(M, N, dtype=torch.float16, device=dev)
+    need = lib.duq_quantize_linear4bit_workspace_bytes(M, N, K)
+    assert need == M * K // 2 + 48 and lib.duq_quantize_linear4bit_workspace_bytes(1, N, K) == 0
+    ws = torch.zeros(need + 16, dtype=torch.uint8, device=dev)
+    st = torch.cuda.current_stream().cuda_stream
+    call = lambda mode, wsp, nbytes, m=M: lib.duq_quantize_linear4bit_forward(
+        mode, X.data_ptr(), 1.0, 6, W.data_ptr(), SW.data_ptr(), None, None, m, N, K, y.data_ptr(), None, None, wsp,
+        nbytes, st)
+    assert call(0, None, 0) == -1
+    assert call(0, ws.data_ptr(), need - 1) == -2
+    assert call(0, ws.data_ptr() + 8, need) == -5
+    assert call(1, ws.data_ptr(), need) == -4 and call(2, ws.data_ptr(), need) == -1  # asym unsupported; dual needs scale 2
+    assert call(0, ws.data_ptr(), need) == 0
+    torch.cuda.synchronize()
+    assert cases.bits_equal(y.cpu().numpy(), want)
+    # the staged codes and scales are the quantizer's
+    assert np.array_equal(ws[:M * K // 2].view(M, K // 2).cpu().numpy(), orc.sym_quant(x, orc.sym_scales(x)))
+    y.zero_()
+    assert call(0, None, 0, 3) == 0  # three rows: one launch, no workspace
+    torch.cuda.synchronize()
+    assert cases.bits_equal(y[:3].cpu().numpy(), want[:3]) and not y[3:].any()
+
+
+def test_config2_all_shapes_one_launch(hip, dev):
+    """Benchmark configuration 2 (M in {1, 4, 16}, K = 4096, N in {4096, 11008}; uniform random nibbles, scales
+    U[0.001, 0.01], activations ~N(0,1)) from binary16 activations through the single entry point."""
+    K = 4096
+    for N in (4096, 11008):
+        wq, sw = cases.weights_random_nibbles(N, K, seed=22)
+        W, SW = cases.t(wq, dev), cases.t(sw, dev)
+        for M in (1, 4, 16):
+            _say("config 2 fp16-in", M, N)
+            x = cases.acts_normal(M, K, seed=2)
+            want, *_ = orc.linear4bit_sq_forward(x, wq, sw)
+            assert cases.bits_equal(hip.quantize_linear4bit_forward(cases.t(x, dev), W, SW).cpu().numpy(), want)

@@ -212,3 +212,54 @@ def test_libtorch_header_compiles_against_the_c_abi(tmp_path):
            "-I", os.path.join(tinc, "torch", "csrc", "api", "include"), "-I", "/opt/rocm/include", str(src)]
     r = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, r.stderr[-3000:]
+
+
+def test_gemm_kernel_selection_keeps_32_bit_offsets_in_range():
+    """The dispatch rule (host arithmetic, exported as duq_gemm_kernel_for): every kernel family that addresses the
+    weight tensor with 32-bit byte offsets (decode rows 1, decode MFMA 2, dot 3, ring 4, skinny 5) is only picked
+    while the packed weights stay below 2^32 - 256 bytes; anything larger goes to the stream / tile kernels
+    (64-bit per-tile bases).  Also pins the shape buckets."""
+    from duqlinear4bitcuda_amd import _lib
+
+    f = _lib.load().duq_gemm_kernel_for
+    small = {1, 2, 3, 4, 5}
+    limit = 0xFFFFFF00
+    rng = np.random.default_rng(0)
+    ks = [64, 128, 4096, 8192, 11008, 12288, 12352, 16384, 16448, 28672, 131008]
+    for M in (1, 2, 3, 4, 5, 8, 16, 17, 32, 64, 65, 128, 256, 257, 2048):
+        for K in ks:
+            kb = K // 2
+            edge = limit // kb
+            for N in {1, 16, 4096, 11008, edge - 1, edge, edge + 1, edge + 4096, 1 << 22} | set(rng.integers(1, 1 << 22, 6).tolist()):
+                if N < 1 or N > (1 << 22):
+                    continue
+                k = f(M, int(N), K)
+                assert k in (1, 2, 3, 4, 5, 6, 7)
+                if int(N) * kb >= limit:
+                    assert k not in small, (M, N, K, k)
+    # buckets at the benchmark shapes
+    assert [f(m, 4096, 4096) for m in (1, 4, 5, 16, 17, 64, 2048)] == [1, 1, 2, 2, 4, 4, 6]
+    assert f(16, 11008, 4096) == 5 and f(16, 4096, 11008) == 2 and f(16, 28672, 8192) == 5
+    assert f(1, 28672, 8192) == 1 and f(1, 8192, 28672) == 3 and f(16, 8192, 28672) == 7
+    assert f(16, 64, 16384) == 4 and f(4, 64, 16384) == 1 and f(16, 4096, 12288) == 2
+    assert f(16, 1 << 22, 4096) == 7 and f(1, 1 << 22, 4096) == 7 and f(64, 1 << 22, 4096) in (6, 7)
+
+
+def test_fp16_input_entry_point_validation_without_launch():
+    from duqlinear4bitcuda_amd import _lib
+
+    lib = _lib.load()
+    P = 0x1000
+    f = lib.duq_quantize_linear4bit_forward
+    assert f(0, P, 1.0, 6, P, P, None, None, 4, 4, 100, P, None, None, None, 0, None) == -3      # K % 64
+    assert f(5, P, 1.0, 6, P, P, None, None, 4, 4, 64, P, None, None, None, 0, None) == -4       # mode
+    assert f(0, P, 1.0, 9, P, P, None, None, 4, 4, 64, P, None, None, None, 0, None) == -4       # qmax
+    assert f(0, None, 1.0, 6, P, P, None, None, 4, 4, 64, P, None, None, None, 0, None) == -1
+    assert f(0, P, 1.0, 6, P, None, None, None, 4, 4, 64, P, None, None, None, 0, None) == -1
+    assert f(2, P, 1.0, 6, P, P, None, None, 4, 4, 64, P, None, None, None, 0, None) == -1       # dual needs scale 2
+    assert f(0, P, 1.0, 6, P, P, None, None, 64, 4, 64, P, None, None, None, 0, None) == -1      # needs a workspace
+    assert f(0, P, 1.0, 6, P, P, None, None, 64, 4, 64, P, None, None, P, 100, None) == -2       # too small
+    assert f(0, None, 1.0, 6, None, None, None, None, 0, 4, 64, None, None, None, None, 0, None) == 0
+    assert lib.duq_quantize_linear4bit_workspace_bytes(64, 4, 64) == 64 * 32 + 128
+    assert lib.duq_quantize_linear4bit_workspace_bytes(4, 4096, 4096) == 0
+    assert lib.duq_quantize_linear4bit_workspace_bytes(4, 28672, 8192) == 4 * 4096 + 16
