@@ -1,8 +1,12 @@
 // Runs the libtorch classes of include/duq_torch.hpp on the current GPU and checks the fused
 // Linear4bit / Linear4bitDUQ forwards against the three-step path (matmul, dequant, bias add)
 // built from the same header, bit for bit.  Prints "OK <checksum>" and exits 0 on success.
+//   duq_torch_check M K N            self-consistency at a given shape
+//   duq_torch_check --fixture DIR    against the CPU oracle's expectations (raw arrays in DIR)
 #include <cstdio>
 #include <cstdlib>
+#include <string>
+#include <vector>
 
 #include "duq_torch.hpp"
 
@@ -11,8 +15,79 @@ static bool same_bits(const torch::Tensor &a, const torch::Tensor &b)
     return a.sizes() == b.sizes() && torch::equal(a.contiguous().view(torch::kInt16), b.contiguous().view(torch::kInt16));
 }
 
+// ---- fixture mode: inputs and expected outputs of the CPU oracle, handed over as raw arrays ----
+static torch::Tensor read_raw(const std::string &dir, const char *name, torch::Dtype dtype, std::vector<int64_t> shape)
+{
+    auto t = torch::empty(shape, torch::dtype(dtype));
+    const std::string path = dir + "/" + name + ".bin";
+    FILE *f = std::fopen(path.c_str(), "rb");
+    if (!f) { std::printf("FAIL cannot open %s\n", path.c_str()); std::exit(1); }
+    const size_t want = (size_t)t.numel() * t.element_size();
+    const size_t got = std::fread(t.data_ptr(), 1, want, f);
+    std::fclose(f);
+    if (got != want) { std::printf("FAIL %s holds %zu bytes, expected %zu\n", path.c_str(), got, want); std::exit(1); }
+    return t;
+}
+
+// The classes against expectations that came from the CPU oracle (the arrays of tests/golden/linear4bit_small.npz
+// written out one file each): quantizer codes and scales, from_float weight codes, and the forwards of both layers.
+static int fixture_check(const std::string &dir)
+{
+    const int64_t M = 24, K = 256, N = 48;
+    auto dev = torch::Device(torch::kCUDA, 0);
+    auto H = torch::kHalf;
+    auto x = read_raw(dir, "sym_x", H, {M, K}).to(dev);
+    auto w_float = read_raw(dir, "sym_w_float", H, {N, K});
+    auto bias = read_raw(dir, "bias", H, {N});
+    auto sw = read_raw(dir, "sym_sw", H, {N, 1}).to(dev);
+
+    torch::nn::Linear lin(torch::nn::LinearOptions(K, N).bias(true));
+    lin->to(dev, H);
+    {
+        torch::NoGradGuard ng;
+        lin->weight.copy_(w_float);
+        lin->bias.copy_(bias);
+    }
+    for (int qmax : {6, 7}) {
+        const std::string tag = "sym_q" + std::to_string(qmax);
+        duq::Quantizer4bit quant(1.0f, qmax);
+        auto p = quant.forward(x);
+        if (!torch::equal(p.quantized_x.cpu(), read_raw(dir, (tag + "_qx").c_str(), torch::kUInt8, {M, K / 2}))) {
+            std::printf("FAIL fixture quantizer codes qmax %d\n", qmax); return 1;
+        }
+        if (!same_bits(p.scale.cpu(), read_raw(dir, (tag + "_sx").c_str(), H, {M, 1}))) {
+            std::printf("FAIL fixture quantizer scales qmax %d\n", qmax); return 1;
+        }
+        auto l = duq::Linear4bit::from_float(lin, sw);  // weight preparation on the device
+        if (!torch::equal(l.weight.cpu(), read_raw(dir, "sym_w", torch::kUInt8, {N, K / 2}))) { std::puts("FAIL fixture from_float codes"); return 1; }
+        auto acc = duq::matmul(p.quantized_x, l.weight);
+        if (!torch::equal(acc.cpu(), read_raw(dir, (tag + "_acc").c_str(), torch::kInt32, {M, N}))) { std::puts("FAIL fixture accumulators"); return 1; }
+        if (!same_bits(l.forward(p).cpu(), read_raw(dir, (tag + "_y").c_str(), H, {M, N}))) {
+            std::printf("FAIL fixture Linear4bit forward qmax %d\n", qmax); return 1;
+        }
+        if (qmax == 6) {
+            // the dual-uniform layer on the same codes with a second scale vector
+            duq::Linear4bitDUQ d(K, N, true);
+            d.weight.copy_(l.weight);
+            d.weight_scale_1.copy_(sw);
+            d.weight_scale_2.copy_(read_raw(dir, "dusq_sw2", H, {N, 1}));
+            d.bias.copy_(bias);
+            if (!same_bits(d.forward(p).cpu(), read_raw(dir, "dusq_y", H, {M, N}))) { std::puts("FAIL fixture Linear4bitDUQ forward"); return 1; }
+            // and as its own from_float prepares it
+            auto d2 = duq::Linear4bitDUQ::from_float(lin, read_raw(dir, "dusq_ff_s1", H, {N, 1}).to(dev),
+                                                     read_raw(dir, "dusq_ff_s2", H, {N, 1}).to(dev));
+            if (!torch::equal(d2.weight.cpu(), read_raw(dir, "dusq_ff_w", torch::kUInt8, {N, K / 2}))) { std::puts("FAIL fixture DUQ from_float codes"); return 1; }
+            if (!same_bits(d2.forward(p).cpu(), read_raw(dir, "dusq_ff_y", H, {M, N}))) { std::puts("FAIL fixture DUQ from_float forward"); return 1; }
+        }
+    }
+    torch::cuda::synchronize();
+    std::puts("OK fixture");
+    return 0;
+}
+
 int main(int argc, char **argv)
 {
+    if (argc > 2 && std::string(argv[1]) == "--fixture") return fixture_check(argv[2]);
     const int64_t M = argc > 1 ? atoll(argv[1]) : 48, K = argc > 2 ? atoll(argv[2]) : 256, N = argc > 3 ? atoll(argv[3]) : 192;
     torch::manual_seed(1234);
     auto dev = torch::Device(torch::kCUDA, 0);

@@ -40,6 +40,15 @@ def main():
     s_w2 = (s_w.astype(np.float32) * 1.5).astype(np.float16)
     y, acc, qx, sx = orc.linear4bit_dusq_forward(x, wq, s_w, s_w2, bias)
     out.update(dusq_sw2=s_w2, dusq_y=y)
+    # the float weights themselves, and the dual-uniform layer as its from_float builds it (columns < 10 divided by
+    # the scale of those columns, the rest by the scale of the rest): for checks of the weight preparation
+    s_w1 = orc.sym_scales(w[:, :10])
+    s_w2b = orc.sym_scales(w[:, 10:])
+    codes = np.concatenate([orc.unpack_i4(orc.weight_sym_from_float(w[:, :10], s_w1)),
+                            orc.unpack_i4(orc.weight_sym_from_float(w[:, 10:], s_w2b))], axis=1)
+    wdu = orc.pack_i4(codes, sym=True)
+    y, *_ = orc.linear4bit_dusq_forward(x, wdu, s_w1, s_w2b, bias)
+    out.update(sym_w_float=w, dusq_ff_s1=s_w1, dusq_ff_s2=s_w2b, dusq_ff_w=wdu, dusq_ff_y=y)
     # asymmetric: U[0,6) activations plus one signed and one constant token
     xa = (torch.rand(M, K, generator=g) * 6)
     xa[1] = torch.randn(K, generator=g)

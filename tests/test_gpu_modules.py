@@ -57,7 +57,7 @@ def test_config1_cpu_fakequant_parity(qnn, dev):
         assert rel.max() <= 1e-3  # the stated bar; bit equality above is stronger
 
 
-@pytest.mark.parametrize("M,N", [(1, 4096), (4, 11008), (16, 4096)])
+@pytest.mark.parametrize("M,N", [(1, 4096), (4, 4096), (16, 4096), (1, 11008), (4, 11008), (16, 11008)])
 def test_config2_decode(qnn, dev, M, N):
     _say("config 2", M, N)
     K = 4096
@@ -87,8 +87,24 @@ def test_config3_prefill_against_c_oracle(qnn, dev):
     acc_want = orc_c.matmul_s4(q_want, wq)
     acc = tu.matmul(p.quantized_x, lin.weight).cpu().numpy()
     assert np.array_equal(acc, acc_want)
+    y_want = orc.sym_dequant(acc_want, s_want, sw)
     y = lin(p).cpu().numpy()
-    assert cases.bits_equal(y, orc.sym_dequant(acc_want, s_want, sw))
+    assert cases.bits_equal(y, y_want)
+    # the same forward on the 6-bit float matrix path (the benchmark's headline kernel at its headline shape),
+    # from the shadow-writing quantizer: directly against the oracle
+    lin.enable_fp6()
+    for shadow in ("only", True):
+        p6 = qnn.SymQuantizer(1.0, shadow=shadow, shadow_min_rows=1)(cases.t(x, dev))
+        assert p6.shadow_x is not None and cases.bits_equal(p6.scales_x.cpu().numpy(), s_want)
+        if shadow is True:
+            assert np.array_equal(p6.quantized_x.cpu().numpy(), q_want)
+        assert lin._use_shadow(p6)
+        assert cases.bits_equal(lin(p6).cpu().numpy(), y_want)
+    from duqlinear4bitcuda_amd import _HIP as hip
+
+    assert np.array_equal(p6.shadow_x.cpu().numpy(), orc.activation_shadow_bf6(q_want))
+    y6 = hip.linear4bit_forward_bf6(hip.EPI_SYM, p6.shadow_x, p6.scales_x, None, lin.weight_shadow, lin.weight_scales)
+    assert cases.bits_equal(y6.cpu().numpy(), y_want)
 
 
 @pytest.mark.parametrize("K,N", [(4096, 11008), (11008, 4096)])
@@ -157,16 +173,19 @@ def test_config5_decode_70b_shapes(qnn, dev, M, K, N):
     assert cases.bits_equal(y, y_want)
 
 
-def test_config5_prefill_70b_shape_by_properties(qnn, dev):
-    """M 4096, K 8192, N 28672 (1.9 T multiply-adds): sampled entries against the oracle and
-    fused == unfused."""
-    _say("config 5 prefill")
+@pytest.mark.parametrize("K,N", [(8192, 28672), (28672, 8192)])
+def test_config5_prefill_70b_shape_by_properties(qnn, dev, K, N):
+    """M 4096 at both Llama-2-70B MLP shapes (1.9 T multiply-adds each): quantizer rows and sampled accumulators
+    against the oracle, fused == unfused, and the 6-bit float matrix path == the integer path == the oracle on the
+    sampled entries."""
+    _say("config 5 prefill", K, N)
     from duqlinear4bitcuda_amd import _HIP as hip
 
-    M, K, N = 4096, 8192, 28672
+    M = 4096
     rng = np.random.default_rng(5)
     x = cases.acts_outliers(M, K, seed=5)
-    q, s = hip.quantize_rows_sym(cases.t(x, dev))
+    X = cases.t(x, dev)
+    q, s = hip.quantize_rows_sym(X)
     assert np.array_equal(q.cpu().numpy()[::97], orc.sym_quant(x[::97], orc.sym_scales(x[::97])))
     wq, sw = cases.weights_random_nibbles(N, K, seed=56)
     W, SW = cases.t(wq, dev), cases.t(sw, dev)
@@ -178,6 +197,13 @@ def test_config5_prefill_70b_shape_by_properties(qnn, dev):
     y_fused = hip.linear4bit_forward(hip.EPI_SYM, q, s, None, W, SW)
     y_unfused = hip.sym_dequant(c, s.view(-1), SW, 32)
     assert torch.equal(y_fused.view(torch.int16), y_unfused.view(torch.int16))
+    del c, y_unfused
+    y_want = orc.sym_dequant(want, s.cpu().numpy()[rows], sw[cols])
+    assert cases.bits_equal(y_fused.cpu().numpy()[np.ix_(rows, cols)], y_want)
+    _, xs, s6 = hip.quantize_rows_sym_bf6(X, with_q=False)
+    assert torch.equal(s6, s)
+    y6 = hip.linear4bit_forward_bf6(hip.EPI_SYM, xs, s6, None, hip.weight_shadow_bf6(W), SW)
+    assert torch.equal(y6.view(torch.int16), y_fused.view(torch.int16))
 
 
 def test_leading_dims_and_odd_widths(qnn, dev):
@@ -266,6 +292,22 @@ def test_libtorch_classes_fused_equals_three_step(shape):
     assert os.path.exists(exe), "tests/cpp/duq_torch_check is not built (run build())"
     r = subprocess.run([exe] + [str(v) for v in shape], capture_output=True, text=True, timeout=100)
     assert r.returncode == 0 and r.stdout.startswith("OK"), (r.returncode, r.stdout[-2000:], r.stderr[-2000:])
+
+
+@pytest.mark.gpu
+def test_libtorch_classes_against_the_oracle_fixture(tmp_path):
+    """The same program fed with the committed fixture (tests/golden/linear4bit_small.npz, every array written out
+    as a raw file): Quantizer4bit codes and scales, Linear4bit::from_float / Linear4bitDUQ::from_float weight codes
+    prepared on the device, int32 accumulators and both layers' forwards equal the CPU oracle's."""
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpp", "duq_torch_check")
+    assert os.path.exists(exe), "tests/cpp/duq_torch_check is not built (run build())"
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "linear4bit_small.npz"))
+    for k in g.files:
+        np.ascontiguousarray(g[k]).tofile(str(tmp_path / f"{k}.bin"))
+    r = subprocess.run([exe, "--fixture", str(tmp_path)], capture_output=True, text=True, timeout=100)
+    assert r.returncode == 0 and r.stdout.startswith("OK fixture"), (r.returncode, r.stdout[-2000:], r.stderr[-2000:])
 
 
 @pytest.mark.gpu
@@ -412,3 +454,63 @@ def test_step_replays_from_a_hip_graph(qnn, dev):
             want = layer(quant(x)).clone()
             torch.cuda.synchronize()
             assert noise.shape == want.shape
+
+
+@pytest.mark.gpu
+def test_weight_preparation_on_the_device_against_the_oracle(qnn, dev):
+    """from_float / from_linear of the four reference-format layers with the float layer ON the device
+    (qlinear4bit/nn/linear.py:58-78, 117-145, 178-206, 252-297): packed codes, scales and zero points equal the
+    oracle's weight preparation, and equal what the same call gives on the CPU."""
+    _say("weight prep on device")
+    K, N = 512, 192
+    g = torch.Generator().manual_seed(77)
+    lin = torch.nn.Linear(K, N, bias=True).half()
+    with torch.no_grad():
+        lin.weight.copy_((torch.randn(N, K, generator=g) * 0.02).half())
+        lin.weight[6, ::2] *= -1
+        lin.bias.copy_(torch.randn(N, generator=g).half())
+    w = lin.weight.detach().numpy()
+    lin_dev = torch.nn.Linear(K, N, bias=True).half().to(dev)
+    lin_dev.load_state_dict(lin.state_dict())
+    split = 10
+
+    def state(m):
+        return {k: v.detach().cpu().numpy() for k, v in m.state_dict().items()}
+
+    def same(a, b):
+        assert a.keys() == b.keys()
+        for k in a:
+            if a[k].dtype == np.float16:
+                assert cases.bits_equal(a[k], b[k]), k
+            else:
+                assert np.array_equal(a[k], b[k]), k
+
+    # Linear4bitSQ.from_float
+    sw = orc.sym_scales(w)
+    on_dev = state(qnn.Linear4bitSQ.from_float(lin_dev, cases.t(sw, dev)))
+    same(on_dev, state(qnn.Linear4bitSQ.from_float(lin, torch.from_numpy(sw))))
+    assert np.array_equal(on_dev["weight"], orc.weight_sym_from_float(w, sw)) and cases.bits_equal(on_dev["weight_scales"], sw)
+    assert cases.bits_equal(on_dev["bias"], lin.bias.detach().numpy())
+    # Linear4bitDUSQ.from_float
+    s1, s2 = orc.sym_scales(w[:, :split]), orc.sym_scales(w[:, split:])
+    on_dev = state(qnn.Linear4bitDUSQ.from_float(lin_dev, cases.t(s1, dev), cases.t(s2, dev)))
+    same(on_dev, state(qnn.Linear4bitDUSQ.from_float(lin, torch.from_numpy(s1), torch.from_numpy(s2))))
+    codes = np.concatenate([orc.unpack_i4(orc.weight_sym_from_float(w[:, :split], s1)),
+                            orc.unpack_i4(orc.weight_sym_from_float(w[:, split:], s2))], axis=1)
+    assert np.array_equal(on_dev["weight"], orc.pack_i4(codes, sym=True))
+    assert cases.bits_equal(on_dev["weight_scales_1"], s1) and cases.bits_equal(on_dev["weight_scales_2"], s2)
+    # Linear4bitASQ.from_linear
+    on_dev = state(qnn.Linear4bitASQ.from_linear(lin_dev))
+    same(on_dev, state(qnn.Linear4bitASQ.from_linear(lin)))
+    wa, sa, za = orc.weight_asym_from_linear(w)
+    assert np.array_equal(on_dev["weight"], wa)
+    assert cases.bits_equal(on_dev["weight_scales"], sa) and cases.bits_equal(on_dev["weight_zeros"], za)
+    # LinearQuant4bitDUASQ.from_linear
+    on_dev = state(qnn.LinearQuant4bitDUASQ.from_linear(lin_dev))
+    same(on_dev, state(qnn.LinearQuant4bitDUASQ.from_linear(lin)))
+    w1, sa1, za1 = orc.weight_asym_from_linear(w[:, :split])
+    w2, sa2, za2 = orc.weight_asym_from_linear(w[:, split:])
+    codes = np.concatenate([orc.unpack_i4(w1, signed=False), orc.unpack_i4(w2, signed=False)], axis=1)
+    assert np.array_equal(on_dev["weight"], orc.pack_i4(codes, sym=False))
+    for k, v in (("weight_scales_1", sa1), ("weight_zeros_1", za1), ("weight_scales_2", sa2), ("weight_zeros_2", za2)):
+        assert cases.bits_equal(on_dev[k], v), k
