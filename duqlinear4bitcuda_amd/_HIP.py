@@ -372,6 +372,15 @@ def gemm_kernel_for(M: int, N: int, K: int) -> int:
     return _lib.load().duq_gemm_kernel_for(M, N, K)
 
 
+def probe_read(t: torch.Tensor):
+    """Measurement aid: read every byte of ``t`` with the decode kernels' access pattern and discard them (the
+    floor of a decode launch over weights of that size)."""
+    _check("probe_read", t)
+    st = _launch(t.device, _lib.load().duq_probe_read, t.data_ptr(), t.numel() * t.element_size(), None)
+    if st:
+        _lib.check(st, "probe_read")
+
+
 def quantize_linear4bit_forward(x, w, w_scale_1, w_scale_2=None, bias=None, clip: float = 1.0, qmax: int = 6,
                                 return_quantized: bool = False):
     """SymQuantizer + Linear4bitSQ / Linear4bitDUSQ forward (qlinear4bit/nn/quantizer.py:10-16,

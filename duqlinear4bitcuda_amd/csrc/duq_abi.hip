@@ -234,6 +234,15 @@ int duq_linear4bit_forward(int32_t mode, const uint8_t *xq, const duq_half *scal
     return duq::launch_gemm_s4(xq, w, M, N, K, nullptr, &e, y, as_stream(stream));
 }
 
+int duq_probe_read(const void *src, uint64_t bytes, uint32_t *sink, duq_stream_t stream)
+{
+    if (bytes == 0) return DUQ_OK;
+    if (!src) return DUQ_E_NULL;
+    if (!aligned(src, 16)) return DUQ_E_ALIGN;
+    if (bytes >= 0xFFFFFF00ull) return DUQ_E_TOO_LARGE;
+    return duq::launch_probe_read(src, bytes, sink, as_stream(stream));
+}
+
 int duq_gemm_kernel_for(uint32_t M, uint32_t N, uint32_t K) { return duq::select_gemm_kernel(M, N, K); }
 
 uint64_t duq_quantize_linear4bit_workspace_bytes(uint32_t M, uint32_t N, uint32_t K)

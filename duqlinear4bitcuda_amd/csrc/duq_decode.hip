@@ -434,6 +434,35 @@ void launch_decode_any(DecodeParams &p, int epi, hipStream_t stream)
 
 }  // namespace
 
+// Measurement aid: the rows kernel's access pattern without its arithmetic (every lane requests 8 x 16 bytes up
+// front, a load instruction covers 1 KB, one workgroup per 32 KB) over `bytes` of memory, nothing stored.  What
+// this takes for N * K / 2 bytes is the floor of a decode launch of that size on the part.
+__global__ __launch_bounds__(256) void probe_read_kernel(const v4u *src, uint32_t nvec, uint32_t *sink)
+{
+    const uint32_t gw = (blockIdx.x * 256 + threadIdx.x) >> 6, lane = threadIdx.x & 63u;
+    const __amdgpu_buffer_rsrc_t r = make_rsrc(src, nvec * 16);
+    v4u v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const uint32_t idx = gw * 512 + i * 64 + lane;
+        v[i] = buf_load16(r, idx < nvec ? idx * 16 : kOobOffset, 0);
+    }
+    uint32_t x = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x ^= (v[i][0] ^ v[i][1]) ^ (v[i][2] ^ v[i][3]);
+    if (x == 0x9E3779B9u && sink) sink[gw & 63u] = x;  // keeps the loads alive; practically never taken
+}
+
+int launch_probe_read(const void *src, uint64_t bytes, uint32_t *sink, hipStream_t stream)
+{
+    const uint32_t nvec = (uint32_t)(bytes / 16);
+    if (nvec == 0) return 0;
+    const uint32_t waves = (nvec + 511) / 512;
+    hipLaunchKernelGGL(probe_read_kernel, dim3((waves + 3) / 4), dim3(256), 0, stream, static_cast<const v4u *>(src), nvec,
+                       sink);
+    return (int)hipGetLastError();
+}
+
 int launch_decode_s4(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N, uint32_t K, int32_t *out_acc,
                      const Epilogue *epi, uint16_t *y, hipStream_t stream)
 {

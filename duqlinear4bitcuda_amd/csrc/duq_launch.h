@@ -74,6 +74,9 @@ int launch_decode_s4(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N,
 int launch_decode_fp16in(const uint16_t *x, float clip, int qmax, const uint8_t *B, uint32_t M, uint32_t N, uint32_t K,
                          const Epilogue &epi, uint16_t *y, uint8_t *q_out, uint16_t *s_out, hipStream_t stream);
 
+// measurement aid: read `bytes` (< 4 GiB) with the decode kernels' access pattern and discard them
+int launch_probe_read(const void *src, uint64_t bytes, uint32_t *sink, hipStream_t stream);
+
 // GEMM: out_acc != nullptr -> int32 accumulators [M,N]; else fused epilogue into y.
 int launch_gemm_s4(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N, uint32_t K, int32_t *out_acc,
                    const Epilogue *epi, uint16_t *y, hipStream_t stream);

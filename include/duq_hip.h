@@ -185,6 +185,13 @@ int duq_linear4bit_forward(int32_t mode, const uint8_t *xq, const duq_half *scal
  * counterpart in the reference (CUTLASS picks its own tile, src/kernels/gemm.cu:17-42). */
 int duq_gemm_kernel_for(uint32_t M, uint32_t N, uint32_t K);
 
+/* Measurement aid, no counterpart in the reference: reads `bytes` (16-byte aligned, < 4 GiB) of device memory
+ * with the access pattern of the decode kernels (every load of a workgroup requested up front, 32 KB per
+ * workgroup) and discards them; `sink` (64 words, may be NULL) only keeps the loads alive.  Its duration for
+ * N * K / 2 bytes is the floor of a decode launch over weights of that size (bench.py reports it beside every
+ * decode row). */
+int duq_probe_read(const void *src, uint64_t bytes, uint32_t *sink, duq_stream_t stream);
+
 /* ---- quantize + GEMM + dequant (+ bias) from binary16 activations ---------------------- */
 
 /* No counterpart in the reference, where this is SymQuantizer.forward followed by Linear4bitSQ.forward /

@@ -255,8 +255,18 @@ def test_gpu_forward_bf6_extreme_accumulation(hip, dev):
     a[2, :] = 0x78                                       # alternating -8 (low nibble) / +7 (high nibble)
     a[3, :] = 0x00
     a[3, 0] = 0x01                                       # a single 1 in a row of zeros
+    # odd products added to an accumulator within 2^14 of 2^23: rows / columns of -8 that share one index holding
+    # +1 (x +1) or +7 (x +1), in the middle of the row and in its last element; an addend aligned below 24 bits
+    # would lose exactly these
+    k1, k2 = 12345, K - 1
+    def put(row, k, v):
+        byte, hi = k // 2, k % 2
+        row[byte] = (row[byte] & (0x0F if hi else 0xF0)) | ((v & 0xF) << (4 if hi else 0))
+    put(a[4], k1, 1), put(b[2], k1, 1)
+    put(a[5], k2, 7), put(b[3], k2, 1)
     acc = orc.matmul_s4(a, b)
     assert acc[0, 0] == 64 * K and acc[0, 1] == -56 * K and acc[3, 0] == -8
+    assert acc[4, 2] == 64 * (K - 1) + 1 and acc[5, 3] == 64 * (K - 1) + 7 and acc[4, 2] > (1 << 23) - (1 << 14)
     one = np.ones((max(M, N), 1), np.float16)
     T = lambda v: cases.t(v, dev)
     # scale 2^-14 per side would underflow; use the asym epilogue with zero points 0 and scales 1 / 2^-10 so that
@@ -274,6 +284,7 @@ def test_gpu_forward_bf6_extreme_accumulation(hip, dev):
                                      hip.weight_shadow_bf6(T(b)), T(one[:N]), T(zc), rowsum_x=T(np.zeros(M, np.int32)),
                                      w_rowsum_adj=T(rc)).cpu().numpy()
     assert np.array_equal(got[0].astype(np.int64), np.zeros(N, np.int64))       # row 0: acc - acc, exactly 0
+    assert int(got[4, 2]) == acc[4, 2] - acc[0, 2] == 9 and int(got[5, 3]) == acc[5, 3] - acc[0, 3] == 15
     assert cases.bits_equal(got, orc.asym_rowsum_dequant(acc, one[:M], zr, np.zeros(M, np.int32), one[:N], zc, rc))
 
 
