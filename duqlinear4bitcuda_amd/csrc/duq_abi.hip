@@ -1,9 +1,39 @@
 // extern "C" boundary of libduq_hip.so: argument validation, then the launchers.
-// Nothing here allocates, synchronises, throws or keeps state.
+// Nothing here allocates, synchronises or throws; the only state is the per-device address of the static
+// scratch array of duq_quantize_linear4bit_forward_static.
+#include <mutex>
+
 #include "../../include/duq_hip.h"
 #include "duq_launch.h"
 
+// Scratch of duq_quantize_linear4bit_forward_static: the packed codes [M, K/2] and then the per-token scales [M]
+// that its quantizer launch hands to its GEMM launch.  Every GPU the library runs on holds its own copy of the
+// array until the process ends.  In host code the name is only a handle for hipGetSymbolAddress: kernels and
+// copies get the device address that static_scratch() looks up once per device.
+static __device__ __align__(256) unsigned char scratch[DUQ_STATIC_SCRATCH_CODE_BYTES + DUQ_STATIC_SCRATCH_ROWS * 2];
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices];  // device address of `scratch` on device i, 0 until first use there
+
+// Address of the current device's copy of `scratch` (looked up on the first call per device).
+int static_scratch(unsigned char **out)
+{
+    int dev = -1;
+    if (hipError_t e = hipGetDevice(&dev)) return static_cast<int>(e);
+    if (dev < 0 || dev >= kMaxDevices) return static_cast<int>(hipErrorInvalidDevice);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        if (hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch))) return static_cast<int>(e);
+        if (!p) return static_cast<int>(hipErrorInvalidSymbol);
+        g_scratch_ptr[dev] = p;
+    }
+    *out = static_cast<unsigned char *>(g_scratch_ptr[dev]);
+    return DUQ_OK;
+}
 
 inline hipStream_t as_stream(duq_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 inline bool aligned(const void *p, uintptr_t a) { return reinterpret_cast<uintptr_t>(p) % a == 0; }
@@ -80,6 +110,8 @@ const char *duq_status_string(int status)
     case DUQ_E_MODE: return "unknown epilogue mode or unsupported qmax";
     case DUQ_E_ALIGN: return "pointer alignment requirement not met";
     case DUQ_E_TOO_LARGE: return "dimension too large";
+    case DUQ_E_SCRATCH:
+        return "input exceeds the static scratch buffer (M * K / 2 <= 8 MiB of packed codes and M <= 32768 rows)";
     default: break;
     }
     if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));
@@ -189,7 +221,7 @@ int duq_sym_dual_dequant_host(const int32_t *q, const duq_half *scale_row, const
 {
     if (rows == 0 || cols == 0) return DUQ_OK;
     if (!q || !scale_row || !scale_col_1 || !scale_col_2 || !x) return DUQ_E_NULL;
-    duq::Epilogue e{DUQ_EPI_SYM_DUAL, scale_row, nullptr, scale_col_1, nullptr, scale_col_2, nullptr, nullptr};
+    duq::Epilogue e{DUQ_EPI_SYM_DUAL, scale_row, nullptr, scale_col_1, nullptr, scale_col_2, nullptr, nullptr, nullptr, nullptr};
     return duq::launch_dequant(q, e, rows, cols, x, as_stream(stream));
 }
 
@@ -261,6 +293,28 @@ int duq_quantize_linear4bit_forward(int32_t mode, const duq_half *x, float clip,
 {
     return quantize_linear_impl(mode, x, clip, qmax, w, w_scale_1, w_scale_2, bias, M, N, K, y, q_out, scale_out,
                                 workspace, workspace_bytes, stream);
+}
+
+int duq_quantize_linear4bit_forward_static(int32_t mode, const duq_half *x, float clip, int32_t qmax, const uint8_t *w,
+                                           const duq_half *w_scale_1, const duq_half *w_scale_2, const duq_half *bias,
+                                           uint32_t M, uint32_t N, uint32_t K, duq_half *y, uint8_t *q_out,
+                                           duq_half *scale_out, duq_stream_t stream)
+{
+    // Same work as duq_quantize_linear4bit_forward with the staging buffer taken from `scratch`.  The size is
+    // checked first, for every shape, so that what a caller may pass does not depend on the launch plan.
+    if ((uint64_t)M * (K / 2) > DUQ_STATIC_SCRATCH_CODE_BYTES || M > DUQ_STATIC_SCRATCH_ROWS) return DUQ_E_SCRATCH;
+    uint8_t *q = q_out;
+    duq_half *sc = scale_out;
+    const bool staged = M != 0 && N != 0 && K != 0 && !duq::decode_fp16in_one_launch(M, N, K) && (!q_out || !scale_out);
+    if (staged) {
+        unsigned char *ws = nullptr;
+        if (int e = static_scratch(&ws)) return e;
+        // codes at the start, scales behind the largest code block: both offsets keep the 256-byte alignment
+        if (!q) q = ws;
+        if (!sc) sc = reinterpret_cast<duq_half *>(ws + DUQ_STATIC_SCRATCH_CODE_BYTES);
+    }
+    return quantize_linear_impl(mode, x, clip, qmax, w, w_scale_1, w_scale_2, bias, M, N, K, y, q, sc, nullptr, 0,
+                                stream);
 }
 
 int duq_asym_rowsum_dequant_host(const int32_t *q, const duq_half *scale_row, const duq_half *zeros_row,

@@ -15,8 +15,9 @@
  *     never exit, abort or throw.
  *
  * All pointers are DEVICE pointers on the current HIP device; inputs are borrowed,
- * outputs are caller-allocated, the library owns no memory and keeps no global state
- * (re-entrant).  No call synchronises the host.
+ * outputs are caller-allocated, the library allocates no memory and keeps no global state
+ * (re-entrant); the one exception is duq_quantize_linear4bit_forward_static and its static
+ * device array.  No call synchronises the host.
  *
  * Packed int4 layout everywhere: element i of a row is in byte i/2, low nibble first
  * (include/int4.h:86-98).
@@ -41,6 +42,7 @@ typedef void *duq_stream_t;  /* hipStream_t */
 #define DUQ_E_MODE (-4)      /* unknown epilogue mode / unsupported qmax */
 #define DUQ_E_ALIGN (-5)     /* a pointer misses the alignment the entry point documents */
 #define DUQ_E_TOO_LARGE (-6) /* a dimension exceeds what the kernels index with 32 bits: K > 131008, N > 2^22, M > 2^24 */
+#define DUQ_E_SCRATCH (-7)   /* the input does not fit the static scratch buffer of an entry point that allocates nothing */
 
 /* symmetric clamp used by the device quantizer of the reference: qmax_sym evaluates to 6
  * (include/common.h:53-54).  7 is the bound of the Python fake-quant path
@@ -215,6 +217,27 @@ int duq_quantize_linear4bit_forward(int32_t mode, const duq_half *x, float clip,
                                     uint32_t M, uint32_t N, uint32_t K, duq_half *y, uint8_t *q_out,
                                     duq_half *scale_out, void *workspace, uint64_t workspace_bytes,
                                     duq_stream_t stream);
+
+/* No counterpart in the reference.  For callers that cannot allocate device memory or carry a workspace around
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc):
+ * duq_quantize_linear4bit_forward without the workspace arguments.  The codes and scales that its quantizer
+ * launch hands to its GEMM launch are staged in a device array that is part of the library's code object
+ * (DUQ_STATIC_SCRATCH_CODE_BYTES + 2 * DUQ_STATIC_SCRATCH_ROWS bytes; every GPU the library runs on holds its own
+ * copy until the process ends).  The call allocates and frees nothing.  y (and q_out / scale_out) are bit-identical
+ * to duq_quantize_linear4bit_forward's.
+ *   limit   M * K / 2 <= DUQ_STATIC_SCRATCH_CODE_BYTES and M <= DUQ_STATIC_SCRATCH_ROWS, whatever the launch plan,
+ *           else DUQ_E_SCRATCH (e.g. 4096 x 4096 or 2048 x 8192 activations fit, 4096 x 8192 do not)
+ *   device  the stream's device must be the current one; the first staged call on a device looks the array's
+ *           address up (hipGetSymbolAddress) and should therefore not be made under stream capture
+ *   sharing all calls on one GPU share that GPU's array: two calls whose work overlaps in time (different
+ *           streams, or graphs replayed concurrently) race on it; calls ordered on one stream do not.  Nothing in
+ *           it has to start at zero: each call overwrites the part it reads. */
+#define DUQ_STATIC_SCRATCH_CODE_BYTES (8u << 20)
+#define DUQ_STATIC_SCRATCH_ROWS 32768u
+int duq_quantize_linear4bit_forward_static(int32_t mode, const duq_half *x, float clip, int32_t qmax, const uint8_t *w,
+                                           const duq_half *w_scale_1, const duq_half *w_scale_2, const duq_half *bias,
+                                           uint32_t M, uint32_t N, uint32_t K, duq_half *y, uint8_t *q_out,
+                                           duq_half *scale_out, duq_stream_t stream);
 
 /* ---- asymmetric forward with exact zero-point correction (row sums) -------------------- */
 
