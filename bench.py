@@ -16,9 +16,18 @@ nibbles with per-channel scales.
 
 Prints ONE JSON line.  ``value`` is 2*M*N*K / (time per step) in TOPS for the whole step.
 ``roofline`` describes the dominant kernel (the fused GEMM): achieved = 2*M*N*K / its own
-average duration, measured with HIP events around ``steps`` back-to-back launches on the
-launch stream, against the published dense peak of the matrix instruction it uses.  ``decode`` and ``quantizer`` report the HBM-bound parts of the metric
-(GB/s with algorithmic bytes), ``cpu_baseline`` the CPU fake-quant path on the host.
+average duration, measured with HIP events around max(steps, 1000) back-to-back launches on the
+launch stream (so the figure does not depend on ``--steps``), against the published dense peak
+of the matrix instruction it uses; ``traffic`` is read from the rocprofv3 summary under
+``profiles/``.  ``decode`` times configuration 2 as it is stated (binary16 activations in,
+quantized per token, GEMM, dequant: the single entry point ``quantize_linear4bit_forward``) with
+its algorithmic bytes 2MK + NK/2 + 2N + 2MN, beside the GEMM alone on pre-quantized activations
+and a read-only kernel over the same weight bytes (the floor of a launch of that size);
+``roofline_decode`` is the WORST of the Llama-2-7B rows.  ``quantizer`` reports the quantizer
+against HBM, ``cpu_baseline`` the CPU fake-quant path on the host.
+
+Every timed loop is preceded by PREWARM_STEPS untimed steps on top of ``--warmup`` (after an idle
+period the part needs about a millisecond of work to reach the clock it then holds).
 """
 from __future__ import annotations
 
@@ -36,8 +45,23 @@ PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, published
 PREWARM_STEPS = 300       # untimed steps before the W warm-up steps of every timed loop (about 10 ms of GPU work)
 PEAK_FP6_TOPS = 10100.0   # MI355X dense fp6 / fp4 MFMA, published
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, published
-GEMM_TRAFFIC_BYTES = (49350 + 16384) * 1024  # fetched + written per launch of the fused GEMM (rocprofv3 counters)
-GEMM_I8_TRAFFIC_BYTES = (33047 + 16384) * 1024
+EVENT_TIMED_LAUNCHES = 1000  # at least this many back-to-back launches behind every per-kernel figure
+
+
+def profile_traffic_bytes(name, kernel):
+    """HBM bytes per launch (fetched + written) of `kernel` from the rocprofv3 --pmc summary profiles/<name>:
+    the line 'dispatches N  fetch avg F KiB (max ..)  write avg W KiB (max ..)' after the kernel's name under
+    'HBM traffic per launch'.  None when the summary is not there."""
+    import re
+
+    try:
+        text = open(os.path.join(ROOT, "profiles", name)).read()
+    except OSError:
+        return None
+    at = text.find("HBM traffic per launch")
+    at = text.find(kernel, at) if at >= 0 else -1
+    m = re.search(r"fetch avg (\d+) KiB.*?write avg (\d+) KiB", text[at:]) if at >= 0 else None
+    return (int(m.group(1)) + int(m.group(2))) * 1024 if m else None
 
 
 def heavy_tail_acts(M, K, seed, frac=0.01):
@@ -115,30 +139,45 @@ def graph_time_us(fns, reps=5):
     return best
 
 
+LLAMA7B_DECODE = [(M, N, 4096) for N in (4096, 11008) for M in (1, 4, 16)]   # configuration 2
+
+
 def decode_section(dev, quick):
-    """HBM-bound decode GEMM (quantized activations in, fp16 out): weights are rotated over
-    more than 512 MB of distinct buffers so that no launch finds its weights in a cache."""
+    """HBM-bound decode at configuration 2 and around it.  Per shape, HIP-graph timed, with the weights rotated
+    over more than 512 MB of distinct buffers so that no launch finds its weights in a cache:
+      us            binary16 activations in -> per-token quantize -> GEMM -> fp16 out, the single entry point
+                    (one launch up to four rows, quantizer + GEMM launches above)
+      gemm_only_us  the GEMM + dequant launch alone on pre-quantized activations
+      read_floor_us a kernel that only reads the same N*K/2 weight bytes with the decode access pattern
+    GBps / frac_hbm use `us` and the algorithmic bytes 2MK + NK/2 + 2N + 2MN."""
     import torch
 
     from duqlinear4bitcuda_amd import _HIP as hip
 
     out = []
-    shapes = [(1, 4096, 4096), (4, 4096, 4096), (16, 4096, 4096), (1, 11008, 4096), (16, 11008, 4096)]
+    shapes = list(LLAMA7B_DECODE)
     if not quick:
-        shapes += [(4, 11008, 4096), (32, 4096, 4096), (64, 11008, 4096), (16, 4096, 11008), (1, 28672, 8192), (1, 8192, 28672),
-                   (16, 28672, 8192)]
+        shapes += [(32, 4096, 4096), (64, 11008, 4096), (1, 4096, 11008), (16, 4096, 11008), (1, 28672, 8192),
+                   (1, 8192, 28672), (16, 28672, 8192)]
     for (M, N, K) in shapes:
         wbytes = N * K // 2
         nbuf = min(96, max(3, int(600e6 // wbytes) + 1))
         ws = [torch.randint(0, 256, (N, K // 2), dtype=torch.uint8, device=dev) for _ in range(nbuf)]
-        xq = torch.randint(0, 256, (M, K // 2), dtype=torch.uint8, device=dev)
-        sx = (torch.rand(M, 1, device=dev) + 0.1).half()
-        sw = (torch.rand(N, 1, device=dev) * 0.01).half()
-        fns = [(lambda w=w: hip.linear4bit_forward(hip.EPI_SYM, xq, sx, None, w, sw)) for w in ws] * 2
-        us = graph_time_us(fns)
-        byts = M * K // 2 + wbytes + 2 * N + 2 * M + 2 * M * N
+        x = torch.randn(M, K, device=dev).half()
+        xq, sx = hip.quantize_rows_sym(x)
+        sw = (torch.rand(N, 1, device=dev) * 0.009 + 0.001).half()
+        us = graph_time_us([(lambda w=w: hip.quantize_linear4bit_forward(x, w, sw)) for w in ws] * 2)
+        us_gemm = graph_time_us([(lambda w=w: hip.linear4bit_forward(hip.EPI_SYM, xq, sx, None, w, sw)) for w in ws] * 2)
+        us_read = graph_time_us([(lambda w=w: hip.probe_read(w)) for w in ws] * 2)
+        byts = 2 * M * K + wbytes + 2 * N + 2 * M * N
         out.append({"M": M, "N": N, "K": K, "us": round(us, 3), "GBps": round(byts / us / 1e3, 1),
-                    "frac_hbm": round(byts / us / 1e3 / PEAK_HBM_GBS, 4), "weight_buffers": nbuf})
+                    "frac_hbm": round(byts / us / 1e3 / PEAK_HBM_GBS, 4),
+                    "launches": 1 if hip.quantize_linear4bit_one_launch(M, N, K) else 2,
+                    "gemm_only_us": round(us_gemm, 3),
+                    "gemm_only_GBps": round((byts - 2 * M * K + M * K // 2 + 2 * M) / us_gemm / 1e3, 1),
+                    "read_floor_us": round(us_read, 3), "read_floor_GBps": round(wbytes / us_read / 1e3, 1),
+                    "frac_of_read_floor": round(us_read / us, 4), "gemm_kernel_family": hip.gemm_kernel_for(M, N, K),
+                    "weight_buffers": nbuf})
         del ws
     return out
 
@@ -403,29 +442,33 @@ def main():
     # ---- dominant kernel (fused GEMM + dequant) alone, HIP events on the launch stream ----
     pq = quant(x)
     xs, sx = pq.shadow_x, pq.scales_x
+    n_timed = max(args.steps, EVENT_TIMED_LAUNCHES)
     gemm_us = event_time_us(lambda: hip.linear4bit_forward_bf6(hip.EPI_SYM, xs, sx, None, lin.weight_shadow, sw),
-                            args.steps, PREWARM_STEPS + args.warmup)
-    quant_us = event_time_us(lambda: hip.quantize_rows_sym_bf6(x, with_q=False), args.steps, PREWARM_STEPS + args.warmup)
+                            n_timed, PREWARM_STEPS + args.warmup)
+    # the quantizer takes less time than a launch from Python: replayed from a HIP graph instead
+    quant_us = graph_time_us([lambda: hip.quantize_rows_sym_bf6(x, with_q=False)] * 40)
     achieved = ops / gemm_us / 1e6
     roofline = {"bound": "mfma", "kernel": "gemm_bf6_kernel<8,4,0,false> (fused GEMM + dequant on v_mfma_f32_16x16x128_f8f6f4, 128 x 256 tiles)",
                 "achieved": round(achieved, 1), "peak": PEAK_FP6_TOPS, "unit": "TOP/s",
                 "frac": round(achieved / PEAK_FP6_TOPS, 4), "frac_of_int8_peak": round(achieved / PEAK_INT8_TOPS, 4),
-                "avg_kernel_us": round(gemm_us, 2),
+                "avg_kernel_us": round(gemm_us, 2), "launches_timed": n_timed,
                 "peak_note": "published dense fp6 peak; the same achieved rate is %.3f of the int8 peak (5.0 POP/s) the "
                              "integer kernel is priced against" % (achieved / PEAK_INT8_TOPS),
                 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this workload, each
                 # scaled by what the counter reads for the 256 MiB copy at the end of this script
-                "traffic": GEMM_TRAFFIC_BYTES, "traffic_source": "profiles/gemm_bf6_kernel__prefill_M2048_K4096_N4096.txt"}
+                "traffic": profile_traffic_bytes("gemm_bf6_kernel__prefill_M2048_K4096_N4096.txt", "gemm_bf6_kernel"),
+                "traffic_source": "profiles/gemm_bf6_kernel__prefill_M2048_K4096_N4096.txt"}
     xq = quant_i8(x).quantized_x
-    i8_gemm_us = event_time_us(lambda: hip.linear4bit_forward(hip.EPI_SYM, xq, sx, None, lin_i8.weight, sw), args.steps,
+    i8_gemm_us = event_time_us(lambda: hip.linear4bit_forward(hip.EPI_SYM, xq, sx, None, lin_i8.weight, sw), n_timed,
                                PREWARM_STEPS + args.warmup)
-    i8_quant_us = event_time_us(lambda: hip.quantize_rows_sym(x), args.steps, PREWARM_STEPS + args.warmup)
+    i8_quant_us = graph_time_us([lambda: hip.quantize_rows_sym(x)] * 40)
     integer_path = {"ms_per_step": round(i8_ms_per_step, 5), "TOPS": round(ops / (i8_ms_per_step * 1e-3) / 1e12, 2),
                     "kernel": "gemm_s4_stream_kernel<4,0,false> (v_mfma_i32_32x32x32_i8)", "gemm_fused_us": round(i8_gemm_us, 2),
                     "quantize_rows_sym_us": round(i8_quant_us, 2),
                     "roofline": {"bound": "mfma", "achieved": round(ops / i8_gemm_us / 1e6, 1), "peak": PEAK_INT8_TOPS,
                                  "unit": "TOP/s", "frac": round(ops / i8_gemm_us / 1e6 / PEAK_INT8_TOPS, 4),
-                                 "traffic": GEMM_I8_TRAFFIC_BYTES,
+                                 "traffic": profile_traffic_bytes("gemm_s4_stream_kernel__prefill_M2048_K4096_N4096.txt",
+                                                                  "gemm_s4_stream_kernel"),
                                  "traffic_source": "profiles/gemm_s4_stream_kernel__prefill_M2048_K4096_N4096.txt"}}
 
     decode = decode_section(dev, args.quick)
@@ -433,10 +476,16 @@ def main():
     asym = None if args.quick else asym_section(dev)
     other = None if args.quick else other_shapes_section(dev)
     int8_layer = int8_layer_section(dev, args.quick)
-    best_decode = max(decode, key=lambda d: d["GBps"])
-    roofline_decode = {"bound": "hbm", "kernel": "gemv_s4_dot_kernel (M=1) / gemm_s4_skinny_kernel (2<=M<=16) / gemm_s4_ring_kernel (17<=M<=64, long rows)", "achieved": best_decode["GBps"],
-                       "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": best_decode["frac_hbm"],
-                       "shape": {k: best_decode[k] for k in ("M", "N", "K")}, "traffic": None}
+    rows_7b = [d for d in decode if (d["M"], d["N"], d["K"]) in LLAMA7B_DECODE]
+    worst = min(rows_7b, key=lambda d: d["frac_hbm"])
+    roofline_decode = {"bound": "hbm", "kernel": "decode_rows_kernel (M <= 4, quantizer inside) / quantize_rows_kernel + "
+                                                 "decode_mfma_kernel or gemm_s4_skinny_kernel (M <= 16)",
+                       "what": "worst of the Llama-2-7B decode rows (M in {1,4,16}, K=4096, N in {4096,11008}), binary16 "
+                               "activations in, quantize + GEMM + dequant, weights never in a cache",
+                       "achieved": worst["GBps"], "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": worst["frac_hbm"],
+                       "shape": {k: worst[k] for k in ("M", "N", "K")},
+                       "best_7b_frac": max(d["frac_hbm"] for d in rows_7b),
+                       "read_floor_frac": round(worst["read_floor_GBps"] / PEAK_HBM_GBS, 4), "traffic": None}
 
     cpu = None
     if not args.no_cpu:
@@ -462,7 +511,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": "prefill Linear4bit forward (quantize + GEMM + dequant), M=2048 K=4096 N=4096, "
                                "symmetric int4 both operands, activations ~N(0,1) with 1% Student-t(3) channels",
-                   "M": M, "N": N, "K": K, "step_kernels": {"quantize_rows_sym_us": round(quant_us, 2),
+                   "M": M, "N": N, "K": K, "step_kernels": {"quantize_rows_sym_bf6_us": round(quant_us, 2),
                                                              "gemm_fused_us": round(gemm_us, 2)}},
         "roofline": roofline,
         "integer_path": integer_path,

@@ -372,6 +372,11 @@ def gemm_kernel_for(M: int, N: int, K: int) -> int:
     return _lib.load().duq_gemm_kernel_for(M, N, K)
 
 
+def quantize_linear4bit_one_launch(M: int, N: int, K: int) -> bool:
+    """True when ``quantize_linear4bit_forward`` runs the shape as one launch (no staging buffer)."""
+    return M > 0 and N > 0 and K > 0 and _lib.load().duq_quantize_linear4bit_workspace_bytes(M, N, K) == 0
+
+
 def probe_read(t: torch.Tensor):
     """Measurement aid: read every byte of ``t`` with the decode kernels' access pattern and discard them (the
     floor of a decode launch over weights of that size)."""
