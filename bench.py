@@ -264,6 +264,48 @@ def other_shapes_section(dev):
     return out
 
 
+def batched_section(dev, quick=False):
+    """Quantized activation x activation products at attention-like shapes (AsymQuantMatMul, n = 32 heads): scores
+    Q K^T (HA = HB = 2048 tokens, W = 128) and P V (HA = 2048, HB = 128, W = 2048).  HIP-graph timed: the fused
+    batched launch, the reference's two steps as two batched launches (GEMM into int32, batched dequant), one fused
+    launch per batch entry (what a loop over the single-problem entry point costs on the GPU alone, without the
+    host time of n launches), and the whole module (two quantizers + the fused launch)."""
+    import torch
+
+    from duqlinear4bitcuda_amd import _HIP as hip
+    from duqlinear4bitcuda_amd.nn import AsymQuantMatMul
+
+    out = []
+    for (n, HA, HB, W) in [(32, 2048, 2048, 128)] if quick else [(32, 2048, 2048, 128), (32, 2048, 128, 2048),
+                                                                  (32, 1, 2048, 128)]:
+        a = torch.randn(n, HA, W, device=dev).half()
+        b = torch.randn(n, HB, W, device=dev).half()
+        mod = AsymQuantMatMul()
+        qa, qb = mod.quantizer_A(a), mod.quantizer_B(b)
+        args = (hip.EPI_ASYM, qa.quantized_x, qa.scales_x, qa.zeros_x, qb.quantized_x, qb.scales_x, qb.zeros_x)
+        us_fused = graph_time_us([lambda: hip.batch_linear4bit_forward(*args)] * 6)
+        acc = hip.batched_matmul(qa.quantized_x, qb.quantized_x)
+        us_mm = graph_time_us([lambda: hip.batched_matmul(qa.quantized_x, qb.quantized_x)] * 6)
+        us_dq = graph_time_us([lambda: hip.asym_batch_dequant(acc, qa.scales_x, qa.zeros_x, qb.scales_x, qb.zeros_x)] * 6)
+
+        def loop():
+            for i in range(n):
+                hip.linear4bit_forward(hip.EPI_ASYM, qa.quantized_x[i], qa.scales_x[i], qa.zeros_x[i], qb.quantized_x[i],
+                                       qb.scales_x[i], qb.zeros_x[i])
+
+        us_loop = graph_time_us([loop] * 3)
+        us_mod = graph_time_us([lambda: mod(a, b)] * 6)
+        ops = 2.0 * n * HA * HB * W
+        byts = n * (HA * W // 2 + HB * W // 2 + 4 * (HA + HB) + 2 * HA * HB)
+        out.append({"n": n, "HA": HA, "HB": HB, "W": W, "fused_us": round(us_fused, 2),
+                    "fused_TOPS": round(ops / us_fused / 1e6, 1), "fused_GBps": round(byts / us_fused / 1e3, 1),
+                    "fused_frac_hbm": round(byts / us_fused / 1e3 / PEAK_HBM_GBS, 4),
+                    "batched_matmul_int32_us": round(us_mm, 2), "asym_batch_dequant_us": round(us_dq, 2),
+                    "per_entry_launches_us": round(us_loop, 2), "module_us": round(us_mod, 2)})
+        del a, b, acc
+    return out
+
+
 def int8_layer_section(dev, quick=False):
     """The 8-bit asymmetric layer (LinearQuant8bitASQ) at the headline shape: float32 activations, quantizer
     launch + fused GEMM launch, float32 result; the GEMM alone against the dense int8 MFMA peak."""
@@ -476,6 +518,7 @@ def main():
     asym = None if args.quick else asym_section(dev)
     other = None if args.quick else other_shapes_section(dev)
     int8_layer = int8_layer_section(dev, args.quick)
+    batched = batched_section(dev, args.quick)
     rows_7b = [d for d in decode if (d["M"], d["N"], d["K"]) in LLAMA7B_DECODE]
     worst = min(rows_7b, key=lambda d: d["frac_hbm"])
     roofline_decode = {"bound": "hbm", "kernel": "decode_rows_kernel (M <= 4, quantizer inside) / quantize_rows_kernel + "
@@ -521,6 +564,7 @@ def main():
         "asym": asym,
         "other_shapes": other,
         "int8_layer": int8_layer,
+        "batched": batched,
         "cpu_baseline": cpu,
         "device": {"name": props.name, "arch": props.gcnArchName, "cus": props.multi_processor_count},
     }

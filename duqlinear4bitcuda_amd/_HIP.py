@@ -85,6 +85,25 @@ def matmul(A: torch.Tensor, B: torch.Tensor) -> torch.Tensor:
     return C
 
 
+def batched_matmul(A: torch.Tensor, B: torch.Tensor) -> torch.Tensor:
+    """A [n, M, K/2], B [n, N, K/2] packed -> int32 [n, M, N], entry i = matmul(A[i], B[i]), in one launch
+    (bindings.cpp:46-86; the reference hands CUTLASS pointer arrays built from the same strides and prints two
+    lines to stdout, which is left out)."""
+    _check("batched_matmul", A, B)
+    _check_dtype("batched_matmul", A, "A", torch.uint8)
+    _check_dtype("batched_matmul", B, "B", torch.uint8)
+    if A.dim() != 3 or B.dim() != 3:
+        raise RuntimeError(f"batched_matmul: expected A [n, M, K/2] and B [n, N, K/2], got {tuple(A.shape)} and {tuple(B.shape)}")
+    n, M, kb = A.shape
+    N = B.size(1)
+    if B.size(0) != n or B.size(2) != kb:
+        raise RuntimeError(f"batched_matmul: batch or packed K differs: A {tuple(A.shape)} vs B {tuple(B.shape)}")
+    C = torch.empty((n, M, N), dtype=torch.int32, device=A.device)
+    st = _launch(A.device, _lib.load().duq_batch_matmul_host_4bit, _ptr(A), _ptr(B), M, N, kb * 2, _ptr(C), n)
+    _lib.check(st, "batched_matmul")
+    return C
+
+
 def sym_quant(x: torch.Tensor, scale: torch.Tensor, qmax: int = 6) -> torch.Tensor:
     """int4Pack(clamp(rint(x / scale), -8, qmax)) -> uint8 [M, ceil(K/2)] (bindings.cpp:88-105).
     ``qmax`` defaults to 6, the bound the reference device kernel really applies
@@ -233,14 +252,9 @@ def asym_batch_dequant(q, scale_row, zeros_row, scale_col, zeros_col, bits: int 
             raise RuntimeError(f"asym_batch_dequant: expected {n} to have size {want} at dimension 1, got {tuple(t.shape)}")
     _check_bits("asym_batch_dequant", bits)
     x = torch.empty(q.shape, dtype=torch.float16, device=q.device)
-    fn = _lib.load().duq_asym_dequant_host
-    esz = 2
-    for b in range(batches):
-        st = _launch(q.device, fn, q.data_ptr() + b * rows * cols * 4, scale_row.data_ptr() + b * rows * esz,
-                     zeros_row.data_ptr() + b * rows * esz, scale_col.data_ptr() + b * cols * esz,
-                     zeros_col.data_ptr() + b * cols * esz, rows, cols, x.data_ptr() + b * rows * cols * esz)
-        if st:
-            _lib.check(st, "asym_batch_dequant")
+    st = _launch(q.device, _lib.load().duq_asym_batch_dequant_host, _ptr(q), _ptr(scale_row), _ptr(zeros_row),
+                 _ptr(scale_col), _ptr(zeros_col), batches, rows, cols, _ptr(x))
+    _lib.check(st, "asym_batch_dequant")
     return x
 
 
@@ -361,6 +375,43 @@ def linear4bit_forward(mode, xq, scale_x, zeros_x, w, w_scale_1, w_zeros_1=None,
     st = _launch(dev, _lib.load().duq_linear4bit_forward, mode, xq.data_ptr(), scale_x.data_ptr(), pz or None,
                  w.data_ptr(), w_scale_1.data_ptr(), ptrs[0] or None, ptrs[1] or None, ptrs[2] or None,
                  ptrs[3] or None, M, N, kb * 2, y.data_ptr())
+    if st:
+        _lib.check(st, name)
+    return y
+
+
+def batch_linear4bit_forward(mode, xq, scale_x, zeros_x, w, w_scale_1, w_zeros_1=None, w_scale_2=None, w_zeros_2=None,
+                             bias=None):
+    """``linear4bit_forward`` over a batch in one launch: ``xq`` uint8 [n, M, K/2], ``w`` uint8 [n, N, K/2],
+    per-row tensors n * M and per-column tensors (and bias) n * N fp16 values, contiguous over the batch.
+    Returns fp16 [n, M, N], entry i bit-identical to ``linear4bit_forward`` on the i-th slices."""
+    name = "batch_linear4bit_forward"
+    if not isinstance(xq, torch.Tensor) or not isinstance(w, torch.Tensor):
+        raise RuntimeError(f"{name}: xq and w must be tensors")
+    dev = xq.device
+    _fast_check(name, "xq", xq, _U8, None)
+    _fast_check(name, "w", w, _U8, dev)
+    if xq.dim() != 3 or w.dim() != 3 or w.shape[0] != xq.shape[0] or w.shape[2] != xq.shape[2]:
+        raise RuntimeError(f"{name}: expected xq [n, M, K/2] and w [n, N, K/2], got {tuple(xq.shape)} and {tuple(w.shape)}")
+    n, M, kb = xq.shape
+    N = w.shape[1]
+    ptrs = []
+    for t, what, cnt, need in ((scale_x, "scale_x", n * M, True), (zeros_x, "zeros_x", n * M, False),
+                               (w_scale_1, "w_scale_1", n * N, True), (w_zeros_1, "w_zeros_1", n * N, False),
+                               (w_scale_2, "w_scale_2", n * N, False), (w_zeros_2, "w_zeros_2", n * N, False),
+                               (bias, "bias", n * N, False)):
+        if t is None:
+            if need:
+                raise RuntimeError(f"{name}: {what} is required")
+            ptrs.append(None)
+            continue
+        _fast_check(name, what, t, _F16, dev)
+        if t.numel() != cnt:
+            raise RuntimeError(f"{name}: expected {what} to hold {cnt} values, got {tuple(t.shape)}")
+        ptrs.append(t.data_ptr())
+    y = torch.empty((n, M, N), dtype=_F16, device=dev)
+    st = _launch(dev, _lib.load().duq_batch_linear4bit_forward, mode, xq.data_ptr(), ptrs[0], ptrs[1], w.data_ptr(),
+                 ptrs[2], ptrs[3], ptrs[4], ptrs[5], ptrs[6], n, M, N, kb * 2, y.data_ptr())
     if st:
         _lib.check(st, name)
     return y

@@ -28,6 +28,10 @@ PROTOTYPES = {
     "duq_quantize_rows_sym": [_c_p, _c_u32, _c_u32, ctypes.c_float, _c_i32, _c_p, _c_p, _c_p],
     "duq_quantize_rows_asym": [_c_p, _c_u32, _c_u32, _c_p, _c_p, _c_p, _c_p],
     "duq_matmul_host_4bit": [_c_p, _c_p, _c_u32, _c_u32, _c_u32, _c_p, _c_p],
+    "duq_batch_matmul_host_4bit": [_c_p, _c_p, _c_u32, _c_u32, _c_u32, _c_p, _c_u32, _c_p],
+    "duq_asym_batch_dequant_host": [_c_p, _c_p, _c_p, _c_p, _c_p, _c_u32, _c_u32, _c_u32, _c_p, _c_p],
+    "duq_batch_linear4bit_forward": [_c_i32, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_u32, _c_u32,
+                                     _c_u32, _c_u32, _c_p, _c_p],
     "duq_sym_dequant_host": [_c_p, _c_p, _c_p, _c_u32, _c_u32, _c_p, _c_p],
     "duq_sym_dual_dequant_host": [_c_p, _c_p, _c_p, _c_p, _c_u32, _c_u32, _c_p, _c_p],
     "duq_asym_dequant_host": [_c_p, _c_p, _c_p, _c_p, _c_p, _c_u32, _c_u32, _c_p, _c_p],

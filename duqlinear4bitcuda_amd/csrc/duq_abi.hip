@@ -266,6 +266,84 @@ int duq_linear4bit_forward(int32_t mode, const uint8_t *xq, const duq_half *scal
     return duq::launch_gemm_s4(xq, w, M, N, K, nullptr, &e, y, as_stream(stream));
 }
 
+// One launch holds at most 65535 batch entries (grid limit of the second and third dimension): longer batches
+// run in slices, every tensor moved on by whole entries.
+constexpr uint32_t kBatchSlice = 65535;
+
+static void advance(duq::Epilogue &e, uint64_t entries, uint32_t rows, uint32_t cols)
+{
+    const uint64_t r = entries * rows, c = entries * cols;
+    if (e.s_row) e.s_row += r;
+    if (e.z_row) e.z_row += r;
+    if (e.rs_row) e.rs_row += r;
+    if (e.s_col_1) e.s_col_1 += c;
+    if (e.z_col_1) e.z_col_1 += c;
+    if (e.s_col_2) e.s_col_2 += c;
+    if (e.z_col_2) e.z_col_2 += c;
+    if (e.bias) e.bias += c;
+    if (e.rs_col) e.rs_col += c;
+}
+
+int duq_batch_matmul_host_4bit(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N, uint32_t K, int32_t *C,
+                               uint32_t batch_count, duq_stream_t stream)
+{
+    if (batch_count == 0) return DUQ_OK;
+    if (int e = check_gemm(A, B, M, N, K)) return e;
+    if (M == 0 || N == 0) return DUQ_OK;
+    if (!C) return DUQ_E_NULL;
+    for (uint32_t b0 = 0; b0 < batch_count; b0 += kBatchSlice) {
+        const uint32_t nb = batch_count - b0 < kBatchSlice ? batch_count - b0 : kBatchSlice;
+        if (int st = duq::launch_gemm_s4_batched(A + (uint64_t)b0 * M * (K / 2), B + (uint64_t)b0 * N * (K / 2), M, N, K,
+                                                 nb, C + (uint64_t)b0 * M * N, nullptr, nullptr, as_stream(stream)))
+            return st;
+    }
+    return DUQ_OK;
+}
+
+int duq_asym_batch_dequant_host(const int32_t *q, const duq_half *scale_row, const duq_half *zeros_row,
+                                const duq_half *scale_col, const duq_half *zeros_col, uint32_t batches,
+                                uint32_t rows, uint32_t cols, duq_half *x, duq_stream_t stream)
+{
+    if (batches == 0 || rows == 0 || cols == 0) return DUQ_OK;
+    if (!q || !scale_row || !zeros_row || !scale_col || !zeros_col || !x) return DUQ_E_NULL;
+    duq::Epilogue e{DUQ_EPI_ASYM, scale_row, zeros_row, scale_col, zeros_col, nullptr, nullptr, nullptr, nullptr, nullptr};
+    for (uint32_t b0 = 0; b0 < batches; b0 += kBatchSlice) {
+        const uint32_t nb = batches - b0 < kBatchSlice ? batches - b0 : kBatchSlice;
+        if (int st = duq::launch_dequant_batched(q + (uint64_t)b0 * rows * cols, e, nb, rows, cols,
+                                                 x + (uint64_t)b0 * rows * cols, as_stream(stream)))
+            return st;
+        advance(e, nb, rows, cols);
+    }
+    return DUQ_OK;
+}
+
+int duq_batch_linear4bit_forward(int32_t mode, const uint8_t *xq, const duq_half *scale_x, const duq_half *zeros_x,
+                                 const uint8_t *w, const duq_half *w_scale_1, const duq_half *w_zeros_1,
+                                 const duq_half *w_scale_2, const duq_half *w_zeros_2, const duq_half *bias,
+                                 uint32_t batch_count, uint32_t M, uint32_t N, uint32_t K, duq_half *y,
+                                 duq_stream_t stream)
+{
+    if (mode < DUQ_EPI_SYM || mode > DUQ_EPI_ASYM_DUAL) return DUQ_E_MODE;
+    if (batch_count == 0) return DUQ_OK;
+    if (int e = check_gemm(xq, w, M, N, K)) return e;
+    if (M == 0 || N == 0) return DUQ_OK;
+    if (!scale_x || !w_scale_1 || !y) return DUQ_E_NULL;
+    const bool asym = mode == DUQ_EPI_ASYM || mode == DUQ_EPI_ASYM_DUAL;
+    const bool dual = mode == DUQ_EPI_SYM_DUAL || mode == DUQ_EPI_ASYM_DUAL;
+    if (asym && (!zeros_x || !w_zeros_1)) return DUQ_E_NULL;
+    if (dual && !w_scale_2) return DUQ_E_NULL;
+    if (asym && dual && !w_zeros_2) return DUQ_E_NULL;
+    duq::Epilogue e{mode, scale_x, zeros_x, w_scale_1, w_zeros_1, w_scale_2, w_zeros_2, bias, nullptr, nullptr};
+    for (uint32_t b0 = 0; b0 < batch_count; b0 += kBatchSlice) {
+        const uint32_t nb = batch_count - b0 < kBatchSlice ? batch_count - b0 : kBatchSlice;
+        if (int st = duq::launch_gemm_s4_batched(xq + (uint64_t)b0 * M * (K / 2), w + (uint64_t)b0 * N * (K / 2), M, N, K,
+                                                 nb, nullptr, &e, y + (uint64_t)b0 * M * N, as_stream(stream)))
+            return st;
+        advance(e, nb, M, N);
+    }
+    return DUQ_OK;
+}
+
 int duq_probe_read(const void *src, uint64_t bytes, uint32_t *sink, duq_stream_t stream)
 {
     if (bytes == 0) return DUQ_OK;

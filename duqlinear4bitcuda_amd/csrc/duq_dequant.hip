@@ -11,6 +11,11 @@ __global__ __launch_bounds__(256) void dequant_kernel(const int32_t *__restrict_
                                                       uint32_t cols, uint16_t *__restrict__ y)
 {
     constexpr int E = VEC ? 8 : 1;
+    if (blockIdx.y) {  // batched launch: one accumulator matrix per blockIdx.y
+        acc += (uint64_t)blockIdx.y * rows * cols;
+        y += (uint64_t)blockIdx.y * rows * cols;
+        batch_shift(epi, blockIdx.y, rows, cols);
+    }
     const uint32_t perRow = cols / E;
     const uint64_t total = (uint64_t)rows * perRow;
     for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
@@ -43,30 +48,39 @@ __global__ __launch_bounds__(256) void dequant_kernel(const int32_t *__restrict_
 }
 
 template <int MODE, bool BIAS>
-static void launch_mode(const int32_t *acc, const Epilogue &epi, uint32_t rows, uint32_t cols, uint16_t *y,
-                        hipStream_t stream)
+static void launch_mode(const int32_t *acc, const Epilogue &epi, uint32_t batches, uint32_t rows, uint32_t cols,
+                        uint16_t *y, hipStream_t stream)
 {
+    // (a batch entry starts rows * cols elements after the previous one: with cols % 8 == 0 every entry keeps the
+    // alignment of the first)
     const bool vec = (cols % 8 == 0) && (reinterpret_cast<uintptr_t>(acc) % 16 == 0) &&
                      (reinterpret_cast<uintptr_t>(y) % 16 == 0);
     const uint64_t total = (uint64_t)rows * (vec ? cols / 8 : cols);
     const uint32_t blocks = (uint32_t)std::min<uint64_t>((total + 255) / 256, 1u << 20);
+    const dim3 grid(blocks, batches);
     if (vec)
-        hipLaunchKernelGGL((dequant_kernel<MODE, BIAS, true>), dim3(blocks), dim3(256), 0, stream, acc, epi, rows, cols, y);
+        hipLaunchKernelGGL((dequant_kernel<MODE, BIAS, true>), grid, dim3(256), 0, stream, acc, epi, rows, cols, y);
     else
-        hipLaunchKernelGGL((dequant_kernel<MODE, BIAS, false>), dim3(blocks), dim3(256), 0, stream, acc, epi, rows, cols, y);
+        hipLaunchKernelGGL((dequant_kernel<MODE, BIAS, false>), grid, dim3(256), 0, stream, acc, epi, rows, cols, y);
 }
 
 int launch_dequant(const int32_t *acc, const Epilogue &epi, uint32_t rows, uint32_t cols, uint16_t *y,
                    hipStream_t stream)
 {
-    if (rows == 0 || cols == 0) return 0;
+    return launch_dequant_batched(acc, epi, 1, rows, cols, y, stream);
+}
+
+int launch_dequant_batched(const int32_t *acc, const Epilogue &epi, uint32_t batches, uint32_t rows, uint32_t cols,
+                           uint16_t *y, hipStream_t stream)
+{
+    if (rows == 0 || cols == 0 || batches == 0) return 0;
     const bool bias = epi.bias != nullptr;
 #define DUQ_DQ(M)                                                          \
     case M:                                                                \
         if (bias)                                                          \
-            launch_mode<M, true>(acc, epi, rows, cols, y, stream);         \
+            launch_mode<M, true>(acc, epi, batches, rows, cols, y, stream);  \
         else                                                               \
-            launch_mode<M, false>(acc, epi, rows, cols, y, stream);        \
+            launch_mode<M, false>(acc, epi, batches, rows, cols, y, stream); \
         break;
     switch (epi.mode) {
         DUQ_DQ(0)

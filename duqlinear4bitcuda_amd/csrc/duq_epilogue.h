@@ -29,6 +29,22 @@ struct RowEpi {
     int rs;  // mode 4
 };
 
+// Batched launches (one problem per blockIdx.z / blockIdx.y, every tensor contiguous over the batch): move the
+// per-row arrays by b * rows and the per-column ones by b * cols elements.
+__device__ __forceinline__ void batch_shift(Epilogue &e, uint32_t b, uint32_t rows, uint32_t cols)
+{
+    const uint64_t r = (uint64_t)b * rows, c = (uint64_t)b * cols;
+    if (e.s_row) e.s_row += r;
+    if (e.z_row) e.z_row += r;
+    if (e.rs_row) e.rs_row += r;
+    if (e.s_col_1) e.s_col_1 += c;
+    if (e.z_col_1) e.z_col_1 += c;
+    if (e.s_col_2) e.s_col_2 += c;
+    if (e.z_col_2) e.z_col_2 += c;
+    if (e.bias) e.bias += c;
+    if (e.rs_col) e.rs_col += c;
+}
+
 template <int MODE>
 __device__ __forceinline__ RowEpi load_row(const Epilogue &e, uint32_t row)
 {

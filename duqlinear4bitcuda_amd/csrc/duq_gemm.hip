@@ -44,6 +44,17 @@ struct GemmParams {
     uint32_t tiles_m, tiles_n;
 };
 
+// Batched launch: problem blockIdx.z of a batch whose tensors are contiguous ([batch, M, K/2], [batch, N, K/2],
+// [batch, M, N], per-row arrays [batch, M], per-column arrays [batch, N]).
+__device__ __forceinline__ void batch_shift(GemmParams &p, uint32_t b)
+{
+    p.A += (uint64_t)b * p.M * (p.K >> 1);
+    p.B += (uint64_t)b * p.N * (p.K >> 1);
+    if (p.C) p.C += (uint64_t)b * p.M * p.N;
+    if (p.y) p.y += (uint64_t)b * p.M * p.N;
+    batch_shift(p.epi, b, p.M, p.N);
+}
+
 __device__ __forceinline__ void expand_nibbles(const v4u w, v4u &even, v4u &odd)
 {
 #pragma unroll
@@ -107,6 +118,7 @@ __global__ __launch_bounds__(256) void gemm_s4_tile_kernel(GemmParams p)
 
     __shared__ __attribute__((aligned(16))) uint8_t lds[2][(BM + BN) * kLdsStride];
 
+    if (blockIdx.z) batch_shift(p, blockIdx.z);
     uint32_t tile_m, tile_n;
     tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
@@ -270,6 +282,7 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
 
     __shared__ __attribute__((aligned(16))) uint8_t lds[3 * kBuf];
 
+    if (blockIdx.z) batch_shift(p, blockIdx.z);
     uint32_t tile_m, tile_n;
     tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
@@ -918,10 +931,13 @@ int select_gemm_kernel(uint32_t M, uint32_t N, uint32_t K)
     return kKernelTile;
 }
 
+// batch > 1: `batch` problems of one shape, tensors contiguous over the batch, one launch (blockIdx.z is the
+// problem): stream or tile kernel only, the choice made on the tiles of the whole batch.
 template <int EPI, bool BIAS>
-static void launch_epi(GemmParams &p, hipStream_t stream)
+static void launch_epi(GemmParams &p, hipStream_t stream, uint32_t batch = 1)
 {
-    const int kernel = select_gemm_kernel(p.M, p.N, p.K);
+    const int kernel = batch > 1 ? (p.M > 32 && ((p.M + 31) / 32) * ((p.N + 255) / 256) * batch >= 32 ? kKernelStream : kKernelTile)
+                                 : select_gemm_kernel(p.M, p.N, p.K);
     if (kernel == kKernelDot) {
         const uint32_t xstride = ((p.K / 2 + 127) / 128) * 128;
         const dim3 grid((p.N + 7) / 8);
@@ -982,7 +998,7 @@ static void launch_epi(GemmParams &p, hipStream_t stream)
     // Stream kernel with 128, 64 or 32 activation rows per workgroup: whole rounds of 256 workgroups
     // (one per CU) cost about nchunks * c + f microseconds each, c and f measured per tile height;
     // the cheapest wins.  Small problems (few column tiles) stay on the tile kernels.
-    auto tiles = [&](uint32_t bm, uint32_t bn) { return ((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn); };
+    auto tiles = [&](uint32_t bm, uint32_t bn) { return ((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn) * batch; };
     int best_tm = 0;
     if (kernel == kKernelStream) {
         const float nch = (float)((p.K + kCK - 1) / kCK);
@@ -997,30 +1013,39 @@ static void launch_epi(GemmParams &p, hipStream_t stream)
             }
         }
     }
+    bool narrow = false;
+    if (batch > 1 && best_tm) {
+        // measured at attention-like batches (32 problems): rows of at most 256 elements leave a workgroup mostly
+        // prologue and epilogue, and 64-row tiles put three workgroups on a CU that overlap them (2048 x 2048 x
+        // 128: 90 us against 115 / 109 us with 128- / 32-row tiles); at most 128 columns fill half of a 256-wide
+        // tile, the 128 x 128 tile kernel is 15 % faster there (2048 x 128 x 2048: 32 against 37 us)
+        if (p.K <= 256 && p.M > 32) best_tm = 2;
+        else if (p.N <= 128 && p.M > 64) { best_tm = 0; narrow = true; }
+    }
     if (best_tm) {
         p.tiles_m = (p.M + 32 * best_tm - 1) / (32 * best_tm);
         p.tiles_n = (p.N + 255) / 256;
-        const dim3 grid(p.tiles_m * p.tiles_n);
+        const dim3 grid(p.tiles_m * p.tiles_n, 1, batch);
         if (best_tm == 4)
             hipLaunchKernelGGL((gemm_s4_stream_kernel<4, EPI, BIAS>), grid, dim3(256), 0, stream, p);
         else if (best_tm == 2)
             hipLaunchKernelGGL((gemm_s4_stream_kernel<2, EPI, BIAS>), grid, dim3(256), 0, stream, p);
         else
             hipLaunchKernelGGL((gemm_s4_stream_kernel<1, EPI, BIAS>), grid, dim3(256), 0, stream, p);
-    } else if (tiles(128, 256) >= 256 && p.M > 64) {
+    } else if (!narrow && tiles(128, 256) >= 256 && p.M > 64) {
         p.tiles_m = (p.M + 127) / 128;
         p.tiles_n = (p.N + 255) / 256;
-        hipLaunchKernelGGL((gemm_s4_tile_kernel<128, 256, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0,
+        hipLaunchKernelGGL((gemm_s4_tile_kernel<128, 256, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(256), 0,
                            stream, p);
-    } else if (tiles(128, 128) >= 256 && p.M > 64) {
+    } else if (narrow || (tiles(128, 128) >= 256 && p.M > 64)) {
         p.tiles_m = (p.M + 127) / 128;
         p.tiles_n = (p.N + 127) / 128;
-        hipLaunchKernelGGL((gemm_s4_tile_kernel<128, 128, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0,
+        hipLaunchKernelGGL((gemm_s4_tile_kernel<128, 128, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(256), 0,
                            stream, p);
     } else {
         p.tiles_m = (p.M + 63) / 64;
         p.tiles_n = (p.N + 63) / 64;
-        hipLaunchKernelGGL((gemm_s4_tile_kernel<64, 64, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0,
+        hipLaunchKernelGGL((gemm_s4_tile_kernel<64, 64, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(256), 0,
                            stream, p);
     }
 }
@@ -1028,8 +1053,14 @@ static void launch_epi(GemmParams &p, hipStream_t stream)
 int launch_gemm_s4(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N, uint32_t K, int32_t *out_acc,
                    const Epilogue *epi, uint16_t *y, hipStream_t stream)
 {
-    if (M == 0 || N == 0) return 0;
-    {
+    return launch_gemm_s4_batched(A, B, M, N, K, 1, out_acc, epi, y, stream);
+}
+
+int launch_gemm_s4_batched(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N, uint32_t K, uint32_t batch,
+                           int32_t *out_acc, const Epilogue *epi, uint16_t *y, hipStream_t stream)
+{
+    if (M == 0 || N == 0 || batch == 0) return 0;
+    if (batch == 1) {
         const int kernel = select_gemm_kernel(M, N, K);
         if (kernel == kKernelDecodeRows || kernel == kKernelDecodeMfma)
             return launch_decode_s4(A, B, M, N, K, out_acc, epi, y, stream);
@@ -1044,15 +1075,15 @@ int launch_gemm_s4(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N, u
     p.y = y;
     if (epi) p.epi = *epi;
     if (out_acc) {
-        launch_epi<-1, false>(p, stream);
+        launch_epi<-1, false>(p, stream, batch);
     } else {
         const bool bias = epi->bias != nullptr;
 #define DUQ_GEMM(MODE)                             \
     case MODE:                                     \
         if (bias)                                  \
-            launch_epi<MODE, true>(p, stream);     \
+            launch_epi<MODE, true>(p, stream, batch);  \
         else                                       \
-            launch_epi<MODE, false>(p, stream);    \
+            launch_epi<MODE, false>(p, stream, batch); \
         break;
         switch (epi->mode) {
             DUQ_GEMM(0)

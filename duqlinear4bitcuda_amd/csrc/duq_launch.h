@@ -42,6 +42,10 @@ struct Epilogue {
 
 int launch_dequant(const int32_t *acc, const Epilogue &epi, uint32_t rows, uint32_t cols, uint16_t *y,
                    hipStream_t stream);
+// the same over `batches` accumulator matrices [batches, rows, cols] in one launch, every batch entry with its
+// own per-row [batches, rows] and per-column [batches, cols] parameters.  batches <= 65535.
+int launch_dequant_batched(const int32_t *acc, const Epilogue &epi, uint32_t batches, uint32_t rows, uint32_t cols,
+                           uint16_t *y, hipStream_t stream);
 
 // Kernel families of the int4 GEMM and the host-side rule that picks one (select_gemm_kernel: host arithmetic
 // only, exported as duq_gemm_kernel_for so that the rule can be tested without a GPU).
@@ -80,6 +84,10 @@ int launch_probe_read(const void *src, uint64_t bytes, uint32_t *sink, hipStream
 // GEMM: out_acc != nullptr -> int32 accumulators [M,N]; else fused epilogue into y.
 int launch_gemm_s4(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N, uint32_t K, int32_t *out_acc,
                    const Epilogue *epi, uint16_t *y, hipStream_t stream);
+// `batch` problems of one shape in one launch: A [batch, M, K/2], B [batch, N, K/2], out [batch, M, N], the
+// epilogue's per-row arrays [batch, M] and per-column arrays [batch, N], all contiguous.  batch <= 65535.
+int launch_gemm_s4_batched(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N, uint32_t K, uint32_t batch,
+                           int32_t *out_acc, const Epilogue *epi, uint16_t *y, hipStream_t stream);
 
 
 // 6-bit float (E3M2) shadows of packed-int4 tensors and the GEMM that multiplies them

@@ -3,9 +3,11 @@
 int4 x int4 and dequantized.  Rows of ``B`` play the part of weight rows: the result is
 ``A @ B^T`` over the last dimension.
 
-Each batch entry runs one fused GEMM + dequant launch (the reference runs a GEMM per batch
-entry into a zero-filled int32 tensor, pads B's rows to a multiple of 32, then one batched
-dequant: matmul.py:46-63); the bits are the same.
+A whole batch runs as ONE fused GEMM + dequant launch, whatever the number of batch entries
+(the reference runs a GEMM per batch entry into a zero-filled int32 tensor, pads B's rows to a
+multiple of 32, then one batched dequant: matmul.py:46-63); the bits are the same.  With
+``fused = False`` the steps are the reference's: one batched GEMM launch into int32, one
+batched dequant launch.
 """
 from __future__ import annotations
 
@@ -19,7 +21,8 @@ from .quantizer import AsymQuantizer, SymQuantizer
 
 
 class SymQuantMatMul(torch.nn.Module):
-    """sym_dequant(matmul(q(A), q(B)), s_A, s_B) (matmul.py:69-84); A [M, K], B [N, K]."""
+    """sym_dequant(matmul(q(A), q(B)), s_A, s_B) (matmul.py:69-84); A [M, K], B [N, K].  Also takes
+    A [..., M, K] and B [..., N, K] with equal leading dimensions (one product per entry, one launch)."""
 
     fused = True
 
@@ -31,9 +34,22 @@ class SymQuantMatMul(torch.nn.Module):
     def forward(self, A: torch.Tensor, B: torch.Tensor) -> torch.Tensor:
         A = self.quantizer_A(A)
         B = self.quantizer_B(B)
-        if self.fused and B.quantized_x.dim() == 2:
-            return tensor_utils.linear_forward(_ops.EPI_SYM, A.quantized_x, A.scales_x, None, B.quantized_x, B.scales_x)
-        out = tensor_utils.matmul(A.quantized_x, B.quantized_x)
+        qa, qb = A.quantized_x, B.quantized_x
+        if qb.dim() > 2:
+            lead = tuple(qb.shape[:-2])
+            assert tuple(qa.shape[:-2]) == lead, "Batch dimensions must match"
+            qa3, qb3 = qa.reshape(-1, *qa.shape[-2:]), qb.reshape(-1, *qb.shape[-2:])
+            if self.fused:
+                out = _ops.batch_linear4bit_forward(_ops.EPI_SYM, qa3, A.scales_x, None, qb3, B.scales_x)
+            else:
+                acc = tensor_utils.batched_matmul(qa3, qb3)
+                n, M, N = acc.shape
+                sa, sb = A.scales_x.reshape(n, M), B.scales_x.reshape(n, N)
+                out = torch.stack([tensor_utils.sym_dequant(acc[b], sa[b], sb[b]) for b in range(n)])
+            return out.view(*lead, qa.shape[-2], qb.shape[-2])
+        if self.fused:
+            return tensor_utils.linear_forward(_ops.EPI_SYM, qa, A.scales_x, None, qb, B.scales_x)
+        out = tensor_utils.matmul(qa, qb)
         return tensor_utils.sym_dequant(out, A.scales_x, B.scales_x)
 
 
@@ -61,11 +77,9 @@ class AsymQuantMatMul(torch.nn.Module):
         qa = self.quantizer_A(A.reshape(n, HA, WA))
         qb = self.quantizer_B(B.reshape(n, HB, WB))
         if self.fused:
-            out = torch.empty((n, HA, HB), dtype=torch.float16, device=A.device)
-            for b in range(n):
-                out[b] = tensor_utils.linear_forward(_ops.EPI_ASYM, qa.quantized_x[b], qa.scales_x[b], qa.zeros_x[b],
-                                                     qb.quantized_x[b], qb.scales_x[b], qb.zeros_x[b])
+            out = _ops.batch_linear4bit_forward(_ops.EPI_ASYM, qa.quantized_x, qa.scales_x, qa.zeros_x,
+                                                qb.quantized_x, qb.scales_x, qb.zeros_x)
         else:
-            acc = torch.stack([tensor_utils.matmul(qa.quantized_x[b], qb.quantized_x[b]) for b in range(n)])
+            acc = tensor_utils.batched_matmul(qa.quantized_x, qb.quantized_x)
             out = tensor_utils.asym_batch_dequant(acc, qa.scales_x, qa.zeros_x, qb.scales_x, qb.zeros_x)
         return out.view(list(ext_a) + [HA, HB])

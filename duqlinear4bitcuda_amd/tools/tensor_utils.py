@@ -58,6 +58,13 @@ def matmul(A, B):
     return _ops.matmul(A2, B2).view(*a_lead, *b_lead)
 
 
+def batched_matmul(A, B):
+    """A [n, M, K/2] x B [n, N, K/2] -> int32 [n, M, N] in one launch (tensor_utils.py:63-68, whose body stops
+    in an interactive ``IPython.embed()`` before the call; that line is not reproduced)."""
+    assert A.shape[-1] % 32 == 0, "A.shape[-1]: {} must be multiplication of 32".format(A.shape[-1])
+    return _ops.batched_matmul(A, B)
+
+
 def matmul_8bit(A, B):
     """int8 x int8 -> int32 (tensor_utils.py:57-61)."""
     assert A.shape[-1] % 32 == 0, "A.shape[-1]: {} must be multiplication of 32".format(A.shape[-1])

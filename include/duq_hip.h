@@ -133,6 +133,15 @@ int duq_quantize_rows_asym_shifted(const duq_half *x, uint32_t rows, uint32_t co
 int duq_matmul_host_4bit(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N, uint32_t K,
                          int32_t *C, duq_stream_t stream);
 
+/* Replaces batch_matmul_host_4bit (include/gemm.h:23-31, src/kernels/gemm.cu:83-117; binding batched_matmul,
+ * src/export/bindings.cpp:46-86): batch_count problems of one shape in ONE launch,
+ * C[i] = s4(A[i]) * s4(B[i])^T.  The reference takes arrays of per-problem pointers that its only caller fills
+ * with base + i * stride of contiguous tensors (bindings.cpp:67-71); here the three tensors are passed as such:
+ * A [batch_count, M, K/2], B [batch_count, N, K/2], C [batch_count, M, N], contiguous.  Same K rules as
+ * duq_matmul_host_4bit (K % 64 == 0 keeps every problem 16-byte aligned). */
+int duq_batch_matmul_host_4bit(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N, uint32_t K,
+                               int32_t *C, uint32_t batch_count, duq_stream_t stream);
+
 /* ---- stand-alone dequant epilogues (int32 accumulators in HBM -> fp16) ---------------- */
 
 /* Replaces sym_dequant_host (include/quant.h:19-26, src/kernels/quant.cu:83-97):
@@ -161,6 +170,13 @@ int duq_asym_dual_dequant_host(const int32_t *q, const duq_half *scale_row, cons
                                const duq_half *scale_col_2, const duq_half *zeros_col_2, uint32_t rows,
                                uint32_t cols, duq_half *x, duq_stream_t stream);
 
+/* Replaces asym_batch_dequant_host (include/quant.h:80-90, src/kernels/quant.cu:190-239): the asymmetric
+ * epilogue of duq_asym_dequant_host over q [batches, rows, cols] in one launch, batch entry b reading
+ * scale_row / zeros_row [b * rows + r] and scale_col / zeros_col [b * cols + c]. */
+int duq_asym_batch_dequant_host(const int32_t *q, const duq_half *scale_row, const duq_half *zeros_row,
+                                const duq_half *scale_col, const duq_half *zeros_col, uint32_t batches,
+                                uint32_t rows, uint32_t cols, duq_half *x, duq_stream_t stream);
+
 /* ---- fused GEMM + dequant (+ bias) ---------------------------------------------------- */
 
 /* One launch replacing matmul_host_4bit + {sym,asym,sym_dual,asym_dual}_dequant_host and
@@ -178,6 +194,18 @@ int duq_linear4bit_forward(int32_t mode, const uint8_t *xq, const duq_half *scal
                            const uint8_t *w, const duq_half *w_scale_1, const duq_half *w_zeros_1,
                            const duq_half *w_scale_2, const duq_half *w_zeros_2, const duq_half *bias,
                            uint32_t M, uint32_t N, uint32_t K, duq_half *y, duq_stream_t stream);
+
+/* duq_linear4bit_forward over batch_count problems of one shape in ONE launch: what the loop of
+ * AsymQuantMatMul.forward (qlinear4bit/nn/matmul.py:55-63: a GEMM per batch entry into an int32 tensor, then
+ * asym_batch_dequant) and a batched SymQuantMatMul compute, without the int32 tensor.  Every tensor is
+ * contiguous over the batch: xq [batch_count, M, K/2], w [batch_count, N, K/2], per-row parameters
+ * [batch_count, M], per-column parameters and bias [batch_count, N], y [batch_count, M, N].  Bit-identical to
+ * batch_count calls of duq_linear4bit_forward. */
+int duq_batch_linear4bit_forward(int32_t mode, const uint8_t *xq, const duq_half *scale_x, const duq_half *zeros_x,
+                                 const uint8_t *w, const duq_half *w_scale_1, const duq_half *w_zeros_1,
+                                 const duq_half *w_scale_2, const duq_half *w_zeros_2, const duq_half *bias,
+                                 uint32_t batch_count, uint32_t M, uint32_t N, uint32_t K, duq_half *y,
+                                 duq_stream_t stream);
 
 /* Which kernel family duq_matmul_host_4bit / duq_linear4bit_forward run for a shape (no GPU work; for tests
  * and tuning): 1 decode rows kernel (M <= 4), 2 decode MFMA kernel (M <= 16), 3 dot kernel (M <= 4, rows longer
