@@ -208,7 +208,7 @@ def asym_section(dev):
     (quantize + GEMM + dequant, two launches) in the reference-faithful mode and in the row-sum mode."""
     import torch
 
-    from duqlinear4bitcuda_amd.nn import Linear4bitASQ, Linear4bitASQRowSum
+    from duqlinear4bitcuda_amd.nn import Linear4bitASQ, Linear4bitASQRowSum, LinearQuant4bitDUASQ, LinearQuant4bitDUASQRowSum
 
     M, K, N = 512, 4096, 4096
     g = torch.Generator().manual_seed(4)
@@ -232,6 +232,16 @@ def asym_section(dev):
         us6 = graph_time_us([lambda: mod(x)] * 20)
         out[name].update({"fp6_step_us": round(us6, 2), "fp6_TOPS": round(2.0 * M * N * K / us6 / 1e6, 1),
                           "fp6_same_bits": same})
+    # the dual-uniform layer (input columns 0..9 of the weights on a scale of their own): the reference's epilogue
+    # (one launch after the quantizer) and the row-sum mode that splits the accumulator at column 10 (quantizer,
+    # GEMM into int32, epilogue)
+    dual_rowsum = LinearQuant4bitDUASQRowSum.from_linear(lin)
+    dual_ref = LinearQuant4bitDUASQ.from_linear(lin.cpu()).to(dev)
+    for name, mod in (("dual_reference_mode", dual_ref), ("dual_rowsum_mode", dual_rowsum)):
+        us = graph_time_us([lambda: mod(x)] * 20)
+        y = mod(x).float()
+        out[name] = {"step_us": round(us, 2), "TOPS": round(2.0 * M * N * K / us / 1e6, 1),
+                     "rel_error_vs_fp32_matmul": round(float((y.detach() - true).norm() / true.norm()), 4)}
     return out
 
 

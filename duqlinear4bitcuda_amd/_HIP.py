@@ -438,12 +438,15 @@ def probe_read(t: torch.Tensor):
 
 
 def quantize_linear4bit_forward(x, w, w_scale_1, w_scale_2=None, bias=None, clip: float = 1.0, qmax: int = 6,
-                                return_quantized: bool = False):
+                                return_quantized: bool = False, static: bool = False):
     """SymQuantizer + Linear4bitSQ / Linear4bitDUSQ forward (qlinear4bit/nn/quantizer.py:10-16,
     qlinear4bit/nn/linear.py:42-56, 167-176) from binary16 activations ``x`` [..., K]: bit-identical to
     ``quantize_rows_sym`` followed by ``linear4bit_forward``.  Up to four rows are ONE launch;
     larger inputs run the two launches with the codes staged in a buffer allocated here.  With
-    ``return_quantized`` also returns (codes uint8 [..., K/2], scales [..., 1])."""
+    ``return_quantized`` also returns (codes uint8 [..., K/2], scales [..., 1]).  ``static=True`` stages in the
+    library's static device array instead (``duq_quantize_linear4bit_forward_static``: nothing but the outputs is
+    allocated, 5..16 rows of up to 8192 elements are ONE launch too; calls that overlap on one GPU race on the
+    array, and M * K / 2 <= 8 MiB)."""
     name = "quantize_linear4bit_forward"
     if not isinstance(x, torch.Tensor) or not isinstance(w, torch.Tensor):
         raise RuntimeError(f"{name}: x and w must be tensors")
@@ -471,11 +474,18 @@ def quantize_linear4bit_forward(x, w, w_scale_1, w_scale_2=None, bias=None, clip
         s = torch.empty(lead + (1,), dtype=_F16, device=dev)
     lib = _lib.load()
     ws, ws_bytes = None, 0
+    mode = EPI_SYM if w_scale_2 is None else EPI_SYM_DUAL
+    if static:
+        st = _launch(dev, lib.duq_quantize_linear4bit_forward_static, mode, x.data_ptr(), float(clip), qmax, w.data_ptr(),
+                     ptrs[0] or None, ptrs[1] or None, ptrs[2] or None, M, N, K, y.data_ptr(), _ptr(q), _ptr(s))
+        if st:
+            _lib.check(st, name)
+        return (y, q, s) if return_quantized else y
     if not return_quantized:
         ws_bytes = lib.duq_quantize_linear4bit_workspace_bytes(M, N, K)
         if ws_bytes:
             ws = torch.empty(ws_bytes, dtype=_U8, device=dev)
-    st = _launch(dev, lib.duq_quantize_linear4bit_forward, EPI_SYM if w_scale_2 is None else EPI_SYM_DUAL,
+    st = _launch(dev, lib.duq_quantize_linear4bit_forward, mode,
                  x.data_ptr(), float(clip), qmax, w.data_ptr(), ptrs[0] or None, ptrs[1] or None, ptrs[2] or None, M, N, K,
                  y.data_ptr(), _ptr(q), _ptr(s), _ptr(ws), ws_bytes)
     if st:
@@ -566,6 +576,41 @@ def asym_rowsum_dequant(q, scale_row, zeros_row, rowsum_row, scale_col, zeros_co
     st = _launch(q.device, _lib.load().duq_asym_rowsum_dequant_host, q.data_ptr(), scale_row.data_ptr(),
                  zeros_row.data_ptr(), rowsum_row.data_ptr(), scale_col.data_ptr(), zeros_col.data_ptr(),
                  rowsum_adj_col.data_ptr(), pb, rows, cols, x.data_ptr())
+    if st:
+        _lib.check(st, name)
+    return x
+
+
+def asym_dual_rowsum_dequant(q, xq, scale_row, zeros_row, rowsum_row, w, scale_col_1, zeros_col_1, scale_col_2,
+                             zeros_col_2, adj_col_1, adj_col_2, bias=None):
+    """Row-sum epilogue of the dual-uniform layer on int32 accumulators ``q`` [rows, cols] = matmul(xq, w): input
+    columns 0..9 dequantized with (scale_col_1, zeros_col_1), the others with (scale_col_2, zeros_col_2); the
+    codes of columns 0..9 are read from the packed operands ``xq`` [rows, K/2] and ``w`` [cols, K/2]."""
+    name = "asym_dual_rowsum_dequant"
+    _check(name, q, xq, w)
+    _check_dtype(name, q, "q", _I32)
+    _check_dtype(name, xq, "xq", _U8)
+    _check_dtype(name, w, "w", _U8)
+    if q.dim() != 2 or xq.dim() != 2 or w.dim() != 2:
+        raise RuntimeError(f"{name}: expected 2-D q, xq and w")
+    rows, cols = q.shape
+    kb = xq.shape[1]
+    if xq.shape[0] != rows or w.shape[0] != cols or w.shape[1] != kb:
+        raise RuntimeError(f"{name}: q {tuple(q.shape)} does not match xq {tuple(xq.shape)} and w {tuple(w.shape)}")
+    dev = q.device
+    for t, what, dt, cnt in ((scale_row, "scale_row", _F16, rows), (zeros_row, "zeros_row", _F16, rows),
+                             (rowsum_row, "rowsum_row", _I32, rows), (scale_col_1, "scale_col_1", _F16, cols),
+                             (zeros_col_1, "zeros_col_1", _F16, cols), (scale_col_2, "scale_col_2", _F16, cols),
+                             (zeros_col_2, "zeros_col_2", _F16, cols), (adj_col_1, "adj_col_1", _I32, cols),
+                             (adj_col_2, "adj_col_2", _I32, cols)) + (((bias, "bias", _F16, cols),) if bias is not None else ()):
+        _fast_check(name, what, t, dt, dev)
+        if t.numel() != cnt:
+            _check_size0(name, t.reshape(-1), what, cnt)
+    x = torch.empty((rows, cols), dtype=_F16, device=dev)
+    st = _launch(dev, _lib.load().duq_asym_dual_rowsum_dequant_host, q.data_ptr(), xq.data_ptr(), scale_row.data_ptr(),
+                 zeros_row.data_ptr(), rowsum_row.data_ptr(), w.data_ptr(), scale_col_1.data_ptr(), zeros_col_1.data_ptr(),
+                 scale_col_2.data_ptr(), zeros_col_2.data_ptr(), adj_col_1.data_ptr(), adj_col_2.data_ptr(), _ptr(bias),
+                 rows, cols, kb * 2, x.data_ptr())
     if st:
         _lib.check(st, name)
     return x

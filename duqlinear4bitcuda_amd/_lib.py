@@ -49,6 +49,8 @@ PROTOTYPES = {
     "duq_linear4bit_forward_rowsum": [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_u32, _c_u32, _c_u32,
                                       _c_p, _c_p],
     "duq_asym_rowsum_dequant_host": [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_u32, _c_u32, _c_p, _c_p],
+    "duq_asym_dual_rowsum_dequant_host": [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p,
+                                          _c_u32, _c_u32, _c_u32, _c_p, _c_p],
     "duq_weight_shadow_bf6": [_c_p, _c_u32, _c_u32, _c_p, _c_p],
     "duq_quantize_rows_sym_bf6": [_c_p, _c_u32, _c_u32, ctypes.c_float, _c_i32, _c_p, _c_p, _c_p, _c_p],
     "duq_quantize_rows_asym_bf6": [_c_p, _c_u32, _c_u32, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p],

@@ -408,6 +408,25 @@ int duq_asym_rowsum_dequant_host(const int32_t *q, const duq_half *scale_row, co
     return duq::launch_dequant(q, e, rows, cols, x, as_stream(stream));
 }
 
+int duq_asym_dual_rowsum_dequant_host(const int32_t *q, const uint8_t *xq, const duq_half *scale_row,
+                                      const duq_half *zeros_row, const int32_t *rowsum_row, const uint8_t *w,
+                                      const duq_half *scale_col_1, const duq_half *zeros_col_1,
+                                      const duq_half *scale_col_2, const duq_half *zeros_col_2,
+                                      const int32_t *adj_col_1, const int32_t *adj_col_2, const duq_half *bias,
+                                      uint32_t rows, uint32_t cols, uint32_t K, duq_half *x, duq_stream_t stream)
+{
+    if (int e = check_gemm(xq, w, rows, cols, K)) return e;
+    if (rows == 0 || cols == 0) return DUQ_OK;
+    if (K == 0) return DUQ_E_KALIGN;
+    if (!q || !scale_row || !zeros_row || !rowsum_row || !scale_col_1 || !zeros_col_1 || !scale_col_2 || !zeros_col_2 ||
+        !adj_col_1 || !adj_col_2 || !x)
+        return DUQ_E_NULL;
+    duq::DualRowsumParams p{q,           xq,          w,           K / 2,     scale_row, zeros_row, rowsum_row, scale_col_1,
+                            zeros_col_1, scale_col_2, zeros_col_2, adj_col_1, adj_col_2, bias,      rows,       cols,
+                            x};
+    return duq::launch_dual_rowsum_dequant(p, as_stream(stream));
+}
+
 int duq_linear4bit_forward_rowsum(const uint8_t *xq, const duq_half *scale_x, const duq_half *zeros_x,
                                   const int32_t *rowsum_x, const uint8_t *w, const duq_half *w_scale,
                                   const duq_half *w_zeros, const int32_t *w_rowsum_adj, const duq_half *bias,

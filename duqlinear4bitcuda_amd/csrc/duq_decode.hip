@@ -107,23 +107,27 @@ __device__ __forceinline__ uint16_t dequant_rt(int acc, const RowEpi &r, const C
 // ---------------------------------------------------------------------------------
 // rows kernel: M <= MR <= 4, K <= XS * 2048
 // ---------------------------------------------------------------------------------
-template <int MR, int XS, bool FUSEQ, int EPI>
-__global__ __launch_bounds__(256) void gemv_s4_rows_kernel(DecodeParams p)
+// WAVES wavefronts of R = 16 / WAVES weight rows each: 16 weight rows per workgroup either way.  Eight wavefronts
+// help when the workgroup quantizes four activation rows itself and a CU holds several workgroups (launcher).
+template <int MR, int XS, bool FUSEQ, int EPI, int WAVES = 4>
+__global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DecodeParams p)
 {
-    constexpr int R = DUQ_DEC_R;     // weight rows per wavefront
+    constexpr int R = 4 * DUQ_DEC_R / WAVES;  // weight rows per wavefront
     constexpr int V = MR * R;        // partial sums per lane: 4, 8 or 16
     constexpr int LPV = 64 / V;      // lanes that finish one sum: 16, 8 or 4
     constexpr int MODE = EPI < 0 ? 0 : EPI;
     constexpr uint32_t XSTRIDE = XS * 1024;
     static_assert(MR == 1 || MR == 2 || MR == 4, "rows");
-    __shared__ __attribute__((aligned(16))) int red[4][V * 64];
+    static_assert(WAVES == 4 || WAVES == 8, "wavefronts per workgroup");
+    static_assert(V >= 4 && (XS * MR * 4) % WAVES == 0, "partial sums per lane, quantize units per lane");
+    __shared__ __attribute__((aligned(16))) int red[WAVES][V * 64];
     __shared__ __attribute__((aligned(16))) uint8_t xs[FUSEQ ? MR * XSTRIDE : 16];
-    __shared__ uint32_t rmax[4];
+    __shared__ uint32_t rmax[WAVES];
     __shared__ uint16_t srow[MR];
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t kbytes = p.K >> 1;
-    const uint32_t n0 = (blockIdx.x * 4 + wave) * R;
+    const uint32_t n0 = (blockIdx.x * WAVES + wave) * R;
 
 
     // ---- loads, in the order their data is needed (loads return in order: waiting for one waits for every
@@ -131,8 +135,8 @@ __global__ __launch_bounds__(256) void gemv_s4_rows_kernel(DecodeParams p)
     // output this lane will finish
     // activations: lane l needs bytes [i*1024 + l*16, +16) of every row
     v4u xr[MR][XS];
-    constexpr int WPR = 4 / MR;              // wavefronts that share a row in the quantize phase
-    constexpr int UPL = FUSEQ ? XS * MR : 1;  // 8-element units per lane in the quantize phase
+    constexpr int WPR = WAVES / MR;           // wavefronts that share a row in the quantize phase
+    constexpr int UPL = FUSEQ ? XS * MR * 4 / WAVES : 1;  // 8-element units per lane in the quantize phase
     const uint32_t qrow = wave / WPR, qpart = wave % WPR;
     v4u raw[UPL];
     const uint32_t nunits = p.K >> 3;
@@ -146,7 +150,7 @@ __global__ __launch_bounds__(256) void gemv_s4_rows_kernel(DecodeParams p)
                 xr[m][i] = buf_load16(rX, off < kbytes ? m * kbytes + off : kOobOffset, 0);
             }
     } else {
-        // the workgroup quantizes the MR rows into LDS: WPR = 4 / MR wavefronts share a row, wavefront `part` of
+        // the workgroup quantizes the MR rows into LDS: WPR = WAVES / MR wavefronts share a row, wavefront `part` of
         // a row owns its 8-element units part*64 + lane, + 64*WPR, ...
         const __amdgpu_buffer_rsrc_t rX = make_rsrc(p.X, p.M * p.K * 2);  // rows past M read as zero
 #pragma unroll
@@ -367,8 +371,17 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_s4_decode_kernel(DecodeParams
 template <int MR, int XS, bool FUSEQ>
 void launch_rows_mode(const DecodeParams &p, int epi, hipStream_t stream)
 {
-    const dim3 grid((p.N + 4 * DUQ_DEC_R - 1) / (4 * DUQ_DEC_R));  // 4 wavefronts x R rows per workgroup
-#define DUQ_ROWS(E) hipLaunchKernelGGL((gemv_s4_rows_kernel<MR, XS, FUSEQ, E>), grid, dim3(256), 0, stream, p)
+    const dim3 grid((p.N + 4 * DUQ_DEC_R - 1) / (4 * DUQ_DEC_R));  // 16 weight rows per workgroup
+    // eight wavefronts when four rows are quantized in the kernel and a CU gets more than one workgroup (measured,
+    // N = 11008, K = 4096: 7.9 against 8.3 us; with one workgroup per CU the vector work per SIMD is the same and
+    // four wavefronts are ahead, N = 4096: 4.8 against 5.1 us)
+    const bool wide = FUSEQ && MR == 4 && grid.x > 256;
+#define DUQ_ROWS(E)                                                                                              \
+    if (wide)                                                                                                    \
+        hipLaunchKernelGGL((gemv_s4_rows_kernel<MR, XS, FUSEQ, E, (FUSEQ && MR == 4) ? 8 : 4>), grid, dim3(512), 0,  \
+                           stream, p);                                                                           \
+    else                                                                                                         \
+        hipLaunchKernelGGL((gemv_s4_rows_kernel<MR, XS, FUSEQ, E, 4>), grid, dim3(256), 0, stream, p)
     switch (epi) {
     case 0: DUQ_ROWS(0); break;
     case 2: DUQ_ROWS(2); break;

@@ -95,4 +95,105 @@ int launch_dequant_batched(const int32_t *acc, const Epilogue &epi, uint32_t bat
     return (int)hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------------
+// row-sum epilogue of the dual-uniform layer
+// ---------------------------------------------------------------------------------
+// A thread owns four consecutive output columns: it keeps the codes of their input columns 0..9 (two words per
+// column, the second masked to its two nibbles by masking the activation side), their two scale / zero / row-sum
+// pairs and the bias in registers and walks kDualRows rows; per row the workgroup needs eight bytes of the
+// activation row and three parameters (the same addresses in every lane).
+constexpr uint32_t kDualRows = 8;
+
+template <bool BIAS>
+__global__ __launch_bounds__(256) void dual_rowsum_dequant_kernel(DualRowsumParams p)
+{
+    const uint32_t n0 = (blockIdx.x * 256 + threadIdx.x) * 4;
+    if (n0 >= p.cols) return;  // (no barrier below)
+    const bool vec = (p.cols % 4 == 0) && (reinterpret_cast<uintptr_t>(p.acc) % 16 == 0) &&
+                     (reinterpret_cast<uintptr_t>(p.y) % 8 == 0);
+    uint32_t wlo[4], whi[4];
+    uint32_t z1[4], z2[4], a1[4], a2[4];
+    float s1[4], s2[4];
+    f16 bias[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t n = min(n0 + j, p.cols - 1);
+        const v2u head = *reinterpret_cast<const v2u *>(p.w + (uint64_t)n * p.kbytes);
+        wlo[j] = head[0];
+        whi[j] = head[1];
+        s1[j] = (float)bits_to_f16(p.s_col_1[n]);
+        s2[j] = (float)bits_to_f16(p.s_col_2[n]);
+        z1[j] = (uint32_t)rint_i32((float)bits_to_f16(p.z_col_1[n]));
+        z2[j] = (uint32_t)rint_i32((float)bits_to_f16(p.z_col_2[n]));
+        a1[j] = (uint32_t)p.adj_col_1[n];
+        a2[j] = (uint32_t)p.adj_col_2[n];
+        bias[j] = BIAS ? bits_to_f16(p.bias[n]) : (f16)0;
+    }
+    const uint32_t r0 = blockIdx.y * kDualRows, r1 = min(r0 + kDualRows, p.rows);
+    for (uint32_t r = r0; r < r1; ++r) {
+        const v2u xh = *reinterpret_cast<const v2u *>(p.xq + (uint64_t)r * p.kbytes);
+        const uint32_t xlo = xh[0], xhi = xh[1] & 0xFFu;  // input columns 0..7 and 8, 9
+        const uint32_t rxl = (uint32_t)__builtin_amdgcn_sdot8((int)xhi, 0x11111111, __builtin_amdgcn_sdot8((int)xlo, 0x11111111, 0, false), false);
+        const uint32_t zx = (uint32_t)rint_i32((float)bits_to_f16(p.z_row[r]));
+        const float sx = (float)bits_to_f16(p.s_row[r]);
+        const uint32_t rxr = (uint32_t)p.rs_row[r] - rxl;
+        int acc[4];
+        if (vec) {
+            const v4i a = *reinterpret_cast<const v4i *>(p.acc + (uint64_t)r * p.cols + n0);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[j] = a[j];
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[j] = p.acc[(uint64_t)r * p.cols + min(n0 + j, p.cols - 1)];
+        }
+        uint16_t out[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t accl = (uint32_t)__builtin_amdgcn_sdot8((int)xhi, (int)whi[j], __builtin_amdgcn_sdot8((int)xlo, (int)wlo[j], 0, false), false);
+            // 32-bit wrapping integer arithmetic, like the single-range row-sum epilogue
+            const int corr_l = (int)(accl - zx * a1[j] - z1[j] * rxl);
+            const int corr_r = (int)(((uint32_t)acc[j] - accl) - zx * a2[j] - z2[j] * rxr);
+            float t1 = (float)corr_l * (sx * s1[j]);  // sx * s: exact (11-bit significands)
+            float t2 = (float)corr_r * (sx * s2[j]);
+            asm volatile("" : "+v"(t1), "+v"(t2));    // each product rounded to float32 on its own
+            float t = t1 + t2;
+            asm volatile("" : "+v"(t));               // the sum rounded to float32, then to binary16
+            f16 y = (f16)t;
+            if (BIAS) y = y + bias[j];
+            out[j] = f16_to_bits(y);
+        }
+        uint16_t *dst = p.y + (uint64_t)r * p.cols + n0;
+        if (vec) {
+            *reinterpret_cast<v2u *>(dst) = v2u{(uint32_t)out[0] | ((uint32_t)out[1] << 16), (uint32_t)out[2] | ((uint32_t)out[3] << 16)};
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (n0 + j < p.cols) dst[j] = out[j];
+        }
+    }
+}
+
+int launch_dual_rowsum_dequant(const DualRowsumParams &p, hipStream_t stream)
+{
+    if (p.rows == 0 || p.cols == 0) return 0;
+    // at most 65535 row groups per launch (grid limit): longer inputs run in slices of rows
+    constexpr uint32_t kSlice = 65535u * kDualRows;
+    for (uint32_t r0 = 0; r0 < p.rows; r0 += kSlice) {
+        DualRowsumParams q = p;
+        q.rows = std::min(p.rows - r0, kSlice);
+        q.acc += (uint64_t)r0 * p.cols;
+        q.y += (uint64_t)r0 * p.cols;
+        q.xq += (uint64_t)r0 * p.kbytes;
+        q.s_row += r0;
+        q.z_row += r0;
+        q.rs_row += r0;
+        const dim3 grid((p.cols + 1023) / 1024, (q.rows + kDualRows - 1) / kDualRows);
+        if (p.bias)
+            hipLaunchKernelGGL((dual_rowsum_dequant_kernel<true>), grid, dim3(256), 0, stream, q);
+        else
+            hipLaunchKernelGGL((dual_rowsum_dequant_kernel<false>), grid, dim3(256), 0, stream, q);
+    }
+    return (int)hipGetLastError();
+}
+
 }  // namespace duq

@@ -47,6 +47,24 @@ int launch_dequant(const int32_t *acc, const Epilogue &epi, uint32_t rows, uint3
 int launch_dequant_batched(const int32_t *acc, const Epilogue &epi, uint32_t batches, uint32_t rows, uint32_t cols,
                            uint16_t *y, hipStream_t stream);
 
+// Row-sum epilogue of the dual-uniform layer on int32 accumulators (definition: include/duq_hip.h,
+// duq_asym_dual_rowsum_dequant_host).  xq / w are the packed operands of the GEMM that made `acc`: the kernel reads
+// the first eight bytes of every row of both (the codes of input columns 0..9).
+struct DualRowsumParams {
+    const int32_t *acc;      // [rows, cols]
+    const uint8_t *xq;       // [rows, kbytes]
+    const uint8_t *w;        // [cols, kbytes]
+    uint32_t kbytes;
+    const uint16_t *s_row, *z_row;   // [rows]
+    const int32_t *rs_row;           // [rows]
+    const uint16_t *s_col_1, *z_col_1, *s_col_2, *z_col_2;  // [cols]
+    const int32_t *adj_col_1, *adj_col_2;                   // [cols]
+    const uint16_t *bias;            // [cols] or nullptr
+    uint32_t rows, cols;
+    uint16_t *y;             // [rows, cols]
+};
+int launch_dual_rowsum_dequant(const DualRowsumParams &p, hipStream_t stream);
+
 // Kernel families of the int4 GEMM and the host-side rule that picks one (select_gemm_kernel: host arithmetic
 // only, exported as duq_gemm_kernel_for so that the rule can be tested without a GPU).
 enum GemmKernelId {

@@ -239,6 +239,77 @@ class Linear4bitASQRowSum(_Linear4bitBase):
         return new
 
 
+class LinearQuant4bitDUASQRowSum(_Linear4bitBase):
+    """Dual-uniform asymmetric layer with the exact zero-point correction.  Not in the reference: its
+    LinearQuant4bitDUASQ (linear.py:209-297) quantizes input columns 0..9 of every weight row with one
+    (scale, zero) pair and the others with a second pair, and its epilogue (src/kernels/quant2.cu:158-186) then
+    applies ONE pair per output column to the whole accumulator.  Here the accumulator is split at input column 10
+    and each part gets the row-sum correction with its own pair:
+        y = s_x * ( s_1 * corr(k < 10) + s_2 * corr(k >= 10) ),  corr = acc - z_x * (R_w - n_k * z_w) - z_w * R_x
+    Codes and zero points are stored minus 8 (the signed GEMM reads them exactly), ``weight_rowsum_1/2`` hold
+    ``R_w - n_k * z_w`` of the two ranges.  The forward is quantizer, GEMM into int32, epilogue (three launches)."""
+
+    def __init__(self, in_features, out_features, bias=False, require_quantizer=True):
+        super().__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+        self.require_quantizer = require_quantizer
+        for k in (1, 2):
+            self.register_buffer(f"weight_scales_{k}", torch.zeros((out_features, 1), requires_grad=False, dtype=torch.float16))
+            self.register_buffer(f"weight_zeros_{k}", torch.zeros((out_features, 1), requires_grad=False, dtype=torch.float16))
+            self.register_buffer(f"weight_rowsum_{k}", torch.zeros((out_features,), requires_grad=False, dtype=torch.int32))
+        self.register_buffer("weight", _placeholder_weight(out_features, in_features))
+        if bias:
+            self.register_buffer("bias", torch.zeros((out_features), dtype=torch.float16))
+        else:
+            self.bias = None
+        if require_quantizer:
+            self.quantizer = AsymQuantizer(shifted=True)
+
+    def forward(self, x):
+        if self.require_quantizer:
+            x = self.quantizer(x)
+        assert type(x) == tensor_utils.PackedQuantizedTensor and x.rowsum_x is not None, \
+            "Input should come from AsymQuantizer(shifted=True), or require_quantizer should be set"
+        xq = x.quantized_x
+        lead = xq.shape[:-1]
+        xq2 = xq.reshape(-1, xq.shape[-1])
+        acc = _ops.matmul(xq2, self.weight)
+        y = _ops.asym_dual_rowsum_dequant(acc, xq2, x.scales_x, x.zeros_x, x.rowsum_x, self.weight,
+                                          self.weight_scales_1, self.weight_zeros_1, self.weight_scales_2,
+                                          self.weight_zeros_2, self.weight_rowsum_1, self.weight_rowsum_2, self.bias)
+        return y.view(*lead, -1)
+
+    @classmethod
+    def from_linear(cls, module: torch.nn.Linear, require_quantizer: bool = True):
+        """Per-output-channel min/max quantization of input columns 0..9 and of the others, each range on its own,
+        on the device the weight lives on (the activation quantizer kernel applied to the two column ranges,
+        each padded with copies of its last column to a width the kernel takes: a copy changes neither the
+        minimum nor the maximum)."""
+        w = module.weight.data
+        assert w.is_cuda, "weight preparation runs on the GPU: move the layer there first"
+        K, split = module.in_features, tensor_utils.get_dual_quant_col()
+        assert K > split and K % 2 == 0
+        new = cls(K, module.out_features, bias=module.bias is not None, require_quantizer=require_quantizer).to(w.device)
+        w = w.to(torch.float16)
+        codes = []
+        for k, (lo, hi) in enumerate(((0, split), (split, K)), start=1):
+            part = w[:, lo:hi]
+            pad = (-(hi - lo)) % 32
+            if pad:
+                part = torch.cat([part, part[:, -1:].expand(-1, pad)], dim=1)
+            q, scale, zeros, _ = tensor_utils.quantize_asym_shifted(part.contiguous())
+            c = quant_utils.unpack_i4(q)[:, :hi - lo]          # signed codes
+            codes.append(c)
+            getattr(new, f"weight_scales_{k}").copy_(scale)
+            getattr(new, f"weight_zeros_{k}").copy_(zeros)
+            getattr(new, f"weight_rowsum_{k}").copy_(c.sum(dim=1, dtype=torch.int32) - (hi - lo) * zeros.view(-1).to(torch.int32))
+        new.weight.copy_(quant_utils.pack_i4(torch.cat(codes, dim=1).to(torch.int8), sym=True))
+        if module.bias is not None:
+            new.bias.copy_(module.bias)
+        return new
+
+
 class Linear4bitDUSQ(_Linear4bitBase):
     """Symmetric layer with two per-row weight scales: input columns < 10 were quantized
     with scale 1, the rest with scale 2; the epilogue picks per OUTPUT column < 10

@@ -292,6 +292,27 @@ int duq_asym_rowsum_dequant_host(const int32_t *q, const duq_half *scale_row, co
                                  const int32_t *rowsum_adj_col, const duq_half *bias, uint32_t rows, uint32_t cols,
                                  duq_half *x, duq_stream_t stream);
 
+/* Row-sum epilogue for the dual-uniform layer (no counterpart in the reference).  LinearQuant4bitDUASQ
+ * (qlinear4bit/nn/linear.py:252-297) quantizes input columns 0..9 of every weight row with (scale_1, zero_1) and
+ * the others with (scale_2, zero_2); the reference epilogue (src/kernels/quant2.cu:158-186) applies ONE of the two
+ * pairs per output column (its selector is non-zero for output column 0 only) to the whole accumulator, which is
+ * not the product of the dequantized operands.  That product needs the accumulator split at input column 10:
+ *   accL = sum_{k<10} c_x[m,k] c_w[n,k],  accR = q[m,n] - accL,  R_xL = sum_{k<10} c_x[m,k],  R_xR = rowsum_row[m] - R_xL
+ *   corrL = accL - z_x[m]*adj_col_1[n] - z_1[n]*R_xL      adj_col_1[n] = sum_{k<10}  c_w[n,k] - 10*z_1[n]
+ *   corrR = accR - z_x[m]*adj_col_2[n] - z_2[n]*R_xR      adj_col_2[n] = sum_{k>=10} c_w[n,k] - (K-10)*z_2[n]
+ *   x[m,n] = h( f32(corrL)*(f32(s_x)*f32(s_1)) + f32(corrR)*(f32(s_x)*f32(s_2)) )   (+ bias: h(x + bias[n]))
+ * with every float32 operator rounded, corrections in wrapping 32-bit integers, codes and zero points signed-shifted
+ * as for duq_linear4bit_forward_rowsum (activations from duq_quantize_rows_asym_shifted).
+ *   q    [rows, cols] int32 from duq_matmul_host_4bit(xq, w)
+ *   xq   [rows, K/2], w [cols, K/2]: the packed operands of that GEMM; the first eight bytes of every row are read
+ *        (16-byte aligned, K % 64 == 0) */
+int duq_asym_dual_rowsum_dequant_host(const int32_t *q, const uint8_t *xq, const duq_half *scale_row,
+                                      const duq_half *zeros_row, const int32_t *rowsum_row, const uint8_t *w,
+                                      const duq_half *scale_col_1, const duq_half *zeros_col_1,
+                                      const duq_half *scale_col_2, const duq_half *zeros_col_2,
+                                      const int32_t *adj_col_1, const int32_t *adj_col_2, const duq_half *bias,
+                                      uint32_t rows, uint32_t cols, uint32_t K, duq_half *x, duq_stream_t stream);
+
 /* ---- the same forward on the 6-bit float matrix path ---------------------------------- */
 
 /* No counterpart in the reference.  Every int4 value is exactly an E3M2 ("bf6") number and

@@ -377,6 +377,73 @@ def linear4bit_asq_rowsum_forward(x, w_packed_shifted, w_scales, w_zeros_shifted
 
 
 # ----------------------------------------------------------------------------------
+# Row-sum mode of the dual-uniform layer.  LinearQuant4bitDUASQ (qlinear4bit/nn/linear.py:252-297) quantizes the
+# first QUANT_COL_K = 10 INPUT columns of every weight row with (scale_1, zero_1) and the rest with
+# (scale_2, zero_2); its epilogue (src/kernels/quant2.cu:158-186) then applies one pair per OUTPUT column,
+# chosen by a selector that is non-zero for column 0 only, to a single accumulator.  The product of the
+# dequantized operands needs the accumulator split at input column 10 instead:
+#   accL = sum_{k<10} c_x c_w,  accR = acc - accL,  R_xL = sum_{k<10} c_x,  R_xR = R_x - R_xL
+#   corrL = accL - z_x * adjL[n] - z_1[n] * R_xL,   adjL[n] = sum_{k<10} c_w[n,k] - 10 * z_1[n]
+#   corrR = accR - z_x * adjR[n] - z_2[n] * R_xR,   adjR[n] = sum_{k>=10} c_w[n,k] - (K-10) * z_2[n]
+#   y = h( f32(corrL) * (f32(s_x) * f32(s_1)) + f32(corrR) * (f32(s_x) * f32(s_2)) ), every float32 operator
+#   rounded; with bias y = h(y + bias).
+# This restates the definition in include/duq_hip.h (no counterpart in the reference); pinned by the integer
+# identities corrL/R == sum (c_x - z_x)(c_w - z_{1,2}) over their k ranges (brute force) and by the float64
+# product of the dequantized operands.
+# ----------------------------------------------------------------------------------
+def weight_asym_dual_shifted_from_linear(w):
+    """Per-row true min/max quantization of the two column ranges, stored shifted.  Returns (packed u8 [N, K/2],
+    scale_1, zeros_1_shifted, scale_2, zeros_2_shifted [N,1] each, adjL int32 [N], adjR int32 [N])."""
+    w = np.asarray(w, _F16)
+    K = w.shape[1]
+    parts = []
+    for lo, hi in ((0, QUANT_COL_K), (QUANT_COL_K, K)):
+        q, s, zs, _ = asym_quant_shifted(np.ascontiguousarray(w[:, lo:hi]) if (hi - lo) % 2 == 0 else
+                                         np.concatenate([w[:, lo:hi], w[:, hi - 1:hi]], axis=1))
+        c = unpack_i4(q, signed=True)[:, :hi - lo].astype(np.int64)
+        z = half_to_int_rn(zs.reshape(-1)).astype(np.int64)
+        parts.append((c, s, zs, _wrap_i32(c.sum(axis=1) - (hi - lo) * z).astype(np.int32)))
+    codes = np.concatenate([parts[0][0], parts[1][0]], axis=1).astype(np.int8)
+    return pack_i4(codes, sym=True), parts[0][1], parts[0][2], parts[1][1], parts[1][2], parts[0][3], parts[1][3]
+
+
+def asym_dual_rowsum_dequant(acc, x_packed_shifted, scale_row, zeros_row, rowsum_row, w_packed_shifted, scale_col_1,
+                             zeros_col_1, scale_col_2, zeros_col_2, adj_col_1, adj_col_2, bias=None):
+    """The epilogue defined above on int32 accumulators; the first 10 codes of every activation and weight row
+    supply accL and R_xL."""
+    cx = unpack_i4(np.asarray(x_packed_shifted)[:, :8], signed=True)[:, :QUANT_COL_K].astype(np.int64)
+    cw = unpack_i4(np.asarray(w_packed_shifted)[:, :8], signed=True)[:, :QUANT_COL_K].astype(np.int64)
+    accL = cx @ cw.T
+    rxL = cx.sum(axis=1)[:, None]
+    acc = np.asarray(acc, np.int64)
+    zr = half_to_int_rn(np.asarray(zeros_row, _F16).reshape(-1)).astype(np.int64)[:, None]
+    z1 = half_to_int_rn(np.asarray(zeros_col_1, _F16).reshape(-1)).astype(np.int64)[None, :]
+    z2 = half_to_int_rn(np.asarray(zeros_col_2, _F16).reshape(-1)).astype(np.int64)[None, :]
+    rx = np.asarray(rowsum_row, np.int64).reshape(-1, 1)
+    a1 = np.asarray(adj_col_1, np.int64).reshape(1, -1)
+    a2 = np.asarray(adj_col_2, np.int64).reshape(1, -1)
+    corrL = _wrap_i32(accL - zr * a1 - z1 * rxL).astype(np.int32)
+    corrR = _wrap_i32((acc - accL) - zr * a2 - z2 * (rx - rxL)).astype(np.int32)
+    sr = _f32(np.asarray(scale_row, _F16).reshape(-1, 1))
+    ss1 = sr * _f32(np.asarray(scale_col_1, _F16).reshape(1, -1))   # exact in float32 (11-bit significands)
+    ss2 = sr * _f32(np.asarray(scale_col_2, _F16).reshape(1, -1))
+    with np.errstate(invalid="ignore", over="ignore"):
+        t = (corrL.astype(_F32) * ss1).astype(_F32) + (corrR.astype(_F32) * ss2).astype(_F32)
+        y = t.astype(_F32).astype(_F16)
+    if bias is not None:
+        y = add_bias(y, bias)
+    return y
+
+
+def linear4bit_duasq_rowsum_forward(x, w_packed_shifted, ws1, wz1, ws2, wz2, adj1, adj2, bias=None):
+    """AsymQuantizer(shifted) + GEMM + dual row-sum epilogue.  Returns (y, acc, q_x, s_x, z_x, rowsum_x)."""
+    q_x, s_x, z_x, r_x = asym_quant_shifted(x)
+    acc = matmul_s4(q_x, w_packed_shifted)
+    y = asym_dual_rowsum_dequant(acc, q_x, s_x, z_x, r_x, w_packed_shifted, ws1, wz1, ws2, wz2, adj1, adj2, bias)
+    return y, acc, q_x, s_x, z_x, r_x
+
+
+# ----------------------------------------------------------------------------------
 # A8  module forwards as compositions (qlinear4bit/nn/linear.py:42-56,104-115,
 #     167-176,239-250)
 # ----------------------------------------------------------------------------------

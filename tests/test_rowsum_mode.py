@@ -73,6 +73,80 @@ def test_oracle_rowsum_bias_and_wrapping():
     assert c1 == -5
 
 
+@pytest.mark.parametrize("M,N,K,seed", [(5, 7, 64, 0), (3, 4, 192, 1), (8, 2, 64, 2)])
+def test_oracle_dual_rowsum_identity_and_closed_form(M, N, K, seed):
+    """Dual-uniform row-sum mode: the two corrections are the brute-force sums over their own k ranges, y is the
+    float64 product of the dequantized operands up to the stated roundings, and the weight preparation quantizes
+    each range with its own true min/max."""
+    rng = np.random.default_rng(seed)
+    x = (rng.random((M, K)) * 6 - (seed == 1) * 2).astype(np.float16)
+    w = (rng.standard_normal((N, K)) * 0.05).astype(np.float16)
+    w[:, :10] *= 8                      # the first ten input columns on another scale: what the layer is for
+    wq, s1, z1, s2, z2, a1, a2 = orc.weight_asym_dual_shifted_from_linear(w)
+    y, acc, qx, sx, zx, rx = orc.linear4bit_duasq_rowsum_forward(x, wq, s1, z1, s2, z2, a1, a2)
+    cx = orc.unpack_i4(qx, signed=True).astype(np.int64)
+    cw = orc.unpack_i4(wq, signed=True).astype(np.int64)
+    zxi, z1i, z2i = _ints(zx).reshape(-1), _ints(z1).reshape(-1), _ints(z2).reshape(-1)
+    # weight preparation: every range is asym_quant_shifted of that range alone
+    for lo, hi, s, z, a in ((0, 10, s1, z1, a1), (10, K, s2, z2, a2)):
+        q_r, s_r, z_r, _ = orc.asym_quant_shifted(np.ascontiguousarray(w[:, lo:hi]))
+        assert np.array_equal(orc.unpack_i4(q_r, signed=True), cw[:, lo:hi]) and np.array_equal(s_r, s) and np.array_equal(z_r, z)
+        assert np.array_equal(a, cw[:, lo:hi].sum(axis=1) - (hi - lo) * _ints(z).reshape(-1))
+    # the two corrections, term by term from brute-force loops
+    want_l = np.zeros((M, N), np.int64)
+    want_r = np.zeros((M, N), np.int64)
+    for m in range(M):
+        for n in range(N):
+            want_l[m, n] = sum(int(cx[m, k] - zxi[m]) * int(cw[n, k] - z1i[n]) for k in range(10))
+            want_r[m, n] = sum(int(cx[m, k] - zxi[m]) * int(cw[n, k] - z2i[n]) for k in range(10, K))
+    acc_l = cx[:, :10] @ cw[:, :10].T
+    rxl = cx[:, :10].sum(axis=1)
+    corr_l = acc_l - zxi[:, None] * a1.astype(np.int64)[None, :] - z1i[None, :] * rxl[:, None]
+    corr_r = (acc.astype(np.int64) - acc_l) - zxi[:, None] * a2.astype(np.int64)[None, :] - z2i[None, :] * (rx.astype(np.int64) - rxl)[:, None]
+    assert np.array_equal(corr_l, want_l) and np.array_equal(corr_r, want_r)
+    # y against the exact value: two float32 products, one float32 sum, one binary16 rounding
+    sx64 = sx.astype(np.float64)
+    e1 = sx64 * s1.astype(np.float64).reshape(1, -1) * want_l
+    e2 = sx64 * s2.astype(np.float64).reshape(1, -1) * want_r
+    exact = e1 + e2
+    bound = (np.abs(e1) + np.abs(e2)) * 2.0 ** -22 + np.abs(exact) * 2.0 ** -11 + 6e-8
+    assert np.all(np.abs(y.astype(np.float64) - exact) <= bound)
+    # exact is the product of the dequantized operands
+    wd = np.concatenate([s1.astype(np.float64) * (cw[:, :10] - z1i[:, None]), s2.astype(np.float64) * (cw[:, 10:] - z2i[:, None])], axis=1)
+    ref = (sx64 * (cx - zxi[:, None])) @ wd.T
+    assert np.allclose(exact, ref, rtol=1e-12, atol=1e-300)
+    # the point of the mode: close to the real product, where the reference's epilogue is not
+    true = x.astype(np.float64) @ w.astype(np.float64).T
+    err = np.abs(y.astype(np.float64) - true).max() / np.abs(true).max()
+    assert err < 0.25
+    # swapping the two pairs (a plausible mistake) must show
+    y_swapped = orc.asym_dual_rowsum_dequant(acc, qx, sx, zx, rx, wq, s2, z2, s1, z1, a2, a1)
+    assert not np.array_equal(y_swapped, y)
+
+
+def test_oracle_dual_rowsum_hand_case():
+    """One row, one column, K = 64, every quantity small enough to do by hand."""
+    cxv = np.zeros(64, np.int8); cwv = np.zeros(64, np.int8)
+    cxv[:12] = [1, -2, 3, 0, 7, -8, 1, 1, 2, -3, 5, 4]
+    cwv[:12] = [2, 2, -1, 5, 1, 1, 0, -4, 3, 3, -2, 6]
+    qx, qw = orc.pack_i4(cxv[None, :], sym=True), orc.pack_i4(cwv[None, :], sym=True)
+    acc = orc.matmul_s4(qx, qw)
+    acc_l = 2 - 4 - 3 + 0 + 7 - 8 + 0 - 4 + 6 - 9          # first ten products
+    assert acc[0, 0] == acc_l + (-10 + 24)
+    rx = int(cxv.sum()); rxl = 1 - 2 + 3 + 0 + 7 - 8 + 1 + 1 + 2 - 3
+    zx, z1, z2 = -8, 3, -2
+    a1 = int(cwv[:10].sum()) - 10 * z1
+    a2 = int(cwv[10:].sum()) - 54 * z2
+    corr_l = acc_l - zx * a1 - z1 * rxl
+    corr_r = 14 - zx * a2 - z2 * (rx - rxl)
+    H = lambda v: np.array([[v]], np.float16)
+    y = orc.asym_dual_rowsum_dequant(acc, qx, H(0.5), H(zx), np.array([rx], np.int32), qw, H(0.25), H(z1), H(2.0), H(z2),
+                                     np.array([a1], np.int32), np.array([a2], np.int32), bias=np.array([1.5], np.float16))
+    want = np.float16(np.float16(np.float32(corr_l) * np.float32(0.125) + np.float32(corr_r) * np.float32(1.0)) + np.float16(1.5))
+    assert y[0, 0] == want
+    assert (corr_l, corr_r) == (acc_l + 8 * a1 - 3 * rxl, 14 + 8 * a2 + 2 * (rx - rxl))
+
+
 def test_abi_validation_rowsum_entries():
     from duqlinear4bitcuda_amd import _lib
     lib = _lib.load()
@@ -84,6 +158,11 @@ def test_abi_validation_rowsum_entries():
     assert lib.duq_linear4bit_forward_rowsum(P, P, P, None, P, P, P, P, None, 4, 4, 64, P, None) == -1
     assert lib.duq_linear4bit_forward_rowsum(P, P, P, P, P, P, P, P, None, 4, 4, 96, P, None) == -3
     assert lib.duq_asym_rowsum_dequant_host(P, P, P, P, P, P, None, None, 4, 4, P, None) == -1
+    dual = lambda *a: lib.duq_asym_dual_rowsum_dequant_host(*a)
+    assert dual(P, P, P, P, P, P, P, P, P, P, P, None, None, 4, 4, 64, P, None) == -1
+    assert dual(P, P, P, P, P, P, P, P, P, P, P, P, None, 4, 4, 96, P, None) == -3
+    assert dual(P, P + 8, P, P, P, P, P, P, P, P, P, P, None, 4, 4, 64, P, None) == -5
+    assert dual(None, None, None, None, None, None, None, None, None, None, None, None, None, 0, 4, 64, None, None) == 0
 
 
 # ------------------------------------------------------------------ GPU parity
@@ -162,3 +241,69 @@ def test_gpu_rowsum_module_config4(dev):
     y_ref_mode, *_ = orc.linear4bit_asq_forward(x, *orc.weight_asym_from_linear(w), bias=lin.bias.detach().cpu().numpy())
     rel_ref_mode = np.linalg.norm(y_ref_mode.astype(np.float64) - true) / np.linalg.norm(true)
     assert rel < 0.25 and rel < 0.5 * rel_ref_mode, (rel, rel_ref_mode)  # 4-bit x 4-bit noise, not a broken correction
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N,K", [(1, 64, 64), (7, 130, 128), (48, 1000, 256), (300, 1027, 320), (512, 4096, 4096),
+                                   (33, 4100, 1024), (2050, 96, 64)])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_gpu_dual_rowsum_dequant(hip, dev, M, N, K, with_bias):
+    """The dual-uniform row-sum epilogue through the C ABI against the oracle: aligned and ragged widths, more
+    than one column block, more rows than one row group."""
+    print("dual rowsum", M, N, K, with_bias, flush=True)
+    rng = np.random.default_rng(M + 3 * N + 7 * K)
+    x = cases.acts_uniform(M, K, seed=M + N + K)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float16)
+    w[:, :10] *= 6
+    wq, s1, z1, s2, z2, a1, a2 = orc.weight_asym_dual_shifted_from_linear(w)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float16) if with_bias else None
+    want, acc, qx, sx, zx, rx = orc.linear4bit_duasq_rowsum_forward(x, wq, s1, z1, s2, z2, a1, a2, bias)
+    T = lambda v: cases.t(v, dev)
+    q, s, z, r = hip.quantize_rows_asym_shifted(T(x))
+    acc_gpu = hip.matmul(q, T(wq))
+    assert np.array_equal(acc_gpu.cpu().numpy(), acc)
+    got = hip.asym_dual_rowsum_dequant(acc_gpu, q, s, z, r, T(wq), T(s1), T(z1), T(s2), T(z2), T(a1), T(a2),
+                                       None if bias is None else T(bias))
+    assert cases.bits_equal(got.cpu().numpy(), want)
+
+
+@pytest.mark.gpu
+def test_gpu_dual_rowsum_module_config4(dev):
+    """Config 4 (M=512, K=N=4096, activations ~U[0,6]) through LinearQuant4bitDUASQRowSum: weights prepared on the
+    device equal the oracle's, the forward equals the oracle, and the result is close to the fp16 layer it
+    replaces, where the reference's dual-uniform epilogue is not."""
+    from duqlinear4bitcuda_amd.nn import LinearQuant4bitDUASQRowSum
+    M, K, N = 512, 4096, 4096
+    x = cases.acts_uniform(M, K, seed=4)
+    g = torch.Generator().manual_seed(45)
+    lin = torch.nn.Linear(K, N, bias=True).half()
+    with torch.no_grad():
+        wt = torch.randn(N, K, generator=g) * 0.02
+        wt[:, :10] *= 6                                  # outlier input channels in the first range
+        lin.weight.copy_(wt.half())
+        lin.bias.copy_(torch.randn(N, generator=g).half())
+    mod = LinearQuant4bitDUASQRowSum.from_linear(lin.to(dev))
+    w = lin.weight.detach().cpu().numpy()
+    wq, s1, z1, s2, z2, a1, a2 = orc.weight_asym_dual_shifted_from_linear(w)
+    assert np.array_equal(mod.weight.cpu().numpy(), wq)
+    for name, want in (("weight_scales_1", s1), ("weight_zeros_1", z1), ("weight_scales_2", s2), ("weight_zeros_2", z2)):
+        assert cases.bits_equal(getattr(mod, name).cpu().numpy(), want), name
+    assert np.array_equal(mod.weight_rowsum_1.cpu().numpy(), a1) and np.array_equal(mod.weight_rowsum_2.cpu().numpy(), a2)
+    y = mod(cases.t(x, dev).view(2, 256, K))
+    assert y.shape == (2, 256, N)
+    b = lin.bias.detach().cpu().numpy()
+    want, *_ = orc.linear4bit_duasq_rowsum_forward(x, wq, s1, z1, s2, z2, a1, a2, b)
+    assert cases.bits_equal(y.view(M, N).cpu().numpy(), want)
+    true = x.astype(np.float64) @ w.astype(np.float64).T + b.astype(np.float64)
+    rel = np.linalg.norm(want.astype(np.float64) - true) / np.linalg.norm(true)
+    # the reference's layer on the same weights (its own preparation and epilogue)
+    from duqlinear4bitcuda_amd.nn import LinearQuant4bitDUASQ
+    ref_mod = LinearQuant4bitDUASQ.from_linear(lin.cpu()).to(dev)
+    y_ref = ref_mod(cases.t(x, dev)).float().cpu().numpy().astype(np.float64)
+    rel_ref = np.linalg.norm(y_ref - true) / np.linalg.norm(true)
+    print("relative error: dual row-sum", rel, "reference dual epilogue", rel_ref, flush=True)
+    assert rel < 0.25 and rel < 0.5 * rel_ref, (rel, rel_ref)
+    # state_dict round trip
+    other = LinearQuant4bitDUASQRowSum(K, N, bias=True).to(dev)
+    other.load_state_dict(mod.state_dict())
+    assert torch.equal(other(cases.t(x, dev)).view(torch.int16), y.view(M, N).view(torch.int16))
