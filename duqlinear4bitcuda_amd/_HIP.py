@@ -445,8 +445,7 @@ def quantize_linear4bit_forward(x, w, w_scale_1, w_scale_2=None, bias=None, clip
     larger inputs run the two launches with the codes staged in a buffer allocated here.  With
     ``return_quantized`` also returns (codes uint8 [..., K/2], scales [..., 1]).  ``static=True`` stages in the
     library's static device array instead (``duq_quantize_linear4bit_forward_static``: nothing but the outputs is
-    allocated, 5..16 rows of up to 8192 elements are ONE launch too; calls that overlap on one GPU race on the
-    array, and M * K / 2 <= 8 MiB)."""
+    allocated; calls that overlap on one GPU race on the array, and M * K / 2 <= 8 MiB)."""
     name = "quantize_linear4bit_forward"
     if not isinstance(x, torch.Tensor) or not isinstance(w, torch.Tensor):
         raise RuntimeError(f"{name}: x and w must be tensors")
