@@ -72,24 +72,6 @@ __device__ __forceinline__ int group_sum(int v)
     return v;
 }
 
-template <int CTRL>
-__device__ __forceinline__ uint32_t dpp_max(uint32_t v)
-{
-    return max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true));
-}
-// maximum over the 64 lanes, the same value in every lane (four DPP steps inside the rows of 16, then the four
-// rows through scalar registers)
-__device__ __forceinline__ uint32_t wave_max_u32_dpp(uint32_t v)
-{
-    v = dpp_max<0xB1>(v);
-    v = dpp_max<0x4E>(v);
-    v = dpp_max<0x141>(v);
-    v = dpp_max<0x140>(v);
-    const uint32_t a = (uint32_t)__builtin_amdgcn_readlane((int)v, 0), b = (uint32_t)__builtin_amdgcn_readlane((int)v, 16);
-    const uint32_t c = (uint32_t)__builtin_amdgcn_readlane((int)v, 32), d = (uint32_t)__builtin_amdgcn_readlane((int)v, 48);
-    return max(max(a, b), max(c, d));
-}
-
 __device__ __forceinline__ v4u load16(const void *p) { return *reinterpret_cast<const v4u *>(p); }
 
 template <int MODE>
@@ -185,7 +167,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DecodeParams p
         for (int j = 0; j < UPL; ++j)
 #pragma unroll
             for (int q = 0; q < 4; ++q) am = pk_absmax_u16(am, raw[j][q]);
-        uint32_t m16 = wave_max_u32_dpp(max(am & 0xFFFFu, am >> 16));
+        uint32_t m16 = wave_max_u32(max(am & 0xFFFFu, am >> 16));
         if (WPR > 1) {  // the row's maximum crosses its wavefronts through LDS
             if (lane == 0) rmax[wave] = m16;
             __syncthreads();

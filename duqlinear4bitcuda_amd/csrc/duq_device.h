@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace duq {
 
 typedef _Float16 f16;
@@ -38,24 +40,47 @@ __device__ __forceinline__ f16 acc_to_f16(int acc) { return (f16)(float)acc; }
 
 __device__ __forceinline__ int clampi(int v, int lo, int hi) { return min(max(v, lo), hi); }
 
-// 64-lane butterfly reductions (wavefront shuffles, no LDS traffic, no barrier).
+// 64-lane reductions, the same value in every lane: four DPP steps inside the rows of 16 lanes (two quad
+// permutations, half-row mirror, row mirror: plain vector instructions, no trip through the LDS crossbar that a
+// lane shuffle takes), then the four rows through scalar registers.
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_get(uint32_t v)
+{
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true);
+}
+template <typename T, typename OP>
+__device__ __forceinline__ T wave_reduce_dpp(T v, OP op)
+{
+    auto step = [&](auto ctrl) {
+        const uint32_t o = dpp_get<decltype(ctrl)::value>(__builtin_bit_cast(uint32_t, v));
+        v = op(v, __builtin_bit_cast(T, o));
+    };
+    step(std::integral_constant<int, 0xB1>{});   // quad_perm [1,0,3,2]
+    step(std::integral_constant<int, 0x4E>{});   // quad_perm [2,3,0,1]
+    step(std::integral_constant<int, 0x141>{});  // row_half_mirror
+    step(std::integral_constant<int, 0x140>{});  // row_mirror
+    const uint32_t bits = __builtin_bit_cast(uint32_t, v);
+    const T a = __builtin_bit_cast(T, (uint32_t)__builtin_amdgcn_readlane((int)bits, 0));
+    const T b = __builtin_bit_cast(T, (uint32_t)__builtin_amdgcn_readlane((int)bits, 16));
+    const T c = __builtin_bit_cast(T, (uint32_t)__builtin_amdgcn_readlane((int)bits, 32));
+    const T d = __builtin_bit_cast(T, (uint32_t)__builtin_amdgcn_readlane((int)bits, 48));
+    return op(op(a, b), op(c, d));
+}
 __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v)
 {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = max(v, (uint32_t)__shfl_xor((int)v, off, kWave));
-    return v;
+    return wave_reduce_dpp(v, [](uint32_t x, uint32_t y) { return max(x, y); });
 }
 __device__ __forceinline__ float wave_max_f32(float v)
 {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
-    return v;
+    return wave_reduce_dpp(v, [](float x, float y) { return fmaxf(x, y); });
 }
 __device__ __forceinline__ float wave_min_f32(float v)
 {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fminf(v, __shfl_xor(v, off, kWave));
-    return v;
+    return wave_reduce_dpp(v, [](float x, float y) { return fminf(x, y); });
+}
+__device__ __forceinline__ int wave_sum_i32(int v)
+{
+    return wave_reduce_dpp(v, [](int x, int y) { return x + y; });
 }
 
 // Reciprocal used for x / s with x, s binary16: float32(x) * rcp is within two float32

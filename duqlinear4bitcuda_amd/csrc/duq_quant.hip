@@ -372,8 +372,7 @@ __global__ __launch_bounds__(WAVES * 64) void quantize_rows_kernel(RowParams p)
         for (uint32_t u = tid; u < nunits; u += T) qrow[u] = quant_unit(xrow[u]);
     }
     if (shifted) {  // uniform branch: sum of (u - 8) over the row
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) code_sum += __shfl_xor(code_sum, off, kWave);
+        code_sum = wave_sum_i32(code_sum);
         if (WAVES > 1) {
             if ((tid & 63u) == 0) red_sum[tid >> 6] = code_sum;
             __syncthreads();
