@@ -232,6 +232,8 @@ __global__ __launch_bounds__(256) void gemm_s4_tile_kernel(GemmParams p)
         }
 }
 
+typedef int v16i __attribute__((ext_vector_type(16)));
+
 // ---------------------------------------------------------------------------------
 // stream kernel (prefill): weights global -> registers, activations through LDS,
 // v_mfma_i32_32x32x32_i8
@@ -266,8 +268,6 @@ __global__ __launch_bounds__(256) void gemm_s4_tile_kernel(GemmParams p)
 // piece at or past the row end is redirected out of bounds and reads as zero).
 constexpr int kCK = 256;         // k elements per chunk (128 packed bytes per row)
 constexpr int kXStride = 272;    // LDS bytes per activation row: 256 expanded + 16 pad
-
-typedef int v16i __attribute__((ext_vector_type(16)));
 
 
 template <int TM, int EPI, bool BIAS>
@@ -413,38 +413,7 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
     }
 
     // ---- epilogue parameters: fetched now so that their latency hides behind the main loop
-    constexpr int MODE = EPI < 0 ? 0 : EPI;
-    const Epilogue &e = p.epi;
-    bool staged = false;
-    v2u raw_s1[TN * 4], raw_z1[TN * 4], raw_s2[TN * 4], raw_z2[TN * 4], raw_bias[TN * 4];
-    v4i raw_rs[TN * 4];
-    RowEpi rowp[TM];
-    if (EPI >= 0) {
-        const bool vec_ld = p.N % 4 == 0 && reinterpret_cast<uintptr_t>(e.s_col_1) % 8 == 0 &&
-                            (MODE == 0 || MODE == 2 || reinterpret_cast<uintptr_t>(e.z_col_1) % 8 == 0) &&
-                            (MODE != 4 || reinterpret_cast<uintptr_t>(e.rs_col) % 16 == 0) &&
-                            (MODE < 2 || reinterpret_cast<uintptr_t>(e.s_col_2) % 8 == 0) &&
-                            (MODE != 3 || reinterpret_cast<uintptr_t>(e.z_col_2) % 8 == 0) &&
-                            (!BIAS || reinterpret_cast<uintptr_t>(e.bias) % 8 == 0);
-        staged = p.N % 8 == 0 && reinterpret_cast<uintptr_t>(p.y) % 16 == 0 && vec_ld;
-#pragma unroll
-        for (int b = 0; b < TM; ++b) {
-            const uint32_t m = min(m0 + b * 32 + l32, p.M - 1);
-            rowp[b] = load_row<MODE>(e, m);
-        }
-        if (staged) {
-#pragma unroll
-            for (int tq = 0; tq < TN * 4; ++tq) {
-                const uint32_t nq = min(n0 + wave * 64 + (tq >> 2) * 32 + (tq & 3) * 8 + h * 4, p.N - 4);
-                raw_s1[tq] = *reinterpret_cast<const v2u *>(e.s_col_1 + nq);
-                if (MODE == 1 || MODE == 3 || MODE == 4) raw_z1[tq] = *reinterpret_cast<const v2u *>(e.z_col_1 + nq);
-                if (MODE == 4) raw_rs[tq] = *reinterpret_cast<const v4i *>(e.rs_col + nq);
-                if (MODE == 2 || MODE == 3) raw_s2[tq] = *reinterpret_cast<const v2u *>(e.s_col_2 + nq);
-                if (MODE == 3) raw_z2[tq] = *reinterpret_cast<const v2u *>(e.z_col_2 + nq);
-                if (BIAS) raw_bias[tq] = *reinterpret_cast<const v2u *>(e.bias + nq);
-            }
-        }
-    }
+#include "duq_stream_epilogue_fetch.inc"
 
     uint32_t cur = 0, nxt = kBuf, nx2 = 2 * kBuf;
     auto rotate = [&]() {
@@ -466,91 +435,104 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
     // before the accumulators are read
     asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 
-    // lane holds, for activation row m = l32 of tile b and weight tile t: registers r = 4*q..4*q+3
-    // are the four consecutive output columns n = 8*q + 4*h + (0..3), q = 0..3
-    if (EPI < 0) {
-        const bool vec_ok = p.N % 4 == 0 && reinterpret_cast<uintptr_t>(p.C) % 16 == 0;
+    constexpr bool kWideStore = false;
+#include "duq_stream_epilogue_store.inc"
+}
+
+// ---------------------------------------------------------------------------------
+// short-row kernel: K <= 256 (one chunk), many tiles; batched products of short rows
+// ---------------------------------------------------------------------------------
+// The stream kernel's tile (32*TM rows x 256 columns, four wavefronts side by side along N, weights global ->
+// registers, activations expanded into LDS, v_mfma_i32_32x32x32_i8, the same epilogue) without its K pipeline: a
+// problem whose rows hold at most 256 elements is one chunk, and a launch is its output stores (a 2048 x 2048 x 128
+// product moves 0.5 MB in and 8 MB out).  One activation buffer that doubles as the epilogue's staging area (37 KB
+// of LDS at 64 rows), only the steps the row length needs, whole-row stores; two workgroups share a CU (about 200
+// registers each) and overlap one another's loads, matrix work and stores.  (Persistent workgroups that request
+// the next tile's operands before the current tile's epilogue measured slower, 93 against 86 us on 32 products of
+// 2048 x 2048 x 128: the loop-carried wait for those loads also waits for the stores issued after them.)
+template <int TM, int EPI, bool BIAS>
+__global__ __launch_bounds__(256, 2) void gemm_s4_shortk_kernel(GemmParams p)
+{
+    constexpr int BM = 32 * TM, BN = 256, TN = 2;
+    constexpr int NXP = TM;  // 16-byte activation pieces per thread
+    constexpr uint32_t kBuf = BM * kXStride, kStage = 4 * BM * 144;
+    __shared__ __attribute__((aligned(16))) uint8_t lds[kBuf > kStage ? kBuf : kStage];
+
+    if (blockIdx.z) batch_shift(p, blockIdx.z);
+    // column blocks fastest: neighbouring workgroups share an activation tile
+    const uint32_t m0 = (blockIdx.x / p.tiles_n) * BM, n0 = (blockIdx.x % p.tiles_n) * BN;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u, wave = tid >> 6;
+    const uint32_t l32 = lane & 31u, h = lane >> 5;
+    const uint32_t kbytes = p.K >> 1;  // <= 128
+
+    const __amdgpu_buffer_rsrc_t rW = make_rsrc(p.B + (uint64_t)n0 * kbytes, min(p.N - n0, (uint32_t)BN) * kbytes);
+    const __amdgpu_buffer_rsrc_t rX = make_rsrc(p.A + (uint64_t)m0 * kbytes, min(p.M - m0, (uint32_t)BM) * kbytes);
+
+    // weights: lane (l32, h) of weight tile j holds piece i = bytes [i*32 + h*16, +16) of row wave*64 + j*32 + l32
+    v4u wreg[TN][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const bool okw = i * 32 + h * 16 < kbytes;  // K % 64 == 0: a piece is all in or all out
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+            wreg[j][i] = buf_load16(rW, okw ? (wave * 64 + j * 32 + l32) * kbytes + i * 32 + h * 16 : kOobOffset, 0);
+    }
+    // activations: thread (row = tid / 8 + 32 * j, piece = tid % 8) -> expanded into LDS (pieces past K as zeros)
+    const uint32_t xq = tid & 7u;
+    v4u xreg[NXP];
+#pragma unroll
+    for (int j = 0; j < NXP; ++j) {
+        const uint32_t row = (tid >> 3) + j * 32;
+        xreg[j] = buf_load16(rX, xq * 16 < kbytes ? row * kbytes + xq * 16 : kOobOffset, 0);
+    }
+#include "duq_stream_epilogue_fetch.inc"
+#pragma unroll
+    for (int j = 0; j < NXP; ++j) {
+        const uint32_t row = (tid >> 3) + j * 32;
+        v4u ev, od;
+        expand_nibbles(xreg[j], ev, od);
+        *reinterpret_cast<v4u *>(lds + row * kXStride + xq * 32) = ev;
+        *reinterpret_cast<v4u *>(lds + row * kXStride + xq * 32 + 16) = od;
+    }
+    __syncthreads();
+
+    v16i acc[TN][TM];
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
         for (int b = 0; b < TM; ++b)
 #pragma unroll
-            for (int t = 0; t < TN; ++t)
+            for (int r = 0; r < 16; ++r) acc[j][b][r] = 0;
+    // step (i, par): weight operand = even (par 0) or odd (par 1) nibbles of piece i, activation fragment at
+    // + i*64 + par*16 of the row; both sides pair the same k values
+    const uint32_t fragX = l32 * kXStride + h * 32;
+    auto steps = [&](int i0, int i1) {
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    v4i v;
+        for (int i = i0; i < i1; ++i) {
+            v4u we[TN], wo[TN];
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) v[r] = acc[t][b][q * 4 + r] >> 8;
-                    store_quad<EPI, BIAS>(p, m0 + b * 32 + l32, n0 + wave * 64 + t * 32 + q * 8 + h * 4, v, vec_ok);
-                }
-    } else {
-        // Fast path (uniform condition): rows of y are 16-byte aligned and the column
-        // parameter arrays 8-byte aligned.  The 128 x 64 fp16 tile of this wavefront goes
-        // through LDS (free now) so that global stores are whole 128-byte lines (the MFMA
-        // layout only offers 16 contiguous bytes per row and instruction), and the code is
-        // branch-free: parameter loads are clamped, stores are buffer stores whose offset
-        // is redirected out of range for rows past M or columns past N.
-        constexpr uint32_t kYStride = 144;  // bytes per staged row: 128 + pad
-        if (staged) {
-            uint8_t *stage = lds + wave * (BM * kYStride);
-            __syncthreads();  // every wavefront is done reading the activation buffers
+            for (int j = 0; j < TN; ++j) expand_nibbles(wreg[j][i], we[j], wo[j]);
 #pragma unroll
-            for (int t = 0; t < TN; ++t)
+            for (int par = 0; par < 2; ++par) {
+                v4i fx[TM];
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const uint32_t ncol = t * 32 + q * 8 + h * 4;  // column inside the wavefront's tile
-                    const uint32_t nq = min(n0 + wave * 64 + ncol, p.N - 4);
-                    const QuadCols<MODE, BIAS> cols = quad_cols_from_raw<MODE, BIAS>(
-                        raw_s1[t * 4 + q], raw_z1[t * 4 + q], raw_s2[t * 4 + q], raw_z2[t * 4 + q], raw_bias[t * 4 + q], nq,
-                        raw_rs[t * 4 + q]);
+                for (int b = 0; b < TM; ++b)
+                    fx[b] = *reinterpret_cast<const v4i *>(lds + fragX + b * 32 * kXStride + i * 64 + par * 16);
 #pragma unroll
-                    for (int b = 0; b < TM; ++b) {
-                        *reinterpret_cast<v2u *>(stage + (b * 32 + l32) * kYStride + ncol * 2) =
-                            v2u{dequant_pair<MODE, BIAS>(acc[t][b][q * 4] >> 8, acc[t][b][q * 4 + 1] >> 8, rowp[b], cols.c[0], cols.c[1]),
-                                dequant_pair<MODE, BIAS>(acc[t][b][q * 4 + 2] >> 8, acc[t][b][q * 4 + 3] >> 8, rowp[b], cols.c[2], cols.c[3])};
-                    }
-                }
-            // the same wavefront wrote and reads its stage: LDS operations complete in order
-            const uint32_t rows_here = min(p.M - m0, (uint32_t)BM);
-            const __amdgpu_buffer_rsrc_t rY = make_rsrc(p.y + (uint64_t)m0 * p.N, rows_here * p.N * 2);
-            const uint32_t piece = lane & 7u, rsub = lane >> 3;
-            const uint32_t ncol0 = n0 + wave * 64 + piece * 8;
+                for (int b = 0; b < TM; ++b)
 #pragma unroll
-            for (int it = 0; it < BM / 8; ++it) {
-                const uint32_t row = it * 8 + rsub;
-                const v4u v = *reinterpret_cast<const v4u *>(stage + row * kYStride + piece * 16);
-                const uint32_t off = (row < rows_here && ncol0 < p.N) ? (row * p.N + ncol0) * 2 : kOobOffset;
-                __builtin_amdgcn_raw_buffer_store_b128(v, rY, (int)off, 0, 0);
-            }
-        } else {
-#pragma unroll 1
-            for (int tq = 0; tq < TN * 4; ++tq) {
-                // generic path (odd N / unaligned pointers): per-element guards; the accumulator
-                // registers are picked with a switch because they cannot be indexed at run time
-                const int t = tq >> 2, q = tq & 3;
-                const uint32_t nq = n0 + wave * 64 + t * 32 + q * 8 + h * 4;
-                if (nq >= p.N) continue;
-                const QuadCols<MODE, BIAS> cols = load_quad_cols<MODE, BIAS>(e.s_col_1, e.z_col_1, e.s_col_2, e.z_col_2,
-                                                                             e.bias, nq, p.N, false, e.rs_col);
-#pragma unroll
-                for (int b = 0; b < TM; ++b) {
-                    const uint32_t m = m0 + b * 32 + l32;
-                    v4i v;
-#pragma unroll
-                    for (int tt = 0; tt < TN; ++tt)
-#pragma unroll
-                        for (int qq = 0; qq < 4; ++qq)
-                            if (tt == t && qq == q) {
-#pragma unroll
-                                for (int r = 0; r < 4; ++r) v[r] = acc[tt][b][qq * 4 + r] >> 8;
-                            }
-                    if (m >= p.M) continue;
-                    uint16_t *dst = p.y + (uint64_t)m * p.N + nq;
-#pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        if (nq + r < p.N) dst[r] = dequant_one<MODE, BIAS>(v[r], rowp[b], cols.c[r]);
-                }
+                    for (int j = 0; j < TN; ++j)
+                        acc[j][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(v4i, par ? wo[j] : we[j]), fx[b],
+                                                                          acc[j][b], 0, 0, 0);
             }
         }
-    }
+    };
+    steps(0, 2);                   // K >= 64 always: pieces 0 and 1 (one of them zeros when K = 64)
+    if (kbytes > 64) steps(2, 4);  // rows of 192 or 256 elements
+    // (the activation buffer becomes the staging area of the epilogue, which waits for every wavefront first)
+    constexpr bool kWideStore = true;
+#include "duq_stream_epilogue_store.inc"
 }
 
 // ---------------------------------------------------------------------------------
@@ -1014,13 +996,19 @@ static void launch_epi(GemmParams &p, hipStream_t stream, uint32_t batch = 1)
         }
     }
     bool narrow = false;
+    if (best_tm && p.K <= 256) {
+        // rows of at most 256 elements: one chunk, the launch is its output stores: the short-row kernel with 64-row
+        // tiles (measured on 32 products of 2048 x 2048 x 128: 86 us against 95 us on the stream kernel's 64-row tiles)
+        p.tiles_m = (p.M + 63) / 64;
+        p.tiles_n = (p.N + 255) / 256;
+        hipLaunchKernelGGL((gemm_s4_shortk_kernel<2, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(256), 0,
+                           stream, p);
+        return;
+    }
     if (batch > 1 && best_tm) {
-        // measured at attention-like batches (32 problems): rows of at most 256 elements leave a workgroup mostly
-        // prologue and epilogue, and 64-row tiles put three workgroups on a CU that overlap them (2048 x 2048 x
-        // 128: 90 us against 115 / 109 us with 128- / 32-row tiles); at most 128 columns fill half of a 256-wide
-        // tile, the 128 x 128 tile kernel is 15 % faster there (2048 x 128 x 2048: 32 against 37 us)
-        if (p.K <= 256 && p.M > 32) best_tm = 2;
-        else if (p.N <= 128 && p.M > 64) { best_tm = 0; narrow = true; }
+        // measured at attention-like batches (32 problems): at most 128 columns fill half of a 256-wide tile, the
+        // 128 x 128 tile kernel is 15 % faster there (2048 x 128 x 2048: 32 against 37 us)
+        if (p.N <= 128 && p.M > 64) { best_tm = 0; narrow = true; }
     }
     if (best_tm) {
         p.tiles_m = (p.M + 32 * best_tm - 1) / (32 * best_tm);
