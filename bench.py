@@ -362,19 +362,26 @@ def int8_layer_section(dev, quick=False):
         return out
     # decode: weights rotated over more than 512 MB of distinct buffers, as in decode_section
     decode = []
-    for (M, K, N) in [(1, 4096, 4096), (16, 4096, 4096), (16, 4096, 11008), (32, 4096, 11008)]:
+    for (M, K, N) in [(1, 4096, 4096), (4, 4096, 4096), (1, 4096, 11008), (16, 4096, 4096), (16, 4096, 11008),
+                      (32, 4096, 11008)]:
         g = torch.Generator().manual_seed(7)
         nbuf = int(600e6 // (N * K)) + 1
         w0 = torch.randint(0, 128, (N, K), dtype=torch.int8, generator=g).to(dev)
-        tiled = [_HIP.weight_tile_8bit(torch.roll(w0, i, 0)) for i in range(nbuf)]
+        # like the layer: up to four rows read `weight` itself (rows kernel), more read its tiled copy
+        few = M <= 4
+        ws = [torch.roll(w0, i, 0).contiguous() if few else _HIP.weight_tile_8bit(torch.roll(w0, i, 0)) for i in range(nbuf)]
         q = torch.randint(0, 127, (M, K), dtype=torch.int8, generator=g).to(dev)
         sx, zx = torch.rand(M, 1, device=dev) + 0.1, torch.zeros(M, 1, device=dev)
         sw, zw = torch.rand(N, 1, device=dev) * 0.01, torch.zeros(N, 1, device=dev)
-        us = graph_time_us([(lambda w=w: _HIP.linear8bit_forward(q, sx, zx, w, sw, zw, tiled_rows=N)) for w in tiled] * 2)
+        us = graph_time_us([(lambda w=w: _HIP.linear8bit_forward(q, sx, zx, w, sw, zw, tiled_rows=None if few else N))
+                            for w in ws] * 2)
+        us_read = graph_time_us([(lambda w=w: _HIP.probe_read(w)) for w in ws] * 2)
         byts = M * K + N * K + 8 * N + 8 * M + 4 * M * N
         decode.append({"M": M, "K": K, "N": N, "gemm_fused_us": round(us, 3), "GBps": round(byts / us / 1e3, 1),
-                       "frac_hbm": round(byts / us / 1e3 / PEAK_HBM_GBS, 4), "weight_buffers": nbuf})
-        del tiled, w0
+                       "frac_hbm": round(byts / us / 1e3 / PEAK_HBM_GBS, 4), "read_floor_us": round(us_read, 3),
+                       "frac_of_read_floor": round(us_read / us, 4), "weight": "row-major" if few else "tiled copy",
+                       "weight_buffers": nbuf})
+        del ws, w0
     out.append({"decode_rotated_weights": decode})
     return out
 

@@ -582,9 +582,122 @@ __global__ __launch_bounds__(256) void gemm_s8_skinny_kernel(Gemm8Params p)
     }
 }
 
+// ---------------------------------------------------------------------------------
+// rows kernel: M <= 4 activation rows on the row-major weight, rows of up to XS KB
+// ---------------------------------------------------------------------------------
+// The 4-bit rows kernel's shape for int8 (src/kernels/gemm.cu:46-81 at M <= 4): v_dot4_i32_i8 straight on the
+// operands, a wavefront owns R weight rows and the whole K range (lane l holds bytes [i*1024 + l*16, +16) of each
+// row: a load instruction covers 1 KB of one row and an activation register serves R rows), every weight load of
+// the workgroup is requested before anything else, the MR * R partial sums of a lane meet the other lanes' through
+// the wavefront's own piece of LDS (no barrier) and a few DPP steps.  A workgroup is four wavefronts: 16 (8 for rows
+// longer than 4 KB) weight rows.
+template <int MR, int XS, bool FUSED, bool BIAS>
+__global__ __launch_bounds__(256) void gemv_s8_rows_kernel(Gemm8Params p)
+{
+    constexpr int R = XS <= 4 ? 4 : 2;  // weight rows per wavefront: at most 16 weight registers of 16 bytes per lane
+    constexpr int V = MR * R;           // partial sums per lane: 2 .. 16
+    constexpr int LPV = 64 / V;         // lanes that finish one sum
+    static_assert((MR == 1 || MR == 2 || MR == 4) && MR * XS <= 16, "activation registers per lane");
+    __shared__ __attribute__((aligned(16))) int red[4][V * 64];
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t n0 = (blockIdx.x * 4 + wave) * R;
+    // loads in the order their data is needed: the activations, then every weight byte of this wavefront, then the
+    // parameters of the output this lane will finish
+    const __amdgpu_buffer_rsrc_t rX = make_rsrc(p.A, p.M * p.K);  // rows past M read as zero
+    v4u xr[MR][XS];
+#pragma unroll
+    for (int m = 0; m < MR; ++m)
+#pragma unroll
+        for (int i = 0; i < XS; ++i) {
+            const uint32_t off = i * 1024 + lane * 16;
+            xr[m][i] = buf_load16(rX, off < p.K ? m * p.K + off : kOobOffset, 0);  // K % 32 == 0 and 16 | off
+        }
+    const __amdgpu_buffer_rsrc_t rW = make_rsrc(p.B + (uint64_t)n0 * p.K, min(p.N - min(n0, p.N), (uint32_t)R) * p.K);
+    v4u w[R][XS];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int i = 0; i < XS; ++i) {
+            const uint32_t off = i * 1024 + lane * 16;
+            w[r][i] = buf_load16(rW, off < p.K ? r * p.K + off : kOobOffset, 0);  // rows past N: beyond the descriptor
+        }
+    const uint32_t myv = lane / LPV, sub = lane % LPV;
+    const uint32_t my_m = myv / R, my_n = n0 + myv % R;
+    float sr = 0.f, zr = 0.f, sc = 0.f, zc = 0.f, bias = 0.f;
+    if (FUSED) {
+        const uint32_t mm = min(my_m, p.M - 1), nn = min(my_n, p.N - 1);
+        sr = p.epi.s_row[mm], zr = p.epi.z_row[mm], sc = p.epi.s_col[nn], zc = p.epi.z_col[nn];
+        if (BIAS) bias = p.epi.bias[nn];
+    }
+
+    int acc[MR][R];
+#pragma unroll
+    for (int m = 0; m < MR; ++m)
+#pragma unroll
+        for (int r = 0; r < R; ++r) acc[m][r] = 0;
+#pragma unroll
+    for (int i = 0; i < XS; ++i)
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int m = 0; m < MR; ++m)
+#pragma unroll
+                for (int d = 0; d < 4; ++d)
+                    acc[m][r] = __builtin_amdgcn_sdot4((int)w[r][i][d], (int)xr[m][i][d], acc[m][r], false);
+
+    // the V sums of 64 lanes each: through this wavefront's piece of LDS (a wavefront's LDS operations execute in
+    // order: no barrier), V entries per lane back, then log2(LPV) DPP steps
+    int *mine = red[wave];
+#pragma unroll
+    for (int v = 0; v < V; ++v) mine[v * 64 + lane] = acc[v / R][v % R];
+    __builtin_amdgcn_wave_barrier();
+    int sum = 0;
+#pragma unroll
+    for (int e = 0; e < V; ++e) sum += mine[lane * V + e];  // = [myv * 64 + sub * V + e]
+    // sum over the LPV consecutive lanes of a group (4 .. 32 lanes)
+    sum += __builtin_amdgcn_update_dpp(0, sum, 0xB1, 0xF, 0xF, true);                  // quad_perm [1,0,3,2]
+    sum += __builtin_amdgcn_update_dpp(0, sum, 0x4E, 0xF, 0xF, true);                  // quad_perm [2,3,0,1]
+    if (LPV >= 8) sum += __builtin_amdgcn_update_dpp(0, sum, 0x141, 0xF, 0xF, true);   // row_half_mirror
+    if (LPV >= 16) sum += __builtin_amdgcn_update_dpp(0, sum, 0x140, 0xF, 0xF, true);  // row_mirror
+    if (LPV >= 32) sum += __shfl_xor(sum, 16, kWave);
+    if (sub == 0 && my_m < p.M && my_n < p.N) {
+        if (FUSED) {
+            float o = dequant_hprec_one(sum, sr, zr, sc, zc);
+            if (BIAS) o = o + bias;
+            p.y[(uint64_t)my_m * p.N + my_n] = o;
+        } else {
+            p.C[(uint64_t)my_m * p.N + my_n] = sum;
+        }
+    }
+}
+
+template <int MR, bool FUSED, bool BIAS>
+static void launch_rows8(const Gemm8Params &p, hipStream_t stream)
+{
+    const uint32_t xs = (p.K + 1023) / 1024;
+#define DUQ_ROWS8K(XS)                                                                                              \
+    hipLaunchKernelGGL((gemv_s8_rows_kernel<MR, XS, FUSED, BIAS>), dim3((p.N + 4 * (XS <= 4 ? 4 : 2) - 1) / (4 * (XS <= 4 ? 4 : 2))), \
+                       dim3(256), 0, stream, p)
+    if (xs <= 2) DUQ_ROWS8K(2);
+    else if (xs <= 4) DUQ_ROWS8K(4);
+    else if constexpr (MR <= 2) DUQ_ROWS8K(8);
+#undef DUQ_ROWS8K
+}
+
+// shapes the rows kernel takes: row-major weight, up to four rows of at most 4096 elements (two rows: 8192), the
+// weight tensor within 32-bit offsets per descriptor (a descriptor covers one wavefront's rows)
+inline bool rows8_takes(uint32_t M, uint32_t K) { return M <= 4 && K <= (M <= 2 ? 8192u : 4096u); }
+
 template <bool FUSED, bool BIAS, bool TILED>
 static void launch_gemm8_variant(Gemm8Params &p, hipStream_t stream)
 {
+    if (!TILED && rows8_takes(p.M, p.K)) {
+        if (p.M == 1) launch_rows8<1, FUSED, BIAS>(p, stream);
+        else if (p.M == 2) launch_rows8<2, FUSED, BIAS>(p, stream);
+        else launch_rows8<4, FUSED, BIAS>(p, stream);
+        return;
+    }
     if (p.M <= 32) {
         const dim3 grid((p.N + 15) / 16);
         if (p.M <= 16)

@@ -457,7 +457,10 @@ class LinearQuant8bitASQ(torch.nn.Module):
         assert type(x) == tensor_utils.PackedQuantizedTensor, \
             "Input should be quantized tensor, or require_quantizer should be passed as initial argument"
         xq, scales_x, zeros_x = x.quantized_x, x.scales_x, x.zeros_x
-        if self.fused and self.tiled:
+        rows = xq.numel() // xq.shape[-1] if xq.shape[-1] else 0
+        # up to four rows (two for rows longer than 4096 elements) run a kernel that reads `weight` itself
+        few_rows = rows <= 4 and self.in_features <= (8192 if rows <= 2 else 4096)
+        if self.fused and self.tiled and not few_rows:
             return tensor_utils.linear8bit_forward(xq, scales_x, zeros_x, self._tiled_weight(), self.weight_scales,
                                                    self.weight_zeros, self.bias, tiled_rows=self.out_features)
         if self.fused:

@@ -371,6 +371,7 @@ def test_gpu_fused_quantizer_8bit_matches_torch_ops(dev, hip):
 
 GEMM_SHAPES = [(1, 1, 32), (5, 7, 64), (32, 64, 96), (16, 16, 32), (9, 40, 96), (17, 250, 416), (32, 1030, 1056),
                (3, 48, 8192), (16, 4096, 4096), (31, 300, 4128),   # skinny kernel: K split over four wavefronts
+               (1, 4096, 4096), (2, 300, 8192), (4, 1000, 4096), (2, 35, 2080), (4, 17, 1056), (1, 5, 8192), (3, 21, 32),   # rows kernel
  (33, 250, 128), (100, 256, 160), (128, 260, 416),
                (129, 512, 1024), (300, 100, 32), (64, 1024, 4096), (65, 300, 224),
                (3, 40, 66560), (40, 300, 33280), (70, 260, 65600),   # long rows
@@ -408,7 +409,7 @@ def test_gpu_asym_dequant_hprec(dev, hip, rows, cols):
     assert got.dtype == F32 and np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
-FWD_SHAPES = [(512, 4096, 128), (300, 3102, 288), (1, 16, 32), (7, 33, 64), (16, 48, 96), (17, 250, 416), (32, 1030, 1056), (4, 4096, 4096), (40, 250, 160), (128, 512, 1024), (130, 1030, 416), (1024, 3072, 256),
+FWD_SHAPES = [(1, 4096, 4096), (2, 250, 5120), (3, 33, 1056), (512, 4096, 128), (300, 3102, 288), (1, 16, 32), (7, 33, 64), (16, 48, 96), (17, 250, 416), (32, 1030, 1056), (4, 4096, 4096), (40, 250, 160), (128, 512, 1024), (130, 1030, 416), (1024, 3072, 256),
               (1000, 3102, 288)]
 
 
