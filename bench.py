@@ -66,6 +66,21 @@ def profile_traffic_bytes(name, kernel):
     return (int(m.group(1)) + int(m.group(2))) * 1024 if m else None
 
 
+def profile_shape_traffic_bytes(name, kernel, workgroups):
+    """HBM bytes per launch (fetched + written) of `kernel` at the launch shape with `workgroups` workgroups, from the
+    per-shape lines 'workgroups W x T threads: ... fetch avg F KiB  write avg W KiB' of profiles/<name>."""
+    import re
+
+    try:
+        text = open(os.path.join(ROOT, "profiles", name)).read()
+    except OSError:
+        return None
+    for m in re.finditer(r"^  (\S.*)\n    workgroups (\d+) x \d+ threads:.*?fetch avg (\d+) KiB\s+write avg (\d+) KiB", text, re.M):
+        if kernel in m.group(1) and int(m.group(2)) == workgroups:
+            return (int(m.group(3)) + int(m.group(4))) * 1024
+    return None
+
+
 def heavy_tail_acts(M, K, seed, frac=0.01):
     import torch
 
@@ -555,7 +570,11 @@ def main():
                        "achieved": worst["GBps"], "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": worst["frac_hbm"],
                        "shape": {k: worst[k] for k in ("M", "N", "K")},
                        "best_7b_frac": max(d["frac_hbm"] for d in rows_7b),
-                       "read_floor_frac": round(worst["read_floor_GBps"] / PEAK_HBM_GBS, 4), "traffic": None}
+                       "read_floor_frac": round(worst["read_floor_GBps"] / PEAK_HBM_GBS, 4),
+                       # the GEMM launch of that row (the quantizer launch of 16 rows before it moves 0.2 MB)
+                       "traffic": profile_shape_traffic_bytes("decode_kernels__bench_shapes.txt", "gemm_s4_decode_kernel<8, 4, 0>", 256)
+                       if (worst["M"], worst["N"]) == (16, 4096) else None,
+                       "traffic_source": "profiles/decode_kernels__bench_shapes.txt"}
 
     cpu = None
     if not args.no_cpu:
