@@ -209,6 +209,8 @@ def test_dequant_kernels(hip, dev, M, N):
                                    # the stream kernel at its three tile heights, aligned and ragged epilogues:
                                    # 64 rows (1024 x 4096, 900 x 4100), 32 rows (200 x 2051), 128 rows (1100 x 8200)
                                    (1024, 4096, 512), (900, 4100, 128), (200, 2051, 192), (1100, 8200, 320),
+                                   # the short-row kernel (K <= 256): whole-line and ragged epilogues, every step count
+                                   (300, 1024, 64), (520, 2048, 256), (1000, 520, 192), (65, 4096, 128),
                                    # two to four rows on either decode kernel
                                    (2, 512, 8192), (3, 300, 20480), (4, 1000, 4096), (2, 300, 4096),
                                    # ring kernel

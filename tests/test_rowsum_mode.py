@@ -190,7 +190,8 @@ def test_gpu_quantize_rows_asym_shifted(hip, dev, M, K):
 @pytest.mark.gpu
 @pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (4, 1000, 512), (16, 4096, 4096), (9, 300, 8192), (48, 96, 256),
                                    (100, 257, 320), (512, 4096, 4096), (300, 1000, 4160), (2048, 4096, 1024),
-                                   (900, 4100, 128), (200, 2051, 192), (48, 4099, 1024), (33, 300, 8192), (12, 300, 11008)])
+                                   (900, 4100, 128), (200, 2051, 192), (48, 4099, 1024), (33, 300, 8192), (12, 300, 11008),
+                                   (520, 2048, 256), (300, 1024, 64)])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_gpu_rowsum_forward(hip, dev, M, N, K, with_bias):
     """Every GEMM kernel family (dot, skinny, tile, stream; aligned and ragged epilogues) in row-sum mode:
