@@ -30,7 +30,9 @@ SHAPES = [(1, 64, 64), (1, 20, 128), (2, 37, 4096), (3, 100, 2048), (4, 4096, 40
           (5, 64, 64), (16, 48, 128), (7, 100, 4096), (16, 4096, 4096), (16, 1000, 11008), (9, 257, 8192),
           (13, 77, 12288), (8, 50, 2112), (16, 32, 6208),
           (16, 11008, 4096), (6, 8200, 8192), (11, 8192, 2048),
-          (12, 40, 16384), (16, 24, 12352)]
+          (12, 40, 16384), (16, 24, 12352),
+          # rows longer than 16384 elements: the dot kernel
+          (1, 300, 20480), (1, 64, 28672), (1, 130, 16448), (2, 100, 20480), (4, 40, 28672)]
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES)
@@ -97,6 +99,32 @@ def test_fp16_input_special_rows_and_clamps(hip, dev, M):
     x[3] = np.float16(3e-7)
     x = np.ascontiguousarray(x[:M]) if M > 1 else np.ascontiguousarray(x[[1]])
     wq, sw = cases.weights_random_nibbles(N, K, seed=9)
+    for clip, qmax in ((1.0, 6), (0.9, 7)):
+        sx = orc.sym_scales(x, clip)
+        q = orc.sym_quant(x, sx, qmax)
+        want = orc.sym_dequant(orc.matmul_s4(q, wq), sx, sw)
+        y, qf, sf = hip.quantize_linear4bit_forward(cases.t(x, dev), cases.t(wq, dev), cases.t(sw, dev), clip=clip,
+                                                    qmax=qmax, return_quantized=True)
+        assert np.array_equal(qf.cpu().numpy(), q) and cases.bits_equal(sf.cpu().numpy(), sx)
+        assert cases.bits_equal(y.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("kind", ["zeros", "inf", "nan", "subnormal", "normal"])
+def test_fp16_input_one_long_row(hip, dev, kind):
+    """One row of 20480 elements (quantizer launch + dot kernel): special rows, clip 0.9 and both upper clamps give
+    the stand-alone quantizer's codes and scales and the oracle's outputs."""
+    _say("long row", kind)
+    N, K = 40, 20480
+    x = cases.acts_normal(1, K, seed=15)
+    if kind == "zeros":
+        x[:] = 0
+    elif kind == "inf":
+        x[0, 20000] = -np.inf
+    elif kind == "nan":
+        x[0, 17] = np.nan
+    elif kind == "subnormal":
+        x[:] = np.float16(-2e-7)
+    wq, sw = cases.weights_random_nibbles(N, K, seed=19)
     for clip, qmax in ((1.0, 6), (0.9, 7)):
         sx = orc.sym_scales(x, clip)
         q = orc.sym_quant(x, sx, qmax)
