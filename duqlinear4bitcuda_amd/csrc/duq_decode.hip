@@ -162,12 +162,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DecodeParams p
     }
 
     if (FUSEQ) {
-        uint32_t am = 0;
+        PkMinMax st;  // units past the row end read as zero, which changes no maximum of |x|
 #pragma unroll
-        for (int j = 0; j < UPL; ++j)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) am = pk_absmax_u16(am, raw[j][q]);
-        uint32_t m16 = wave_max_u32(max(am & 0xFFFFu, am >> 16));
+        for (int j = 0; j < UPL; ++j) st.add8(raw[j]);
+        uint32_t m16 = wave_max_u32(st.absmax_bits());
         if (WPR > 1) {  // the row's maximum crosses its wavefronts through LDS
             if (lane == 0) rmax[wave] = m16;
             __syncthreads();

@@ -237,22 +237,9 @@ __global__ __launch_bounds__(WAVES * 64) void quantize_rows_kernel(RowParams p)
     auto unit_of = [&](int i) -> uint32_t { return tid + i * T; };
 
     v4u regs[kMaxUnits];
-    uint32_t amax = 0;        // sym: packed max of |x| bit patterns (NaN patterns win, as in torch.max)
-    float fmin_ = INFINITY;   // asym
-    float fmax_ = -INFINITY;
+    PkMinMax st;  // packed running maximum and minimum of this lane's elements
 
-    auto reduce_unit = [&](const v4u &g) {
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            amax = pk_absmax_u16(amax, g[w]);  // asym: only to see NaNs, which fminf / fmaxf drop
-            if (ASYM) {
-                const float lo = (float)bits_to_f16((uint16_t)(g[w] & 0xFFFFu));
-                const float hi = (float)bits_to_f16((uint16_t)(g[w] >> 16));
-                fmin_ = fminf(fmin_, fminf(lo, hi));
-                fmax_ = fmaxf(fmax_, fmaxf(lo, hi));
-            }
-        }
-    };
+    auto reduce_unit = [&](const v4u &g) { st.add8(g); };
 
     if (CACHED) {
 #pragma unroll
@@ -267,14 +254,17 @@ __global__ __launch_bounds__(WAVES * 64) void quantize_rows_kernel(RowParams p)
         for (uint32_t u = tid; u < nunits; u += T) reduce_unit(xrow[u]);
     }
 
-    // ---- row reduction: shuffles inside a wavefront, one LDS hop across wavefronts ----
+    // ---- row reduction: DPP steps inside a wavefront, one LDS hop across wavefronts ----
     float a, b = 0.f;
-    uint32_t m16 = wave_max_u32(max(amax & 0xFFFFu, amax >> 16));  // largest |x| bit pattern; above 0x7C00: a NaN
+    uint32_t m16;  // largest |x| bit pattern; above 0x7C00: a NaN (which fminf / fmaxf would drop)
     if (!ASYM) {
+        m16 = wave_max_u32(st.absmax_bits());
         a = __builtin_bit_cast(float, m16);  // carried as raw bits
     } else {
-        a = wave_min_f32(fmin_);
-        b = wave_max_f32(fmax_);
+        st.wave_reduce();
+        m16 = st.absmax_bits();
+        a = st.min_f32();
+        b = st.max_f32();
     }
     if (WAVES > 1) {
         const uint32_t wave = tid >> 6;
