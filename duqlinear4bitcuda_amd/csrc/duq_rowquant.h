@@ -85,7 +85,7 @@ struct RowQuant {
     f16 s, z;
     float rcp, rcp_fast;
     int zi, qmax;
-    bool fast, clamped;
+    bool fast, clamp_lo, clamp_hi;
     v2h lo2, hi2;
     uint32_t zadd;
 
@@ -142,9 +142,9 @@ struct RowQuant {
         // large for exact binary16 bounds runs the element-wise path.
         //
         // h(x * rcp) grows with x, so the row's extreme values bound every quotient of the row, and a row whose
-        // bounds already round into the code range needs no clamp at all: `clamped` is false for it.
-        //   sym : |x| <= am, so every quotient lies in [-t, t] with t = h(am * rcp); no clamp when t rounds to at
-        //         most min(qmax, 8) (t < qmax + 0.5 and t <= 8.5: ties go to the even integer).
+        // bound already rounds into the code range needs no clamp on that side.
+        //   sym : |x| <= am, so every quotient lies in [-t, t] with t = h(am * rcp); no lower clamp when
+        //         t <= 8.5 (ties go to the even integer), no upper one when t < qmax + 0.5.
         //   asym: the zero point is -rint(h(mn * rcp)) (rounding is symmetric), so the smallest code of the row
         //         is exactly 0 and the lower clamp never acts on a finite row; the upper one does not when
         //         rint(h(mx * rcp)) + zi <= 15.
@@ -157,19 +157,22 @@ struct RowQuant {
             float tf = (float)bits_to_f16((uint16_t)am_bits) * rcp_fast;
             asm volatile("" : "+v"(tf));
             const float t = (float)(f16)tf;
-            clamped = !(t < (float)qmax + 0.5f && t <= 8.5f);
+            clamp_lo = !(t <= 8.5f);
+            clamp_hi = !(t < (float)qmax + 0.5f);
         } else {
             fast = fabsf(mn_f) < 65520.f && fabsf(mx_f) < 65520.f && s_bits != 0 && s_bits < 0x7C00u && zi >= -480 &&
                    zi <= 480;
             float tf = mx_f * rcp_fast;
             asm volatile("" : "+v"(tf));
             const float t = __builtin_rintf((float)(f16)tf);
-            clamped = !(t + (float)zi <= 15.f);
+            clamp_lo = false;
+            clamp_hi = !(t + (float)zi <= 15.f);
         }
         // every lane of a wavefront holds the same row statistics: tell the compiler, so that the choice of
         // path is a scalar branch
         fast = __builtin_amdgcn_readfirstlane((int)fast) != 0;
-        clamped = __builtin_amdgcn_readfirstlane((int)clamped) != 0;
+        clamp_lo = __builtin_amdgcn_readfirstlane((int)clamp_lo) != 0;
+        clamp_hi = __builtin_amdgcn_readfirstlane((int)clamp_hi) != 0;
         lo2 = ASYM ? v2h{(f16)(float)(-zi), (f16)(float)(-zi)} : v2h{(f16)-8.0f, (f16)-8.0f};
         hi2 = ASYM ? v2h{(f16)(float)(15 - zi), (f16)(float)(15 - zi)} : v2h{(f16)(float)qmax, (f16)(float)qmax};
         zadd = ASYM ? (((uint32_t)zi & 0xFFFFu) * 0x00010001u) : 0u;
@@ -180,7 +183,7 @@ struct RowQuant {
     // arithmetic, binary16 result); clamp; add 1536, which leaves the codes in the low nibbles of bytes 0 and 2
     // (the high nibbles of those bytes hold the sign extension); asym adds the zero point.  The four pairs go
     // through each stage together so that no instruction waits for the one before it.
-    template <bool CLAMP>
+    template <bool LO, bool HI>
     __device__ __forceinline__ uint32_t quant8_packed(const v4u raw) const
     {
         uint32_t d[4];
@@ -190,15 +193,14 @@ struct RowQuant {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
             asm("v_fma_mixhi_f16 %0, %1, %2, 0 op_sel:[0,1,0] op_sel_hi:[0,1,0]" : "+v"(d[i]) : "v"(rcp_fast), "v"(raw[i]));
-        if (CLAMP) {
-            // written out: the generic minimum / maximum would first canonicalize the opaque results above, one
-            // more instruction per pair that a finite row has no use for
-            if (!ASYM)
+        // written out: the generic minimum / maximum would first canonicalize the opaque results above, one
+        // more instruction per pair that a finite row has no use for
+        if (LO)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) asm("v_pk_max_f16 %0, %0, %1" : "+v"(d[i]) : "v"(lo2));
+            for (int i = 0; i < 4; ++i) asm("v_pk_max_f16 %0, %0, %1" : "+v"(d[i]) : "v"(lo2));
+        if (HI)
 #pragma unroll
             for (int i = 0; i < 4; ++i) asm("v_pk_min_f16 %0, %0, %1" : "+v"(d[i]) : "v"(hi2));
-        }
         uint32_t b[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -224,7 +226,8 @@ struct RowQuant {
     __device__ __forceinline__ uint32_t quant8(const v4u raw) const
     {
         if (!fast) return quant8_exact<ASYM>(raw, rcp, qmax, zi);
-        return clamped ? quant8_packed<true>(raw) : quant8_packed<false>(raw);
+        if (!ASYM && clamp_lo) return quant8_packed<true, true>(raw);
+        return clamp_hi ? quant8_packed<false, true>(raw) : quant8_packed<false, false>(raw);
     }
 };
 

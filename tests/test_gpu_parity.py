@@ -94,7 +94,7 @@ def test_quantize_rows_sym(hip, dev, M, K):
         x[4, :] = 0
         x[4, 9] = 6e-8            # max/7 underflows to a zero scale on a non-zero row
         x[5, :] *= 1e-4           # a subnormal-range row
-    for qmax, clip in ((6, 1.0), (7, 1.0), (6, 0.9)):
+    for qmax, clip in ((6, 1.0), (7, 1.0), (6, 0.9), (6, 0.5), (3, 1.0)):
         s_want = orc.sym_scales(x, clip)
         q_want = orc.sym_quant(x, s_want, qmax)
         q, s = hip.quantize_rows_sym(cases.t(x, dev), clip=clip, qmax=qmax)
@@ -120,6 +120,37 @@ def test_quantize_rows_asym(hip, dev, M, K):
     assert cases.bits_equal(s.cpu().numpy(), s_want)
     assert cases.bits_equal(z.cpu().numpy(), z_want)
     assert np.array_equal(q.cpu().numpy(), q_want)
+
+
+def test_quantize_rows_magnitude_sweep(hip, dev):
+    """Rows of every magnitude binary16 holds, clip ratios on both sides of the point where the lower clamp starts to
+    act (row maximum over scale = 8.5) and upper bounds below, at and above 7: the kernel decides per row which
+    clamps it can leave out, and every such decision has to give the oracle's codes."""
+    M, K = 4096, 64
+    _say("quantize_rows magnitude sweep", M, K)
+    rng = np.random.default_rng(77)
+    mag = np.exp2(rng.uniform(-24.0, 15.9, (M, 1)))
+    with np.errstate(over="ignore"):  # the largest rows overflow to inf here and there: those rows are cases too
+        x = (rng.standard_normal((M, K)) * mag).astype(np.float16)
+        x[::7] = np.round(x[::7] / mag[::7] * 3.0) * (mag[::7] / 3.0).astype(np.float16)  # many exact ties
+    xt = cases.t(x, dev)
+    for qmax, clip in ((6, 1.0), (7, 1.0), (7, 0.83), (7, 0.82), (6, 0.8), (7, 0.5), (2, 1.0), (7, 1.2)):
+        s_want = orc.sym_scales(x, clip)
+        q_want = orc.sym_quant(x, s_want, qmax)
+        q, s = hip.quantize_rows_sym(xt, clip=clip, qmax=qmax)
+        assert cases.bits_equal(s.cpu().numpy(), s_want), (qmax, clip)
+        bad = np.argwhere(q.cpu().numpy() != q_want)
+        assert bad.size == 0, f"qmax {qmax} clip {clip}: first mismatches (row, byte) {bad[:8]}"
+    for shift in (0.0, 0.37, -2.5):
+        with np.errstate(over="ignore", invalid="ignore"):
+            xa = (x.astype(np.float32) + shift * mag).astype(np.float16)
+        s_want, z_want = orc.asym_scales_zeros(xa)
+        q_want = orc.asym_quant(xa, s_want, z_want)
+        q, s, z = hip.quantize_rows_asym(cases.t(xa, dev))
+        assert cases.bits_equal(s.cpu().numpy(), s_want), shift
+        assert cases.bits_equal(z.cpu().numpy(), z_want), shift
+        bad = np.argwhere(q.cpu().numpy() != q_want)
+        assert bad.size == 0, f"shift {shift}: first mismatches (row, byte) {bad[:8]}"
 
 
 # ---------------------------------------------------------------- GEMM
