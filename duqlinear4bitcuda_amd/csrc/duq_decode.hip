@@ -238,19 +238,24 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DecodeParams p
 }
 
 // ---------------------------------------------------------------------------------
-// MFMA kernel: M <= 16, K <= WAVES * SEGS * 128 <= 12288
+// MFMA kernel: M <= 16 * MT, K <= WAVES * SEGS * 128 <= 12288
 // ---------------------------------------------------------------------------------
 // WAVES wavefronts split K: wavefront v owns the 64-byte row segments [v*SEGS, (v+1)*SEGS); lane (l16, g)
-// holds bytes [g*16, +16) of each, of weight row l16 of the tile (MFMA "A" side) and of activation row l16
-// ("B" side), so it ends up with four consecutive output columns of row l16.  Nibble -> byte as in the
+// holds bytes [g*16, +16) of each, of weight row l16 of the tile (MFMA "A" side) and of activation rows
+// 16*t + l16 of the MT row tiles ("B" side), so it ends up with four consecutive output columns of those rows.
+// A weight fragment is expanded once and meets all MT activation fragments: more rows cost matrix instructions
+// and registers (MT * SEGS * 4 for the packed activations), not weight traffic.  Nibble -> byte as in the
 // GEMM kernels: (w & 0xF0F0F0F0) is the four odd-k nibbles times 16, ((w << 4) & 0xF0F0F0F0) the even ones;
 // every product is 256 * a * b and one arithmetic shift recovers the sum.
-template <int WAVES, int SEGS, int EPI>
+template <int WAVES, int SEGS, int EPI, int MT = 1>
 __global__ __launch_bounds__(WAVES * 64) void gemm_s4_decode_kernel(DecodeParams p)
 {
     constexpr int MODE = EPI < 0 ? 0 : EPI;
     static_assert(WAVES == 4 || WAVES == 8, "wavefronts per workgroup");
-    __shared__ v4i part[2][WAVES][64];
+    static_assert(MT >= 1 && MT <= 4, "16-row activation tiles");
+    constexpr int NG = WAVES / 4;             // groups of 256 finishing threads
+    constexpr int FT = (MT + NG - 1) / NG;    // row tiles a finishing thread completes
+    __shared__ v4i part[2][MT][WAVES][64];
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t l16 = lane & 15u, g = lane >> 4;
@@ -278,58 +283,79 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_s4_decode_kernel(DecodeParams
     // ---- loads in the order their data is needed (loads return in order): the activation fragments of this
     // wavefront's k range (packed; expanded when used), the first tile's weights, the parameters of the outputs
     // this thread will finish
-    v4u xp[SEGS];
+    v4u xp[MT][SEGS];
     const __amdgpu_buffer_rsrc_t rX = make_rsrc(p.A, p.M * kbytes);  // rows past M read as zero
 #pragma unroll
-    for (int u = 0; u < SEGS; ++u)
-        xp[u] = buf_load16(rX, koff[u] != kOobOffset ? l16 * kbytes + koff[u] : kOobOffset, 0);
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int u = 0; u < SEGS; ++u)
+            xp[t][u] = buf_load16(rX, koff[u] != kOobOffset ? (t * 16 + l16) * kbytes + koff[u] : kOobOffset, 0);
     v4u w0[SEGS], w1[SEGS];
     load_tile(tile0, w0);
 
-    // threads 0..255 finish one output each: element er of MFMA lane src_lane
-    const uint32_t src_lane = (tid >> 2) & 63u, er = tid & 3u;
+    // threads finish one output per row tile they own: element er of MFMA lane src_lane; the 256-thread group
+    // fg owns row tiles fg, fg + NG, ...
+    const uint32_t src_lane = (tid >> 2) & 63u, er = tid & 3u, fg = tid >> 8;
     const uint32_t my_m = src_lane & 15u, my_c = (src_lane >> 4) * 4 + er;
     const bool bias = p.epi.bias != nullptr;
-    const bool finisher = tid < 256;
+    const bool finisher = fg < (uint32_t)MT;
     ColParams cp{};
-    RowEpi rp{};
+    RowEpi rp[FT];
     auto load_cp = [&](uint32_t tile) {
         ColParams c{};
         if (EPI >= 0 && finisher) c = load_col_rt<MODE>(p.epi, min(tile * 16 + my_c, p.N - 1), bias);
         return c;
     };
     cp = load_cp(tile0);
-    if (EPI >= 0 && finisher) rp = load_row<MODE>(p.epi, min(my_m, p.M - 1));
+#pragma unroll
+    for (int f = 0; f < FT; ++f) {
+        rp[f] = RowEpi{};
+        if (EPI >= 0 && finisher) rp[f] = load_row<MODE>(p.epi, min((fg + f * NG) * 16 + my_m, p.M - 1));
+    }
 
     auto compute_tile = [&](uint32_t tile, const v4u(&w)[SEGS], uint32_t buf) {
         const ColParams cpn = load_cp(tile + 1 < tile_end ? tile + 1 : tile);  // next tile's, under this tile's work
-        v4i acc = v4i{0, 0, 0, 0};
+        v4i acc[MT];
+#pragma unroll
+        for (int t = 0; t < MT; ++t) acc[t] = v4i{0, 0, 0, 0};
 #pragma unroll
         for (int u = 0; u < SEGS; ++u) {
-            v4u we, wo, xe, xo;
+            v4u we, wo;
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 we[q] = (w[u][q] << 4) & kNibbleMaskD;
                 wo[q] = w[u][q] & kNibbleMaskD;
-                xe[q] = (xp[u][q] << 4) & kNibbleMaskD;
-                xo[q] = xp[u][q] & kNibbleMaskD;
             }
-            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i, we), __builtin_bit_cast(v4i, xe), acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i, wo), __builtin_bit_cast(v4i, xo), acc, 0, 0, 0);
-        }
-        part[buf][wave][lane] = acc;
-        __syncthreads();
-        if (finisher) {
-            int sum = 0;
 #pragma unroll
-            for (int w2 = 0; w2 < WAVES; ++w2) sum += part[buf][w2][src_lane][er];
-            sum >>= 8;
-            const uint32_t n = tile * 16 + my_c;
-            if (my_m < p.M && n < p.N) {
-                if (EPI < 0)
-                    p.C[(uint64_t)my_m * p.N + n] = sum;
-                else
-                    p.y[(uint64_t)my_m * p.N + n] = dequant_rt<MODE>(sum, rp, cp, bias);
+            for (int t = 0; t < MT; ++t) {
+                v4u xe, xo;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    xe[q] = (xp[t][u][q] << 4) & kNibbleMaskD;
+                    xo[q] = xp[t][u][q] & kNibbleMaskD;
+                }
+                acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i, we), __builtin_bit_cast(v4i, xe), acc[t], 0, 0, 0);
+                acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i, wo), __builtin_bit_cast(v4i, xo), acc[t], 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < MT; ++t) part[buf][t][wave][lane] = acc[t];
+        __syncthreads();
+#pragma unroll
+        for (int f = 0; f < FT; ++f) {
+            const uint32_t t = fg + f * NG;
+            if (t < (uint32_t)MT) {
+                int sum = 0;
+#pragma unroll
+                for (int w2 = 0; w2 < WAVES; ++w2) sum += part[buf][t][w2][src_lane][er];
+                sum >>= 8;
+                const uint32_t m = t * 16 + my_m, n = tile * 16 + my_c;
+                if (m < p.M && n < p.N) {
+                    if (EPI < 0)
+                        p.C[(uint64_t)m * p.N + n] = sum;
+                    else
+                        p.y[(uint64_t)m * p.N + n] = dequant_rt<MODE>(sum, rp[f], cp, bias);
+                }
             }
         }
         cp = cpn;
@@ -388,12 +414,12 @@ void launch_rows_xs(const DecodeParams &p, int epi, hipStream_t stream)
     else launch_rows_mode<MR, 8, FUSEQ>(p, epi, stream);
 }
 
-template <int WAVES, int SEGS>
+template <int WAVES, int SEGS, int MT = 1>
 void launch_mfma_mode(const DecodeParams &p, int epi, hipStream_t stream)
 {
     const uint32_t ntiles = (p.N + 15) / 16;
     const dim3 grid((ntiles + p.tiles_per_wg - 1) / p.tiles_per_wg);
-#define DUQ_DEC(E) hipLaunchKernelGGL((gemm_s4_decode_kernel<WAVES, SEGS, E>), grid, dim3(WAVES * 64), 0, stream, p)
+#define DUQ_DEC(E) hipLaunchKernelGGL((gemm_s4_decode_kernel<WAVES, SEGS, E, MT>), grid, dim3(WAVES * 64), 0, stream, p)
     switch (epi) {
     case -1: DUQ_DEC(-1); break;
     case 0: DUQ_DEC(0); break;
@@ -419,9 +445,19 @@ void launch_decode_any(DecodeParams &p, int epi, hipStream_t stream)
         const uint32_t ntiles = (p.N + 15) / 16;
         p.tiles_per_wg = decode_tiles_per_workgroup(ntiles);
         constexpr int W = DUQ_DEC_WAVES, S = 32 / W;  // 64-byte segments per wavefront for 2 KB of a row
-        if (kbytes <= 2048) launch_mfma_mode<W, S>(p, epi, stream);
-        else if (kbytes <= 4096) launch_mfma_mode<W, 2 * S>(p, epi, stream);
+        const uint32_t mt = (p.M + 15) / 16;  // 2..4 only with rows of at most 8192 elements (select_gemm_kernel)
+#define DUQ_DEC_MT(T)                                                     \
+    do {                                                                  \
+        if (kbytes <= 2048) launch_mfma_mode<W, S, T>(p, epi, stream);    \
+        else launch_mfma_mode<W, 2 * S, T>(p, epi, stream);               \
+    } while (0)
+        // (three and four row tiles of rows longer than 4096 elements would spill registers: not instantiated)
+        if (mt == 4 && kbytes <= 2048) launch_mfma_mode<W, S, 4>(p, epi, stream);
+        else if (mt == 3 && kbytes <= 2048) launch_mfma_mode<W, S, 3>(p, epi, stream);
+        else if (mt == 2) DUQ_DEC_MT(2);
+        else if (kbytes <= 4096) DUQ_DEC_MT(1);
         else launch_mfma_mode<8, 12>(p, epi, stream);
+#undef DUQ_DEC_MT
     }
 }
 

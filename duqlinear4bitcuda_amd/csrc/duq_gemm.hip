@@ -882,14 +882,16 @@ int select_gemm_kernel(uint32_t M, uint32_t N, uint32_t K)
 {
     const uint64_t wbytes = (uint64_t)N * (K / 2);
     const bool small_offsets = wbytes < 0xFFFFFF00ull && K > 0;
-    // decode: up to 16 rows.  Rows kernel for up to four rows (8 KB of every weight row per wavefront); above,
-    // the MFMA decode kernel (6 KB per row over eight wavefronts), or the skinny kernel once there are 512
-    // column tiles (its whole-line weight loads measure 7-9 % faster there)
+    // decode.  Rows kernel for up to four rows (8 KB of every weight row per wavefront); above, the MFMA decode
+    // kernel (6 KB per row over eight wavefronts; up to 64 rows of at most 4096 elements and 32 of at most 8192 as
+    // two to four row tiles against the same weight fragments), except 9..16 rows on very wide layers, where the
+    // skinny kernel's whole-line weight loads measure 5 % faster (N = 28672, K = 4096)
     if (M <= 4 && K <= 16384 && small_offsets) return kKernelDecodeRows;
     if (M <= 16 && small_offsets) {
-        if ((N + 15) / 16 >= 512 && K <= 8192) return kKernelSkinny;
+        if (M > 8 && (N + 15) / 16 >= 1536 && K <= 4096) return kKernelSkinny;
         if (K <= 12288) return kKernelDecodeMfma;
     }
+    if (M <= 64 && small_offsets && (K <= 4096 || (K <= 8192 && M <= 32))) return kKernelDecodeMfma;
     const uint32_t xstride = ((K / 2 + 127) / 128) * 128;
     // dot kernel: up to four rows too long for the decode kernels
     if (M <= 4 && small_offsets && 4 * xstride <= 60 * 1024) return kKernelDot;

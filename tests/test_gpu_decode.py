@@ -1,4 +1,4 @@
-"""GPU parity of the decode kernels (up to 16 activation rows) and of the quantize + GEMM + dequant entry point
+"""GPU parity of the decode kernels (up to 64 activation rows) and of the quantize + GEMM + dequant entry point
 that takes binary16 activations, against the oracle, through the C ABI."""
 import ctypes
 
@@ -24,13 +24,21 @@ def hip(dev):
 
 
 # rows kernel (M <= 4: every K bucket, K and N tails), MFMA decode kernel (5..16 rows: K buckets of 4096 / 8192 /
-# 12288, tiles that end inside N), skinny kernel (512 or more column tiles), ring kernel for long rows
+# 12288, tiles that end inside N, several tiles per workgroup), ring kernel for long rows
 SHAPES = [(1, 64, 64), (1, 20, 128), (2, 37, 4096), (3, 100, 2048), (4, 4096, 4096), (1, 4096, 4096), (1, 515, 11008),
           (4, 130, 8192), (2, 64, 16384), (3, 33, 12352), (1, 11008, 4096),
           (5, 64, 64), (16, 48, 128), (7, 100, 4096), (16, 4096, 4096), (16, 1000, 11008), (9, 257, 8192),
           (13, 77, 12288), (8, 50, 2112), (16, 32, 6208),
           (16, 11008, 4096), (6, 8200, 8192), (11, 8192, 2048),
           (12, 40, 16384), (16, 24, 12352),
+          # MFMA decode kernel with two to four row tiles (17..64 rows of at most 4096 elements, 17..32 of at most
+          # 8192), one to several column tiles per workgroup, tiles that end inside M and N
+          (17, 4096, 4096), (32, 300, 4096), (33, 4099, 2048), (48, 1000, 4096), (64, 11008, 4096), (50, 72, 64),
+          (64, 40, 128), (20, 520, 8192), (32, 4100, 8192), (29, 9000, 4160), (64, 5000, 1024),
+          # and their neighbours on the ring kernel: more than 32 rows of more than 4096 elements
+          (33, 300, 8192), (64, 130, 4160),
+          # 9..16 rows on 1536 or more column tiles: the skinny kernel
+          (9, 24600, 64), (16, 28672, 256),
           # rows longer than 16384 elements: the dot kernel
           (1, 300, 20480), (1, 64, 28672), (1, 130, 16448), (2, 100, 20480), (4, 40, 28672)]
 
