@@ -89,9 +89,12 @@ __device__ __forceinline__ uint16_t dequant_rt(int acc, const RowEpi &r, const C
 // ---------------------------------------------------------------------------------
 // rows kernel: M <= MR <= 4, K <= XS * 2048
 // ---------------------------------------------------------------------------------
-// WAVES wavefronts of R = 16 / WAVES weight rows each: 16 weight rows per workgroup either way.  Eight wavefronts
-// help when the workgroup quantizes four activation rows itself and a CU holds several workgroups (launcher).
-template <int MR, int XS, bool FUSEQ, int EPI, int WAVES = 4>
+// WAVES wavefronts of R = 16 / WAVES weight rows each: 16 weight rows ("a tile") per workgroup either way.  Eight
+// wavefronts help when the workgroup quantizes four activation rows itself and a CU holds several workgroups
+// (launcher).  MULTI: a workgroup owns p.tiles_per_wg consecutive tiles and keeps two tiles' weights in flight
+// (two register sets that alternate), so that a launch is one round of at most 256 workgroups: the activations
+// are fetched, and with FUSEQ quantized, once per CU and not once per tile.
+template <int MR, int XS, bool FUSEQ, int EPI, int WAVES = 4, bool MULTI = false>
 __global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DecodeParams p)
 {
     constexpr int R = 4 * DUQ_DEC_R / WAVES;  // weight rows per wavefront
@@ -109,12 +112,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DecodeParams p
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t kbytes = p.K >> 1;
-    const uint32_t n0 = (blockIdx.x * WAVES + wave) * R;
-
+    const uint32_t tile0 = MULTI ? blockIdx.x * p.tiles_per_wg : blockIdx.x;
+    const uint32_t tile_end = MULTI ? min(tile0 + p.tiles_per_wg, (p.N + 4 * DUQ_DEC_R - 1) / (4 * DUQ_DEC_R)) : tile0 + 1;
 
     // ---- loads, in the order their data is needed (loads return in order: waiting for one waits for every
-    // earlier one): the activations first, then every weight byte of this wavefront, then the parameters of the
-    // output this lane will finish
+    // earlier one): the activations first, then every weight byte of this wavefront's first tile, then the
+    // parameters of the output this lane will finish
     // activations: lane l needs bytes [i*1024 + l*16, +16) of every row
     v4u xr[MR][XS];
     constexpr int WPR = WAVES / MR;           // wavefronts that share a row in the quantize phase
@@ -142,24 +145,33 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DecodeParams p
         }
     }
     const __amdgpu_buffer_rsrc_t rW = make_rsrc(p.B, p.N * kbytes);
-    v4u w[R][XS];
+    // the weights of tile t for this wavefront (tiles past the workgroup's last read as zero, unused)
+    auto load_w = [&](uint32_t tile, v4u(&w)[R][XS]) {
+        const uint32_t n0 = (tile * WAVES + wave) * R;
+        const uint32_t nrows = (!MULTI || tile < tile_end) ? p.N : 0u;
 #pragma unroll
-    for (int r = 0; r < R; ++r)
+        for (int r = 0; r < R; ++r)
 #pragma unroll
-        for (int i = 0; i < XS; ++i) {
-            const uint32_t off = i * 1024 + lane * 16;
-            const bool ok = off < kbytes && n0 + r < p.N;  // K % 64 == 0: a 16-byte piece is all in or all out
-            w[r][i] = buf_load16(rW, ok ? (n0 + r) * kbytes + off : kOobOffset, 0);
-        }
+            for (int i = 0; i < XS; ++i) {
+                const uint32_t off = i * 1024 + lane * 16;
+                // K % 64 == 0: a 16-byte piece is all in or all out
+                const bool ok = off < kbytes && n0 + r < nrows;
+                w[r][i] = buf_load16(rW, ok ? (n0 + r) * kbytes + off : kOobOffset, 0);
+            }
+    };
+    v4u w0[R][XS], w1[MULTI ? R : 1][MULTI ? XS : 1];
+    load_w(tile0, w0);
     const uint32_t myv = lane / LPV, sub = lane % LPV;
-    const uint32_t my_m = myv / R, my_n = n0 + myv % R;
+    const uint32_t my_m = myv / R, my_r = wave * R + myv % R;  // my_r: weight row inside a tile
     const bool bias = p.epi.bias != nullptr;
-    ColParams cp{};
+    auto load_cp = [&](uint32_t tile) {
+        ColParams c{};
+        if (EPI >= 0) c = load_col_rt<MODE>(p.epi, min(tile * (4 * DUQ_DEC_R) + my_r, p.N - 1), bias);
+        return c;
+    };
+    ColParams cp = load_cp(tile0);
     RowEpi rp{};
-    if (EPI >= 0) {
-        cp = load_col_rt<MODE>(p.epi, min(my_n, p.N - 1), bias);
-        if (!FUSEQ) rp = load_row<MODE>(p.epi, min(my_m, p.M - 1));
-    }
+    if (EPI >= 0 && !FUSEQ) rp = load_row<MODE>(p.epi, min(my_m, p.M - 1));
 
     if (FUSEQ) {
         PkMinMax st;  // units past the row end read as zero, which changes no maximum of |x|
@@ -200,40 +212,57 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DecodeParams p
         rp.s = bits_to_f16(srow[min(my_m, (uint32_t)MR - 1)]);
     }
 
-    // ---- dot products on the packed nibbles
-    int acc[MR][R];
+    auto do_tile = [&](uint32_t tile, const v4u(&w)[R][XS], const ColParams &c) {
+        // ---- dot products on the packed nibbles
+        int acc[MR][R];
 #pragma unroll
-    for (int m = 0; m < MR; ++m)
+        for (int m = 0; m < MR; ++m)
 #pragma unroll
-        for (int r = 0; r < R; ++r) acc[m][r] = 0;
+            for (int r = 0; r < R; ++r) acc[m][r] = 0;
 #pragma unroll
-    for (int i = 0; i < XS; ++i)
+        for (int i = 0; i < XS; ++i)
 #pragma unroll
-        for (int r = 0; r < R; ++r)
+            for (int r = 0; r < R; ++r)
 #pragma unroll
-            for (int m = 0; m < MR; ++m)
+                for (int m = 0; m < MR; ++m)
 #pragma unroll
-                for (int d = 0; d < 4; ++d)
-                    acc[m][r] = __builtin_amdgcn_sdot8((int)w[r][i][d], (int)xr[m][i][d], acc[m][r], false);
+                    for (int d = 0; d < 4; ++d)
+                        acc[m][r] = __builtin_amdgcn_sdot8((int)w[r][i][d], (int)xr[m][i][d], acc[m][r], false);
 
-    // ---- the V sums of 64 lanes each: through this wavefront's piece of LDS (a wavefront's LDS operations
-    // execute in order: no barrier), V entries per lane back, then log2(LPV) DPP steps
-    int *mine = red[wave];
+        // ---- the V sums of 64 lanes each: through this wavefront's piece of LDS (a wavefront's LDS operations
+        // execute in order: no barrier), V entries per lane back, then log2(LPV) DPP steps
+        int *mine = red[wave];
 #pragma unroll
-    for (int v = 0; v < V; ++v) mine[v * 64 + lane] = acc[v / R][v % R];
-    __builtin_amdgcn_wave_barrier();
-    int sum = 0;
+        for (int v = 0; v < V; ++v) mine[v * 64 + lane] = acc[v / R][v % R];
+        __builtin_amdgcn_wave_barrier();
+        int sum = 0;
 #pragma unroll
-    for (int e = 0; e < V / 4; ++e) {
-        const v4i t = *reinterpret_cast<const v4i *>(&mine[lane * V + e * 4]);  // = [myv * 64 + sub * V + e * 4]
-        sum += (t[0] + t[1]) + (t[2] + t[3]);
-    }
-    sum = group_sum<LPV>(sum);
-    if (sub == 0 && my_m < p.M && my_n < p.N) {
-        if (EPI < 0)
-            p.C[(uint64_t)my_m * p.N + my_n] = sum;
-        else
-            p.y[(uint64_t)my_m * p.N + my_n] = dequant_rt<MODE>(sum, rp, cp, bias);
+        for (int e = 0; e < V / 4; ++e) {
+            const v4i t = *reinterpret_cast<const v4i *>(&mine[lane * V + e * 4]);  // = [myv * 64 + sub * V + e * 4]
+            sum += (t[0] + t[1]) + (t[2] + t[3]);
+        }
+        __builtin_amdgcn_wave_barrier();
+        sum = group_sum<LPV>(sum);
+        const uint32_t my_n = tile * (4 * DUQ_DEC_R) + my_r;
+        if (sub == 0 && my_m < p.M && my_n < p.N) {
+            if (EPI < 0)
+                p.C[(uint64_t)my_m * p.N + my_n] = sum;
+            else
+                p.y[(uint64_t)my_m * p.N + my_n] = dequant_rt<MODE>(sum, rp, c, bias);
+        }
+    };
+
+    if constexpr (!MULTI) {
+        do_tile(tile0, w0, cp);
+    } else {
+        for (uint32_t t = tile0; t < tile_end; t += 2) {
+            load_w(t + 1, w1);
+            const ColParams cp1 = load_cp(t + 1 < tile_end ? t + 1 : t);
+            do_tile(t, w0, cp);
+            load_w(t + 2, w0);
+            cp = load_cp(t + 2 < tile_end ? t + 2 : t);
+            if (t + 1 < tile_end) do_tile(t + 1, w1, cp1);
+        }
     }
 }
 
@@ -375,15 +404,26 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_s4_decode_kernel(DecodeParams
 // dispatch
 // ---------------------------------------------------------------------------------
 template <int MR, int XS, bool FUSEQ>
-void launch_rows_mode(const DecodeParams &p, int epi, hipStream_t stream)
+void launch_rows_mode(DecodeParams &p, int epi, hipStream_t stream)
 {
-    const dim3 grid((p.N + 4 * DUQ_DEC_R - 1) / (4 * DUQ_DEC_R));  // 16 weight rows per workgroup
-    // eight wavefronts when four rows are quantized in the kernel and a CU gets more than one workgroup (measured,
-    // N = 11008, K = 4096: 7.9 against 8.3 us; with one workgroup per CU the vector work per SIMD is the same and
-    // four wavefronts are ahead, N = 4096: 4.8 against 5.1 us)
-    const bool wide = FUSEQ && MR == 4 && grid.x > 256;
+    const uint32_t ntiles = (p.N + 4 * DUQ_DEC_R - 1) / (4 * DUQ_DEC_R);  // 16 weight rows per tile
+    // One tile per workgroup.  Four rows quantized in the kernel, more than 256 tiles: every workgroup quantizes
+    // the rows again, so one round of at most 256 workgroups of eight wavefronts with several tiles each when two
+    // register sets of weights fit (rows of at most 8192 elements; measured at K = 4096: N = 6144 5.76 against
+    // 6.21 us, N = 11008 7.18 against 7.73), else eight wavefronts and one tile (N = 11008: 7.9 against 8.3 us with
+    // four; with one workgroup per CU the vector work per SIMD is the same and four wavefronts are ahead,
+    // N = 4096: 4.8 against 5.1 us).  On pre-quantized rows, or with one or two rows, several tiles per workgroup
+    // measured 3-15 % slower than one (four wavefronts per CU keep too few loads in flight): not used there.
+    constexpr bool kCanMulti = FUSEQ && MR == 4 && XS <= 4;
+    const bool multi = kCanMulti && ntiles > 256;
+    p.tiles_per_wg = multi ? (ntiles + 255) / 256 : 1;
+    const dim3 grid((ntiles + p.tiles_per_wg - 1) / p.tiles_per_wg);
+    const bool wide = FUSEQ && MR == 4 && !multi && grid.x > 256;
 #define DUQ_ROWS(E)                                                                                              \
-    if (wide)                                                                                                    \
+    if (multi) {                                                                                                 \
+        if constexpr (kCanMulti)                                                                                 \
+            hipLaunchKernelGGL((gemv_s4_rows_kernel<MR, XS, FUSEQ, E, 8, true>), grid, dim3(512), 0, stream, p);     \
+    } else if (wide)                                                                                             \
         hipLaunchKernelGGL((gemv_s4_rows_kernel<MR, XS, FUSEQ, E, (FUSEQ && MR == 4) ? 8 : 4>), grid, dim3(512), 0,  \
                            stream, p);                                                                           \
     else                                                                                                         \
@@ -405,7 +445,7 @@ void launch_rows_mode(const DecodeParams &p, int epi, hipStream_t stream)
 }
 
 template <int MR, bool FUSEQ>
-void launch_rows_xs(const DecodeParams &p, int epi, hipStream_t stream)
+void launch_rows_xs(DecodeParams &p, int epi, hipStream_t stream)
 {
     const uint32_t kbytes = p.K / 2;
     if (kbytes <= 2048) launch_rows_mode<MR, 2, FUSEQ>(p, epi, stream);

@@ -27,6 +27,8 @@ def hip(dev):
 # 12288, tiles that end inside N, several tiles per workgroup), ring kernel for long rows
 SHAPES = [(1, 64, 64), (1, 20, 128), (2, 37, 4096), (3, 100, 2048), (4, 4096, 4096), (1, 4096, 4096), (1, 515, 11008),
           (4, 130, 8192), (2, 64, 16384), (3, 33, 12352), (1, 11008, 4096),
+          # three or four rows from binary16 on more than 256 column tiles: several tiles per workgroup
+          (4, 11008, 4096), (3, 4500, 8192), (4, 9001, 2048), (4, 16384, 64), (4, 4112, 12288),
           (5, 64, 64), (16, 48, 128), (7, 100, 4096), (16, 4096, 4096), (16, 1000, 11008), (9, 257, 8192),
           (13, 77, 12288), (8, 50, 2112), (16, 32, 6208),
           (16, 11008, 4096), (6, 8200, 8192), (11, 8192, 2048),
