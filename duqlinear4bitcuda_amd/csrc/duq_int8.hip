@@ -583,6 +583,178 @@ __global__ __launch_bounds__(256) void gemm_s8_skinny_kernel(Gemm8Params p)
 }
 
 // ---------------------------------------------------------------------------------
+// decode kernel (5 <= M <= 64 on the row-major weight): one round of workgroups, activations held in registers
+// ---------------------------------------------------------------------------------
+// The 4-bit MFMA decode kernel's shape for int8 (src/kernels/gemm.cu:46-81 at small M): eight wavefronts split K
+// for one 16-column tile (wavefront v owns the 64-byte row segments [v*SEGS, (v+1)*SEGS)); lane (l16, g) holds
+// bytes [g*16, +16) of each segment, of weight row l16 of the tile (MFMA "A" side) and of activation rows
+// 16*t + l16 of the MT row tiles ("B" side), the operand layout of v_mfma_i32_16x16x64_i8.  A lane keeps its
+// activation fragments in registers for the whole launch and a workgroup owns p.tiles_n consecutive column tiles
+// with two tiles' weights in flight (two register sets alternate), so a launch is one round of at most 256
+// workgroups and the activations (as many bytes as a tile's weights at 16 rows) enter a CU once.  The partial
+// tiles meet in LDS; MT * 64 threads finish four consecutive columns of one row each.
+template <int SEGS, int MT, bool FUSED, bool BIAS, bool TILED>
+__global__ __launch_bounds__(512) void gemm_s8_decode_kernel(Gemm8Params p)
+{
+    constexpr int WAVES = 8;
+    __shared__ v4i part[2][MT][WAVES][64];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t l16 = lane & 15u, g = lane >> 4;
+    const uint32_t ntiles = (p.N + 15) / 16;
+    const uint32_t tile0 = blockIdx.x * p.tiles_n;
+    const uint32_t tile_end = min(tile0 + p.tiles_n, ntiles);
+
+    // rows past N read as zero (the tiled copy holds whole 32-row tiles, zero-padded); N * K < 2^32 - 32 * K (launcher)
+    const __amdgpu_buffer_rsrc_t rW = make_rsrc(p.B, (TILED ? (p.N + 31u) / 32u * 32u : p.N) * p.K);
+    const __amdgpu_buffer_rsrc_t rX = make_rsrc(p.A, p.M * p.K);  // rows past M read as zero
+    uint32_t koff[SEGS];  // byte offset inside a row, or out of range for pieces past K (K % 32 == 0 and 16 | off)
+#pragma unroll
+    for (int u = 0; u < SEGS; ++u) {
+        const uint32_t off = (wave * SEGS + u) * 64 + g * 16;
+        koff[u] = off < p.K ? off : kOobOffset;
+    }
+    // row-major: 16 rows x 64 contiguous bytes per load instruction.  Tiled copy (fragments of 32 rows x 32 bytes,
+    // 1 KB each in lane order (r, h) -> (h * 32 + r) * 16): the 16 bytes of (row, 64 * j + 16 * g) sit in fragment
+    // ks = 2 * j + g / 2 at lane (h = g % 2, r = row % 32): four runs of 256 contiguous bytes per instruction
+    auto load_tile = [&](uint32_t tile, v4i(&w)[SEGS]) {
+        const uint32_t row = tile * 16 + l16;
+        const uint32_t nrows = tile < tile_end ? p.N : 0u;
+        const uint32_t base = TILED ? (tile >> 1) * 32u * p.K + (g >> 1) * 1024u + ((g & 1u) * 32u + l16 + (tile & 1u) * 16u) * 16u
+                                    : row * p.K;
+#pragma unroll
+        for (int u = 0; u < SEGS; ++u) {
+            const uint32_t off = TILED ? base + (wave * SEGS + u) * 2048u : base + koff[u];
+            w[u] = __builtin_bit_cast(v4i, buf_load16(rW, (row < nrows && koff[u] != kOobOffset) ? off : kOobOffset, 0));
+        }
+    };
+    // loads in the order their data is needed: activations, the first tile's weights, the finishing threads' row
+    // parameters
+    v4i x[MT][SEGS];
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int u = 0; u < SEGS; ++u)
+            x[t][u] = __builtin_bit_cast(v4i, buf_load16(rX, koff[u] != kOobOffset ? (t * 16 + l16) * p.K + koff[u] : kOobOffset, 0));
+    v4i w0[SEGS], w1[SEGS];
+    load_tile(tile0, w0);
+
+    // thread (mt = tid / 64, lane) finishes C[mt*16 + l16][tile*16 + 4*g + (0..3)]
+    const bool finisher = tid < MT * 64;
+    const uint32_t m = wave * 16 + l16;
+    float sr = 0.f, zr = 0.f;
+    if (FUSED && finisher) {
+        const uint32_t mm = min(m, p.M - 1);
+        sr = p.epi.s_row[mm], zr = p.epi.z_row[mm];
+    }
+    const void *outp = FUSED ? (const void *)p.y : (const void *)p.C;
+    const bool vec_all = p.N % 4 == 0 && reinterpret_cast<uintptr_t>(outp) % 16 == 0;
+
+    auto compute_tile = [&](uint32_t tile, const v4i(&w)[SEGS], uint32_t buf) {
+        const uint32_t n = tile * 16 + g * 4;
+        float sc[4], zc[4], bs[4];
+        if (FUSED && finisher) {  // requested now, used after the matrix work and the barrier
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const uint32_t nn = min(n + r, p.N - 1);
+                sc[r] = p.epi.s_col[nn];
+                zc[r] = p.epi.z_col[nn];
+                bs[r] = BIAS ? p.epi.bias[nn] : 0.f;
+            }
+        }
+        v4i acc[MT];
+#pragma unroll
+        for (int t = 0; t < MT; ++t) acc[t] = v4i{0, 0, 0, 0};
+#pragma unroll
+        for (int u = 0; u < SEGS; ++u)
+#pragma unroll
+            for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[u], x[t][u], acc[t], 0, 0, 0);
+#pragma unroll
+        for (int t = 0; t < MT; ++t) part[buf][t][wave][lane] = acc[t];
+        __syncthreads();
+        if (finisher) {
+            v4i sum = part[buf][wave][0][lane];
+#pragma unroll
+            for (int w2 = 1; w2 < WAVES; ++w2) {
+                const v4i o = part[buf][wave][w2][lane];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) sum[r] += o[r];
+            }
+            if (m < p.M && n < p.N) {
+                const bool vec_ok = vec_all && n + 3 < p.N;
+                if (FUSED) {
+                    v4f32 v;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        float o = dequant_hprec_one(sum[r], sr, zr, sc[r], zc[r]);
+                        if (BIAS) o = o + bs[r];
+                        v[r] = o;
+                    }
+                    float *dst = p.y + (uint64_t)m * p.N + n;
+                    if (vec_ok) {
+                        *reinterpret_cast<v4f32 *>(dst) = v;
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            if (n + r < p.N) dst[r] = v[r];
+                    }
+                } else {
+                    int32_t *dst = p.C + (uint64_t)m * p.N + n;
+                    if (vec_ok) {
+                        *reinterpret_cast<v4i *>(dst) = sum;
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            if (n + r < p.N) dst[r] = sum[r];
+                    }
+                }
+            }
+        }
+    };
+
+    // the partial-sum buffers alternate with the register sets: one barrier per tile
+    for (uint32_t t = tile0; t < tile_end; t += 2) {
+        load_tile(t + 1, w1);
+        compute_tile(t, w0, 0);
+        load_tile(t + 2, w0);
+        if (t + 1 < tile_end) compute_tile(t + 1, w1, 1);
+    }
+}
+
+// shapes the decode kernel takes: up to 64 rows of at most 4096 elements (the activation fragments of more would
+// not fit in registers next to two sets of weights; with 8192 it measured slower than the skinny kernel: 11.9
+// against 10.5 us at 16 x 4096 x 8192), the weight tensor within 32-bit offsets; above 32 rows only up to 1024
+// column tiles (64 rows, N = 28672: the 64-row tiles of the GEMM kernel take 27 us, this kernel 33).  Measured
+// on the tiled copy, K = 4096, against the skinny kernel (64 rows: the GEMM kernel): N = 4096 M16 6.5 against
+// 6.6 us, M32 7.7 against 8.9, M64 11.8 against 22.3; N = 11008 M16 11.1 against 14.7, M32 12.3 against 21.6, M64
+// 17.3 against 24.9; N = 28672 M32 26.6 against 47.5; on the row-major weight it is 5-15 % slower than on the copy.
+inline bool decode8_takes(uint32_t M, uint32_t N, uint32_t K)
+{
+    return M <= 64 && K <= 4096 && (M <= 32 || (N + 15) / 16 <= 1024) && ((uint64_t)N + 32) * K < 0xFFFFFF00ull;
+}
+
+template <bool FUSED, bool BIAS, bool TILED>
+static void launch_decode8(Gemm8Params &p, hipStream_t stream)
+{
+    const uint32_t ntiles = (p.N + 15) / 16;
+    p.tiles_n = (ntiles + 255) / 256;  // column tiles per workgroup: one round of at most 256 workgroups
+    const dim3 grid((ntiles + p.tiles_n - 1) / p.tiles_n);
+    const uint32_t mt = (p.M + 15) / 16;
+#define DUQ_DEC8(S, T) hipLaunchKernelGGL((gemm_s8_decode_kernel<S, T, FUSED, BIAS, TILED>), grid, dim3(512), 0, stream, p)
+    if (p.K > 2048) {
+        if (mt == 1) DUQ_DEC8(8, 1);
+        else if (mt == 2) DUQ_DEC8(8, 2);
+        else if (mt == 3) DUQ_DEC8(8, 3);
+        else DUQ_DEC8(8, 4);
+    } else {
+        if (mt == 1) DUQ_DEC8(4, 1);
+        else if (mt == 2) DUQ_DEC8(4, 2);
+        else if (mt == 3) DUQ_DEC8(4, 3);
+        else DUQ_DEC8(4, 4);
+    }
+#undef DUQ_DEC8
+}
+
+// ---------------------------------------------------------------------------------
 // rows kernel: M <= 4 activation rows on the row-major weight, rows of up to XS KB
 // ---------------------------------------------------------------------------------
 // The 4-bit rows kernel's shape for int8 (src/kernels/gemm.cu:46-81 at M <= 4): v_dot4_i32_i8 straight on the
@@ -696,6 +868,10 @@ static void launch_gemm8_variant(Gemm8Params &p, hipStream_t stream)
         if (p.M == 1) launch_rows8<1, FUSED, BIAS>(p, stream);
         else if (p.M == 2) launch_rows8<2, FUSED, BIAS>(p, stream);
         else launch_rows8<4, FUSED, BIAS>(p, stream);
+        return;
+    }
+    if (decode8_takes(p.M, p.N, p.K)) {
+        launch_decode8<FUSED, BIAS, TILED>(p, stream);
         return;
     }
     if (p.M <= 32) {

@@ -370,7 +370,10 @@ def test_gpu_fused_quantizer_8bit_matches_torch_ops(dev, hip):
 
 
 GEMM_SHAPES = [(1, 1, 32), (5, 7, 64), (32, 64, 96), (16, 16, 32), (9, 40, 96), (17, 250, 416), (32, 1030, 1056),
-               (3, 48, 8192), (16, 4096, 4096), (31, 300, 4128),   # skinny kernel: K split over four wavefronts
+               (3, 48, 8192), (16, 4096, 8192), (31, 300, 4128),   # skinny kernel: K split over four wavefronts
+               # decode kernel: up to 64 rows of at most 4096 elements, one to several column tiles per workgroup
+               (16, 4096, 4096), (5, 4100, 4096), (16, 11008, 2048), (33, 5000, 1056), (48, 300, 4096), (64, 4099, 4096),
+               (20, 8200, 96), (64, 16384, 32), (64, 17000, 64), (32, 17000, 64),
                (1, 4096, 4096), (2, 300, 8192), (4, 1000, 4096), (2, 35, 2080), (4, 17, 1056), (1, 5, 8192), (3, 21, 32),   # rows kernel
  (33, 250, 128), (100, 256, 160), (128, 260, 416),
                (129, 512, 1024), (300, 100, 32), (64, 1024, 4096), (65, 300, 224),
@@ -409,7 +412,8 @@ def test_gpu_asym_dequant_hprec(dev, hip, rows, cols):
     assert got.dtype == F32 and np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
-FWD_SHAPES = [(1, 4096, 4096), (2, 250, 5120), (3, 33, 1056), (512, 4096, 128), (300, 3102, 288), (1, 16, 32), (7, 33, 64), (16, 48, 96), (17, 250, 416), (32, 1030, 1056), (4, 4096, 4096), (40, 250, 160), (128, 512, 1024), (130, 1030, 416), (1024, 3072, 256),
+FWD_SHAPES = [(5, 4100, 4096), (16, 11008, 1056), (33, 5000, 416), (64, 4099, 2080), (48, 260, 4096), (17, 40, 32),
+              (1, 4096, 4096), (2, 250, 5120), (3, 33, 1056), (512, 4096, 128), (300, 3102, 288), (1, 16, 32), (7, 33, 64), (16, 48, 96), (17, 250, 416), (32, 1030, 1056), (4, 4096, 4096), (40, 250, 160), (128, 512, 1024), (130, 1030, 416), (1024, 3072, 256),
               (1000, 3102, 288)]
 
 
