@@ -276,7 +276,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DecodeParams p
 // and registers (MT * SEGS * 4 for the packed activations), not weight traffic.  Nibble -> byte as in the
 // GEMM kernels: (w & 0xF0F0F0F0) is the four odd-k nibbles times 16, ((w << 4) & 0xF0F0F0F0) the even ones;
 // every product is 256 * a * b and one arithmetic shift recovers the sum.
-template <int WAVES, int SEGS, int EPI, int MT = 1>
+template <int WAVES, int SEGS, int EPI, int MT = 1, bool DB = true>
 __global__ __launch_bounds__(WAVES * 64) void gemm_s4_decode_kernel(DecodeParams p)
 {
     constexpr int MODE = EPI < 0 ? 0 : EPI;
@@ -319,7 +319,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_s4_decode_kernel(DecodeParams
 #pragma unroll
         for (int u = 0; u < SEGS; ++u)
             xp[t][u] = buf_load16(rX, koff[u] != kOobOffset ? (t * 16 + l16) * kbytes + koff[u] : kOobOffset, 0);
-    v4u w0[SEGS], w1[SEGS];
+    v4u w0[SEGS], w1[DB ? SEGS : 1];
     load_tile(tile0, w0);
 
     // threads finish one output per row tile they own: element er of MFMA lane src_lane; the 256-thread group
@@ -357,11 +357,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_s4_decode_kernel(DecodeParams
             }
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
-                v4u xe, xo;
+                v4u xe, xo, xv = xp[t][u];
+                // many fragments: keep their expansion here (hoisted out of the tile loop it would double the
+                // registers they take)
+                if (MT * SEGS > 16) asm volatile("" : "+v"(xv));
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
-                    xe[q] = (xp[t][u][q] << 4) & kNibbleMaskD;
-                    xo[q] = xp[t][u][q] & kNibbleMaskD;
+                    xe[q] = (xv[q] << 4) & kNibbleMaskD;
+                    xo[q] = xv[q] & kNibbleMaskD;
                 }
                 acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i, we), __builtin_bit_cast(v4i, xe), acc[t], 0, 0, 0);
                 acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i, wo), __builtin_bit_cast(v4i, xo), acc[t], 0, 0, 0);
@@ -391,12 +394,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_s4_decode_kernel(DecodeParams
     };
 
     // two register sets alternate so that one tile's loads are in flight during the other's MFMAs; the
-    // partial-sum buffers alternate too: one barrier per tile
-    for (uint32_t t = tile0; t < tile_end; t += 2) {
-        load_tile(t + 1, w1);
-        compute_tile(t, w0, 0);
-        load_tile(t + 2, w0);
-        if (t + 1 < tile_end) compute_tile(t + 1, w1, 1);
+    // partial-sum buffers alternate too: one barrier per tile.  (DB = false: one set, for the long rows whose
+    // fragments leave no room for a second; their layers have at most 256 column tiles, one per workgroup.)
+    if constexpr (DB) {
+        for (uint32_t t = tile0; t < tile_end; t += 2) {
+            load_tile(t + 1, w1);
+            compute_tile(t, w0, 0);
+            load_tile(t + 2, w0);
+            if (t + 1 < tile_end) compute_tile(t + 1, w1, 1);
+        }
+    } else {
+        for (uint32_t t = tile0; t < tile_end; ++t) {
+            if (t != tile0) load_tile(t, w0);
+            compute_tile(t, w0, (t - tile0) & 1u);
+        }
     }
 }
 
@@ -454,12 +465,12 @@ void launch_rows_xs(DecodeParams &p, int epi, hipStream_t stream)
     else launch_rows_mode<MR, 8, FUSEQ>(p, epi, stream);
 }
 
-template <int WAVES, int SEGS, int MT = 1>
+template <int WAVES, int SEGS, int MT = 1, bool DB = true>
 void launch_mfma_mode(const DecodeParams &p, int epi, hipStream_t stream)
 {
     const uint32_t ntiles = (p.N + 15) / 16;
     const dim3 grid((ntiles + p.tiles_per_wg - 1) / p.tiles_per_wg);
-#define DUQ_DEC(E) hipLaunchKernelGGL((gemm_s4_decode_kernel<WAVES, SEGS, E, MT>), grid, dim3(WAVES * 64), 0, stream, p)
+#define DUQ_DEC(E) hipLaunchKernelGGL((gemm_s4_decode_kernel<WAVES, SEGS, E, MT, DB>), grid, dim3(WAVES * 64), 0, stream, p)
     switch (epi) {
     case -1: DUQ_DEC(-1); break;
     case 0: DUQ_DEC(0); break;
@@ -486,18 +497,23 @@ void launch_decode_any(DecodeParams &p, int epi, hipStream_t stream)
         p.tiles_per_wg = decode_tiles_per_workgroup(ntiles);
         constexpr int W = DUQ_DEC_WAVES, S = 32 / W;  // 64-byte segments per wavefront for 2 KB of a row
         const uint32_t mt = (p.M + 15) / 16;  // 2..4 only with rows of at most 8192 elements (select_gemm_kernel)
-#define DUQ_DEC_MT(T)                                                     \
-    do {                                                                  \
-        if (kbytes <= 2048) launch_mfma_mode<W, S, T>(p, epi, stream);    \
-        else launch_mfma_mode<W, 2 * S, T>(p, epi, stream);               \
-    } while (0)
-        // (three and four row tiles of rows longer than 4096 elements would spill registers: not instantiated)
-        if (mt == 4 && kbytes <= 2048) launch_mfma_mode<W, S, 4>(p, epi, stream);
-        else if (mt == 3 && kbytes <= 2048) launch_mfma_mode<W, S, 3>(p, epi, stream);
-        else if (mt == 2) DUQ_DEC_MT(2);
-        else if (kbytes <= 4096) DUQ_DEC_MT(1);
-        else launch_mfma_mode<8, 12>(p, epi, stream);
-#undef DUQ_DEC_MT
+        // rows of up to 4096 / 8192 / 12288 elements: S, 2 S, 12 segments per wavefront; the row tiles whose
+        // fragments fit in registers next to two sets of weights (select_gemm_kernel admits no others)
+        if (kbytes <= 2048) {
+            if (mt == 1) launch_mfma_mode<W, S, 1>(p, epi, stream);
+            else if (mt == 2) launch_mfma_mode<W, S, 2>(p, epi, stream);
+            else if (mt == 3) launch_mfma_mode<W, S, 3>(p, epi, stream);
+            else launch_mfma_mode<W, S, 4>(p, epi, stream);
+        } else if (kbytes <= 4096) {
+            if (mt == 1) launch_mfma_mode<W, 2 * S, 1>(p, epi, stream);
+            else if (mt == 2) launch_mfma_mode<W, 2 * S, 2>(p, epi, stream);
+            else if (mt == 3) launch_mfma_mode<W, 2 * S, 3>(p, epi, stream);
+            else launch_mfma_mode<W, 2 * S, 4>(p, epi, stream);
+        } else {
+            if (mt == 1) launch_mfma_mode<8, 12, 1>(p, epi, stream);
+            else if (mt == 2) launch_mfma_mode<8, 12, 2, false>(p, epi, stream);
+            else launch_mfma_mode<8, 12, 3, false>(p, epi, stream);
+        }
     }
 }
 

@@ -883,15 +883,21 @@ int select_gemm_kernel(uint32_t M, uint32_t N, uint32_t K)
     const uint64_t wbytes = (uint64_t)N * (K / 2);
     const bool small_offsets = wbytes < 0xFFFFFF00ull && K > 0;
     // decode.  Rows kernel for up to four rows (8 KB of every weight row per wavefront); above, the MFMA decode
-    // kernel (6 KB per row over eight wavefronts; up to 64 rows of at most 4096 elements and 32 of at most 8192 as
-    // two to four row tiles against the same weight fragments), except 9..16 rows on very wide layers, where the
-    // skinny kernel's whole-line weight loads measure 5 % faster (N = 28672, K = 4096)
+    // kernel (6 KB per row over eight wavefronts), with two to four row tiles against the same weight fragments
+    // for 17..64 rows as far as the fragments fit in registers (64 rows of at most 8192 elements, 48 of at most
+    // 12288).  Two exceptions, both measured: 9..16 rows on very wide layers run the skinny kernel (whole-line
+    // weight loads, 5 % faster at N = 28672, K = 4096), and the long-row forms (more than 32 rows of more than 4096
+    // elements, any of more than 8192) need 192 column tiles: on narrower layers the ring kernel, which splits K
+    // over workgroups, is ahead (48 x 1024 x 8192: 7.9 against 10.2 us; 48 x 3072 x 12288: 20.6 against 14.1).
     if (M <= 4 && K <= 16384 && small_offsets) return kKernelDecodeRows;
     if (M <= 16 && small_offsets) {
         if (M > 8 && (N + 15) / 16 >= 1536 && K <= 4096) return kKernelSkinny;
         if (K <= 12288) return kKernelDecodeMfma;
     }
-    if (M <= 64 && small_offsets && (K <= 4096 || (K <= 8192 && M <= 32))) return kKernelDecodeMfma;
+    if (M <= 64 && small_offsets) {
+        if (K <= 4096 || (K <= 8192 && M <= 32)) return kKernelDecodeMfma;
+        if ((N + 15) / 16 >= 192 && (K <= 8192 || (K <= 12288 && M <= 48))) return kKernelDecodeMfma;
+    }
     const uint32_t xstride = ((K / 2 + 127) / 128) * 128;
     // dot kernel: up to four rows too long for the decode kernels
     if (M <= 4 && small_offsets && 4 * xstride <= 60 * 1024) return kKernelDot;

@@ -69,7 +69,7 @@ int launch_dual_rowsum_dequant(const DualRowsumParams &p, hipStream_t stream);
 // only, exported as duq_gemm_kernel_for so that the rule can be tested without a GPU).
 enum GemmKernelId {
     kKernelDecodeRows = 1,  // duq_decode.hip, v_dot8_i32_i4, M <= 4
-    kKernelDecodeMfma = 2,  // duq_decode.hip, MFMA, 5 <= M <= 16 (K <= 12288), 17 <= M <= 64 (K <= 4096; 32 rows: 8192)
+    kKernelDecodeMfma = 2,  // duq_decode.hip, MFMA, 5 <= M <= 16 (K <= 12288), 17 <= M <= 64 (K <= 8192; 48 rows: 12288)
     kKernelDot = 3,         // duq_gemm.hip, M <= 4 with rows longer than 16384 elements
     kKernelRing = 4,        // duq_gemm.hip, 17 <= M <= 256 on narrow problems the decode kernel does not take
     kKernelSkinny = 5,      // duq_gemm.hip, 9 <= M <= 16 with 1536 or more column tiles, K <= 4096

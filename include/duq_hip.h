@@ -208,8 +208,8 @@ int duq_batch_linear4bit_forward(int32_t mode, const uint8_t *xq, const duq_half
                                  duq_stream_t stream);
 
 /* Which kernel family duq_matmul_host_4bit / duq_linear4bit_forward run for a shape (no GPU work; for tests
- * and tuning): 1 decode rows kernel (M <= 4), 2 decode MFMA kernel (M <= 16; up to 64 rows of at most 4096
- * elements, 32 of at most 8192), 3 dot kernel (M <= 4, rows longer than 16384 elements), 4 ring kernel, 5 skinny
+ * and tuning): 1 decode rows kernel (M <= 4), 2 decode MFMA kernel (M <= 16; up to 64 rows of at most 8192
+ * elements, 48 of at most 12288), 3 dot kernel (M <= 4, rows longer than 16384 elements), 4 ring kernel, 5 skinny
  * kernel (9 <= M <= 16, very wide problems), 6 stream kernel (prefill), 7 tile kernel.  Families 1-5 address the weight tensor with 32-bit byte offsets and are only picked while
  * N * K / 2 < 2^32 - 256; larger tensors run the stream / tile kernels, whose bases are 64-bit per tile.  No
  * counterpart in the reference (CUTLASS picks its own tile, src/kernels/gemm.cu:17-42). */

@@ -37,8 +37,10 @@ SHAPES = [(1, 64, 64), (1, 20, 128), (2, 37, 4096), (3, 100, 2048), (4, 4096, 40
           # 8192), one to several column tiles per workgroup, tiles that end inside M and N
           (17, 4096, 4096), (32, 300, 4096), (33, 4099, 2048), (48, 1000, 4096), (64, 11008, 4096), (50, 72, 64),
           (64, 40, 128), (20, 520, 8192), (32, 4100, 8192), (29, 9000, 4160), (64, 5000, 1024),
-          # and their neighbours on the ring kernel: more than 32 rows of more than 4096 elements
-          (33, 300, 8192), (64, 130, 4160),
+          # the long-row forms (three and four row tiles of up to 8192 elements, two and three of up to 12288: from
+          # 192 column tiles on) and their neighbours on the ring kernel
+          (33, 3072, 8192), (64, 3100, 4160), (48, 4096, 11008), (20, 3080, 12288), (40, 6200, 8256),
+          (33, 300, 8192), (64, 130, 4160), (49, 3072, 11008),
           # 9..16 rows on 1536 or more column tiles: the skinny kernel
           (9, 24600, 64), (16, 28672, 256),
           # rows longer than 16384 elements: the dot kernel

@@ -241,7 +241,8 @@ def test_gemm_kernel_selection_keeps_32_bit_offsets_in_range():
     assert [f(m, 4096, 4096) for m in (1, 4, 5, 16, 17, 64, 65, 2048)] == [1, 1, 2, 2, 2, 2, 4, 6]
     assert f(16, 11008, 4096) == 2 and f(16, 4096, 11008) == 2 and f(16, 28672, 8192) == 2
     assert f(16, 28672, 4096) == 5 and f(8, 28672, 4096) == 2 and f(64, 28672, 4096) == 2
-    assert f(32, 4096, 8192) == 2 and f(33, 4096, 8192) == 4 and f(17, 4096, 11008) != 2
+    assert f(32, 4096, 8192) == 2 and f(33, 4096, 8192) == 2 and f(17, 4096, 11008) == 2 and f(48, 4096, 12288) == 2
+    assert f(33, 1024, 8192) == 4 and f(32, 1024, 8192) == 2 and f(49, 4096, 11008) != 2 and f(17, 2048, 11008) == 4
     assert f(1, 28672, 8192) == 1 and f(1, 8192, 28672) == 3 and f(16, 8192, 28672) == 7
     assert f(16, 64, 16384) == 4 and f(4, 64, 16384) == 1 and f(16, 4096, 12288) == 2
     assert f(16, 1 << 22, 4096) == 7 and f(1, 1 << 22, 4096) == 7 and f(64, 1 << 22, 4096) in (6, 7)
