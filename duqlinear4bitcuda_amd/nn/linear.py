@@ -38,9 +38,10 @@ def _asym_params(w: torch.Tensor):
 class _Linear4bitBase(torch.nn.Module):
     fused = True
     # 6-bit float matrix path (not in the reference): taken when the layer holds a weight shadow
-    # (enable_fp6) and the input brings one, for more than 64 rows (more than 32 when rows are longer than 4096
-    # elements) and at least fp6_min_tiles output tiles of 64 x 256, or more than 256 rows and 5/8 of that (below,
-    # the integer kernels' smaller tiles and the decode kernels do better; measured crossover on an MI355X)
+    # (enable_fp6) and the input brings one, for more rows than the integer decode kernel takes (64 of up to 8192
+    # elements, 48 of up to 12288, 32 beyond) and at least fp6_min_tiles output tiles of 64 x 256, or more than 256
+    # rows and 5/8 of that (below, the integer kernels' smaller tiles and the decode kernels do better; measured
+    # crossover on an MI355X)
     fp6_min_tiles = 32
     _shadow_key = None
 
@@ -68,7 +69,8 @@ class _Linear4bitBase(torch.nn.Module):
 
     def _fp6_wanted(self, rows):
         tiles = -(-rows // 64) * -(-self.out_features // 256)
-        return self._fp6_ready() and rows > (64 if self.in_features <= 4096 else 32) and \
+        decode_rows = 64 if self.in_features <= 8192 else (48 if self.in_features <= 12288 else 32)
+        return self._fp6_ready() and rows > decode_rows and \
             (tiles >= self.fp6_min_tiles or (rows > 256 and 8 * tiles >= 5 * self.fp6_min_tiles))
 
     def _use_shadow(self, x):

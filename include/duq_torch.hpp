@@ -224,15 +224,15 @@ inline torch::Tensor weight_shadow(const torch::Tensor &weight)
     return out;
 }
 
-// The 6-bit float matrix path is taken when both shadows exist and the problem has more than 64 rows (more than 32
-// when rows are longer than 4096 elements: a shadow row holds 3/4 byte per element) and at least 32 output tiles
-// of 64 x 256 (below, the integer kernels do better); same bits either way.
+// The 6-bit float matrix path is taken when both shadows exist and the problem has more rows than the integer
+// decode kernel takes (64 of up to 8192 elements, 48 of up to 12288, 32 beyond; a shadow row holds 3/4 byte per
+// element) and at least 32 output tiles of 64 x 256 (below, the integer kernels do better); same bits either way.
 inline bool use_shadow(const PackedQuantizedTensor &input, const torch::Tensor &w_shadow, int64_t N)
 {
     if (!input.shadow_x.defined() || !w_shadow.defined()) return false;
     const int64_t rows = input.shadow_x.numel() / input.shadow_x.size(-1);
     const int64_t K = input.shadow_x.size(-1) * 4 / 3;
-    return rows > (K <= 4096 ? 64 : 32) && ((rows + 63) / 64) * ((N + 255) / 256) >= 32;
+    return rows > (K <= 8192 ? 64 : (K <= 12288 ? 48 : 32)) && ((rows + 63) / 64) * ((N + 255) / 256) >= 32;
 }
 
 inline torch::Tensor fused_forward_shadow(int mode, const PackedQuantizedTensor &input, const torch::Tensor &w_shadow,
