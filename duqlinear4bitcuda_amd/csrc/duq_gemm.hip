@@ -270,12 +270,14 @@ constexpr int kCK = 256;         // k elements per chunk (128 packed bytes per r
 constexpr int kXStride = 272;    // LDS bytes per activation row: 256 expanded + 16 pad
 
 
-template <int TM, int EPI, bool BIAS>
+template <int TM, int EPI, bool BIAS, int TN = 2>
 __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
 {
     static_assert(TM == 4 || TM == 2 || TM == 1, "32-row activation tiles per wavefront");
-    constexpr int BM = 32 * TM, BN = 256;
-    constexpr int TN = 2;              // 32x32 tiles per wavefront: BM x 64
+    // TN = 32-column weight tiles per wavefront: tiles of 256 columns (TN = 2), or of 128 with 64 rows (TN = 1):
+    // as many outputs per workgroup as 32 x 256 with a third less operand bytes into the CU
+    static_assert(TN == 2 || (TN == 1 && TM == 2), "column tiles per wavefront");
+    constexpr int BM = 32 * TM, BN = 128 * TN;
     constexpr int S = TM * TN;         // MFMA slots per step
     constexpr int NXP = TM;            // 16-byte activation pieces per thread and chunk
     constexpr uint32_t kBuf = BM * kXStride;
@@ -298,7 +300,7 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
 
     uint32_t woff[TN];
 #pragma unroll
-    for (int t = 0; t < TN; ++t) woff[t] = (wave * 64 + t * 32 + l32) * kbytes + h * 16;
+    for (int t = 0; t < TN; ++t) woff[t] = (wave * (32 * TN) + t * 32 + l32) * kbytes + h * 16;
     uint32_t xoff[NXP], xlds[NXP];
     const uint32_t xq = tid & 7u;  // which 16-byte piece of the 128-byte row segment
 #pragma unroll
@@ -340,7 +342,7 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
             const bool okw = !G || (koff1 + i * 32 + h * 16 < kbytes);
 #pragma unroll
             for (int slot = 0; slot < S; ++slot) {
-                const int b = slot >> 1, t = slot & 1;
+                const int b = slot / TN, t = slot % TN;
                 asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0"
                              : "+a"(acc[t][b])
                              : "v"(wexp[i & 1][par][t]), "v"(fx[step & 1][b]));
@@ -357,12 +359,13 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
                     xreg[slot] = buf_load16(rX, okx ? xoff[slot] : kOobOffset, koff2);
                 // expand the next weight piece of tile `par`: its four words over the last four slots (or
                 // two / one per slot when a step has fewer than four slots)
-                {
+                if (par < TN) {
                     const int np = (i + 1) & 3;  // pieces 1, 2, 3 of this chunk, then piece 0 of the next
 #pragma unroll
                     for (int w = 0; w < 4; ++w)
                         if ((S >= 4 ? S - 4 + w : w * S / 4) == slot)
-                            expand_word(wreg[par][np], wexp[(i + 1) & 1][0][par], wexp[(i + 1) & 1][1][par], w);
+                            expand_word(wreg[par < TN ? par : 0][np], wexp[(i + 1) & 1][0][par < TN ? par : 0],
+                                        wexp[(i + 1) & 1][1][par < TN ? par : 0], w);
                 }
                 if (step >= 8 - NXP) {  // activations two chunks ahead -> third LDS buffer, one piece per step
 #pragma unroll
@@ -901,6 +904,12 @@ int select_gemm_kernel(uint32_t M, uint32_t N, uint32_t K)
     const uint32_t xstride = ((K / 2 + 127) / 128) * 128;
     // dot kernel: up to four rows too long for the decode kernels
     if (M <= 4 && small_offsets && 4 * xstride <= 60 * 1024) return kKernelDot;
+    // more than 64 rows whose 64 x 128 tiles make one round of 64..256 workgroups: the stream kernel on those tiles
+    // (measured against the ring kernel, N = 4096: 128 x 4096 11.9 against 14.6 us, 192 x 4096 12.1 against 18.3,
+    // 128 x 11008 (K) 25.1 against 42.2; with fewer tiles the ring kernel, which splits K over workgroups, is far
+    // ahead: 200 x 520 x 8192 8.2 against 28.8 us)
+    const uint32_t narrow_tiles = ((M + 63) / 64) * ((N + 127) / 128);
+    const bool narrow_round = M > 64 && narrow_tiles >= 64 && narrow_tiles <= 256;
     {
         // ring kernel: 17..256 rows in groups whose packed activations fit in LDS (a few groups only, or a
         // problem too narrow to fill the chip with stream-kernel tiles)
@@ -914,10 +923,10 @@ int select_gemm_kernel(uint32_t M, uint32_t N, uint32_t K)
         const bool few_groups = row_groups <= 2 || (row_groups <= 6 && tiles32 < 64) || tiles32 < 48;
         const bool mid_rows = M > 16 && M <= 256 && few_groups && !(row_groups > 1 && tiles32 >= 128);
         const bool long_rows = M <= 16 && K > 8192;  // 5..16 rows of 12289..16384 elements
-        if ((long_rows || mid_rows) && K <= 16384 && small_offsets) return kKernelRing;
+        if ((long_rows || mid_rows) && K <= 16384 && small_offsets && !narrow_round) return kKernelRing;
     }
     auto tiles = [&](uint32_t bm, uint32_t bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-    if (M > 32 && tiles(32, 256) >= 32) return kKernelStream;
+    if (narrow_round || (M > 32 && tiles(32, 256) >= 32)) return kKernelStream;
     return kKernelTile;
 }
 
@@ -985,25 +994,29 @@ static void launch_epi(GemmParams &p, hipStream_t stream, uint32_t batch = 1)
 #undef DUQ_RING
         return;
     }
-    // Stream kernel with 128, 64 or 32 activation rows per workgroup: whole rounds of 256 workgroups
-    // (one per CU) cost about nchunks * c + f microseconds each, c and f measured per tile height;
-    // the cheapest wins.  Small problems (few column tiles) stay on the tile kernels.
+    // Stream kernel with 128, 64 or 32 activation rows x 256 columns per workgroup, or 64 x 128: whole rounds of
+    // 256 workgroups (one per CU) cost about nchunks * c + f microseconds each, c and f measured per tile shape;
+    // the cheapest wins.  A 64 x 128 tile has the outputs of a 32 x 256 one with a third less operand bytes into the
+    // CU (192 rows of K / 2 bytes against 288; the L2 -> CU path is what bounds these tiles): 512 x 4096 x 4096 13.1
+    // against 19.8 us, 512 x 4096 x 11008 (K) 34.1 against 52.  Small problems (few column tiles) stay on the tile
+    // kernels.
     auto tiles = [&](uint32_t bm, uint32_t bn) { return ((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn) * batch; };
     int best_tm = 0;
+    bool half_width = false;  // 64 x 128 tiles
     if (kernel == kKernelStream) {
         const float nch = (float)((p.K + kCK - 1) / kCK);
-        const float c_us[3] = {1.5f, 1.0f, 0.8f}, f_us[3] = {9.f, 7.f, 6.f};
+        const float c_us[4] = {1.5f, 1.0f, 0.8f, 0.78f}, f_us[4] = {9.f, 7.f, 6.f, 1.f};
         float best = 0.f;
-        for (int k = 0; k < 3; ++k) {
-            const uint32_t t = tiles(128u >> k, 256);
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t t = k < 3 ? tiles(128u >> k, 256) : tiles(64, 128);
             const float cost = (float)((t + 255) / 256) * (nch * c_us[k] + f_us[k]);
             if (best_tm == 0 || cost < best) {
                 best = cost;
-                best_tm = 4 >> k;
+                best_tm = k < 3 ? 4 >> k : 2;
+                half_width = k == 3;
             }
         }
     }
-    bool narrow = false;
     if (best_tm && p.K <= 256) {
         // rows of at most 256 elements: one chunk, the launch is its output stores: the short-row kernel with 64-row
         // tiles (measured on 32 products of 2048 x 2048 x 128: 86 us against 95 us on the stream kernel's 64-row tiles)
@@ -1013,12 +1026,12 @@ static void launch_epi(GemmParams &p, hipStream_t stream, uint32_t batch = 1)
                            stream, p);
         return;
     }
-    if (batch > 1 && best_tm) {
-        // measured at attention-like batches (32 problems): at most 128 columns fill half of a 256-wide tile, the
-        // 128 x 128 tile kernel is 15 % faster there (2048 x 128 x 2048: 32 against 37 us)
-        if (p.N <= 128 && p.M > 64) { best_tm = 0; narrow = true; }
-    }
-    if (best_tm) {
+    if (best_tm && half_width) {
+        p.tiles_m = (p.M + 63) / 64;
+        p.tiles_n = (p.N + 127) / 128;
+        hipLaunchKernelGGL((gemm_s4_stream_kernel<2, EPI, BIAS, 1>), dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(256), 0,
+                           stream, p);
+    } else if (best_tm) {
         p.tiles_m = (p.M + 32 * best_tm - 1) / (32 * best_tm);
         p.tiles_n = (p.N + 255) / 256;
         const dim3 grid(p.tiles_m * p.tiles_n, 1, batch);
@@ -1028,12 +1041,12 @@ static void launch_epi(GemmParams &p, hipStream_t stream, uint32_t batch = 1)
             hipLaunchKernelGGL((gemm_s4_stream_kernel<2, EPI, BIAS>), grid, dim3(256), 0, stream, p);
         else
             hipLaunchKernelGGL((gemm_s4_stream_kernel<1, EPI, BIAS>), grid, dim3(256), 0, stream, p);
-    } else if (!narrow && tiles(128, 256) >= 256 && p.M > 64) {
+    } else if (tiles(128, 256) >= 256 && p.M > 64) {
         p.tiles_m = (p.M + 127) / 128;
         p.tiles_n = (p.N + 255) / 256;
         hipLaunchKernelGGL((gemm_s4_tile_kernel<128, 256, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(256), 0,
                            stream, p);
-    } else if (narrow || (tiles(128, 128) >= 256 && p.M > 64)) {
+    } else if (tiles(128, 128) >= 256 && p.M > 64) {
         p.tiles_m = (p.M + 127) / 128;
         p.tiles_n = (p.N + 127) / 128;
         hipLaunchKernelGGL((gemm_s4_tile_kernel<128, 128, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(256), 0,

@@ -238,7 +238,8 @@ def test_gemm_kernel_selection_keeps_32_bit_offsets_in_range():
                 if int(N) * kb >= limit:
                     assert k not in small, (M, N, K, k)
     # buckets at the benchmark shapes
-    assert [f(m, 4096, 4096) for m in (1, 4, 5, 16, 17, 64, 65, 2048)] == [1, 1, 2, 2, 2, 2, 4, 6]
+    assert [f(m, 4096, 4096) for m in (1, 4, 5, 16, 17, 64, 65, 2048)] == [1, 1, 2, 2, 2, 2, 6, 6]
+    assert f(100, 1000, 4096) == 4 and f(200, 520, 8192) == 4 and f(128, 11008, 4096) == 6 and f(128, 28672, 8192) == 6
     assert f(16, 11008, 4096) == 2 and f(16, 4096, 11008) == 2 and f(16, 28672, 8192) == 2
     assert f(16, 28672, 4096) == 5 and f(8, 28672, 4096) == 2 and f(64, 28672, 4096) == 2
     assert f(32, 4096, 8192) == 2 and f(33, 4096, 8192) == 2 and f(17, 4096, 11008) == 2 and f(48, 4096, 12288) == 2
