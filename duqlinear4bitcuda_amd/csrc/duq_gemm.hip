@@ -276,7 +276,7 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
     static_assert(TM == 4 || TM == 2 || TM == 1, "32-row activation tiles per wavefront");
     // TN = 32-column weight tiles per wavefront: tiles of 256 columns (TN = 2), or of 128 with 64 rows (TN = 1):
     // as many outputs per workgroup as 32 x 256 with a third less operand bytes into the CU
-    static_assert(TN == 2 || (TN == 1 && TM == 2), "column tiles per wavefront");
+    static_assert(TN == 2 || (TN == 1 && TM >= 2), "column tiles per wavefront");
     constexpr int BM = 32 * TM, BN = 128 * TN;
     constexpr int S = TM * TN;         // MFMA slots per step
     constexpr int NXP = TM;            // 16-byte activation pieces per thread and chunk
@@ -994,26 +994,30 @@ static void launch_epi(GemmParams &p, hipStream_t stream, uint32_t batch = 1)
 #undef DUQ_RING
         return;
     }
-    // Stream kernel with 128, 64 or 32 activation rows x 256 columns per workgroup, or 64 x 128: whole rounds of
-    // 256 workgroups (one per CU) cost about nchunks * c + f microseconds each, c and f measured per tile shape;
-    // the cheapest wins.  A 64 x 128 tile has the outputs of a 32 x 256 one with a third less operand bytes into the
-    // CU (192 rows of K / 2 bytes against 288; the L2 -> CU path is what bounds these tiles): 512 x 4096 x 4096 13.1
-    // against 19.8 us, 512 x 4096 x 11008 (K) 34.1 against 52.  Small problems (few column tiles) stay on the tile
-    // kernels.
+    // Stream kernel with 128, 64 or 32 activation rows x 256 columns per workgroup, or 128 or 64 x 128: whole rounds
+    // of 256 workgroups (one per CU) cost about nchunks * c + f microseconds each, c and f measured per tile shape;
+    // the cheapest wins.  The L2 -> CU path bounds these tiles, so what counts is operand rows per output: a
+    // 64 x 128 tile has the outputs of a 32 x 256 one with a third less operand bytes into the CU (192 rows of K / 2
+    // bytes against 288): 512 x 4096 x 4096 13.1 against 19.8 us, 512 x 4096 x 11008 (K) 34.1 against 52; a 128 x 128
+    // tile those of a 64 x 256 one with a fifth less (256 against 320): 1024 x 4096 x 4096 21.5 against 26.1 us on one
+    // box, 768 rows 18.9 against 22.4, 1024 x 4096 x 11008 (K) 50.5 against 58.5.  Small problems (few column tiles)
+    // stay on the tile kernels.
     auto tiles = [&](uint32_t bm, uint32_t bn) { return ((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn) * batch; };
     int best_tm = 0;
-    bool half_width = false;  // 64 x 128 tiles
+    bool half_width = false;  // 128-column tiles
     if (kernel == kKernelStream) {
         const float nch = (float)((p.K + kCK - 1) / kCK);
-        const float c_us[4] = {1.5f, 1.0f, 0.8f, 0.78f}, f_us[4] = {9.f, 7.f, 6.f, 1.f};
+        const int tm[5] = {4, 2, 1, 2, 4};
+        const bool hw[5] = {false, false, false, true, true};
+        const float c_us[5] = {1.5f, 1.0f, 0.8f, 0.78f, 0.9f}, f_us[5] = {9.f, 7.f, 6.f, 1.f, 4.5f};
         float best = 0.f;
-        for (int k = 0; k < 4; ++k) {
-            const uint32_t t = k < 3 ? tiles(128u >> k, 256) : tiles(64, 128);
+        for (int k = 0; k < 5; ++k) {
+            const uint32_t t = tiles(32u * tm[k], hw[k] ? 128 : 256);
             const float cost = (float)((t + 255) / 256) * (nch * c_us[k] + f_us[k]);
             if (best_tm == 0 || cost < best) {
                 best = cost;
-                best_tm = k < 3 ? 4 >> k : 2;
-                half_width = k == 3;
+                best_tm = tm[k];
+                half_width = hw[k];
             }
         }
     }
@@ -1027,10 +1031,13 @@ static void launch_epi(GemmParams &p, hipStream_t stream, uint32_t batch = 1)
         return;
     }
     if (best_tm && half_width) {
-        p.tiles_m = (p.M + 63) / 64;
+        p.tiles_m = (p.M + 32 * best_tm - 1) / (32 * best_tm);
         p.tiles_n = (p.N + 127) / 128;
-        hipLaunchKernelGGL((gemm_s4_stream_kernel<2, EPI, BIAS, 1>), dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(256), 0,
-                           stream, p);
+        const dim3 grid(p.tiles_m * p.tiles_n, 1, batch);
+        if (best_tm == 4)
+            hipLaunchKernelGGL((gemm_s4_stream_kernel<4, EPI, BIAS, 1>), grid, dim3(256), 0, stream, p);
+        else
+            hipLaunchKernelGGL((gemm_s4_stream_kernel<2, EPI, BIAS, 1>), grid, dim3(256), 0, stream, p);
     } else if (best_tm) {
         p.tiles_m = (p.M + 32 * best_tm - 1) / (32 * best_tm);
         p.tiles_n = (p.N + 255) / 256;

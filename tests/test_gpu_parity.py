@@ -172,6 +172,8 @@ def _rand_packed(rng, rows, K):
     (100, 1000, 4096), (200, 520, 8192), (90, 300, 11008), (256, 1024, 8192),
     # stream kernel on 64 x 128 tiles (one round of 64..256 of them), tiles that end inside M, N and K
     (128, 4096, 4096), (65, 4100, 320), (130, 8000, 4160), (200, 3000, 8192), (500, 4099, 448), (512, 4096, 1024),
+    # and on 128 x 128 tiles (one round where 64 x 128 tiles need two)
+    (700, 4000, 1024), (650, 4100, 1088),
 ])
 def test_matmul_bit_exact(hip, dev, M, N, K):
     _say("matmul", M, N, K)
@@ -244,6 +246,8 @@ def test_dequant_kernels(hip, dev, M, N):
                                    (1024, 4096, 512), (900, 4100, 128), (200, 2051, 192), (1100, 8200, 320),
                                    # and on its 64 x 128 tiles
                                    (128, 4096, 512), (300, 3100, 320), (250, 8190, 384), (100, 4097, 1088),
+                                   # and on its 128 x 128 tiles
+                                   (700, 4000, 1024), (650, 4100, 1088),
                                    # the short-row kernel (K <= 256): whole-line and ragged epilogues, every step count
                                    (300, 1024, 64), (520, 2048, 256), (1000, 520, 192), (65, 4096, 128),
                                    # two to four rows on either decode kernel
