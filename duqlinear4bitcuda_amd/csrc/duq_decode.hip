@@ -1,4 +1,4 @@
-// Decode kernels (M <= 16 activation rows, K <= 16384): weight streaming for problems of a few MB,
+// Decode kernels (M <= 64 activation rows, K <= 16384): weight streaming for problems of a few MB,
 // where a launch lives for two or three microseconds and what counts is that every byte is requested
 // in the kernel's first instructions and nothing else sits on the critical path.
 //
@@ -20,8 +20,9 @@
 //    whole K range: lane l holds bytes [i*1024 + l*16, +16) of each row, so a load instruction covers 1 KB
 //    of one row and an activation register serves four rows.  The 4*M partial sums of a lane meet the other
 //    lanes' through the wavefront's own piece of LDS (no barrier) and a few DPP steps.
-//  MFMA kernel (M <= 16): v_mfma_i32_16x16x64_i8, eight wavefronts split K for one 16-column tile, the partial
-//    tiles meet in LDS, the first 256 threads finish one output each.
+//  MFMA kernel (5 <= M <= 64): v_mfma_i32_16x16x64_i8, eight wavefronts split K for one 16-column tile, one to
+//    four tiles of 16 rows against the same weight fragments, the partial tiles meet in LDS, 256 threads finish
+//    one output each per row tile; one round of at most 256 workgroups with several column tiles each.
 #include "duq_epilogue.h"
 #include "duq_launch.h"
 #include "duq_rowquant.h"

@@ -10,16 +10,17 @@
 // 256*|C| stays below 2^31 for K <= 131008.  Integer accumulation is order-free, so the
 // k order inside a tile only has to be the same for A and B.
 //
-// Five kernels here, picked by shape in select_gemm_kernel() (decode shapes of a few MB run the two kernels of
-// duq_decode.hip):
-//  * stream kernel (prefill, M >= 128; tiles of 128, 64 or 32 rows x 256 columns, the height
-//    picked per shape): weights go from global memory straight to registers, activations are
+// Six kernels here, picked by shape in select_gemm_kernel() (up to 64 rows run the two kernels of
+// duq_decode.hip as far as they reach):
+//  * stream kernel (prefill, more than 64 rows; tiles of 128, 64 or 32 rows x 256 columns or of 128 or 64 rows x
+//    128, the shape picked per problem): weights go from global memory straight to registers, activations are
 //    expanded once into LDS, v_mfma_i32_32x32x32_i8 with a hand-ordered schedule (see the kernel);
-//  * tile kernel (everything else above 16 rows, and any tensor of 4 GiB or more): BM x BN x 128 tiles,
-//    4 wavefronts (2 x 2), both operands expanded on the way into double-buffered LDS, v_mfma_i32_16x16x64_i8;
-//  * ring kernel (17 <= M <= 256 on narrow problems, and 5..16 rows of 12289..16384 elements): packed
-//    activations of all rows in LDS, every wavefront streams whole weight rows through a ring of loads;
-//  * skinny kernel (5 <= M <= 16 with 512 or more column tiles): one workgroup owns 16 output columns, its
+//  * short-row kernel (rows of at most 256 elements): the stream kernel's tile without its K pipeline;
+//  * tile kernel (what is left, and any tensor of 4 GiB or more): BM x BN x 128 tiles, 4 wavefronts (2 x 2),
+//    both operands expanded on the way into double-buffered LDS, v_mfma_i32_16x16x64_i8;
+//  * ring kernel (17 <= M <= 256 on narrow problems or long rows, and 5..16 rows of 12289..16384 elements):
+//    packed activations of all rows in LDS, every wavefront streams whole weight rows through a ring of loads;
+//  * skinny kernel (9 <= M <= 16 with 1536 or more column tiles): one workgroup owns 16 output columns, its
 //    wavefronts split K, whole-line weight loads turned into fragments through LDS;
 //  * dot kernel (M <= 4 with rows longer than 16384 elements): v_dot8_i32_i4 on the packed nibbles, a
 //    pure HBM stream.
