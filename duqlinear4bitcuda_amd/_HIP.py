@@ -615,6 +615,41 @@ def asym_dual_rowsum_dequant(q, xq, scale_row, zeros_row, rowsum_row, w, scale_c
     return x
 
 
+def linear4bit_forward_dual_rowsum(xq, scale_x, zeros_x, rowsum_x, w, w_scale_1, w_zeros_1, w_scale_2, w_zeros_2,
+                                   w_adj_1, w_adj_2, bias=None):
+    """``asym_dual_rowsum_dequant(matmul(xq, w), ...)`` as the library runs it best: one launch where the GEMM
+    kernel of the shape applies the epilogue itself, else the GEMM into a scratch int32 tensor and the stand-alone
+    epilogue.  Same bits either way.  ``xq`` uint8 [M, K/2], ``w`` uint8 [N, K/2]; returns fp16 [M, N]."""
+    name = "linear4bit_forward_dual_rowsum"
+    _check(name, xq, w)
+    _check_dtype(name, xq, "xq", _U8)
+    _check_dtype(name, w, "w", _U8)
+    if xq.dim() != 2 or w.dim() != 2 or xq.shape[1] != w.shape[1]:
+        raise RuntimeError(f"{name}: expected xq [M, K/2] and w [N, K/2], got {tuple(xq.shape)} and {tuple(w.shape)}")
+    M, kb = xq.shape
+    N = w.shape[0]
+    dev = xq.device
+    for t, what, dt, cnt in ((scale_x, "scale_x", _F16, M), (zeros_x, "zeros_x", _F16, M), (rowsum_x, "rowsum_x", _I32, M),
+                             (w_scale_1, "w_scale_1", _F16, N), (w_zeros_1, "w_zeros_1", _F16, N),
+                             (w_scale_2, "w_scale_2", _F16, N), (w_zeros_2, "w_zeros_2", _F16, N),
+                             (w_adj_1, "w_adj_1", _I32, N), (w_adj_2, "w_adj_2", _I32, N)) + \
+            (((bias, "bias", _F16, N),) if bias is not None else ()):
+        _fast_check(name, what, t, dt, dev)
+        if t.numel() != cnt:
+            _check_size0(name, t.reshape(-1), what, cnt)
+    lib = _lib.load()
+    y = torch.empty((M, N), dtype=_F16, device=dev)
+    need = int(lib.duq_linear4bit_dual_rowsum_workspace_bytes(M, N, kb * 2))
+    ws = torch.empty(need // 4, dtype=_I32, device=dev) if need else None
+    st = _launch(dev, lib.duq_linear4bit_forward_dual_rowsum, xq.data_ptr(), scale_x.data_ptr(), zeros_x.data_ptr(),
+                 rowsum_x.data_ptr(), w.data_ptr(), w_scale_1.data_ptr(), w_zeros_1.data_ptr(), w_scale_2.data_ptr(),
+                 w_zeros_2.data_ptr(), w_adj_1.data_ptr(), w_adj_2.data_ptr(), _ptr(bias), M, N, kb * 2, y.data_ptr(),
+                 ws.data_ptr() if ws is not None else None, need)
+    if st:
+        _lib.check(st, name)
+    return y
+
+
 # ---- the forward on the 6-bit float matrix path (exact; not in the reference) --------------
 
 EPI_ASYM_ROWSUM = 4

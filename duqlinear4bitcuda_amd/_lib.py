@@ -51,6 +51,9 @@ PROTOTYPES = {
     "duq_asym_rowsum_dequant_host": [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_u32, _c_u32, _c_p, _c_p],
     "duq_asym_dual_rowsum_dequant_host": [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p,
                                           _c_u32, _c_u32, _c_u32, _c_p, _c_p],
+    "duq_linear4bit_dual_rowsum_workspace_bytes": [_c_u32, _c_u32, _c_u32],  # returns uint64_t (restype set in load())
+    "duq_linear4bit_forward_dual_rowsum": [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p,
+                                           _c_u32, _c_u32, _c_u32, _c_p, _c_p, ctypes.c_uint64, _c_p],
     "duq_weight_shadow_bf6": [_c_p, _c_u32, _c_u32, _c_p, _c_p],
     "duq_quantize_rows_sym_bf6": [_c_p, _c_u32, _c_u32, ctypes.c_float, _c_i32, _c_p, _c_p, _c_p, _c_p],
     "duq_quantize_rows_asym_bf6": [_c_p, _c_u32, _c_u32, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p],
@@ -89,6 +92,7 @@ def load():
         fn.argtypes = argtypes
         fn.restype = ctypes.c_int
     lib.duq_quantize_linear4bit_workspace_bytes.restype = ctypes.c_uint64
+    lib.duq_linear4bit_dual_rowsum_workspace_bytes.restype = ctypes.c_uint64
     lib.duq_status_string.argtypes = [ctypes.c_int]
     lib.duq_status_string.restype = ctypes.c_char_p
     _lib = lib

@@ -427,6 +427,41 @@ int duq_asym_dual_rowsum_dequant_host(const int32_t *q, const uint8_t *xq, const
     return duq::launch_dual_rowsum_dequant(p, as_stream(stream));
 }
 
+uint64_t duq_linear4bit_dual_rowsum_workspace_bytes(uint32_t M, uint32_t N, uint32_t K)
+{
+    if (M == 0 || N == 0 || K == 0) return 0;
+    return duq::gemm_fuses_dual_rowsum(M, N, K) ? 0 : (uint64_t)M * N * 4;
+}
+
+int duq_linear4bit_forward_dual_rowsum(const uint8_t *xq, const duq_half *scale_x, const duq_half *zeros_x,
+                                       const int32_t *rowsum_x, const uint8_t *w, const duq_half *w_scale_1,
+                                       const duq_half *w_zeros_1, const duq_half *w_scale_2,
+                                       const duq_half *w_zeros_2, const int32_t *w_adj_1, const int32_t *w_adj_2,
+                                       const duq_half *bias, uint32_t M, uint32_t N, uint32_t K, duq_half *y,
+                                       void *acc_workspace, uint64_t workspace_bytes, duq_stream_t stream)
+{
+    if (int e = check_gemm(xq, w, M, N, K)) return e;
+    if (M == 0 || N == 0) return DUQ_OK;
+    if (K == 0) return DUQ_E_KALIGN;
+    if (!scale_x || !zeros_x || !rowsum_x || !w_scale_1 || !w_zeros_1 || !w_scale_2 || !w_zeros_2 || !w_adj_1 || !w_adj_2 || !y)
+        return DUQ_E_NULL;
+    if (!aligned(y, 16)) return DUQ_E_ALIGN;
+    const uint64_t need = duq_linear4bit_dual_rowsum_workspace_bytes(M, N, K);
+    if (need == 0) {
+        duq::Epilogue e{DUQ_EPI_ASYM_DUAL_ROWSUM, scale_x, zeros_x, w_scale_1, w_zeros_1, w_scale_2, w_zeros_2, bias, rowsum_x,
+                        w_adj_1,                  w_adj_2};
+        return duq::launch_gemm_s4(xq, w, M, N, K, nullptr, &e, y, as_stream(stream));
+    }
+    if (!acc_workspace) return DUQ_E_NULL;
+    if (workspace_bytes < need) return DUQ_E_SHAPE;
+    if (!aligned(acc_workspace, 16)) return DUQ_E_ALIGN;
+    int32_t *acc = static_cast<int32_t *>(acc_workspace);
+    if (int e = duq::launch_gemm_s4(xq, w, M, N, K, acc, nullptr, nullptr, as_stream(stream))) return e;
+    duq::DualRowsumParams p{acc,       xq,        w,         K / 2,   scale_x, zeros_x, rowsum_x, w_scale_1, w_zeros_1,
+                            w_scale_2, w_zeros_2, w_adj_1,   w_adj_2, bias,    M,       N,        y};
+    return duq::launch_dual_rowsum_dequant(p, as_stream(stream));
+}
+
 int duq_linear4bit_forward_rowsum(const uint8_t *xq, const duq_half *scale_x, const duq_half *zeros_x,
                                   const int32_t *rowsum_x, const uint8_t *w, const duq_half *w_scale,
                                   const duq_half *w_zeros, const int32_t *w_rowsum_adj, const duq_half *bias,

@@ -129,39 +129,41 @@ __global__ __launch_bounds__(256) void dual_rowsum_dequant_kernel(DualRowsumPara
         a2[j] = (uint32_t)p.adj_col_2[n];
         bias[j] = BIAS ? bits_to_f16(p.bias[n]) : (f16)0;
     }
-    const uint32_t r0 = blockIdx.y * kDualRows, r1 = min(r0 + kDualRows, p.rows);
-    for (uint32_t r = r0; r < r1; ++r) {
-        const v2u xh = *reinterpret_cast<const v2u *>(p.xq + (uint64_t)r * p.kbytes);
-        const uint32_t xlo = xh[0], xhi = xh[1] & 0xFFu;  // input columns 0..7 and 8, 9
-        const uint32_t rxl = (uint32_t)__builtin_amdgcn_sdot8((int)xhi, 0x11111111, __builtin_amdgcn_sdot8((int)xlo, 0x11111111, 0, false), false);
-        const uint32_t zx = (uint32_t)rint_i32((float)bits_to_f16(p.z_row[r]));
-        const float sx = (float)bits_to_f16(p.s_row[r]);
-        const uint32_t rxr = (uint32_t)p.rs_row[r] - rxl;
-        int acc[4];
-        if (vec) {
-            const v4i a = *reinterpret_cast<const v4i *>(p.acc + (uint64_t)r * p.cols + n0);
+    // every load of the kDualRows rows is requested before the first result is needed (rows past the end repeat
+    // the last one and store nothing)
+    const uint32_t r0 = blockIdx.y * kDualRows;
+    v2u xh[kDualRows];
+    uint32_t zxs[kDualRows], rss[kDualRows];
+    float sxs[kDualRows];
+    v4i accv[kDualRows];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc[j] = a[j];
+    for (uint32_t i = 0; i < kDualRows; ++i) {
+        const uint32_t r = min(r0 + i, p.rows - 1);
+        xh[i] = *reinterpret_cast<const v2u *>(p.xq + (uint64_t)r * p.kbytes);
+        zxs[i] = (uint32_t)rint_i32((float)bits_to_f16(p.z_row[r]));
+        sxs[i] = (float)bits_to_f16(p.s_row[r]);
+        rss[i] = (uint32_t)p.rs_row[r];
+        if (vec) {
+            accv[i] = *reinterpret_cast<const v4i *>(p.acc + (uint64_t)r * p.cols + n0);
         } else {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc[j] = p.acc[(uint64_t)r * p.cols + min(n0 + j, p.cols - 1)];
+            for (int j = 0; j < 4; ++j) accv[i][j] = p.acc[(uint64_t)r * p.cols + min(n0 + j, p.cols - 1)];
         }
+    }
+#pragma unroll
+    for (uint32_t i = 0; i < kDualRows; ++i) {
+        const uint32_t r = r0 + i;
+        const uint32_t xlo = xh[i][0], xhi = xh[i][1] & 0xFFu;  // input columns 0..7 and 8, 9
+        const uint32_t rxl = (uint32_t)__builtin_amdgcn_sdot8((int)xhi, 0x11111111, __builtin_amdgcn_sdot8((int)xlo, 0x11111111, 0, false), false);
+        const uint32_t zx = zxs[i];
+        const float sx = sxs[i];
+        const uint32_t rxr = rss[i] - rxl;
         uint16_t out[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const uint32_t accl = (uint32_t)__builtin_amdgcn_sdot8((int)xhi, (int)whi[j], __builtin_amdgcn_sdot8((int)xlo, (int)wlo[j], 0, false), false);
-            // 32-bit wrapping integer arithmetic, like the single-range row-sum epilogue
-            const int corr_l = (int)(accl - zx * a1[j] - z1[j] * rxl);
-            const int corr_r = (int)(((uint32_t)acc[j] - accl) - zx * a2[j] - z2[j] * rxr);
-            float t1 = (float)corr_l * (sx * s1[j]);  // sx * s: exact (11-bit significands)
-            float t2 = (float)corr_r * (sx * s2[j]);
-            asm volatile("" : "+v"(t1), "+v"(t2));    // each product rounded to float32 on its own
-            float t = t1 + t2;
-            asm volatile("" : "+v"(t));               // the sum rounded to float32, then to binary16
-            f16 y = (f16)t;
-            if (BIAS) y = y + bias[j];
-            out[j] = f16_to_bits(y);
-        }
+        for (int j = 0; j < 4; ++j)
+            out[j] = dual_rowsum_one(accv[i][j], xlo, xhi, zx, rxl, rxr, sx, wlo[j], whi[j], s1[j], s2[j], z1[j], z2[j], a1[j],
+                                     a2[j], BIAS, bias[j]);
+        if (r >= p.rows) continue;
         uint16_t *dst = p.y + (uint64_t)r * p.cols + n0;
         if (vec) {
             *reinterpret_cast<v2u *>(dst) = v2u{(uint32_t)out[0] | ((uint32_t)out[1] << 16), (uint32_t)out[2] | ((uint32_t)out[3] << 16)};

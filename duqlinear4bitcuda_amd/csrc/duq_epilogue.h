@@ -43,6 +43,7 @@ __device__ __forceinline__ void batch_shift(Epilogue &e, uint32_t b, uint32_t ro
     if (e.z_col_2) e.z_col_2 += c;
     if (e.bias) e.bias += c;
     if (e.rs_col) e.rs_col += c;
+    if (e.rs_col_2) e.rs_col_2 += c;
 }
 
 template <int MODE>
@@ -149,6 +150,29 @@ __device__ __forceinline__ uint32_t dequant_pair(ACC acc0, ACC acc1, const RowEp
     }
     if (BIAS) y = y + v2h{c0.bias, c1.bias};
     return __builtin_bit_cast(uint32_t, y);
+}
+
+// Row-sum epilogue of the dual-uniform layer for one output (definition: include/duq_hip.h,
+// duq_asym_dual_rowsum_dequant_host), shared by the stand-alone kernel and the fused GEMM so that both give
+// identical bits.  xlo / xhi and wlo / whi: the first eight bytes of the packed activation and weight rows, xhi
+// masked to its two nibbles (input columns 8, 9); rxl = sum of the activation row's codes 0..9, rxr = of the others.
+__device__ __forceinline__ uint16_t dual_rowsum_one(int acc, uint32_t xlo, uint32_t xhi, uint32_t zx, uint32_t rxl,
+                                                    uint32_t rxr, float sx, uint32_t wlo, uint32_t whi, float s1, float s2,
+                                                    uint32_t z1, uint32_t z2, uint32_t a1, uint32_t a2, bool with_bias,
+                                                    f16 bias)
+{
+    const uint32_t accl = (uint32_t)__builtin_amdgcn_sdot8((int)xhi, (int)whi, __builtin_amdgcn_sdot8((int)xlo, (int)wlo, 0, false), false);
+    // 32-bit wrapping integer arithmetic, like the single-range row-sum epilogue
+    const int corr_l = (int)(accl - zx * a1 - z1 * rxl);
+    const int corr_r = (int)(((uint32_t)acc - accl) - zx * a2 - z2 * rxr);
+    float t1 = (float)corr_l * (sx * s1);  // sx * s: exact (11-bit significands)
+    float t2 = (float)corr_r * (sx * s2);
+    asm volatile("" : "+v"(t1), "+v"(t2));  // each product rounded to float32 on its own
+    float t = t1 + t2;
+    asm volatile("" : "+v"(t));             // the sum rounded to float32, then to binary16
+    f16 y = (f16)t;
+    if (with_bias) y = y + bias;
+    return f16_to_bits(y);
 }
 
 // Column parameters of four consecutive output columns n0 .. n0+3, fetched with 64-bit

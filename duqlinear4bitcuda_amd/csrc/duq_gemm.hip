@@ -284,6 +284,11 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
     constexpr uint32_t kBuf = BM * kXStride;
 
     __shared__ __attribute__((aligned(16))) uint8_t lds[3 * kBuf];
+    // dual-uniform row-sum epilogue (EPI 5): its parameters, eight words per column of the tile and per row,
+    // fetched by the first BN / BM threads before the loop and read back from here after it
+    //   column: wlo, whi (first eight bytes of the weight row), s1 | s2 << 16, z1, z2, adj1, adj2, bias
+    //   row   : xlo, xhi & 0xFF (first ten codes of the activation row), float(s), z, rx - rxl, rxl
+    __shared__ __attribute__((aligned(16))) uint32_t dpar[EPI == 5 ? (BN + BM) * 8 : 4];
 
     if (blockIdx.z) batch_shift(p, blockIdx.z);
     uint32_t tile_m, tile_n;
@@ -295,6 +300,36 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
     const uint32_t kbytes = p.K >> 1;
     const uint32_t nfull = p.K / kCK;
     const uint32_t nchunks = (p.K + kCK - 1) / kCK;
+
+    if constexpr (EPI == 5) {
+        if (tid < (uint32_t)BN) {
+            const uint32_t n = min(n0 + tid, p.N - 1);
+            const v2u head = *reinterpret_cast<const v2u *>(p.B + (uint64_t)n * kbytes);
+            uint32_t *d = dpar + tid * 8;
+            d[0] = head[0];
+            d[1] = head[1];
+            d[2] = (uint32_t)p.epi.s_col_1[n] | ((uint32_t)p.epi.s_col_2[n] << 16);
+            d[3] = (uint32_t)rint_i32((float)bits_to_f16(p.epi.z_col_1[n]));
+            d[4] = (uint32_t)rint_i32((float)bits_to_f16(p.epi.z_col_2[n]));
+            d[5] = (uint32_t)p.epi.rs_col[n];
+            d[6] = (uint32_t)p.epi.rs_col_2[n];
+            d[7] = BIAS ? (uint32_t)p.epi.bias[n] : 0u;
+        }
+        if (tid < (uint32_t)BM) {
+            const uint32_t m = min(m0 + tid, p.M - 1);
+            const v2u head = *reinterpret_cast<const v2u *>(p.A + (uint64_t)m * kbytes);
+            const uint32_t xlo = head[0], xhi = head[1] & 0xFFu;  // input columns 0..7 and 8, 9
+            const uint32_t rxl = (uint32_t)__builtin_amdgcn_sdot8((int)xhi, 0x11111111, __builtin_amdgcn_sdot8((int)xlo, 0x11111111, 0, false), false);
+            uint32_t *d = dpar + (BN + tid) * 8;
+            d[0] = xlo;
+            d[1] = xhi;
+            d[2] = __builtin_bit_cast(uint32_t, (float)bits_to_f16(p.epi.s_row[m]));
+            d[3] = (uint32_t)rint_i32((float)bits_to_f16(p.epi.z_row[m]));
+            d[4] = (uint32_t)p.epi.rs_row[m] - rxl;
+            d[5] = rxl;
+        }
+        // (the barrier that ends the prologue below orders these writes before the epilogue's reads)
+    }
 
     const __amdgpu_buffer_rsrc_t rW = make_rsrc(p.B + (uint64_t)n0 * kbytes, min(p.N - n0, (uint32_t)BN) * kbytes);
     const __amdgpu_buffer_rsrc_t rX = make_rsrc(p.A + (uint64_t)m0 * kbytes, min(p.M - m0, (uint32_t)BM) * kbytes);
@@ -461,6 +496,7 @@ __global__ __launch_bounds__(256, 2) void gemm_s4_shortk_kernel(GemmParams p)
     constexpr int NXP = TM;  // 16-byte activation pieces per thread
     constexpr uint32_t kBuf = BM * kXStride, kStage = 4 * BM * 144;
     __shared__ __attribute__((aligned(16))) uint8_t lds[kBuf > kStage ? kBuf : kStage];
+    uint32_t *const dpar = nullptr;  // named by the shared epilogue text for an epilogue this kernel never runs
 
     if (blockIdx.z) batch_shift(p, blockIdx.z);
     // column blocks fastest: neighbouring workgroups share an activation tile
@@ -938,6 +974,8 @@ static void launch_epi(GemmParams &p, hipStream_t stream, uint32_t batch = 1)
 {
     const int kernel = batch > 1 ? (p.M > 32 && ((p.M + 31) / 32) * ((p.N + 255) / 256) * batch >= 32 ? kKernelStream : kKernelTile)
                                  : select_gemm_kernel(p.M, p.N, p.K);
+    // (EPI 5, the dual-uniform row-sum epilogue, exists in the stream kernel only: gemm_fuses_dual_rowsum)
+    if constexpr (EPI != 5) {
     if (kernel == kKernelDot) {
         const uint32_t xstride = ((p.K / 2 + 127) / 128) * 128;
         const dim3 grid((p.N + 7) / 8);
@@ -995,6 +1033,7 @@ static void launch_epi(GemmParams &p, hipStream_t stream, uint32_t batch = 1)
 #undef DUQ_RING
         return;
     }
+    }
     // Stream kernel with 128, 64 or 32 activation rows x 256 columns per workgroup, or 128 or 64 x 128: whole rounds
     // of 256 workgroups (one per CU) cost about nchunks * c + f microseconds each, c and f measured per tile shape;
     // the cheapest wins.  The L2 -> CU path bounds these tiles, so what counts is operand rows per output: a
@@ -1022,7 +1061,7 @@ static void launch_epi(GemmParams &p, hipStream_t stream, uint32_t batch = 1)
             }
         }
     }
-    if (best_tm && p.K <= 256) {
+    if constexpr (EPI != 5) if (best_tm && p.K <= 256) {
         // rows of at most 256 elements: one chunk, the launch is its output stores: the short-row kernel with 64-row
         // tiles (measured on 32 products of 2048 x 2048 x 128: 86 us against 95 us on the stream kernel's 64-row tiles)
         p.tiles_m = (p.M + 63) / 64;
@@ -1049,21 +1088,23 @@ static void launch_epi(GemmParams &p, hipStream_t stream, uint32_t batch = 1)
             hipLaunchKernelGGL((gemm_s4_stream_kernel<2, EPI, BIAS>), grid, dim3(256), 0, stream, p);
         else
             hipLaunchKernelGGL((gemm_s4_stream_kernel<1, EPI, BIAS>), grid, dim3(256), 0, stream, p);
-    } else if (tiles(128, 256) >= 256 && p.M > 64) {
-        p.tiles_m = (p.M + 127) / 128;
-        p.tiles_n = (p.N + 255) / 256;
-        hipLaunchKernelGGL((gemm_s4_tile_kernel<128, 256, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(256), 0,
-                           stream, p);
-    } else if (tiles(128, 128) >= 256 && p.M > 64) {
-        p.tiles_m = (p.M + 127) / 128;
-        p.tiles_n = (p.N + 127) / 128;
-        hipLaunchKernelGGL((gemm_s4_tile_kernel<128, 128, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(256), 0,
-                           stream, p);
-    } else {
-        p.tiles_m = (p.M + 63) / 64;
-        p.tiles_n = (p.N + 63) / 64;
-        hipLaunchKernelGGL((gemm_s4_tile_kernel<64, 64, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(256), 0,
-                           stream, p);
+    } else if constexpr (EPI != 5) {
+        if (tiles(128, 256) >= 256 && p.M > 64) {
+            p.tiles_m = (p.M + 127) / 128;
+            p.tiles_n = (p.N + 255) / 256;
+            hipLaunchKernelGGL((gemm_s4_tile_kernel<128, 256, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(256),
+                               0, stream, p);
+        } else if (tiles(128, 128) >= 256 && p.M > 64) {
+            p.tiles_m = (p.M + 127) / 128;
+            p.tiles_n = (p.N + 127) / 128;
+            hipLaunchKernelGGL((gemm_s4_tile_kernel<128, 128, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(256),
+                               0, stream, p);
+        } else {
+            p.tiles_m = (p.M + 63) / 64;
+            p.tiles_n = (p.N + 63) / 64;
+            hipLaunchKernelGGL((gemm_s4_tile_kernel<64, 64, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(256), 0,
+                               stream, p);
+        }
     }
 }
 
@@ -1108,6 +1149,13 @@ int launch_gemm_s4_batched(const uint8_t *A, const uint8_t *B, uint32_t M, uint3
             DUQ_GEMM(2)
             DUQ_GEMM(3)
             DUQ_GEMM(4)
+        case 5:
+            if (batch != 1 || !gemm_fuses_dual_rowsum(M, N, K)) return (int)hipErrorInvalidValue;
+            if (bias)
+                launch_epi<5, true>(p, stream, 1);
+            else
+                launch_epi<5, false>(p, stream, 1);
+            break;
         default:
             return (int)hipErrorInvalidValue;
         }

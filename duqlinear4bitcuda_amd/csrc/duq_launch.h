@@ -25,8 +25,8 @@ int launch_quantize_rows_asym(const uint16_t *x, uint32_t rows, uint32_t cols, u
                               uint16_t *zeros, int32_t *rowsum, uint8_t *bf6, hipStream_t stream);
 
 // Epilogue description shared by the stand-alone dequant kernels and the fused GEMM.
-// mode: 0 sym, 1 asym, 2 sym-dual, 3 asym-dual, 4 asym with row-sum zero-point correction
-// (DUQ_EPI_* of the public header).
+// mode: 0 sym, 1 asym, 2 sym-dual, 3 asym-dual, 4 asym with row-sum zero-point correction, 5 the same for the
+// dual-uniform layer (fused GEMM only, shapes of gemm_fuses_dual_rowsum) (DUQ_EPI_* of the public header).
 struct Epilogue {
     int mode;
     const uint16_t *s_row;   // [rows]
@@ -37,7 +37,9 @@ struct Epilogue {
     const uint16_t *z_col_2; // [cols]  asym-dual
     const uint16_t *bias;    // [cols] or nullptr
     const int32_t *rs_row;   // [rows]  mode 4: sum over k of the row's shifted codes
-    const int32_t *rs_col;   // [cols]  mode 4: sum over k of the column's shifted codes minus K * zero
+    const int32_t *rs_col;   // [cols]  mode 4: sum over k of the column's shifted codes minus K * zero (mode 5: of
+                             //         input columns 0..9)
+    const int32_t *rs_col_2; // [cols]  mode 5: the same over the other input columns
 };
 
 int launch_dequant(const int32_t *acc, const Epilogue &epi, uint32_t rows, uint32_t cols, uint16_t *y,
@@ -77,6 +79,13 @@ enum GemmKernelId {
     kKernelTile = 7,        // duq_gemm.hip, everything else (per-tile 64-bit bases: any tensor size)
 };
 int select_gemm_kernel(uint32_t M, uint32_t N, uint32_t K);
+// Shapes whose GEMM can apply the dual-uniform row-sum epilogue itself (mode 5): those of the stream kernel with
+// rows longer than 256 elements and N % 8 == 0 (its staged stores); the others run the GEMM into int32 and
+// launch_dual_rowsum_dequant.
+inline bool gemm_fuses_dual_rowsum(uint32_t M, uint32_t N, uint32_t K)
+{
+    return select_gemm_kernel(M, N, K) == kKernelStream && K > 256 && N % 8 == 0;
+}
 inline bool decode_uses_rows_kernel(uint32_t M) { return M <= 4; }
 // MFMA decode kernel: one round of at most 256 workgroups, each with its share of the 16-column tiles.  The
 // activations enter a CU once, and a workgroup has two tiles' weights in flight whatever their number; measured

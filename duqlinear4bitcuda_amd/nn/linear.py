@@ -276,10 +276,16 @@ class LinearQuant4bitDUASQRowSum(_Linear4bitBase):
         xq = x.quantized_x
         lead = xq.shape[:-1]
         xq2 = xq.reshape(-1, xq.shape[-1])
-        acc = _ops.matmul(xq2, self.weight)
-        y = _ops.asym_dual_rowsum_dequant(acc, xq2, x.scales_x, x.zeros_x, x.rowsum_x, self.weight,
-                                          self.weight_scales_1, self.weight_zeros_1, self.weight_scales_2,
-                                          self.weight_zeros_2, self.weight_rowsum_1, self.weight_rowsum_2, self.bias)
+        if self.fused:
+            y = _ops.linear4bit_forward_dual_rowsum(xq2, x.scales_x, x.zeros_x, x.rowsum_x, self.weight,
+                                                    self.weight_scales_1, self.weight_zeros_1, self.weight_scales_2,
+                                                    self.weight_zeros_2, self.weight_rowsum_1, self.weight_rowsum_2,
+                                                    self.bias)
+        else:
+            acc = _ops.matmul(xq2, self.weight)
+            y = _ops.asym_dual_rowsum_dequant(acc, xq2, x.scales_x, x.zeros_x, x.rowsum_x, self.weight,
+                                              self.weight_scales_1, self.weight_zeros_1, self.weight_scales_2,
+                                              self.weight_zeros_2, self.weight_rowsum_1, self.weight_rowsum_2, self.bias)
         return y.view(*lead, -1)
 
     @classmethod

@@ -57,6 +57,7 @@ typedef void *duq_stream_t;  /* hipStream_t */
 #define DUQ_EPI_SYM_DUAL 2   /* src/kernels/quant2.cu:62-83  */
 #define DUQ_EPI_ASYM_DUAL 3  /* src/kernels/quant2.cu:158-186 */
 #define DUQ_EPI_ASYM_ROWSUM 4 /* exact zero-point correction with row sums; not in the reference */
+#define DUQ_EPI_ASYM_DUAL_ROWSUM 5 /* the same for the dual-uniform layer (duq_linear4bit_forward_dual_rowsum only) */
 
 /* ---- library info ------------------------------------------------------------------ */
 
@@ -312,6 +313,21 @@ int duq_asym_dual_rowsum_dequant_host(const int32_t *q, const uint8_t *xq, const
                                       const duq_half *scale_col_2, const duq_half *zeros_col_2,
                                       const int32_t *adj_col_1, const int32_t *adj_col_2, const duq_half *bias,
                                       uint32_t rows, uint32_t cols, uint32_t K, duq_half *x, duq_stream_t stream);
+
+/* GEMM + that epilogue: y[M,N] = dual row-sum epilogue of xq[M,K/2] x w[N,K/2]^T, bit-identical to
+ * duq_matmul_host_4bit followed by duq_asym_dual_rowsum_dequant_host (no counterpart in the reference).  Shapes for
+ * which duq_linear4bit_dual_rowsum_workspace_bytes(M, N, K) is 0 (the prefill kernel with rows longer than 256
+ * elements and N % 8 == 0) run as one launch and `acc_workspace` may be NULL; the others run those two launches and
+ * stage the int32 accumulators in `acc_workspace` (at least the bytes the query returns, 16-byte aligned, owned by
+ * the caller: the library allocates nothing).  y 16-byte aligned, the column arrays as torch allocates them
+ * (16-byte aligned). */
+uint64_t duq_linear4bit_dual_rowsum_workspace_bytes(uint32_t M, uint32_t N, uint32_t K);
+int duq_linear4bit_forward_dual_rowsum(const uint8_t *xq, const duq_half *scale_x, const duq_half *zeros_x,
+                                       const int32_t *rowsum_x, const uint8_t *w, const duq_half *w_scale_1,
+                                       const duq_half *w_zeros_1, const duq_half *w_scale_2,
+                                       const duq_half *w_zeros_2, const int32_t *w_adj_1, const int32_t *w_adj_2,
+                                       const duq_half *bias, uint32_t M, uint32_t N, uint32_t K, duq_half *y,
+                                       void *acc_workspace, uint64_t workspace_bytes, duq_stream_t stream);
 
 /* ---- the same forward on the 6-bit float matrix path ---------------------------------- */
 

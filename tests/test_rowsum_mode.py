@@ -245,7 +245,8 @@ def test_gpu_rowsum_module_config4(dev):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("M,N,K", [(1, 64, 64), (7, 130, 128), (48, 1000, 256), (300, 1027, 320), (512, 4096, 4096),
+@pytest.mark.parametrize("M,N,K", [(128, 4096, 512), (300, 3104, 320), (700, 4000, 1024), (1024, 4096, 320), (65, 8192, 448),
+                                   (1, 64, 64), (7, 130, 128), (48, 1000, 256), (300, 1027, 320), (512, 4096, 4096),
                                    (33, 4100, 1024), (2050, 96, 64)])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_gpu_dual_rowsum_dequant(hip, dev, M, N, K, with_bias):
@@ -266,6 +267,32 @@ def test_gpu_dual_rowsum_dequant(hip, dev, M, N, K, with_bias):
     got = hip.asym_dual_rowsum_dequant(acc_gpu, q, s, z, r, T(wq), T(s1), T(z1), T(s2), T(z2), T(a1), T(a2),
                                        None if bias is None else T(bias))
     assert cases.bits_equal(got.cpu().numpy(), want)
+    # GEMM + epilogue through one entry point (one launch where the GEMM kernel of the shape applies it itself)
+    got = hip.linear4bit_forward_dual_rowsum(q, s, z, r, T(wq), T(s1), T(z1), T(s2), T(z2), T(a1), T(a2),
+                                             None if bias is None else T(bias))
+    assert cases.bits_equal(got.cpu().numpy(), want)
+
+
+def test_dual_rowsum_fused_shapes_and_validation():
+    """Which shapes the fused entry point runs as one launch (no workspace), and its argument checks."""
+    from duqlinear4bitcuda_amd import _lib
+
+    lib = _lib.load()
+    ws = lib.duq_linear4bit_dual_rowsum_workspace_bytes
+    assert ws(512, 4096, 4096) == 0 and ws(128, 4096, 512) == 0 and ws(2048, 4096, 4096) == 0 and ws(700, 4000, 1024) == 0
+    assert ws(16, 4096, 4096) == 16 * 4096 * 4      # decode kernels
+    assert ws(300, 1028, 320) == 300 * 1028 * 4     # N % 8 != 0
+    assert ws(512, 4096, 256) == 512 * 4096 * 4     # short rows
+    assert ws(0, 4096, 4096) == 0
+    P = 0x1000
+    f = lib.duq_linear4bit_forward_dual_rowsum
+    args = lambda M, N, K, y=P, w=None, nb=0: (P, P, P, P, P, P, P, P, P, P, P, None, M, N, K, y, w, nb, None)
+    assert f(*args(16, 64, 100)) == -3                      # K % 64
+    assert f(*args(16, 64, 128, y=None)) == -1
+    assert f(*args(16, 64, 128, y=P + 2)) == -5
+    assert f(*args(16, 64, 128)) == -1                      # needs a workspace
+    assert f(*args(16, 64, 128, w=P, nb=100)) == -2         # too small
+    assert f(*args(0, 64, 128)) == 0
 
 
 @pytest.mark.gpu
