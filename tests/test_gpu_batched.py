@@ -26,7 +26,8 @@ def _nibbles(n, rows, K, seed):
 # of the batched kernel choice (more or fewer than 32 tiles of 32 x 256 over the whole batch), a tile-kernel
 # shape with 128-row tiles, short rows (64-row tiles) and a narrow B (128 x 128 tiles)
 SHAPES = [(3, 40, 33, 128), (5, 1, 70, 64), (2, 130, 300, 512), (8, 160, 520, 320), (4, 33, 2100, 256),
-          (2, 520, 2100, 192), (1, 77, 130, 128), (7, 16, 16, 64), (3, 100, 600, 256), (6, 200, 100, 512)]
+          (2, 520, 2100, 192), (1, 77, 130, 128), (7, 16, 16, 64), (3, 100, 600, 256), (6, 200, 100, 512),
+          (3, 700, 1024, 1024)]
 
 
 @pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
