@@ -161,8 +161,8 @@ __global__ __launch_bounds__(256) void dual_rowsum_dequant_kernel(DualRowsumPara
         uint16_t out[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-            out[j] = dual_rowsum_one(accv[i][j], xlo, xhi, zx, rxl, rxr, sx, wlo[j], whi[j], s1[j], s2[j], z1[j], z2[j], a1[j],
-                                     a2[j], BIAS, bias[j]);
+            out[j] = dual_rowsum_one<false>(accv[i][j], xlo, xhi, zx, rxl, rxr, sx, wlo[j], whi[j], s1[j], s2[j], z1[j], z2[j],
+                                            a1[j], a2[j], BIAS, bias[j]);
         if (r >= p.rows) continue;
         uint16_t *dst = p.y + (uint64_t)r * p.cols + n0;
         if (vec) {

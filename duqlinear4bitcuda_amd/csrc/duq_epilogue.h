@@ -156,6 +156,11 @@ __device__ __forceinline__ uint32_t dequant_pair(ACC acc0, ACC acc1, const RowEp
 // duq_asym_dual_rowsum_dequant_host), shared by the stand-alone kernel and the fused GEMM so that both give
 // identical bits.  xlo / xhi and wlo / whi: the first eight bytes of the packed activation and weight rows, xhi
 // masked to its two nibbles (input columns 8, 9); rxl = sum of the activation row's codes 0..9, rxr = of the others.
+// I24: every factor of the four products is known to lie inside the signed 24-bit range (fits_i24), so they run
+// on the full-rate 24-bit multiplier; the low 32 bits of those products are the wrapping 32-bit products.
+__device__ __forceinline__ bool fits_i24(uint32_t v) { return (uint32_t)((int)v + (1 << 23)) < (1u << 24); }
+
+template <bool I24 = false>
 __device__ __forceinline__ uint16_t dual_rowsum_one(int acc, uint32_t xlo, uint32_t xhi, uint32_t zx, uint32_t rxl,
                                                     uint32_t rxr, float sx, uint32_t wlo, uint32_t whi, float s1, float s2,
                                                     uint32_t z1, uint32_t z2, uint32_t a1, uint32_t a2, bool with_bias,
@@ -163,8 +168,11 @@ __device__ __forceinline__ uint16_t dual_rowsum_one(int acc, uint32_t xlo, uint3
 {
     const uint32_t accl = (uint32_t)__builtin_amdgcn_sdot8((int)xhi, (int)whi, __builtin_amdgcn_sdot8((int)xlo, (int)wlo, 0, false), false);
     // 32-bit wrapping integer arithmetic, like the single-range row-sum epilogue
-    const int corr_l = (int)(accl - zx * a1 - z1 * rxl);
-    const int corr_r = (int)(((uint32_t)acc - accl) - zx * a2 - z2 * rxr);
+    auto mul = [](uint32_t a, uint32_t b) -> uint32_t {
+        return I24 ? (uint32_t)__mul24((int)a, (int)b) : a * b;
+    };
+    const int corr_l = (int)(accl - mul(zx, a1) - mul(z1, rxl));
+    const int corr_r = (int)(((uint32_t)acc - accl) - mul(zx, a2) - mul(z2, rxr));
     float t1 = (float)corr_l * (sx * s1);  // sx * s: exact (11-bit significands)
     float t2 = (float)corr_r * (sx * s2);
     asm volatile("" : "+v"(t1), "+v"(t2));  // each product rounded to float32 on its own

@@ -289,6 +289,7 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
     //   column: wlo, whi (first eight bytes of the weight row), s1 | s2 << 16, z1, z2, adj1, adj2, bias
     //   row   : xlo, xhi & 0xFF (first ten codes of the activation row), float(s), z, rx - rxl, rxl
     __shared__ __attribute__((aligned(16))) uint32_t dpar[EPI == 5 ? (BN + BM) * 8 : 4];
+    __shared__ uint32_t dwide;  // EPI 5: non-zero when a factor of the corrections leaves the signed 24-bit range
 
     if (blockIdx.z) batch_shift(p, blockIdx.z);
     uint32_t tile_m, tile_n;
@@ -302,6 +303,9 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
     const uint32_t nchunks = (p.K + kCK - 1) / kCK;
 
     if constexpr (EPI == 5) {
+        if (tid == 0) dwide = 0;
+        __syncthreads();
+        bool wide = false;
         if (tid < (uint32_t)BN) {
             const uint32_t n = min(n0 + tid, p.N - 1);
             const v2u head = *reinterpret_cast<const v2u *>(p.B + (uint64_t)n * kbytes);
@@ -314,6 +318,7 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
             d[5] = (uint32_t)p.epi.rs_col[n];
             d[6] = (uint32_t)p.epi.rs_col_2[n];
             d[7] = BIAS ? (uint32_t)p.epi.bias[n] : 0u;
+            wide = !(fits_i24(d[3]) && fits_i24(d[4]) && fits_i24(d[5]) && fits_i24(d[6]));
         }
         if (tid < (uint32_t)BM) {
             const uint32_t m = min(m0 + tid, p.M - 1);
@@ -327,7 +332,9 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
             d[3] = (uint32_t)rint_i32((float)bits_to_f16(p.epi.z_row[m]));
             d[4] = (uint32_t)p.epi.rs_row[m] - rxl;
             d[5] = rxl;
+            wide = wide || !(fits_i24(d[3]) && fits_i24(d[4]));
         }
+        if (wide) dwide = 1;  // (same value from every writer)
         // (the barrier that ends the prologue below orders these writes before the epilogue's reads)
     }
 
@@ -497,6 +504,7 @@ __global__ __launch_bounds__(256, 2) void gemm_s4_shortk_kernel(GemmParams p)
     constexpr uint32_t kBuf = BM * kXStride, kStage = 4 * BM * 144;
     __shared__ __attribute__((aligned(16))) uint8_t lds[kBuf > kStage ? kBuf : kStage];
     uint32_t *const dpar = nullptr;  // named by the shared epilogue text for an epilogue this kernel never runs
+    const uint32_t dwide = 0;
 
     if (blockIdx.z) batch_shift(p, blockIdx.z);
     // column blocks fastest: neighbouring workgroups share an activation tile

@@ -273,6 +273,35 @@ def test_gpu_dual_rowsum_dequant(hip, dev, M, N, K, with_bias):
     assert cases.bits_equal(got.cpu().numpy(), want)
 
 
+@pytest.mark.gpu
+def test_gpu_dual_rowsum_wide_factors(hip, dev):
+    """Row-sum terms outside the signed 24-bit range (no genuine layer has them; the arrays are inputs): the fused
+    kernel leaves its 24-bit multiplier path and still gives the oracle's wrapping 32-bit arithmetic, like the
+    stand-alone epilogue."""
+    M, N, K = 128, 4096, 512
+    print("dual rowsum wide factors", M, N, K, flush=True)
+    rng = np.random.default_rng(99)
+    x = cases.acts_uniform(M, K, seed=7)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float16)
+    wq, s1, z1, s2, z2, a1, a2 = orc.weight_asym_dual_shifted_from_linear(w)
+    T = lambda v: cases.t(v, dev)
+    q, s, z, r = hip.quantize_rows_asym_shifted(T(x))
+    acc = hip.matmul(q, T(wq))
+    for which in ("adj", "rowsum"):
+        a1w, a2w, rw = a1.copy(), a2.copy(), r.cpu().numpy().copy()
+        if which == "adj":
+            a1w[5] = 2 ** 30 + 12345
+            a2w[4000] = -(2 ** 29) - 7
+        else:
+            rw[77] = 2 ** 31 - 5
+        want = orc.asym_dual_rowsum_dequant(acc.cpu().numpy(), q.cpu().numpy(), s.cpu().numpy(), z.cpu().numpy(), rw, wq,
+                                            s1, z1, s2, z2, a1w, a2w)
+        got = hip.linear4bit_forward_dual_rowsum(q, s, z, T(rw), T(wq), T(s1), T(z1), T(s2), T(z2), T(a1w), T(a2w))
+        assert cases.bits_equal(got.cpu().numpy(), want), which
+        got = hip.asym_dual_rowsum_dequant(acc, q, s, z, T(rw), T(wq), T(s1), T(z1), T(s2), T(z2), T(a1w), T(a2w))
+        assert cases.bits_equal(got.cpu().numpy(), want), which
+
+
 def test_dual_rowsum_fused_shapes_and_validation():
     """Which shapes the fused entry point runs as one launch (no workspace), and its argument checks."""
     from duqlinear4bitcuda_amd import _lib
