@@ -441,7 +441,7 @@ def quantize_linear4bit_forward(x, w, w_scale_1, w_scale_2=None, bias=None, clip
                                 return_quantized: bool = False, static: bool = False):
     """SymQuantizer + Linear4bitSQ / Linear4bitDUSQ forward (qlinear4bit/nn/quantizer.py:10-16,
     qlinear4bit/nn/linear.py:42-56, 167-176) from binary16 activations ``x`` [..., K]: bit-identical to
-    ``quantize_rows_sym`` followed by ``linear4bit_forward``.  Up to four rows are ONE launch;
+    ``quantize_rows_sym`` followed by ``linear4bit_forward``.  Up to eight rows are ONE launch;
     larger inputs run the two launches with the codes staged in a buffer allocated here.  With
     ``return_quantized`` also returns (codes uint8 [..., K/2], scales [..., 1]).  ``static=True`` stages in the
     library's static device array instead (``duq_quantize_linear4bit_forward_static``: nothing but the outputs is

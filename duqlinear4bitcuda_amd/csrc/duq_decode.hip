@@ -88,7 +88,7 @@ __device__ __forceinline__ uint16_t dequant_rt(int acc, const RowEpi &r, const C
 }
 
 // ---------------------------------------------------------------------------------
-// rows kernel: M <= MR <= 4, K <= XS * 2048
+// rows kernel: M <= MR <= 4 (8 with binary16 activations quantized inside), K <= XS * 2048
 // ---------------------------------------------------------------------------------
 // WAVES wavefronts of R = 16 / WAVES weight rows each: 16 weight rows ("a tile") per workgroup either way.  Eight
 // wavefronts help when the workgroup quantizes four activation rows itself and a CU holds several workgroups
@@ -103,9 +103,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DecodeParams p
     constexpr int LPV = 64 / V;      // lanes that finish one sum: 16, 8 or 4
     constexpr int MODE = EPI < 0 ? 0 : EPI;
     constexpr uint32_t XSTRIDE = XS * 1024;
-    static_assert(MR == 1 || MR == 2 || MR == 4, "rows");
+    static_assert(MR == 1 || MR == 2 || MR == 4 || (MR == 8 && WAVES == 8), "rows");
     static_assert(WAVES == 4 || WAVES == 8, "wavefronts per workgroup");
-    static_assert(V >= 4 && (XS * MR * 4) % WAVES == 0, "partial sums per lane, quantize units per lane");
+    static_assert(V >= 4 && V <= 16 && (XS * MR * 4) % WAVES == 0, "partial sums per lane, quantize units per lane");
     __shared__ __attribute__((aligned(16))) int red[WAVES][V * 64];
     __shared__ __attribute__((aligned(16))) uint8_t xs[FUSEQ ? MR * XSTRIDE : 16];
     __shared__ uint32_t rmax[WAVES];
@@ -426,30 +426,33 @@ void launch_rows_mode(DecodeParams &p, int epi, hipStream_t stream)
     // four; with one workgroup per CU the vector work per SIMD is the same and four wavefronts are ahead,
     // N = 4096: 4.8 against 5.1 us).  On pre-quantized rows, or with one or two rows, several tiles per workgroup
     // measured 3-15 % slower than one (four wavefronts per CU keep too few loads in flight): not used there.
-    constexpr bool kCanMulti = FUSEQ && MR == 4 && XS <= 4;
+    // Eight rows (binary16 in only): always eight wavefronts, one per row in the quantize phase.
+    constexpr bool kCanMulti = FUSEQ && MR >= 4 && XS <= (MR == 4 ? 4 : 2);
     const bool multi = kCanMulti && ntiles > 256;
     p.tiles_per_wg = multi ? (ntiles + 255) / 256 : 1;
     const dim3 grid((ntiles + p.tiles_per_wg - 1) / p.tiles_per_wg);
-    const bool wide = FUSEQ && MR == 4 && !multi && grid.x > 256;
+    const bool wide = MR == 8 || (FUSEQ && MR == 4 && !multi && grid.x > 256);
 #define DUQ_ROWS(E)                                                                                              \
     if (multi) {                                                                                                 \
         if constexpr (kCanMulti)                                                                                 \
             hipLaunchKernelGGL((gemv_s4_rows_kernel<MR, XS, FUSEQ, E, 8, true>), grid, dim3(512), 0, stream, p);     \
-    } else if (wide)                                                                                             \
-        hipLaunchKernelGGL((gemv_s4_rows_kernel<MR, XS, FUSEQ, E, (FUSEQ && MR == 4) ? 8 : 4>), grid, dim3(512), 0,  \
-                           stream, p);                                                                           \
-    else                                                                                                         \
-        hipLaunchKernelGGL((gemv_s4_rows_kernel<MR, XS, FUSEQ, E, 4>), grid, dim3(256), 0, stream, p)
+    } else if (wide) {                                                                                           \
+        if constexpr (FUSEQ && MR >= 4)                                                                          \
+            hipLaunchKernelGGL((gemv_s4_rows_kernel<MR, XS, FUSEQ, E, 8>), grid, dim3(512), 0, stream, p);           \
+    } else {                                                                                                     \
+        if constexpr (MR <= 4)                                                                                   \
+            hipLaunchKernelGGL((gemv_s4_rows_kernel<MR, XS, FUSEQ, E, 4>), grid, dim3(256), 0, stream, p);           \
+    }
     switch (epi) {
-    case 0: DUQ_ROWS(0); break;
-    case 2: DUQ_ROWS(2); break;
+    case 0: DUQ_ROWS(0) break;
+    case 2: DUQ_ROWS(2) break;
     default:
         if constexpr (!FUSEQ) {
             switch (epi) {
-            case -1: DUQ_ROWS(-1); break;
-            case 1: DUQ_ROWS(1); break;
-            case 3: DUQ_ROWS(3); break;
-            case 4: DUQ_ROWS(4); break;
+            case -1: DUQ_ROWS(-1) break;
+            case 1: DUQ_ROWS(1) break;
+            case 3: DUQ_ROWS(3) break;
+            case 4: DUQ_ROWS(4) break;
             }
         }
     }
@@ -462,8 +465,10 @@ void launch_rows_xs(DecodeParams &p, int epi, hipStream_t stream)
     const uint32_t kbytes = p.K / 2;
     if (kbytes <= 2048) launch_rows_mode<MR, 2, FUSEQ>(p, epi, stream);
     else if (kbytes <= 4096) launch_rows_mode<MR, 4, FUSEQ>(p, epi, stream);
-    else if (kbytes <= 6144) launch_rows_mode<MR, 6, FUSEQ>(p, epi, stream);
-    else launch_rows_mode<MR, 8, FUSEQ>(p, epi, stream);
+    else if constexpr (MR <= 4) {  // (eight rows: up to 8192 elements, decode_fp16in_one_launch)
+        if (kbytes <= 6144) launch_rows_mode<MR, 6, FUSEQ>(p, epi, stream);
+        else launch_rows_mode<MR, 8, FUSEQ>(p, epi, stream);
+    }
 }
 
 template <int WAVES, int SEGS, int MT = 1, bool DB = true>
@@ -491,6 +496,10 @@ void launch_decode_any(DecodeParams &p, int epi, hipStream_t stream)
         if (p.M == 1) launch_rows_xs<1, FUSEQ>(p, epi, stream);
         else if (p.M == 2) launch_rows_xs<2, FUSEQ>(p, epi, stream);
         else launch_rows_xs<4, FUSEQ>(p, epi, stream);
+        return;
+    }
+    if constexpr (FUSEQ) {
+        launch_rows_xs<8, true>(p, epi, stream);  // 5..8 rows (decode_fp16in_one_launch admits no others)
         return;
     }
     if constexpr (!FUSEQ) {

@@ -92,12 +92,17 @@ inline bool decode_uses_rows_kernel(uint32_t M) { return M <= 4; }
 // against one tile per workgroup (16 rows, K = 4096): N = 4800 4.96 against 6.54 us, N = 8192 5.67 against 6.89,
 // N = 11008 7.05 against 8.78; 64 rows, N = 11008: 10.95 against 15.7.
 inline uint32_t decode_tiles_per_workgroup(uint32_t ntiles) { return (ntiles + 255) / 256; }
-// quantize + GEMM + dequant from binary16 activations in one launch: shapes of the rows kernel; from two rows on
-// only up to 16384 output columns (every workgroup quantizes the rows again: measured slower than two launches
-// beyond)
+// quantize + GEMM + dequant from binary16 activations in one launch: shapes of the rows kernel, and 5..8 rows
+// of at most 4096 elements, or 8192 on at most 4096 columns (the rows kernel with eight rows, one wavefront
+// quantizing each; measured against quantizer + MFMA decode kernel at 8 rows: N = K = 4096 6.3 against 7.2 us,
+// N = 11008 8.5 against 9.8, K = 2048 4.9 against 6.4, N = K = 8192 16.9 against 13.5); from two rows on only up to
+// 16384 output columns (every workgroup quantizes the rows again: measured slower than two launches beyond)
 inline bool decode_fp16in_one_launch(uint32_t M, uint32_t N, uint32_t K)
 {
-    return select_gemm_kernel(M, N, K) == kKernelDecodeRows && (M == 1 || N <= 16384);
+    const int kernel = select_gemm_kernel(M, N, K);
+    if (kernel == kKernelDecodeRows) return M == 1 || N <= 16384;
+    return M <= 8 && N <= 16384 && (K <= 4096 || (K <= 8192 && N <= 4096)) &&
+           (kernel == kKernelDecodeMfma || kernel == kKernelSkinny);
 }
 // decode kernels (duq_decode.hip); the shape must be one select_gemm_kernel gives to them
 int launch_decode_s4(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N, uint32_t K, int32_t *out_acc,

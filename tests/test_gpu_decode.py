@@ -33,6 +33,8 @@ SHAPES = [(1, 64, 64), (1, 20, 128), (2, 37, 4096), (3, 100, 2048), (4, 4096, 40
           (13, 77, 12288), (8, 50, 2112), (16, 32, 6208),
           (16, 11008, 4096), (6, 8200, 8192), (11, 8192, 2048),
           (12, 40, 16384), (16, 24, 12352),
+          # five to eight rows: from binary16 the rows kernel with eight rows (one launch), pre-quantized the MFMA kernel
+          (5, 4096, 4096), (8, 11008, 4096), (6, 300, 2048), (7, 4100, 8192), (8, 16384, 64), (8, 8200, 8192), (8, 20000, 128),
           # MFMA decode kernel with two to four row tiles (17..64 rows of at most 4096 elements, 17..32 of at most
           # 8192), one to several column tiles per workgroup, tiles that end inside M and N
           (17, 4096, 4096), (32, 300, 4096), (33, 4099, 2048), (48, 1000, 4096), (64, 11008, 4096), (50, 72, 64),
@@ -98,13 +100,13 @@ def test_decode_rowsum_epilogue(hip, dev):
         assert cases.bits_equal(y.cpu().numpy(), want)
 
 
-@pytest.mark.parametrize("M", [1, 2, 4])
+@pytest.mark.parametrize("M", [1, 2, 4, 7])
 def test_fp16_input_special_rows_and_clamps(hip, dev, M):
     """Rows of zeros, with an infinity, with a NaN, with subnormals only, clip 0.9 and both upper clamps: the
     one-launch path gives the stand-alone quantizer's codes and scales and the oracle's outputs."""
     _say("decode special rows", M)
     N, K = 72, 1024
-    x = cases.acts_normal(4, K, seed=5)
+    x = cases.acts_normal(max(M, 4), K, seed=5)
     x[0] = 0
     x[1, 7] = np.inf
     x[2, 100] = np.nan
