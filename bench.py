@@ -163,7 +163,7 @@ def decode_section(dev, quick):
     """HBM-bound decode at configuration 2 and around it.  Per shape, HIP-graph timed, with the weights rotated
     over more than 512 MB of distinct buffers so that no launch finds its weights in a cache:
       us            binary16 activations in -> per-token quantize -> GEMM -> fp16 out, the single entry point
-                    (one launch up to four rows, quantizer + GEMM launches above)
+                    (one launch up to eight rows, quantizer + GEMM launches above)
       gemm_only_us  the GEMM + dequant launch alone on pre-quantized activations
       read_floor_us a kernel that only reads the same N*K/2 weight bytes with the decode access pattern
     GBps / frac_hbm use `us` and the algorithmic bytes 2MK + NK/2 + 2N + 2MN."""
@@ -174,7 +174,7 @@ def decode_section(dev, quick):
     out = []
     shapes = list(LLAMA7B_DECODE)
     if not quick:
-        shapes += [(32, 4096, 4096), (64, 11008, 4096), (1, 4096, 11008), (16, 4096, 11008), (1, 28672, 8192),
+        shapes += [(8, 4096, 4096), (32, 4096, 4096), (64, 11008, 4096), (1, 4096, 11008), (16, 4096, 11008), (1, 28672, 8192),
                    (1, 8192, 28672), (16, 28672, 8192)]
     for (M, N, K) in shapes:
         wbytes = N * K // 2
@@ -547,7 +547,7 @@ def main():
                                PREWARM_STEPS + args.warmup)
     i8_quant_us = graph_time_us([lambda: hip.quantize_rows_sym(x)] * 40)
     integer_path = {"ms_per_step": round(i8_ms_per_step, 5), "TOPS": round(ops / (i8_ms_per_step * 1e-3) / 1e12, 2),
-                    "kernel": "gemm_s4_stream_kernel<4,0,false> (v_mfma_i32_32x32x32_i8)", "gemm_fused_us": round(i8_gemm_us, 2),
+                    "kernel": "gemm_s4_stream_kernel<4,0,false,2> (v_mfma_i32_32x32x32_i8, 128 x 256 tiles)", "gemm_fused_us": round(i8_gemm_us, 2),
                     "quantize_rows_sym_us": round(i8_quant_us, 2),
                     "roofline": {"bound": "mfma", "achieved": round(ops / i8_gemm_us / 1e6, 1), "peak": PEAK_INT8_TOPS,
                                  "unit": "TOP/s", "frac": round(ops / i8_gemm_us / 1e6 / PEAK_INT8_TOPS, 4),
@@ -563,8 +563,8 @@ def main():
     batched = batched_section(dev, args.quick)
     rows_7b = [d for d in decode if (d["M"], d["N"], d["K"]) in LLAMA7B_DECODE]
     worst = min(rows_7b, key=lambda d: d["frac_hbm"])
-    roofline_decode = {"bound": "hbm", "kernel": "decode_rows_kernel (M <= 4, quantizer inside) / quantize_rows_kernel + "
-                                                 "decode_mfma_kernel or gemm_s4_skinny_kernel (M <= 16)",
+    roofline_decode = {"bound": "hbm", "kernel": "gemv_s4_rows_kernel (M <= 8, quantizer inside) / quantize_rows_kernel + "
+                                                 "gemm_s4_decode_kernel (M <= 64)",
                        "what": "worst of the Llama-2-7B decode rows (M in {1,4,16}, K=4096, N in {4096,11008}), binary16 "
                                "activations in, quantize + GEMM + dequant, weights never in a cache",
                        "achieved": worst["GBps"], "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": worst["frac_hbm"],
@@ -572,7 +572,7 @@ def main():
                        "best_7b_frac": max(d["frac_hbm"] for d in rows_7b),
                        "read_floor_frac": round(worst["read_floor_GBps"] / PEAK_HBM_GBS, 4),
                        # the GEMM launch of that row (the quantizer launch of 16 rows before it moves 0.2 MB)
-                       "traffic": profile_shape_traffic_bytes("decode_kernels__bench_shapes.txt", "gemm_s4_decode_kernel<8, 4, 0>", 256)
+                       "traffic": profile_shape_traffic_bytes("decode_kernels__bench_shapes.txt", "gemm_s4_decode_kernel<8, 4, 0, 1,", 256)
                        if (worst["M"], worst["N"]) == (16, 4096) else None,
                        "traffic_source": "profiles/decode_kernels__bench_shapes.txt"}
 
