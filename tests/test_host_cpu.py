@@ -174,6 +174,24 @@ def test_bench_refuses_more_than_one_gpu():
     assert "ONE GPU" in r.stderr
 
 
+def test_bench_finds_its_traffic_figures_in_the_profiles():
+    """bench.py reads the HBM traffic of its roofline kernels from the committed rocprofv3 summaries by kernel
+    name: the names it looks for must be the ones the summaries hold."""
+    import re
+
+    sys.path.insert(0, ROOT)
+    import bench
+
+    src = open(os.path.join(ROOT, "bench.py")).read()
+    calls = re.findall(r'profile_traffic_bytes\(\s*"([^"]+)",\s*"([^"]+)"\)', src)
+    shaped = re.findall(r'profile_shape_traffic_bytes\(\s*"([^"]+)",\s*"([^"]+)",\s*(\d+)\)', src)
+    assert len(calls) >= 2 and len(shaped) >= 1
+    for name, kernel in calls:
+        assert bench.profile_traffic_bytes(name, kernel), (name, kernel)
+    for name, kernel, wgs in shaped:
+        assert bench.profile_shape_traffic_bytes(name, kernel, int(wgs)), (name, kernel, wgs)
+
+
 def test_reference_package_name_is_importable():
     import qlinear4bit._CUDA as ops
     import qlinear4bit.nn as rnn
