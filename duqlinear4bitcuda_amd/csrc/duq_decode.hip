@@ -145,6 +145,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DecodeParams p
             raw[j] = buf_load16(rX, c < nunits ? (qrow * p.K + c * 8) * 2 : kOobOffset, 0);
         }
     }
+    // Eight wavefronts that quantize: all of them request their activations before any requests weights (the CU
+    // serves requests in order, and a wavefront whose activations queue behind another's weights holds up the
+    // whole workgroup at the staging barrier below; measured at 8 rows, K = 4096: N = 4096 5.6 against 6.2 us,
+    // N = 11008 8.2 against 8.5; with four wavefronts it changes nothing)
+    if (FUSEQ && WAVES == 8) __builtin_amdgcn_s_barrier();
     const __amdgpu_buffer_rsrc_t rW = make_rsrc(p.B, p.N * kbytes);
     // the weights of tile t for this wavefront (tiles past the workgroup's last read as zero, unused)
     auto load_w = [&](uint32_t tile, v4u(&w)[R][XS]) {
