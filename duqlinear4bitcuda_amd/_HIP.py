@@ -438,14 +438,14 @@ def probe_read(t: torch.Tensor):
 
 
 def quantize_linear4bit_forward(x, w, w_scale_1, w_scale_2=None, bias=None, clip: float = 1.0, qmax: int = 6,
-                                return_quantized: bool = False, static: bool = False):
+                                return_quantized: bool = False, static: bool = False, slot: int = 0):
     """SymQuantizer + Linear4bitSQ / Linear4bitDUSQ forward (qlinear4bit/nn/quantizer.py:10-16,
     qlinear4bit/nn/linear.py:42-56, 167-176) from binary16 activations ``x`` [..., K]: bit-identical to
     ``quantize_rows_sym`` followed by ``linear4bit_forward``.  Up to eight rows are ONE launch;
     larger inputs run the two launches with the codes staged in a buffer allocated here.  With
     ``return_quantized`` also returns (codes uint8 [..., K/2], scales [..., 1]).  ``static=True`` stages in the
     library's static device array instead (``duq_quantize_linear4bit_forward_static``: nothing but the outputs is
-    allocated; calls that overlap on one GPU race on the array, and M * K / 2 <= 8 MiB)."""
+    allocated; M * K / 2 <= 8 MiB; calls that may overlap on one GPU must name different ``slot``s, 0..3)."""
     name = "quantize_linear4bit_forward"
     if not isinstance(x, torch.Tensor) or not isinstance(w, torch.Tensor):
         raise RuntimeError(f"{name}: x and w must be tensors")
@@ -476,7 +476,7 @@ def quantize_linear4bit_forward(x, w, w_scale_1, w_scale_2=None, bias=None, clip
     mode = EPI_SYM if w_scale_2 is None else EPI_SYM_DUAL
     if static:
         st = _launch(dev, lib.duq_quantize_linear4bit_forward_static, mode, x.data_ptr(), float(clip), qmax, w.data_ptr(),
-                     ptrs[0] or None, ptrs[1] or None, ptrs[2] or None, M, N, K, y.data_ptr(), _ptr(q), _ptr(s))
+                     ptrs[0] or None, ptrs[1] or None, ptrs[2] or None, M, N, K, y.data_ptr(), _ptr(q), _ptr(s), slot)
         if st:
             _lib.check(st, name)
         return (y, q, s) if return_quantized else y
@@ -490,6 +490,143 @@ def quantize_linear4bit_forward(x, w, w_scale_1, w_scale_2=None, bias=None, clip
     if st:
         _lib.check(st, name)
     return (y, q, s) if return_quantized else y
+
+
+def quantize_linear4bit_forward_asym(mode, x, w, w_scale_1, w_zeros_1, w_scale_2=None, w_zeros_2=None,
+                                     w_rowsum_adj=None, bias=None, return_quantized: bool = False):
+    """AsymQuantizer + Linear4bitASQ / LinearQuant4bitDUASQ forward (qlinear4bit/nn/quantizer.py:24-35,
+    qlinear4bit/nn/linear.py:104-115, 239-250) from binary16 activations ``x`` [..., K], and the row-sum layer's
+    (``mode`` EPI_ASYM_ROWSUM with ``w_rowsum_adj``: the signed-shifted quantizer): bit-identical to
+    ``quantize_rows_asym`` (``quantize_rows_asym_shifted``) followed by ``linear4bit_forward``
+    (``linear4bit_forward_rowsum``).  Up to eight rows are ONE launch; larger inputs run the two launches with the
+    codes staged in a buffer allocated here.  With ``return_quantized`` also returns (codes, scales [..., 1],
+    zeros [..., 1][, rowsum [...]])."""
+    name = "quantize_linear4bit_forward_asym"
+    if mode not in (EPI_ASYM, EPI_ASYM_DUAL, EPI_ASYM_ROWSUM):
+        raise RuntimeError(f"{name}: mode must be EPI_ASYM, EPI_ASYM_DUAL or EPI_ASYM_ROWSUM")
+    if not isinstance(x, torch.Tensor) or not isinstance(w, torch.Tensor):
+        raise RuntimeError(f"{name}: x and w must be tensors")
+    dev = x.device
+    _fast_check(name, "x", x, _F16, None)
+    _fast_check(name, "w", w, _U8, dev)
+    K = x.shape[-1]
+    if w.dim() != 2 or w.shape[1] * 2 != K:
+        raise RuntimeError(f"{name}: K differs: x {tuple(x.shape)} vs packed w {tuple(w.shape)}")
+    M = x.numel() // K if K else 0
+    N = w.shape[0]
+    ptrs = []
+    for t, what, dt in ((w_scale_1, "w_scale_1", _F16), (w_zeros_1, "w_zeros_1", _F16), (w_scale_2, "w_scale_2", _F16),
+                        (w_zeros_2, "w_zeros_2", _F16), (w_rowsum_adj, "w_rowsum_adj", _I32), (bias, "bias", _F16)):
+        if t is None:
+            ptrs.append(None)
+            continue
+        _fast_check(name, what, t, dt, dev)
+        if t.numel() != N:
+            _check_size0(name, t.reshape(-1), what, N)
+        ptrs.append(t.data_ptr())
+    lead = x.shape[:-1]
+    y = torch.empty(lead + (N,), dtype=_F16, device=dev)
+    q = s = z = r = None
+    rowsum = mode == EPI_ASYM_ROWSUM
+    if return_quantized:
+        q = torch.empty(lead + (K // 2,), dtype=_U8, device=dev)
+        s = torch.empty(lead + (1,), dtype=_F16, device=dev)
+        z = torch.empty(lead + (1,), dtype=_F16, device=dev)
+        r = torch.empty(lead, dtype=_I32, device=dev) if rowsum else None
+    lib = _lib.load()
+    ws, ws_bytes = None, 0
+    if not return_quantized:
+        ws_bytes = lib.duq_quantize_linear4bit_asym_workspace_bytes(mode, M, N, K)
+        if ws_bytes:
+            ws = torch.empty(ws_bytes, dtype=_U8, device=dev)
+    st = _launch(dev, lib.duq_quantize_linear4bit_forward_asym, mode, x.data_ptr(), w.data_ptr(), *ptrs, M, N, K,
+                 y.data_ptr(), _ptr(q), _ptr(s), _ptr(z), _ptr(r), _ptr(ws), ws_bytes)
+    if st:
+        _lib.check(st, name)
+    if not return_quantized:
+        return y
+    return (y, q, s, z, r) if rowsum else (y, q, s, z)
+
+
+class FusedDecode:
+    """One layer's arguments for the one-launch entry points (``duq_quantize_linear4bit_forward`` for the symmetric
+    modes, ``duq_quantize_linear4bit_forward_asym`` for EPI_ASYM / EPI_ASYM_DUAL / EPI_ASYM_ROWSUM), checked once
+    and kept as a prepared argument list, so that a decode step of a module costs one ``torch.empty`` and one
+    foreign call.  The tensors are held (``tensors``) so that a caller can tell when the layer's buffers were
+    replaced; a change of their contents in place needs no new object."""
+
+    __slots__ = ("mode", "N", "K", "device", "index", "tensors", "w_ptr", "_fn", "_head", "_tail", "_one", "_lib")
+
+    def __init__(self, mode, w, w_scale_1, w_zeros_1=None, w_scale_2=None, w_zeros_2=None, w_rowsum_adj=None, bias=None):
+        name = "FusedDecode"
+        if not isinstance(w, torch.Tensor):
+            raise RuntimeError(f"{name}: w must be a tensor")
+        _fast_check(name, "w", w, _U8, None)
+        if w.dim() != 2:
+            raise RuntimeError(f"{name}: expected w [N, K/2], got {tuple(w.shape)}")
+        dev = w.device
+        N, K = w.shape[0], w.shape[1] * 2
+        asym = mode in (EPI_ASYM, EPI_ASYM_DUAL, EPI_ASYM_ROWSUM)
+        dual = mode in (EPI_SYM_DUAL, EPI_ASYM_DUAL)
+        if mode not in (EPI_SYM, EPI_SYM_DUAL) and not asym:
+            raise RuntimeError(f"{name}: unknown mode {mode}")
+        need = {"w_scale_1": True, "w_zeros_1": asym, "w_scale_2": dual, "w_zeros_2": asym and dual,
+                "w_rowsum_adj": mode == EPI_ASYM_ROWSUM, "bias": False}
+        ptrs = {}
+        for t, what, dt in ((w_scale_1, "w_scale_1", _F16), (w_zeros_1, "w_zeros_1", _F16), (w_scale_2, "w_scale_2", _F16),
+                            (w_zeros_2, "w_zeros_2", _F16), (w_rowsum_adj, "w_rowsum_adj", _I32), (bias, "bias", _F16)):
+            if t is None:
+                if need[what]:
+                    raise RuntimeError(f"{name}: {what} is required for mode {mode}")
+                ptrs[what] = None
+                continue
+            _fast_check(name, what, t, dt, dev)
+            if t.numel() != N:
+                _check_size0(name, t.reshape(-1), what, N)
+            ptrs[what] = t.data_ptr()
+        self.mode, self.N, self.K, self.device, self.index = mode, N, K, dev, dev.index
+        self.tensors = (w, w_scale_1, w_zeros_1, w_scale_2, w_zeros_2, w_rowsum_adj, bias)
+        self.w_ptr = w.data_ptr()
+        lib = self._lib = _lib.load()
+        if asym:
+            self._fn = lib.duq_quantize_linear4bit_forward_asym
+            self._head = (w.data_ptr(), ptrs["w_scale_1"], ptrs["w_zeros_1"], ptrs["w_scale_2"], ptrs["w_zeros_2"],
+                          ptrs["w_rowsum_adj"], ptrs["bias"])
+            self._tail = (None, None, None, None, None, 0)   # q_out, scale_out, zeros_out, rowsum_out, workspace, bytes
+        else:
+            self._fn = lib.duq_quantize_linear4bit_forward
+            self._head = (w.data_ptr(), ptrs["w_scale_1"], ptrs["w_scale_2"], ptrs["bias"])
+            self._tail = (None, None, None, 0)               # q_out, scale_out, workspace, bytes
+        self._one = {}
+
+    def admits(self, M: int) -> bool:
+        """True when M rows of this layer run as ONE launch with nothing staged."""
+        one = self._one.get(M)
+        if one is None:
+            one = self._one[M] = M > 0 and self._lib.duq_quantize_linear4bit_workspace_bytes(M, self.N, self.K) == 0
+        return one
+
+    def run(self, x: torch.Tensor, M: int, clip: float = 1.0, qmax: int = 6) -> torch.Tensor:
+        """x: contiguous binary16 [..., K] on the layer's device, 16-byte aligned, M = its rows with admits(M);
+        clip / qmax: the symmetric quantizer's settings (unused by the asymmetric modes).  Returns binary16
+        [..., N]."""
+        if x.dtype is not _F16 or not x.is_contiguous() or x.shape[-1] != self.K or x.device != self.device:
+            raise RuntimeError(f"FusedDecode: expected a contiguous float16 tensor [..., {self.K}] on {self.device}, got "
+                               f"{x.dtype} {tuple(x.shape)} on {x.device}")
+        y = torch.empty(x.shape[:-1] + (self.N,), dtype=_F16, device=self.device)
+        idx = self.index
+        if self.mode == EPI_SYM or self.mode == EPI_SYM_DUAL:
+            args = (self.mode, x.data_ptr(), clip, qmax, *self._head, M, self.N, self.K, y.data_ptr(), *self._tail)
+        else:
+            args = (self.mode, x.data_ptr(), *self._head, M, self.N, self.K, y.data_ptr(), *self._tail)
+        if idx == torch._C._cuda_getDevice():
+            st = self._fn(*args, _raw_stream(idx))
+        else:
+            with torch.cuda.device(idx):
+                st = self._fn(*args, _raw_stream(idx))
+        if st:
+            _lib.check(st, "quantize_linear4bit_forward")
+        return y
 
 
 # ---- asymmetric path with exact zero-point correction (row sums); not in the reference ----

@@ -1,37 +1,50 @@
 // extern "C" boundary of libduq_hip.so: argument validation, then the launchers.
 // Nothing here allocates, synchronises or throws; the only state is the per-device address of the static
 // scratch array of duq_quantize_linear4bit_forward_static.
-#include <mutex>
+#include <atomic>
 
 #include "../../include/duq_hip.h"
 #include "duq_launch.h"
 
-// Scratch of duq_quantize_linear4bit_forward_static: the packed codes [M, K/2] and then the per-token scales [M]
-// that its quantizer launch hands to its GEMM launch.  Every GPU the library runs on holds its own copy of the
-// array until the process ends.  In host code the name is only a handle for hipGetSymbolAddress: kernels and
-// copies get the device address that static_scratch() looks up once per device.
-static __device__ __align__(256) unsigned char scratch[DUQ_STATIC_SCRATCH_CODE_BYTES + DUQ_STATIC_SCRATCH_ROWS * 2];
+// Scratch of duq_quantize_linear4bit_forward_static: DUQ_STATIC_SCRATCH_SLOTS slots, each the packed codes
+// [M, K/2] and then the per-token scales [M] that the call's quantizer launch hands to its GEMM launch.  Every GPU
+// the library runs on holds its own copy of the array until the process ends.  In host code the name is only a
+// handle for hipGetSymbolAddress: kernels and copies get the device address that static_scratch() looks up once per
+// device.
+constexpr uint64_t kSlotBytes = (uint64_t)DUQ_STATIC_SCRATCH_CODE_BYTES + DUQ_STATIC_SCRATCH_ROWS * 2;
+static __device__ __align__(256) unsigned char scratch[DUQ_STATIC_SCRATCH_SLOTS * kSlotBytes];
 
 namespace {
 
 constexpr int kMaxDevices = 64;
-std::mutex g_scratch_mutex;
-void *g_scratch_ptr[kMaxDevices];  // device address of `scratch` on device i, 0 until first use there
+std::atomic<void *> g_scratch_ptr[kMaxDevices];  // device address of `scratch` on device i, null until first use there
 
-// Address of the current device's copy of `scratch` (looked up on the first call per device).
-int static_scratch(unsigned char **out)
+// Address of `scratch` on the device of `stream`, which must be the current device (the lookup and the launches
+// that follow act on the current device).  The first call per device asks the runtime, which a stream under
+// capture may not do: such a call is refused instead (call duq_static_scratch_init first).  Later calls read one
+// atomic pointer.  Two threads that race on the first call both look the address up and store the same value.
+int static_scratch(hipStream_t stream, unsigned char **out)
 {
     int dev = -1;
     if (hipError_t e = hipGetDevice(&dev)) return static_cast<int>(e);
     if (dev < 0 || dev >= kMaxDevices) return static_cast<int>(hipErrorInvalidDevice);
-    std::lock_guard<std::mutex> lock(g_scratch_mutex);
-    if (!g_scratch_ptr[dev]) {
-        void *p = nullptr;
+    if (stream) {
+        hipDevice_t sdev = -1;
+        if (hipError_t e = hipStreamGetDevice(stream, &sdev)) return static_cast<int>(e);
+        if (static_cast<int>(sdev) != dev) return DUQ_E_DEVICE;
+    }
+    void *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        if (stream) {
+            hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+            if (hipError_t e = hipStreamIsCapturing(stream, &cap)) return static_cast<int>(e);
+            if (cap != hipStreamCaptureStatusNone) return DUQ_E_CAPTURE;
+        }
         if (hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch))) return static_cast<int>(e);
         if (!p) return static_cast<int>(hipErrorInvalidSymbol);
-        g_scratch_ptr[dev] = p;
+        g_scratch_ptr[dev].store(p, std::memory_order_release);
     }
-    *out = static_cast<unsigned char *>(g_scratch_ptr[dev]);
+    *out = static_cast<unsigned char *>(p);
     return DUQ_OK;
 }
 
@@ -60,38 +73,73 @@ int check_gemm(const void *A, const void *B, uint32_t M, uint32_t N, uint32_t K)
 }
 
 // quantize + GEMM + dequant from binary16 activations: one launch for decode shapes, otherwise the quantizer
-// into `workspace` (codes, then scales) followed by the GEMM
-int quantize_linear_impl(int32_t mode, const duq_half *x, float clip, int32_t qmax, const uint8_t *w,
-                         const duq_half *w_scale_1, const duq_half *w_scale_2, const duq_half *bias, uint32_t M,
-                         uint32_t N, uint32_t K, duq_half *y, uint8_t *q_out, duq_half *scale_out, void *workspace,
-                         uint64_t workspace_bytes, duq_stream_t stream)
+// into `workspace` (codes, scales, then zero points and row sums for the asymmetric modes) followed by the GEMM.
+// The epilogue mode decides the quantizer: symmetric for DUQ_EPI_SYM / SYM_DUAL, asymmetric for DUQ_EPI_ASYM /
+// ASYM_DUAL, its signed-shifted form for DUQ_EPI_ASYM_ROWSUM.
+struct FusedOut {
+    uint8_t *q;
+    duq_half *scale, *zeros;
+    int32_t *rowsum;
+};
+
+inline uint64_t up16(uint64_t v) { return (v + 15) & ~(uint64_t)15; }
+
+uint64_t staging_bytes(int32_t mode, uint32_t M, uint32_t K)
 {
-    if (mode != DUQ_EPI_SYM && mode != DUQ_EPI_SYM_DUAL) return DUQ_E_MODE;
-    if (int e = check_qmax(qmax)) return e;
+    uint64_t b = up16((uint64_t)M * (K / 2)) + up16((uint64_t)M * 2);
+    if (mode == DUQ_EPI_ASYM || mode == DUQ_EPI_ASYM_DUAL || mode == DUQ_EPI_ASYM_ROWSUM) b += up16((uint64_t)M * 2);
+    if (mode == DUQ_EPI_ASYM_ROWSUM) b += up16((uint64_t)M * 4);
+    return b;
+}
+
+int quantize_linear_impl(duq::Epilogue e, const duq_half *x, float clip, int32_t qmax, const uint8_t *w, uint32_t M,
+                         uint32_t N, uint32_t K, duq_half *y, FusedOut out, void *workspace, uint64_t workspace_bytes,
+                         duq_stream_t stream)
+{
+    const int32_t mode = e.mode;
+    const bool asym = mode == DUQ_EPI_ASYM || mode == DUQ_EPI_ASYM_DUAL || mode == DUQ_EPI_ASYM_ROWSUM;
+    const bool dual = mode == DUQ_EPI_SYM_DUAL || mode == DUQ_EPI_ASYM_DUAL;
+    const bool rowsum = mode == DUQ_EPI_ASYM_ROWSUM;
+    if (mode < DUQ_EPI_SYM || mode > DUQ_EPI_ASYM_ROWSUM) return DUQ_E_MODE;
+    if (int st = check_qmax(qmax)) return st;
     if (M == 0 || N == 0) return DUQ_OK;
     if (!x) return DUQ_E_NULL;
-    if (int e = check_gemm(x, w, M, N, K)) return e;
+    if (int st = check_gemm(x, w, M, N, K)) return st;
     if (K == 0) return DUQ_E_KALIGN;
-    if (!w_scale_1 || !y) return DUQ_E_NULL;
-    if (mode == DUQ_EPI_SYM_DUAL && !w_scale_2) return DUQ_E_NULL;
-    if ((q_out && !aligned(q_out, 16))) return DUQ_E_ALIGN;
-    duq::Epilogue e{mode, nullptr, nullptr, w_scale_1, nullptr, w_scale_2, nullptr, bias, nullptr, nullptr};
+    if (!e.s_col_1 || !y) return DUQ_E_NULL;
+    if (asym && !e.z_col_1) return DUQ_E_NULL;
+    if (dual && (!e.s_col_2 || (asym && !e.z_col_2))) return DUQ_E_NULL;
+    if (rowsum && !e.rs_col) return DUQ_E_NULL;
+    if ((out.q && !aligned(out.q, 16))) return DUQ_E_ALIGN;
     if (duq::decode_fp16in_one_launch(M, N, K))
-        return duq::launch_decode_fp16in(x, clip, qmax, w, M, N, K, e, y, q_out, scale_out, as_stream(stream));
-    // two launches: the codes and scales go to the caller's outputs when given, else to the workspace
-    const uint64_t code_bytes = ((uint64_t)M * (K / 2) + 15) & ~(uint64_t)15;
-    uint8_t *q = q_out;
-    duq_half *s = scale_out;
-    if (!q || !s) {
+        return duq::launch_decode_fp16in(x, clip, qmax, w, M, N, K, e, y, out.q, out.scale, asym ? out.zeros : nullptr,
+                                         rowsum ? out.rowsum : nullptr, as_stream(stream));
+    // two launches: codes and per-token parameters go to the caller's outputs where given, else to the workspace
+    const bool need_ws = !out.q || !out.scale || (asym && !out.zeros) || (rowsum && !out.rowsum);
+    if (need_ws) {
         if (!workspace) return DUQ_E_NULL;
         if (!aligned(workspace, 16)) return DUQ_E_ALIGN;
-        if (workspace_bytes < code_bytes + (((uint64_t)M * 2 + 15) & ~(uint64_t)15)) return DUQ_E_SHAPE;
-        if (!q) q = static_cast<uint8_t *>(workspace);
-        if (!s) s = reinterpret_cast<duq_half *>(static_cast<uint8_t *>(workspace) + code_bytes);
+        if (workspace_bytes < staging_bytes(mode, M, K)) return DUQ_E_SHAPE;
+        uint8_t *at = static_cast<uint8_t *>(workspace);
+        if (!out.q) out.q = at;
+        at += up16((uint64_t)M * (K / 2));
+        if (!out.scale) out.scale = reinterpret_cast<duq_half *>(at);
+        at += up16((uint64_t)M * 2);
+        if (asym && !out.zeros) out.zeros = reinterpret_cast<duq_half *>(at);
+        at += up16((uint64_t)M * 2);
+        if (rowsum && !out.rowsum) out.rowsum = reinterpret_cast<int32_t *>(at);
     }
-    if (int st = duq::launch_quantize_rows_sym(x, M, K, clip, qmax, q, s, nullptr, as_stream(stream))) return st;
-    e.s_row = s;
-    return duq::launch_gemm_s4(q, w, M, N, K, nullptr, &e, y, as_stream(stream));
+    int st;
+    if (!asym)
+        st = duq::launch_quantize_rows_sym(x, M, K, clip, qmax, out.q, out.scale, nullptr, as_stream(stream));
+    else
+        st = duq::launch_quantize_rows_asym(x, M, K, out.q, out.scale, out.zeros, rowsum ? out.rowsum : nullptr, nullptr,
+                                            as_stream(stream));
+    if (st) return st;
+    e.s_row = out.scale;
+    e.z_row = asym ? out.zeros : nullptr;
+    e.rs_row = rowsum ? out.rowsum : nullptr;
+    return duq::launch_gemm_s4(out.q, w, M, N, K, nullptr, &e, y, as_stream(stream));
 }
 
 }  // namespace
@@ -111,7 +159,10 @@ const char *duq_status_string(int status)
     case DUQ_E_ALIGN: return "pointer alignment requirement not met";
     case DUQ_E_TOO_LARGE: return "dimension too large";
     case DUQ_E_SCRATCH:
-        return "input exceeds the static scratch buffer (M * K / 2 <= 8 MiB of packed codes and M <= 32768 rows)";
+        return "input exceeds a slot of the static scratch buffer (M * K / 2 <= 8 MiB of packed codes and M <= 32768 rows), or no such slot";
+    case DUQ_E_DEVICE: return "the stream belongs to another device than the current one";
+    case DUQ_E_CAPTURE:
+        return "first use of the static scratch buffer on this device under stream capture: call duq_static_scratch_init() before capturing";
     default: break;
     }
     if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));
@@ -360,7 +411,7 @@ uint64_t duq_quantize_linear4bit_workspace_bytes(uint32_t M, uint32_t N, uint32_
     if (M == 0 || N == 0 || K == 0) return 0;
     if (duq::decode_fp16in_one_launch(M, N, K)) return 0;  // nothing staged
     // packed codes [M, K/2] (rounded up to 16 bytes so that the scales stay aligned), then the scales [M]
-    return (((uint64_t)M * (K / 2) + 15) & ~(uint64_t)15) + (((uint64_t)M * 2 + 15) & ~(uint64_t)15);
+    return staging_bytes(DUQ_EPI_SYM, M, K);
 }
 
 int duq_quantize_linear4bit_forward(int32_t mode, const duq_half *x, float clip, int32_t qmax, const uint8_t *w,
@@ -369,30 +420,62 @@ int duq_quantize_linear4bit_forward(int32_t mode, const duq_half *x, float clip,
                                     duq_half *scale_out, void *workspace, uint64_t workspace_bytes,
                                     duq_stream_t stream)
 {
-    return quantize_linear_impl(mode, x, clip, qmax, w, w_scale_1, w_scale_2, bias, M, N, K, y, q_out, scale_out,
+    if (mode != DUQ_EPI_SYM && mode != DUQ_EPI_SYM_DUAL) return DUQ_E_MODE;
+    duq::Epilogue e{mode, nullptr, nullptr, w_scale_1, nullptr, w_scale_2, nullptr, bias, nullptr, nullptr};
+    return quantize_linear_impl(e, x, clip, qmax, w, M, N, K, y, FusedOut{q_out, scale_out, nullptr, nullptr}, workspace,
+                                workspace_bytes, stream);
+}
+
+uint64_t duq_quantize_linear4bit_asym_workspace_bytes(int32_t mode, uint32_t M, uint32_t N, uint32_t K)
+{
+    if (M == 0 || N == 0 || K == 0) return 0;
+    if (mode != DUQ_EPI_ASYM && mode != DUQ_EPI_ASYM_DUAL && mode != DUQ_EPI_ASYM_ROWSUM) return 0;
+    if (duq::decode_fp16in_one_launch(M, N, K)) return 0;
+    return staging_bytes(mode, M, K);
+}
+
+int duq_quantize_linear4bit_forward_asym(int32_t mode, const duq_half *x, const uint8_t *w, const duq_half *w_scale_1,
+                                         const duq_half *w_zeros_1, const duq_half *w_scale_2,
+                                         const duq_half *w_zeros_2, const int32_t *w_rowsum_adj, const duq_half *bias,
+                                         uint32_t M, uint32_t N, uint32_t K, duq_half *y, uint8_t *q_out,
+                                         duq_half *scale_out, duq_half *zeros_out, int32_t *rowsum_out, void *workspace,
+                                         uint64_t workspace_bytes, duq_stream_t stream)
+{
+    if (mode != DUQ_EPI_ASYM && mode != DUQ_EPI_ASYM_DUAL && mode != DUQ_EPI_ASYM_ROWSUM) return DUQ_E_MODE;
+    duq::Epilogue e{mode, nullptr, nullptr, w_scale_1, w_zeros_1, w_scale_2, w_zeros_2, bias, nullptr, w_rowsum_adj};
+    return quantize_linear_impl(e, x, 1.0f, DUQ_QMAX_SYM_DEVICE, w, M, N, K, y, FusedOut{q_out, scale_out, zeros_out, rowsum_out},
                                 workspace, workspace_bytes, stream);
+}
+
+int duq_static_scratch_init(void)
+{
+    unsigned char *p = nullptr;
+    return static_scratch(nullptr, &p);
 }
 
 int duq_quantize_linear4bit_forward_static(int32_t mode, const duq_half *x, float clip, int32_t qmax, const uint8_t *w,
                                            const duq_half *w_scale_1, const duq_half *w_scale_2, const duq_half *bias,
                                            uint32_t M, uint32_t N, uint32_t K, duq_half *y, uint8_t *q_out,
-                                           duq_half *scale_out, duq_stream_t stream)
+                                           duq_half *scale_out, uint32_t slot, duq_stream_t stream)
 {
     // Same work as duq_quantize_linear4bit_forward with the staging buffer taken from `scratch`.  The size is
     // checked first, for every shape, so that what a caller may pass does not depend on the launch plan.
+    if (mode != DUQ_EPI_SYM && mode != DUQ_EPI_SYM_DUAL) return DUQ_E_MODE;
+    if (slot >= DUQ_STATIC_SCRATCH_SLOTS) return DUQ_E_SCRATCH;
     if ((uint64_t)M * (K / 2) > DUQ_STATIC_SCRATCH_CODE_BYTES || M > DUQ_STATIC_SCRATCH_ROWS) return DUQ_E_SCRATCH;
     uint8_t *q = q_out;
     duq_half *sc = scale_out;
     const bool staged = M != 0 && N != 0 && K != 0 && !duq::decode_fp16in_one_launch(M, N, K) && (!q_out || !scale_out);
     if (staged) {
         unsigned char *ws = nullptr;
-        if (int e = static_scratch(&ws)) return e;
-        // codes at the start, scales behind the largest code block: both offsets keep the 256-byte alignment
+        if (int e = static_scratch(as_stream(stream), &ws)) return e;
+        ws += (uint64_t)slot * kSlotBytes;
+        // codes at the start of the slot, scales behind the largest code block: both offsets keep the 256-byte alignment
         if (!q) q = ws;
         if (!sc) sc = reinterpret_cast<duq_half *>(ws + DUQ_STATIC_SCRATCH_CODE_BYTES);
     }
-    return quantize_linear_impl(mode, x, clip, qmax, w, w_scale_1, w_scale_2, bias, M, N, K, y, q, sc, nullptr, 0,
-                                stream);
+    duq::Epilogue e{mode, nullptr, nullptr, w_scale_1, nullptr, w_scale_2, nullptr, bias, nullptr, nullptr};
+    return quantize_linear_impl(e, x, clip, qmax, w, M, N, K, y, FusedOut{q, sc, nullptr, nullptr}, nullptr, 0, stream);
 }
 
 int duq_asym_rowsum_dequant_host(const int32_t *q, const duq_half *scale_row, const duq_half *zeros_row,

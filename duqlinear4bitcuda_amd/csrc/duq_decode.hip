@@ -53,6 +53,8 @@ struct DecodeParams {
     int qmax;            // FUSEQ
     uint8_t *q_out;      // FUSEQ, optional: the packed codes [M, K/2] (written by workgroup 0)
     uint16_t *s_out;     // FUSEQ, optional: the per-token scales [M]
+    uint16_t *z_out;     // FUSEQ with an asymmetric epilogue, optional: the per-token zero points [M]
+    int32_t *rs_out;     // FUSEQ with the row-sum epilogue, optional: the per-token sums of the shifted codes [M]
     uint32_t tiles_per_wg;
 };
 
@@ -109,7 +111,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DecodeParams p
     __shared__ __attribute__((aligned(16))) int red[WAVES][V * 64];
     __shared__ __attribute__((aligned(16))) uint8_t xs[FUSEQ ? MR * XSTRIDE : 16];
     __shared__ uint32_t rmax[WAVES];
-    __shared__ uint16_t srow[MR];
+    __shared__ float rlo[WAVES], rhi[WAVES];
+    __shared__ int rsum[WAVES];
+    __shared__ uint16_t srow[MR], zrow[MR];
+    __shared__ int rsrow[MR];
+    // binary16 rows in: the epilogue decides the quantizer (SymQuantizer for the symmetric epilogues, AsymQuantizer
+    // for the asymmetric ones; the row-sum epilogue takes the signed-shifted codes, code - 8 and zero - 8, and the
+    // per-token sum of the shifted codes)
+    constexpr bool ASYMQ = FUSEQ && (MODE == 1 || MODE == 3 || MODE == 4);
+    constexpr bool SHIFTQ = FUSEQ && MODE == 4;
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t kbytes = p.K >> 1;
@@ -180,42 +190,100 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DecodeParams p
     if (EPI >= 0 && !FUSEQ) rp = load_row<MODE>(p.epi, min(my_m, p.M - 1));
 
     if (FUSEQ) {
-        PkMinMax st;  // units past the row end read as zero, which changes no maximum of |x|
+        // statistics of this wavefront's share of its row.  Units past the row end read as zero: that changes no
+        // maximum of |x|, but it would change a minimum or a maximum, so the asymmetric form skips them.
+        PkMinMax st;
 #pragma unroll
-        for (int j = 0; j < UPL; ++j) st.add8(raw[j]);
-        uint32_t m16 = wave_max_u32(st.absmax_bits());
-        if (WPR > 1) {  // the row's maximum crosses its wavefronts through LDS
-            if (lane == 0) rmax[wave] = m16;
+        for (int j = 0; j < UPL; ++j)
+            if (!ASYMQ || qpart * 64 + lane + j * (64 * WPR) < nunits) st.add8(raw[j]);
+        uint32_t m16;
+        float lo = 0.f, hi = 0.f;
+        if (!ASYMQ) {
+            m16 = wave_max_u32(st.absmax_bits());
+        } else {
+            st.wave_reduce();
+            m16 = st.absmax_bits();
+            lo = st.min_f32();
+            hi = st.max_f32();
+        }
+        if (WPR > 1) {  // the row's statistics cross its wavefronts through LDS
+            if (lane == 0) {
+                rmax[wave] = m16;
+                if (ASYMQ) {
+                    rlo[wave] = lo;
+                    rhi[wave] = hi;
+                }
+            }
             __syncthreads();
             m16 = rmax[qrow * WPR];
+            if (ASYMQ) {
+                lo = rlo[qrow * WPR];
+                hi = rhi[qrow * WPR];
+            }
 #pragma unroll
-            for (int i = 1; i < WPR; ++i) m16 = max(m16, rmax[qrow * WPR + i]);
+            for (int i = 1; i < WPR; ++i) {
+                m16 = max(m16, rmax[qrow * WPR + i]);
+                if (ASYMQ) {
+                    lo = fminf(lo, rlo[qrow * WPR + i]);
+                    hi = fmaxf(hi, rhi[qrow * WPR + i]);
+                }
+            }
         }
-        {
-            RowQuant<false> rq;
-            rq.init(m16, 0.f, 0.f, p.clip, p.qmax);
-            const bool copy_out = blockIdx.x == 0 && qrow < p.M;
+        if (ASYMQ && m16 > 0x7C00u) lo = hi = __builtin_nanf("");  // torch's min / max return NaN for a row that holds one
+        int code_sum = 0;
+        // rows past M (the last rows of the MR the kernel is built for) are neither quantized nor used
+        if (qrow < p.M) {
+            RowQuant<ASYMQ> rq;
+            rq.init(m16, lo, hi, p.clip, p.qmax);
+            const bool copy_out = blockIdx.x == 0;
 #pragma unroll
             for (int j = 0; j < UPL; ++j) {
                 const uint32_t c = qpart * 64 + lane + j * (64 * WPR);
                 if (c < nunits) {
-                    const uint32_t word = rq.quant8(raw[j]);
+                    uint32_t word = rq.quant8(raw[j]);
+                    if (SHIFTQ) {
+                        // eight unsigned codes: sum them, then u - 8 as a signed nibble is u with bit 3 flipped
+                        const uint32_t pairs = (word & 0x0F0F0F0Fu) + ((word >> 4) & 0x0F0F0F0Fu);
+                        code_sum = (int)__builtin_amdgcn_udot4(pairs, 0x01010101u, (uint32_t)code_sum, false);
+                        word ^= 0x88888888u;
+                    }
                     *reinterpret_cast<uint32_t *>(xs + qrow * XSTRIDE + c * 4) = word;
                     if (copy_out && p.q_out) reinterpret_cast<uint32_t *>(p.q_out + (uint64_t)qrow * kbytes)[c] = word;
                 }
             }
+            if (SHIFTQ) {
+                code_sum = wave_sum_i32(code_sum);
+                if (lane == 0) rsum[wave] = code_sum;
+            }
             if (qpart == 0 && lane == 0) {
+                const f16 z = SHIFTQ ? rq.z - (f16)8.0f : rq.z;
                 srow[qrow] = f16_to_bits(rq.s);
+                if (ASYMQ) zrow[qrow] = f16_to_bits(z);
                 if (copy_out && p.s_out) p.s_out[qrow] = f16_to_bits(rq.s);
+                if (ASYMQ && copy_out && p.z_out) p.z_out[qrow] = f16_to_bits(z);
             }
         }
         __syncthreads();
+        if (SHIFTQ) {
+            // per-token sum of the shifted codes: the parts of a row's wavefronts, minus 8 per element
+            if (tid < (uint32_t)MR && tid < p.M) {
+                int t = -8 * (int)p.K;
+#pragma unroll
+                for (int i = 0; i < WPR; ++i) t += rsum[tid * WPR + i];
+                rsrow[tid] = t;
+                if (blockIdx.x == 0 && p.rs_out) p.rs_out[tid] = t;
+            }
+            __syncthreads();
+        }
         // (bytes past the row end are never written: the weights read as zero there)
 #pragma unroll
         for (int m = 0; m < MR; ++m)
 #pragma unroll
             for (int i = 0; i < XS; ++i) xr[m][i] = load16(xs + m * XSTRIDE + i * 1024 + lane * 16);
-        rp.s = bits_to_f16(srow[min(my_m, (uint32_t)MR - 1)]);
+        const uint32_t rm = min(my_m, (uint32_t)MR - 1);
+        rp.s = bits_to_f16(srow[rm]);
+        if (ASYMQ) rp.z = bits_to_f16(zrow[rm]);
+        if (SHIFTQ) rp.rs = rsrow[rm];
     }
 
     auto do_tile = [&](uint32_t tile, const v4u(&w)[R][XS], const ColParams &c) {
@@ -420,8 +488,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_s4_decode_kernel(DecodeParams
 // ---------------------------------------------------------------------------------
 // dispatch
 // ---------------------------------------------------------------------------------
+// Every dispatcher below returns whether it launched a kernel: a shape or mode that no instantiated template
+// covers launches nothing, and the entry points turn that into an error instead of returning success with the
+// output unwritten.
 template <int MR, int XS, bool FUSEQ>
-void launch_rows_mode(DecodeParams &p, int epi, hipStream_t stream)
+bool launch_rows_mode(DecodeParams &p, int epi, hipStream_t stream)
 {
     const uint32_t ntiles = (p.N + 4 * DUQ_DEC_R - 1) / (4 * DUQ_DEC_R);  // 16 weight rows per tile
     // One tile per workgroup.  Four rows quantized in the kernel, more than 256 tiles: every workgroup quantizes
@@ -437,47 +508,54 @@ void launch_rows_mode(DecodeParams &p, int epi, hipStream_t stream)
     p.tiles_per_wg = multi ? (ntiles + 255) / 256 : 1;
     const dim3 grid((ntiles + p.tiles_per_wg - 1) / p.tiles_per_wg);
     const bool wide = MR == 8 || (FUSEQ && MR == 4 && !multi && grid.x > 256);
+    bool launched = false;
 #define DUQ_ROWS(E)                                                                                              \
     if (multi) {                                                                                                 \
-        if constexpr (kCanMulti)                                                                                 \
+        if constexpr (kCanMulti) {                                                                               \
             hipLaunchKernelGGL((gemv_s4_rows_kernel<MR, XS, FUSEQ, E, 8, true>), grid, dim3(512), 0, stream, p);     \
+            launched = true;                                                                                     \
+        }                                                                                                        \
     } else if (wide) {                                                                                           \
-        if constexpr (FUSEQ && MR >= 4)                                                                          \
+        if constexpr (FUSEQ && MR >= 4) {                                                                        \
             hipLaunchKernelGGL((gemv_s4_rows_kernel<MR, XS, FUSEQ, E, 8>), grid, dim3(512), 0, stream, p);           \
+            launched = true;                                                                                     \
+        }                                                                                                        \
     } else {                                                                                                     \
-        if constexpr (MR <= 4)                                                                                   \
+        if constexpr (MR <= 4) {                                                                                 \
             hipLaunchKernelGGL((gemv_s4_rows_kernel<MR, XS, FUSEQ, E, 4>), grid, dim3(256), 0, stream, p);           \
+            launched = true;                                                                                     \
+        }                                                                                                        \
     }
     switch (epi) {
     case 0: DUQ_ROWS(0) break;
+    case 1: DUQ_ROWS(1) break;
     case 2: DUQ_ROWS(2) break;
+    case 3: DUQ_ROWS(3) break;
+    case 4: DUQ_ROWS(4) break;
     default:
         if constexpr (!FUSEQ) {
-            switch (epi) {
-            case -1: DUQ_ROWS(-1) break;
-            case 1: DUQ_ROWS(1) break;
-            case 3: DUQ_ROWS(3) break;
-            case 4: DUQ_ROWS(4) break;
-            }
+            if (epi == -1) { DUQ_ROWS(-1) }
         }
     }
 #undef DUQ_ROWS
+    return launched;
 }
 
 template <int MR, bool FUSEQ>
-void launch_rows_xs(DecodeParams &p, int epi, hipStream_t stream)
+bool launch_rows_xs(DecodeParams &p, int epi, hipStream_t stream)
 {
     const uint32_t kbytes = p.K / 2;
-    if (kbytes <= 2048) launch_rows_mode<MR, 2, FUSEQ>(p, epi, stream);
-    else if (kbytes <= 4096) launch_rows_mode<MR, 4, FUSEQ>(p, epi, stream);
-    else if constexpr (MR <= 4) {  // (eight rows: up to 8192 elements, decode_fp16in_one_launch)
-        if (kbytes <= 6144) launch_rows_mode<MR, 6, FUSEQ>(p, epi, stream);
-        else launch_rows_mode<MR, 8, FUSEQ>(p, epi, stream);
+    if (kbytes <= 2048) return launch_rows_mode<MR, 2, FUSEQ>(p, epi, stream);
+    if (kbytes <= 4096) return launch_rows_mode<MR, 4, FUSEQ>(p, epi, stream);
+    if constexpr (MR <= 4) {  // (eight rows: up to 8192 elements, decode_fp16in_one_launch)
+        if (kbytes <= 6144) return launch_rows_mode<MR, 6, FUSEQ>(p, epi, stream);
+        if (kbytes <= 8192) return launch_rows_mode<MR, 8, FUSEQ>(p, epi, stream);
     }
+    return false;
 }
 
 template <int WAVES, int SEGS, int MT = 1, bool DB = true>
-void launch_mfma_mode(const DecodeParams &p, int epi, hipStream_t stream)
+bool launch_mfma_mode(const DecodeParams &p, int epi, hipStream_t stream)
 {
     const uint32_t ntiles = (p.N + 15) / 16;
     const dim3 grid((ntiles + p.tiles_per_wg - 1) / p.tiles_per_wg);
@@ -489,46 +567,48 @@ void launch_mfma_mode(const DecodeParams &p, int epi, hipStream_t stream)
     case 2: DUQ_DEC(2); break;
     case 3: DUQ_DEC(3); break;
     case 4: DUQ_DEC(4); break;
+    default: return false;
     }
 #undef DUQ_DEC
+    return true;
 }
 
 template <bool FUSEQ>
-void launch_decode_any(DecodeParams &p, int epi, hipStream_t stream)
+bool launch_decode_any(DecodeParams &p, int epi, hipStream_t stream)
 {
     const uint32_t kbytes = p.K / 2;
     if (decode_uses_rows_kernel(p.M)) {
-        if (p.M == 1) launch_rows_xs<1, FUSEQ>(p, epi, stream);
-        else if (p.M == 2) launch_rows_xs<2, FUSEQ>(p, epi, stream);
-        else launch_rows_xs<4, FUSEQ>(p, epi, stream);
-        return;
+        if (p.M == 1) return launch_rows_xs<1, FUSEQ>(p, epi, stream);
+        if (p.M == 2) return launch_rows_xs<2, FUSEQ>(p, epi, stream);
+        return launch_rows_xs<4, FUSEQ>(p, epi, stream);
     }
     if constexpr (FUSEQ) {
-        launch_rows_xs<8, true>(p, epi, stream);  // 5..8 rows (decode_fp16in_one_launch admits no others)
-        return;
-    }
-    if constexpr (!FUSEQ) {
+        if (p.M > 8) return false;
+        return launch_rows_xs<8, true>(p, epi, stream);  // 5..8 rows
+    } else {
         const uint32_t ntiles = (p.N + 15) / 16;
         p.tiles_per_wg = decode_tiles_per_workgroup(ntiles);
         constexpr int W = DUQ_DEC_WAVES, S = 32 / W;  // 64-byte segments per wavefront for 2 KB of a row
-        const uint32_t mt = (p.M + 15) / 16;  // 2..4 only with rows of at most 8192 elements (select_gemm_kernel)
+        const uint32_t mt = (p.M + 15) / 16;
         // rows of up to 4096 / 8192 / 12288 elements: S, 2 S, 12 segments per wavefront; the row tiles whose
-        // fragments fit in registers next to two sets of weights (select_gemm_kernel admits no others)
+        // fragments fit in registers next to two sets of weights (what select_gemm_kernel sends here)
+        if (mt > 4 || kbytes > 6144) return false;
         if (kbytes <= 2048) {
-            if (mt == 1) launch_mfma_mode<W, S, 1>(p, epi, stream);
-            else if (mt == 2) launch_mfma_mode<W, S, 2>(p, epi, stream);
-            else if (mt == 3) launch_mfma_mode<W, S, 3>(p, epi, stream);
-            else launch_mfma_mode<W, S, 4>(p, epi, stream);
-        } else if (kbytes <= 4096) {
-            if (mt == 1) launch_mfma_mode<W, 2 * S, 1>(p, epi, stream);
-            else if (mt == 2) launch_mfma_mode<W, 2 * S, 2>(p, epi, stream);
-            else if (mt == 3) launch_mfma_mode<W, 2 * S, 3>(p, epi, stream);
-            else launch_mfma_mode<W, 2 * S, 4>(p, epi, stream);
-        } else {
-            if (mt == 1) launch_mfma_mode<8, 12, 1>(p, epi, stream);
-            else if (mt == 2) launch_mfma_mode<8, 12, 2, false>(p, epi, stream);
-            else launch_mfma_mode<8, 12, 3, false>(p, epi, stream);
+            if (mt == 1) return launch_mfma_mode<W, S, 1>(p, epi, stream);
+            if (mt == 2) return launch_mfma_mode<W, S, 2>(p, epi, stream);
+            if (mt == 3) return launch_mfma_mode<W, S, 3>(p, epi, stream);
+            return launch_mfma_mode<W, S, 4>(p, epi, stream);
         }
+        if (kbytes <= 4096) {
+            if (mt == 1) return launch_mfma_mode<W, 2 * S, 1>(p, epi, stream);
+            if (mt == 2) return launch_mfma_mode<W, 2 * S, 2>(p, epi, stream);
+            if (mt == 3) return launch_mfma_mode<W, 2 * S, 3>(p, epi, stream);
+            return launch_mfma_mode<W, 2 * S, 4>(p, epi, stream);
+        }
+        if (mt == 1) return launch_mfma_mode<8, 12, 1>(p, epi, stream);
+        if (mt == 2) return launch_mfma_mode<8, 12, 2, false>(p, epi, stream);
+        if (mt == 3) return launch_mfma_mode<8, 12, 3, false>(p, epi, stream);
+        return false;
     }
 }
 
@@ -575,12 +655,13 @@ int launch_decode_s4(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N,
     p.C = out_acc;
     p.y = y;
     if (epi) p.epi = *epi;
-    launch_decode_any<false>(p, out_acc ? -1 : epi->mode, stream);
+    if (!launch_decode_any<false>(p, out_acc ? -1 : epi->mode, stream)) return (int)hipErrorInvalidValue;
     return (int)hipGetLastError();
 }
 
 int launch_decode_fp16in(const uint16_t *x, float clip, int qmax, const uint8_t *B, uint32_t M, uint32_t N, uint32_t K,
-                         const Epilogue &epi, uint16_t *y, uint8_t *q_out, uint16_t *s_out, hipStream_t stream)
+                         const Epilogue &epi, uint16_t *y, uint8_t *q_out, uint16_t *s_out, uint16_t *z_out,
+                         int32_t *rs_out, hipStream_t stream)
 {
     DecodeParams p{};
     p.X = x;
@@ -594,7 +675,9 @@ int launch_decode_fp16in(const uint16_t *x, float clip, int qmax, const uint8_t 
     p.qmax = qmax;
     p.q_out = q_out;
     p.s_out = s_out;
-    launch_decode_any<true>(p, epi.mode, stream);
+    p.z_out = z_out;
+    p.rs_out = rs_out;
+    if (!launch_decode_any<true>(p, epi.mode, stream)) return (int)hipErrorInvalidValue;
     return (int)hipGetLastError();
 }
 

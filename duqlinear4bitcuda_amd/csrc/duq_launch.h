@@ -101,18 +101,20 @@ inline bool decode_fp16in_one_launch(uint32_t M, uint32_t N, uint32_t K)
 {
     const int kernel = select_gemm_kernel(M, N, K);
     if (kernel == kKernelDecodeRows) return M == 1 || N <= 16384;
-    return M <= 8 && N <= 16384 && (K <= 4096 || (K <= 8192 && N <= 4096)) &&
-           (kernel == kKernelDecodeMfma || kernel == kKernelSkinny);
+    return M <= 8 && N <= 16384 && (K <= 4096 || (K <= 8192 && N <= 4096)) && kernel == kKernelDecodeMfma;
 }
 // decode kernels (duq_decode.hip); the shape must be one select_gemm_kernel gives to them
 int launch_decode_s4(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N, uint32_t K, int32_t *out_acc,
                      const Epilogue *epi, uint16_t *y, hipStream_t stream);
-// the same with binary16 activations in: per-token symmetric quantization (scale = h(h(max|x| / 7) * clip), codes
-// clamp(rint(h(x / scale)), -8, qmax)) happens inside the launch; epi.s_row is ignored; q_out / s_out (optional)
-// receive the codes and scales.  Modes DUQ_EPI_SYM and DUQ_EPI_SYM_DUAL; shapes of the rows kernel only
-// (select_gemm_kernel(M, N, K) == kKernelDecodeRows).
+// the same with binary16 activations in: the per-token quantizer runs inside the launch, SymQuantizer for the
+// symmetric epilogues (scale = h(h(max|x| / 7) * clip), codes clamp(rint(h(x / scale)), -8, qmax)), AsymQuantizer for
+// modes 1 and 3 (unsigned codes, as the reference stores them) and its signed-shifted form for mode 4 (codes and
+// zero points minus 8, plus the per-token sums of the shifted codes); epi.s_row / z_row / rs_row are ignored.
+// q_out / s_out / z_out / rs_out (optional) receive the codes, scales, zero points and sums.  Shapes of
+// decode_fp16in_one_launch only.
 int launch_decode_fp16in(const uint16_t *x, float clip, int qmax, const uint8_t *B, uint32_t M, uint32_t N, uint32_t K,
-                         const Epilogue &epi, uint16_t *y, uint8_t *q_out, uint16_t *s_out, hipStream_t stream);
+                         const Epilogue &epi, uint16_t *y, uint8_t *q_out, uint16_t *s_out, uint16_t *z_out,
+                         int32_t *rs_out, hipStream_t stream);
 
 // measurement aid: read `bytes` (< 4 GiB) with the decode kernels' access pattern and discard them
 int launch_probe_read(const void *src, uint64_t bytes, uint32_t *sink, hipStream_t stream);

@@ -48,6 +48,44 @@ class _Linear4bitBase(torch.nn.Module):
     def _finish(self, y):
         return y if self.bias is None else y + self.bias
 
+    # ---- decode: quantizer + GEMM + dequant as ONE launch (up to eight rows of binary16 activations) ----
+    _decode = None
+
+    def _decode_args(self):
+        """(mode, weight, w_scale_1, w_zeros_1, w_scale_2, w_zeros_2, w_rowsum_adj) of the layer, or None when
+        it has no one-launch form."""
+        return None
+
+    def _decode_call(self):
+        """The layer's prepared one-launch call (``_HIP.FusedDecode``), rebuilt when a buffer was replaced (moved,
+        cast, reloaded into a new tensor); None for a layer that has none or is not on a GPU."""
+        args = self._decode_args()
+        if args is None:
+            return None
+        d = self._decode
+        if d is not None:
+            held = d.tensors
+            if held[0] is args[1] and held[1] is args[2] and held[2] is args[3] and held[3] is args[4] and \
+                    held[4] is args[5] and held[5] is args[6] and held[6] is self.bias and d.w_ptr == args[1].data_ptr():
+                return d
+        if not args[1].is_cuda:
+            return None
+        d = self._decode = _ops.FusedDecode(*args, bias=self.bias)
+        return d
+
+    def _decode_forward(self, x, clip=1.0, qmax=6):
+        """y for binary16 rows ``x`` when the layer runs them as one launch (quantizer inside), else None."""
+        K = self.in_features
+        if not self.fused or x.shape[-1] != K or K % 64:
+            return None
+        M = x.numel() // K
+        if M > 8 or M == 0:
+            return None
+        d = self._decode_call()
+        if d is None or not d.admits(M):
+            return None
+        return d.run(x, M, clip, qmax)
+
     def enable_fp6(self):
         """Build the E3M2 shadow of ``weight`` (3/4 byte per element next to the 1/2 byte of the packed
         nibbles; not part of the state_dict; rebuilt when ``weight`` changes).  Results are bit-identical;
@@ -83,6 +121,14 @@ class _Linear4bitBase(torch.nn.Module):
             return True
         return self._fp6_wanted(x.shadow_x.numel() // x.shadow_x.shape[-1])
 
+    def _own_quantizer_decode(self, x):
+        """Layers with their own AsymQuantizer: a few contiguous binary16 rows on the GPU run quantizer + GEMM +
+        dequant as one launch (the quantizer inside the GEMM kernel, same bits); None for anything else."""
+        if type(x) is not torch.Tensor or x.dtype is not torch.float16 or not x.is_cuda or not x.is_contiguous() or \
+                x.data_ptr() % 16:
+            return None
+        return self._decode_forward(x)
+
     def _quantize(self, x):
         """Own quantizer of the asymmetric layers: shadow only when this call will take the 6-bit float path."""
         rows = x.numel() // x.shape[-1]
@@ -103,8 +149,16 @@ class Linear4bitSQ(_Linear4bitBase):
         else:
             self.bias = None
 
+    def _decode_args(self):
+        b = self._buffers
+        return (_ops.EPI_SYM, b["weight"], b["weight_scales"], None, None, None, None)
+
     def forward(self, x):
         assert type(x) == tensor_utils.PackedQuantizedTensor  # quantized input is required
+        if x._src is not None:  # a few rows straight from SymQuantizer: quantized inside the GEMM launch
+            y = self._decode_forward(x.source(), x._clip, x._qmax)
+            if y is not None:
+                return y
         xq, scales_x = x.quantized_x, x.scales_x
         if self.fused and self._use_shadow(x):
             return tensor_utils.linear_forward_shadow(_ops.EPI_SYM, x.shadow_x, scales_x, None, self.weight_shadow,
@@ -150,8 +204,15 @@ class Linear4bitASQ(_Linear4bitBase):
         if require_quantizer:
             self.quantizer = AsymQuantizer()
 
+    def _decode_args(self):
+        b = self._buffers
+        return (_ops.EPI_ASYM, b["weight"], b["weight_scales"], b["weight_zeros"], None, None, None)
+
     def forward(self, x):
         if self.require_quantizer:
+            y = self._own_quantizer_decode(x)
+            if y is not None:
+                return y
             x = self._quantize(x) if self.fused else self.quantizer(x)
         assert type(x) == tensor_utils.PackedQuantizedTensor, \
             "Input should be quantized tensor, or require_quantizer should be passed as initial argument"
@@ -204,8 +265,15 @@ class Linear4bitASQRowSum(_Linear4bitBase):
         if require_quantizer:
             self.quantizer = AsymQuantizer(shifted=True)
 
+    def _decode_args(self):
+        b = self._buffers
+        return (_ops.EPI_ASYM_ROWSUM, b["weight"], b["weight_scales"], b["weight_zeros"], None, None, b["weight_rowsum"])
+
     def forward(self, x):
         if self.require_quantizer:
+            y = self._own_quantizer_decode(x)
+            if y is not None:
+                return y
             x = self._quantize(x) if self.fused else self.quantizer(x)
         assert type(x) == tensor_utils.PackedQuantizedTensor and x.rowsum_x is not None, \
             "Input should come from AsymQuantizer(shifted=True), or require_quantizer should be set"
@@ -335,8 +403,16 @@ class Linear4bitDUSQ(_Linear4bitBase):
         else:
             self.bias = None
 
+    def _decode_args(self):
+        b = self._buffers
+        return (_ops.EPI_SYM_DUAL, b["weight"], b["weight_scales_1"], None, b["weight_scales_2"], None, None)
+
     def forward(self, x):
         assert type(x) == tensor_utils.PackedQuantizedTensor
+        if x._src is not None:  # a few rows straight from SymQuantizer: quantized inside the GEMM launch
+            y = self._decode_forward(x.source(), x._clip, x._qmax)
+            if y is not None:
+                return y
         xq, scales_x = x.quantized_x, x.scales_x
         if self.fused and self._use_shadow(x):
             return tensor_utils.linear_forward_shadow(_ops.EPI_SYM_DUAL, x.shadow_x, scales_x, None, self.weight_shadow,
@@ -386,8 +462,16 @@ class LinearQuant4bitDUASQ(_Linear4bitBase):
         if self.require_quantizer:
             self.quantizer = AsymQuantizer()
 
+    def _decode_args(self):
+        b = self._buffers
+        return (_ops.EPI_ASYM_DUAL, b["weight"], b["weight_scales_1"], b["weight_zeros_1"], b["weight_scales_2"],
+                b["weight_zeros_2"], None)
+
     def forward(self, x):
         if self.require_quantizer:
+            y = self._own_quantizer_decode(x)
+            if y is not None:
+                return y
             x = self._quantize(x) if self.fused else self.quantizer(x)
         assert type(x) == tensor_utils.PackedQuantizedTensor, \
             "Input should be quantized tensor, or require_quantizer should be passed as initial argument"

@@ -27,6 +27,12 @@ class SymQuantizer(torch.nn.Module):
     clamp of the codes: 6 is what the reference's device kernel applies
     (include/common.h:53-54), 7 what its Python fake-quant path applies."""
 
+    # Inputs of at most this many rows (decode) are handed on unquantized inside the PackedQuantizedTensor: a
+    # Linear4bitSQ / Linear4bitDUSQ that follows quantizes them inside its own launch (quantizer + GEMM + dequant
+    # are then ONE launch), and anything else that reads quantized_x / scales_x triggers this quantizer's launch
+    # then, with the same bits.  0 switches that off.
+    defer_rows = 8
+
     def __init__(self, input_clip_ratio=1.0, qmax: int = 6, shadow=False, shadow_min_rows: int = 96):
         super().__init__()
         self.input_clip_ratio = input_clip_ratio
@@ -40,6 +46,10 @@ class SymQuantizer(torch.nn.Module):
     def forward(self, x, shadow=None) -> tensor_utils.PackedQuantizedTensor:
         if not x.is_contiguous():
             x = x.contiguous()
+        cols = x.shape[-1]
+        if shadow is None and self.defer_rows and cols % 64 == 0 and 0 < x.numel() <= self.defer_rows * cols and \
+                x.is_cuda and x.dtype is torch.float16 and x.data_ptr() % 16 == 0:
+            return tensor_utils.PackedQuantizedTensor.deferred(x, self.input_clip_ratio, self.qmax)
         shadow = _shadow_choice(self, x, shadow)
         if shadow:
             q, sh, scales = tensor_utils.quantize_sym_shadow(x, self.input_clip_ratio, self.qmax, shadow != "only")

@@ -13,27 +13,87 @@ from .. import _HIP as _ops
 
 class PackedQuantizedTensor:
     """A quantized activation: packed nibbles plus per-token scale (and zero point)
-    (tensor_utils.py:20-38)."""
+    (tensor_utils.py:20-38).
+
+    A few rows (decode) may arrive *deferred* from ``SymQuantizer``: the object then holds the binary16 rows and
+    the quantizer's settings, a ``Linear4bitSQ`` / ``Linear4bitDUSQ`` that can run quantize + GEMM + dequant as one
+    launch consumes those directly, and ``quantized_x`` / ``scales_x`` are computed (one quantizer launch, the same
+    bits) the first time anything reads them."""
+
+    __slots__ = ("_q", "_s", "zeros_x", "rowsum_x", "shadow_x", "_src", "_src_version", "_clip", "_qmax")
 
     def __init__(self, quantized_x: torch.Tensor, scales_x: torch.Tensor, zeros_x: torch.Tensor = None,
                  rowsum_x: torch.Tensor = None, shadow_x: torch.Tensor = None):
-        self.quantized_x = quantized_x
-        self.scales_x = scales_x
+        self._q = quantized_x
+        self._s = scales_x
         self.zeros_x = zeros_x
         # set only by the signed-shifted asymmetric quantizer (codes - 8, zeros - 8): per-token sums of the codes
         self.rowsum_x = rowsum_x
         # set by a quantizer with shadow=True / "only": the same codes as 6-bit floats [..., 3K/4] for the
         # 6-bit float matrix path; with "only", quantized_x is None
         self.shadow_x = shadow_x
+        self._src = None
+
+    @classmethod
+    def deferred(cls, x: torch.Tensor, clip: float, qmax: int):
+        """The symmetric quantization of ``x`` (contiguous binary16 [..., K], K % 32 == 0, 16-byte aligned), not
+        yet computed."""
+        self = cls.__new__(cls)
+        self._q = self._s = self.zeros_x = self.rowsum_x = self.shadow_x = None
+        self._src = x
+        self._src_version = x._version
+        self._clip = clip
+        self._qmax = qmax
+        return self
+
+    def source(self):
+        """The binary16 rows of a deferred tensor (None once quantized, or when it never was deferred).  Raises
+        when they were written to since the quantizer saw them: the codes would be those of the new values."""
+        x = self._src
+        if x is not None and x._version != self._src_version:
+            raise RuntimeError("PackedQuantizedTensor: the activations were modified in place between the quantizer "
+                               "and the first use of its result")
+        return x
+
+    def _materialize(self):
+        x = self.source()
+        self._q, self._s = _ops.quantize_rows_sym(x, self._clip, self._qmax)
+        self._src = None
+
+    @property
+    def quantized_x(self):
+        if self._src is not None:
+            self._materialize()
+        return self._q
+
+    @quantized_x.setter
+    def quantized_x(self, v):
+        if self._src is not None:
+            self._materialize()
+        self._q = v
+
+    @property
+    def scales_x(self):
+        if self._src is not None:
+            self._materialize()
+        return self._s
+
+    @scales_x.setter
+    def scales_x(self, v):
+        if self._src is not None:
+            self._materialize()
+        self._s = v
 
     def size(self):
-        if self.quantized_x is not None:
-            return self.quantized_x.size()
+        if self._src is not None:
+            return torch.Size(self._src.shape[:-1] + (self._src.shape[-1] // 2,))
+        if self._q is not None:
+            return self._q.size()
         return torch.Size(self.shadow_x.shape[:-1] + (self.shadow_x.shape[-1] * 2 // 3,))
 
     @property
     def device(self):
-        return self.scales_x.device
+        return self._src.device if self._src is not None else self._s.device
 
     @property
     def dtype(self):

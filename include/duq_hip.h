@@ -17,7 +17,7 @@
  * All pointers are DEVICE pointers on the current HIP device; inputs are borrowed,
  * outputs are caller-allocated, the library allocates no memory and keeps no global state
  * (re-entrant); the one exception is duq_quantize_linear4bit_forward_static and its static
- * device array.  No call synchronises the host.
+ * device array (and duq_static_scratch_init, which belongs to it).  No call synchronises the host.
  *
  * Packed int4 layout everywhere: element i of a row is in byte i/2, low nibble first
  * (include/int4.h:86-98).
@@ -42,7 +42,9 @@ typedef void *duq_stream_t;  /* hipStream_t */
 #define DUQ_E_MODE (-4)      /* unknown epilogue mode / unsupported qmax */
 #define DUQ_E_ALIGN (-5)     /* a pointer misses the alignment the entry point documents */
 #define DUQ_E_TOO_LARGE (-6) /* a dimension exceeds what the kernels index with 32 bits: K > 131008, N > 2^22, M > 2^24 */
-#define DUQ_E_SCRATCH (-7)   /* the input does not fit the static scratch buffer of an entry point that allocates nothing */
+#define DUQ_E_SCRATCH (-7)   /* the input does not fit a slot of the static scratch buffer of the entry point that allocates nothing, or the slot does not exist */
+#define DUQ_E_DEVICE (-8)    /* the stream belongs to another device than the current one */
+#define DUQ_E_CAPTURE (-9)   /* a call that must query the runtime was made on a stream under capture */
 
 /* symmetric clamp used by the device quantizer of the reference: qmax_sym evaluates to 6
  * (include/common.h:53-54).  7 is the bound of the Python fake-quant path
@@ -247,26 +249,50 @@ int duq_quantize_linear4bit_forward(int32_t mode, const duq_half *x, float clip,
                                     duq_half *scale_out, void *workspace, uint64_t workspace_bytes,
                                     duq_stream_t stream);
 
+/* The same from binary16 activations for the asymmetric layers (no counterpart in the reference, where this is
+ * AsymQuantizer.forward followed by Linear4bitASQ.forward / LinearQuant4bitDUASQ.forward,
+ * qlinear4bit/nn/quantizer.py:24-35, qlinear4bit/nn/linear.py:104-115, 239-250), and for the row-sum mode:
+ *   mode DUQ_EPI_ASYM       y = duq_quantize_rows_asym, then duq_linear4bit_forward(DUQ_EPI_ASYM), bit for bit
+ *        DUQ_EPI_ASYM_DUAL  the same with the dual-uniform epilogue (w_scale_2, w_zeros_2)
+ *        DUQ_EPI_ASYM_ROWSUM  duq_quantize_rows_asym_shifted, then duq_linear4bit_forward_rowsum (w_rowsum_adj)
+ *   q_out [M,K/2], scale_out [M], zeros_out [M], rowsum_out [M] (row-sum mode): optional (NULL)
+ * The shapes that run as ONE launch are those of duq_quantize_linear4bit_forward; the others run quantizer + GEMM
+ * and stage codes, scales, zero points (and row sums) in `workspace`
+ * (duq_quantize_linear4bit_asym_workspace_bytes(mode, M, N, K) bytes, 16-byte aligned; whatever the caller's own
+ * output pointers cover is written there instead). */
+uint64_t duq_quantize_linear4bit_asym_workspace_bytes(int32_t mode, uint32_t M, uint32_t N, uint32_t K);
+int duq_quantize_linear4bit_forward_asym(int32_t mode, const duq_half *x, const uint8_t *w, const duq_half *w_scale_1,
+                                         const duq_half *w_zeros_1, const duq_half *w_scale_2,
+                                         const duq_half *w_zeros_2, const int32_t *w_rowsum_adj, const duq_half *bias,
+                                         uint32_t M, uint32_t N, uint32_t K, duq_half *y, uint8_t *q_out,
+                                         duq_half *scale_out, duq_half *zeros_out, int32_t *rowsum_out, void *workspace,
+                                         uint64_t workspace_bytes, duq_stream_t stream);
+
 /* No counterpart in the reference.  For callers that cannot allocate device memory or carry a workspace around
  * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc):
  * duq_quantize_linear4bit_forward without the workspace arguments.  The codes and scales that its quantizer
- * launch hands to its GEMM launch are staged in a device array that is part of the library's code object
- * (DUQ_STATIC_SCRATCH_CODE_BYTES + 2 * DUQ_STATIC_SCRATCH_ROWS bytes; every GPU the library runs on holds its own
- * copy until the process ends).  The call allocates and frees nothing.  y (and q_out / scale_out) are bit-identical
- * to duq_quantize_linear4bit_forward's.
+ * launch hands to its GEMM launch are staged in a device array that is part of the library's code object:
+ * DUQ_STATIC_SCRATCH_SLOTS slots of DUQ_STATIC_SCRATCH_CODE_BYTES + 2 * DUQ_STATIC_SCRATCH_ROWS bytes (33 MiB in
+ * all; every GPU the library runs on holds its own copy until the process ends).  The call allocates and frees
+ * nothing.  y (and q_out / scale_out) are bit-identical to duq_quantize_linear4bit_forward's.
  *   limit   M * K / 2 <= DUQ_STATIC_SCRATCH_CODE_BYTES and M <= DUQ_STATIC_SCRATCH_ROWS, whatever the launch plan,
  *           else DUQ_E_SCRATCH (e.g. 4096 x 4096 or 2048 x 8192 activations fit, 4096 x 8192 do not)
- *   device  the stream's device must be the current one; the first staged call on a device looks the array's
- *           address up (hipGetSymbolAddress) and should therefore not be made under stream capture
- *   sharing all calls on one GPU share that GPU's array: two calls whose work overlaps in time (different
- *           streams, or graphs replayed concurrently) race on it; calls ordered on one stream do not.  Nothing in
- *           it has to start at zero: each call overwrites the part it reads. */
+ *   slot    which slot the call stages in, 0 .. DUQ_STATIC_SCRATCH_SLOTS - 1 (else DUQ_E_SCRATCH).  Calls whose work
+ *           may overlap in time on one GPU (different streams, graphs replayed concurrently) must use different
+ *           slots: two overlapping calls on one slot race on it with no error.  Calls ordered on one stream may
+ *           share a slot.  Nothing in a slot has to start at zero: each call overwrites the part it reads.
+ *   device  the stream must belong to the current device (DUQ_E_DEVICE otherwise).  The first staged call on a
+ *           device asks the runtime for the array's address (hipGetSymbolAddress), which a stream under capture
+ *           may not do: such a call returns DUQ_E_CAPTURE.  duq_static_scratch_init() does the lookup for the
+ *           current device up front; afterwards a call reads one atomic pointer and takes no lock. */
 #define DUQ_STATIC_SCRATCH_CODE_BYTES (8u << 20)
 #define DUQ_STATIC_SCRATCH_ROWS 32768u
+#define DUQ_STATIC_SCRATCH_SLOTS 4u
+int duq_static_scratch_init(void);
 int duq_quantize_linear4bit_forward_static(int32_t mode, const duq_half *x, float clip, int32_t qmax, const uint8_t *w,
                                            const duq_half *w_scale_1, const duq_half *w_scale_2, const duq_half *bias,
                                            uint32_t M, uint32_t N, uint32_t K, duq_half *y, uint8_t *q_out,
-                                           duq_half *scale_out, duq_stream_t stream);
+                                           duq_half *scale_out, uint32_t slot, duq_stream_t stream);
 
 /* ---- asymmetric forward with exact zero-point correction (row sums) -------------------- */
 

@@ -50,6 +50,10 @@ inline std::pair<torch::Tensor, std::vector<int64_t>> flatten_last_dim_and_retur
 }
 
 // ---- quantized activation (include/quant_tensor.h:11-27)
+// A few rows (decode) may arrive *deferred* from Quantizer4bit: the object then holds the binary16 rows
+// (`source_x`) and the quantizer's settings, quantized_x / scale are undefined, and a Linear4bit / Linear4bitDUQ
+// that can run quantizer + GEMM + dequant as one launch consumes the rows directly.  Anything else calls
+// materialize() first (one quantizer launch, the same bits); Quantizer4bit(clip, qmax, shadow, 0) never defers.
 class PackedQuantizedTensor {
 public:
     torch::Tensor quantized_x;
@@ -57,10 +61,51 @@ public:
     // not in the reference: the same codes as 6-bit floats [..., 3K/4] for the 6-bit float matrix path
     // (Quantizer4bit with shadow = true); undefined otherwise
     torch::Tensor shadow_x;
+    // not in the reference: the deferred form (see above); undefined otherwise
+    torch::Tensor source_x;
+    float clip = 1.0f;
+    int qmax = DUQ_QMAX_SYM_DEVICE;
+
     PackedQuantizedTensor(torch::Tensor quantized_x, torch::Tensor scale, torch::Tensor shadow_x = torch::Tensor())
         : quantized_x(std::move(quantized_x)), scale(std::move(scale)), shadow_x(std::move(shadow_x)) {}
-    torch::IntArrayRef sizes() const { return quantized_x.sizes(); }
-    torch::Device device() const { return quantized_x.device(); }
+
+    static PackedQuantizedTensor deferred(torch::Tensor x, float clip, int qmax)
+    {
+        PackedQuantizedTensor p{torch::Tensor(), torch::Tensor()};
+        p.packed_sizes_.assign(x.sizes().begin(), x.sizes().end());
+        p.packed_sizes_.back() /= 2;
+        p.source_x = std::move(x);
+        p.clip = clip;
+        p.qmax = qmax;
+        return p;
+    }
+    bool is_deferred() const { return source_x.defined(); }
+
+    // Run the quantizer now (no-op unless deferred): quantized_x [..., K/2] and scale [..., 1] as Quantizer4bit
+    // writes them for larger inputs.
+    PackedQuantizedTensor &materialize()
+    {
+        if (!source_x.defined()) return *this;
+        const torch::Tensor &x = source_x;
+        const uint32_t cols = x.size(-1), rows = cols ? x.numel() / cols : 0;
+        std::vector<int64_t> qshape(x.sizes().begin(), x.sizes().end()), sshape = qshape;
+        qshape.back() = cols / 2;
+        sshape.back() = 1;
+        quantized_x = torch::empty(qshape, torch::dtype(torch::kUInt8).device(x.device()));
+        scale = torch::empty(sshape, torch::dtype(torch::kHalf).device(x.device()));
+        const int st = duq_quantize_rows_sym(reinterpret_cast<const duq_half *>(x.data_ptr()), rows, cols, clip, qmax,
+                                             quantized_x.data_ptr<uint8_t>(), reinterpret_cast<duq_half *>(scale.data_ptr()),
+                                             static_cast<duq_stream_t>(c10::hip::getCurrentHIPStream(x.device().index()).stream()));
+        TORCH_CHECK(st == DUQ_OK, "PackedQuantizedTensor::materialize: ", duq_status_string(st));
+        source_x = torch::Tensor();
+        return *this;
+    }
+
+    torch::IntArrayRef sizes() const { return source_x.defined() ? torch::IntArrayRef(packed_sizes_) : quantized_x.sizes(); }
+    torch::Device device() const { return source_x.defined() ? source_x.device() : quantized_x.device(); }
+
+private:
+    std::vector<int64_t> packed_sizes_;
 };
 
 // quantized activation with two scales: columns < 10 and the rest (include/quant_tensor.h:29-45)
@@ -169,15 +214,21 @@ public:
     float input_clip_ratio;
     int qmax;
     bool shadow;  // also write the 6-bit float shadow (inputs whose width is a multiple of 128)
-    explicit Quantizer4bit(float input_clip_ratio, int qmax = DUQ_QMAX_SYM_DEVICE, bool shadow = false)
-        : input_clip_ratio(input_clip_ratio), qmax(qmax), shadow(shadow) {}
+    // inputs of at most this many rows are handed on unquantized (PackedQuantizedTensor::deferred): the linear
+    // layer behind quantizes them inside its own launch; 0 switches that off
+    uint32_t defer_rows;
+    explicit Quantizer4bit(float input_clip_ratio, int qmax = DUQ_QMAX_SYM_DEVICE, bool shadow = false, uint32_t defer_rows = 8)
+        : input_clip_ratio(input_clip_ratio), qmax(qmax), shadow(shadow), defer_rows(defer_rows) {}
     PackedQuantizedTensor forward(torch::Tensor x)
     {
         x = x.contiguous();
         check_device_tensor(x, "Quantizer4bit::forward", "x");
+        half_ptr(x);  // binary16 only (bf16 storage is rejected)
         auto [x2, lead] = flatten_last_dim_and_return_shape(x);
         const uint32_t rows = x2.size(0), cols = x2.size(1);
         TORCH_CHECK(cols % 32 == 0, "Quantizer4bit::forward: the last dimension must be a multiple of 32");
+        if (!shadow && rows > 0 && rows <= defer_rows && cols % 64 == 0 && reinterpret_cast<uintptr_t>(x.data_ptr()) % 16 == 0)
+            return PackedQuantizedTensor::deferred(x, input_clip_ratio, qmax);
         auto q = torch::empty({rows, cols / 2}, torch::dtype(torch::kUInt8).device(x.device()));
         auto s = torch::empty({rows, 1}, torch::dtype(torch::kHalf).device(x.device()));
         auto qshape = lead;
@@ -257,6 +308,29 @@ inline torch::Tensor fused_forward_shadow(int mode, const PackedQuantizedTensor 
     return y.view(lead);
 }
 
+// A deferred input on a shape that runs quantizer + GEMM + dequant as ONE launch: the result; else an undefined
+// tensor (the caller then materializes the input and takes the usual route).
+inline torch::Tensor fused_decode(int mode, const PackedQuantizedTensor &input, const torch::Tensor &weight,
+                                  const torch::Tensor &s1, const torch::Tensor &s2, const torch::Tensor &bias)
+{
+    const torch::Tensor &x = input.source_x;
+    check_device_tensor(weight, "Linear4bit::forward", "B");
+    TORCH_CHECK(x.device() == weight.device(), "Linear4bit::forward: operands on different devices");
+    TORCH_CHECK(weight.size(1) * 2 == x.size(-1), "Linear4bit::forward: K differs");
+    const uint32_t K = x.size(-1), M = x.numel() / K, N = weight.size(0);
+    if (duq_quantize_linear4bit_workspace_bytes(M, N, K) != 0) return torch::Tensor();
+    std::vector<int64_t> shape(x.sizes().begin(), x.sizes().end());
+    shape.back() = N;
+    auto y = torch::empty(shape, torch::dtype(torch::kHalf).device(x.device()));
+    check_status(duq_quantize_linear4bit_forward(mode, half_ptr(x), input.clip, input.qmax, weight.data_ptr<uint8_t>(),
+                                                 half_ptr(s1), s2.defined() ? half_ptr(s2) : nullptr,
+                                                 bias.defined() ? half_ptr(bias) : nullptr, M, N, K,
+                                                 reinterpret_cast<duq_half *>(y.data_ptr()), nullptr, nullptr, nullptr, 0,
+                                                 current_stream(x)),
+                 "Linear4bit::forward");
+    return y;
+}
+
 inline torch::Tensor fused_forward(int mode, const PackedQuantizedTensor &input, const torch::Tensor &weight,
                                    const torch::Tensor &s1, const torch::Tensor &s2, const torch::Tensor &bias)
 {
@@ -308,6 +382,11 @@ public:
 
     torch::Tensor forward(PackedQuantizedTensor input)
     {
+        if (input.is_deferred()) {  // a few rows straight from Quantizer4bit: quantized inside the GEMM launch
+            auto y = detail::fused_decode(DUQ_EPI_SYM, input, weight, weight_scale.view(-1), torch::Tensor(), bias);
+            if (y.defined()) return y;
+            input.materialize();
+        }
         if (detail::use_shadow(input, weight_shadow, weight.size(0)))
             return detail::fused_forward_shadow(DUQ_EPI_SYM, input, weight_shadow, weight_scale.view(-1), torch::Tensor(), bias);
         return detail::fused_forward(DUQ_EPI_SYM, input, weight, weight_scale.view(-1), torch::Tensor(), bias);
@@ -353,6 +432,11 @@ public:
 
     torch::Tensor forward(PackedQuantizedTensor input)
     {
+        if (input.is_deferred()) {
+            auto y = detail::fused_decode(DUQ_EPI_SYM_DUAL, input, weight, weight_scale_1.view(-1), weight_scale_2.view(-1), bias);
+            if (y.defined()) return y;
+            input.materialize();
+        }
         if (detail::use_shadow(input, weight_shadow, weight.size(0)))
             return detail::fused_forward_shadow(DUQ_EPI_SYM_DUAL, input, weight_shadow, weight_scale_1.view(-1),
                                                 weight_scale_2.view(-1), bias);

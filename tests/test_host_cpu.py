@@ -285,3 +285,56 @@ def test_fp16_input_entry_point_validation_without_launch():
     assert lib.duq_quantize_linear4bit_workspace_bytes(64, 4, 64) == 64 * 32 + 128
     assert lib.duq_quantize_linear4bit_workspace_bytes(4, 4096, 4096) == 0
     assert lib.duq_quantize_linear4bit_workspace_bytes(4, 28672, 8192) == 4 * 4096 + 16
+
+
+def test_asym_fp16_input_entry_point_validation_without_launch():
+    from duqlinear4bitcuda_amd import _lib
+
+    lib = _lib.load()
+    P = 0x1000
+    f = lib.duq_quantize_linear4bit_forward_asym
+    tail = (None, None, None, None, None, 0, None)
+    assert f(0, P, P, P, P, None, None, None, None, 4, 4, 64, P, *tail) == -4      # symmetric modes: the other entry point
+    assert f(5, P, P, P, P, None, None, None, None, 4, 4, 64, P, *tail) == -4
+    assert f(1, P, P, P, P, None, None, None, None, 4, 4, 100, P, *tail) == -3     # K % 64
+    assert f(1, None, P, P, P, None, None, None, None, 4, 4, 64, P, *tail) == -1
+    assert f(1, P, P, P, None, None, None, None, None, 4, 4, 64, P, *tail) == -1   # asym needs weight zeros
+    assert f(3, P, P, P, P, P, None, None, None, 4, 4, 64, P, *tail) == -1         # dual needs the second pair
+    assert f(4, P, P, P, P, None, None, None, None, 4, 4, 64, P, *tail) == -1      # row-sum needs the weight term
+    assert f(1, P, P, P, P, None, None, None, None, 64, 4, 64, P, *tail) == -1     # needs a workspace
+    assert f(1, P, P, P, P, None, None, None, None, 64, 4, 64, P, None, None, None, None, P, 100, None) == -2
+    assert f(1, None, None, None, None, None, None, None, None, 0, 4, 64, None, *tail) == 0
+    g = lib.duq_quantize_linear4bit_asym_workspace_bytes
+    assert g(1, 64, 4, 64) == 64 * 32 + 128 + 128 and g(4, 64, 4, 64) == 64 * 32 + 128 + 128 + 256
+    assert g(1, 8, 4096, 4096) == 0 and g(2, 64, 4, 64) == 0
+    # the entry point that allocates nothing: slot and size limits are checked before anything else
+    s = lib.duq_quantize_linear4bit_forward_static
+    assert s(0, P, 1.0, 6, P, P, None, None, 8, 64, 64, P, None, None, 4, None) == -7   # no such slot
+    assert s(0, P, 1.0, 6, P, P, None, None, 4097, 64, 4096, P, None, None, 0, None) == -7
+    assert s(1, P, 1.0, 6, P, P, None, None, 8, 64, 64, P, None, None, 0, None) == -4
+    for code in (-7, -8, -9):
+        assert len(lib.duq_status_string(code)) > 10
+
+
+def test_deferred_quantized_tensor_host_side():
+    """What SymQuantizer hands over for a few rows: shape, device and the check that the rows were not written to,
+    without anything being computed (quantizing needs the GPU)."""
+    from duqlinear4bitcuda_amd import nn as qnn
+    from duqlinear4bitcuda_amd.tools import tensor_utils as tu
+
+    x = torch.zeros(2, 3, 128, dtype=torch.float16)
+    p = tu.PackedQuantizedTensor.deferred(x, 0.9, 7)
+    assert type(p) is tu.PackedQuantizedTensor
+    assert tuple(p.size()) == (2, 3, 64) and p.device.type == "cpu" and p.dtype == torch.uint8
+    assert p.source() is x and p.zeros_x is None and p.shadow_x is None and p.rowsum_x is None
+    x.add_(1)
+    with pytest.raises(RuntimeError, match="modified in place"):
+        p.source()
+    # CPU inputs are never deferred (the quantizer then fails in the op, like the reference binding)
+    with pytest.raises(RuntimeError):
+        qnn.SymQuantizer(1.0)(torch.zeros(2, 128, dtype=torch.float16))
+    # explicit fields behave like the reference's plain attributes
+    q = tu.PackedQuantizedTensor(torch.zeros(3, 8, dtype=torch.uint8), torch.ones(3, 1))
+    q.scales_x = torch.full((3, 1), 2.0)
+    q.quantized_x = torch.ones(3, 8, dtype=torch.uint8)
+    assert q.scales_x[0, 0] == 2 and q.quantized_x[0, 0] == 1 and q.source() is None

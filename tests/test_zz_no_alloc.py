@@ -15,7 +15,7 @@ def _say(*a):
     print(*a, flush=True)
 
 
-def _run_both(lib, dev, M, N, K, seed, dual_bias):
+def _run_both(lib, dev, M, N, K, seed, dual_bias, slot=0):
     x = cases.acts_outliers(M, K, seed=seed)
     wq, sw = cases.weights_random_nibbles(N, K, seed=seed + 1)
     rng = np.random.default_rng(seed)
@@ -34,7 +34,7 @@ def _run_both(lib, dev, M, N, K, seed, dual_bias):
                                                y_ref.data_ptr(), None, None, ws.data_ptr(), need, st) == 0
     before = torch.cuda.mem_get_info()[0]
     assert lib.duq_quantize_linear4bit_forward_static(mode, X.data_ptr(), 1.0, 6, W.data_ptr(), SW.data_ptr(), p2, pb, M,
-                                                      N, K, y_new.data_ptr(), None, None, st) == 0
+                                                      N, K, y_new.data_ptr(), None, None, slot, st) == 0
     torch.cuda.synchronize()
     after = torch.cuda.mem_get_info()[0]
     got, ref = y_new.cpu().numpy(), y_ref.cpu().numpy()
@@ -61,6 +61,9 @@ def test_static_scratch_entry_point_two_calls_second_smaller(dev):
     # a one-launch shape (up to four rows) goes through untouched by the scratch
     _say("static scratch: call 3, 3 x 2048 -> 128")
     _run_both(lib, dev, 3, 128, 2048, seed=45, dual_bias=False)
+    # another slot of the array: same bits (callers whose work may overlap on one GPU name different slots)
+    _say("static scratch: call 4, 40 x 512 -> 96, slot 3")
+    _run_both(lib, dev, 40, 96, 512, seed=47, dual_bias=True, slot=3)
 
 
 def test_static_scratch_limits_and_errors(dev):
@@ -70,8 +73,8 @@ def test_static_scratch_limits_and_errors(dev):
     st = torch.cuda.current_stream().cuda_stream
     one = torch.zeros(64, dtype=torch.uint8, device=dev)   # never dereferenced: every call below is rejected first
     p = one.data_ptr()
-    call = lambda M, N, K, mode=0: lib.duq_quantize_linear4bit_forward_static(mode, p, 1.0, 6, p, p, None, None, M, N, K,
-                                                                              p, None, None, st)
+    call = lambda M, N, K, mode=0, slot=0: lib.duq_quantize_linear4bit_forward_static(mode, p, 1.0, 6, p, p, None, None, M, N,
+                                                                                      K, p, None, None, slot, st)
     _say("static scratch: limits")
     assert call(4096, 64, 8192) == -7          # 16 MiB of codes
     assert call(4097, 64, 4096) == -7          # one row too many for 8 MiB
@@ -79,5 +82,43 @@ def test_static_scratch_limits_and_errors(dev):
     assert call(2, 64, 131072) == -6           # fits the scratch, rejected like everywhere else: K too large
     assert call(8, 64, 96) == -3 and call(8, 64, 256, mode=1) == -4
     assert b"scratch" in lib.duq_status_string(-7)
+    assert call(8, 64, 64, slot=4) == -7       # slots 0..3
+    assert lib.duq_static_scratch_init() == 0  # the address lookup, for callers that capture their first call
     assert call(0, 64, 64) == 0 and call(8, 0, 64) == 0   # nothing to do
     torch.cuda.synchronize()
+
+
+def test_static_scratch_two_streams_two_slots(dev):
+    """Two calls that may overlap in time (two streams, nothing ordering them) on two slots of the array: each gives
+    the bits of the workspace form."""
+    from duqlinear4bitcuda_amd import _lib
+
+    lib = _lib.load()
+    assert lib.duq_static_scratch_init() == 0
+    M, N, K = 512, 1024, 4096
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    work = []
+    for i, s in enumerate(streams):
+        x = cases.acts_outliers(M, K, seed=71 + i)
+        wq, sw = cases.weights_random_nibbles(N, K, seed=81 + i)
+        X, W, SW = (cases.t(a, dev) for a in (x, wq, sw))
+        need = lib.duq_quantize_linear4bit_workspace_bytes(M, N, K)
+        ws = torch.zeros(need, dtype=torch.uint8, device=dev)
+        y_ref = torch.zeros(M, N, dtype=torch.float16, device=dev)
+        y_new = torch.zeros(M, N, dtype=torch.float16, device=dev)
+        work.append((X, W, SW, ws, need, y_ref, y_new))
+    torch.cuda.synchronize()
+    _say("static scratch: two streams, slots 1 and 2")
+    for rep in range(3):
+        for i, s in enumerate(streams):
+            X, W, SW, ws, need, y_ref, y_new = work[i]
+            assert lib.duq_quantize_linear4bit_forward_static(0, X.data_ptr(), 1.0, 6, W.data_ptr(), SW.data_ptr(), None, None,
+                                                              M, N, K, y_new.data_ptr(), None, None, 1 + i, s.cuda_stream) == 0
+    torch.cuda.synchronize()
+    st = torch.cuda.current_stream().cuda_stream
+    for X, W, SW, ws, need, y_ref, y_new in work:
+        assert lib.duq_quantize_linear4bit_forward(0, X.data_ptr(), 1.0, 6, W.data_ptr(), SW.data_ptr(), None, None, M, N, K,
+                                                   y_ref.data_ptr(), None, None, ws.data_ptr(), need, st) == 0
+    torch.cuda.synchronize()
+    for X, W, SW, ws, need, y_ref, y_new in work:
+        assert cases.bits_equal(y_new.cpu().numpy(), y_ref.cpu().numpy())
