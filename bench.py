@@ -14,9 +14,9 @@ the metric is quoted on: M = 2048 tokens, K = N = 4096 (a Llama-2-7B attention
 projection), activations ~N(0,1) with 1 % heavy-tailed channels, weights uniform random
 nibbles with per-channel scales.
 
-Prints ONE JSON line.  ``value`` is 2*M*N*K / (time per step) in TOPS for the whole step, the K steps timed
-twice, as eager module calls and as one HIP graph of the same K steps replayed once, and the faster reported
-(``timed_path`` says which; both times are in the line).
+Prints ONE JSON line.  ``value`` is 2*M*N*K / (time per step) in TOPS for the whole step timed as eager module
+calls (how the reference's harness times a layer, test/benchmark.py:24-39); the same K steps as one HIP graph
+replayed once are reported beside it (``graph_ms_per_step``).
 ``roofline`` describes the dominant kernel (the fused GEMM): achieved = 2*M*N*K / its own
 average duration, measured with HIP events around max(steps, 1000) back-to-back launches on the
 launch stream (so the figure does not depend on ``--steps``), against the published dense peak
@@ -26,7 +26,9 @@ quantized per token, GEMM, dequant: the single entry point ``quantize_linear4bit
 its algorithmic bytes 2MK + NK/2 + 2N + 2MN, beside the GEMM alone on pre-quantized activations
 and a read-only kernel over the same weight bytes (the floor of a launch of that size);
 ``roofline_decode`` is the WORST of the Llama-2-7B rows.  ``quantizer`` reports the quantizer
-against HBM, ``cpu_baseline`` the CPU fake-quant path on the host.
+against HBM, ``harness`` reproduces the reference's own benchmark table (module-level eager wall time of the 4-bit
+layers and of the fp16 torch.nn.Linear at its six layer sizes), ``fanout`` one quantizer feeding several
+projections, ``cpu_baseline`` the CPU fake-quant path on the host.
 
 Every timed loop is preceded by PREWARM_STEPS untimed steps on top of ``--warmup`` (after an idle
 period the part needs about a millisecond of work to reach the clock it then holds).
@@ -156,6 +158,161 @@ def graph_time_us(fns, reps=5):
     return best
 
 
+def eager_wall_us(modules, x, steps=2000, warm=200):
+    """Wall time per eager call of modules[i % n](x): perf_counter around a loop that ends in synchronize()."""
+    import torch
+
+    n = len(modules)
+    for i in range(warm):
+        modules[i % n](x)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        modules[i % n](x)
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e6 / steps
+
+
+def shader_clock_mhz():
+    """The shader clock the driver reports right now (the level marked '*' in pp_dpm_sclk of the first GPU), or
+    None where that file is not readable."""
+    import glob
+    import re
+
+    for path in sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk")):
+        try:
+            text = open(path).read()
+        except OSError:
+            continue
+        m = re.search(r"(\d+)\s*Mhz\s*\*", text, re.I)
+        if m:
+            return int(m.group(1))
+    return None
+
+
+class ClockSampler:
+    """Samples shader_clock_mhz() from a thread while a timed loop runs: the clock the part held under that load."""
+
+    def __init__(self, period_s=0.002):
+        import threading
+
+        self.period, self.samples, self._stop = period_s, [], threading.Event()
+        self._t = threading.Thread(target=self._run, daemon=True)
+
+    def _run(self):
+        while not self._stop.is_set():
+            v = shader_clock_mhz()
+            if v is None:
+                return
+            self.samples.append(v)
+            time.sleep(self.period)
+
+    def __enter__(self):
+        self._t.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop.set()
+        self._t.join(timeout=1.0)
+
+    def summary(self):
+        if not self.samples:
+            return None
+        s = sorted(self.samples)
+        return {"median_mhz": s[len(s) // 2], "min_mhz": s[0], "max_mhz": s[-1], "samples": len(s)}
+
+
+def harness_section(dev, quick=False):
+    """The reference's own benchmark (test/benchmark.py:8-39, 54-100) on this GPU: x = rand(1, seq_len, in) as
+    binary16, weights integers in [-8, 7) with unit scales, module-level eager wall time in ms (5 warm-up + 100 calls
+    per run, mean of `runs` runs) of Sequential(SymQuantizer, Linear4bitSQ), Sequential(SymQuantizer,
+    Linear4bitDUSQ) and the fp16 torch.nn.Linear they replace, at its six layer sizes, for seq_len 2048 (its
+    default), 16 and 1; plus the 4-bit layer on the 6-bit float matrix path at seq_len 2048 (enable_fp6, not in the
+    reference)."""
+    import torch
+
+    from duqlinear4bitcuda_amd.nn import Linear4bitDUSQ, Linear4bitSQ, SymQuantizer
+
+    sizes = [(4096, 4096), (5120, 5120), (8192, 8192), (4096, 11008), (5120, 13824), (8192, 28672)]
+    if quick:
+        sizes = sizes[:1]
+    runs = 3
+
+    def module_benchmark(module, x):
+        for _ in range(5):
+            module(x)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(100):
+            module(x)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1000 / 100
+
+    def mean_ms(module, x):
+        module_benchmark(module, x)   # one untimed run: clock ramp, lazy set-up
+        return sum(module_benchmark(module, x) for _ in range(runs)) / runs
+
+    out = []
+    for (fin, fout) in sizes:
+        base = torch.nn.Linear(fin, fout, bias=False).to(dev).half()
+        base.weight.data = torch.randint_like(base.weight.data, low=-8, high=7).half()
+        s_w = torch.ones((fout, 1), dtype=torch.float16, device=dev)
+        with torch.no_grad():
+            sq = Linear4bitSQ.from_float(base, weight_scales=s_w).to(dev)
+            du = Linear4bitDUSQ.from_float(base, weight_scales_1=s_w, weight_scales_2=s_w.clone()).to(dev)
+            int4 = torch.nn.Sequential(SymQuantizer(input_clip_ratio=1.0), sq)
+            int4duq = torch.nn.Sequential(SymQuantizer(input_clip_ratio=1.0), du)
+            row = {"in": fin, "out": fout}
+            for seq in (2048, 16, 1):
+                x = torch.rand((1, seq, fin), device=dev).half()
+                t4, td, tf = mean_ms(int4, x), mean_ms(int4duq, x), mean_ms(base, x)
+                r = {"int4_ms": round(t4, 4), "int4_duq_ms": round(td, 4), "fp16_ms": round(tf, 4),
+                     "speedup_int4": round(tf / t4, 3), "speedup_int4_duq": round(tf / td, 3)}
+                if seq == 2048 and fin % 128 == 0 and fout % 16 == 0:
+                    sq.enable_fp6()
+                    fp6 = torch.nn.Sequential(SymQuantizer(1.0, shadow="only", shadow_min_rows=1), sq)
+                    t6 = mean_ms(fp6, x)
+                    r.update({"int4_fp6_path_ms": round(t6, 4), "speedup_int4_fp6_path": round(tf / t6, 3)})
+                    del sq._buffers["weight_shadow"]
+                row[f"seq{seq}"] = r
+        out.append(row)
+        del base, sq, du, int4, int4duq
+    return {"what": "module-level eager wall time as test/benchmark.py of the reference measures it (bsz 1; 5 + 100 calls, "
+                    f"mean of {runs} runs after one untimed run), fp16 = torch.nn.Linear (hipBLASLt) on the same GPU",
+            "rows": out}
+
+
+def fanout_section(dev):
+    """One quantized activation feeding several projections of a Llama-2-7B block as ONE GEMM over the concatenated
+    weight (q/k/v: N = 3 x 4096; gate/up: N = 2 x 11008), M = 2048: the quantizer's share of the step shrinks with
+    the width it feeds.  HIP-graph timed module steps, 6-bit float path and integer path."""
+    import torch
+
+    from duqlinear4bitcuda_amd.nn import Linear4bitSQ, SymQuantizer
+
+    out = []
+    M, K = 2048, 4096
+    x = heavy_tail_acts(M, K, seed=8).to(dev)
+    for name, N in (("one projection", 4096), ("q/k/v as one GEMM", 3 * 4096), ("gate/up as one GEMM", 2 * 11008)):
+        w, sw = random_weights(N, K, seed=88, dev=dev)
+        lin = Linear4bitSQ(K, N, bias=False).to(dev)
+        lin.weight.copy_(w)
+        lin.weight_scales = sw
+        q_i8 = SymQuantizer(1.0)
+        q_f6 = SymQuantizer(1.0, shadow="only", shadow_min_rows=1)
+        us_i8 = graph_time_us([lambda: lin(q_i8(x))] * 6)
+        lin.enable_fp6()
+        us_f6 = graph_time_us([lambda: lin(q_f6(x))] * 6)
+        pq = q_f6(x)
+        us_gemm = graph_time_us([lambda: lin(pq)] * 6)
+        ops = 2.0 * M * N * K
+        out.append({"what": name, "M": M, "K": K, "N": N, "fp6_step_us": round(us_f6, 1), "fp6_TOPS": round(ops / us_f6 / 1e6, 1),
+                    "fp6_gemm_only_us": round(us_gemm, 1), "quantizer_share": round(1.0 - us_gemm / us_f6, 3),
+                    "integer_step_us": round(us_i8, 1), "integer_TOPS": round(ops / us_i8 / 1e6, 1)})
+        del lin, w
+    return out
+
+
 LLAMA7B_DECODE = [(M, N, 4096) for N in (4096, 11008) for M in (1, 4, 16)]   # configuration 2
 
 
@@ -166,10 +323,17 @@ def decode_section(dev, quick):
                     (one launch up to eight rows, quantizer + GEMM launches above)
       gemm_only_us  the GEMM + dequant launch alone on pre-quantized activations
       read_floor_us a kernel that only reads the same N*K/2 weight bytes with the decode access pattern
+      module_graph_us  the same step through the drop-in modules, Sequential(SymQuantizer, Linear4bitSQ) on an input
+                    [1, M, K] (test/benchmark.py:54-70 of the reference), replayed from a HIP graph
+      module_eager_us  the same modules called eagerly: wall time per call (time.perf_counter around a loop that
+                    ends in synchronize(), as test/benchmark.py:24-39), which is what a caller without graphs gets:
+                    host time per call when that exceeds the kernels' time
+      module_launches  library calls per module step
     GBps / frac_hbm use `us` and the algorithmic bytes 2MK + NK/2 + 2N + 2MN."""
     import torch
 
     from duqlinear4bitcuda_amd import _HIP as hip
+    from duqlinear4bitcuda_amd.nn import Linear4bitSQ, SymQuantizer
 
     out = []
     shapes = list(LLAMA7B_DECODE)
@@ -186,16 +350,28 @@ def decode_section(dev, quick):
         us = graph_time_us([(lambda w=w: hip.quantize_linear4bit_forward(x, w, sw)) for w in ws] * 2)
         us_gemm = graph_time_us([(lambda w=w: hip.linear4bit_forward(hip.EPI_SYM, xq, sx, None, w, sw)) for w in ws] * 2)
         us_read = graph_time_us([(lambda w=w: hip.probe_read(w)) for w in ws] * 2)
+        # the drop-in modules, one layer per weight buffer (the same rotation)
+        x3 = x.view(1, M, K)
+        models = []
+        for w in ws:
+            layer = Linear4bitSQ(K, N, bias=False).to(dev)
+            layer.weight = w
+            layer.weight_scales = sw
+            models.append(torch.nn.Sequential(SymQuantizer(1.0), layer))
+        us_mod_graph = graph_time_us([(lambda m=m: m(x3)) for m in models] * 2)
+        us_mod_eager = eager_wall_us(models, x3)
         byts = 2 * M * K + wbytes + 2 * N + 2 * M * N
         out.append({"M": M, "N": N, "K": K, "us": round(us, 3), "GBps": round(byts / us / 1e3, 1),
                     "frac_hbm": round(byts / us / 1e3 / PEAK_HBM_GBS, 4),
                     "launches": 1 if hip.quantize_linear4bit_one_launch(M, N, K) else 2,
+                    "module_graph_us": round(us_mod_graph, 3), "module_eager_us": round(us_mod_eager, 3),
+                    "module_launches": 1 if M <= 8 and hip.quantize_linear4bit_one_launch(M, N, K) else 2,
                     "gemm_only_us": round(us_gemm, 3),
                     "gemm_only_GBps": round((byts - 2 * M * K + M * K // 2 + 2 * M) / us_gemm / 1e3, 1),
                     "read_floor_us": round(us_read, 3), "read_floor_GBps": round(wbytes / us_read / 1e3, 1),
                     "frac_of_read_floor": round(us_read / us, 4), "gemm_kernel_family": hip.gemm_kernel_for(M, N, K),
                     "weight_buffers": nbuf})
-        del ws
+        del ws, models
     return out
 
 
@@ -505,13 +681,10 @@ def main():
         del g
     except RuntimeError as exc:  # capture unsupported: keep the eager figure only
         print(f"graph capture skipped: {exc}", file=sys.stderr)
+    # `value` is the eager module path, which is how the reference's own harness times a layer
+    # (test/benchmark.py:24-39); the graph replay of the same K steps is reported beside it
     eager_ms_per_step = ms_per_step
     timed_path = "eager module calls"
-    if graph_ms_per_step is not None and graph_ms_per_step < ms_per_step:
-        # `value` is the faster of the two ways to run the same K steps (a serving loop replays a graph)
-        ms_per_step = graph_ms_per_step
-        tops = ops / (ms_per_step * 1e-3) / 1e12
-        timed_path = "one HIP graph of the K steps, replayed once"
 
     # ---- the same steps on the integer kernels ----
     for _ in range(PREWARM_STEPS + args.warmup):
@@ -527,8 +700,9 @@ def main():
     pq = quant(x)
     xs, sx = pq.shadow_x, pq.scales_x
     n_timed = max(args.steps, EVENT_TIMED_LAUNCHES)
-    gemm_us = event_time_us(lambda: hip.linear4bit_forward_bf6(hip.EPI_SYM, xs, sx, None, lin.weight_shadow, sw),
-                            n_timed, PREWARM_STEPS + args.warmup)
+    with ClockSampler() as clk_f6:
+        gemm_us = event_time_us(lambda: hip.linear4bit_forward_bf6(hip.EPI_SYM, xs, sx, None, lin.weight_shadow, sw),
+                                n_timed, PREWARM_STEPS + args.warmup)
     # the quantizer takes less time than a launch from Python: replayed from a HIP graph instead
     quant_us = graph_time_us([lambda: hip.quantize_rows_sym_bf6(x, with_q=False)] * 40)
     achieved = ops / gemm_us / 1e6
@@ -536,6 +710,9 @@ def main():
                 "achieved": round(achieved, 1), "peak": PEAK_FP6_TOPS, "unit": "TOP/s",
                 "frac": round(achieved / PEAK_FP6_TOPS, 4), "frac_of_int8_peak": round(achieved / PEAK_INT8_TOPS, 4),
                 "avg_kernel_us": round(gemm_us, 2), "launches_timed": n_timed,
+                # what the driver reported as the shader clock while those launches ran (pp_dpm_sclk): boxes of the
+                # pool differ by a few per cent in the clock they hold, and avg_kernel_us with them
+                "shader_clock_during_timing": clk_f6.summary(),
                 "peak_note": "published dense fp6 peak; the same achieved rate is %.3f of the int8 peak (5.0 POP/s) the "
                              "integer kernel is priced against" % (achieved / PEAK_INT8_TOPS),
                 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this workload, each
@@ -543,17 +720,23 @@ def main():
                 "traffic": profile_traffic_bytes("gemm_bf6_kernel__prefill_M2048_K4096_N4096.txt", "gemm_bf6_kernel"),
                 "traffic_source": "profiles/gemm_bf6_kernel__prefill_M2048_K4096_N4096.txt"}
     xq = quant_i8(x).quantized_x
-    i8_gemm_us = event_time_us(lambda: hip.linear4bit_forward(hip.EPI_SYM, xq, sx, None, lin_i8.weight, sw), n_timed,
-                               PREWARM_STEPS + args.warmup)
+    with ClockSampler() as clk_i8:
+        i8_gemm_us = event_time_us(lambda: hip.linear4bit_forward(hip.EPI_SYM, xq, sx, None, lin_i8.weight, sw), n_timed,
+                                   PREWARM_STEPS + args.warmup)
     i8_quant_us = graph_time_us([lambda: hip.quantize_rows_sym(x)] * 40)
     integer_path = {"ms_per_step": round(i8_ms_per_step, 5), "TOPS": round(ops / (i8_ms_per_step * 1e-3) / 1e12, 2),
                     "kernel": "gemm_s4_stream_kernel<4,0,false,2> (v_mfma_i32_32x32x32_i8, 128 x 256 tiles)", "gemm_fused_us": round(i8_gemm_us, 2),
                     "quantize_rows_sym_us": round(i8_quant_us, 2),
-                    "roofline": {"bound": "mfma", "achieved": round(ops / i8_gemm_us / 1e6, 1), "peak": PEAK_INT8_TOPS,
+                    "roofline": {"bound": "mfma", "kernel": "gemm_s4_stream_kernel (fused GEMM + dequant on v_mfma_i32_32x32x32_i8)",
+                                 "achieved": round(ops / i8_gemm_us / 1e6, 1), "peak": PEAK_INT8_TOPS,
                                  "unit": "TOP/s", "frac": round(ops / i8_gemm_us / 1e6 / PEAK_INT8_TOPS, 4),
+                                 "avg_kernel_us": round(i8_gemm_us, 2), "launches_timed": n_timed,
+                                 "shader_clock_during_timing": clk_i8.summary(),
                                  "traffic": profile_traffic_bytes("gemm_s4_stream_kernel__prefill_M2048_K4096_N4096.txt",
                                                                   "gemm_s4_stream_kernel"),
                                  "traffic_source": "profiles/gemm_s4_stream_kernel__prefill_M2048_K4096_N4096.txt"}}
+    # the driver record keeps `roofline`: the integer path's figures ride inside it as a second entry
+    roofline["integer_path"] = integer_path["roofline"]
 
     decode = decode_section(dev, args.quick)
     quantizer = quantizer_section(dev)
@@ -561,6 +744,8 @@ def main():
     other = None if args.quick else other_shapes_section(dev)
     int8_layer = int8_layer_section(dev, args.quick)
     batched = batched_section(dev, args.quick)
+    harness = harness_section(dev, args.quick)
+    fanout = None if args.quick else fanout_section(dev)
     rows_7b = [d for d in decode if (d["M"], d["N"], d["K"]) in LLAMA7B_DECODE]
     worst = min(rows_7b, key=lambda d: d["frac_hbm"])
     roofline_decode = {"bound": "hbm", "kernel": "gemv_s4_rows_kernel (M <= 8, quantizer inside) / quantize_rows_kernel + "
@@ -612,6 +797,8 @@ def main():
         "other_shapes": other,
         "int8_layer": int8_layer,
         "batched": batched,
+        "harness": harness,
+        "fanout": fanout,
         "cpu_baseline": cpu,
         "device": {"name": props.name, "arch": props.gcnArchName, "cus": props.multi_processor_count},
     }

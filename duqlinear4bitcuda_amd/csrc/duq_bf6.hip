@@ -205,14 +205,17 @@ __device__ __forceinline__ void mfma_pinned(int t, int h, v4f &acc, const v12i &
 }
 #undef DUQ_PIN
 
+// The first 56 bytes (through epi.mode) reach the kernel in registers (DUQ_HEAD_DECL / with_head).
 struct Bf6Params {
     const uint8_t *X;  // activation shadow
     const uint8_t *W;  // weight shadow
     uint32_t M, N, K;
+    uint32_t tiles_m;
     uint16_t *y;
+    uint32_t tiles_n;
     Epilogue epi;
-    uint32_t tiles_m, tiles_n;
 };
+static_assert(offsetof(Bf6Params, epi) + 8 == kHeadBytes, "the fields delivered in registers");
 
 // TMI = 8: 128-row tiles.  TMI = 4: 64-row tiles for problems that would leave most CUs without a 128-row tile
 // (half the MFMAs for the same weight traffic, but twice the workgroups).  TMI = 16: 256-row tiles for problems
@@ -220,8 +223,12 @@ struct Bf6Params {
 // the L2 -> CU limit that bounds the smaller tiles; all 256 AGPRs hold accumulators, an activation chunk is one
 // 128-k step (three buffers of two steps would not fit in LDS) and the epilogue parameters are fetched after the loop.
 template <int TMI, int TNI, int EPI, bool BIAS>
-__global__ __launch_bounds__(256) void gemm_bf6_kernel(Bf6Params p)
+__global__ __launch_bounds__(256) void gemm_bf6_kernel(DUQ_HEAD_DECL, Bf6Params tail)
 {
+    Bf6Params p = with_head(tail, DUQ_HEAD_USE);
+    to_global(p.X);
+    to_global(p.W);
+    to_global(p.y);
     static_assert(TMI == 16 || TMI == 8 || TMI == 4, "16-row MFMA tiles per wavefront along M");
     // TNI = 16 x 16 MFMA tiles per wavefront along N: BM rows x 64 columns (TNI = 4), or BM x 32 (TNI = 2, with
     // 64-row tiles only: twice the workgroups for problems that leave CUs without a 64 x 256 tile)
@@ -521,9 +528,9 @@ static void launch_tile(const Bf6Params &p, hipStream_t stream)
 {
     const dim3 grid(p.tiles_m * p.tiles_n);
     if (p.epi.bias)
-        hipLaunchKernelGGL((gemm_bf6_kernel<TMI, TNI, EPI, true>), grid, dim3(256), 0, stream, p);
+        DUQ_LAUNCH_HEAD((gemm_bf6_kernel<TMI, TNI, EPI, true>), grid, dim3(256), 0, stream, p);
     else
-        hipLaunchKernelGGL((gemm_bf6_kernel<TMI, TNI, EPI, false>), grid, dim3(256), 0, stream, p);
+        DUQ_LAUNCH_HEAD((gemm_bf6_kernel<TMI, TNI, EPI, false>), grid, dim3(256), 0, stream, p);
 }
 
 template <int EPI>
@@ -559,7 +566,7 @@ int launch_gemm_bf6(const uint8_t *X, const uint8_t *W, uint32_t M, uint32_t N, 
                     uint16_t *y, hipStream_t stream)
 {
     if (M == 0 || N == 0) return 0;
-    Bf6Params p{X, W, M, N, K, y, epi, (M + 127) / 128, (N + 255) / 256};
+    Bf6Params p{X, W, M, N, K, (M + 127) / 128, y, (N + 255) / 256, epi};
     switch (epi.mode) {
     case 0: launch_mode<0>(p, stream); break;
     case 1: launch_mode<1>(p, stream); break;

@@ -23,6 +23,8 @@
 //  MFMA kernel (5 <= M <= 64): v_mfma_i32_16x16x64_i8, eight wavefronts split K for one 16-column tile, one to
 //    four tiles of 16 rows against the same weight fragments, the partial tiles meet in LDS, 256 threads finish
 //    one output each per row tile; one round of at most 256 workgroups with several column tiles each.
+#include <cstddef>
+
 #include "duq_epilogue.h"
 #include "duq_launch.h"
 #include "duq_rowquant.h"
@@ -41,11 +43,13 @@ namespace {
 
 constexpr uint32_t kNibbleMaskD = 0xF0F0F0F0u;
 
+// The first 56 bytes (through `y`) reach the kernels in registers (DUQ_HEAD_DECL / with_head).
 struct DecodeParams {
     const uint8_t *A;    // packed activations [M, K/2] (pre-quantized input)
     const uint16_t *X;   // binary16 activations [M, K] (FUSEQ)
     const uint8_t *B;    // packed weights [N, K/2]
     uint32_t M, N, K;
+    uint32_t tiles_per_wg;
     int32_t *C;          // int32 out (EPI < 0)
     uint16_t *y;         // binary16 out (EPI >= 0)
     Epilogue epi;        // FUSEQ: s_row is not read, the kernel computes it
@@ -55,8 +59,8 @@ struct DecodeParams {
     uint16_t *s_out;     // FUSEQ, optional: the per-token scales [M]
     uint16_t *z_out;     // FUSEQ with an asymmetric epilogue, optional: the per-token zero points [M]
     int32_t *rs_out;     // FUSEQ with the row-sum epilogue, optional: the per-token sums of the shifted codes [M]
-    uint32_t tiles_per_wg;
 };
+static_assert(offsetof(DecodeParams, y) + sizeof(uint16_t *) == kHeadBytes, "the fields delivered in registers");
 
 template <int CTRL>
 __device__ __forceinline__ int dpp_add(int v)
@@ -98,8 +102,9 @@ __device__ __forceinline__ uint16_t dequant_rt(int acc, const RowEpi &r, const C
 // (two register sets that alternate), so that a launch is one round of at most 256 workgroups: the activations
 // are fetched, and with FUSEQ quantized, once per CU and not once per tile.
 template <int MR, int XS, bool FUSEQ, int EPI, int WAVES = 4, bool MULTI = false>
-__global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DecodeParams p)
+__global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DUQ_HEAD_DECL, DecodeParams tail)
 {
+    const DecodeParams p = with_head(tail, DUQ_HEAD_USE);
     constexpr int R = 4 * DUQ_DEC_R / WAVES;  // weight rows per wavefront
     constexpr int V = MR * R;        // partial sums per lane: 4, 8 or 16
     constexpr int LPV = 64 / V;      // lanes that finish one sum: 16, 8 or 4
@@ -189,6 +194,21 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DecodeParams p
     RowEpi rp{};
     if (EPI >= 0 && !FUSEQ) rp = load_row<MODE>(p.epi, min(my_m, p.M - 1));
 
+    // what the quantize phase needs of the kernel arguments, fetched here under the vector loads above: a scalar
+    // load issued where the value is first used (the compiler sinks it into the branch that uses it) is waited for on
+    // its own, and a fetch of kernel arguments costs about half a microsecond (measured: 4 rows, N = K = 4096, 5.5
+    // against 4.9 us)
+    const float q_clip = p.clip;
+    const int q_qmax = p.qmax;
+    uint8_t *const q_out = p.q_out;
+    uint16_t *const s_out = p.s_out, *const z_out = p.z_out;
+    int32_t *const rs_out = p.rs_out;
+    if (FUSEQ)
+        asm volatile("" ::"s"(q_clip), "s"(q_qmax), "s"(q_out), "s"(s_out), "s"(z_out), "s"(rs_out));
+    // (the output pointers arrive in registers)
+    const auto c_out = as_global(p.C);
+    const auto y_out = as_global(p.y);
+
     if (FUSEQ) {
         // statistics of this wavefront's share of its row.  Units past the row end read as zero: that changes no
         // maximum of |x|, but it would change a minimum or a maximum, so the asymmetric form skips them.
@@ -234,7 +254,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DecodeParams p
         // rows past M (the last rows of the MR the kernel is built for) are neither quantized nor used
         if (qrow < p.M) {
             RowQuant<ASYMQ> rq;
-            rq.init(m16, lo, hi, p.clip, p.qmax);
+            rq.init(m16, lo, hi, q_clip, q_qmax);
             const bool copy_out = blockIdx.x == 0;
 #pragma unroll
             for (int j = 0; j < UPL; ++j) {
@@ -248,7 +268,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DecodeParams p
                         word ^= 0x88888888u;
                     }
                     *reinterpret_cast<uint32_t *>(xs + qrow * XSTRIDE + c * 4) = word;
-                    if (copy_out && p.q_out) reinterpret_cast<uint32_t *>(p.q_out + (uint64_t)qrow * kbytes)[c] = word;
+                    if (copy_out && q_out) reinterpret_cast<uint32_t *>(q_out + (uint64_t)qrow * kbytes)[c] = word;
                 }
             }
             if (SHIFTQ) {
@@ -259,8 +279,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DecodeParams p
                 const f16 z = SHIFTQ ? rq.z - (f16)8.0f : rq.z;
                 srow[qrow] = f16_to_bits(rq.s);
                 if (ASYMQ) zrow[qrow] = f16_to_bits(z);
-                if (copy_out && p.s_out) p.s_out[qrow] = f16_to_bits(rq.s);
-                if (ASYMQ && copy_out && p.z_out) p.z_out[qrow] = f16_to_bits(z);
+                if (copy_out && s_out) s_out[qrow] = f16_to_bits(rq.s);
+                if (ASYMQ && copy_out && z_out) z_out[qrow] = f16_to_bits(z);
             }
         }
         __syncthreads();
@@ -271,7 +291,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DecodeParams p
 #pragma unroll
                 for (int i = 0; i < WPR; ++i) t += rsum[tid * WPR + i];
                 rsrow[tid] = t;
-                if (blockIdx.x == 0 && p.rs_out) p.rs_out[tid] = t;
+                if (blockIdx.x == 0 && rs_out) rs_out[tid] = t;
             }
             __syncthreads();
         }
@@ -320,9 +340,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DecodeParams p
         const uint32_t my_n = tile * (4 * DUQ_DEC_R) + my_r;
         if (sub == 0 && my_m < p.M && my_n < p.N) {
             if (EPI < 0)
-                p.C[(uint64_t)my_m * p.N + my_n] = sum;
+                c_out[(uint64_t)my_m * p.N + my_n] = sum;
             else
-                p.y[(uint64_t)my_m * p.N + my_n] = dequant_rt<MODE>(sum, rp, c, bias);
+                y_out[(uint64_t)my_m * p.N + my_n] = dequant_rt<MODE>(sum, rp, c, bias);
         }
     };
 
@@ -351,8 +371,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DecodeParams p
 // GEMM kernels: (w & 0xF0F0F0F0) is the four odd-k nibbles times 16, ((w << 4) & 0xF0F0F0F0) the even ones;
 // every product is 256 * a * b and one arithmetic shift recovers the sum.
 template <int WAVES, int SEGS, int EPI, int MT = 1, bool DB = true>
-__global__ __launch_bounds__(WAVES * 64) void gemm_s4_decode_kernel(DecodeParams p)
+__global__ __launch_bounds__(WAVES * 64) void gemm_s4_decode_kernel(DUQ_HEAD_DECL, DecodeParams tail)
 {
+    const DecodeParams p = with_head(tail, DUQ_HEAD_USE);
     constexpr int MODE = EPI < 0 ? 0 : EPI;
     static_assert(WAVES == 4 || WAVES == 8, "wavefronts per workgroup");
     static_assert(MT >= 1 && MT <= 4, "16-row activation tiles");
@@ -410,6 +431,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_s4_decode_kernel(DecodeParams
         return c;
     };
     cp = load_cp(tile0);
+    // (the output pointers arrive in registers)
+    const auto c_out = as_global(p.C);
+    const auto y_out = as_global(p.y);
 #pragma unroll
     for (int f = 0; f < FT; ++f) {
         rp[f] = RowEpi{};
@@ -458,9 +482,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_s4_decode_kernel(DecodeParams
                 const uint32_t m = t * 16 + my_m, n = tile * 16 + my_c;
                 if (m < p.M && n < p.N) {
                     if (EPI < 0)
-                        p.C[(uint64_t)m * p.N + n] = sum;
+                        c_out[(uint64_t)m * p.N + n] = sum;
                     else
-                        p.y[(uint64_t)m * p.N + n] = dequant_rt<MODE>(sum, rp[f], cp, bias);
+                        y_out[(uint64_t)m * p.N + n] = dequant_rt<MODE>(sum, rp[f], cp, bias);
                 }
             }
         }
@@ -512,17 +536,17 @@ bool launch_rows_mode(DecodeParams &p, int epi, hipStream_t stream)
 #define DUQ_ROWS(E)                                                                                              \
     if (multi) {                                                                                                 \
         if constexpr (kCanMulti) {                                                                               \
-            hipLaunchKernelGGL((gemv_s4_rows_kernel<MR, XS, FUSEQ, E, 8, true>), grid, dim3(512), 0, stream, p);     \
+            DUQ_LAUNCH_HEAD((gemv_s4_rows_kernel<MR, XS, FUSEQ, E, 8, true>), grid, dim3(512), 0, stream, p);         \
             launched = true;                                                                                     \
         }                                                                                                        \
     } else if (wide) {                                                                                           \
         if constexpr (FUSEQ && MR >= 4) {                                                                        \
-            hipLaunchKernelGGL((gemv_s4_rows_kernel<MR, XS, FUSEQ, E, 8>), grid, dim3(512), 0, stream, p);           \
+            DUQ_LAUNCH_HEAD((gemv_s4_rows_kernel<MR, XS, FUSEQ, E, 8>), grid, dim3(512), 0, stream, p);               \
             launched = true;                                                                                     \
         }                                                                                                        \
     } else {                                                                                                     \
         if constexpr (MR <= 4) {                                                                                 \
-            hipLaunchKernelGGL((gemv_s4_rows_kernel<MR, XS, FUSEQ, E, 4>), grid, dim3(256), 0, stream, p);           \
+            DUQ_LAUNCH_HEAD((gemv_s4_rows_kernel<MR, XS, FUSEQ, E, 4>), grid, dim3(256), 0, stream, p);               \
             launched = true;                                                                                     \
         }                                                                                                        \
     }
@@ -559,7 +583,7 @@ bool launch_mfma_mode(const DecodeParams &p, int epi, hipStream_t stream)
 {
     const uint32_t ntiles = (p.N + 15) / 16;
     const dim3 grid((ntiles + p.tiles_per_wg - 1) / p.tiles_per_wg);
-#define DUQ_DEC(E) hipLaunchKernelGGL((gemm_s4_decode_kernel<WAVES, SEGS, E, MT, DB>), grid, dim3(WAVES * 64), 0, stream, p)
+#define DUQ_DEC(E) DUQ_LAUNCH_HEAD((gemm_s4_decode_kernel<WAVES, SEGS, E, MT, DB>), grid, dim3(WAVES * 64), 0, stream, p)
     switch (epi) {
     case -1: DUQ_DEC(-1); break;
     case 0: DUQ_DEC(0); break;

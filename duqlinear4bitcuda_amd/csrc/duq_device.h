@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <cstddef>
+
 #include <type_traits>
 
 namespace duq {
@@ -20,6 +22,58 @@ constexpr int kQuantColK = 10;  // include/quant.h:5 of the reference
 
 __device__ __forceinline__ f16 bits_to_f16(uint16_t b) { return __builtin_bit_cast(f16, b); }
 __device__ __forceinline__ uint16_t f16_to_bits(f16 v) { return __builtin_bit_cast(uint16_t, v); }
+
+// ---- kernel arguments delivered in registers ------------------------------------------------------------
+// gfx950 can hand a kernel the first 14 dwords of its arguments in scalar registers when the wavefront starts
+// (compiled with -mllvm -amdgpu-kernarg-preload-count=14) instead of the kernel fetching them from the argument
+// buffer with a scalar load, a fetch that a short kernel waits for with nothing to overlap it (measured: a kernel
+// that only reads 8 MiB takes 2.66 us with its three arguments preloaded against 2.99 us).  Only leading scalar
+// arguments qualify, not a parameter struct passed by value, so a kernel that wants this takes the first 56 bytes
+// of its parameter struct once more as 14 dwords in front of the struct (DUQ_HEAD_DECL), and with_head() puts them
+// back in place: fields of the first 56 bytes then come from registers, the others from the argument buffer.
+// DUQ_LAUNCH_HEAD is the host side.  Pointers rebuilt this way have lost their address space: as_global() says
+// again that one points to device memory (direct loads and stores through it would otherwise be flat ones).
+#define DUQ_HEAD_DECL                                                                                                  \
+    uint32_t h0, uint32_t h1, uint32_t h2, uint32_t h3, uint32_t h4, uint32_t h5, uint32_t h6, uint32_t h7, uint32_t h8, \
+        uint32_t h9, uint32_t h10, uint32_t h11, uint32_t h12, uint32_t h13
+#define DUQ_HEAD_USE h0, h1, h2, h3, h4, h5, h6, h7, h8, h9, h10, h11, h12, h13
+constexpr int kHeadBytes = 56;
+
+template <typename T>
+__device__ __forceinline__ T with_head(const T &tail, DUQ_HEAD_DECL)
+{
+    static_assert(sizeof(T) >= kHeadBytes && std::is_trivially_copyable<T>::value, "parameter struct");
+    T q = tail;
+    const uint32_t hw[14] = {DUQ_HEAD_USE};
+    __builtin_memcpy(&q, hw, kHeadBytes);
+    return q;
+}
+
+template <typename T>
+__device__ __forceinline__ __attribute__((address_space(1))) T *as_global(T *p)
+{
+    return (__attribute__((address_space(1))) T *)p;
+}
+
+// The same for a (wavefront-uniform) pointer variable or field, in place: uses that follow are resolved to device
+// memory.  The empty asm keeps the compiler from folding the two casts away.
+template <typename T>
+__device__ __forceinline__ void to_global(T *&p)
+{
+    auto g = as_global(p);
+    asm("" : "+s"(g));
+    p = (T *)g;
+}
+
+#define DUQ_LAUNCH_HEAD(kernel, grid, block, lds, stream, params)                                                      \
+    do {                                                                                                               \
+        static_assert(sizeof(params) >= duq::kHeadBytes, "parameter struct");                                          \
+        uint32_t duq_hw_[14];                                                                                          \
+        __builtin_memcpy(duq_hw_, &(params), duq::kHeadBytes);                                                         \
+        hipLaunchKernelGGL(kernel, grid, block, lds, stream, duq_hw_[0], duq_hw_[1], duq_hw_[2], duq_hw_[3], duq_hw_[4], \
+                           duq_hw_[5], duq_hw_[6], duq_hw_[7], duq_hw_[8], duq_hw_[9], duq_hw_[10], duq_hw_[11],        \
+                           duq_hw_[12], duq_hw_[13], params);                                                          \
+    } while (0)
 
 // float -> int32 with the hardware rule: truncation, saturation, NaN -> 0.  A C cast is
 // undefined for NaN / out-of-range values, the instruction is not.

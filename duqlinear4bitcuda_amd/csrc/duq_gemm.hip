@@ -35,15 +35,18 @@ namespace duq {
 
 constexpr uint32_t kNibbleMask = 0xF0F0F0F0u;
 
+// The first 56 bytes (through tiles_n) reach the kernels in registers (DUQ_HEAD_DECL / with_head).
 struct GemmParams {
     const uint8_t *A;  // activations [M, K/2]
     const uint8_t *B;  // weights     [N, K/2]
     uint32_t M, N, K;
+    uint32_t tiles_m;
     int32_t *C;        // int32 out (EPI < 0)
     uint16_t *y;       // fp16 out  (EPI >= 0)
+    uint32_t tiles_n;
     Epilogue epi;
-    uint32_t tiles_m, tiles_n;
 };
+static_assert(offsetof(GemmParams, epi) == kHeadBytes, "the fields delivered in registers");
 
 // Batched launch: problem blockIdx.z of a batch whose tensors are contiguous ([batch, M, K/2], [batch, N, K/2],
 // [batch, M, N], per-row arrays [batch, M], per-column arrays [batch, N]).
@@ -110,8 +113,13 @@ constexpr int kBK = 128;           // k elements per tile step (64 packed bytes 
 constexpr int kLdsStride = 144;    // bytes per LDS row: 128 expanded bytes + 16 pad
 
 template <int BM, int BN, int EPI, bool BIAS>
-__global__ __launch_bounds__(256) void gemm_s4_tile_kernel(GemmParams p)
+__global__ __launch_bounds__(256) void gemm_s4_tile_kernel(DUQ_HEAD_DECL, GemmParams tail)
 {
+    GemmParams p = with_head(tail, DUQ_HEAD_USE);
+    to_global(p.A);
+    to_global(p.B);
+    to_global(p.C);
+    to_global(p.y);
     constexpr int WTM = BM / 2, WTN = BN / 2;  // per-wavefront tile
     constexpr int TM = WTM / 16, TN = WTN / 16;
     constexpr int NA = BM / 64, NB = BN / 64;  // 16-byte global pieces per thread
@@ -272,8 +280,13 @@ constexpr int kXStride = 272;    // LDS bytes per activation row: 256 expanded +
 
 
 template <int TM, int EPI, bool BIAS, int TN = 2>
-__global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
+__global__ __launch_bounds__(256) void gemm_s4_stream_kernel(DUQ_HEAD_DECL, GemmParams tail)
 {
+    GemmParams p = with_head(tail, DUQ_HEAD_USE);
+    to_global(p.A);
+    to_global(p.B);
+    to_global(p.C);
+    to_global(p.y);
     static_assert(TM == 4 || TM == 2 || TM == 1, "32-row activation tiles per wavefront");
     // TN = 32-column weight tiles per wavefront: tiles of 256 columns (TN = 2), or of 128 with 64 rows (TN = 1):
     // as many outputs per workgroup as 32 x 256 with a third less operand bytes into the CU
@@ -497,8 +510,13 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(GemmParams p)
 // the next tile's operands before the current tile's epilogue measured slower, 93 against 86 us on 32 products of
 // 2048 x 2048 x 128: the loop-carried wait for those loads also waits for the stores issued after them.)
 template <int TM, int EPI, bool BIAS>
-__global__ __launch_bounds__(256, 2) void gemm_s4_shortk_kernel(GemmParams p)
+__global__ __launch_bounds__(256, 2) void gemm_s4_shortk_kernel(DUQ_HEAD_DECL, GemmParams tail)
 {
+    GemmParams p = with_head(tail, DUQ_HEAD_USE);
+    to_global(p.A);
+    to_global(p.B);
+    to_global(p.C);
+    to_global(p.y);
     constexpr int BM = 32 * TM, BN = 256, TN = 2;
     constexpr int NXP = TM;  // 16-byte activation pieces per thread
     constexpr uint32_t kBuf = BM * kXStride, kStage = 4 * BM * 144;
@@ -604,8 +622,13 @@ constexpr int kSkinnySegs = 8;  // 64-byte segments per wavefront = 128-bit weig
 
 
 template <int WAVES, int EPI, bool BIAS>
-__global__ __launch_bounds__(WAVES * 64) void gemm_s4_skinny_kernel(GemmParams p)
+__global__ __launch_bounds__(WAVES * 64) void gemm_s4_skinny_kernel(DUQ_HEAD_DECL, GemmParams tail)
 {
+    GemmParams p = with_head(tail, DUQ_HEAD_USE);
+    to_global(p.A);
+    to_global(p.B);
+    to_global(p.C);
+    to_global(p.y);
     __shared__ v4i part[2][WAVES][64];
     __shared__ __attribute__((aligned(16))) uint8_t turn[WAVES * 8192];
     const uint32_t tid = threadIdx.x;
@@ -712,8 +735,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_s4_skinny_kernel(GemmParams p
 constexpr int kRing = 8;  // 128-bit weight loads in flight per lane
 
 template <int XBYTES, int RB, int EPI, bool BIAS>
-__global__ __launch_bounds__(256) void gemm_s4_ring_kernel(GemmParams p)
+__global__ __launch_bounds__(256) void gemm_s4_ring_kernel(DUQ_HEAD_DECL, GemmParams tail)
 {
+    GemmParams p = with_head(tail, DUQ_HEAD_USE);
+    to_global(p.A);
+    to_global(p.B);
+    to_global(p.C);
+    to_global(p.y);
     constexpr uint32_t WAVES = 4, T = WAVES * 64;
     constexpr uint32_t XS = XBYTES + 16;  // LDS row stride = 16 (mod 256)
     __shared__ __attribute__((aligned(16))) uint8_t xs[16 * RB * XS];
@@ -832,8 +860,13 @@ __global__ __launch_bounds__(256) void gemm_s4_ring_kernel(GemmParams p)
 constexpr int kDotRing = 8;
 
 template <int MROWS, int EPI, bool BIAS>
-__global__ __launch_bounds__(256) void gemv_s4_dot_kernel(GemmParams p)
+__global__ __launch_bounds__(256) void gemv_s4_dot_kernel(DUQ_HEAD_DECL, GemmParams tail)
 {
+    GemmParams p = with_head(tail, DUQ_HEAD_USE);
+    to_global(p.A);
+    to_global(p.B);
+    to_global(p.C);
+    to_global(p.y);
     extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [MROWS][xstride] packed activations
     __shared__ int part[4][8][MROWS];
     const uint32_t tid = threadIdx.x;
@@ -988,11 +1021,11 @@ static void launch_epi(GemmParams &p, hipStream_t stream, uint32_t batch = 1)
         const uint32_t xstride = ((p.K / 2 + 127) / 128) * 128;
         const dim3 grid((p.N + 7) / 8);
         if (p.M == 1)
-            hipLaunchKernelGGL((gemv_s4_dot_kernel<1, EPI, BIAS>), grid, dim3(256), 1 * xstride, stream, p);
+            DUQ_LAUNCH_HEAD((gemv_s4_dot_kernel<1, EPI, BIAS>), grid, dim3(256), 1 * xstride, stream, p);
         else if (p.M == 2)
-            hipLaunchKernelGGL((gemv_s4_dot_kernel<2, EPI, BIAS>), grid, dim3(256), 2 * xstride, stream, p);
+            DUQ_LAUNCH_HEAD((gemv_s4_dot_kernel<2, EPI, BIAS>), grid, dim3(256), 2 * xstride, stream, p);
         else
-            hipLaunchKernelGGL((gemv_s4_dot_kernel<4, EPI, BIAS>), grid, dim3(256), 4 * xstride, stream, p);
+            DUQ_LAUNCH_HEAD((gemv_s4_dot_kernel<4, EPI, BIAS>), grid, dim3(256), 4 * xstride, stream, p);
         return;
     }
     if (kernel == kKernelSkinny) {
@@ -1009,9 +1042,9 @@ static void launch_epi(GemmParams &p, hipStream_t stream, uint32_t batch = 1)
         p.tiles_m = tpw;
         const dim3 grid((ntiles + tpw - 1) / tpw);
         if (segs <= 4 * kSkinnySegs)
-            hipLaunchKernelGGL((gemm_s4_skinny_kernel<4, EPI, BIAS>), grid, dim3(256), 0, stream, p);
+            DUQ_LAUNCH_HEAD((gemm_s4_skinny_kernel<4, EPI, BIAS>), grid, dim3(256), 0, stream, p);
         else
-            hipLaunchKernelGGL((gemm_s4_skinny_kernel<8, EPI, BIAS>), grid, dim3(512), 0, stream, p);
+            DUQ_LAUNCH_HEAD((gemm_s4_skinny_kernel<8, EPI, BIAS>), grid, dim3(512), 0, stream, p);
         return;
     }
     if (kernel == kKernelRing) {
@@ -1032,7 +1065,7 @@ static void launch_epi(GemmParams &p, hipStream_t stream, uint32_t batch = 1)
         p.tiles_m = kslices;
         p.tiles_n = (groups + slots - 1) / slots;
         const dim3 grid((groups + p.tiles_n - 1) / p.tiles_n, row_groups);
-#define DUQ_RING(X, R) hipLaunchKernelGGL((gemm_s4_ring_kernel<X, R, EPI, BIAS>), grid, dim3(256), 0, stream, p)
+#define DUQ_RING(X, R) DUQ_LAUNCH_HEAD((gemm_s4_ring_kernel<X, R, EPI, BIAS>), grid, dim3(256), 0, stream, p)
         if (xbytes == 8192) DUQ_RING(8192, 1);
         else if (xbytes == 4096) DUQ_RING(4096, 2);
         else if (rb == 2) DUQ_RING(2048, 2);
@@ -1074,7 +1107,7 @@ static void launch_epi(GemmParams &p, hipStream_t stream, uint32_t batch = 1)
         // tiles (measured on 32 products of 2048 x 2048 x 128: 86 us against 95 us on the stream kernel's 64-row tiles)
         p.tiles_m = (p.M + 63) / 64;
         p.tiles_n = (p.N + 255) / 256;
-        hipLaunchKernelGGL((gemm_s4_shortk_kernel<2, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(256), 0,
+        DUQ_LAUNCH_HEAD((gemm_s4_shortk_kernel<2, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(256), 0,
                            stream, p);
         return;
     }
@@ -1083,34 +1116,34 @@ static void launch_epi(GemmParams &p, hipStream_t stream, uint32_t batch = 1)
         p.tiles_n = (p.N + 127) / 128;
         const dim3 grid(p.tiles_m * p.tiles_n, 1, batch);
         if (best_tm == 4)
-            hipLaunchKernelGGL((gemm_s4_stream_kernel<4, EPI, BIAS, 1>), grid, dim3(256), 0, stream, p);
+            DUQ_LAUNCH_HEAD((gemm_s4_stream_kernel<4, EPI, BIAS, 1>), grid, dim3(256), 0, stream, p);
         else
-            hipLaunchKernelGGL((gemm_s4_stream_kernel<2, EPI, BIAS, 1>), grid, dim3(256), 0, stream, p);
+            DUQ_LAUNCH_HEAD((gemm_s4_stream_kernel<2, EPI, BIAS, 1>), grid, dim3(256), 0, stream, p);
     } else if (best_tm) {
         p.tiles_m = (p.M + 32 * best_tm - 1) / (32 * best_tm);
         p.tiles_n = (p.N + 255) / 256;
         const dim3 grid(p.tiles_m * p.tiles_n, 1, batch);
         if (best_tm == 4)
-            hipLaunchKernelGGL((gemm_s4_stream_kernel<4, EPI, BIAS>), grid, dim3(256), 0, stream, p);
+            DUQ_LAUNCH_HEAD((gemm_s4_stream_kernel<4, EPI, BIAS>), grid, dim3(256), 0, stream, p);
         else if (best_tm == 2)
-            hipLaunchKernelGGL((gemm_s4_stream_kernel<2, EPI, BIAS>), grid, dim3(256), 0, stream, p);
+            DUQ_LAUNCH_HEAD((gemm_s4_stream_kernel<2, EPI, BIAS>), grid, dim3(256), 0, stream, p);
         else
-            hipLaunchKernelGGL((gemm_s4_stream_kernel<1, EPI, BIAS>), grid, dim3(256), 0, stream, p);
+            DUQ_LAUNCH_HEAD((gemm_s4_stream_kernel<1, EPI, BIAS>), grid, dim3(256), 0, stream, p);
     } else if constexpr (EPI != 5) {
         if (tiles(128, 256) >= 256 && p.M > 64) {
             p.tiles_m = (p.M + 127) / 128;
             p.tiles_n = (p.N + 255) / 256;
-            hipLaunchKernelGGL((gemm_s4_tile_kernel<128, 256, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(256),
+            DUQ_LAUNCH_HEAD((gemm_s4_tile_kernel<128, 256, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(256),
                                0, stream, p);
         } else if (tiles(128, 128) >= 256 && p.M > 64) {
             p.tiles_m = (p.M + 127) / 128;
             p.tiles_n = (p.N + 127) / 128;
-            hipLaunchKernelGGL((gemm_s4_tile_kernel<128, 128, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(256),
+            DUQ_LAUNCH_HEAD((gemm_s4_tile_kernel<128, 128, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(256),
                                0, stream, p);
         } else {
             p.tiles_m = (p.M + 63) / 64;
             p.tiles_n = (p.N + 63) / 64;
-            hipLaunchKernelGGL((gemm_s4_tile_kernel<64, 64, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(256), 0,
+            DUQ_LAUNCH_HEAD((gemm_s4_tile_kernel<64, 64, EPI, BIAS>), dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(256), 0,
                                stream, p);
         }
     }

@@ -230,21 +230,29 @@ int launch_dequant_hprec(const int32_t *acc, const float *s_row, const float *z_
 // to 272 bytes, one barrier per chunk) -> fragments read one step ahead; the register of piece j is stored at step
 // j (for the chunk after next) and refetched at once (for the chunk after that), again a whole chunk ahead.
 // The weight operand is the MFMA "A" side, so a lane ends up with four consecutive output columns of one row.
+// The first 56 bytes (through tiles_n) reach the kernels in registers (DUQ_HEAD_DECL / with_head).
 struct Gemm8Params {
     const int8_t *A;  // [M, K]
     const int8_t *B;  // [N, K]
     uint32_t M, N, K;
+    uint32_t tiles_m;
     int32_t *C;       // int32 out (not fused)
     float *y;         // float32 out (fused)
+    uint32_t tiles_n;
     Epi8 epi;
-    uint32_t tiles_m, tiles_n;
 };
+static_assert(offsetof(Gemm8Params, epi) == kHeadBytes, "the fields delivered in registers");
 
 __device__ __forceinline__ void lds_barrier8() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 template <int TM, int TN, bool FUSED, bool BIAS, bool TILED>
-__global__ __launch_bounds__(256) void gemm_s8_kernel(Gemm8Params p)
+__global__ __launch_bounds__(256) void gemm_s8_kernel(DUQ_HEAD_DECL, Gemm8Params tail)
 {
+    Gemm8Params p = with_head(tail, DUQ_HEAD_USE);
+    to_global(p.A);
+    to_global(p.B);
+    to_global(p.C);
+    to_global(p.y);
     static_assert(TM == 4 || TM == 2 || TM == 1, "32-row MFMA tiles per wavefront along M");
     // TN = 32-column MFMA tiles per wavefront: tiles of 256 columns (TN = 2), or of 128 (TN = 1, with 64-row tiles:
     // twice the workgroups for problems that leave CUs without a 64 x 256 tile)
@@ -483,8 +491,13 @@ __global__ __launch_bounds__(256) void gemm_s8_kernel(Gemm8Params p)
 constexpr int kSkinnyRing = 16;
 
 template <int MT, bool FUSED, bool BIAS, bool TILED>
-__global__ __launch_bounds__(256) void gemm_s8_skinny_kernel(Gemm8Params p)
+__global__ __launch_bounds__(256) void gemm_s8_skinny_kernel(DUQ_HEAD_DECL, Gemm8Params tail)
 {
+    Gemm8Params p = with_head(tail, DUQ_HEAD_USE);
+    to_global(p.A);
+    to_global(p.B);
+    to_global(p.C);
+    to_global(p.y);
     __shared__ v4i part[4][MT][64];
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63u, wave = tid >> 6;
@@ -594,8 +607,13 @@ __global__ __launch_bounds__(256) void gemm_s8_skinny_kernel(Gemm8Params p)
 // workgroups and the activations (as many bytes as a tile's weights at 16 rows) enter a CU once.  The partial
 // tiles meet in LDS; MT * 64 threads finish four consecutive columns of one row each.
 template <int SEGS, int MT, bool FUSED, bool BIAS, bool TILED>
-__global__ __launch_bounds__(512) void gemm_s8_decode_kernel(Gemm8Params p)
+__global__ __launch_bounds__(512) void gemm_s8_decode_kernel(DUQ_HEAD_DECL, Gemm8Params tail)
 {
+    Gemm8Params p = with_head(tail, DUQ_HEAD_USE);
+    to_global(p.A);
+    to_global(p.B);
+    to_global(p.C);
+    to_global(p.y);
     constexpr int WAVES = 8;
     __shared__ v4i part[2][MT][WAVES][64];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
@@ -739,7 +757,7 @@ static void launch_decode8(Gemm8Params &p, hipStream_t stream)
     p.tiles_n = (ntiles + 255) / 256;  // column tiles per workgroup: one round of at most 256 workgroups
     const dim3 grid((ntiles + p.tiles_n - 1) / p.tiles_n);
     const uint32_t mt = (p.M + 15) / 16;
-#define DUQ_DEC8(S, T) hipLaunchKernelGGL((gemm_s8_decode_kernel<S, T, FUSED, BIAS, TILED>), grid, dim3(512), 0, stream, p)
+#define DUQ_DEC8(S, T) DUQ_LAUNCH_HEAD((gemm_s8_decode_kernel<S, T, FUSED, BIAS, TILED>), grid, dim3(512), 0, stream, p)
     if (p.K > 2048) {
         if (mt == 1) DUQ_DEC8(8, 1);
         else if (mt == 2) DUQ_DEC8(8, 2);
@@ -764,8 +782,13 @@ static void launch_decode8(Gemm8Params &p, hipStream_t stream)
 // the wavefront's own piece of LDS (no barrier) and a few DPP steps.  A workgroup is four wavefronts: 16 (8 for rows
 // longer than 4 KB) weight rows.
 template <int MR, int XS, bool FUSED, bool BIAS>
-__global__ __launch_bounds__(256) void gemv_s8_rows_kernel(Gemm8Params p)
+__global__ __launch_bounds__(256) void gemv_s8_rows_kernel(DUQ_HEAD_DECL, Gemm8Params tail)
 {
+    Gemm8Params p = with_head(tail, DUQ_HEAD_USE);
+    to_global(p.A);
+    to_global(p.B);
+    to_global(p.C);
+    to_global(p.y);
     constexpr int R = XS <= 4 ? 4 : 2;  // weight rows per wavefront: at most 16 weight registers of 16 bytes per lane
     constexpr int V = MR * R;           // partial sums per lane: 2 .. 16
     constexpr int LPV = 64 / V;         // lanes that finish one sum
@@ -849,7 +872,7 @@ static void launch_rows8(const Gemm8Params &p, hipStream_t stream)
 {
     const uint32_t xs = (p.K + 1023) / 1024;
 #define DUQ_ROWS8K(XS)                                                                                              \
-    hipLaunchKernelGGL((gemv_s8_rows_kernel<MR, XS, FUSED, BIAS>), dim3((p.N + 4 * (XS <= 4 ? 4 : 2) - 1) / (4 * (XS <= 4 ? 4 : 2))), \
+    DUQ_LAUNCH_HEAD((gemv_s8_rows_kernel<MR, XS, FUSED, BIAS>), dim3((p.N + 4 * (XS <= 4 ? 4 : 2) - 1) / (4 * (XS <= 4 ? 4 : 2))), \
                        dim3(256), 0, stream, p)
     if (xs <= 2) DUQ_ROWS8K(2);
     else if (xs <= 4) DUQ_ROWS8K(4);
@@ -877,9 +900,9 @@ static void launch_gemm8_variant(Gemm8Params &p, hipStream_t stream)
     if (p.M <= 32) {
         const dim3 grid((p.N + 15) / 16);
         if (p.M <= 16)
-            hipLaunchKernelGGL((gemm_s8_skinny_kernel<1, FUSED, BIAS, TILED>), grid, dim3(256), 0, stream, p);
+            DUQ_LAUNCH_HEAD((gemm_s8_skinny_kernel<1, FUSED, BIAS, TILED>), grid, dim3(256), 0, stream, p);
         else
-            hipLaunchKernelGGL((gemm_s8_skinny_kernel<2, FUSED, BIAS, TILED>), grid, dim3(256), 0, stream, p);
+            DUQ_LAUNCH_HEAD((gemm_s8_skinny_kernel<2, FUSED, BIAS, TILED>), grid, dim3(256), 0, stream, p);
         return;
     }
     p.tiles_n = (p.N + 255) / 256;
@@ -887,20 +910,20 @@ static void launch_gemm8_variant(Gemm8Params &p, hipStream_t stream)
     const uint32_t t128 = ((p.M + 127) / 128) * p.tiles_n, t64 = ((p.M + 63) / 64) * p.tiles_n;
     if (p.M > 64 && t128 >= 160) {
         p.tiles_m = (p.M + 127) / 128;
-        hipLaunchKernelGGL((gemm_s8_kernel<4, 2, FUSED, BIAS, TILED>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, stream, p);
+        DUQ_LAUNCH_HEAD((gemm_s8_kernel<4, 2, FUSED, BIAS, TILED>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, stream, p);
     } else if (p.M > 32 && t64 >= 48) {
         p.tiles_m = (p.M + 63) / 64;
         // one round of 64 x 256 tiles would leave CUs idle: 64 x 128 tiles, twice as many (measured 21-24 % faster at
         // 128 such tiles, 9 % at 64)
         if (t64 <= 128) {
             p.tiles_n = (p.N + 127) / 128;
-            hipLaunchKernelGGL((gemm_s8_kernel<2, 1, FUSED, BIAS, TILED>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, stream, p);
+            DUQ_LAUNCH_HEAD((gemm_s8_kernel<2, 1, FUSED, BIAS, TILED>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, stream, p);
         } else {
-            hipLaunchKernelGGL((gemm_s8_kernel<2, 2, FUSED, BIAS, TILED>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, stream, p);
+            DUQ_LAUNCH_HEAD((gemm_s8_kernel<2, 2, FUSED, BIAS, TILED>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, stream, p);
         }
     } else {
         p.tiles_m = (p.M + 31) / 32;
-        hipLaunchKernelGGL((gemm_s8_kernel<1, 2, FUSED, BIAS, TILED>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, stream, p);
+        DUQ_LAUNCH_HEAD((gemm_s8_kernel<1, 2, FUSED, BIAS, TILED>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, stream, p);
     }
 }
 
@@ -909,7 +932,7 @@ int launch_gemm_s8(const int8_t *A, const int8_t *B, bool b_tiled, uint32_t M, u
                    float *y, hipStream_t stream)
 {
     if (M == 0 || N == 0) return 0;
-    Gemm8Params p{A, B, M, N, K, C, y, Epi8{s_row, z_row, s_col, z_col, bias}, 0, 0};
+    Gemm8Params p{A, B, M, N, K, 0, C, y, 0, Epi8{s_row, z_row, s_col, z_col, bias}};
     if (C)
         launch_gemm8_variant<false, false, false>(p, stream);
     else if (b_tiled && bias)

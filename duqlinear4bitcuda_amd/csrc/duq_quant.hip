@@ -36,8 +36,15 @@ struct QuantParams {
 // scalar kernel: any shape, one thread per output byte (odd K, unaligned rows)
 // ---------------------------------------------------------------------------------
 template <int KIND>
-__global__ __launch_bounds__(256) void quant_scalar_kernel(QuantParams p)
+__global__ __launch_bounds__(256) void quant_scalar_kernel(DUQ_HEAD_DECL, QuantParams tail)
 {
+    QuantParams p = with_head(tail, DUQ_HEAD_USE);
+    to_global(p.x);
+    to_global(p.s1);
+    to_global(p.z1);
+    to_global(p.s2);
+    to_global(p.z2);
+    to_global(p.q);
     const uint64_t total = (uint64_t)p.rows * p.colsDst;
     for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
          i += (uint64_t)gridDim.x * blockDim.x) {
@@ -98,8 +105,15 @@ __device__ __forceinline__ uint32_t quant8(const v4u raw, uint32_t col0, float r
 }
 
 template <int KIND>
-__global__ __launch_bounds__(256) void quant_vec_kernel(QuantParams p)
+__global__ __launch_bounds__(256) void quant_vec_kernel(DUQ_HEAD_DECL, QuantParams tail)
 {
+    QuantParams p = with_head(tail, DUQ_HEAD_USE);
+    to_global(p.x);
+    to_global(p.s1);
+    to_global(p.z1);
+    to_global(p.s2);
+    to_global(p.z2);
+    to_global(p.q);
     const uint32_t vecPerRow = p.colsSrc >> 3;
     const uint64_t total = (uint64_t)p.rows * vecPerRow;
     const v4u *x4 = reinterpret_cast<const v4u *>(p.x);
@@ -132,11 +146,11 @@ static int launch_quant(const QuantParams &p, hipStream_t stream)
     if (vec_ok) {
         const uint64_t total = (uint64_t)p.rows * (p.colsSrc / 8);
         const uint32_t blocks = (uint32_t)std::min<uint64_t>((total + 255) / 256, 1u << 20);
-        hipLaunchKernelGGL(quant_vec_kernel<KIND>, dim3(blocks), dim3(256), 0, stream, p);
+        DUQ_LAUNCH_HEAD((quant_vec_kernel<KIND>), dim3(blocks), dim3(256), 0, stream, p);
     } else {
         const uint64_t total = (uint64_t)p.rows * p.colsDst;
         const uint32_t blocks = (uint32_t)std::min<uint64_t>((total + 255) / 256, 1u << 20);
-        hipLaunchKernelGGL(quant_scalar_kernel<KIND>, dim3(blocks), dim3(256), 0, stream, p);
+        DUQ_LAUNCH_HEAD((quant_scalar_kernel<KIND>), dim3(blocks), dim3(256), 0, stream, p);
     }
     return (int)hipGetLastError();
 }
@@ -178,17 +192,19 @@ int launch_asym_dual_quant(const uint16_t *x, const uint16_t *s1, const uint16_t
 // run the same code with CACHED = false: the units are read a second time (from L2).
 constexpr int kMaxUnits = 8;  // 64 elements = 32 VGPRs of row data per lane
 
+// The first 56 bytes (through qmax) reach the kernel in registers (DUQ_HEAD_DECL / with_head).
 struct RowParams {
     const uint16_t *x;
     uint8_t *q;
     uint16_t *scale;
     uint16_t *zeros;
+    uint8_t *bf6;     // BF6 kernels: E3M2 shadow of the codes, [rows][cols/32 x 16 B | cols/32 x 8 B]; q may be null
     uint32_t rows, cols;
     float clip;
     int qmax;
     int32_t *rowsum;  // asym only: non-null selects the signed-shifted form (code - 8, zero - 8, sum of codes)
-    uint8_t *bf6;     // BF6 kernels: E3M2 shadow of the codes, [rows][cols/32 x 16 B | cols/32 x 8 B]; q may be null
 };
+static_assert(offsetof(RowParams, rowsum) == kHeadBytes, "the fields delivered in registers");
 
 typedef _Float16 v32h __attribute__((ext_vector_type(32)));
 typedef unsigned int v6u __attribute__((ext_vector_type(6)));
@@ -220,8 +236,14 @@ __device__ __forceinline__ v6u bf6_block(const uint32_t (&w)[4])
 // coalesced unit-per-lane pattern and a lane still converts whole blocks.  The packed nibbles
 // are written only when p.q is given.
 template <int WAVES, bool ASYM, bool CACHED, bool BF6 = false>
-__global__ __launch_bounds__(WAVES * 64) void quantize_rows_kernel(RowParams p)
+__global__ __launch_bounds__(WAVES * 64) void quantize_rows_kernel(DUQ_HEAD_DECL, RowParams tail)
 {
+    RowParams p = with_head(tail, DUQ_HEAD_USE);
+    to_global(p.x);
+    to_global(p.q);
+    to_global(p.scale);
+    to_global(p.zeros);
+    to_global(p.bf6);
     constexpr int T = WAVES * 64;
     __shared__ float red[3][WAVES];
     __shared__ int red_sum[WAVES];
@@ -394,9 +416,9 @@ static int launch_rows(const RowParams &p, hipStream_t stream)
     const bool cached = waves * 64 * kMaxUnits >= nunits;
 #define DUQ_ROWS_LAUNCH(W, C)                                                                                \
     if (p.bf6)                                                                                               \
-        hipLaunchKernelGGL((quantize_rows_kernel<W, ASYM, C, true>), grid, dim3(W * 64), 0, stream, p);      \
+        DUQ_LAUNCH_HEAD((quantize_rows_kernel<W, ASYM, C, true>), grid, dim3(W * 64), 0, stream, p);      \
     else                                                                                                     \
-        hipLaunchKernelGGL((quantize_rows_kernel<W, ASYM, C, false>), grid, dim3(W * 64), 0, stream, p);
+        DUQ_LAUNCH_HEAD((quantize_rows_kernel<W, ASYM, C, false>), grid, dim3(W * 64), 0, stream, p);
 #define DUQ_ROWS_CASE(W)                                                                                     \
     case W:                                                                                                  \
         if (cached) {                                                                                        \
@@ -420,13 +442,13 @@ static int launch_rows(const RowParams &p, hipStream_t stream)
 int launch_quantize_rows_sym(const uint16_t *x, uint32_t rows, uint32_t cols, float clip, int qmax, uint8_t *q,
                              uint16_t *scale, uint8_t *bf6, hipStream_t stream)
 {
-    RowParams p{x, q, scale, nullptr, rows, cols, clip, qmax, nullptr, bf6};
+    RowParams p{x, q, scale, nullptr, bf6, rows, cols, clip, qmax, nullptr};
     return launch_rows<false>(p, stream);
 }
 int launch_quantize_rows_asym(const uint16_t *x, uint32_t rows, uint32_t cols, uint8_t *q, uint16_t *scale,
                               uint16_t *zeros, int32_t *rowsum, uint8_t *bf6, hipStream_t stream)
 {
-    RowParams p{x, q, scale, zeros, rows, cols, 1.0f, 15, rowsum, bf6};
+    RowParams p{x, q, scale, zeros, bf6, rows, cols, 1.0f, 15, rowsum};
     return launch_rows<true>(p, stream);
 }
 

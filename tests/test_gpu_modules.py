@@ -206,6 +206,47 @@ def test_config5_prefill_70b_shape_by_properties(qnn, dev, K, N):
     assert torch.equal(y6.view(torch.int16), y_fused.view(torch.int16))
 
 
+@pytest.mark.parametrize("K,N", [(5120, 5120), (5120, 13824), (13824, 5120)])
+def test_llama13b_shapes_by_properties(qnn, dev, K, N):
+    """The Llama-2-13B layer sizes of the reference's own benchmark (test/benchmark.py:8-18: 5120 x 5120 and
+    5120 x 13824; 320 / 864 output tiles of 128 x 256 at 2048 tokens, i.e. ragged rounds on 256 CUs) on both matrix
+    paths: quantizer rows and sampled accumulators against the oracle, fused == unfused, the 6-bit float path == the
+    integer path, and the module forward at 2048, 16 and 1 tokens against the oracle on sampled outputs."""
+    _say("13B shape", K, N)
+    from duqlinear4bitcuda_amd import _HIP as hip
+
+    M = 2048
+    rng = np.random.default_rng(K + 3 * N)
+    x = cases.acts_heavy_tail(M, K, seed=13)
+    X = cases.t(x, dev)
+    q, s = hip.quantize_rows_sym(X)
+    assert np.array_equal(q.cpu().numpy()[::131], orc.sym_quant(x[::131], orc.sym_scales(x[::131])))
+    wq, sw = cases.weights_random_nibbles(N, K, seed=130)
+    W, SW = cases.t(wq, dev), cases.t(sw, dev)
+    c = hip.matmul(q, W)
+    rows = np.concatenate([rng.choice(M, 14, replace=False), [0, M - 1]])
+    cols = np.concatenate([rng.choice(N, 30, replace=False), [0, N - 1]])
+    want = orc.unpack_i4(q.cpu().numpy()[rows]).astype(np.int64) @ orc.unpack_i4(wq[cols]).astype(np.int64).T
+    assert np.array_equal(c.cpu().numpy()[np.ix_(rows, cols)], want)
+    y_fused = hip.linear4bit_forward(hip.EPI_SYM, q, s, None, W, SW)
+    assert torch.equal(y_fused.view(torch.int16), hip.sym_dequant(c, s.view(-1), SW, 32).view(torch.int16))
+    y_want = orc.sym_dequant(want, s.cpu().numpy()[rows], sw[cols])
+    assert cases.bits_equal(y_fused.cpu().numpy()[np.ix_(rows, cols)], y_want)
+    lin = _sq_module(qnn, dev, wq, sw)
+    lin.enable_fp6()
+    p6 = qnn.SymQuantizer(1.0, shadow="only", shadow_min_rows=1)(X)
+    assert lin._use_shadow(p6)
+    assert torch.equal(lin(p6).view(torch.int16), y_fused.view(torch.int16))
+    # decode through the modules at the same layer: 16 tokens (two launches) and 1 token (one launch), full oracle
+    for m in (16, 1):
+        xm = x[:m]
+        y_m = torch.nn.Sequential(qnn.SymQuantizer(1.0), lin)(cases.t(xm, dev).view(1, m, K)).cpu().numpy().reshape(m, N)
+        sm = orc.sym_scales(xm)
+        acc_cols = orc.unpack_i4(orc.sym_quant(xm, sm)).astype(np.int64) @ orc.unpack_i4(wq[cols]).astype(np.int64).T
+        assert cases.bits_equal(y_m[:, cols], orc.sym_dequant(acc_cols, sm, sw[cols]))
+        assert cases.bits_equal(y_m, y_fused.cpu().numpy()[:m])
+
+
 def test_leading_dims_and_odd_widths(qnn, dev):
     """[B, S, K] inputs keep their leading dims; a width that is not a multiple of 32 takes
     the torch-scale + given-scale kernel route and gives the same bits."""
