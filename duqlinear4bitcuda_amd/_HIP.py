@@ -331,6 +331,8 @@ def quantize_rows_asym(x: torch.Tensor):
 
 
 EPI_SYM, EPI_ASYM, EPI_SYM_DUAL, EPI_ASYM_DUAL = 0, 1, 2, 3
+EPI_ASYM_ROWSUM = 4        # exact zero-point correction with row sums; not in the reference
+EPI_ASYM_DUAL_ROWSUM = 5   # the same for the dual-uniform layer (one-launch decode entry point only)
 
 
 def linear4bit_forward(mode, xq, scale_x, zeros_x, w, w_scale_1, w_zeros_1=None, w_scale_2=None, w_zeros_2=None,
@@ -493,17 +495,18 @@ def quantize_linear4bit_forward(x, w, w_scale_1, w_scale_2=None, bias=None, clip
 
 
 def quantize_linear4bit_forward_asym(mode, x, w, w_scale_1, w_zeros_1, w_scale_2=None, w_zeros_2=None,
-                                     w_rowsum_adj=None, bias=None, return_quantized: bool = False):
+                                     w_rowsum_adj=None, bias=None, return_quantized: bool = False, w_rowsum_adj_2=None):
     """AsymQuantizer + Linear4bitASQ / LinearQuant4bitDUASQ forward (qlinear4bit/nn/quantizer.py:24-35,
     qlinear4bit/nn/linear.py:104-115, 239-250) from binary16 activations ``x`` [..., K], and the row-sum layer's
-    (``mode`` EPI_ASYM_ROWSUM with ``w_rowsum_adj``: the signed-shifted quantizer): bit-identical to
+    (``mode`` EPI_ASYM_ROWSUM with ``w_rowsum_adj``, or EPI_ASYM_DUAL_ROWSUM with ``w_rowsum_adj`` /
+    ``w_rowsum_adj_2`` for the dual-uniform layer: the signed-shifted quantizer): bit-identical to
     ``quantize_rows_asym`` (``quantize_rows_asym_shifted``) followed by ``linear4bit_forward``
-    (``linear4bit_forward_rowsum``).  Up to eight rows are ONE launch; larger inputs run the two launches with the
+    (``linear4bit_forward_rowsum`` / ``linear4bit_forward_dual_rowsum``).  Up to eight rows are ONE launch; larger inputs run the two launches with the
     codes staged in a buffer allocated here.  With ``return_quantized`` also returns (codes, scales [..., 1],
     zeros [..., 1][, rowsum [...]])."""
     name = "quantize_linear4bit_forward_asym"
-    if mode not in (EPI_ASYM, EPI_ASYM_DUAL, EPI_ASYM_ROWSUM):
-        raise RuntimeError(f"{name}: mode must be EPI_ASYM, EPI_ASYM_DUAL or EPI_ASYM_ROWSUM")
+    if mode not in (EPI_ASYM, EPI_ASYM_DUAL, EPI_ASYM_ROWSUM, EPI_ASYM_DUAL_ROWSUM):
+        raise RuntimeError(f"{name}: mode must be EPI_ASYM, EPI_ASYM_DUAL, EPI_ASYM_ROWSUM or EPI_ASYM_DUAL_ROWSUM")
     if not isinstance(x, torch.Tensor) or not isinstance(w, torch.Tensor):
         raise RuntimeError(f"{name}: x and w must be tensors")
     dev = x.device
@@ -516,7 +519,8 @@ def quantize_linear4bit_forward_asym(mode, x, w, w_scale_1, w_zeros_1, w_scale_2
     N = w.shape[0]
     ptrs = []
     for t, what, dt in ((w_scale_1, "w_scale_1", _F16), (w_zeros_1, "w_zeros_1", _F16), (w_scale_2, "w_scale_2", _F16),
-                        (w_zeros_2, "w_zeros_2", _F16), (w_rowsum_adj, "w_rowsum_adj", _I32), (bias, "bias", _F16)):
+                        (w_zeros_2, "w_zeros_2", _F16), (w_rowsum_adj, "w_rowsum_adj", _I32),
+                        (w_rowsum_adj_2, "w_rowsum_adj_2", _I32), (bias, "bias", _F16)):
         if t is None:
             ptrs.append(None)
             continue
@@ -527,7 +531,7 @@ def quantize_linear4bit_forward_asym(mode, x, w, w_scale_1, w_zeros_1, w_scale_2
     lead = x.shape[:-1]
     y = torch.empty(lead + (N,), dtype=_F16, device=dev)
     q = s = z = r = None
-    rowsum = mode == EPI_ASYM_ROWSUM
+    rowsum = mode in (EPI_ASYM_ROWSUM, EPI_ASYM_DUAL_ROWSUM)
     if return_quantized:
         q = torch.empty(lead + (K // 2,), dtype=_U8, device=dev)
         s = torch.empty(lead + (1,), dtype=_F16, device=dev)
@@ -535,7 +539,7 @@ def quantize_linear4bit_forward_asym(mode, x, w, w_scale_1, w_zeros_1, w_scale_2
         r = torch.empty(lead, dtype=_I32, device=dev) if rowsum else None
     lib = _lib.load()
     ws, ws_bytes = None, 0
-    if not return_quantized:
+    if not return_quantized or mode == EPI_ASYM_DUAL_ROWSUM:  # (that mode may also stage its accumulators)
         ws_bytes = lib.duq_quantize_linear4bit_asym_workspace_bytes(mode, M, N, K)
         if ws_bytes:
             ws = torch.empty(ws_bytes, dtype=_U8, device=dev)
@@ -550,14 +554,15 @@ def quantize_linear4bit_forward_asym(mode, x, w, w_scale_1, w_zeros_1, w_scale_2
 
 class FusedDecode:
     """One layer's arguments for the one-launch entry points (``duq_quantize_linear4bit_forward`` for the symmetric
-    modes, ``duq_quantize_linear4bit_forward_asym`` for EPI_ASYM / EPI_ASYM_DUAL / EPI_ASYM_ROWSUM), checked once
+    modes, ``duq_quantize_linear4bit_forward_asym`` for the asymmetric and row-sum modes), checked once
     and kept as a prepared argument list, so that a decode step of a module costs one ``torch.empty`` and one
     foreign call.  The tensors are held (``tensors``) so that a caller can tell when the layer's buffers were
     replaced; a change of their contents in place needs no new object."""
 
     __slots__ = ("mode", "N", "K", "device", "index", "tensors", "w_ptr", "_fn", "_head", "_tail", "_one", "_lib")
 
-    def __init__(self, mode, w, w_scale_1, w_zeros_1=None, w_scale_2=None, w_zeros_2=None, w_rowsum_adj=None, bias=None):
+    def __init__(self, mode, w, w_scale_1, w_zeros_1=None, w_scale_2=None, w_zeros_2=None, w_rowsum_adj=None,
+                 w_rowsum_adj_2=None, bias=None):
         name = "FusedDecode"
         if not isinstance(w, torch.Tensor):
             raise RuntimeError(f"{name}: w must be a tensor")
@@ -566,15 +571,17 @@ class FusedDecode:
             raise RuntimeError(f"{name}: expected w [N, K/2], got {tuple(w.shape)}")
         dev = w.device
         N, K = w.shape[0], w.shape[1] * 2
-        asym = mode in (EPI_ASYM, EPI_ASYM_DUAL, EPI_ASYM_ROWSUM)
-        dual = mode in (EPI_SYM_DUAL, EPI_ASYM_DUAL)
+        asym = mode in (EPI_ASYM, EPI_ASYM_DUAL, EPI_ASYM_ROWSUM, EPI_ASYM_DUAL_ROWSUM)
+        dual = mode in (EPI_SYM_DUAL, EPI_ASYM_DUAL, EPI_ASYM_DUAL_ROWSUM)
         if mode not in (EPI_SYM, EPI_SYM_DUAL) and not asym:
             raise RuntimeError(f"{name}: unknown mode {mode}")
         need = {"w_scale_1": True, "w_zeros_1": asym, "w_scale_2": dual, "w_zeros_2": asym and dual,
-                "w_rowsum_adj": mode == EPI_ASYM_ROWSUM, "bias": False}
+                "w_rowsum_adj": mode in (EPI_ASYM_ROWSUM, EPI_ASYM_DUAL_ROWSUM),
+                "w_rowsum_adj_2": mode == EPI_ASYM_DUAL_ROWSUM, "bias": False}
         ptrs = {}
         for t, what, dt in ((w_scale_1, "w_scale_1", _F16), (w_zeros_1, "w_zeros_1", _F16), (w_scale_2, "w_scale_2", _F16),
-                            (w_zeros_2, "w_zeros_2", _F16), (w_rowsum_adj, "w_rowsum_adj", _I32), (bias, "bias", _F16)):
+                            (w_zeros_2, "w_zeros_2", _F16), (w_rowsum_adj, "w_rowsum_adj", _I32),
+                            (w_rowsum_adj_2, "w_rowsum_adj_2", _I32), (bias, "bias", _F16)):
             if t is None:
                 if need[what]:
                     raise RuntimeError(f"{name}: {what} is required for mode {mode}")
@@ -585,13 +592,13 @@ class FusedDecode:
                 _check_size0(name, t.reshape(-1), what, N)
             ptrs[what] = t.data_ptr()
         self.mode, self.N, self.K, self.device, self.index = mode, N, K, dev, dev.index
-        self.tensors = (w, w_scale_1, w_zeros_1, w_scale_2, w_zeros_2, w_rowsum_adj, bias)
+        self.tensors = (w, w_scale_1, w_zeros_1, w_scale_2, w_zeros_2, w_rowsum_adj, w_rowsum_adj_2, bias)
         self.w_ptr = w.data_ptr()
         lib = self._lib = _lib.load()
         if asym:
             self._fn = lib.duq_quantize_linear4bit_forward_asym
             self._head = (w.data_ptr(), ptrs["w_scale_1"], ptrs["w_zeros_1"], ptrs["w_scale_2"], ptrs["w_zeros_2"],
-                          ptrs["w_rowsum_adj"], ptrs["bias"])
+                          ptrs["w_rowsum_adj"], ptrs["w_rowsum_adj_2"], ptrs["bias"])
             self._tail = (None, None, None, None, None, 0)   # q_out, scale_out, zeros_out, rowsum_out, workspace, bytes
         else:
             self._fn = lib.duq_quantize_linear4bit_forward
@@ -788,8 +795,6 @@ def linear4bit_forward_dual_rowsum(xq, scale_x, zeros_x, rowsum_x, w, w_scale_1,
 
 
 # ---- the forward on the 6-bit float matrix path (exact; not in the reference) --------------
-
-EPI_ASYM_ROWSUM = 4
 
 
 def weight_shadow_bf6(w: torch.Tensor) -> torch.Tensor:

@@ -84,11 +84,14 @@ struct FusedOut {
 
 inline uint64_t up16(uint64_t v) { return (v + 15) & ~(uint64_t)15; }
 
-uint64_t staging_bytes(int32_t mode, uint32_t M, uint32_t K)
+// codes, scales, zero points (asymmetric modes), row sums (row-sum modes), and for the dual-uniform row-sum mode
+// on a shape whose GEMM cannot apply that epilogue itself the int32 accumulators
+uint64_t staging_bytes(int32_t mode, uint32_t M, uint32_t N, uint32_t K)
 {
     uint64_t b = up16((uint64_t)M * (K / 2)) + up16((uint64_t)M * 2);
-    if (mode == DUQ_EPI_ASYM || mode == DUQ_EPI_ASYM_DUAL || mode == DUQ_EPI_ASYM_ROWSUM) b += up16((uint64_t)M * 2);
-    if (mode == DUQ_EPI_ASYM_ROWSUM) b += up16((uint64_t)M * 4);
+    if (mode == DUQ_EPI_ASYM || mode == DUQ_EPI_ASYM_DUAL || mode >= DUQ_EPI_ASYM_ROWSUM) b += up16((uint64_t)M * 2);
+    if (mode >= DUQ_EPI_ASYM_ROWSUM) b += up16((uint64_t)M * 4);
+    if (mode == DUQ_EPI_ASYM_DUAL_ROWSUM && !duq::gemm_fuses_dual_rowsum(M, N, K)) b += up16((uint64_t)M * N * 4);
     return b;
 }
 
@@ -97,10 +100,10 @@ int quantize_linear_impl(duq::Epilogue e, const duq_half *x, float clip, int32_t
                          duq_stream_t stream)
 {
     const int32_t mode = e.mode;
-    const bool asym = mode == DUQ_EPI_ASYM || mode == DUQ_EPI_ASYM_DUAL || mode == DUQ_EPI_ASYM_ROWSUM;
-    const bool dual = mode == DUQ_EPI_SYM_DUAL || mode == DUQ_EPI_ASYM_DUAL;
-    const bool rowsum = mode == DUQ_EPI_ASYM_ROWSUM;
-    if (mode < DUQ_EPI_SYM || mode > DUQ_EPI_ASYM_ROWSUM) return DUQ_E_MODE;
+    const bool asym = mode == DUQ_EPI_ASYM || mode == DUQ_EPI_ASYM_DUAL || mode >= DUQ_EPI_ASYM_ROWSUM;
+    const bool dual = mode == DUQ_EPI_SYM_DUAL || mode == DUQ_EPI_ASYM_DUAL || mode == DUQ_EPI_ASYM_DUAL_ROWSUM;
+    const bool rowsum = mode >= DUQ_EPI_ASYM_ROWSUM;
+    if (mode < DUQ_EPI_SYM || mode > DUQ_EPI_ASYM_DUAL_ROWSUM) return DUQ_E_MODE;
     if (int st = check_qmax(qmax)) return st;
     if (M == 0 || N == 0) return DUQ_OK;
     if (!x) return DUQ_E_NULL;
@@ -110,16 +113,19 @@ int quantize_linear_impl(duq::Epilogue e, const duq_half *x, float clip, int32_t
     if (asym && !e.z_col_1) return DUQ_E_NULL;
     if (dual && (!e.s_col_2 || (asym && !e.z_col_2))) return DUQ_E_NULL;
     if (rowsum && !e.rs_col) return DUQ_E_NULL;
+    if (mode == DUQ_EPI_ASYM_DUAL_ROWSUM && !e.rs_col_2) return DUQ_E_NULL;
     if ((out.q && !aligned(out.q, 16))) return DUQ_E_ALIGN;
     if (duq::decode_fp16in_one_launch(M, N, K))
         return duq::launch_decode_fp16in(x, clip, qmax, w, M, N, K, e, y, out.q, out.scale, asym ? out.zeros : nullptr,
                                          rowsum ? out.rowsum : nullptr, as_stream(stream));
     // two launches: codes and per-token parameters go to the caller's outputs where given, else to the workspace
-    const bool need_ws = !out.q || !out.scale || (asym && !out.zeros) || (rowsum && !out.rowsum);
+    const bool acc_ws = mode == DUQ_EPI_ASYM_DUAL_ROWSUM && !duq::gemm_fuses_dual_rowsum(M, N, K);
+    const bool need_ws = !out.q || !out.scale || (asym && !out.zeros) || (rowsum && !out.rowsum) || acc_ws;
+    int32_t *acc = nullptr;
     if (need_ws) {
         if (!workspace) return DUQ_E_NULL;
         if (!aligned(workspace, 16)) return DUQ_E_ALIGN;
-        if (workspace_bytes < staging_bytes(mode, M, K)) return DUQ_E_SHAPE;
+        if (workspace_bytes < staging_bytes(mode, M, N, K)) return DUQ_E_SHAPE;
         uint8_t *at = static_cast<uint8_t *>(workspace);
         if (!out.q) out.q = at;
         at += up16((uint64_t)M * (K / 2));
@@ -128,6 +134,8 @@ int quantize_linear_impl(duq::Epilogue e, const duq_half *x, float clip, int32_t
         if (asym && !out.zeros) out.zeros = reinterpret_cast<duq_half *>(at);
         at += up16((uint64_t)M * 2);
         if (rowsum && !out.rowsum) out.rowsum = reinterpret_cast<int32_t *>(at);
+        at += up16((uint64_t)M * 4);
+        if (acc_ws) acc = reinterpret_cast<int32_t *>(at);
     }
     int st;
     if (!asym)
@@ -139,6 +147,12 @@ int quantize_linear_impl(duq::Epilogue e, const duq_half *x, float clip, int32_t
     e.s_row = out.scale;
     e.z_row = asym ? out.zeros : nullptr;
     e.rs_row = rowsum ? out.rowsum : nullptr;
+    if (acc_ws) {  // GEMM into int32, then the stand-alone epilogue
+        if (int st2 = duq::launch_gemm_s4(out.q, w, M, N, K, acc, nullptr, nullptr, as_stream(stream))) return st2;
+        duq::DualRowsumParams dp{acc,       out.q,     w,         K / 2,    out.scale, out.zeros, out.rowsum, e.s_col_1, e.z_col_1,
+                                 e.s_col_2, e.z_col_2, e.rs_col,  e.rs_col_2, e.bias,  M,         N,          y};
+        return duq::launch_dual_rowsum_dequant(dp, as_stream(stream));
+    }
     return duq::launch_gemm_s4(out.q, w, M, N, K, nullptr, &e, y, as_stream(stream));
 }
 
@@ -411,7 +425,7 @@ uint64_t duq_quantize_linear4bit_workspace_bytes(uint32_t M, uint32_t N, uint32_
     if (M == 0 || N == 0 || K == 0) return 0;
     if (duq::decode_fp16in_one_launch(M, N, K)) return 0;  // nothing staged
     // packed codes [M, K/2] (rounded up to 16 bytes so that the scales stay aligned), then the scales [M]
-    return staging_bytes(DUQ_EPI_SYM, M, K);
+    return staging_bytes(DUQ_EPI_SYM, M, N, K);
 }
 
 int duq_quantize_linear4bit_forward(int32_t mode, const duq_half *x, float clip, int32_t qmax, const uint8_t *w,
@@ -429,20 +443,24 @@ int duq_quantize_linear4bit_forward(int32_t mode, const duq_half *x, float clip,
 uint64_t duq_quantize_linear4bit_asym_workspace_bytes(int32_t mode, uint32_t M, uint32_t N, uint32_t K)
 {
     if (M == 0 || N == 0 || K == 0) return 0;
-    if (mode != DUQ_EPI_ASYM && mode != DUQ_EPI_ASYM_DUAL && mode != DUQ_EPI_ASYM_ROWSUM) return 0;
+    if (mode != DUQ_EPI_ASYM && mode != DUQ_EPI_ASYM_DUAL && mode != DUQ_EPI_ASYM_ROWSUM && mode != DUQ_EPI_ASYM_DUAL_ROWSUM)
+        return 0;
     if (duq::decode_fp16in_one_launch(M, N, K)) return 0;
-    return staging_bytes(mode, M, K);
+    return staging_bytes(mode, M, N, K);
 }
 
 int duq_quantize_linear4bit_forward_asym(int32_t mode, const duq_half *x, const uint8_t *w, const duq_half *w_scale_1,
                                          const duq_half *w_zeros_1, const duq_half *w_scale_2,
-                                         const duq_half *w_zeros_2, const int32_t *w_rowsum_adj, const duq_half *bias,
-                                         uint32_t M, uint32_t N, uint32_t K, duq_half *y, uint8_t *q_out,
-                                         duq_half *scale_out, duq_half *zeros_out, int32_t *rowsum_out, void *workspace,
+                                         const duq_half *w_zeros_2, const int32_t *w_rowsum_adj,
+                                         const int32_t *w_rowsum_adj_2, const duq_half *bias, uint32_t M, uint32_t N,
+                                         uint32_t K, duq_half *y, uint8_t *q_out, duq_half *scale_out,
+                                         duq_half *zeros_out, int32_t *rowsum_out, void *workspace,
                                          uint64_t workspace_bytes, duq_stream_t stream)
 {
-    if (mode != DUQ_EPI_ASYM && mode != DUQ_EPI_ASYM_DUAL && mode != DUQ_EPI_ASYM_ROWSUM) return DUQ_E_MODE;
-    duq::Epilogue e{mode, nullptr, nullptr, w_scale_1, w_zeros_1, w_scale_2, w_zeros_2, bias, nullptr, w_rowsum_adj};
+    if (mode != DUQ_EPI_ASYM && mode != DUQ_EPI_ASYM_DUAL && mode != DUQ_EPI_ASYM_ROWSUM && mode != DUQ_EPI_ASYM_DUAL_ROWSUM)
+        return DUQ_E_MODE;
+    duq::Epilogue e{mode,      nullptr, nullptr, w_scale_1,    w_zeros_1,     w_scale_2,
+                    w_zeros_2, bias,    nullptr, w_rowsum_adj, w_rowsum_adj_2};
     return quantize_linear_impl(e, x, 1.0f, DUQ_QMAX_SYM_DEVICE, w, M, N, K, y, FusedOut{q_out, scale_out, zeros_out, rowsum_out},
                                 workspace, workspace_bytes, stream);
 }

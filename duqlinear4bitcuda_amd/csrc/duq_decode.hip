@@ -81,16 +81,46 @@ __device__ __forceinline__ int group_sum(int v)
 
 __device__ __forceinline__ v4u load16(const void *p) { return *reinterpret_cast<const v4u *>(p); }
 
+// Epilogue records of one output row / one output column, by mode: modes 0..4 the shared ColParams / RowEpi,
+// mode 5 (row-sum epilogue of the dual-uniform layer) the records that also carry the codes of input columns 0..9.
 template <int MODE>
-__device__ __forceinline__ ColParams load_col_rt(const Epilogue &e, uint32_t col, bool bias)
+struct EpiRec {
+    using Col = ColParams;
+    using Row = RowEpi;
+};
+template <>
+struct EpiRec<5> {
+    using Col = DualCol;
+    using Row = DualRow;
+};
+
+// B / A: the packed operands (mode 5 reads the first eight bytes of the row)
+template <int MODE>
+__device__ __forceinline__ typename EpiRec<MODE>::Col load_col_rt(const Epilogue &e, uint32_t col, bool bias, const uint8_t *B,
+                                                                  uint32_t kbytes)
 {
-    return bias ? load_col<MODE, true>(e.s_col_1, e.z_col_1, e.s_col_2, e.z_col_2, e.bias, col, e.rs_col)
-                : load_col<MODE, false>(e.s_col_1, e.z_col_1, e.s_col_2, e.z_col_2, e.bias, col, e.rs_col);
+    if constexpr (MODE == 5)
+        return load_dual_col(e, B, kbytes, col, bias);
+    else
+        return bias ? load_col<MODE, true>(e.s_col_1, e.z_col_1, e.s_col_2, e.z_col_2, e.bias, col, e.rs_col)
+                    : load_col<MODE, false>(e.s_col_1, e.z_col_1, e.s_col_2, e.z_col_2, e.bias, col, e.rs_col);
 }
 template <int MODE>
-__device__ __forceinline__ uint16_t dequant_rt(int acc, const RowEpi &r, const ColParams &c, bool bias)
+__device__ __forceinline__ typename EpiRec<MODE>::Row load_row_rt(const Epilogue &e, uint32_t row, const uint8_t *A, uint32_t kbytes)
 {
-    return bias ? dequant_one<MODE, true>(acc, r, c) : dequant_one<MODE, false>(acc, r, c);
+    if constexpr (MODE == 5)
+        return load_dual_row(e, A, kbytes, row);
+    else
+        return load_row<MODE>(e, row);
+}
+template <int MODE>
+__device__ __forceinline__ uint16_t dequant_rt(int acc, const typename EpiRec<MODE>::Row &r, const typename EpiRec<MODE>::Col &c,
+                                               bool bias)
+{
+    if constexpr (MODE == 5)
+        return dual_finish(acc, r, c, bias);
+    else
+        return bias ? dequant_one<MODE, true>(acc, r, c) : dequant_one<MODE, false>(acc, r, c);
 }
 
 // ---------------------------------------------------------------------------------
@@ -123,8 +153,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DUQ_HEAD_DECL,
     // binary16 rows in: the epilogue decides the quantizer (SymQuantizer for the symmetric epilogues, AsymQuantizer
     // for the asymmetric ones; the row-sum epilogue takes the signed-shifted codes, code - 8 and zero - 8, and the
     // per-token sum of the shifted codes)
-    constexpr bool ASYMQ = FUSEQ && (MODE == 1 || MODE == 3 || MODE == 4);
-    constexpr bool SHIFTQ = FUSEQ && MODE == 4;
+    constexpr bool ASYMQ = FUSEQ && (MODE == 1 || MODE == 3 || MODE == 4 || MODE == 5);
+    constexpr bool SHIFTQ = FUSEQ && (MODE == 4 || MODE == 5);
+    using ColRec = typename EpiRec<MODE>::Col;
+    using RowRec = typename EpiRec<MODE>::Row;
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t kbytes = p.K >> 1;
@@ -186,13 +218,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DUQ_HEAD_DECL,
     const uint32_t my_m = myv / R, my_r = wave * R + myv % R;  // my_r: weight row inside a tile
     const bool bias = p.epi.bias != nullptr;
     auto load_cp = [&](uint32_t tile) {
-        ColParams c{};
-        if (EPI >= 0) c = load_col_rt<MODE>(p.epi, min(tile * (4 * DUQ_DEC_R) + my_r, p.N - 1), bias);
+        ColRec c{};
+        if (EPI >= 0) c = load_col_rt<MODE>(p.epi, min(tile * (4 * DUQ_DEC_R) + my_r, p.N - 1), bias, p.B, kbytes);
         return c;
     };
-    ColParams cp = load_cp(tile0);
-    RowEpi rp{};
-    if (EPI >= 0 && !FUSEQ) rp = load_row<MODE>(p.epi, min(my_m, p.M - 1));
+    ColRec cp = load_cp(tile0);
+    RowRec rp{};
+    if (EPI >= 0 && !FUSEQ) rp = load_row_rt<MODE>(p.epi, min(my_m, p.M - 1), p.A, kbytes);
 
     // what the quantize phase needs of the kernel arguments, fetched here under the vector loads above: a scalar
     // load issued where the value is first used (the compiler sinks it into the branch that uses it) is waited for on
@@ -301,12 +333,23 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DUQ_HEAD_DECL,
 #pragma unroll
             for (int i = 0; i < XS; ++i) xr[m][i] = load16(xs + m * XSTRIDE + i * 1024 + lane * 16);
         const uint32_t rm = min(my_m, (uint32_t)MR - 1);
-        rp.s = bits_to_f16(srow[rm]);
-        if (ASYMQ) rp.z = bits_to_f16(zrow[rm]);
-        if (SHIFTQ) rp.rs = rsrow[rm];
+        if constexpr (MODE == 5) {
+            // the row record from the codes this workgroup just wrote
+            const v2u head = *reinterpret_cast<const v2u *>(xs + rm * XSTRIDE);
+            rp.xlo = head[0];
+            rp.xhi = head[1] & 0xFFu;
+            rp.zx = (uint32_t)rint_i32((float)bits_to_f16(zrow[rm]));
+            rp.sx = (float)bits_to_f16(srow[rm]);
+            rp.rxl = dual_head_sum(rp.xlo, rp.xhi);
+            rp.rxr = (uint32_t)rsrow[rm] - rp.rxl;
+        } else {
+            rp.s = bits_to_f16(srow[rm]);
+            if (ASYMQ) rp.z = bits_to_f16(zrow[rm]);
+            if (SHIFTQ) rp.rs = rsrow[rm];
+        }
     }
 
-    auto do_tile = [&](uint32_t tile, const v4u(&w)[R][XS], const ColParams &c) {
+    auto do_tile = [&](uint32_t tile, const v4u(&w)[R][XS], const ColRec &c) {
         // ---- dot products on the packed nibbles
         int acc[MR][R];
 #pragma unroll
@@ -351,7 +394,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DUQ_HEAD_DECL,
     } else {
         for (uint32_t t = tile0; t < tile_end; t += 2) {
             load_w(t + 1, w1);
-            const ColParams cp1 = load_cp(t + 1 < tile_end ? t + 1 : t);
+            const ColRec cp1 = load_cp(t + 1 < tile_end ? t + 1 : t);
             do_tile(t, w0, cp);
             load_w(t + 2, w0);
             cp = load_cp(t + 2 < tile_end ? t + 2 : t);
@@ -423,11 +466,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_s4_decode_kernel(DUQ_HEAD_DEC
     const uint32_t my_m = src_lane & 15u, my_c = (src_lane >> 4) * 4 + er;
     const bool bias = p.epi.bias != nullptr;
     const bool finisher = fg < (uint32_t)MT;
-    ColParams cp{};
-    RowEpi rp[FT];
+    using ColRec = typename EpiRec<MODE>::Col;
+    using RowRec = typename EpiRec<MODE>::Row;
+    ColRec cp{};
+    RowRec rp[FT];
     auto load_cp = [&](uint32_t tile) {
-        ColParams c{};
-        if (EPI >= 0 && finisher) c = load_col_rt<MODE>(p.epi, min(tile * 16 + my_c, p.N - 1), bias);
+        ColRec c{};
+        if (EPI >= 0 && finisher) c = load_col_rt<MODE>(p.epi, min(tile * 16 + my_c, p.N - 1), bias, p.B, kbytes);
         return c;
     };
     cp = load_cp(tile0);
@@ -436,12 +481,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_s4_decode_kernel(DUQ_HEAD_DEC
     const auto y_out = as_global(p.y);
 #pragma unroll
     for (int f = 0; f < FT; ++f) {
-        rp[f] = RowEpi{};
-        if (EPI >= 0 && finisher) rp[f] = load_row<MODE>(p.epi, min((fg + f * NG) * 16 + my_m, p.M - 1));
+        rp[f] = RowRec{};
+        if (EPI >= 0 && finisher) rp[f] = load_row_rt<MODE>(p.epi, min((fg + f * NG) * 16 + my_m, p.M - 1), p.A, kbytes);
     }
 
     auto compute_tile = [&](uint32_t tile, const v4u(&w)[SEGS], uint32_t buf) {
-        const ColParams cpn = load_cp(tile + 1 < tile_end ? tile + 1 : tile);  // next tile's, under this tile's work
+        const ColRec cpn = load_cp(tile + 1 < tile_end ? tile + 1 : tile);  // next tile's, under this tile's work
         v4i acc[MT];
 #pragma unroll
         for (int t = 0; t < MT; ++t) acc[t] = v4i{0, 0, 0, 0};
@@ -556,6 +601,7 @@ bool launch_rows_mode(DecodeParams &p, int epi, hipStream_t stream)
     case 2: DUQ_ROWS(2) break;
     case 3: DUQ_ROWS(3) break;
     case 4: DUQ_ROWS(4) break;
+    case 5: DUQ_ROWS(5) break;
     default:
         if constexpr (!FUSEQ) {
             if (epi == -1) { DUQ_ROWS(-1) }
@@ -591,6 +637,7 @@ bool launch_mfma_mode(const DecodeParams &p, int epi, hipStream_t stream)
     case 2: DUQ_DEC(2); break;
     case 3: DUQ_DEC(3); break;
     case 4: DUQ_DEC(4); break;
+    case 5: DUQ_DEC(5); break;
     default: return false;
     }
 #undef DUQ_DEC

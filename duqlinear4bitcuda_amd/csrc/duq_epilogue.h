@@ -183,6 +183,62 @@ __device__ __forceinline__ uint16_t dual_rowsum_one(int acc, uint32_t xlo, uint3
     return f16_to_bits(y);
 }
 
+// Row-side and column-side records of that epilogue for kernels that finish one output per thread (the decode
+// kernels): everything dual_rowsum_one needs of one activation row / one weight row.
+struct DualRow {
+    uint32_t xlo, xhi;  // codes of input columns 0..7 / 8, 9 (xhi masked to its two nibbles)
+    uint32_t zx, rxl, rxr;
+    float sx;
+};
+struct DualCol {
+    uint32_t wlo, whi;
+    uint32_t z1, z2, a1, a2;
+    float s1, s2;
+    f16 bias;
+};
+
+// sum of the ten codes held in xlo (eight signed nibbles) and xhi (two)
+__device__ __forceinline__ uint32_t dual_head_sum(uint32_t xlo, uint32_t xhi)
+{
+    return (uint32_t)__builtin_amdgcn_sdot8((int)xhi, 0x11111111, __builtin_amdgcn_sdot8((int)xlo, 0x11111111, 0, false), false);
+}
+
+// xq: the packed activation row (its first eight bytes are read), kbytes = K / 2
+__device__ __forceinline__ DualRow load_dual_row(const Epilogue &e, const uint8_t *xq, uint32_t kbytes, uint32_t row)
+{
+    DualRow r;
+    const v2u head = *reinterpret_cast<const v2u *>(xq + (uint64_t)row * kbytes);
+    r.xlo = head[0];
+    r.xhi = head[1] & 0xFFu;
+    r.zx = (uint32_t)rint_i32((float)bits_to_f16(e.z_row[row]));
+    r.sx = (float)bits_to_f16(e.s_row[row]);
+    r.rxl = dual_head_sum(r.xlo, r.xhi);
+    r.rxr = (uint32_t)e.rs_row[row] - r.rxl;
+    return r;
+}
+
+__device__ __forceinline__ DualCol load_dual_col(const Epilogue &e, const uint8_t *w, uint32_t kbytes, uint32_t col, bool bias)
+{
+    DualCol c;
+    const v2u head = *reinterpret_cast<const v2u *>(w + (uint64_t)col * kbytes);
+    c.wlo = head[0];
+    c.whi = head[1];
+    c.s1 = (float)bits_to_f16(e.s_col_1[col]);
+    c.s2 = (float)bits_to_f16(e.s_col_2[col]);
+    c.z1 = (uint32_t)rint_i32((float)bits_to_f16(e.z_col_1[col]));
+    c.z2 = (uint32_t)rint_i32((float)bits_to_f16(e.z_col_2[col]));
+    c.a1 = (uint32_t)e.rs_col[col];
+    c.a2 = (uint32_t)e.rs_col_2[col];
+    c.bias = bias ? bits_to_f16(e.bias[col]) : (f16)0;
+    return c;
+}
+
+__device__ __forceinline__ uint16_t dual_finish(int acc, const DualRow &r, const DualCol &c, bool bias)
+{
+    return dual_rowsum_one<false>(acc, r.xlo, r.xhi, r.zx, r.rxl, r.rxr, r.sx, c.wlo, c.whi, c.s1, c.s2, c.z1, c.z2, c.a1, c.a2,
+                                  bias, c.bias);
+}
+
 // Column parameters of four consecutive output columns n0 .. n0+3, fetched with 64-bit
 // loads when the arrays allow it (`vec`: 8-byte aligned bases and n0 + 3 < cols).
 template <int MODE, bool BIAS>

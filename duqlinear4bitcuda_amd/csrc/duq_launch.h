@@ -79,12 +79,14 @@ enum GemmKernelId {
     kKernelTile = 7,        // duq_gemm.hip, everything else (per-tile 64-bit bases: any tensor size)
 };
 int select_gemm_kernel(uint32_t M, uint32_t N, uint32_t K);
-// Shapes whose GEMM can apply the dual-uniform row-sum epilogue itself (mode 5): those of the stream kernel with
-// rows longer than 256 elements and N % 8 == 0 (its staged stores); the others run the GEMM into int32 and
-// launch_dual_rowsum_dequant.
+// Shapes whose GEMM can apply the dual-uniform row-sum epilogue itself (mode 5): those of the decode kernels, and those
+// of the stream kernel with rows longer than 256 elements and N % 8 == 0 (its staged stores); the others run the GEMM
+// into int32 and launch_dual_rowsum_dequant.
 inline bool gemm_fuses_dual_rowsum(uint32_t M, uint32_t N, uint32_t K)
 {
-    return select_gemm_kernel(M, N, K) == kKernelStream && K > 256 && N % 8 == 0;
+    const int kernel = select_gemm_kernel(M, N, K);
+    if (kernel == kKernelDecodeRows || kernel == kKernelDecodeMfma) return true;
+    return kernel == kKernelStream && K > 256 && N % 8 == 0;
 }
 inline bool decode_uses_rows_kernel(uint32_t M) { return M <= 4; }
 // MFMA decode kernel: one round of at most 256 workgroups, each with its share of the 16-column tiles.  The
@@ -108,7 +110,7 @@ int launch_decode_s4(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N,
                      const Epilogue *epi, uint16_t *y, hipStream_t stream);
 // the same with binary16 activations in: the per-token quantizer runs inside the launch, SymQuantizer for the
 // symmetric epilogues (scale = h(h(max|x| / 7) * clip), codes clamp(rint(h(x / scale)), -8, qmax)), AsymQuantizer for
-// modes 1 and 3 (unsigned codes, as the reference stores them) and its signed-shifted form for mode 4 (codes and
+// modes 1 and 3 (unsigned codes, as the reference stores them) and its signed-shifted form for modes 4 and 5 (codes and
 // zero points minus 8, plus the per-token sums of the shifted codes); epi.s_row / z_row / rs_row are ignored.
 // q_out / s_out / z_out / rs_out (optional) receive the codes, scales, zero points and sums.  Shapes of
 // decode_fp16in_one_launch only.

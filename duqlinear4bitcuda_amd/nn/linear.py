@@ -52,8 +52,8 @@ class _Linear4bitBase(torch.nn.Module):
     _decode = None
 
     def _decode_args(self):
-        """(mode, weight, w_scale_1, w_zeros_1, w_scale_2, w_zeros_2, w_rowsum_adj) of the layer, or None when
-        it has no one-launch form."""
+        """(mode, weight, w_scale_1, w_zeros_1, w_scale_2, w_zeros_2, w_rowsum_adj, w_rowsum_adj_2) of the layer, or
+        None when it has no one-launch form."""
         return None
 
     def _decode_call(self):
@@ -66,7 +66,8 @@ class _Linear4bitBase(torch.nn.Module):
         if d is not None:
             held = d.tensors
             if held[0] is args[1] and held[1] is args[2] and held[2] is args[3] and held[3] is args[4] and \
-                    held[4] is args[5] and held[5] is args[6] and held[6] is self.bias and d.w_ptr == args[1].data_ptr():
+                    held[4] is args[5] and held[5] is args[6] and held[6] is args[7] and held[7] is self.bias and \
+                    d.w_ptr == args[1].data_ptr():
                 return d
         if not args[1].is_cuda:
             return None
@@ -151,7 +152,7 @@ class Linear4bitSQ(_Linear4bitBase):
 
     def _decode_args(self):
         b = self._buffers
-        return (_ops.EPI_SYM, b["weight"], b["weight_scales"], None, None, None, None)
+        return (_ops.EPI_SYM, b["weight"], b["weight_scales"], None, None, None, None, None)
 
     def forward(self, x):
         assert type(x) == tensor_utils.PackedQuantizedTensor  # quantized input is required
@@ -206,7 +207,7 @@ class Linear4bitASQ(_Linear4bitBase):
 
     def _decode_args(self):
         b = self._buffers
-        return (_ops.EPI_ASYM, b["weight"], b["weight_scales"], b["weight_zeros"], None, None, None)
+        return (_ops.EPI_ASYM, b["weight"], b["weight_scales"], b["weight_zeros"], None, None, None, None)
 
     def forward(self, x):
         if self.require_quantizer:
@@ -267,7 +268,7 @@ class Linear4bitASQRowSum(_Linear4bitBase):
 
     def _decode_args(self):
         b = self._buffers
-        return (_ops.EPI_ASYM_ROWSUM, b["weight"], b["weight_scales"], b["weight_zeros"], None, None, b["weight_rowsum"])
+        return (_ops.EPI_ASYM_ROWSUM, b["weight"], b["weight_scales"], b["weight_zeros"], None, None, b["weight_rowsum"], None)
 
     def forward(self, x):
         if self.require_quantizer:
@@ -317,7 +318,8 @@ class LinearQuant4bitDUASQRowSum(_Linear4bitBase):
     and each part gets the row-sum correction with its own pair:
         y = s_x * ( s_1 * corr(k < 10) + s_2 * corr(k >= 10) ),  corr = acc - z_x * (R_w - n_k * z_w) - z_w * R_x
     Codes and zero points are stored minus 8 (the signed GEMM reads them exactly), ``weight_rowsum_1/2`` hold
-    ``R_w - n_k * z_w`` of the two ranges.  The forward is quantizer, GEMM into int32, epilogue (three launches)."""
+    ``R_w - n_k * z_w`` of the two ranges.  The forward is one launch for up to eight rows, quantizer + GEMM with the
+    epilogue inside for the shapes of the decode and prefill kernels, else quantizer, GEMM into int32, epilogue."""
 
     def __init__(self, in_features, out_features, bias=False, require_quantizer=True):
         super().__init__()
@@ -336,8 +338,16 @@ class LinearQuant4bitDUASQRowSum(_Linear4bitBase):
         if require_quantizer:
             self.quantizer = AsymQuantizer(shifted=True)
 
+    def _decode_args(self):
+        b = self._buffers
+        return (_ops.EPI_ASYM_DUAL_ROWSUM, b["weight"], b["weight_scales_1"], b["weight_zeros_1"], b["weight_scales_2"],
+                b["weight_zeros_2"], b["weight_rowsum_1"], b["weight_rowsum_2"])
+
     def forward(self, x):
         if self.require_quantizer:
+            y = self._own_quantizer_decode(x)
+            if y is not None:
+                return y
             x = self.quantizer(x)
         assert type(x) == tensor_utils.PackedQuantizedTensor and x.rowsum_x is not None, \
             "Input should come from AsymQuantizer(shifted=True), or require_quantizer should be set"
@@ -405,7 +415,7 @@ class Linear4bitDUSQ(_Linear4bitBase):
 
     def _decode_args(self):
         b = self._buffers
-        return (_ops.EPI_SYM_DUAL, b["weight"], b["weight_scales_1"], None, b["weight_scales_2"], None, None)
+        return (_ops.EPI_SYM_DUAL, b["weight"], b["weight_scales_1"], None, b["weight_scales_2"], None, None, None)
 
     def forward(self, x):
         assert type(x) == tensor_utils.PackedQuantizedTensor
@@ -465,7 +475,7 @@ class LinearQuant4bitDUASQ(_Linear4bitBase):
     def _decode_args(self):
         b = self._buffers
         return (_ops.EPI_ASYM_DUAL, b["weight"], b["weight_scales_1"], b["weight_zeros_1"], b["weight_scales_2"],
-                b["weight_zeros_2"], None)
+                b["weight_zeros_2"], None, None)
 
     def forward(self, x):
         if self.require_quantizer:

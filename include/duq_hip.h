@@ -255,17 +255,21 @@ int duq_quantize_linear4bit_forward(int32_t mode, const duq_half *x, float clip,
  *   mode DUQ_EPI_ASYM       y = duq_quantize_rows_asym, then duq_linear4bit_forward(DUQ_EPI_ASYM), bit for bit
  *        DUQ_EPI_ASYM_DUAL  the same with the dual-uniform epilogue (w_scale_2, w_zeros_2)
  *        DUQ_EPI_ASYM_ROWSUM  duq_quantize_rows_asym_shifted, then duq_linear4bit_forward_rowsum (w_rowsum_adj)
- *   q_out [M,K/2], scale_out [M], zeros_out [M], rowsum_out [M] (row-sum mode): optional (NULL)
+ *        DUQ_EPI_ASYM_DUAL_ROWSUM  duq_quantize_rows_asym_shifted, then duq_linear4bit_forward_dual_rowsum
+ *                           (w_rowsum_adj = its w_adj_1, w_rowsum_adj_2 = its w_adj_2)
+ *   q_out [M,K/2], scale_out [M], zeros_out [M], rowsum_out [M] (row-sum modes): optional (NULL)
  * The shapes that run as ONE launch are those of duq_quantize_linear4bit_forward; the others run quantizer + GEMM
- * and stage codes, scales, zero points (and row sums) in `workspace`
+ * and stage codes, scales, zero points (and row sums; in the dual-uniform row-sum mode also the int32 accumulators,
+ * for shapes whose GEMM cannot apply that epilogue itself) in `workspace`
  * (duq_quantize_linear4bit_asym_workspace_bytes(mode, M, N, K) bytes, 16-byte aligned; whatever the caller's own
  * output pointers cover is written there instead). */
 uint64_t duq_quantize_linear4bit_asym_workspace_bytes(int32_t mode, uint32_t M, uint32_t N, uint32_t K);
 int duq_quantize_linear4bit_forward_asym(int32_t mode, const duq_half *x, const uint8_t *w, const duq_half *w_scale_1,
                                          const duq_half *w_zeros_1, const duq_half *w_scale_2,
-                                         const duq_half *w_zeros_2, const int32_t *w_rowsum_adj, const duq_half *bias,
-                                         uint32_t M, uint32_t N, uint32_t K, duq_half *y, uint8_t *q_out,
-                                         duq_half *scale_out, duq_half *zeros_out, int32_t *rowsum_out, void *workspace,
+                                         const duq_half *w_zeros_2, const int32_t *w_rowsum_adj,
+                                         const int32_t *w_rowsum_adj_2, const duq_half *bias, uint32_t M, uint32_t N,
+                                         uint32_t K, duq_half *y, uint8_t *q_out, duq_half *scale_out,
+                                         duq_half *zeros_out, int32_t *rowsum_out, void *workspace,
                                          uint64_t workspace_bytes, duq_stream_t stream);
 
 /* No counterpart in the reference.  For callers that cannot allocate device memory or carry a workspace around
@@ -342,8 +346,8 @@ int duq_asym_dual_rowsum_dequant_host(const int32_t *q, const uint8_t *xq, const
 
 /* GEMM + that epilogue: y[M,N] = dual row-sum epilogue of xq[M,K/2] x w[N,K/2]^T, bit-identical to
  * duq_matmul_host_4bit followed by duq_asym_dual_rowsum_dequant_host (no counterpart in the reference).  Shapes for
- * which duq_linear4bit_dual_rowsum_workspace_bytes(M, N, K) is 0 (the prefill kernel with rows longer than 256
- * elements and N % 8 == 0) run as one launch and `acc_workspace` may be NULL; the others run those two launches and
+ * which duq_linear4bit_dual_rowsum_workspace_bytes(M, N, K) is 0 (the decode kernels, up to 64 rows, and the prefill
+ * kernel with rows longer than 256 elements and N % 8 == 0) run as one launch and `acc_workspace` may be NULL; the others run those two launches and
  * stage the int32 accumulators in `acc_workspace` (at least the bytes the query returns, 16-byte aligned, owned by
  * the caller: the library allocates nothing).  y 16-byte aligned, the column arrays as torch allocates them
  * (16-byte aligned). */

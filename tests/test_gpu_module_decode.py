@@ -266,11 +266,57 @@ def test_asym_fp16_input_two_launch_shapes_and_errors(dev):
     need = lib.duq_quantize_linear4bit_asym_workspace_bytes(1, M, N, K)
     ws = torch.zeros(need + 16, dtype=torch.uint8, device=dev)
     call = lambda mode, wsp, nbytes, zp=ZW.data_ptr(): lib.duq_quantize_linear4bit_forward_asym(
-        mode, X.data_ptr(), W.data_ptr(), SW.data_ptr(), zp, None, None, None, None, M, N, K, y.data_ptr(), None, None, None,
-        None, wsp, nbytes, st)
+        mode, X.data_ptr(), W.data_ptr(), SW.data_ptr(), zp, None, None, None, None, None, M, N, K, y.data_ptr(), None, None,
+        None, None, wsp, nbytes, st)
     assert call(1, None, 0) == -1 and call(1, ws.data_ptr(), need - 1) == -2 and call(1, ws.data_ptr() + 8, need) == -5
     assert call(0, ws.data_ptr(), need) == -4 and call(2, ws.data_ptr(), need) == -4   # symmetric modes: the other entry point
     assert call(1, ws.data_ptr(), need, None) == -1 and call(3, ws.data_ptr(), need) == -1 and call(4, ws.data_ptr(), need) == -1
     assert call(1, ws.data_ptr(), need) == 0
     torch.cuda.synchronize()
     assert cases.bits_equal(y.cpu().numpy(), orc.linear4bit_asq_forward(x, wq, sw, zw)[0])
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (4, 11008, 4096), (8, 512, 2048), (3, 100, 8192), (16, 4096, 4096),
+                                    (40, 1000, 1024), (100, 1000, 512)])
+def test_dual_uniform_rowsum_layer_decode(dev, library_calls, M, N, K):
+    """LinearQuant4bitDUASQRowSum from binary16 rows: one launch up to eight rows (quantizer inside the rows
+    kernel), quantizer + GEMM with the epilogue inside for the MFMA decode kernel's shapes, three launches on the
+    ring kernel's; the oracle's bits everywhere, and the op's codes / scales / zero points / row sums."""
+    from duqlinear4bitcuda_amd import _HIP as hip
+    from duqlinear4bitcuda_amd.nn import LinearQuant4bitDUASQRowSum
+    _say("dual row-sum decode", M, N, K)
+    rng = np.random.default_rng(M + N + K)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float16)
+    w[:, :10] *= 6
+    bias = rng.standard_normal(N).astype(np.float16)
+    lin = torch.nn.Linear(K, N, bias=True).half()
+    with torch.no_grad():
+        lin.weight.copy_(torch.from_numpy(w))
+        lin.bias.copy_(torch.from_numpy(bias))
+        layer = LinearQuant4bitDUASQRowSum.from_linear(lin.to(dev))
+    wq, s1, z1, s2, z2, a1, a2 = orc.weight_asym_dual_shifted_from_linear(w)
+    assert np.array_equal(layer.weight.cpu().numpy(), wq)
+    x = cases.acts_uniform(M, K, seed=70 + M)
+    X = cases.t(x, dev)
+    want, acc, qx, sx, zx, rx = orc.linear4bit_duasq_rowsum_forward(x, wq, s1, z1, s2, z2, a1, a2, bias)
+    layer(X)
+    library_calls.clear()
+    y = layer(X)
+    if M <= 8:
+        assert library_calls == ["duq_quantize_linear4bit_forward_asym"], library_calls
+    elif M <= 64:
+        assert library_calls == ["duq_quantize_rows_asym_shifted", "duq_linear4bit_forward_dual_rowsum"], library_calls
+    assert cases.bits_equal(y.detach().cpu().numpy(), want)
+    layer.fused = False
+    assert cases.bits_equal(layer(X).detach().cpu().numpy(), want)
+    T = lambda a: cases.t(a, dev)
+    y, qf, sf, zf, rf = hip.quantize_linear4bit_forward_asym(hip.EPI_ASYM_DUAL_ROWSUM, X, T(wq), T(s1), T(z1), T(s2), T(z2),
+                                                             T(a1), T(bias), return_quantized=True, w_rowsum_adj_2=T(a2))
+    assert np.array_equal(qf.cpu().numpy(), qx) and cases.bits_equal(sf.cpu().numpy(), sx) and cases.bits_equal(zf.cpu().numpy(), zx)
+    assert np.array_equal(rf.cpu().numpy(), rx)
+    assert cases.bits_equal(y.cpu().numpy(), want)
+    # without the caller's buffers: staged in a workspace allocated by the op (with the accumulators where the GEMM
+    # of the shape cannot apply the epilogue itself)
+    y = hip.quantize_linear4bit_forward_asym(hip.EPI_ASYM_DUAL_ROWSUM, X, T(wq), T(s1), T(z1), T(s2), T(z2), T(a1), None,
+                                             w_rowsum_adj_2=T(a2))
+    assert cases.bits_equal(y.cpu().numpy(), orc.linear4bit_duasq_rowsum_forward(x, wq, s1, z1, s2, z2, a1, a2)[0])

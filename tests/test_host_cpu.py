@@ -294,19 +294,21 @@ def test_asym_fp16_input_entry_point_validation_without_launch():
     P = 0x1000
     f = lib.duq_quantize_linear4bit_forward_asym
     tail = (None, None, None, None, None, 0, None)
-    assert f(0, P, P, P, P, None, None, None, None, 4, 4, 64, P, *tail) == -4      # symmetric modes: the other entry point
-    assert f(5, P, P, P, P, None, None, None, None, 4, 4, 64, P, *tail) == -4
-    assert f(1, P, P, P, P, None, None, None, None, 4, 4, 100, P, *tail) == -3     # K % 64
-    assert f(1, None, P, P, P, None, None, None, None, 4, 4, 64, P, *tail) == -1
-    assert f(1, P, P, P, None, None, None, None, None, 4, 4, 64, P, *tail) == -1   # asym needs weight zeros
-    assert f(3, P, P, P, P, P, None, None, None, 4, 4, 64, P, *tail) == -1         # dual needs the second pair
-    assert f(4, P, P, P, P, None, None, None, None, 4, 4, 64, P, *tail) == -1      # row-sum needs the weight term
-    assert f(1, P, P, P, P, None, None, None, None, 64, 4, 64, P, *tail) == -1     # needs a workspace
-    assert f(1, P, P, P, P, None, None, None, None, 64, 4, 64, P, None, None, None, None, P, 100, None) == -2
-    assert f(1, None, None, None, None, None, None, None, None, 0, 4, 64, None, *tail) == 0
+    assert f(0, P, P, P, P, None, None, None, None, None, 4, 4, 64, P, *tail) == -4      # symmetric modes: the other entry point
+    assert f(6, P, P, P, P, None, None, None, None, None, 4, 4, 64, P, *tail) == -4
+    assert f(1, P, P, P, P, None, None, None, None, None, 4, 4, 100, P, *tail) == -3     # K % 64
+    assert f(1, None, P, P, P, None, None, None, None, None, 4, 4, 64, P, *tail) == -1
+    assert f(1, P, P, P, None, None, None, None, None, None, 4, 4, 64, P, *tail) == -1   # asym needs weight zeros
+    assert f(3, P, P, P, P, P, None, None, None, None, 4, 4, 64, P, *tail) == -1         # dual needs the second pair
+    assert f(4, P, P, P, P, None, None, None, None, None, 4, 4, 64, P, *tail) == -1      # row-sum needs the weight term
+    assert f(5, P, P, P, P, P, P, P, None, None, 4, 4, 64, P, *tail) == -1               # dual row-sum needs both terms
+    assert f(1, P, P, P, P, None, None, None, None, None, 64, 4, 64, P, *tail) == -1     # needs a workspace
+    assert f(1, P, P, P, P, None, None, None, None, None, 64, 4, 64, P, None, None, None, None, P, 100, None) == -2
+    assert f(1, None, None, None, None, None, None, None, None, None, 0, 4, 64, None, *tail) == 0
     g = lib.duq_quantize_linear4bit_asym_workspace_bytes
     assert g(1, 64, 4, 64) == 64 * 32 + 128 + 128 and g(4, 64, 4, 64) == 64 * 32 + 128 + 128 + 256
-    assert g(1, 8, 4096, 4096) == 0 and g(2, 64, 4, 64) == 0
+    assert g(5, 64, 4, 64) == 64 * 32 + 128 + 128 + 256 and g(5, 100, 8, 128) == 100 * 64 + 208 + 208 + 400 + 3200
+    assert g(1, 8, 4096, 4096) == 0 and g(5, 8, 4096, 4096) == 0 and g(2, 64, 4, 64) == 0
     # the entry point that allocates nothing: slot and size limits are checked before anything else
     s = lib.duq_quantize_linear4bit_forward_static
     assert s(0, P, 1.0, 6, P, P, None, None, 8, 64, 64, P, None, None, 4, None) == -7   # no such slot

@@ -309,18 +309,19 @@ def test_dual_rowsum_fused_shapes_and_validation():
     lib = _lib.load()
     ws = lib.duq_linear4bit_dual_rowsum_workspace_bytes
     assert ws(512, 4096, 4096) == 0 and ws(128, 4096, 512) == 0 and ws(2048, 4096, 4096) == 0 and ws(700, 4000, 1024) == 0
-    assert ws(16, 4096, 4096) == 16 * 4096 * 4      # decode kernels
+    assert ws(16, 4096, 4096) == 0 and ws(1, 64, 64) == 0 and ws(64, 11008, 4096) == 0   # decode kernels apply it too
+    assert ws(100, 1000, 4096) == 100 * 1000 * 4    # ring kernel
     assert ws(300, 1028, 320) == 300 * 1028 * 4     # N % 8 != 0
     assert ws(512, 4096, 256) == 512 * 4096 * 4     # short rows
     assert ws(0, 4096, 4096) == 0
     P = 0x1000
     f = lib.duq_linear4bit_forward_dual_rowsum
     args = lambda M, N, K, y=P, w=None, nb=0: (P, P, P, P, P, P, P, P, P, P, P, None, M, N, K, y, w, nb, None)
-    assert f(*args(16, 64, 100)) == -3                      # K % 64
-    assert f(*args(16, 64, 128, y=None)) == -1
-    assert f(*args(16, 64, 128, y=P + 2)) == -5
-    assert f(*args(16, 64, 128)) == -1                      # needs a workspace
-    assert f(*args(16, 64, 128, w=P, nb=100)) == -2         # too small
+    assert f(*args(100, 64, 100)) == -3                      # K % 64
+    assert f(*args(100, 64, 128, y=None)) == -1
+    assert f(*args(100, 64, 128, y=P + 2)) == -5
+    assert f(*args(100, 64, 128)) == -1                      # needs a workspace
+    assert f(*args(100, 64, 128, w=P, nb=100)) == -2         # too small
     assert f(*args(0, 64, 128)) == 0
 
 
