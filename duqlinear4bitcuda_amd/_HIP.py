@@ -873,6 +873,41 @@ def linear4bit_forward_bf6(mode, x_bf6, scale_x, zeros_x, w_bf6, w_scale_1, w_ze
     return y
 
 
+def linear4bit_forward_dual_rowsum_bf6(x_bf6, xq, scale_x, zeros_x, rowsum_x, w_bf6, w, w_scale_1, w_zeros_1, w_scale_2, w_zeros_2,
+                                       w_adj_1, w_adj_2, bias=None):
+    """``linear4bit_forward_dual_rowsum`` on the 6-bit float matrix path: the GEMM on the shadows ``x_bf6``
+    [M, 3K/4] and ``w_bf6``, the epilogue (same launch) with the first ten codes of every row of the packed
+    operands ``xq`` [M, K/2] and ``w`` [N, K/2].  Bit-identical results."""
+    name = "linear4bit_forward_dual_rowsum_bf6"
+    _check(name, x_bf6, xq, w_bf6, w)
+    for t, what in ((x_bf6, "x_bf6"), (xq, "xq"), (w_bf6, "w_bf6"), (w, "w")):
+        _check_dtype(name, t, what, _U8)
+    if xq.dim() != 2 or w.dim() != 2 or x_bf6.dim() != 2 or w_bf6.dim() != 2 or xq.shape[1] != w.shape[1] or \
+            x_bf6.shape != (xq.shape[0], xq.shape[1] * 3 // 2) or \
+            w_bf6.shape != ((w.shape[0] + 31) // 32 * 32, w.shape[1] * 3 // 2):
+        raise RuntimeError(f"{name}: operands and shadows do not match: xq {tuple(xq.shape)}, x_bf6 {tuple(x_bf6.shape)}, "
+                           f"w {tuple(w.shape)}, w_bf6 {tuple(w_bf6.shape)}")
+    M, kb = xq.shape
+    N = w.shape[0]
+    dev = xq.device
+    for t, what, dt, cnt in ((scale_x, "scale_x", _F16, M), (zeros_x, "zeros_x", _F16, M), (rowsum_x, "rowsum_x", _I32, M),
+                             (w_scale_1, "w_scale_1", _F16, N), (w_zeros_1, "w_zeros_1", _F16, N),
+                             (w_scale_2, "w_scale_2", _F16, N), (w_zeros_2, "w_zeros_2", _F16, N),
+                             (w_adj_1, "w_adj_1", _I32, N), (w_adj_2, "w_adj_2", _I32, N)) + \
+            (((bias, "bias", _F16, N),) if bias is not None else ()):
+        _fast_check(name, what, t, dt, dev)
+        if t.numel() != cnt:
+            _check_size0(name, t.reshape(-1), what, cnt)
+    y = torch.empty((M, N), dtype=_F16, device=dev)
+    st = _launch(dev, _lib.load().duq_linear4bit_forward_dual_rowsum_bf6, x_bf6.data_ptr(), xq.data_ptr(), scale_x.data_ptr(),
+                 zeros_x.data_ptr(), rowsum_x.data_ptr(), w_bf6.data_ptr(), w.data_ptr(), w_scale_1.data_ptr(),
+                 w_zeros_1.data_ptr(), w_scale_2.data_ptr(), w_zeros_2.data_ptr(), w_adj_1.data_ptr(), w_adj_2.data_ptr(),
+                 _ptr(bias), M, N, kb * 2, y.data_ptr())
+    if st:
+        _lib.check(st, name)
+    return y
+
+
 def quantize_rows_sym_bf6(x: torch.Tensor, clip: float = 1.0, qmax: int = 6, with_q: bool = True):
     """``quantize_rows_sym`` that also writes the E3M2 shadow of the codes: returns
     (q or None, x_bf6 uint8 [..., 3K/4], scales).  K % 128 == 0."""

@@ -64,6 +64,7 @@ PROTOTYPES = {
     "duq_activation_shadow_bf6": [_c_p, _c_u32, _c_u32, _c_p, _c_p],
     "duq_linear4bit_forward_bf6": [_c_i32, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_u32,
                                    _c_u32, _c_u32, _c_p, _c_p],
+    "duq_linear4bit_forward_dual_rowsum_bf6": [_c_p] * 14 + [_c_u32, _c_u32, _c_u32, _c_p, _c_p],
     "duq_asym_quant_host_8bit": [_c_p, _c_p, _c_p, _c_u32, _c_u32, _c_p, _c_p],
     "duq_matmul_host_8bit": [_c_p, _c_p, _c_u32, _c_u32, _c_u32, _c_p, _c_p],
     "duq_asym_dequant_host_hprec": [_c_p, _c_p, _c_p, _c_p, _c_p, _c_u32, _c_u32, _c_p, _c_p],

@@ -645,6 +645,26 @@ int duq_linear4bit_forward_bf6(int32_t mode, const uint8_t *x_bf6, const duq_hal
     return duq::launch_gemm_bf6(x_bf6, w_bf6, M, N, K, e, y, as_stream(stream));
 }
 
+int duq_linear4bit_forward_dual_rowsum_bf6(const uint8_t *x_bf6, const uint8_t *xq, const duq_half *scale_x,
+                                           const duq_half *zeros_x, const int32_t *rowsum_x, const uint8_t *w_bf6,
+                                           const uint8_t *w, const duq_half *w_scale_1, const duq_half *w_zeros_1,
+                                           const duq_half *w_scale_2, const duq_half *w_zeros_2, const int32_t *w_adj_1,
+                                           const int32_t *w_adj_2, const duq_half *bias, uint32_t M, uint32_t N,
+                                           uint32_t K, duq_half *y, duq_stream_t stream)
+{
+    if (M == 0 || N == 0) return DUQ_OK;
+    if (!x_bf6 || !xq || !w_bf6 || !w || !scale_x || !zeros_x || !rowsum_x || !w_scale_1 || !w_zeros_1 || !w_scale_2 ||
+        !w_zeros_2 || !w_adj_1 || !w_adj_2 || !y)
+        return DUQ_E_NULL;
+    if (K == 0 || K % 128 != 0) return DUQ_E_KALIGN;
+    if (N % 16 != 0) return DUQ_E_SHAPE;
+    if (K > 131008u || N > (1u << 22) || M > (1u << 24)) return DUQ_E_TOO_LARGE;
+    if (!aligned(x_bf6, 16) || !aligned(w_bf6, 16) || !aligned(y, 16) || !aligned(xq, 16) || !aligned(w, 16)) return DUQ_E_ALIGN;
+    duq::Epilogue e{DUQ_EPI_ASYM_DUAL_ROWSUM, scale_x, zeros_x, w_scale_1, w_zeros_1, w_scale_2, w_zeros_2, bias, rowsum_x,
+                    w_adj_1,                  w_adj_2};
+    return duq::launch_gemm_bf6(x_bf6, w_bf6, M, N, K, e, y, as_stream(stream), xq, w);
+}
+
 // ---- 8-bit asymmetric layer ----------------------------------------------------------------
 
 static int check_gemm8(const void *A, const void *B, uint32_t M, uint32_t N, uint32_t K)

@@ -214,6 +214,10 @@ struct Bf6Params {
     uint16_t *y;
     uint32_t tiles_n;
     Epilogue epi;
+    // epilogue mode 5 only: the packed-int4 operands the shadows were made from (the first eight bytes of every row
+    // are read: the codes of input columns 0..9)
+    const uint8_t *xq;
+    const uint8_t *wq;
 };
 static_assert(offsetof(Bf6Params, epi) + 8 == kHeadBytes, "the fields delivered in registers");
 
@@ -249,6 +253,13 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(DUQ_HEAD_DECL, Bf6Params 
     constexpr int MODE = EPI;
 
     __shared__ __attribute__((aligned(16))) uint8_t lds[kLds];
+    // dual-uniform row-sum epilogue (EPI 5): its parameters, eight words per column of the tile and per row, fetched
+    // by the first BN / BM threads before the loop and read back from here after it (the records of the integer
+    // kernel's epilogue, gemm_s4_stream_kernel)
+    //   column: wlo, whi (first eight bytes of the packed weight row), s1 | s2 << 16, z1, z2, adj1, adj2, bias
+    //   row   : xlo, xhi & 0xFF (first ten codes of the packed activation row), float(s), z, rx - rxl, rxl
+    __shared__ __attribute__((aligned(16))) uint32_t dpar[EPI == 5 ? (BN + BM) * 8 : 4];
+    __shared__ uint32_t dwide;  // EPI 5: non-zero when a factor of the corrections leaves the signed 24-bit range
 
     uint32_t tile_m, tile_n;
     tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
@@ -256,6 +267,42 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(DUQ_HEAD_DECL, Bf6Params 
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63u, wave = tid >> 6;
     const uint32_t l16 = lane & 15u, kb = lane >> 4;
+    if constexpr (EPI == 5) {
+        const uint32_t kbytes = p.K >> 1;
+        if (tid == 0) dwide = 0;
+        __syncthreads();
+        bool wide = false;
+        for (uint32_t i = tid; i < (uint32_t)BN; i += 256) {
+            const uint32_t n = min(n0 + i, p.N - 1);
+            const v2u head = *reinterpret_cast<const v2u *>(p.wq + (uint64_t)n * kbytes);
+            uint32_t *d = dpar + i * 8;
+            d[0] = head[0];
+            d[1] = head[1];
+            d[2] = (uint32_t)p.epi.s_col_1[n] | ((uint32_t)p.epi.s_col_2[n] << 16);
+            d[3] = (uint32_t)rint_i32((float)bits_to_f16(p.epi.z_col_1[n]));
+            d[4] = (uint32_t)rint_i32((float)bits_to_f16(p.epi.z_col_2[n]));
+            d[5] = (uint32_t)p.epi.rs_col[n];
+            d[6] = (uint32_t)p.epi.rs_col_2[n];
+            d[7] = BIAS ? (uint32_t)p.epi.bias[n] : 0u;
+            wide = wide || !(fits_i24(d[3]) && fits_i24(d[4]) && fits_i24(d[5]) && fits_i24(d[6]));
+        }
+        for (uint32_t i = tid; i < (uint32_t)BM; i += 256) {
+            const uint32_t m = min(m0 + i, p.M - 1);
+            const v2u head = *reinterpret_cast<const v2u *>(p.xq + (uint64_t)m * kbytes);
+            const uint32_t xlo = head[0], xhi = head[1] & 0xFFu;  // input columns 0..7 and 8, 9
+            const uint32_t rxl = dual_head_sum(xlo, xhi);
+            uint32_t *d = dpar + (BN + i) * 8;
+            d[0] = xlo;
+            d[1] = xhi;
+            d[2] = __builtin_bit_cast(uint32_t, (float)bits_to_f16(p.epi.s_row[m]));
+            d[3] = (uint32_t)rint_i32((float)bits_to_f16(p.epi.z_row[m]));
+            d[4] = (uint32_t)p.epi.rs_row[m] - rxl;
+            d[5] = rxl;
+            wide = wide || !(fits_i24(d[3]) && fits_i24(d[4]));
+        }
+        if (wide) dwide = 1;  // (same value from every writer)
+        // (the barriers of the main loop order these writes before the epilogue's reads)
+    }
     const uint32_t nblk = p.K / 32;
     const uint32_t row_bytes = nblk * 24, p1off = nblk * 16;
     const uint32_t ksteps = p.K / 128;
@@ -366,8 +413,9 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(DUQ_HEAD_DECL, Bf6Params 
     v4i raw_rs[TNI];
     RowEpi rowp[TMI];
     auto load_params = [&]() {
+        if constexpr (EPI == 5) return;  // staged in LDS above
 #pragma unroll
-        for (int mi = 0; mi < TMI; ++mi) rowp[mi] = load_row<MODE>(e, min(m0 + mi * 16 + l16, p.M - 1));
+        for (int mi = 0; mi < TMI; ++mi) rowp[mi] = load_row<MODE == 5 ? 0 : MODE>(e, min(m0 + mi * 16 + l16, p.M - 1));
 #pragma unroll
         for (int ni = 0; ni < TNI; ++ni) {
             const uint32_t nq = min(n0 + wave * (16 * TNI) + ni * 16 + kb * 4, p.N - 4);
@@ -496,6 +544,44 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(DUQ_HEAD_DECL, Bf6Params 
     // 128 x 64 fp16 tile of the wavefront goes through LDS so that global stores are whole
     // 128-byte lines.
     uint8_t *stage = lds + wave * (BM * kYStride);
+    if constexpr (EPI == 5) {
+        // every wavefront has passed the loop's last barrier: dpar is complete.  The staging area overlaps the
+        // activation buffers that other wavefronts may still read in their last chunk: wait for them.
+        __syncthreads();
+        const bool wide = dwide != 0;
+#pragma unroll
+        for (int ni = 0; ni < TNI; ++ni) {
+            const uint32_t ncol = ni * 16 + kb * 4;
+            v4u c0[4], c1[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const uint32_t *d = dpar + (wave * (16 * TNI) + ncol + r) * 8;
+                c0[r] = *reinterpret_cast<const v4u *>(d);
+                c1[r] = *reinterpret_cast<const v4u *>(d + 4);
+            }
+#pragma unroll
+            for (int mi = 0; mi < TMI; ++mi) {
+                const uint32_t *d = dpar + (BN + mi * 16 + l16) * 8;
+                const v4u r0 = *reinterpret_cast<const v4u *>(d);
+                const v2u r1 = *reinterpret_cast<const v2u *>(d + 4);
+                const uint32_t s_bits = r0[2];  // (a copy: a bit cast of a vector element would read element 0)
+                const float sx = __builtin_bit_cast(float, s_bits);
+                uint16_t out[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float s1 = (float)bits_to_f16((uint16_t)(c0[r][2] & 0xFFFFu)), s2 = (float)bits_to_f16((uint16_t)(c0[r][2] >> 16));
+                    const f16 b = bits_to_f16((uint16_t)c1[r][3]);
+                    const int a = (int)acc[mi][ni][r];
+                    out[r] = wide ? dual_rowsum_one<false>(a, r0[0], r0[1], r0[3], r1[1], r1[0], sx, c0[r][0], c0[r][1], s1, s2,
+                                                           c0[r][3], c1[r][0], c1[r][1], c1[r][2], BIAS, b)
+                                  : dual_rowsum_one<true>(a, r0[0], r0[1], r0[3], r1[1], r1[0], sx, c0[r][0], c0[r][1], s1, s2,
+                                                          c0[r][3], c1[r][0], c1[r][1], c1[r][2], BIAS, b);
+                }
+                *reinterpret_cast<v2u *>(stage + (mi * 16 + l16) * kYStride + ncol * 2) =
+                    v2u{(uint32_t)out[0] | ((uint32_t)out[1] << 16), (uint32_t)out[2] | ((uint32_t)out[3] << 16)};
+            }
+        }
+    } else {
 #pragma unroll
     for (int ni = 0; ni < TNI; ++ni) {
         const uint32_t ncol = ni * 16 + kb * 4;
@@ -508,6 +594,7 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(DUQ_HEAD_DECL, Bf6Params 
                 v2u{dequant_pair<MODE, BIAS>(acc[mi][ni][0], acc[mi][ni][1], rowp[mi], cols.c[0], cols.c[1]),
                     dequant_pair<MODE, BIAS>(acc[mi][ni][2], acc[mi][ni][3], rowp[mi], cols.c[2], cols.c[3])};
         }
+    }
     }
     const uint32_t rows_here = min(p.M - m0, (uint32_t)BM);
     const __amdgpu_buffer_rsrc_t rY = make_rsrc(p.y + (uint64_t)m0 * p.N, rows_here * p.N * 2);
@@ -543,9 +630,10 @@ static void launch_mode(Bf6Params &p, hipStream_t stream)
                    t64 = ((p.M + 63) / 64) * p.tiles_n;
     const float c256 = kCost256 * (float)((t256 + 255) / 256), c128 = (float)((t128 + 255) / 256),
                 c64 = kCost64 * (float)((t64 + 255) / 256);
-    if (c256 < c128 && c256 <= c64) {
+    // (the 256-row tile leaves no LDS for the staged parameters of epilogue 5)
+    if (EPI != 5 && c256 < c128 && c256 <= c64) {
         p.tiles_m = (p.M + 255) / 256;
-        launch_tile<16, 4, EPI>(p, stream);
+        if constexpr (EPI != 5) launch_tile<16, 4, EPI>(p, stream);
     } else if (c64 < c128) {
         p.tiles_m = (p.M + 63) / 64;
         // CUs left without a 64 x 256 tile: 64 x 128 tiles, twice as many, as long as they still run in one round
@@ -563,16 +651,21 @@ static void launch_mode(Bf6Params &p, hipStream_t stream)
 }
 
 int launch_gemm_bf6(const uint8_t *X, const uint8_t *W, uint32_t M, uint32_t N, uint32_t K, const Epilogue &epi,
-                    uint16_t *y, hipStream_t stream)
+                    uint16_t *y, hipStream_t stream, const uint8_t *xq, const uint8_t *wq)
 {
     if (M == 0 || N == 0) return 0;
-    Bf6Params p{X, W, M, N, K, (M + 127) / 128, y, (N + 255) / 256, epi};
+    Bf6Params p{X, W, M, N, K, (M + 127) / 128, y, (N + 255) / 256, epi, xq, wq};
     switch (epi.mode) {
     case 0: launch_mode<0>(p, stream); break;
     case 1: launch_mode<1>(p, stream); break;
     case 2: launch_mode<2>(p, stream); break;
     case 3: launch_mode<3>(p, stream); break;
-    default: launch_mode<4>(p, stream); break;
+    case 4: launch_mode<4>(p, stream); break;
+    case 5:
+        if (!xq || !wq) return (int)hipErrorInvalidValue;
+        launch_mode<5>(p, stream);
+        break;
+    default: return (int)hipErrorInvalidValue;
     }
     return (int)hipGetLastError();
 }

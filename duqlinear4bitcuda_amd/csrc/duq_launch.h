@@ -134,8 +134,10 @@ int launch_gemm_s4_batched(const uint8_t *A, const uint8_t *B, uint32_t M, uint3
 // (duq_bf6.hip).  K % 128 == 0, N % 16 == 0.
 int launch_weight_shadow_bf6(const uint8_t *w, uint32_t N, uint32_t K, uint8_t *out, hipStream_t stream);
 int launch_activation_shadow_bf6(const uint8_t *q, uint32_t M, uint32_t K, uint8_t *out, hipStream_t stream);
+// epi.mode 5 (row-sum epilogue of the dual-uniform layer) also needs the packed-int4 operands the shadows were made
+// from, xq [M, K/2] and wq [N, K/2]: the first eight bytes of every row are read.
 int launch_gemm_bf6(const uint8_t *X, const uint8_t *W, uint32_t M, uint32_t N, uint32_t K, const Epilogue &epi,
-                    uint16_t *y, hipStream_t stream);
+                    uint16_t *y, hipStream_t stream, const uint8_t *xq = nullptr, const uint8_t *wq = nullptr);
 
 // 8-bit asymmetric layer (duq_int8.hip): float32 activations, int8 codes, int32 accumulators, float32 results.
 int launch_asym_quant8(const float *x, const float *scale, const float *zeros, uint32_t rows, uint32_t cols, int8_t *q,

@@ -348,13 +348,21 @@ class LinearQuant4bitDUASQRowSum(_Linear4bitBase):
             y = self._own_quantizer_decode(x)
             if y is not None:
                 return y
-            x = self.quantizer(x)
+            # (the 6-bit float path of this layer reads the packed codes too: shadow and codes)
+            rows = x.numel() // x.shape[-1]
+            x = self.quantizer(x, shadow=True if self.fused and self._fp6_wanted(rows) else False)
         assert type(x) == tensor_utils.PackedQuantizedTensor and x.rowsum_x is not None, \
             "Input should come from AsymQuantizer(shifted=True), or require_quantizer should be set"
         xq = x.quantized_x
         lead = xq.shape[:-1]
         xq2 = xq.reshape(-1, xq.shape[-1])
-        if self.fused:
+        if self.fused and x.shadow_x is not None and self._fp6_wanted(xq2.shape[0]):
+            y = _ops.linear4bit_forward_dual_rowsum_bf6(x.shadow_x.reshape(xq2.shape[0], -1), xq2, x.scales_x, x.zeros_x,
+                                                        x.rowsum_x, self.weight_shadow, self.weight,
+                                                        self.weight_scales_1, self.weight_zeros_1, self.weight_scales_2,
+                                                        self.weight_zeros_2, self.weight_rowsum_1, self.weight_rowsum_2,
+                                                        self.bias)
+        elif self.fused:
             y = _ops.linear4bit_forward_dual_rowsum(xq2, x.scales_x, x.zeros_x, x.rowsum_x, self.weight,
                                                     self.weight_scales_1, self.weight_zeros_1, self.weight_scales_2,
                                                     self.weight_zeros_2, self.weight_rowsum_1, self.weight_rowsum_2,

@@ -390,6 +390,17 @@ int duq_linear4bit_forward_bf6(int32_t mode, const uint8_t *x_bf6, const duq_hal
                                const int32_t *w_rowsum_adj, const duq_half *bias, uint32_t M, uint32_t N, uint32_t K,
                                duq_half *y, duq_stream_t stream);
 
+/* duq_linear4bit_forward_dual_rowsum on the 6-bit float matrix path (no counterpart in the reference): the GEMM reads
+ * the shadows, the epilogue (inside the same launch) the first eight bytes of every row of the packed operands the
+ * shadows were made from, xq [M,K/2] and w [N,K/2] (the codes of input columns 0..9).  y is bit-identical to
+ * duq_linear4bit_forward_dual_rowsum's.  K % 128 == 0, N % 16 == 0; shadows, packed operands and y 16-byte aligned. */
+int duq_linear4bit_forward_dual_rowsum_bf6(const uint8_t *x_bf6, const uint8_t *xq, const duq_half *scale_x,
+                                           const duq_half *zeros_x, const int32_t *rowsum_x, const uint8_t *w_bf6,
+                                           const uint8_t *w, const duq_half *w_scale_1, const duq_half *w_zeros_1,
+                                           const duq_half *w_scale_2, const duq_half *w_zeros_2, const int32_t *w_adj_1,
+                                           const int32_t *w_adj_2, const duq_half *bias, uint32_t M, uint32_t N,
+                                           uint32_t K, duq_half *y, duq_stream_t stream);
+
 /* ---- the 8-bit asymmetric layer (LinearQuant8bitASQ, qlinear4bit/nn/linear.py:300-368) ---- */
 
 /* float32 activations [rows, cols], per-row float32 scale and zero point ->

@@ -302,6 +302,40 @@ def test_gpu_dual_rowsum_wide_factors(hip, dev):
         assert cases.bits_equal(got.cpu().numpy(), want), which
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N,K", [(512, 4096, 4096), (100, 4096, 512), (300, 3104, 384), (2048, 1024, 1024), (70, 8192, 128),
+                                   (1100, 4096, 256), (200, 512, 640)])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_gpu_dual_rowsum_on_the_6bit_float_path(hip, dev, M, N, K, with_bias):
+    """The dual-uniform row-sum epilogue inside the 6-bit float GEMM (128-, 64-row and 64 x 128 tiles, ragged M, N
+    ending inside a tile, one chunk and several) against the oracle, and row-sum terms outside the signed 24-bit
+    range (the kernel then leaves its 24-bit multiplier)."""
+    print("dual rowsum fp6", M, N, K, with_bias, flush=True)
+    rng = np.random.default_rng(M + 3 * N + 7 * K)
+    x = cases.acts_uniform(M, K, seed=M + N + K)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float16)
+    w[:, :10] *= 6
+    wq, s1, z1, s2, z2, a1, a2 = orc.weight_asym_dual_shifted_from_linear(w)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float16) if with_bias else None
+    want, acc, qx, sx, zx, rx = orc.linear4bit_duasq_rowsum_forward(x, wq, s1, z1, s2, z2, a1, a2, bias)
+    T = lambda v: cases.t(v, dev)
+    q, b6, s, z, r = hip.quantize_rows_asym_bf6(T(x), shifted=True, with_q=True)
+    assert np.array_equal(q.cpu().numpy(), qx) and np.array_equal(r.cpu().numpy(), rx)
+    W = T(wq)
+    W6 = hip.weight_shadow_bf6(W)
+    B = None if bias is None else T(bias)
+    got = hip.linear4bit_forward_dual_rowsum_bf6(b6, q, s, z, r, W6, W, T(s1), T(z1), T(s2), T(z2), T(a1), T(a2), B)
+    assert cases.bits_equal(got.cpu().numpy(), want)
+    if with_bias and M <= 512:
+        a1w, a2w, rw = a1.copy(), a2.copy(), rx.copy()
+        a1w[5] = 2 ** 30 + 12345
+        a2w[N - 3] = -(2 ** 29) - 7
+        rw[M // 2] = 2 ** 31 - 5
+        want = orc.asym_dual_rowsum_dequant(acc, qx, sx, zx, rw, wq, s1, z1, s2, z2, a1w, a2w, bias)
+        got = hip.linear4bit_forward_dual_rowsum_bf6(b6, q, s, z, T(rw), W6, W, T(s1), T(z1), T(s2), T(z2), T(a1w), T(a2w), B)
+        assert cases.bits_equal(got.cpu().numpy(), want)
+
+
 def test_dual_rowsum_fused_shapes_and_validation():
     """Which shapes the fused entry point runs as one launch (no workspace), and its argument checks."""
     from duqlinear4bitcuda_amd import _lib
@@ -364,4 +398,8 @@ def test_gpu_dual_rowsum_module_config4(dev):
     # state_dict round trip
     other = LinearQuant4bitDUASQRowSum(K, N, bias=True).to(dev)
     other.load_state_dict(mod.state_dict())
+    assert torch.equal(other(cases.t(x, dev)).view(torch.int16), y.view(M, N).view(torch.int16))
+    # the same layer on the 6-bit float matrix path: same bits
+    other.enable_fp6()
+    assert other._fp6_wanted(M)
     assert torch.equal(other(cases.t(x, dev)).view(torch.int16), y.view(M, N).view(torch.int16))
