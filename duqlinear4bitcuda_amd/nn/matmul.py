@@ -21,8 +21,14 @@ from .quantizer import AsymQuantizer, SymQuantizer
 
 
 class SymQuantMatMul(torch.nn.Module):
-    """sym_dequant(matmul(q(A), q(B)), s_A, s_B) (matmul.py:69-84); A [M, K], B [N, K].  Also takes
-    A [..., M, K] and B [..., N, K] with equal leading dimensions (one product per entry, one launch)."""
+    """sym_dequant(matmul(q(A), q(B)), s_A, s_B) (matmul.py:69-84): A [..., M, K] against a 2-D B [N, K] gives
+    [..., M, N], as in the reference (its wrappers flatten the leading dimensions of A).
+
+    Extension: a B of more than two dimensions, [..., N, K] with the leading dimensions of A, is one product per
+    batch entry (per-entry scales, one launch), result [..., M, N].  The reference has no such case: its
+    ``tensor_utils.matmul`` would form the cross product of all rows of A with all rows of B and its
+    ``sym_dequant`` then rejects the scale sizes (src/export/bindings.cpp:152-155).  Leading dimensions that differ
+    raise ``RuntimeError``."""
 
     fused = True
 
@@ -37,7 +43,9 @@ class SymQuantMatMul(torch.nn.Module):
         qa, qb = A.quantized_x, B.quantized_x
         if qb.dim() > 2:
             lead = tuple(qb.shape[:-2])
-            assert tuple(qa.shape[:-2]) == lead, "Batch dimensions must match"
+            if tuple(qa.shape[:-2]) != lead:
+                raise RuntimeError(f"SymQuantMatMul: a batched B {tuple(qb.shape[:-2])} x [N, K] needs an A with the same "
+                                   f"leading dimensions, got {tuple(qa.shape[:-2])} x [M, K]")
             qa3, qb3 = qa.reshape(-1, *qa.shape[-2:]), qb.reshape(-1, *qb.shape[-2:])
             if self.fused:
                 out = _ops.batch_linear4bit_forward(_ops.EPI_SYM, qa3, A.scales_x, None, qb3, B.scales_x)

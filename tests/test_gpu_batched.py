@@ -199,3 +199,23 @@ def test_batched_argument_errors(dev):
         ops.batched_matmul(torch.zeros((2, 4, 24), dtype=torch.uint8, device=dev),
                            torch.zeros((2, 4, 24), dtype=torch.uint8, device=dev))
     assert ops.batched_matmul(a[:0], a[:0]).shape == (0, 4, 4)
+
+
+def test_sym_quant_matmul_shapes_of_the_reference_and_mismatch(dev):
+    """A with leading dimensions against a 2-D B gives [..., M, N] as the reference's flattening wrappers do
+    (qlinear4bit/tools/tensor_utils.py:51-55, nn/matmul.py:76-84); a batched B whose leading dimensions differ from
+    A's is rejected with a RuntimeError."""
+    from duqlinear4bitcuda_amd.nn import SymQuantMatMul
+    a = cases.acts_normal(3 * 20, 128, seed=41).reshape(3, 20, 128)
+    b = cases.acts_normal(24, 128, seed=42)
+    mod = SymQuantMatMul()
+    got = mod(cases.t(a, dev), cases.t(b, dev))
+    assert got.shape == (3, 20, 24)
+    a2 = a.reshape(60, 128)
+    sa, sb = orc.sym_scales(a2), orc.sym_scales(b)
+    want = orc.sym_dequant(orc.matmul_s4(orc.sym_quant(a2, sa), orc.sym_quant(b, sb)), sa, sb)
+    assert cases.bits_equal(got.cpu().numpy().reshape(60, 24), want)
+    with pytest.raises(RuntimeError, match="leading dimensions"):
+        mod(cases.t(a[0], dev), cases.t(np.stack([b, b]), dev))
+    with pytest.raises(RuntimeError, match="leading dimensions"):
+        mod(cases.t(a, dev), cases.t(np.stack([b, b]), dev))
