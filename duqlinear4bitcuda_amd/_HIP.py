@@ -8,6 +8,8 @@ device, and calls the C ABI on the current torch stream.  Argument errors raise
 """
 from __future__ import annotations
 
+import ctypes
+
 import torch
 
 from . import _lib
@@ -553,13 +555,14 @@ def quantize_linear4bit_forward_asym(mode, x, w, w_scale_1, w_zeros_1, w_scale_2
 
 
 class FusedDecode:
-    """One layer's arguments for the one-launch entry points (``duq_quantize_linear4bit_forward`` for the symmetric
-    modes, ``duq_quantize_linear4bit_forward_asym`` for the asymmetric and row-sum modes), checked once
-    and kept as a prepared argument list, so that a decode step of a module costs one ``torch.empty`` and one
-    foreign call.  The tensors are held (``tensors``) so that a caller can tell when the layer's buffers were
-    replaced; a change of their contents in place needs no new object."""
+    """One layer's side of the one-launch decode (what ``duq_quantize_linear4bit_forward`` takes for the symmetric
+    modes and ``duq_quantize_linear4bit_forward_asym`` for the asymmetric and row-sum modes), checked once and kept
+    as a ``duq_fused_layer`` struct for ``duq_quantize_linear4bit_forward_layer``: a decode step of a module then
+    costs one ``torch.empty`` and one foreign call with five arguments.  The tensors are held (``tensors``) so that
+    a caller can tell when the layer's buffers were replaced; a change of their contents in place needs no new
+    object."""
 
-    __slots__ = ("mode", "N", "K", "device", "index", "tensors", "w_ptr", "_fn", "_head", "_tail", "_one", "_lib")
+    __slots__ = ("mode", "N", "K", "device", "index", "tensors", "w_ptr", "_fn", "_ptrs", "_structs", "_one", "_lib")
 
     def __init__(self, mode, w, w_scale_1, w_zeros_1=None, w_scale_2=None, w_zeros_2=None, w_rowsum_adj=None,
                  w_rowsum_adj_2=None, bias=None):
@@ -595,16 +598,21 @@ class FusedDecode:
         self.tensors = (w, w_scale_1, w_zeros_1, w_scale_2, w_zeros_2, w_rowsum_adj, w_rowsum_adj_2, bias)
         self.w_ptr = w.data_ptr()
         lib = self._lib = _lib.load()
-        if asym:
-            self._fn = lib.duq_quantize_linear4bit_forward_asym
-            self._head = (w.data_ptr(), ptrs["w_scale_1"], ptrs["w_zeros_1"], ptrs["w_scale_2"], ptrs["w_zeros_2"],
-                          ptrs["w_rowsum_adj"], ptrs["w_rowsum_adj_2"], ptrs["bias"])
-            self._tail = (None, None, None, None, None, 0)   # q_out, scale_out, zeros_out, rowsum_out, workspace, bytes
-        else:
-            self._fn = lib.duq_quantize_linear4bit_forward
-            self._head = (w.data_ptr(), ptrs["w_scale_1"], ptrs["w_scale_2"], ptrs["bias"])
-            self._tail = (None, None, None, 0)               # q_out, scale_out, workspace, bytes
+        self._fn = lib.duq_quantize_linear4bit_forward_layer
+        # one struct per quantizer setting (clip, qmax), built on first use
+        self._ptrs = ptrs
+        self._structs = {}
         self._one = {}
+
+    def _layer(self, clip, qmax):
+        key = (clip, qmax)
+        ref = self._structs.get(key)
+        if ref is None:
+            p = self._ptrs
+            st = _lib.FusedLayer(self.mode, float(clip), int(qmax), self.N, self.K, self.w_ptr, p["w_scale_1"], p["w_zeros_1"],
+                                 p["w_scale_2"], p["w_zeros_2"], p["w_rowsum_adj"], p["w_rowsum_adj_2"], p["bias"])
+            ref = self._structs[key] = (ctypes.addressof(st), st)   # (the struct is kept alive beside its address)
+        return ref[0]
 
     def admits(self, M: int) -> bool:
         """True when M rows of this layer run as ONE launch with nothing staged."""
@@ -613,24 +621,23 @@ class FusedDecode:
             one = self._one[M] = M > 0 and self._lib.duq_quantize_linear4bit_workspace_bytes(M, self.N, self.K) == 0
         return one
 
-    def run(self, x: torch.Tensor, M: int, clip: float = 1.0, qmax: int = 6) -> torch.Tensor:
+    def run(self, x: torch.Tensor, M: int, clip: float = 1.0, qmax: int = 6, checked: bool = False) -> torch.Tensor:
         """x: contiguous binary16 [..., K] on the layer's device, 16-byte aligned, M = its rows with admits(M);
-        clip / qmax: the symmetric quantizer's settings (unused by the asymmetric modes).  Returns binary16
-        [..., N]."""
-        if x.dtype is not _F16 or not x.is_contiguous() or x.shape[-1] != self.K or x.device != self.device:
+        clip / qmax: the symmetric quantizer's settings (unused by the asymmetric modes).  ``checked``: the caller
+        has verified dtype and contiguity already.  Returns binary16 [..., N]."""
+        if x.get_device() != self.index or x.shape[-1] != self.K or \
+                not (checked or (x.dtype is _F16 and x.is_contiguous())):
             raise RuntimeError(f"FusedDecode: expected a contiguous float16 tensor [..., {self.K}] on {self.device}, got "
                                f"{x.dtype} {tuple(x.shape)} on {x.device}")
         y = torch.empty(x.shape[:-1] + (self.N,), dtype=_F16, device=self.device)
         idx = self.index
-        if self.mode == EPI_SYM or self.mode == EPI_SYM_DUAL:
-            args = (self.mode, x.data_ptr(), clip, qmax, *self._head, M, self.N, self.K, y.data_ptr(), *self._tail)
-        else:
-            args = (self.mode, x.data_ptr(), *self._head, M, self.N, self.K, y.data_ptr(), *self._tail)
+        ref = self._structs.get((clip, qmax))
+        layer = ref[0] if ref is not None else self._layer(clip, qmax)
         if idx == torch._C._cuda_getDevice():
-            st = self._fn(*args, _raw_stream(idx))
+            st = self._fn(layer, x.data_ptr(), M, y.data_ptr(), _raw_stream(idx))
         else:
             with torch.cuda.device(idx):
-                st = self._fn(*args, _raw_stream(idx))
+                st = self._fn(layer, x.data_ptr(), M, y.data_ptr(), _raw_stream(idx))
         if st:
             _lib.check(st, "quantize_linear4bit_forward")
         return y

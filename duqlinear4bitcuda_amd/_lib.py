@@ -46,6 +46,7 @@ PROTOTYPES = {
     "duq_quantize_linear4bit_forward_static": [_c_i32, _c_p, ctypes.c_float, _c_i32, _c_p, _c_p, _c_p, _c_p, _c_u32,
                                                _c_u32, _c_u32, _c_p, _c_p, _c_p, _c_u32, _c_p],
     "duq_static_scratch_init": [],
+    "duq_quantize_linear4bit_forward_layer": [_c_p, _c_p, _c_u32, _c_p, _c_p],
     "duq_quantize_linear4bit_asym_workspace_bytes": [_c_i32, _c_u32, _c_u32, _c_u32],  # returns uint64_t
     "duq_quantize_linear4bit_forward_asym": [_c_i32, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_u32, _c_u32,
                                              _c_u32, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, ctypes.c_uint64, _c_p],
@@ -73,6 +74,15 @@ PROTOTYPES = {
     "duq_linear8bit_forward_tiled": [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_u32, _c_u32, _c_u32, _c_p, _c_p],
     "duq_linear8bit_forward": [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_u32, _c_u32, _c_u32, _c_p, _c_p],
 }
+
+
+
+class FusedLayer(ctypes.Structure):
+    """``duq_fused_layer`` of include/duq_hip.h."""
+    _fields_ = [("mode", _c_i32), ("clip", ctypes.c_float), ("qmax", _c_i32), ("N", _c_u32), ("K", _c_u32),
+                ("w", _c_p), ("w_scale_1", _c_p), ("w_zeros_1", _c_p), ("w_scale_2", _c_p), ("w_zeros_2", _c_p),
+                ("w_rowsum_adj", _c_p), ("w_rowsum_adj_2", _c_p), ("bias", _c_p)]
+
 
 _lib = None
 

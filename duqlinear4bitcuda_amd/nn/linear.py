@@ -49,32 +49,36 @@ class _Linear4bitBase(torch.nn.Module):
         return y if self.bias is None else y + self.bias
 
     # ---- decode: quantizer + GEMM + dequant as ONE launch (up to eight rows of binary16 activations) ----
+    # _decode_spec: (epilogue mode, ((argument of _HIP.FusedDecode, buffer name), ...)) of a layer class that has a
+    # one-launch form; the weight comes first.
+    _decode_spec = None
     _decode = None
-
-    def _decode_args(self):
-        """(mode, weight, w_scale_1, w_zeros_1, w_scale_2, w_zeros_2, w_rowsum_adj, w_rowsum_adj_2) of the layer, or
-        None when it has no one-launch form."""
-        return None
+    _decode_held = ()
 
     def _decode_call(self):
         """The layer's prepared one-launch call (``_HIP.FusedDecode``), rebuilt when a buffer was replaced (moved,
         cast, reloaded into a new tensor); None for a layer that has none or is not on a GPU."""
-        args = self._decode_args()
-        if args is None:
+        spec = self._decode_spec
+        if spec is None:
             return None
+        b = self._buffers
         d = self._decode
         if d is not None:
-            held = d.tensors
-            if held[0] is args[1] and held[1] is args[2] and held[2] is args[3] and held[3] is args[4] and \
-                    held[4] is args[5] and held[5] is args[6] and held[6] is args[7] and held[7] is self.bias and \
-                    d.w_ptr == args[1].data_ptr():
-                return d
-        if not args[1].is_cuda:
+            for name, t in self._decode_held:
+                if b.get(name) is not t:
+                    break
+            else:
+                if d.w_ptr == self._decode_held[0][1].data_ptr():
+                    return d
+        names = spec[1] + (("bias", "bias"),)
+        held = tuple((buf, b.get(buf)) for _, buf in names)
+        if not held[0][1].is_cuda:
             return None
-        d = self._decode = _ops.FusedDecode(*args, bias=self.bias)
+        d = self._decode = _ops.FusedDecode(spec[0], **{arg: t for (arg, _), (_, t) in zip(names, held)})
+        self._decode_held = held
         return d
 
-    def _decode_forward(self, x, clip=1.0, qmax=6):
+    def _decode_forward(self, x, clip=1.0, qmax=6, checked=False):
         """y for binary16 rows ``x`` when the layer runs them as one launch (quantizer inside), else None."""
         K = self.in_features
         if not self.fused or x.shape[-1] != K or K % 64:
@@ -85,7 +89,7 @@ class _Linear4bitBase(torch.nn.Module):
         d = self._decode_call()
         if d is None or not d.admits(M):
             return None
-        return d.run(x, M, clip, qmax)
+        return d.run(x, M, clip, qmax, checked)
 
     def enable_fp6(self):
         """Build the E3M2 shadow of ``weight`` (3/4 byte per element next to the 1/2 byte of the packed
@@ -150,14 +154,12 @@ class Linear4bitSQ(_Linear4bitBase):
         else:
             self.bias = None
 
-    def _decode_args(self):
-        b = self._buffers
-        return (_ops.EPI_SYM, b["weight"], b["weight_scales"], None, None, None, None, None)
+    _decode_spec = (_ops.EPI_SYM, (("w", "weight"), ("w_scale_1", "weight_scales")))
 
     def forward(self, x):
         assert type(x) == tensor_utils.PackedQuantizedTensor  # quantized input is required
         if x._src is not None:  # a few rows straight from SymQuantizer: quantized inside the GEMM launch
-            y = self._decode_forward(x.source(), x._clip, x._qmax)
+            y = self._decode_forward(x.source(), x._clip, x._qmax, True)
             if y is not None:
                 return y
         xq, scales_x = x.quantized_x, x.scales_x
@@ -205,9 +207,7 @@ class Linear4bitASQ(_Linear4bitBase):
         if require_quantizer:
             self.quantizer = AsymQuantizer()
 
-    def _decode_args(self):
-        b = self._buffers
-        return (_ops.EPI_ASYM, b["weight"], b["weight_scales"], b["weight_zeros"], None, None, None, None)
+    _decode_spec = (_ops.EPI_ASYM, (("w", "weight"), ("w_scale_1", "weight_scales"), ("w_zeros_1", "weight_zeros")))
 
     def forward(self, x):
         if self.require_quantizer:
@@ -266,9 +266,8 @@ class Linear4bitASQRowSum(_Linear4bitBase):
         if require_quantizer:
             self.quantizer = AsymQuantizer(shifted=True)
 
-    def _decode_args(self):
-        b = self._buffers
-        return (_ops.EPI_ASYM_ROWSUM, b["weight"], b["weight_scales"], b["weight_zeros"], None, None, b["weight_rowsum"], None)
+    _decode_spec = (_ops.EPI_ASYM_ROWSUM, (("w", "weight"), ("w_scale_1", "weight_scales"), ("w_zeros_1", "weight_zeros"),
+                                           ("w_rowsum_adj", "weight_rowsum")))
 
     def forward(self, x):
         if self.require_quantizer:
@@ -338,10 +337,9 @@ class LinearQuant4bitDUASQRowSum(_Linear4bitBase):
         if require_quantizer:
             self.quantizer = AsymQuantizer(shifted=True)
 
-    def _decode_args(self):
-        b = self._buffers
-        return (_ops.EPI_ASYM_DUAL_ROWSUM, b["weight"], b["weight_scales_1"], b["weight_zeros_1"], b["weight_scales_2"],
-                b["weight_zeros_2"], b["weight_rowsum_1"], b["weight_rowsum_2"])
+    _decode_spec = (_ops.EPI_ASYM_DUAL_ROWSUM, (("w", "weight"), ("w_scale_1", "weight_scales_1"), ("w_zeros_1", "weight_zeros_1"),
+                                                ("w_scale_2", "weight_scales_2"), ("w_zeros_2", "weight_zeros_2"),
+                                                ("w_rowsum_adj", "weight_rowsum_1"), ("w_rowsum_adj_2", "weight_rowsum_2")))
 
     def forward(self, x):
         if self.require_quantizer:
@@ -421,14 +419,12 @@ class Linear4bitDUSQ(_Linear4bitBase):
         else:
             self.bias = None
 
-    def _decode_args(self):
-        b = self._buffers
-        return (_ops.EPI_SYM_DUAL, b["weight"], b["weight_scales_1"], None, b["weight_scales_2"], None, None, None)
+    _decode_spec = (_ops.EPI_SYM_DUAL, (("w", "weight"), ("w_scale_1", "weight_scales_1"), ("w_scale_2", "weight_scales_2")))
 
     def forward(self, x):
         assert type(x) == tensor_utils.PackedQuantizedTensor
         if x._src is not None:  # a few rows straight from SymQuantizer: quantized inside the GEMM launch
-            y = self._decode_forward(x.source(), x._clip, x._qmax)
+            y = self._decode_forward(x.source(), x._clip, x._qmax, True)
             if y is not None:
                 return y
         xq, scales_x = x.quantized_x, x.scales_x
@@ -480,10 +476,8 @@ class LinearQuant4bitDUASQ(_Linear4bitBase):
         if self.require_quantizer:
             self.quantizer = AsymQuantizer()
 
-    def _decode_args(self):
-        b = self._buffers
-        return (_ops.EPI_ASYM_DUAL, b["weight"], b["weight_scales_1"], b["weight_zeros_1"], b["weight_scales_2"],
-                b["weight_zeros_2"], None, None)
+    _decode_spec = (_ops.EPI_ASYM_DUAL, (("w", "weight"), ("w_scale_1", "weight_scales_1"), ("w_zeros_1", "weight_zeros_1"),
+                                         ("w_scale_2", "weight_scales_2"), ("w_zeros_2", "weight_zeros_2")))
 
     def forward(self, x):
         if self.require_quantizer:

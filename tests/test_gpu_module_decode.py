@@ -77,7 +77,7 @@ def test_sequential_symquantizer_linear_is_one_library_call(dev, library_calls, 
         model(X)  # first call builds the layer's prepared call
         library_calls.clear()
         y = model(X)
-        assert library_calls == ["duq_quantize_linear4bit_forward"], library_calls
+        assert library_calls == ["duq_quantize_linear4bit_forward_layer"], library_calls
         assert y.shape == (1, M, N)
         assert cases.bits_equal(y.cpu().numpy().reshape(M, N), want)
     # what the quantizer hands over still reads as a quantized tensor
@@ -107,7 +107,7 @@ def test_symquantizer_settings_reach_the_one_launch_path(dev, library_calls):
         want = orc.linear4bit_sq_forward(x, wq, sw, None, clip, qmax)[0]
         library_calls.clear()
         y = torch.nn.Sequential(SymQuantizer(clip, qmax=qmax), sq)(X)
-        assert library_calls == ["duq_quantize_linear4bit_forward"], library_calls
+        assert library_calls == ["duq_quantize_linear4bit_forward_layer"], library_calls
         assert cases.bits_equal(y.cpu().numpy(), want), (clip, qmax)
     want = orc.linear4bit_sq_forward(x, wq, sw)[0]
     eager = SymQuantizer(1.0)
@@ -152,7 +152,7 @@ def test_one_launch_follows_the_layer_buffers(dev, library_calls):
     fresh = fresh.half().to(dev)                     # a new module holds float32 scales until cast (linear.py:32-33); .to() replaces every buffer
     library_calls.clear()
     y = torch.nn.Sequential(SymQuantizer(1.0), fresh)(X)
-    assert library_calls == ["duq_quantize_linear4bit_forward"], library_calls
+    assert library_calls == ["duq_quantize_linear4bit_forward_layer"], library_calls
     assert cases.bits_equal(y.cpu().numpy(), orc.linear4bit_sq_forward(x, wq2, sw2, b)[0])
 
 
@@ -192,7 +192,7 @@ def test_asymmetric_layers_decode_in_one_library_call(dev, library_calls, M, N, 
         layer(X)
         library_calls.clear()
         y = layer(X)
-        assert library_calls == ["duq_quantize_linear4bit_forward_asym"], (type(layer).__name__, library_calls)
+        assert library_calls == ["duq_quantize_linear4bit_forward_layer"], (type(layer).__name__, library_calls)
         assert cases.bits_equal(y.detach().cpu().numpy(), want), type(layer).__name__
         layer.fused = False   # the reference's sequence of steps: same bits
         assert cases.bits_equal(layer(X).cpu().numpy(), want), type(layer).__name__
@@ -303,7 +303,7 @@ def test_dual_uniform_rowsum_layer_decode(dev, library_calls, M, N, K):
     library_calls.clear()
     y = layer(X)
     if M <= 8:
-        assert library_calls == ["duq_quantize_linear4bit_forward_asym"], library_calls
+        assert library_calls == ["duq_quantize_linear4bit_forward_layer"], library_calls
     elif M <= 64:
         assert library_calls == ["duq_quantize_rows_asym_shifted", "duq_linear4bit_forward_dual_rowsum"], library_calls
     assert cases.bits_equal(y.detach().cpu().numpy(), want)
