@@ -128,6 +128,13 @@ int launch_activation_shadow_bf6(const uint8_t *q, uint32_t M, uint32_t K, uint8
 // prefetches issued just before it (a full memory latency per chunk).
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+// Cache policy of the output stores: 2 = non-temporal.  The output is written once and read by nobody in this
+// launch; streamed past the L2 it leaves the operand panels there and the launch ends sooner (measured at
+// M = 2048, N = K = 4096: 21.8 against 23.0 us; same bits).
+#ifndef DUQ_BF6_STORE_AUX
+#define DUQ_BF6_STORE_AUX 2
+#endif
+
 #ifndef DUQ_BF6_COST256
 #define DUQ_BF6_COST256 1.78f
 #endif
@@ -606,7 +613,7 @@ __global__ __launch_bounds__(256) void gemm_bf6_kernel(DUQ_HEAD_DECL, Bf6Params 
         const uint32_t row = it * RPI + rsub;
         const v4u v = *reinterpret_cast<const v4u *>(stage + row * kYStride + piece * 16);
         const uint32_t off = (row < rows_here && ncol0 < p.N) ? (row * p.N + ncol0) * 2 : kOobOffset;
-        __builtin_amdgcn_raw_buffer_store_b128(v, rY, (int)off, 0, 0);
+        __builtin_amdgcn_raw_buffer_store_b128(v, rY, (int)off, 0, DUQ_BF6_STORE_AUX);
     }
 }
 
