@@ -33,6 +33,13 @@
 #ifndef DUQ_DEC_R
 #define DUQ_DEC_R 4
 #endif
+// Cache policy of the rows kernel's weight loads (and of the read probe that mirrors them): 2 = non-temporal.  A
+// load instruction of that kernel covers whole cache lines that nobody reads again (measured, one row: N = K = 4096
+// 3.00 against 3.08 us, N = 28672 K = 8192 19.6 against 21.2).  The MFMA kernel reads a line in two instructions (64
+// bytes of a row each) and loses with it (16 rows, N = K = 4096: 4.13 against 3.90 us): it keeps the default.
+#ifndef DUQ_DEC_WLOAD_AUX
+#define DUQ_DEC_WLOAD_AUX 2
+#endif
 #ifndef DUQ_DEC_WAVES
 #define DUQ_DEC_WAVES 8
 #endif
@@ -209,7 +216,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DUQ_HEAD_DECL,
                 const uint32_t off = i * 1024 + lane * 16;
                 // K % 64 == 0: a 16-byte piece is all in or all out
                 const bool ok = off < kbytes && n0 + r < nrows;
-                w[r][i] = buf_load16(rW, ok ? (n0 + r) * kbytes + off : kOobOffset, 0);
+                w[r][i] = __builtin_bit_cast(
+                    v4u, __builtin_amdgcn_raw_buffer_load_b128(rW, (int)(ok ? (n0 + r) * kbytes + off : kOobOffset), 0, DUQ_DEC_WLOAD_AUX));
             }
     };
     v4u w0[R][XS], w1[MULTI ? R : 1][MULTI ? XS : 1];
@@ -696,7 +704,8 @@ __global__ __launch_bounds__(256) void probe_read_kernel(const v4u *src, uint32_
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         const uint32_t idx = gw * 512 + i * 64 + lane;
-        v[i] = buf_load16(r, idx < nvec ? idx * 16 : kOobOffset, 0);
+        v[i] = __builtin_bit_cast(
+            v4u, __builtin_amdgcn_raw_buffer_load_b128(r, (int)(idx < nvec ? idx * 16 : kOobOffset), 0, DUQ_DEC_WLOAD_AUX));
     }
     uint32_t x = 0;
 #pragma unroll

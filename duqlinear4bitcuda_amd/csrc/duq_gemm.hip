@@ -29,6 +29,20 @@
 #include "duq_epilogue.h"
 // Cache policy of the stream / short-row kernels' output stores: 2 = non-temporal (the output is written once and
 // read by nobody in the launch; measured at M = 2048, N = K = 4096: 30.2 against 31.5 us, M = 4096: 58.8 against 61.1)
+// Cache policy of the weight loads of the kernels that read every weight byte once: 2 = non-temporal.  Measured:
+// skinny kernel 16 x 28672 x 4096 13.2 against 14.1 us, dot kernel 1 x 8192 x 28672 20.9 against 22.8 and 4 x 4096 x
+// 20480 11.5 against 13.2; the ring kernel (row groups read the weights again; a lane fetches 16 bytes of a row, a
+// quarter of a cache line, per instruction) loses on most shapes (100 x 1000 x 4096: 7.9 against 7.3) and keeps the
+// default.
+#ifndef DUQ_SKINNY_WLOAD_AUX
+#define DUQ_SKINNY_WLOAD_AUX 2
+#endif
+#ifndef DUQ_RING_WLOAD_AUX
+#define DUQ_RING_WLOAD_AUX 0
+#endif
+#ifndef DUQ_DOT_WLOAD_AUX
+#define DUQ_DOT_WLOAD_AUX 2
+#endif
 #ifndef DUQ_STREAM_STORE_AUX
 #define DUQ_STREAM_STORE_AUX 2
 #endif
@@ -669,7 +683,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_s4_skinny_kernel(DUQ_HEAD_DEC
             const uint32_t rt = (u & 1) * 8 + r8, row = tile * 16 + rt;
             const uint32_t off = seg0 * 64 + (u >> 1) * 128 + ((j8 ^ ((rt >> 1) & 7u)) << 4);
             const bool ok = tile < tile_end && row < p.N && off < kbytes;
-            w[u] = buf_load16(rW, ok ? row * kbytes + off : kOobOffset, 0);
+            w[u] = buf_load16_aux<DUQ_SKINNY_WLOAD_AUX>(rW, ok ? row * kbytes + off : kOobOffset, 0);
         }
     };
     auto compute_tile = [&](uint32_t tile, const v4u(&w)[kSkinnySegs], uint32_t buf) {
@@ -775,7 +789,7 @@ __global__ __launch_bounds__(256) void gemm_s4_ring_kernel(DUQ_HEAD_DECL, GemmPa
         const uint32_t sg = blk * kRing + j;
         const uint32_t off = (seg_lo + sg) * 64 + g * 16;
         const bool ok = it < items && row < p.N && sg < sps && off < kbytes;
-        ring[j] = buf_load16(rW, ok ? row * kbytes + off : kOobOffset, 0);
+        ring[j] = buf_load16_aux<DUQ_RING_WLOAD_AUX>(rW, ok ? row * kbytes + off : kOobOffset, 0);
     };
 #pragma unroll
     for (int j = 0; j < kRing; ++j) issue(0, 0, j);  // the first weights are under way before the activations
@@ -895,7 +909,7 @@ __global__ __launch_bounds__(256) void gemv_s4_dot_kernel(DUQ_HEAD_DECL, GemmPar
 
     v4u ring[kDotRing];
 #pragma unroll
-    for (int u = 0; u < kDotRing; ++u) ring[u] = buf_load16(rW, w_off(u), 0);
+    for (int u = 0; u < kDotRing; ++u) ring[u] = buf_load16_aux<DUQ_DOT_WLOAD_AUX>(rW, w_off(u), 0);
 
     // activations -> LDS (all rows, whole K), zero beyond the row end
     for (uint32_t i = tid; i < MROWS * (xstride / 16); i += 256) {
@@ -914,7 +928,7 @@ __global__ __launch_bounds__(256) void gemv_s4_dot_kernel(DUQ_HEAD_DECL, GemmPar
 #pragma unroll
         for (int u = 0; u < kDotRing; ++u) {
             const v4u w = ring[u];
-            ring[u] = buf_load16(rW, w_off(s + u + kDotRing), 0);
+            ring[u] = buf_load16_aux<DUQ_DOT_WLOAD_AUX>(rW, w_off(s + u + kDotRing), 0);
             const uint32_t xo = (step0 + s + u) * 128 + j * 16;
             if (s + u < nsteps) {
 #pragma unroll

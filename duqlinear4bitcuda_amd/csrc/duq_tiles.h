@@ -36,5 +36,11 @@ __device__ __forceinline__ v4u buf_load16(__amdgpu_buffer_rsrc_t r, uint32_t vof
 {
     return __builtin_bit_cast(v4u, __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)soff, 0));
 }
+// The same with a cache policy (2 = non-temporal: for bytes that are read once, in whole cache lines).
+template <int AUX>
+__device__ __forceinline__ v4u buf_load16_aux(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff)
+{
+    return __builtin_bit_cast(v4u, __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)soff, AUX));
+}
 
 }  // namespace duq
