@@ -316,7 +316,7 @@ def fanout_section(dev):
 LLAMA7B_DECODE = [(M, N, 4096) for N in (4096, 11008) for M in (1, 4, 16)]   # configuration 2
 
 
-def decode_section(dev, quick):
+def decode_section(dev, quick, eager=True):
     """HBM-bound decode at configuration 2 and around it.  Per shape, HIP-graph timed, with the weights rotated
     over more than 512 MB of distinct buffers so that no launch finds its weights in a cache:
       us            binary16 activations in -> per-token quantize -> GEMM -> fp16 out, the single entry point
@@ -359,12 +359,12 @@ def decode_section(dev, quick):
             layer.weight_scales = sw
             models.append(torch.nn.Sequential(SymQuantizer(1.0), layer))
         us_mod_graph = graph_time_us([(lambda m=m: m(x3)) for m in models] * 2)
-        us_mod_eager = eager_wall_us(models, x3)
+        us_mod_eager = eager_wall_us(models, x3) if eager else float("nan")
         byts = 2 * M * K + wbytes + 2 * N + 2 * M * N
         out.append({"M": M, "N": N, "K": K, "us": round(us, 3), "GBps": round(byts / us / 1e3, 1),
                     "frac_hbm": round(byts / us / 1e3 / PEAK_HBM_GBS, 4),
                     "launches": 1 if hip.quantize_linear4bit_one_launch(M, N, K) else 2,
-                    "module_graph_us": round(us_mod_graph, 3), "module_eager_us": round(us_mod_eager, 3),
+                    "module_graph_us": round(us_mod_graph, 3), "module_eager_us": round(us_mod_eager, 3) if eager else None,
                     "module_launches": 1 if M <= 8 and hip.quantize_linear4bit_one_launch(M, N, K) else 2,
                     "gemm_only_us": round(us_gemm, 3),
                     "gemm_only_GBps": round((byts - 2 * M * K + M * K // 2 + 2 * M) / us_gemm / 1e3, 1),
@@ -606,6 +606,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=300)
     ap.add_argument("--quick", action="store_true", help="skip the larger decode shapes and shorten the CPU baseline")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-harness", action="store_true",
+                    help="skip the eager wall-clock sections (the reference's harness table, the modules' eager decode "
+                         "figures): for runs under a profiler, where every launch is slow")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU path exists or is measured)",
@@ -738,13 +741,13 @@ def main():
     # the driver record keeps `roofline`: the integer path's figures ride inside it as a second entry
     roofline["integer_path"] = integer_path["roofline"]
 
-    decode = decode_section(dev, args.quick)
+    decode = decode_section(dev, args.quick, eager=not args.no_harness)
     quantizer = quantizer_section(dev)
     asym = None if args.quick else asym_section(dev)
     other = None if args.quick else other_shapes_section(dev)
     int8_layer = int8_layer_section(dev, args.quick)
     batched = batched_section(dev, args.quick)
-    harness = harness_section(dev, args.quick)
+    harness = None if args.no_harness else harness_section(dev, args.quick)
     fanout = None if args.quick else fanout_section(dev)
     rows_7b = [d for d in decode if (d["M"], d["N"], d["K"]) in LLAMA7B_DECODE]
     worst = min(rows_7b, key=lambda d: d["frac_hbm"])

@@ -135,6 +135,9 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 #define DUQ_BF6_STORE_AUX 2
 #endif
 
+#ifndef DUQ_BF6_COST64
+#define DUQ_BF6_COST64 0.68f
+#endif
 #ifndef DUQ_BF6_COST256
 #define DUQ_BF6_COST256 1.78f
 #endif
@@ -632,7 +635,7 @@ static void launch_mode(Bf6Params &p, hipStream_t stream)
 {
     // Tile height: whole rounds of 256 workgroups, with a 64-row / 256-row tile priced relative to a 128-row one
     // (the weight traffic per tile is the same, the MFMAs are half / twice; measured on an MI355X).
-    constexpr float kCost64 = 0.68f, kCost256 = DUQ_BF6_COST256;
+    constexpr float kCost64 = DUQ_BF6_COST64, kCost256 = DUQ_BF6_COST256;
     const uint32_t t256 = ((p.M + 255) / 256) * p.tiles_n, t128 = ((p.M + 127) / 128) * p.tiles_n,
                    t64 = ((p.M + 63) / 64) * p.tiles_n;
     const float c256 = kCost256 * (float)((t256 + 255) / 256), c128 = (float)((t128 + 255) / 256),
