@@ -365,7 +365,8 @@ def decode_section(dev, quick, eager=True):
                     "frac_hbm": round(byts / us / 1e3 / PEAK_HBM_GBS, 4),
                     "launches": 1 if hip.quantize_linear4bit_one_launch(M, N, K) else 2,
                     "module_graph_us": round(us_mod_graph, 3), "module_eager_us": round(us_mod_eager, 3) if eager else None,
-                    "module_launches": 1 if M <= 8 and hip.quantize_linear4bit_one_launch(M, N, K) else 2,
+                    "module_launches": 1 if hip.quantize_linear4bit_one_launch(M, N, K) else 2,
+                    "module_library_calls": 1 if M <= 64 else 2,
                     "gemm_only_us": round(us_gemm, 3),
                     "gemm_only_GBps": round((byts - 2 * M * K + M * K // 2 + 2 * M) / us_gemm / 1e3, 1),
                     "read_floor_us": round(us_read, 3), "read_floor_GBps": round(wbytes / us_read / 1e3, 1),

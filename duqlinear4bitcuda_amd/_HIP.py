@@ -558,7 +558,7 @@ class FusedDecode:
     """One layer's side of the one-launch decode (what ``duq_quantize_linear4bit_forward`` takes for the symmetric
     modes and ``duq_quantize_linear4bit_forward_asym`` for the asymmetric and row-sum modes), checked once and kept
     as a ``duq_fused_layer`` struct for ``duq_quantize_linear4bit_forward_layer``: a decode step of a module then
-    costs one ``torch.empty`` and one foreign call with five arguments.  The tensors are held (``tensors``) so that
+    costs one ``torch.empty`` (two above eight rows: the staging buffer) and one foreign call with seven arguments.  The tensors are held (``tensors``) so that
     a caller can tell when the layer's buffers were replaced; a change of their contents in place needs no new
     object."""
 
@@ -614,12 +614,30 @@ class FusedDecode:
             ref = self._structs[key] = (ctypes.addressof(st), st)   # (the struct is kept alive beside its address)
         return ref[0]
 
+    # Rows up to which a module hands binary16 activations to this call: the decode kernels' range.  Up to eight
+    # rows (and N <= 16384) it is one launch; above, the quantizer launch and the GEMM launch of one library call.
+    max_rows = 64
+
+    def _staging(self, M: int) -> int:
+        """Bytes the library stages between its two launches at M rows (0: one launch); -1 when M is out of range."""
+        b = self._one.get(M)
+        if b is None:
+            if not 0 < M <= self.max_rows:
+                b = -1
+            elif self.mode in (EPI_SYM, EPI_SYM_DUAL):
+                b = self._lib.duq_quantize_linear4bit_workspace_bytes(M, self.N, self.K)
+            else:
+                b = self._lib.duq_quantize_linear4bit_asym_workspace_bytes(self.mode, M, self.N, self.K)
+            self._one[M] = b
+        return b
+
     def admits(self, M: int) -> bool:
-        """True when M rows of this layer run as ONE launch with nothing staged."""
-        one = self._one.get(M)
-        if one is None:
-            one = self._one[M] = M > 0 and self._lib.duq_quantize_linear4bit_workspace_bytes(M, self.N, self.K) == 0
-        return one
+        """True when M rows of this layer run through one library call from binary16 rows."""
+        return self._staging(M) >= 0
+
+    def one_launch(self, M: int) -> bool:
+        """True when M rows run as ONE launch with nothing staged."""
+        return self._staging(M) == 0
 
     def run(self, x: torch.Tensor, M: int, clip: float = 1.0, qmax: int = 6, checked: bool = False) -> torch.Tensor:
         """x: contiguous binary16 [..., K] on the layer's device, 16-byte aligned, M = its rows with admits(M);
@@ -629,15 +647,25 @@ class FusedDecode:
                 not (checked or (x.dtype is _F16 and x.is_contiguous())):
             raise RuntimeError(f"FusedDecode: expected a contiguous float16 tensor [..., {self.K}] on {self.device}, got "
                                f"{x.dtype} {tuple(x.shape)} on {x.device}")
+        nbytes = self._one.get(M)
+        if nbytes is None:
+            nbytes = self._staging(M)
+        if nbytes < 0:
+            raise RuntimeError(f"FusedDecode: {M} rows (at most {self.max_rows})")
         y = torch.empty(x.shape[:-1] + (self.N,), dtype=_F16, device=self.device)
         idx = self.index
         ref = self._structs.get((clip, qmax))
         layer = ref[0] if ref is not None else self._layer(clip, qmax)
+        if nbytes:
+            ws = torch.empty(nbytes, dtype=_U8, device=self.device)
+            ws_ptr = ws.data_ptr()
+        else:
+            ws_ptr = None
         if idx == torch._C._cuda_getDevice():
-            st = self._fn(layer, x.data_ptr(), M, y.data_ptr(), _raw_stream(idx))
+            st = self._fn(layer, x.data_ptr(), M, y.data_ptr(), ws_ptr, nbytes, _raw_stream(idx))
         else:
             with torch.cuda.device(idx):
-                st = self._fn(layer, x.data_ptr(), M, y.data_ptr(), _raw_stream(idx))
+                st = self._fn(layer, x.data_ptr(), M, y.data_ptr(), ws_ptr, nbytes, _raw_stream(idx))
         if st:
             _lib.check(st, "quantize_linear4bit_forward")
         return y

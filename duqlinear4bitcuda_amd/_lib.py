@@ -46,7 +46,7 @@ PROTOTYPES = {
     "duq_quantize_linear4bit_forward_static": [_c_i32, _c_p, ctypes.c_float, _c_i32, _c_p, _c_p, _c_p, _c_p, _c_u32,
                                                _c_u32, _c_u32, _c_p, _c_p, _c_p, _c_u32, _c_p],
     "duq_static_scratch_init": [],
-    "duq_quantize_linear4bit_forward_layer": [_c_p, _c_p, _c_u32, _c_p, _c_p],
+    "duq_quantize_linear4bit_forward_layer": [_c_p, _c_p, _c_u32, _c_p, _c_p, ctypes.c_uint64, _c_p],
     "duq_quantize_linear4bit_asym_workspace_bytes": [_c_i32, _c_u32, _c_u32, _c_u32],  # returns uint64_t
     "duq_quantize_linear4bit_forward_asym": [_c_i32, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_u32, _c_u32,
                                              _c_u32, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, ctypes.c_uint64, _c_p],

@@ -466,18 +466,18 @@ int duq_quantize_linear4bit_forward_asym(int32_t mode, const duq_half *x, const 
 }
 
 int duq_quantize_linear4bit_forward_layer(const duq_fused_layer *layer, const duq_half *x, uint32_t M, duq_half *y,
-                                          duq_stream_t stream)
+                                          void *workspace, uint64_t workspace_bytes, duq_stream_t stream)
 {
     if (!layer) return DUQ_E_NULL;
     const duq_fused_layer &l = *layer;
     if (l.mode < DUQ_EPI_SYM || l.mode > DUQ_EPI_ASYM_DUAL_ROWSUM) return DUQ_E_MODE;
     if (M == 0 || l.N == 0) return DUQ_OK;
-    if (l.K == 0 || !duq::decode_fp16in_one_launch(M, l.N, l.K)) return DUQ_E_SHAPE;
+    if (l.K == 0) return DUQ_E_SHAPE;
     const bool sym = l.mode == DUQ_EPI_SYM || l.mode == DUQ_EPI_SYM_DUAL;
     duq::Epilogue e{l.mode,      nullptr, nullptr, l.w_scale_1,    sym ? nullptr : l.w_zeros_1, l.w_scale_2,
                     sym ? nullptr : l.w_zeros_2, l.bias,  nullptr, l.w_rowsum_adj, l.w_rowsum_adj_2};
     return quantize_linear_impl(e, x, sym ? l.clip : 1.0f, sym ? l.qmax : DUQ_QMAX_SYM_DEVICE, l.w, M, l.N, l.K, y,
-                                FusedOut{nullptr, nullptr, nullptr, nullptr}, nullptr, 0, stream);
+                                FusedOut{nullptr, nullptr, nullptr, nullptr}, workspace, workspace_bytes, stream);
 }
 
 int duq_static_scratch_init(void)

@@ -79,12 +79,13 @@ class _Linear4bitBase(torch.nn.Module):
         return d
 
     def _decode_forward(self, x, clip=1.0, qmax=6, checked=False):
-        """y for binary16 rows ``x`` when the layer runs them as one launch (quantizer inside), else None."""
+        """y for binary16 rows ``x`` when the layer takes them in one library call (up to eight rows: one launch,
+        quantizer inside; up to 64: quantizer launch + GEMM launch), else None."""
         K = self.in_features
         if not self.fused or x.shape[-1] != K or K % 64:
             return None
         M = x.numel() // K
-        if M > 8 or M == 0:
+        if M > _ops.FusedDecode.max_rows or M == 0:
             return None
         d = self._decode_call()
         if d is None or not d.admits(M):

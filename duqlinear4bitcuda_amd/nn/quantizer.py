@@ -28,10 +28,12 @@ class SymQuantizer(torch.nn.Module):
     (include/common.h:53-54), 7 what its Python fake-quant path applies."""
 
     # Inputs of at most this many rows (decode) are handed on unquantized inside the PackedQuantizedTensor: a
-    # Linear4bitSQ / Linear4bitDUSQ that follows quantizes them inside its own launch (quantizer + GEMM + dequant
-    # are then ONE launch), and anything else that reads quantized_x / scales_x triggers this quantizer's launch
-    # then, with the same bits.  0 switches that off.
-    defer_rows = 8
+    # Linear4bitSQ / Linear4bitDUSQ that follows quantizes them inside its own library call (up to eight rows
+    # quantizer + GEMM + dequant are ONE launch; above, the quantizer launch and the GEMM launch of one call: at
+    # these sizes a step costs more on the host than on the GPU, and a call less is most of it), and anything
+    # else that reads quantized_x / scales_x triggers this quantizer's launch then, with the same bits.  0
+    # switches that off.
+    defer_rows = 64
 
     def __init__(self, input_clip_ratio=1.0, qmax: int = 6, shadow=False, shadow_min_rows: int = 96):
         super().__init__()

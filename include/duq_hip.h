@@ -273,10 +273,12 @@ int duq_quantize_linear4bit_forward_asym(int32_t mode, const duq_half *x, const 
                                          uint64_t workspace_bytes, duq_stream_t stream);
 
 /* The two entry points above with the layer's side of the arguments in a struct the caller fills once per layer
- * (no counterpart in the reference): a decode step then passes five arguments instead of seventeen to twenty, which
+ * (no counterpart in the reference): a decode step then passes seven arguments instead of seventeen to twenty, which
  * is what a step costs on the host when it goes through a foreign-function interface (ctypes: about 0.1 us per
- * argument).  Only shapes that run as ONE launch are taken (duq_quantize_linear4bit_workspace_bytes(M, N, K) == 0):
- * others return DUQ_E_SHAPE before anything is launched, and the caller uses the full entry points.
+ * argument).  Shapes that run as ONE launch take no workspace (NULL, 0); the others stage what the quantizer
+ * launch hands to the GEMM launch in `workspace`, of duq_quantize_linear4bit_workspace_bytes(M, N, K) bytes for the
+ * symmetric modes and duq_quantize_linear4bit_asym_workspace_bytes(mode, M, N, K) for the others, 16-byte aligned
+ * (DUQ_E_NULL without one, DUQ_E_SHAPE for one that is too small, before anything is launched).
  *   mode  DUQ_EPI_SYM / DUQ_EPI_SYM_DUAL (clip, qmax as duq_quantize_rows_sym) or one of the asymmetric modes of
  *         duq_quantize_linear4bit_forward_asym (clip, qmax ignored); pointers a mode does not use are NULL */
 typedef struct duq_fused_layer {
@@ -290,7 +292,7 @@ typedef struct duq_fused_layer {
     const duq_half *bias;
 } duq_fused_layer;
 int duq_quantize_linear4bit_forward_layer(const duq_fused_layer *layer, const duq_half *x, uint32_t M, duq_half *y,
-                                          duq_stream_t stream);
+                                          void *workspace, uint64_t workspace_bytes, duq_stream_t stream);
 
 /* No counterpart in the reference.  For callers that cannot allocate device memory or carry a workspace around
  * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc):

@@ -214,10 +214,14 @@ public:
     float input_clip_ratio;
     int qmax;
     bool shadow;  // also write the 6-bit float shadow (inputs whose width is a multiple of 128)
-    // inputs of at most this many rows are handed on unquantized (PackedQuantizedTensor::deferred): the linear
-    // layer behind quantizes them inside its own launch; 0 switches that off
+    // defer_rows > 0 (at most 64 is useful): inputs of at most that many rows are handed on unquantized
+    // (PackedQuantizedTensor::deferred) and the linear layer behind quantizes them inside its own library call (one
+    // launch up to eight rows, the quantizer launch and the GEMM launch of one call above).  Off by default: the
+    // fields quantized_x and scale of such a tensor are undefined until materialize(), and code written against the
+    // reference reads them as plain members (test/test.cu:238-242).  A decode pipeline that only passes the tensor
+    // on, torch::nn::Sequential(Quantizer4bit(clip, qmax, false, 64), Linear4bit) (test/pipeline.cu:107-110), turns it on.
     uint32_t defer_rows;
-    explicit Quantizer4bit(float input_clip_ratio, int qmax = DUQ_QMAX_SYM_DEVICE, bool shadow = false, uint32_t defer_rows = 8)
+    explicit Quantizer4bit(float input_clip_ratio, int qmax = DUQ_QMAX_SYM_DEVICE, bool shadow = false, uint32_t defer_rows = 0)
         : input_clip_ratio(input_clip_ratio), qmax(qmax), shadow(shadow), defer_rows(defer_rows) {}
     PackedQuantizedTensor forward(torch::Tensor x)
     {
@@ -308,8 +312,9 @@ inline torch::Tensor fused_forward_shadow(int mode, const PackedQuantizedTensor 
     return y.view(lead);
 }
 
-// A deferred input on a shape that runs quantizer + GEMM + dequant as ONE launch: the result; else an undefined
-// tensor (the caller then materializes the input and takes the usual route).
+// A deferred input of at most 64 rows: quantizer + GEMM + dequant in one library call (ONE launch where the shape
+// allows, else two with the codes and scales staged in a workspace allocated here); else an undefined tensor (the
+// caller then materializes the input and takes the usual route).
 inline torch::Tensor fused_decode(int mode, const PackedQuantizedTensor &input, const torch::Tensor &weight,
                                   const torch::Tensor &s1, const torch::Tensor &s2, const torch::Tensor &bias)
 {
@@ -318,15 +323,18 @@ inline torch::Tensor fused_decode(int mode, const PackedQuantizedTensor &input, 
     TORCH_CHECK(x.device() == weight.device(), "Linear4bit::forward: operands on different devices");
     TORCH_CHECK(weight.size(1) * 2 == x.size(-1), "Linear4bit::forward: K differs");
     const uint32_t K = x.size(-1), M = x.numel() / K, N = weight.size(0);
-    if (duq_quantize_linear4bit_workspace_bytes(M, N, K) != 0) return torch::Tensor();
+    if (M > 64) return torch::Tensor();
+    const uint64_t ws_bytes = duq_quantize_linear4bit_workspace_bytes(M, N, K);
+    torch::Tensor ws;
+    if (ws_bytes) ws = torch::empty({(int64_t)ws_bytes}, torch::dtype(torch::kUInt8).device(x.device()));
     std::vector<int64_t> shape(x.sizes().begin(), x.sizes().end());
     shape.back() = N;
     auto y = torch::empty(shape, torch::dtype(torch::kHalf).device(x.device()));
     check_status(duq_quantize_linear4bit_forward(mode, half_ptr(x), input.clip, input.qmax, weight.data_ptr<uint8_t>(),
                                                  half_ptr(s1), s2.defined() ? half_ptr(s2) : nullptr,
                                                  bias.defined() ? half_ptr(bias) : nullptr, M, N, K,
-                                                 reinterpret_cast<duq_half *>(y.data_ptr()), nullptr, nullptr, nullptr, 0,
-                                                 current_stream(x)),
+                                                 reinterpret_cast<duq_half *>(y.data_ptr()), nullptr, nullptr,
+                                                 ws_bytes ? ws.data_ptr() : nullptr, ws_bytes, current_stream(x)),
                  "Linear4bit::forward");
     return y;
 }

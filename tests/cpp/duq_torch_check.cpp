@@ -98,7 +98,7 @@ int main(int argc, char **argv)
     auto w = lin->weight.detach();
     auto ws = (w.abs().amax(1, true).to(torch::kFloat32) / 7.0).to(torch::kHalf);
 
-    duq::Quantizer4bit quant(1.0f, DUQ_QMAX_SYM_DEVICE, false, 0);  // always quantizes at once (the decode hand-over is checked below)
+    duq::Quantizer4bit quant(1.0f);  // quantizes at once (the default; the decode hand-over is checked below)
     auto p = quant.forward(x);
     if (p.quantized_x.size(-1) != K / 2 || p.scale.size(-1) != 1 || p.scale.dim() != 3) { std::puts("FAIL quantizer shapes"); return 1; }
 
@@ -159,19 +159,19 @@ int main(int argc, char **argv)
         if (!same_bits(l.forward(p4), y4)) { std::puts("FAIL Linear4bit without an activation shadow"); return 1; }
     }
 
-    // decode: up to eight rows are handed from Quantizer4bit to the layer unquantized and run as ONE launch
-    // (torch::nn::Sequential(Quantizer4bit, Linear4bit), test/pipeline.cu:107-110 of the reference); same bits as
-    // the quantizer launch followed by the GEMM launch, and as the three steps
+    // decode: up to 64 rows are handed from Quantizer4bit to the layer unquantized and run in one library call (ONE
+    // launch up to eight rows) (torch::nn::Sequential(Quantizer4bit, Linear4bit), test/pipeline.cu:107-110 of the
+    // reference); same bits as the quantizer call followed by the GEMM call, and as the three steps
     if (K % 64 == 0) {
         duq::Quantizer4bit &eager = quant;
-        duq::Quantizer4bit handover(1.0f);
-        for (int64_t rows : {1, 4, 8}) {
+        duq::Quantizer4bit handover(1.0f, DUQ_QMAX_SYM_DEVICE, false, 64);
+        for (int64_t rows : {1, 4, 8, 16, 64}) {
             if (rows > M) continue;
             auto xd = x.view({-1, K}).slice(0, 0, rows).contiguous().view({1, rows, K});
             auto pd8 = handover.forward(xd);
             if (!pd8.is_deferred() || pd8.sizes() != torch::IntArrayRef({1, rows, K / 2})) { std::puts("FAIL decode input not deferred"); return 1; }
             auto pe = eager.forward(xd);
-            if (pe.is_deferred()) { std::puts("FAIL defer_rows = 0 deferred"); return 1; }
+            if (pe.is_deferred()) { std::puts("FAIL deferred by default"); return 1; }
             auto y1 = l.forward(pd8), y2 = l.forward(pe);
             auto acc8 = duq::matmul(pe.quantized_x.view({-1, K / 2}), l.weight);
             auto y38 = (duq::sym_dequant(acc8, pe.scale.view(-1), l.weight_scale.view(-1), 32) + l.bias).view({1, rows, N});
@@ -182,7 +182,7 @@ int main(int argc, char **argv)
                 std::puts("FAIL materialize"); return 1;
             }
         }
-        torch::nn::Sequential seq(duq::Quantizer4bit(1.0f), duq::Linear4bit::from_float(lin, ws));
+        torch::nn::Sequential seq(duq::Quantizer4bit(1.0f, DUQ_QMAX_SYM_DEVICE, false, 64), duq::Linear4bit::from_float(lin, ws));
         auto xs = x.view({-1, K}).slice(0, 0, 3).contiguous();
         if (!same_bits(seq->forward(xs), l.forward(eager.forward(xs)))) { std::puts("FAIL Sequential decode"); return 1; }
     }

@@ -1,6 +1,6 @@
 """Decode through the drop-in modules: Sequential(SymQuantizer, Linear4bitSQ / Linear4bitDUSQ) and the layers with
-their own AsymQuantizer run quantizer + GEMM + dequant as ONE library call for up to eight rows, with the bits of
-the oracle; and the binary16-input entry point of the asymmetric modes against the oracle, through the C ABI."""
+their own AsymQuantizer run quantizer + GEMM + dequant as ONE library call for up to 64 rows (one launch up to
+eight), with the bits of the oracle; and the binary16-input entry point of the asymmetric modes against the oracle, through the C ABI."""
 import numpy as np
 import pytest
 import torch
@@ -59,11 +59,11 @@ def _sq_layers(dev, N, K, seed, bias):
     return sq, du, wq, sw, sw2, b
 
 
-@pytest.mark.parametrize("M", [1, 4, 8])
+@pytest.mark.parametrize("M", [1, 4, 8, 16, 64])
 @pytest.mark.parametrize("N", [4096, 11008])
 def test_sequential_symquantizer_linear_is_one_library_call(dev, library_calls, M, N):
-    """Configuration 2 shapes through the reference's own usage (test/benchmark.py:67-70): one launch, the oracle's
-    bits, for Linear4bitSQ and Linear4bitDUSQ; reading the quantized tensor afterwards still gives the quantizer's
+    """Configuration 2 shapes through the reference's own usage (test/benchmark.py:67-70): one library call, the
+    oracle's bits, for Linear4bitSQ and Linear4bitDUSQ; reading the quantized tensor afterwards still gives the quantizer's
     codes and scales."""
     from duqlinear4bitcuda_amd.nn import SymQuantizer
     K = 4096
@@ -97,7 +97,7 @@ def test_sequential_symquantizer_linear_is_one_library_call(dev, library_calls, 
 
 def test_symquantizer_settings_reach_the_one_launch_path(dev, library_calls):
     """clip ratio and upper clamp of the quantizer in front, a quantizer with deferral switched off, a layer with
-    fused = False, more than eight rows, and an input written to between the quantizer and the layer."""
+    fused = False, nine and 65 rows, and an input written to between the quantizer and the layer."""
     from duqlinear4bitcuda_amd.nn import SymQuantizer
     M, N, K = 3, 200, 1024
     sq, _, wq, sw, _, _ = _sq_layers(dev, N, K, seed=5, bias=False)
@@ -120,11 +120,12 @@ def test_symquantizer_settings_reach_the_one_launch_path(dev, library_calls):
     assert cases.bits_equal(torch.nn.Sequential(SymQuantizer(1.0), sq)(X).cpu().numpy(), want)
     assert library_calls == ["duq_quantize_rows_sym", "duq_matmul_host_4bit", "duq_sym_dequant_host"], library_calls
     sq.fused = True
-    x9 = cases.acts_normal(9, K, seed=7)
-    library_calls.clear()
-    y9 = torch.nn.Sequential(SymQuantizer(1.0), sq)(cases.t(x9, dev))
-    assert library_calls == ["duq_quantize_rows_sym", "duq_linear4bit_forward"], library_calls
-    assert cases.bits_equal(y9.cpu().numpy(), orc.linear4bit_sq_forward(x9, wq, sw)[0])
+    for rows, calls in ((9, ["duq_quantize_linear4bit_forward_layer"]), (65, ["duq_quantize_rows_sym", "duq_linear4bit_forward"])):
+        x9 = cases.acts_normal(rows, K, seed=7)
+        library_calls.clear()
+        y9 = torch.nn.Sequential(SymQuantizer(1.0), sq)(cases.t(x9, dev))
+        assert library_calls == calls, (rows, library_calls)
+        assert cases.bits_equal(y9.cpu().numpy(), orc.linear4bit_sq_forward(x9, wq, sw)[0])
     pq = SymQuantizer(1.0)(X)
     X.add_(1)
     with pytest.raises(RuntimeError, match="modified in place"):
@@ -162,10 +163,11 @@ def _asym_weights(N, K, seed):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (4, 11008, 4096), (8, 4096, 4096), (3, 100, 2048), (2, 64, 8192),
-                                    (7, 300, 1024), (4, 16000, 128)])
+                                    (7, 300, 1024), (4, 16000, 128), (16, 4096, 4096), (40, 1000, 1024), (64, 11008, 4096)])
 def test_asymmetric_layers_decode_in_one_library_call(dev, library_calls, M, N, K):
     """Linear4bitASQ, LinearQuant4bitDUASQ (qlinear4bit/nn/linear.py:104-115, 239-250) and the row-sum layer from
-    binary16 rows: one launch, the oracle's bits (activations ~U[0, 6] as in configuration 4)."""
+    binary16 rows: one library call (one launch up to eight rows), the oracle's bits (activations ~U[0, 6] as in
+    configuration 4)."""
     from duqlinear4bitcuda_amd.nn import Linear4bitASQ, Linear4bitASQRowSum, LinearQuant4bitDUASQ
     _say("module decode asym", M, N, K)
     w = _asym_weights(N, K, seed=N + K)
@@ -279,9 +281,9 @@ def test_asym_fp16_input_two_launch_shapes_and_errors(dev):
 @pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (4, 11008, 4096), (8, 512, 2048), (3, 100, 8192), (16, 4096, 4096),
                                     (40, 1000, 1024), (100, 1000, 512)])
 def test_dual_uniform_rowsum_layer_decode(dev, library_calls, M, N, K):
-    """LinearQuant4bitDUASQRowSum from binary16 rows: one launch up to eight rows (quantizer inside the rows
-    kernel), quantizer + GEMM with the epilogue inside for the MFMA decode kernel's shapes, three launches on the
-    ring kernel's; the oracle's bits everywhere, and the op's codes / scales / zero points / row sums."""
+    """LinearQuant4bitDUASQRowSum from binary16 rows: one library call up to 64 rows (one launch up to eight, the
+    quantizer inside the rows kernel; quantizer + GEMM with the epilogue inside for the MFMA decode kernel's shapes;
+    three launches on the ring kernel's), two calls above; the oracle's bits everywhere, and the op's codes / scales / zero points / row sums."""
     from duqlinear4bitcuda_amd import _HIP as hip
     from duqlinear4bitcuda_amd.nn import LinearQuant4bitDUASQRowSum
     _say("dual row-sum decode", M, N, K)
@@ -302,9 +304,9 @@ def test_dual_uniform_rowsum_layer_decode(dev, library_calls, M, N, K):
     layer(X)
     library_calls.clear()
     y = layer(X)
-    if M <= 8:
+    if M <= 64:
         assert library_calls == ["duq_quantize_linear4bit_forward_layer"], library_calls
-    elif M <= 64:
+    else:
         assert library_calls == ["duq_quantize_rows_asym_shifted", "duq_linear4bit_forward_dual_rowsum"], library_calls
     assert cases.bits_equal(y.detach().cpu().numpy(), want)
     layer.fused = False

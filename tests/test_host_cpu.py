@@ -316,15 +316,17 @@ def test_asym_fp16_input_entry_point_validation_without_launch():
     assert s(1, P, 1.0, 6, P, P, None, None, 8, 64, 64, P, None, None, 0, None) == -4
     for code in (-7, -8, -9):
         assert len(lib.duq_status_string(code)) > 10
-    # the prepared-layer form: only one-launch shapes, checked before anything else is touched
+    # the prepared-layer form: a shape of two launches needs its workspace, checked before anything else is touched
     layer = _lib.FusedLayer(0, 1.0, 6, 4096, 4096, P, P, None, None, None, None, None, None)
     g = lib.duq_quantize_linear4bit_forward_layer
-    assert g(ctypes.addressof(layer), P, 9, P, None) == -2 and g(None, P, 1, P, None) == -1
-    assert g(ctypes.addressof(layer), P, 0, P, None) == 0
+    assert g(ctypes.addressof(layer), P, 9, P, None, 0, None) == -1 and g(None, P, 1, P, None, 0, None) == -1
+    assert g(ctypes.addressof(layer), P, 9, P, P, 100, None) == -2
+    assert g(ctypes.addressof(layer), P, 9, P, ctypes.c_void_p(4104), 1 << 20, None) == -5
+    assert g(ctypes.addressof(layer), P, 0, P, None, 0, None) == 0
     layer.mode = 9
-    assert g(ctypes.addressof(layer), P, 1, P, None) == -4
+    assert g(ctypes.addressof(layer), P, 1, P, None, 0, None) == -4
     layer.mode, layer.w_scale_1 = 0, None
-    assert g(ctypes.addressof(layer), P, 1, P, None) == -1
+    assert g(ctypes.addressof(layer), P, 1, P, None, 0, None) == -1
 
 
 def test_deferred_quantized_tensor_host_side():
