@@ -22,6 +22,7 @@ def _stream(t: torch.Tensor):
 
 
 _raw_stream = torch._C._cuda_getCurrentRawStream  # (device index) -> hipStream_t as int; no Stream object built
+_current_device = torch._C._cuda_getDevice
 _F16, _U8 = torch.float16, torch.uint8
 
 
@@ -643,8 +644,9 @@ class FusedDecode:
         """x: contiguous binary16 [..., K] on the layer's device, 16-byte aligned, M = its rows with admits(M);
         clip / qmax: the symmetric quantizer's settings (unused by the asymmetric modes).  ``checked``: the caller
         has verified dtype and contiguity already.  Returns binary16 [..., N]."""
-        if x.get_device() != self.index or x.shape[-1] != self.K or \
-                not (checked or (x.dtype is _F16 and x.is_contiguous())):
+        idx = self.index
+        shape = x.shape
+        if x.get_device() != idx or shape[-1] != self.K or not (checked or (x.dtype is _F16 and x.is_contiguous())):
             raise RuntimeError(f"FusedDecode: expected a contiguous float16 tensor [..., {self.K}] on {self.device}, got "
                                f"{x.dtype} {tuple(x.shape)} on {x.device}")
         nbytes = self._one.get(M)
@@ -652,8 +654,7 @@ class FusedDecode:
             nbytes = self._staging(M)
         if nbytes < 0:
             raise RuntimeError(f"FusedDecode: {M} rows (at most {self.max_rows})")
-        y = torch.empty(x.shape[:-1] + (self.N,), dtype=_F16, device=self.device)
-        idx = self.index
+        y = x.new_empty((*shape[:-1], self.N))
         ref = self._structs.get((clip, qmax))
         layer = ref[0] if ref is not None else self._layer(clip, qmax)
         if nbytes:
@@ -661,7 +662,7 @@ class FusedDecode:
             ws_ptr = ws.data_ptr()
         else:
             ws_ptr = None
-        if idx == torch._C._cuda_getDevice():
+        if idx == _current_device():
             st = self._fn(layer, x.data_ptr(), M, y.data_ptr(), ws_ptr, nbytes, _raw_stream(idx))
         else:
             with torch.cuda.device(idx):

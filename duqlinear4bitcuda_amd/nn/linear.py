@@ -58,11 +58,8 @@ class _Linear4bitBase(torch.nn.Module):
     def _decode_call(self):
         """The layer's prepared one-launch call (``_HIP.FusedDecode``), rebuilt when a buffer was replaced (moved,
         cast, reloaded into a new tensor); None for a layer that has none or is not on a GPU."""
-        spec = self._decode_spec
-        if spec is None:
-            return None
-        b = self._buffers
         d = self._decode
+        b = self._buffers
         if d is not None:
             for name, t in self._decode_held:
                 if b.get(name) is not t:
@@ -70,6 +67,9 @@ class _Linear4bitBase(torch.nn.Module):
             else:
                 if d.w_ptr == self._decode_held[0][1].data_ptr():
                     return d
+        spec = self._decode_spec
+        if spec is None:
+            return None
         names = spec[1] + (("bias", "bias"),)
         held = tuple((buf, b.get(buf)) for _, buf in names)
         if not held[0][1].is_cuda:
@@ -81,14 +81,16 @@ class _Linear4bitBase(torch.nn.Module):
     def _decode_forward(self, x, clip=1.0, qmax=6, checked=False):
         """y for binary16 rows ``x`` when the layer takes them in one library call (up to eight rows: one launch,
         quantizer inside; up to 64: quantizer launch + GEMM launch), else None."""
-        K = self.in_features
-        if not self.fused or x.shape[-1] != K or K % 64:
-            return None
-        M = x.numel() // K
-        if M > _ops.FusedDecode.max_rows or M == 0:
+        if not self.fused:
             return None
         d = self._decode_call()
-        if d is None or not d.admits(M):
+        if d is None:
+            return None
+        K = d.K
+        if K % 64 or x.shape[-1] != K:
+            return None
+        M = x.numel() // K
+        if d._one.get(M, -1) < 0 and not d.admits(M):
             return None
         return d.run(x, M, clip, qmax, checked)
 
