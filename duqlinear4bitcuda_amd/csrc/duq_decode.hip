@@ -30,6 +30,28 @@
 #include "duq_rowquant.h"
 #include "duq_tiles.h"
 
+// Wavefronts per workgroup of the rows kernel when it quantizes its rows itself (binary16 in).  The quantize phase is
+// vector arithmetic (about 27 instructions per eight elements), the same for every workgroup, and sits between the
+// arrival of the activations and the dot products: a wavefront alone on its SIMD issues it at half the rate that
+// two reach together.  Measured (us, N = K = 4096 unless said): two rows 3.25 with four wavefronts, 3.21 with eight;
+// three / four rows 4.11 / 4.17 with four, 3.67 / 3.68 with eight (and with sixteen); four rows of 8192 / 11008
+// elements 7.5 / 8.9 with four, 6.5 / 7.1 with sixteen; eight rows 5.0 with eight, 5.1 with sixteen, of 8192
+// elements 9.1 with eight, 8.7 with sixteen.
+#ifndef DUQ_DEC_FUSEQ_WAVES
+#define DUQ_DEC_FUSEQ_WAVES 8     // eight rows; and several tiles per workgroup
+#endif
+#ifndef DUQ_DEC_FUSEQ_WAVES_M4
+#define DUQ_DEC_FUSEQ_WAVES_M4 8  // three or four rows of up to 4096 elements
+#endif
+#ifndef DUQ_DEC_FUSEQ_WAVES_M4L
+#define DUQ_DEC_FUSEQ_WAVES_M4L 16  // of more
+#endif
+#ifndef DUQ_DEC_FUSEQ_WAVES_M8L
+#define DUQ_DEC_FUSEQ_WAVES_M8L 16  // eight rows of more than 4096 elements
+#endif
+#ifndef DUQ_DEC_FUSEQ_WAVES_M2
+#define DUQ_DEC_FUSEQ_WAVES_M2 4
+#endif
 #ifndef DUQ_DEC_R
 #define DUQ_DEC_R 4
 #endif
@@ -147,8 +169,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DUQ_HEAD_DECL,
     constexpr int LPV = 64 / V;      // lanes that finish one sum: 16, 8 or 4
     constexpr int MODE = EPI < 0 ? 0 : EPI;
     constexpr uint32_t XSTRIDE = XS * 1024;
-    static_assert(MR == 1 || MR == 2 || MR == 4 || (MR == 8 && WAVES == 8), "rows");
-    static_assert(WAVES == 4 || WAVES == 8, "wavefronts per workgroup");
+    static_assert(MR == 1 || MR == 2 || MR == 4 || (MR == 8 && WAVES >= 8), "rows");
+    static_assert(WAVES == 4 || WAVES == 8 || WAVES == 16, "wavefronts per workgroup");
     static_assert(V >= 4 && V <= 16 && (XS * MR * 4) % WAVES == 0, "partial sums per lane, quantize units per lane");
     __shared__ __attribute__((aligned(16))) int red[WAVES][V * 64];
     __shared__ __attribute__((aligned(16))) uint8_t xs[FUSEQ ? MR * XSTRIDE : 16];
@@ -203,7 +225,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DUQ_HEAD_DECL,
     // serves requests in order, and a wavefront whose activations queue behind another's weights holds up the
     // whole workgroup at the staging barrier below; measured at 8 rows, K = 4096: N = 4096 5.6 against 6.2 us,
     // N = 11008 8.2 against 8.5; with four wavefronts it changes nothing)
-    if (FUSEQ && WAVES == 8) __builtin_amdgcn_s_barrier();
+    if (FUSEQ && WAVES >= 8) __builtin_amdgcn_s_barrier();
     const __amdgpu_buffer_rsrc_t rW = make_rsrc(p.B, p.N * kbytes);
     // the weights of tile t for this wavefront (tiles past the workgroup's last read as zero, unused)
     auto load_w = [&](uint32_t tile, v4u(&w)[R][XS]) {
@@ -575,33 +597,29 @@ bool launch_rows_mode(DecodeParams &p, int epi, hipStream_t stream)
     // One tile per workgroup.  Four rows quantized in the kernel, more than 256 tiles: every workgroup quantizes
     // the rows again, so one round of at most 256 workgroups of eight wavefronts with several tiles each when two
     // register sets of weights fit (rows of at most 8192 elements; measured at K = 4096: N = 6144 5.76 against
-    // 6.21 us, N = 11008 7.18 against 7.73), else eight wavefronts and one tile (N = 11008: 7.9 against 8.3 us with
-    // four; with one workgroup per CU the vector work per SIMD is the same and four wavefronts are ahead,
-    // N = 4096: 4.8 against 5.1 us).  On pre-quantized rows, or with one or two rows, several tiles per workgroup
-    // measured 3-15 % slower than one (four wavefronts per CU keep too few loads in flight): not used there.
-    // Eight rows (binary16 in only): always eight wavefronts, one per row in the quantize phase.
+    // 6.21 us, N = 11008 7.18 against 7.73).  On pre-quantized rows, or with one or two rows, several tiles per
+    // workgroup measured 3-15 % slower than one (four wavefronts per CU keep too few loads in flight): not used
+    // there.
     constexpr bool kCanMulti = FUSEQ && MR >= 4 && XS <= (MR == 4 ? 4 : 2);
     const bool multi = kCanMulti && ntiles > 256;
     p.tiles_per_wg = multi ? (ntiles + 255) / 256 : 1;
     const dim3 grid((ntiles + p.tiles_per_wg - 1) / p.tiles_per_wg);
-    const bool wide = MR == 8 || (FUSEQ && MR == 4 && !multi && grid.x > 256);
+    // wavefronts per workgroup: four, or with three or more rows to quantize WQ (DUQ_DEC_FUSEQ_WAVES above)
+    constexpr int WQ = !FUSEQ || MR == 1 ? 4
+                       : MR == 2         ? DUQ_DEC_FUSEQ_WAVES_M2
+                       : MR == 8         ? (XS >= 4 ? DUQ_DEC_FUSEQ_WAVES_M8L : DUQ_DEC_FUSEQ_WAVES)
+                                         : (XS >= 4 ? DUQ_DEC_FUSEQ_WAVES_M4L : DUQ_DEC_FUSEQ_WAVES_M4);
+    constexpr int WMULTI = DUQ_DEC_FUSEQ_WAVES;
     bool launched = false;
 #define DUQ_ROWS(E)                                                                                              \
     if (multi) {                                                                                                 \
         if constexpr (kCanMulti) {                                                                               \
-            DUQ_LAUNCH_HEAD((gemv_s4_rows_kernel<MR, XS, FUSEQ, E, 8, true>), grid, dim3(512), 0, stream, p);         \
-            launched = true;                                                                                     \
-        }                                                                                                        \
-    } else if (wide) {                                                                                           \
-        if constexpr (FUSEQ && MR >= 4) {                                                                        \
-            DUQ_LAUNCH_HEAD((gemv_s4_rows_kernel<MR, XS, FUSEQ, E, 8>), grid, dim3(512), 0, stream, p);               \
+            DUQ_LAUNCH_HEAD((gemv_s4_rows_kernel<MR, XS, FUSEQ, E, WMULTI, true>), grid, dim3(WMULTI * 64), 0, stream, p); \
             launched = true;                                                                                     \
         }                                                                                                        \
     } else {                                                                                                     \
-        if constexpr (MR <= 4) {                                                                                 \
-            DUQ_LAUNCH_HEAD((gemv_s4_rows_kernel<MR, XS, FUSEQ, E, 4>), grid, dim3(256), 0, stream, p);               \
-            launched = true;                                                                                     \
-        }                                                                                                        \
+        DUQ_LAUNCH_HEAD((gemv_s4_rows_kernel<MR, XS, FUSEQ, E, WQ>), grid, dim3(WQ * 64), 0, stream, p);              \
+        launched = true;                                                                                         \
     }
     switch (epi) {
     case 0: DUQ_ROWS(0) break;
