@@ -541,7 +541,13 @@ def int8_layer_section(dev, quick=False):
         us_rowmajor = graph_time_us([lambda: _HIP.linear8bit_forward(p.quantized_x, p.scales_x, p.zeros_x, layer.weight,
                                                                      layer.weight_scales, layer.weight_zeros)] * 10)
         us_quant = graph_time_us([lambda: layer.quantizer(x)] * 10)
-        out.append({"M": M, "K": K, "N": N, "step_us": round(us_step, 2), "step_TOPS": round(ops / us_step / 1e6, 1),
+        eager = {}
+        if M <= 256:  # a step of a few rows is bound by the host: one library call (the default) against two
+            eager["module_eager_us"] = round(eager_wall_us([layer], x), 2)
+            layer.one_call_rows = 0
+            eager["module_eager_two_calls_us"] = round(eager_wall_us([layer], x), 2)
+            layer.one_call_rows = 256
+        out.append({"M": M, "K": K, "N": N, "step_us": round(us_step, 2), "step_TOPS": round(ops / us_step / 1e6, 1), **eager,
                     "three_step_us": round(us3, 2), "fused_equals_three_steps": same,
                     "quantize_us": round(us_quant, 2),
                     "quantize_GBps": round((M * K * 5 + M * 8) / us_quant / 1e3, 1),

@@ -1111,3 +1111,43 @@ def linear8bit_forward(xq, scale_x, zeros_x, w, w_scale, w_zeros, bias=None, til
     if st:
         _lib.check(st, name)
     return y
+
+
+def quantize_linear8bit_forward(x, w, w_tiled, w_scale, w_zeros, bias=None):
+    """AsymQuantizer8bit + linear8bit_forward in one library call (two launches, the codes staged in a workspace
+    allocated here): x float32 [..., K] -> float32 [..., N], the bits of the two calls.  ``w`` the weight [N, K]
+    int8, ``w_tiled`` its tiled copy from weight_tile_8bit or None."""
+    name = "quantize_linear8bit_forward"
+    if not isinstance(x, torch.Tensor) or not isinstance(w, torch.Tensor):
+        raise RuntimeError(f"{name}: x and w must be tensors")
+    dev = x.device
+    _fast_check(name, "x", x, _F32, None)
+    _fast_check(name, "w", w, _I8, dev)
+    K = x.shape[-1]
+    M = x.numel() // K if K else 0
+    if w.dim() != 2 or w.size(1) != K:
+        raise RuntimeError(f"{name}: K differs: x {tuple(x.shape)} vs w {tuple(w.shape)}")
+    N = w.size(0)
+    if w_tiled is not None:
+        _fast_check(name, "w_tiled", w_tiled, _I8, dev)
+        if w_tiled.numel() != (N + 31) // 32 * 32 * K:
+            raise RuntimeError(f"{name}: the tiled weight has {w_tiled.numel()} bytes, expected {(N + 31) // 32 * 32 * K}")
+    for t, what in ((w_scale, "w_scale"), (w_zeros, "w_zeros"), (bias, "bias")):
+        if t is None and what == "bias":
+            continue
+        if not isinstance(t, torch.Tensor):
+            raise RuntimeError(f"{name}: {what} is not a tensor")
+        _fast_check(name, what, t, _F32, dev)
+        if t.numel() != N:
+            raise RuntimeError(f"{name}: expected {what} to have {N} elements, got {tuple(t.shape)}")
+    lib = _lib.load()
+    y = x.new_empty((*x.shape[:-1], N))
+    if M == 0 or N == 0:
+        return y
+    nbytes = lib.duq_quantize_linear8bit_workspace_bytes(M, K)
+    ws = torch.empty(nbytes, dtype=_U8, device=dev)
+    st = _launch(dev, lib.duq_quantize_linear8bit_forward, x.data_ptr(), w.data_ptr(), _ptr(w_tiled), w_scale.data_ptr(),
+                 w_zeros.data_ptr(), _ptr(bias), M, N, K, y.data_ptr(), ws.data_ptr(), nbytes)
+    if st:
+        _lib.check(st, name)
+    return y

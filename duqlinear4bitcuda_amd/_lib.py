@@ -46,6 +46,9 @@ PROTOTYPES = {
     "duq_quantize_linear4bit_forward_static": [_c_i32, _c_p, ctypes.c_float, _c_i32, _c_p, _c_p, _c_p, _c_p, _c_u32,
                                                _c_u32, _c_u32, _c_p, _c_p, _c_p, _c_u32, _c_p],
     "duq_static_scratch_init": [],
+    "duq_quantize_linear8bit_workspace_bytes": [_c_u32, _c_u32],  # returns uint64_t
+    "duq_quantize_linear8bit_forward": [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_u32, _c_u32, _c_u32, _c_p, _c_p,
+                                        ctypes.c_uint64, _c_p],
     "duq_quantize_linear4bit_forward_layer": [_c_p, _c_p, _c_u32, _c_p, _c_p, ctypes.c_uint64, _c_p],
     "duq_quantize_linear4bit_asym_workspace_bytes": [_c_i32, _c_u32, _c_u32, _c_u32],  # returns uint64_t
     "duq_quantize_linear4bit_forward_asym": [_c_i32, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_u32, _c_u32,
@@ -109,6 +112,7 @@ def load():
     lib.duq_quantize_linear4bit_workspace_bytes.restype = ctypes.c_uint64
     lib.duq_linear4bit_dual_rowsum_workspace_bytes.restype = ctypes.c_uint64
     lib.duq_quantize_linear4bit_asym_workspace_bytes.restype = ctypes.c_uint64
+    lib.duq_quantize_linear8bit_workspace_bytes.restype = ctypes.c_uint64
     lib.duq_status_string.argtypes = [ctypes.c_int]
     lib.duq_status_string.restype = ctypes.c_char_p
     _lib = lib

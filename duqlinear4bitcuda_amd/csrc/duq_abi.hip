@@ -766,4 +766,32 @@ int duq_linear8bit_forward_tiled(const int8_t *xq, const float *scale_x, const f
                                as_stream(stream));
 }
 
+uint64_t duq_quantize_linear8bit_workspace_bytes(uint32_t M, uint32_t K)
+{
+    return up16((uint64_t)M * K) + 2 * up16((uint64_t)M * 4);
+}
+
+int duq_quantize_linear8bit_forward(const float *x, const int8_t *w, const int8_t *w_tiled, const float *w_scale,
+                                    const float *w_zeros, const float *bias, uint32_t M, uint32_t N, uint32_t K, float *y,
+                                    void *workspace, uint64_t workspace_bytes, duq_stream_t stream)
+{
+    if (M == 0 || N == 0) return DUQ_OK;
+    if (!x || (!w && !w_tiled) || !workspace) return DUQ_E_NULL;
+    if (!aligned(x, 16) || !aligned(workspace, 16)) return DUQ_E_ALIGN;
+    if (workspace_bytes < duq_quantize_linear8bit_workspace_bytes(M, K)) return DUQ_E_SHAPE;
+    // few rows run the kernel that reads the weight as stored, the others the tiled copy when there is one
+    const bool rows_kernel = w && M <= 4 && K <= (M <= 2 ? 8192u : 4096u);
+    const bool tiled = w_tiled && !rows_kernel;
+    const int8_t *weight = tiled ? w_tiled : w;
+    if (!weight) return DUQ_E_NULL;
+    int8_t *q = static_cast<int8_t *>(workspace);
+    float *sx = reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + up16((uint64_t)M * K));
+    float *zx = reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(sx) + up16((uint64_t)M * 4));
+    if (int e = check_gemm8(q, weight, M, N, K)) return e;
+    if (!w_scale || !w_zeros || !y) return DUQ_E_NULL;
+    if (!aligned(y, 4)) return DUQ_E_ALIGN;
+    if (int e = duq::launch_quantize_rows_asym8(x, M, K, q, sx, zx, as_stream(stream))) return e;
+    return duq::launch_gemm_s8(q, weight, tiled, M, N, K, nullptr, sx, zx, w_scale, w_zeros, bias, y, as_stream(stream));
+}
+
 }  // extern "C"

@@ -558,8 +558,18 @@ class LinearQuant8bitASQ(torch.nn.Module):
         if require_quantizer:
             self.quantizer = AsymQuantizer8bit()
 
+    # rows up to which the layer's own quantizer and the GEMM go through one library call (a step of a few rows
+    # costs more on the host than on the GPU; larger inputs hide the second call behind the first launch)
+    one_call_rows = 256
+
     def forward(self, x):
         if self.require_quantizer:
+            if self.fused and type(x) is torch.Tensor and x.dtype is torch.float32 and x.is_cuda and x.is_contiguous() \
+                    and x.shape[-1] == self.in_features and self.in_features % 32 == 0 and x.data_ptr() % 16 == 0 \
+                    and 0 < x.numel() <= self.one_call_rows * self.in_features and type(self.quantizer) is AsymQuantizer8bit \
+                    and self.quantizer.fused:
+                return _ops.quantize_linear8bit_forward(x, self.weight, self._tiled_weight() if self.tiled else None,
+                                                        self.weight_scales, self.weight_zeros, self.bias)
             x = self.quantizer(x)
         assert type(x) == tensor_utils.PackedQuantizedTensor, \
             "Input should be quantized tensor, or require_quantizer should be passed as initial argument"

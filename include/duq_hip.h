@@ -473,6 +473,18 @@ int duq_linear8bit_forward_tiled(const int8_t *xq, const float *scale_x, const f
                                  const float *w_scale, const float *w_zeros, const float *bias, uint32_t M, uint32_t N,
                                  uint32_t K, float *y, duq_stream_t stream);
 
+/* No counterpart in the reference: LinearQuant8bitASQ.forward with its own quantizer (qlinear4bit/nn/linear.py:323-335)
+ * in one call: duq_quantize_rows_asym_8bit into `workspace`, then duq_linear8bit_forward(_tiled) on it; the same
+ * bits as the two calls.  x [M,K] float32, 16-byte aligned, K % 32 == 0; w the weight as stored and / or w_tiled its
+ * tiled copy (one may be NULL): up to four rows (two of more than 4096 elements) read w when it is given, everything
+ * else w_tiled when it is given.  workspace: duq_quantize_linear8bit_workspace_bytes(M, K) bytes (codes, scales,
+ * zero points), 16-byte aligned.  What a step of the layer costs at a few rows is mostly the host's share of a
+ * call; this halves it. */
+uint64_t duq_quantize_linear8bit_workspace_bytes(uint32_t M, uint32_t K);
+int duq_quantize_linear8bit_forward(const float *x, const int8_t *w, const int8_t *w_tiled, const float *w_scale,
+                                    const float *w_zeros, const float *bias, uint32_t M, uint32_t N, uint32_t K, float *y,
+                                    void *workspace, uint64_t workspace_bytes, duq_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

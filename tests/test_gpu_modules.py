@@ -407,6 +407,36 @@ def _bits(t):
 
 
 @pytest.mark.gpu
+def test_enable_fp6_over_a_model(qnn, dev, monkeypatch):
+    """nn.enable_fp6(model): every 4-bit layer it can take gets its weight shadow, every quantizer writes the
+    activation shadow, the model's output keeps its bits and the large input runs the 6-bit float entry point."""
+    from duqlinear4bitcuda_amd import _lib
+    torch.manual_seed(11)
+    K, N = 512, 1024
+    lin = torch.nn.Linear(K, N, bias=True).half().to(dev)
+    sw = (lin.weight.abs().amax(dim=1, keepdim=True) / 7).half()
+    odd = torch.nn.Linear(K, 40, bias=False).half().to(dev)   # 40 columns: not a shape the path takes
+    model = torch.nn.ModuleList([
+        torch.nn.Sequential(qnn.SymQuantizer(1.0), qnn.Linear4bitSQ.from_float(lin, sw).to(dev)),
+        qnn.Linear4bitASQ.from_linear(lin).to(dev),
+        torch.nn.Sequential(qnn.SymQuantizer(1.0), qnn.Linear4bitSQ.from_float(odd, (odd.weight.abs().amax(dim=1, keepdim=True) / 7).half()).to(dev)),
+    ])
+    x = torch.randn(600, K, device=dev).half()
+    want = [m(x) for m in model]
+    assert qnn.enable_fp6(model) == 2
+    assert model[0][0].shadow is True and model[2][0].shadow is True
+    lib = _lib.load()
+    calls = []
+    real = lib.duq_linear4bit_forward_bf6
+    monkeypatch.setattr(lib, "duq_linear4bit_forward_bf6", lambda *a: (calls.append(1), real(*a))[1], raising=False)
+    got = [m(x) for m in model]
+    assert len(calls) == 2
+    for g, w in zip(got, want):
+        assert torch.equal(_bits(g), _bits(w))
+    assert qnn.enable_fp6(torch.nn.Sequential(qnn.SymQuantizer(1.0)), "only") == 0
+
+
+@pytest.mark.gpu
 def test_fp6_matrix_path_in_the_layers(qnn, dev):
     """enable_fp6(): every layer class gives the same bits through the 6-bit float matrix path as through the
     integer kernels; the shadow stays out of the state_dict and follows the weights."""

@@ -268,6 +268,17 @@ def test_abi_validation_8bit_entries():
     assert lib.duq_quantize_rows_asym_8bit(P, 2, 6, P, P, P, None) == -2      # cols % 4
     assert lib.duq_quantize_rows_asym_8bit(P + 4, 2, 8, P, P, P, None) == -5
     assert lib.duq_quantize_rows_asym_8bit(P, 2, 8, None, P, P, None) == -1
+    # quantizer + forward in one call
+    ql = lib.duq_quantize_linear8bit_forward
+    nb = lib.duq_quantize_linear8bit_workspace_bytes
+    assert nb(4, 32) == 128 + 16 + 16 and nb(5, 4096) == 5 * 4096 + 32 + 32
+    assert ql(P, P, None, P, P, None, 4, 8, 40, P, P, 1024, None) == -3          # K % 32
+    assert ql(P, None, None, P, P, None, 4, 8, 32, P, P, 1024, None) == -1       # no weight at all
+    assert ql(P, P, None, P, P, None, 4, 8, 32, P, None, 0, None) == -1          # no workspace
+    assert ql(P, P, None, P, P, None, 4, 8, 32, P, P, 100, None) == -2           # too small
+    assert ql(P + 4, P, None, P, P, None, 4, 8, 32, P, P, 1024, None) == -5
+    assert ql(P, P, None, None, P, None, 4, 8, 32, P, P, 1024, None) == -1
+    assert ql(None, None, None, None, None, None, 0, 8, 32, None, None, 0, None) == 0
 
 
 def test_python_ops_reject_bad_arguments():
@@ -504,6 +515,42 @@ def test_gpu_layer_8bit(dev):
     # wrappers keep leading dimensions
     p = AsymQuantizer8bit()(xt)
     assert tuple(tensor_utils.matmul_8bit(p.quantized_x, layer.weight).shape) == (2, 37, N)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows", [1, 4, 5, 16, 74, 256, 300])
+def test_gpu_layer_8bit_one_call(dev, monkeypatch, rows):
+    """LinearQuant8bitASQ with its own quantizer: up to 256 rows quantizer + GEMM are one library call, the bits of
+    the oracle and of the two calls; above, two calls."""
+    import torch
+    from duqlinear4bitcuda_amd import _lib
+    from duqlinear4bitcuda_amd.nn import LinearQuant8bitASQ
+    print("8-bit layer, one call", rows, flush=True)
+    rng = np.random.default_rng(rows)
+    K, N = 1024, 320
+    lin = torch.nn.Linear(K, N, bias=True)
+    with torch.no_grad():
+        lin.weight.copy_(torch.from_numpy((rng.standard_normal((N, K)) * 0.03).astype(F32)))
+        lin.bias.copy_(torch.from_numpy(rng.standard_normal(N).astype(F32)))
+    layer = LinearQuant8bitASQ.from_linear(lin).to(dev)
+    wq, ws, wz = orc.weight_asym8_from_linear(lin.weight.detach().numpy())
+    x = _acts(rng, rows, K)
+    want = orc.linear8bit_asq_forward(x, wq, ws, wz, lin.bias.detach().numpy())[0]
+    xt = _t(x, dev)
+    layer(xt)
+    lib = _lib.load()
+    calls = []
+    for name in ("duq_quantize_linear8bit_forward", "duq_quantize_rows_asym_8bit", "duq_linear8bit_forward",
+                 "duq_linear8bit_forward_tiled"):
+        real = getattr(lib, name)
+        monkeypatch.setattr(lib, name, (lambda *a, _r=real, _n=name: (calls.append(_n), _r(*a))[1]), raising=False)
+    y = layer(xt)
+    tiled_fwd = "duq_linear8bit_forward" if rows <= 4 else "duq_linear8bit_forward_tiled"
+    assert calls == (["duq_quantize_linear8bit_forward"] if rows <= 256 else ["duq_quantize_rows_asym_8bit", tiled_fwd]), calls
+    assert np.array_equal(y.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    for tiled, one_call in ((False, 256), (True, 0)):
+        layer.tiled, layer.one_call_rows = tiled, one_call
+        assert torch.equal(layer(xt), y), (tiled, one_call)
 
 
 @pytest.mark.gpu
