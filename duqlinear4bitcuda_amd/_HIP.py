@@ -422,6 +422,12 @@ def batch_linear4bit_forward(mode, xq, scale_x, zeros_x, w, w_scale_1, w_zeros_1
     return y
 
 
+def gemm_stream_tile_for(M: int, N: int, K: int) -> int:
+    """Tile of the stream kernel for a shape (rows * 1000 + columns), 0 for shapes other kernels run; see
+    ``duq_gemm_stream_tile_for`` in include/duq_hip.h."""
+    return _lib.load().duq_gemm_stream_tile_for(M, N, K)
+
+
 def gemm_kernel_for(M: int, N: int, K: int) -> int:
     """Which kernel family the int4 GEMM runs for a shape (host arithmetic, no GPU work): see
     ``duq_gemm_kernel_for`` in include/duq_hip.h."""

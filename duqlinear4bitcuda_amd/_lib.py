@@ -39,6 +39,7 @@ PROTOTYPES = {
     "duq_linear4bit_forward": [_c_i32, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_u32, _c_u32,
                                _c_u32, _c_p, _c_p],
     "duq_gemm_kernel_for": [_c_u32, _c_u32, _c_u32],
+    "duq_gemm_stream_tile_for": [_c_u32, _c_u32, _c_u32],
     "duq_probe_read": [_c_p, ctypes.c_uint64, _c_p, _c_p],
     "duq_quantize_linear4bit_workspace_bytes": [_c_u32, _c_u32, _c_u32],  # returns uint64_t (restype set in load())
     "duq_quantize_linear4bit_forward": [_c_i32, _c_p, ctypes.c_float, _c_i32, _c_p, _c_p, _c_p, _c_p, _c_u32, _c_u32,

@@ -420,6 +420,13 @@ int duq_probe_read(const void *src, uint64_t bytes, uint32_t *sink, duq_stream_t
 
 int duq_gemm_kernel_for(uint32_t M, uint32_t N, uint32_t K) { return duq::select_gemm_kernel(M, N, K); }
 
+int duq_gemm_stream_tile_for(uint32_t M, uint32_t N, uint32_t K)
+{
+    if (duq::select_gemm_kernel(M, N, K) != duq::kKernelStream) return 0;
+    const duq::StreamTile t = duq::select_stream_tile(M, N, K, 1, false);
+    return (int)(t.rows * 1000 + t.cols);
+}
+
 uint64_t duq_quantize_linear4bit_workspace_bytes(uint32_t M, uint32_t N, uint32_t K)
 {
     if (M == 0 || N == 0 || K == 0) return 0;

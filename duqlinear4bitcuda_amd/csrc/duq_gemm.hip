@@ -518,6 +518,192 @@ __global__ __launch_bounds__(256) void gemm_s4_stream_kernel(DUQ_HEAD_DECL, Gemm
 }
 
 // ---------------------------------------------------------------------------------
+// stream kernel, 256-row tiles: problems with at least one 256 x 256 tile per CU
+// ---------------------------------------------------------------------------------
+// The stream kernel's schedule with twice the activation rows per workgroup: the weight bytes a wavefront fetches
+// and expands (the loop's main side work: two vector instructions per packed word) meet eight activation tiles
+// instead of four, and a tile's prologue and epilogue are paid once per 65536 outputs instead of twice.  All 256
+// accumulation registers hold accumulators (2 weight tiles x 8 activation tiles x 16), so the epilogue parameters
+// are fetched after the loop, and a chunk is 128 k (three LDS buffers of 256 rows x 144 bytes; the epilogue's staging
+// area, 4 x 256 x 144 bytes, is what sizes the array).  A chunk is four steps (piece, nibble parity) of sixteen
+// MFMAs; per step: slots 0-7 read the next step's eight activation fragments, 8-9 refetch the weight piece just
+// consumed (even steps), 10-13 expand one weight piece of one tile, 8, 9, 14, 15 expand one activation piece (stored
+// in slot 15), and the activations ride two chunks of registers deep: a chunk's packed activations are requested a
+// whole chunk before they are expanded into the buffer that is read two chunks later.
+constexpr int kCK2 = 128;        // k elements per chunk
+constexpr int kXStride2 = 144;   // LDS bytes per activation row: 128 expanded + 16 pad
+
+template <int EPI, bool BIAS>
+__global__ __launch_bounds__(256) void gemm_s4_stream256_kernel(DUQ_HEAD_DECL, GemmParams tail)
+{
+    GemmParams p = with_head(tail, DUQ_HEAD_USE);
+    to_global(p.A);
+    to_global(p.B);
+    to_global(p.C);
+    to_global(p.y);
+    static_assert(EPI != 5, "the dual-uniform row-sum epilogue stages its parameters in LDS: stream kernel");
+    constexpr int TM = 8, TN = 2, BM = 256, BN = 256, S = TM * TN, NXP = 4;
+    constexpr uint32_t kBuf = BM * kXStride2;
+    constexpr uint32_t kLds = 4 * BM * 144 > 3 * kBuf ? 4 * BM * 144 : 3 * kBuf;
+    __shared__ __attribute__((aligned(16))) uint8_t lds[kLds];
+    uint32_t *const dpar = nullptr;  // named by the shared epilogue text for an epilogue this kernel never runs
+    const uint32_t dwide = 0;
+
+    if (blockIdx.z) batch_shift(p, blockIdx.z);
+    uint32_t tile_m, tile_n;
+    tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+    const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u, wave = tid >> 6;
+    const uint32_t l32 = lane & 31u, h = lane >> 5;
+    const uint32_t kbytes = p.K >> 1;
+    const uint32_t nchunks = (p.K + kCK2 - 1) / kCK2;
+
+    const __amdgpu_buffer_rsrc_t rW = make_rsrc(p.B + (uint64_t)n0 * kbytes, min(p.N - n0, (uint32_t)BN) * kbytes);
+    const __amdgpu_buffer_rsrc_t rX = make_rsrc(p.A + (uint64_t)m0 * kbytes, min(p.M - m0, (uint32_t)BM) * kbytes);
+
+    // weights: lane (l32, h) of tile t holds piece i = bytes [i*32 + h*16, +16) of the chunk's 64-byte row segment
+    uint32_t woff[TN];
+#pragma unroll
+    for (int t = 0; t < TN; ++t) woff[t] = (wave * (32 * TN) + t * 32 + l32) * kbytes + h * 16;
+    // activations: thread -> 16-byte piece xq of the segment of row xrow + 64 * i.  The sixteen lanes that an LDS
+    // write instruction serves together hold rows r, r + 1, r + 8, r + 9 (r even): with 144-byte rows their four
+    // pieces each land in sixteen different 16-byte columns of the banks (rows r .. r + 3 would collide in pairs)
+    uint32_t xoff[NXP], xlds[NXP];
+    const uint32_t xq = tid & 3u;
+    const uint32_t xrow = ((tid >> 2) & 1u) + 8u * ((tid >> 3) & 1u) + 2u * ((tid >> 4) & 3u) + 16u * (tid >> 6);
+#pragma unroll
+    for (int i = 0; i < NXP; ++i) {
+        const uint32_t row = xrow + i * 64;
+        xoff[i] = row * kbytes + xq * 16;
+        xlds[i] = row * kXStride2 + xq * 32;
+    }
+    // K % 64 == 0: a 16-byte piece is all inside the row or all outside (then redirected out of range: zero)
+    auto load_w = [&](int t, int i, uint32_t koff) {
+        return buf_load16(rW, koff + i * 32 + h * 16 < kbytes ? woff[t] + i * 32 : kOobOffset, koff);
+    };
+    auto load_x = [&](int j, uint32_t koff) {
+        return buf_load16(rX, koff + xq * 16 < kbytes ? xoff[j] : kOobOffset, koff);
+    };
+
+    v4u wreg[TN][2];      // raw weight pieces [tile][piece]
+    v4u xr[2][NXP];       // raw activation pieces, two chunks of them
+    v4u wexp[2][2][TN];   // expanded weights [piece][parity][tile]
+    v4i fx[2][TM];        // activation fragments [step & 1][tile]
+    v16i acc[TN][TM];
+#pragma unroll
+    for (int t = 0; t < TN; ++t)
+#pragma unroll
+        for (int b = 0; b < TM; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[t][b][r] = 0;
+
+    // fragment of step (i, par) for activation tile b: + b*32*kXStride2 + i*64 + par*16
+    const uint32_t fragX = l32 * kXStride2 + h * 32;
+    auto expand_word = [&](const v4u &raw, v4u &even, v4u &odd, int w) {
+        even[w] = (raw[w] << 4) & kNibbleMask;
+        odd[w] = raw[w] & kNibbleMask;
+    };
+
+    // chunk c; PAR = c & 1: xr[PAR] holds the packed activations of chunk c + 2, xr[PAR ^ 1] receives those of c + 3
+    auto body = [&](auto parity, uint32_t c, uint32_t cur, uint32_t nxt, uint32_t nx2) {
+        constexpr int PAR = decltype(parity)::value;
+        const uint32_t koff1 = (c + 1) * (kCK2 / 2), koff3 = (c + 3) * (kCK2 / 2);
+        v4u xe, xo;
+#pragma unroll
+        for (int step = 0; step < 4; ++step) {
+            const int i = step >> 1, par = step & 1;
+#pragma unroll
+            for (int slot = 0; slot < S; ++slot) {
+                const int b = slot / TN, t = slot % TN;
+                asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0"
+                             : "+a"(acc[t][b])
+                             : "v"(wexp[i][par][t]), "v"(fx[step & 1][b]));
+                __builtin_amdgcn_sched_barrier(0);
+                // ---- side work in the shadow of this MFMA
+                if (slot < TM) {  // next step's activation fragment for tile `slot`
+                    const uint8_t *src = step < 3 ? lds + cur + fragX + ((step + 1) >> 1) * 64 + ((step + 1) & 1) * 16
+                                                  : lds + nxt + fragX;
+                    fx[(step + 1) & 1][slot] = *reinterpret_cast<const v4i *>(src + slot * 32 * kXStride2);
+                }
+                if (par == 0 && slot >= 8 && slot < 8 + TN)  // piece i was expanded earlier: refetch it for the next chunk
+                    wreg[slot - 8][i] = load_w(slot - 8, i, koff1);
+                if (slot >= 10 && slot < 14)  // the next piece (this chunk's second, then the next chunk's first) of tile `par`
+                    expand_word(wreg[par][(i + 1) & 1], wexp[(i + 1) & 1][0][par], wexp[(i + 1) & 1][1][par], slot - 10);
+                if (step == 0 && slot >= 12) xr[PAR ^ 1][slot - 12] = load_x(slot - 12, koff3);
+                // chunk c + 2 -> third LDS buffer: piece `step`, its four words in the slots without a fragment read
+                // or a weight word, then both halves stored
+                if (slot == 8 || slot == 9 || slot == 14 || slot == 15) {
+                    const int w = slot < 10 ? slot - 8 : slot - 12;
+                    expand_word(xr[PAR][step], xe, xo, w);
+                    if (w == 3) {
+                        *reinterpret_cast<v4u *>(lds + nx2 + xlds[step]) = xe;
+                        *reinterpret_cast<v4u *>(lds + nx2 + xlds[step] + 16) = xo;
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        __syncthreads();
+    };
+
+    // ---- prologue: chunks 0 and 1 activations -> LDS, chunk 2 -> registers, chunk 0 weights -> registers
+    {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int t = 0; t < TN; ++t) wreg[t][i] = load_w(t, i, 0);
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+#pragma unroll
+            for (int j = 0; j < NXP; ++j) xr[q][j] = load_x(j, q * (kCK2 / 2));
+        }
+#pragma unroll
+        for (int q = 0; q < 2; ++q)
+#pragma unroll
+            for (int j = 0; j < NXP; ++j) {
+                v4u ev, od;
+                expand_nibbles(xr[q][j], ev, od);
+                *reinterpret_cast<v4u *>(lds + q * kBuf + xlds[j]) = ev;
+                *reinterpret_cast<v4u *>(lds + q * kBuf + xlds[j] + 16) = od;
+            }
+#pragma unroll
+        for (int j = 0; j < NXP; ++j) xr[0][j] = load_x(j, 2 * (kCK2 / 2));
+#pragma unroll
+        for (int t = 0; t < TN; ++t) expand_nibbles(wreg[t][0], wexp[0][0][t], wexp[0][1][t]);
+        __syncthreads();
+#pragma unroll
+        for (int b = 0; b < TM; ++b) fx[0][b] = *reinterpret_cast<const v4i *>(lds + fragX + b * 32 * kXStride2);
+    }
+
+    uint32_t cur = 0, nxt = kBuf, nx2 = 2 * kBuf;
+    auto rotate = [&]() {
+        const uint32_t t = cur;
+        cur = nxt;
+        nxt = nx2;
+        nx2 = t;
+    };
+    using P0 = std::integral_constant<int, 0>;
+    using P1 = std::integral_constant<int, 1>;
+    uint32_t c = 0;
+    for (; c + 1 < nchunks; c += 2) {
+        body(P0{}, c, cur, nxt, nx2);
+        rotate();
+        body(P1{}, c + 1, cur, nxt, nx2);
+        rotate();
+    }
+    if (c < nchunks) body(P0{}, c, cur, nxt, nx2);
+    // the MFMAs above are opaque to the compiler's hazard tracking: let the last ones retire
+    // before the accumulators are read
+    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+
+    // ---- epilogue parameters (after the loop: no registers to spare inside it), then the epilogue
+#include "duq_stream_epilogue_fetch.inc"
+    constexpr bool kWideStore = false;
+#include "duq_stream_epilogue_store.inc"
+}
+
+// ---------------------------------------------------------------------------------
 // short-row kernel: K <= 256 (one chunk), many tiles; batched products of short rows
 // ---------------------------------------------------------------------------------
 // The stream kernel's tile (32*TM rows x 256 columns, four wavefronts side by side along N, weights global ->
@@ -1094,32 +1280,24 @@ static void launch_epi(GemmParams &p, hipStream_t stream, uint32_t batch = 1)
         return;
     }
     }
-    // Stream kernel with 128, 64 or 32 activation rows x 256 columns per workgroup, or 128 or 64 x 128: whole rounds
-    // of 256 workgroups (one per CU) cost about nchunks * c + f microseconds each, c and f measured per tile shape;
-    // the cheapest wins.  The L2 -> CU path bounds these tiles, so what counts is operand rows per output: a
-    // 64 x 128 tile has the outputs of a 32 x 256 one with a third less operand bytes into the CU (192 rows of K / 2
-    // bytes against 288): 512 x 4096 x 4096 13.1 against 19.8 us, 512 x 4096 x 11008 (K) 34.1 against 52; a 128 x 128
-    // tile those of a 64 x 256 one with a fifth less (256 against 320): 1024 x 4096 x 4096 21.5 against 26.1 us on one
-    // box, 768 rows 18.9 against 22.4, 1024 x 4096 x 11008 (K) 50.5 against 58.5.  Small problems (few column tiles)
-    // stay on the tile kernels.
+    // Stream kernel: the tile that select_stream_tile prices cheapest; small problems (few column tiles) stay on
+    // the tile kernels.
     auto tiles = [&](uint32_t bm, uint32_t bn) { return ((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn) * batch; };
     int best_tm = 0;
     bool half_width = false;  // 128-column tiles
     if (kernel == kKernelStream) {
-        const float nch = (float)((p.K + kCK - 1) / kCK);
-        const int tm[5] = {4, 2, 1, 2, 4};
-        const bool hw[5] = {false, false, false, true, true};
-        const float c_us[5] = {1.5f, 1.0f, 0.8f, 0.78f, 0.9f}, f_us[5] = {9.f, 7.f, 6.f, 1.f, 4.5f};
-        float best = 0.f;
-        for (int k = 0; k < 5; ++k) {
-            const uint32_t t = tiles(32u * tm[k], hw[k] ? 128 : 256);
-            const float cost = (float)((t + 255) / 256) * (nch * c_us[k] + f_us[k]);
-            if (best_tm == 0 || cost < best) {
-                best = cost;
-                best_tm = tm[k];
-                half_width = hw[k];
+        const StreamTile tile = select_stream_tile(p.M, p.N, p.K, batch, EPI == 5);
+        if constexpr (EPI != 5) {
+            if (tile.rows == 256) {
+                p.tiles_m = (p.M + 255) / 256;
+                p.tiles_n = (p.N + 255) / 256;
+                DUQ_LAUNCH_HEAD((gemm_s4_stream256_kernel<EPI, BIAS>), dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(256), 0,
+                                stream, p);
+                return;
             }
         }
+        best_tm = (int)(tile.rows / 32);
+        half_width = tile.cols == 128;
     }
     if constexpr (EPI != 5) if (best_tm && p.K <= 256) {
         // rows of at most 256 elements: one chunk, the launch is its output stores: the short-row kernel with 64-row

@@ -88,6 +88,42 @@ inline bool gemm_fuses_dual_rowsum(uint32_t M, uint32_t N, uint32_t K)
     if (kernel == kKernelDecodeRows || kernel == kKernelDecodeMfma) return true;
     return kernel == kKernelStream && K > 256 && N % 8 == 0;
 }
+// Tile of the stream kernel for a problem select_gemm_kernel gives to it (rows 0: none, the tile kernels run).
+// Whole rounds of 256 workgroups (one per CU) cost about nchunks * c + f microseconds each, c (per 256 k) and f
+// measured per tile shape; the cheapest wins.  The L2 -> CU path bounds these tiles, so what counts is operand rows
+// per output: a 64 x 128 tile has the outputs of a 32 x 256 one with a third less operand bytes into the CU (192 rows
+// of K / 2 bytes against 288): 512 x 4096 x 4096 13.1 against 19.8 us, 512 x 4096 x 11008 (K) 34.1 against 52; a
+// 128 x 128 tile those of a 64 x 256 one with a fifth less (256 against 320): 1024 x 4096 x 4096 21.5 against 26.1 us
+// on one box, 768 rows 18.9 against 22.4, 1024 x 4096 x 11008 (K) 50.5 against 58.5.  A round of 256 x 256 tiles
+// (gemm_s4_stream256_kernel; not with the dual-uniform row-sum epilogue, `mode5`) costs 1.91 rounds of 128 x 256
+// ones for twice the outputs, measured (us, 256-row against 128-row tiles): 4096 x 4096 x 4096 56.5 / 58.9,
+// 4096 x 11008 x 4096 149 / 160, 2048 x 22016 x 4096 150 / 160, 4096 x 28672 x 8192 668 / 707,
+// 4096 x 8192 x 28672 (K) 634 / 667; and 4000 x 8200 x 4160, three ragged rounds against five: 160 / 145.
+struct StreamTile {
+    uint32_t rows, cols;
+};
+inline StreamTile select_stream_tile(uint32_t M, uint32_t N, uint32_t K, uint32_t batch, bool mode5)
+{
+    auto tiles = [&](uint32_t bm, uint32_t bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn) * batch; };
+    const float nch = (float)((K + 255) / 256);
+    const uint32_t tm[5] = {4, 2, 1, 2, 4};
+    const bool hw[5] = {false, false, false, true, true};
+    const float c_us[5] = {1.5f, 1.0f, 0.8f, 0.78f, 0.9f}, f_us[5] = {9.f, 7.f, 6.f, 1.f, 4.5f};
+    StreamTile best{0, 0};
+    float best_cost = 0.f;
+    for (int k = 0; k < 5; ++k) {
+        const uint32_t t = tiles(32u * tm[k], hw[k] ? 128 : 256);
+        const float cost = (float)((t + 255) / 256) * (nch * c_us[k] + f_us[k]);
+        if (best.rows == 0 || cost < best_cost) {
+            best_cost = cost;
+            best = StreamTile{32u * tm[k], hw[k] ? 128u : 256u};
+        }
+    }
+    const uint32_t t256 = tiles(256, 256);
+    if (!mode5 && K > 256 && t256 >= 256 && 1.91f * (float)((t256 + 255) / 256) * (nch * c_us[0] + f_us[0]) < best_cost)
+        best = StreamTile{256, 256};
+    return best;
+}
 inline bool decode_uses_rows_kernel(uint32_t M) { return M <= 4; }
 // MFMA decode kernel: one round of at most 256 workgroups, each with its share of the 16-column tiles.  The
 // activations enter a CU once, and a workgroup has two tiles' weights in flight whatever their number; measured

@@ -217,6 +217,9 @@ int duq_batch_linear4bit_forward(int32_t mode, const uint8_t *xq, const duq_half
  * N * K / 2 < 2^32 - 256; larger tensors run the stream / tile kernels, whose bases are 64-bit per tile.  No
  * counterpart in the reference (CUTLASS picks its own tile, src/kernels/gemm.cu:17-42). */
 int duq_gemm_kernel_for(uint32_t M, uint32_t N, uint32_t K);
+/* For a shape of family 6: the stream kernel's tile as rows * 1000 + columns (256256, 128256, 64256, 32256, 128128,
+ * 64128); 0 for the other families.  (The dual-uniform row-sum epilogue never runs the 256-row tile.) */
+int duq_gemm_stream_tile_for(uint32_t M, uint32_t N, uint32_t K);
 
 /* Measurement aid, no counterpart in the reference: reads `bytes` (16-byte aligned, < 4 GiB) of device memory
  * with the access pattern of the decode kernels (every load of a workgroup requested up front, 32 KB per

@@ -11,7 +11,7 @@ from tests import cases
 pytestmark = pytest.mark.gpu
 
 # entry points that launch nothing (queries, set-up)
-_QUERIES = {"duq_abi_version", "duq_get_dual_quant_col_k", "duq_gemm_kernel_for", "duq_quantize_linear4bit_workspace_bytes",
+_QUERIES = {"duq_abi_version", "duq_get_dual_quant_col_k", "duq_gemm_kernel_for", "duq_gemm_stream_tile_for", "duq_quantize_linear4bit_workspace_bytes", "duq_quantize_linear8bit_workspace_bytes",
             "duq_quantize_linear4bit_asym_workspace_bytes", "duq_linear4bit_dual_rowsum_workspace_bytes",
             "duq_static_scratch_init"}
 

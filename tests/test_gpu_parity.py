@@ -278,3 +278,35 @@ def test_fused_forward_equals_unfused_and_oracle(hip, dev, M, N, K, with_bias):
     got = hip.linear4bit_forward(hip.EPI_ASYM_DUAL, T(a), T(sr), T(zr), T(b), T(sc1), T(zc1), T(sc2), T(zc2),
                                  bias=tb).cpu().numpy()
     assert cases.bits_equal(got, fin(orc.asym_dual_dequant(acc, sr, zr, sc1, zc1, sc2, zc2)))
+
+
+@pytest.mark.parametrize("M,N,K,with_bias", [(4090, 4088, 4160, True), (4096, 4090, 4096, False)])
+def test_stream_kernel_256_row_tiles(hip, dev, M, N, K, with_bias):
+    """The stream kernel's 256 x 256 tiles (problems with at least one per CU): ragged last row tile, a last column
+    tile that ends inside a 32-column fragment, an odd number of 64-element row segments, whole-line and
+    per-element epilogues; int32 accumulators, the four reference epilogues and the row-sum one against the oracle
+    over the whole output."""
+    _say("256-row tiles", M, N, K, with_bias)
+    assert hip.gemm_kernel_for(M, N, K) == 6 and hip.gemm_stream_tile_for(M, N, K) == 256256
+    rng = np.random.default_rng(M + N + K)
+    a = _rand_packed(rng, M, K)
+    b = _rand_packed(rng, N, K)
+    sr, zr, sc1, zc1, sc2, zc2, bias = _epi_inputs(rng, M, N)
+    acc = orc.matmul_s4(a, b)
+    T = lambda v: cases.t(v, dev)
+    A, B = T(a), T(b)
+    tb = T(bias) if with_bias else None
+    fin = (lambda y: orc.add_bias(y, bias)) if with_bias else (lambda y: y)
+    assert np.array_equal(hip.matmul(A, B).cpu().numpy(), acc)
+    got = hip.linear4bit_forward(hip.EPI_SYM, A, T(sr), None, B, T(sc1), bias=tb).cpu().numpy()
+    assert cases.bits_equal(got, fin(orc.sym_dequant(acc, sr, sc1)))
+    got = hip.linear4bit_forward(hip.EPI_ASYM, A, T(sr), T(zr), B, T(sc1), T(zc1), bias=tb).cpu().numpy()
+    assert cases.bits_equal(got, fin(orc.asym_dequant(acc, sr, zr, sc1, zc1)))
+    got = hip.linear4bit_forward(hip.EPI_SYM_DUAL, A, T(sr), None, B, T(sc1), None, T(sc2), bias=tb).cpu().numpy()
+    assert cases.bits_equal(got, fin(orc.sym_dual_dequant(acc, sr, sc1, sc2)))
+    got = hip.linear4bit_forward(hip.EPI_ASYM_DUAL, A, T(sr), T(zr), B, T(sc1), T(zc1), T(sc2), T(zc2), bias=tb).cpu().numpy()
+    assert cases.bits_equal(got, fin(orc.asym_dual_dequant(acc, sr, zr, sc1, zc1, sc2, zc2)))
+    rs_row = rng.integers(-8 * K, 8 * K, (M,)).astype(np.int32)
+    adj = rng.integers(-8 * K, 8 * K, (N,)).astype(np.int32)
+    got = hip.linear4bit_forward_rowsum(A, T(sr), T(zr), T(rs_row), B, T(sc1), T(zc1), T(adj), tb).cpu().numpy()
+    assert cases.bits_equal(got, orc.asym_rowsum_dequant(acc, sr, zr, rs_row, sc1, zc1, adj, bias if with_bias else None))

@@ -329,6 +329,20 @@ def test_asym_fp16_input_entry_point_validation_without_launch():
     assert g(ctypes.addressof(layer), P, 1, P, None, 0, None) == -1
 
 
+def test_stream_tile_rule():
+    """Tile of the stream kernel per shape (host arithmetic, duq_gemm_stream_tile_for): 256-row tiles only with at
+    least one per CU and when their rounds come out cheaper."""
+    from duqlinear4bitcuda_amd import _lib
+    f = _lib.load().duq_gemm_stream_tile_for
+    assert f(2048, 4096, 4096) == 128256          # the headline shape: 256 tiles of 128 rows
+    assert f(4096, 4096, 4096) == 256256 and f(4096, 11008, 4096) == 256256 and f(2048, 22016, 4096) == 256256
+    assert f(4096, 28672, 8192) == 256256 and f(4096, 8192, 28672) == 256256
+    assert f(4000, 8200, 4160) == 128256          # three ragged rounds of 256-row tiles against five of 128-row ones
+    assert f(2048, 11008, 4096) == 128256         # 344 tiles of 256 rows: two rounds, the second a third full
+    assert f(512, 4096, 4096) == 64128 and f(1024, 4096, 4096) == 128128
+    assert f(16, 4096, 4096) == 0 and f(1, 4096, 4096) == 0   # decode kernels
+
+
 def test_deferred_quantized_tensor_host_side():
     """What SymQuantizer hands over for a few rows: shape, device and the check that the rows were not written to,
     without anything being computed (quantizing needs the GPU)."""
