@@ -158,19 +158,24 @@ def graph_time_us(fns, reps=5):
     return best
 
 
-def eager_wall_us(modules, x, steps=2000, warm=200):
-    """Wall time per eager call of modules[i % n](x): perf_counter around a loop that ends in synchronize()."""
+def eager_wall_us(modules, x, steps=1000, warm=200, reps=3):
+    """Wall time per eager call of modules[i % n](x): perf_counter around a loop that ends in synchronize(); the
+    best of `reps` such loops (a host-bound figure of a few microseconds picks up every hiccup of the host)."""
     import torch
 
     n = len(modules)
     for i in range(warm):
         modules[i % n](x)
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(steps):
-        modules[i % n](x)
-    torch.cuda.synchronize()
-    return (time.perf_counter() - t0) * 1e6 / steps
+    best = None
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        for i in range(steps):
+            modules[i % n](x)
+        torch.cuda.synchronize()
+        t = (time.perf_counter() - t0) * 1e6 / steps
+        best = t if best is None else min(best, t)
+    return best
 
 
 def shader_clock_mhz():
