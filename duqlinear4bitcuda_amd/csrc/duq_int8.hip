@@ -265,16 +265,19 @@ __global__ __launch_bounds__(256) void gemm_s8_kernel(DUQ_HEAD_DECL, Gemm8Params
     to_global(p.B);
     to_global(p.C);
     to_global(p.y);
-    static_assert(TM == 4 || TM == 2 || TM == 1, "32-row MFMA tiles per wavefront along M");
+    static_assert(TM == 8 || TM == 4 || TM == 2 || TM == 1, "32-row MFMA tiles per wavefront along M");
     // TN = 32-column MFMA tiles per wavefront: tiles of 256 columns (TN = 2), or of 128 (TN = 1, with 64-row tiles:
     // twice the workgroups for problems that leave CUs without a 64 x 256 tile)
     static_assert(TN == 2 || (TN == 1 && TM == 2), "column tiles per wavefront");
     constexpr int BM = 32 * TM, BN = 128 * TN;
-    constexpr int NS = 8;                 // steps (of 32 k) per chunk
-    constexpr uint32_t kChunk = 32 * NS;  // 256
+    // steps (of 32 k) per chunk: 8, or 4 with 256-row tiles (TM = 8: all 256 accumulation registers hold accumulators
+    // and three activation buffers of 256-k chunks would not fit in LDS)
+    constexpr int NS = TM == 8 ? 4 : 8;
+    constexpr uint32_t kChunk = 32 * NS;  // 256 (128)
     constexpr uint32_t kStride = kChunk + 16;
     constexpr uint32_t kBuf = BM * kStride;
-    constexpr int NXP = BM / 16;          // 16-byte activation pieces per thread and chunk: 8, 4, 2
+    constexpr int PPR = kChunk / 16;      // 16-byte pieces per row of a chunk
+    constexpr int NXP = BM * PPR / 256;   // 16-byte activation pieces per thread and chunk: 8, 4, 2 (TM = 8: 8)
 
     constexpr uint32_t kEStride = 32 * TN * 4 + 16;  // epilogue staging: 32 rows of 32*TN int32 per wavefront
     constexpr uint32_t kLds = 3 * kBuf > 4 * 32 * kEStride ? 3 * kBuf : 4 * 32 * kEStride;
@@ -307,10 +310,10 @@ __global__ __launch_bounds__(256) void gemm_s8_kernel(DUQ_HEAD_DECL, Gemm8Params
         return __builtin_bit_cast(v4i, buf_load16(rW, k < p.K ? wrow[t] + (TILED ? k * 32 : k) : kOobOffset, 0));
     };
     uint32_t xrow[NXP], xlds[NXP];
-    const uint32_t xpiece = tid & 15u;
+    const uint32_t xpiece = tid % PPR;
 #pragma unroll
     for (int j = 0; j < NXP; ++j) {
-        const uint32_t row = (tid >> 4) + j * 16;
+        const uint32_t row = tid / PPR + j * (256 / PPR);
         xrow[j] = row * p.K + xpiece * 16;
         xlds[j] = row * kStride + xpiece * 16;
     }
@@ -407,10 +410,12 @@ __global__ __launch_bounds__(256) void gemm_s8_kernel(DUQ_HEAD_DECL, Gemm8Params
                         fx[(s + 1) & 1][b] = s + 1 < NS ? read_x(cur, b, s + 1) : read_x(nxt, b, 0);
                     if (b == TM - 1)  // last use of this step's weight register: refetch it for the next chunk
                         wreg[W][t][s] = load_w(t, s, c + WR);
-                    if (t == TN - 1 && b == 0) {  // activation pieces: chunk c+2 -> its LDS buffer, then fetch chunk c+3
+                    // activation pieces: chunk c+2 -> its LDS buffer, then fetch chunk c+3; the pieces of a step in
+                    // one slot, or (TM = 8: two pieces per step) in slots of their own
+                    if (t == TN - 1 && (TM == 8 || b == 0)) {
 #pragma unroll
                         for (int j = 0; j < NXP; ++j)
-                            if (j * NS / NXP == s) {
+                            if (j * NS / NXP == s && (TM != 8 || b == 2 + 4 * (j % 2))) {
                                 *reinterpret_cast<v4u *>(lds + nx2 + xlds[j]) = xreg[j];
                                 xreg[j] = load_x(j, c + 3);
                             }
@@ -896,6 +901,11 @@ static void launch_rows8(const Gemm8Params &p, hipStream_t stream)
 // weight tensor within 32-bit offsets per descriptor (a descriptor covers one wavefront's rows)
 inline bool rows8_takes(uint32_t M, uint32_t K) { return M <= 4 && K <= (M <= 2 ? 8192u : 4096u); }
 
+// a round of 256 x 256 tiles in rounds of 128 x 256 ones (measured 1.86 - 1.97: 4096 x 4096 x 4096 73.4 against
+// 74.4 us, 4096 x 11008 x 4096 188 against 202, 4096 x 8192 x 8192 240 against 251)
+#ifndef DUQ_S8_COST256
+#define DUQ_S8_COST256 1.95f
+#endif
 template <bool FUSED, bool BIAS, bool TILED>
 static void launch_gemm8_variant(Gemm8Params &p, hipStream_t stream)
 {
@@ -920,7 +930,13 @@ static void launch_gemm8_variant(Gemm8Params &p, hipStream_t stream)
     p.tiles_n = (p.N + 255) / 256;
     // the tallest tile that still gives most of the 256 CUs a workgroup
     const uint32_t t128 = ((p.M + 127) / 128) * p.tiles_n, t64 = ((p.M + 63) / 64) * p.tiles_n;
-    if (p.M > 64 && t128 >= 160) {
+    const uint32_t t256 = ((p.M + 255) / 256) * p.tiles_n;
+    // 256-row tiles where every CU gets one and their rounds (each DUQ_S8_COST256 rounds of 128-row tiles for twice
+    // the outputs) come out cheaper
+    if (t256 >= 256 && DUQ_S8_COST256 * (float)((t256 + 255) / 256) < (float)((t128 + 255) / 256)) {
+        p.tiles_m = (p.M + 255) / 256;
+        DUQ_LAUNCH_HEAD((gemm_s8_kernel<8, 2, FUSED, BIAS, TILED>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, stream, p);
+    } else if (p.M > 64 && t128 >= 160) {
         p.tiles_m = (p.M + 127) / 128;
         DUQ_LAUNCH_HEAD((gemm_s8_kernel<4, 2, FUSED, BIAS, TILED>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, stream, p);
     } else if (p.M > 32 && t64 >= 48) {

@@ -391,7 +391,8 @@ GEMM_SHAPES = [(1, 1, 32), (5, 7, 64), (32, 64, 96), (16, 16, 32), (9, 40, 96), 
                (3, 40, 66560), (40, 300, 33280), (70, 260, 65600),   # long rows
                (512, 4096, 256), (300, 3100, 288), (200, 3990, 96),   # 64 x 128 tiles (48..128 tiles of 64 x 256)
                (1024, 3072, 256),   # 64 x 256 tiles
-               (1000, 3100, 288), (2048, 4096, 4096)]
+               (1000, 3100, 288), (2048, 4096, 4096),
+               (4090, 4088, 4128)]   # 256 x 256 tiles (at least one per CU): ragged rows and columns, a last chunk of 32 k
 
 
 @pytest.mark.gpu
@@ -425,7 +426,8 @@ def test_gpu_asym_dequant_hprec(dev, hip, rows, cols):
 
 FWD_SHAPES = [(5, 4100, 4096), (16, 11008, 1056), (33, 5000, 416), (64, 4099, 2080), (48, 260, 4096), (17, 40, 32),
               (1, 4096, 4096), (2, 250, 5120), (3, 33, 1056), (512, 4096, 128), (300, 3102, 288), (1, 16, 32), (7, 33, 64), (16, 48, 96), (17, 250, 416), (32, 1030, 1056), (4, 4096, 4096), (40, 250, 160), (128, 512, 1024), (130, 1030, 416), (1024, 3072, 256),
-              (1000, 3102, 288)]
+              (1000, 3102, 288),
+              (4090, 4088, 1056)]   # 256 x 256 tiles
 
 
 @pytest.mark.gpu
