@@ -515,6 +515,34 @@ def batched_section(dev, quick=False):
     return out
 
 
+def stack_section(dev):
+    """A stack of eight Sequential(SymQuantizer, Linear4bitSQ) layers of 4096 x 4096 (a decode step through eight
+    projections): wall time per step called eagerly and replayed as one HIP graph (tools.graphs.GraphedForward;
+    the graphed figure includes the copy of the input into the recording and the replay's launch)."""
+    import torch
+
+    from duqlinear4bitcuda_amd.nn import Linear4bitSQ, SymQuantizer
+    from duqlinear4bitcuda_amd.tools.graphs import GraphedForward
+
+    K = N = 4096
+    g = torch.Generator().manual_seed(9)
+    layers = []
+    for _ in range(8):
+        layer = Linear4bitSQ(K, N, bias=False).to(dev)
+        layer.weight = torch.randint(0, 256, (N, K // 2), dtype=torch.uint8, generator=g).to(dev)
+        layer.weight_scales = (torch.rand(N, 1, generator=g) * 0.002 + 0.0005).half().to(dev)
+        layers += [SymQuantizer(1.0), layer]
+    model = torch.nn.Sequential(*layers)
+    out = []
+    for M in (1, 4, 16):
+        x = torch.randn(1, M, K, generator=g).half().to(dev)
+        graphed = GraphedForward(model, x)
+        same = bool(torch.equal(graphed(x).view(torch.int16), model(x).view(torch.int16)))
+        out.append({"layers": 8, "M": M, "K": K, "N": N, "eager_us_per_step": round(eager_wall_us([model], x, steps=300, warm=50), 2),
+                    "graphed_us_per_step": round(eager_wall_us([graphed], x, steps=300, warm=50), 2), "same_bits": same})
+    return out
+
+
 def int8_layer_section(dev, quick=False):
     """The 8-bit asymmetric layer (LinearQuant8bitASQ) at the headline shape: float32 activations, quantizer
     launch + fused GEMM launch, float32 result; the GEMM alone against the dense int8 MFMA peak."""
@@ -761,6 +789,7 @@ def main():
     batched = batched_section(dev, args.quick)
     harness = None if args.no_harness else harness_section(dev, args.quick)
     fanout = None if args.quick else fanout_section(dev)
+    stack = None if args.quick or args.no_harness else stack_section(dev)
     rows_7b = [d for d in decode if (d["M"], d["N"], d["K"]) in LLAMA7B_DECODE]
     worst = min(rows_7b, key=lambda d: d["frac_hbm"])
     roofline_decode = {"bound": "hbm", "kernel": "gemv_s4_rows_kernel (M <= 8, quantizer inside) / quantize_rows_kernel + "
@@ -814,6 +843,7 @@ def main():
         "batched": batched,
         "harness": harness,
         "fanout": fanout,
+        "stack": stack,
         "cpu_baseline": cpu,
         "device": {"name": props.name, "arch": props.gcnArchName, "cus": props.multi_processor_count},
     }

@@ -13,6 +13,7 @@ _ALIASES = {
     "tools": "tools",
     "tools.tensor_utils": "tools.tensor_utils",
     "tools.quantization": "tools.quantization",
+    "tools.graphs": "tools.graphs",
     "_CUDA": "_HIP",
 }
 for _alias, _target in _ALIASES.items():
