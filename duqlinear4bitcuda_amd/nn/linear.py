@@ -80,7 +80,7 @@ class _Linear4bitBase(torch.nn.Module):
 
     def _decode_forward(self, x, clip=1.0, qmax=6, checked=False):
         """y for binary16 rows ``x`` when the layer takes them in one library call (up to eight rows: one launch,
-        quantizer inside; up to 64: quantizer launch + GEMM launch), else None."""
+        quantizer inside; up to 256: quantizer launch + GEMM launch), else None."""
         if not self.fused:
             return None
         d = self._decode_call()
@@ -92,7 +92,19 @@ class _Linear4bitBase(torch.nn.Module):
         M = x.numel() // K
         if d._one.get(M, -1) < 0 and not d.admits(M):
             return None
+        if M > 64 and self._fp6_wanted(M):  # large enough for the 6-bit float path, and the layer holds a shadow
+            return None
         return d.run(x, M, clip, qmax, checked)
+
+    def _take_deferred(self, x):
+        """A PackedQuantizedTensor that SymQuantizer handed on unquantized: the result of the one-call path, or None
+        after quantizing it now (with the 6-bit float shadow when this layer will take that path)."""
+        y = self._decode_forward(x.source(), x._clip, x._qmax, True)
+        if y is None:
+            src = x._src
+            rows = src.numel() // src.shape[-1]
+            x.materialize(shadow=bool(self.fused and src.shape[-1] % 128 == 0 and self._fp6_wanted(rows)))
+        return y
 
     def enable_fp6(self):
         """Build the E3M2 shadow of ``weight`` (3/4 byte per element next to the 1/2 byte of the packed
@@ -161,8 +173,8 @@ class Linear4bitSQ(_Linear4bitBase):
 
     def forward(self, x):
         assert type(x) == tensor_utils.PackedQuantizedTensor  # quantized input is required
-        if x._src is not None:  # a few rows straight from SymQuantizer: quantized inside the GEMM launch
-            y = self._decode_forward(x.source(), x._clip, x._qmax, True)
+        if x._src is not None:  # up to 256 rows straight from SymQuantizer: quantizer and GEMM in one library call
+            y = self._take_deferred(x)
             if y is not None:
                 return y
         xq, scales_x = x.quantized_x, x.scales_x
@@ -426,8 +438,8 @@ class Linear4bitDUSQ(_Linear4bitBase):
 
     def forward(self, x):
         assert type(x) == tensor_utils.PackedQuantizedTensor
-        if x._src is not None:  # a few rows straight from SymQuantizer: quantized inside the GEMM launch
-            y = self._decode_forward(x.source(), x._clip, x._qmax, True)
+        if x._src is not None:  # up to 256 rows straight from SymQuantizer: quantizer and GEMM in one library call
+            y = self._take_deferred(x)
             if y is not None:
                 return y
         xq, scales_x = x.quantized_x, x.scales_x

@@ -31,9 +31,9 @@ class SymQuantizer(torch.nn.Module):
     # Linear4bitSQ / Linear4bitDUSQ that follows quantizes them inside its own library call (up to eight rows
     # quantizer + GEMM + dequant are ONE launch; above, the quantizer launch and the GEMM launch of one call: at
     # these sizes a step costs more on the host than on the GPU, and a call less is most of it), and anything
-    # else that reads quantized_x / scales_x triggers this quantizer's launch then, with the same bits.  0
-    # switches that off.
-    defer_rows = 64
+    # else that reads quantized_x / scales_x triggers this quantizer's launch then, with the same bits.  Not for
+    # inputs this quantizer is set to write the 6-bit float shadow for.  0 switches that off.
+    defer_rows = 256
 
     def __init__(self, input_clip_ratio=1.0, qmax: int = 6, shadow=False, shadow_min_rows: int = 96):
         super().__init__()
@@ -50,7 +50,8 @@ class SymQuantizer(torch.nn.Module):
             x = x.contiguous()
         cols = x.shape[-1]
         if shadow is None and self.defer_rows and cols % 64 == 0 and 0 < x.numel() <= self.defer_rows * cols and \
-                x.is_cuda and x.dtype is torch.float16 and x.data_ptr() % 16 == 0:
+                x.is_cuda and x.dtype is torch.float16 and x.data_ptr() % 16 == 0 and \
+                not (self.shadow and x.numel() >= self.shadow_min_rows * cols and cols % 128 == 0):
             return tensor_utils.PackedQuantizedTensor.deferred(x, self.input_clip_ratio, self.qmax)
         shadow = _shadow_choice(self, x, shadow)
         if shadow:

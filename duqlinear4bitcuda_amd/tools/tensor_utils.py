@@ -55,10 +55,20 @@ class PackedQuantizedTensor:
                                "and the first use of its result")
         return x
 
-    def _materialize(self):
+    def _materialize(self, shadow=False):
         x = self.source()
-        self._q, self._s = _ops.quantize_rows_sym(x, self._clip, self._qmax)
+        if shadow:
+            self._q, self.shadow_x, self._s = quantize_sym_shadow(x, self._clip, self._qmax, shadow != "only")
+        else:
+            self._q, self._s = _ops.quantize_rows_sym(x, self._clip, self._qmax)
         self._src = None
+
+    def materialize(self, shadow=False):
+        """Quantize a deferred tensor now (no effect on one that is quantized already).  ``shadow``: True also
+        writes the 6-bit float shadow of the codes (inputs whose width is a multiple of 128), "only" nothing else."""
+        if self._src is not None:
+            self._materialize(shadow)
+        return self
 
     @property
     def quantized_x(self):

@@ -1,5 +1,5 @@
 """Decode through the drop-in modules: Sequential(SymQuantizer, Linear4bitSQ / Linear4bitDUSQ) and the layers with
-their own AsymQuantizer run quantizer + GEMM + dequant as ONE library call for up to 64 rows (one launch up to
+their own AsymQuantizer run quantizer + GEMM + dequant as ONE library call for up to 256 rows (one launch up to
 eight), with the bits of the oracle; and the binary16-input entry point of the asymmetric modes against the oracle, through the C ABI."""
 import numpy as np
 import pytest
@@ -97,7 +97,7 @@ def test_sequential_symquantizer_linear_is_one_library_call(dev, library_calls, 
 
 def test_symquantizer_settings_reach_the_one_launch_path(dev, library_calls):
     """clip ratio and upper clamp of the quantizer in front, a quantizer with deferral switched off, a layer with
-    fused = False, nine and 65 rows, and an input written to between the quantizer and the layer."""
+    fused = False, 9, 130 and 257 rows, and an input written to between the quantizer and the layer."""
     from duqlinear4bitcuda_amd.nn import SymQuantizer
     M, N, K = 3, 200, 1024
     sq, _, wq, sw, _, _ = _sq_layers(dev, N, K, seed=5, bias=False)
@@ -120,7 +120,8 @@ def test_symquantizer_settings_reach_the_one_launch_path(dev, library_calls):
     assert cases.bits_equal(torch.nn.Sequential(SymQuantizer(1.0), sq)(X).cpu().numpy(), want)
     assert library_calls == ["duq_quantize_rows_sym", "duq_matmul_host_4bit", "duq_sym_dequant_host"], library_calls
     sq.fused = True
-    for rows, calls in ((9, ["duq_quantize_linear4bit_forward_layer"]), (65, ["duq_quantize_rows_sym", "duq_linear4bit_forward"])):
+    for rows, calls in ((9, ["duq_quantize_linear4bit_forward_layer"]), (130, ["duq_quantize_linear4bit_forward_layer"]),
+                        (257, ["duq_quantize_rows_sym", "duq_linear4bit_forward"])):
         x9 = cases.acts_normal(rows, K, seed=7)
         library_calls.clear()
         y9 = torch.nn.Sequential(SymQuantizer(1.0), sq)(cases.t(x9, dev))
@@ -281,9 +282,9 @@ def test_asym_fp16_input_two_launch_shapes_and_errors(dev):
 @pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (4, 11008, 4096), (8, 512, 2048), (3, 100, 8192), (16, 4096, 4096),
                                     (40, 1000, 1024), (100, 1000, 512)])
 def test_dual_uniform_rowsum_layer_decode(dev, library_calls, M, N, K):
-    """LinearQuant4bitDUASQRowSum from binary16 rows: one library call up to 64 rows (one launch up to eight, the
+    """LinearQuant4bitDUASQRowSum from binary16 rows: one library call up to 256 rows (one launch up to eight, the
     quantizer inside the rows kernel; quantizer + GEMM with the epilogue inside for the MFMA decode kernel's shapes;
-    three launches on the ring kernel's), two calls above; the oracle's bits everywhere, and the op's codes / scales / zero points / row sums."""
+    three launches on the ring kernel's); the oracle's bits everywhere, and the op's codes / scales / zero points / row sums."""
     from duqlinear4bitcuda_amd import _HIP as hip
     from duqlinear4bitcuda_amd.nn import LinearQuant4bitDUASQRowSum
     _say("dual row-sum decode", M, N, K)
@@ -304,10 +305,7 @@ def test_dual_uniform_rowsum_layer_decode(dev, library_calls, M, N, K):
     layer(X)
     library_calls.clear()
     y = layer(X)
-    if M <= 64:
-        assert library_calls == ["duq_quantize_linear4bit_forward_layer"], library_calls
-    else:
-        assert library_calls == ["duq_quantize_rows_asym_shifted", "duq_linear4bit_forward_dual_rowsum"], library_calls
+    assert library_calls == ["duq_quantize_linear4bit_forward_layer"], library_calls
     assert cases.bits_equal(y.detach().cpu().numpy(), want)
     layer.fused = False
     assert cases.bits_equal(layer(X).detach().cpu().numpy(), want)
@@ -322,3 +320,29 @@ def test_dual_uniform_rowsum_layer_decode(dev, library_calls, M, N, K):
     y = hip.quantize_linear4bit_forward_asym(hip.EPI_ASYM_DUAL_ROWSUM, X, T(wq), T(s1), T(z1), T(s2), T(z2), T(a1), None,
                                              w_rowsum_adj_2=T(a2))
     assert cases.bits_equal(y.cpu().numpy(), orc.linear4bit_duasq_rowsum_forward(x, wq, s1, z1, s2, z2, a1, a2)[0])
+
+
+def test_deferred_input_meets_a_layer_on_the_6bit_float_path(dev, library_calls):
+    """130 rows from a plain SymQuantizer into a layer with enable_fp6(): the layer quantizes them with the shadow
+    and takes the 6-bit float kernel; without enable_fp6() the same rows are one library call; same bits."""
+    from duqlinear4bitcuda_amd.nn import SymQuantizer
+    M, N, K = 130, 4096, 512
+    sq, _, wq, sw, _, _ = _sq_layers(dev, N, K, seed=9, bias=False)
+    x = cases.acts_normal(M, K, seed=10)
+    X = cases.t(x, dev)
+    want = orc.linear4bit_sq_forward(x, wq, sw)[0]
+    library_calls.clear()
+    y = torch.nn.Sequential(SymQuantizer(1.0), sq)(X)
+    assert library_calls == ["duq_quantize_linear4bit_forward_layer"], library_calls
+    assert cases.bits_equal(y.cpu().numpy(), want)
+    sq.enable_fp6()
+    assert sq._fp6_wanted(M)
+    library_calls.clear()
+    pq = SymQuantizer(1.0)(X)
+    y = sq(pq)
+    assert library_calls == ["duq_quantize_rows_sym_bf6", "duq_linear4bit_forward_bf6"], library_calls
+    assert cases.bits_equal(y.cpu().numpy(), want)
+    assert pq.shadow_x is not None and np.array_equal(pq.quantized_x.cpu().numpy(), orc.sym_quant(x, orc.sym_scales(x)))
+    # a quantizer that is set to write the shadow itself does not hand such rows on
+    p2 = SymQuantizer(1.0, shadow="only")(X)
+    assert p2._src is None and p2.shadow_x is not None and p2.quantized_x is None
