@@ -622,9 +622,9 @@ class FusedDecode:
         return ref[0]
 
     # Rows up to which a module hands binary16 activations to this call.  Up to eight rows (and N <= 16384) it is one
-    # launch; above, the quantizer launch and the GEMM launch of one library call: up to a few hundred rows the two
-    # kernels take less time than two calls cost on the host.
-    max_rows = 256
+    # launch; above, the quantizer launch and the GEMM launch of one library call: up to about 700 rows (N = K = 4096)
+    # the two kernels take less time than two calls cost on the host (23 us).
+    max_rows = 1024
 
     def _staging(self, M: int) -> int:
         """Bytes the library stages between its two launches at M rows (0: one launch); -1 when M is out of range."""

@@ -80,7 +80,7 @@ class _Linear4bitBase(torch.nn.Module):
 
     def _decode_forward(self, x, clip=1.0, qmax=6, checked=False):
         """y for binary16 rows ``x`` when the layer takes them in one library call (up to eight rows: one launch,
-        quantizer inside; up to 256: quantizer launch + GEMM launch), else None."""
+        quantizer inside; up to 1024: quantizer launch + GEMM launch), else None."""
         if not self.fused:
             return None
         d = self._decode_call()
@@ -173,7 +173,7 @@ class Linear4bitSQ(_Linear4bitBase):
 
     def forward(self, x):
         assert type(x) == tensor_utils.PackedQuantizedTensor  # quantized input is required
-        if x._src is not None:  # up to 256 rows straight from SymQuantizer: quantizer and GEMM in one library call
+        if x._src is not None:  # up to 1024 rows straight from SymQuantizer: quantizer and GEMM in one library call
             y = self._take_deferred(x)
             if y is not None:
                 return y
@@ -438,7 +438,7 @@ class Linear4bitDUSQ(_Linear4bitBase):
 
     def forward(self, x):
         assert type(x) == tensor_utils.PackedQuantizedTensor
-        if x._src is not None:  # up to 256 rows straight from SymQuantizer: quantizer and GEMM in one library call
+        if x._src is not None:  # up to 1024 rows straight from SymQuantizer: quantizer and GEMM in one library call
             y = self._take_deferred(x)
             if y is not None:
                 return y

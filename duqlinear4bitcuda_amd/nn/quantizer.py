@@ -33,7 +33,7 @@ class SymQuantizer(torch.nn.Module):
     # these sizes a step costs more on the host than on the GPU, and a call less is most of it), and anything
     # else that reads quantized_x / scales_x triggers this quantizer's launch then, with the same bits.  Not for
     # inputs this quantizer is set to write the 6-bit float shadow for.  0 switches that off.
-    defer_rows = 256
+    defer_rows = 1024
 
     def __init__(self, input_clip_ratio=1.0, qmax: int = 6, shadow=False, shadow_min_rows: int = 96):
         super().__init__()

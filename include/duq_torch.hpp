@@ -214,7 +214,7 @@ public:
     float input_clip_ratio;
     int qmax;
     bool shadow;  // also write the 6-bit float shadow (inputs whose width is a multiple of 128)
-    // defer_rows > 0 (at most 256 is useful): inputs of at most that many rows are handed on unquantized
+    // defer_rows > 0 (at most 1024 is useful): inputs of at most that many rows are handed on unquantized
     // (PackedQuantizedTensor::deferred) and the linear layer behind quantizes them inside its own library call (one
     // launch up to eight rows, the quantizer launch and the GEMM launch of one call above).  Off by default: the
     // fields quantized_x and scale of such a tensor are undefined until materialize(), and code written against the
@@ -312,7 +312,7 @@ inline torch::Tensor fused_forward_shadow(int mode, const PackedQuantizedTensor 
     return y.view(lead);
 }
 
-// A deferred input of at most 256 rows: quantizer + GEMM + dequant in one library call (ONE launch where the shape
+// A deferred input of at most 1024 rows: quantizer + GEMM + dequant in one library call (ONE launch where the shape
 // allows, else two with the codes and scales staged in a workspace allocated here); else an undefined tensor (the
 // caller then materializes the input and takes the usual route).
 inline torch::Tensor fused_decode(int mode, const PackedQuantizedTensor &input, const torch::Tensor &weight,
@@ -323,7 +323,7 @@ inline torch::Tensor fused_decode(int mode, const PackedQuantizedTensor &input, 
     TORCH_CHECK(x.device() == weight.device(), "Linear4bit::forward: operands on different devices");
     TORCH_CHECK(weight.size(1) * 2 == x.size(-1), "Linear4bit::forward: K differs");
     const uint32_t K = x.size(-1), M = x.numel() / K, N = weight.size(0);
-    if (M > 256) return torch::Tensor();
+    if (M > 1024) return torch::Tensor();
     const uint64_t ws_bytes = duq_quantize_linear4bit_workspace_bytes(M, N, K);
     torch::Tensor ws;
     if (ws_bytes) ws = torch::empty({(int64_t)ws_bytes}, torch::dtype(torch::kUInt8).device(x.device()));

@@ -1,5 +1,5 @@
 """Decode through the drop-in modules: Sequential(SymQuantizer, Linear4bitSQ / Linear4bitDUSQ) and the layers with
-their own AsymQuantizer run quantizer + GEMM + dequant as ONE library call for up to 256 rows (one launch up to
+their own AsymQuantizer run quantizer + GEMM + dequant as ONE library call for up to 1024 rows (one launch up to
 eight), with the bits of the oracle; and the binary16-input entry point of the asymmetric modes against the oracle, through the C ABI."""
 import numpy as np
 import pytest
@@ -97,7 +97,7 @@ def test_sequential_symquantizer_linear_is_one_library_call(dev, library_calls, 
 
 def test_symquantizer_settings_reach_the_one_launch_path(dev, library_calls):
     """clip ratio and upper clamp of the quantizer in front, a quantizer with deferral switched off, a layer with
-    fused = False, 9, 130 and 257 rows, and an input written to between the quantizer and the layer."""
+    fused = False, 9, 130 and 1025 rows, and an input written to between the quantizer and the layer."""
     from duqlinear4bitcuda_amd.nn import SymQuantizer
     M, N, K = 3, 200, 1024
     sq, _, wq, sw, _, _ = _sq_layers(dev, N, K, seed=5, bias=False)
@@ -121,7 +121,7 @@ def test_symquantizer_settings_reach_the_one_launch_path(dev, library_calls):
     assert library_calls == ["duq_quantize_rows_sym", "duq_matmul_host_4bit", "duq_sym_dequant_host"], library_calls
     sq.fused = True
     for rows, calls in ((9, ["duq_quantize_linear4bit_forward_layer"]), (130, ["duq_quantize_linear4bit_forward_layer"]),
-                        (257, ["duq_quantize_rows_sym", "duq_linear4bit_forward"])):
+                        (1025, ["duq_quantize_rows_sym", "duq_linear4bit_forward"])):
         x9 = cases.acts_normal(rows, K, seed=7)
         library_calls.clear()
         y9 = torch.nn.Sequential(SymQuantizer(1.0), sq)(cases.t(x9, dev))
@@ -282,7 +282,7 @@ def test_asym_fp16_input_two_launch_shapes_and_errors(dev):
 @pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (4, 11008, 4096), (8, 512, 2048), (3, 100, 8192), (16, 4096, 4096),
                                     (40, 1000, 1024), (100, 1000, 512)])
 def test_dual_uniform_rowsum_layer_decode(dev, library_calls, M, N, K):
-    """LinearQuant4bitDUASQRowSum from binary16 rows: one library call up to 256 rows (one launch up to eight, the
+    """LinearQuant4bitDUASQRowSum from binary16 rows: one library call up to 1024 rows (one launch up to eight, the
     quantizer inside the rows kernel; quantizer + GEMM with the epilogue inside for the MFMA decode kernel's shapes;
     three launches on the ring kernel's); the oracle's bits everywhere, and the op's codes / scales / zero points / row sums."""
     from duqlinear4bitcuda_amd import _HIP as hip
