@@ -579,7 +579,7 @@ def int8_layer_section(dev, quick=False):
             eager["module_eager_us"] = round(eager_wall_us([layer], x), 2)
             layer.one_call_rows = 0
             eager["module_eager_two_calls_us"] = round(eager_wall_us([layer], x), 2)
-            layer.one_call_rows = 256
+            layer.one_call_rows = 1024
         out.append({"M": M, "K": K, "N": N, "step_us": round(us_step, 2), "step_TOPS": round(ops / us_step / 1e6, 1), **eager,
                     "three_step_us": round(us3, 2), "fused_equals_three_steps": same,
                     "quantize_us": round(us_quant, 2),

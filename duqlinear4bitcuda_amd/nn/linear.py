@@ -572,7 +572,7 @@ class LinearQuant8bitASQ(torch.nn.Module):
 
     # rows up to which the layer's own quantizer and the GEMM go through one library call (a step of a few rows
     # costs more on the host than on the GPU; larger inputs hide the second call behind the first launch)
-    one_call_rows = 256
+    one_call_rows = 1024
 
     def forward(self, x):
         if self.require_quantizer:

@@ -520,9 +520,9 @@ def test_gpu_layer_8bit(dev):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("rows", [1, 4, 5, 16, 74, 256, 300])
+@pytest.mark.parametrize("rows", [1, 4, 5, 16, 74, 256, 1024, 1030])
 def test_gpu_layer_8bit_one_call(dev, monkeypatch, rows):
-    """LinearQuant8bitASQ with its own quantizer: up to 256 rows quantizer + GEMM are one library call, the bits of
+    """LinearQuant8bitASQ with its own quantizer: up to 1024 rows quantizer + GEMM are one library call, the bits of
     the oracle and of the two calls; above, two calls."""
     import torch
     from duqlinear4bitcuda_amd import _lib
@@ -548,9 +548,9 @@ def test_gpu_layer_8bit_one_call(dev, monkeypatch, rows):
         monkeypatch.setattr(lib, name, (lambda *a, _r=real, _n=name: (calls.append(_n), _r(*a))[1]), raising=False)
     y = layer(xt)
     tiled_fwd = "duq_linear8bit_forward" if rows <= 4 else "duq_linear8bit_forward_tiled"
-    assert calls == (["duq_quantize_linear8bit_forward"] if rows <= 256 else ["duq_quantize_rows_asym_8bit", tiled_fwd]), calls
+    assert calls == (["duq_quantize_linear8bit_forward"] if rows <= 1024 else ["duq_quantize_rows_asym_8bit", tiled_fwd]), calls
     assert np.array_equal(y.cpu().numpy().view(np.uint32), want.view(np.uint32))
-    for tiled, one_call in ((False, 256), (True, 0)):
+    for tiled, one_call in ((False, 1024), (True, 0)):
         layer.tiled, layer.one_call_rows = tiled, one_call
         assert torch.equal(layer(xt), y), (tiled, one_call)
 
