@@ -452,8 +452,8 @@ def quantize_linear4bit_forward(x, w, w_scale_1, w_scale_2=None, bias=None, clip
                                 return_quantized: bool = False, static: bool = False, slot: int = 0):
     """SymQuantizer + Linear4bitSQ / Linear4bitDUSQ forward (qlinear4bit/nn/quantizer.py:10-16,
     qlinear4bit/nn/linear.py:42-56, 167-176) from binary16 activations ``x`` [..., K]: bit-identical to
-    ``quantize_rows_sym`` followed by ``linear4bit_forward``.  Up to eight rows are ONE launch;
-    larger inputs run the two launches with the codes staged in a buffer allocated here.  With
+    ``quantize_rows_sym`` followed by ``linear4bit_forward``.  Up to eight rows (and nine to sixteen that hold at
+    most 32768 elements together) are ONE launch; larger inputs run the two launches with the codes staged in a buffer allocated here.  With
     ``return_quantized`` also returns (codes uint8 [..., K/2], scales [..., 1]).  ``static=True`` stages in the
     library's static device array instead (``duq_quantize_linear4bit_forward_static``: nothing but the outputs is
     allocated; M * K / 2 <= 8 MiB; calls that may overlap on one GPU must name different ``slot``s, 0..3)."""
@@ -510,7 +510,8 @@ def quantize_linear4bit_forward_asym(mode, x, w, w_scale_1, w_zeros_1, w_scale_2
     (``mode`` EPI_ASYM_ROWSUM with ``w_rowsum_adj``, or EPI_ASYM_DUAL_ROWSUM with ``w_rowsum_adj`` /
     ``w_rowsum_adj_2`` for the dual-uniform layer: the signed-shifted quantizer): bit-identical to
     ``quantize_rows_asym`` (``quantize_rows_asym_shifted``) followed by ``linear4bit_forward``
-    (``linear4bit_forward_rowsum`` / ``linear4bit_forward_dual_rowsum``).  Up to eight rows are ONE launch; larger inputs run the two launches with the
+    (``linear4bit_forward_rowsum`` / ``linear4bit_forward_dual_rowsum``).  Up to eight rows (sixteen short ones) are
+    ONE launch; larger inputs run the two launches with the
     codes staged in a buffer allocated here.  With ``return_quantized`` also returns (codes, scales [..., 1],
     zeros [..., 1][, rowsum [...]])."""
     name = "quantize_linear4bit_forward_asym"
@@ -565,7 +566,8 @@ class FusedDecode:
     """One layer's side of the one-launch decode (what ``duq_quantize_linear4bit_forward`` takes for the symmetric
     modes and ``duq_quantize_linear4bit_forward_asym`` for the asymmetric and row-sum modes), checked once and kept
     as a ``duq_fused_layer`` struct for ``duq_quantize_linear4bit_forward_layer``: a decode step of a module then
-    costs one ``torch.empty`` (two above eight rows: the staging buffer) and one foreign call with seven arguments.  The tensors are held (``tensors``) so that
+    costs one ``torch.empty`` (two for the shapes of two launches: the staging buffer) and one foreign call with seven
+    arguments.  The tensors are held (``tensors``) so that
     a caller can tell when the layer's buffers were replaced; a change of their contents in place needs no new
     object."""
 
@@ -621,7 +623,7 @@ class FusedDecode:
             ref = self._structs[key] = (ctypes.addressof(st), st)   # (the struct is kept alive beside its address)
         return ref[0]
 
-    # Rows up to which a module hands binary16 activations to this call.  Up to eight rows (and N <= 16384) it is one
+    # Rows up to which a module hands binary16 activations to this call.  Up to eight rows, sixteen short ones (and N <= 16384) it is one
     # launch; above, the quantizer launch and the GEMM launch of one library call: up to about 700 rows (N = K = 4096)
     # the two kernels take less time than two calls cost on the host (23 us).
     max_rows = 1024

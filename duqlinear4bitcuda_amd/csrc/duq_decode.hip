@@ -65,6 +65,11 @@
 #ifndef DUQ_DEC_WAVES
 #define DUQ_DEC_WAVES 8
 #endif
+// wavefronts per workgroup of the MFMA kernel when it quantizes its 16 rows itself
+// (16 rows, N = 4096: sixteen against eight wavefronts K = 4096 7.2 against 7.9 us, K = 2048 4.9 against 5.4)
+#ifndef DUQ_DEC_MFMA_FUSEQ_WAVES
+#define DUQ_DEC_MFMA_FUSEQ_WAVES 16
+#endif
 
 namespace duq {
 
@@ -443,16 +448,32 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DUQ_HEAD_DECL,
 // and registers (MT * SEGS * 4 for the packed activations), not weight traffic.  Nibble -> byte as in the
 // GEMM kernels: (w & 0xF0F0F0F0) is the four odd-k nibbles times 16, ((w << 4) & 0xF0F0F0F0) the even ones;
 // every product is 256 * a * b and one arithmetic shift recovers the sum.
-template <int WAVES, int SEGS, int EPI, int MT = 1, bool DB = true>
+//
+// FUSEQ (one row tile, EPI >= 0): the activations arrive as binary16 and the workgroup quantizes its 16 rows itself,
+// 16 / WAVES whole rows per wavefront (so a row's statistics never leave its wavefront), into LDS; the fragments
+// then come from there.  Every workgroup repeats that work: it pays while the quantizer's own launch (about 2.6 us
+// with the wait between the two) costs more than sixteen rows on a CU's vector units.
+template <int WAVES, int SEGS, int EPI, int MT = 1, bool DB = true, bool FUSEQ = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_s4_decode_kernel(DUQ_HEAD_DECL, DecodeParams tail)
 {
     const DecodeParams p = with_head(tail, DUQ_HEAD_USE);
     constexpr int MODE = EPI < 0 ? 0 : EPI;
-    static_assert(WAVES == 4 || WAVES == 8, "wavefronts per workgroup");
+    static_assert(WAVES == 4 || WAVES == 8 || (WAVES == 16 && FUSEQ), "wavefronts per workgroup");
     static_assert(MT >= 1 && MT <= 4, "16-row activation tiles");
+    static_assert(!FUSEQ || (MT == 1 && EPI >= 0 && WAVES >= 8 && (WAVES * SEGS) % 4 == 0), "rows quantized in the kernel");
     constexpr int NG = WAVES / 4;             // groups of 256 finishing threads
     constexpr int FT = (MT + NG - 1) / NG;    // row tiles a finishing thread completes
     __shared__ v4i part[2][MT][WAVES][64];
+    // FUSEQ: the codes of the 16 rows (a row every XSTRIDE bytes: 16 bytes more than the longest row, so that the 16
+    // rows a fragment read touches fall on different banks) and their per-token parameters
+    constexpr int RPW = FUSEQ ? 16 / WAVES : 1;        // rows a wavefront quantizes
+    constexpr int UPR = FUSEQ ? WAVES * SEGS / 4 : 1;  // 8-element units per lane and row
+    constexpr uint32_t XSTRIDE = WAVES * SEGS * 64 + 16;
+    __shared__ __attribute__((aligned(16))) uint8_t xs[FUSEQ ? 16 * XSTRIDE : 16];
+    __shared__ uint16_t srow[16], zrow[16];
+    __shared__ int rsrow[16];
+    constexpr bool ASYMQ = FUSEQ && (MODE == 1 || MODE == 3 || MODE == 4 || MODE == 5);
+    constexpr bool SHIFTQ = FUSEQ && (MODE == 4 || MODE == 5);
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t l16 = lane & 15u, g = lane >> 4;
@@ -481,12 +502,28 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_s4_decode_kernel(DUQ_HEAD_DEC
     // wavefront's k range (packed; expanded when used), the first tile's weights, the parameters of the outputs
     // this thread will finish
     v4u xp[MT][SEGS];
-    const __amdgpu_buffer_rsrc_t rX = make_rsrc(p.A, p.M * kbytes);  // rows past M read as zero
+    v4u raw[RPW][UPR];
+    const uint32_t nunits = p.K >> 3;
+    if constexpr (!FUSEQ) {
+        const __amdgpu_buffer_rsrc_t rX = make_rsrc(p.A, p.M * kbytes);  // rows past M read as zero
 #pragma unroll
-    for (int t = 0; t < MT; ++t)
+        for (int t = 0; t < MT; ++t)
 #pragma unroll
-        for (int u = 0; u < SEGS; ++u)
-            xp[t][u] = buf_load16(rX, koff[u] != kOobOffset ? (t * 16 + l16) * kbytes + koff[u] : kOobOffset, 0);
+            for (int u = 0; u < SEGS; ++u)
+                xp[t][u] = buf_load16(rX, koff[u] != kOobOffset ? (t * 16 + l16) * kbytes + koff[u] : kOobOffset, 0);
+    } else {
+        // wavefront v quantizes rows v * RPW ..; lane l owns the 8-element units l, l + 64, ... of each
+        const __amdgpu_buffer_rsrc_t rX = make_rsrc(p.X, p.M * p.K * 2);  // rows past M read as zero
+#pragma unroll
+        for (int r = 0; r < RPW; ++r)
+#pragma unroll
+            for (int j = 0; j < UPR; ++j) {
+                const uint32_t c = lane + j * 64;
+                raw[r][j] = buf_load16(rX, c < nunits ? ((wave * RPW + r) * p.K + c * 8) * 2 : kOobOffset, 0);
+            }
+        // every wavefront requests its activations before any requests weights (requests are served in order)
+        __builtin_amdgcn_s_barrier();
+    }
     v4u w0[SEGS], w1[DB ? SEGS : 1];
     load_tile(tile0, w0);
 
@@ -512,7 +549,90 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_s4_decode_kernel(DUQ_HEAD_DEC
 #pragma unroll
     for (int f = 0; f < FT; ++f) {
         rp[f] = RowRec{};
-        if (EPI >= 0 && finisher) rp[f] = load_row_rt<MODE>(p.epi, min((fg + f * NG) * 16 + my_m, p.M - 1), p.A, kbytes);
+        if (EPI >= 0 && finisher && !FUSEQ)
+            rp[f] = load_row_rt<MODE>(p.epi, min((fg + f * NG) * 16 + my_m, p.M - 1), p.A, kbytes);
+    }
+
+    if constexpr (FUSEQ) {
+        // the quantizer's arguments, fetched under the vector loads above (a scalar load issued where its value is
+        // first used is waited for on its own)
+        const float q_clip = p.clip;
+        const int q_qmax = p.qmax;
+        uint8_t *const q_out = p.q_out;
+        uint16_t *const s_out = p.s_out, *const z_out = p.z_out;
+        int32_t *const rs_out = p.rs_out;
+        asm volatile("" ::"s"(q_clip), "s"(q_qmax), "s"(q_out), "s"(s_out), "s"(z_out), "s"(rs_out));
+        const bool copy_out = blockIdx.x == 0;
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) {
+            const uint32_t qrow = wave * RPW + r;
+            // units past the row end read as zero: no maximum of |x| changes, a minimum or maximum would
+            PkMinMax st;
+#pragma unroll
+            for (int j = 0; j < UPR; ++j)
+                if (!ASYMQ || lane + j * 64 < nunits) st.add8(raw[r][j]);
+            uint32_t m16;
+            float lo = 0.f, hi = 0.f;
+            if (!ASYMQ) {
+                m16 = wave_max_u32(st.absmax_bits());
+            } else {
+                st.wave_reduce();
+                m16 = st.absmax_bits();
+                lo = st.min_f32();
+                hi = st.max_f32();
+                if (m16 > 0x7C00u) lo = hi = __builtin_nanf("");  // torch's min / max of a row that holds a NaN
+            }
+            if (qrow < p.M) {  // rows past M are neither quantized nor used
+                RowQuant<ASYMQ> rq;
+                rq.init(m16, lo, hi, q_clip, q_qmax);
+                int code_sum = 0;
+#pragma unroll
+                for (int j = 0; j < UPR; ++j) {
+                    const uint32_t c = lane + j * 64;
+                    if (c < nunits) {
+                        uint32_t word = rq.quant8(raw[r][j]);
+                        if (SHIFTQ) {
+                            const uint32_t pairs = (word & 0x0F0F0F0Fu) + ((word >> 4) & 0x0F0F0F0Fu);
+                            code_sum = (int)__builtin_amdgcn_udot4(pairs, 0x01010101u, (uint32_t)code_sum, false);
+                            word ^= 0x88888888u;  // u - 8 as a signed nibble
+                        }
+                        *reinterpret_cast<uint32_t *>(xs + qrow * XSTRIDE + c * 4) = word;
+                        if (copy_out && q_out) reinterpret_cast<uint32_t *>(q_out + (uint64_t)qrow * kbytes)[c] = word;
+                    }
+                }
+                if (SHIFTQ) code_sum = wave_sum_i32(code_sum) - 8 * (int)p.K;
+                if (lane == 0) {
+                    const f16 z = SHIFTQ ? rq.z - (f16)8.0f : rq.z;
+                    srow[qrow] = f16_to_bits(rq.s);
+                    if (ASYMQ) zrow[qrow] = f16_to_bits(z);
+                    if (SHIFTQ) rsrow[qrow] = code_sum;
+                    if (copy_out && s_out) s_out[qrow] = f16_to_bits(rq.s);
+                    if (ASYMQ && copy_out && z_out) z_out[qrow] = f16_to_bits(z);
+                    if (SHIFTQ && copy_out && rs_out) rs_out[qrow] = code_sum;
+                }
+            }
+        }
+        __syncthreads();
+        // (bytes past the row end, and rows past M, are never written: the weights read as zero there, and a row's
+        // codes only reach that row's outputs)
+#pragma unroll
+        for (int u = 0; u < SEGS; ++u)
+            xp[0][u] = koff[u] != kOobOffset ? load16(xs + l16 * XSTRIDE + koff[u]) : v4u{0, 0, 0, 0};
+        if (finisher) {
+            if constexpr (MODE == 5) {
+                const v2u head = *reinterpret_cast<const v2u *>(xs + my_m * XSTRIDE);
+                rp[0].xlo = head[0];
+                rp[0].xhi = head[1] & 0xFFu;
+                rp[0].zx = (uint32_t)rint_i32((float)bits_to_f16(zrow[my_m]));
+                rp[0].sx = (float)bits_to_f16(srow[my_m]);
+                rp[0].rxl = dual_head_sum(rp[0].xlo, rp[0].xhi);
+                rp[0].rxr = (uint32_t)rsrow[my_m] - rp[0].rxl;
+            } else {
+                rp[0].s = bits_to_f16(srow[my_m]);
+                if (ASYMQ) rp[0].z = bits_to_f16(zrow[my_m]);
+                if (SHIFTQ) rp[0].rs = rsrow[my_m];
+            }
+        }
     }
 
     auto compute_tile = [&](uint32_t tile, const v4u(&w)[SEGS], uint32_t buf) {
@@ -650,14 +770,18 @@ bool launch_rows_xs(DecodeParams &p, int epi, hipStream_t stream)
     return false;
 }
 
-template <int WAVES, int SEGS, int MT = 1, bool DB = true>
+template <int WAVES, int SEGS, int MT = 1, bool DB = true, bool FUSEQ = false>
 bool launch_mfma_mode(const DecodeParams &p, int epi, hipStream_t stream)
 {
     const uint32_t ntiles = (p.N + 15) / 16;
     const dim3 grid((ntiles + p.tiles_per_wg - 1) / p.tiles_per_wg);
-#define DUQ_DEC(E) DUQ_LAUNCH_HEAD((gemm_s4_decode_kernel<WAVES, SEGS, E, MT, DB>), grid, dim3(WAVES * 64), 0, stream, p)
+#define DUQ_DEC(E) \
+    DUQ_LAUNCH_HEAD((gemm_s4_decode_kernel<WAVES, SEGS, E, MT, DB, FUSEQ>), grid, dim3(WAVES * 64), 0, stream, p)
     switch (epi) {
-    case -1: DUQ_DEC(-1); break;
+    case -1:
+        if constexpr (FUSEQ) return false;
+        else DUQ_DEC(-1);
+        break;
     case 0: DUQ_DEC(0); break;
     case 1: DUQ_DEC(1); break;
     case 2: DUQ_DEC(2); break;
@@ -680,8 +804,13 @@ bool launch_decode_any(DecodeParams &p, int epi, hipStream_t stream)
         return launch_rows_xs<4, FUSEQ>(p, epi, stream);
     }
     if constexpr (FUSEQ) {
-        if (p.M > 8) return false;
-        return launch_rows_xs<8, true>(p, epi, stream);  // 5..8 rows
+        if (p.M <= 8) return launch_rows_xs<8, true>(p, epi, stream);  // 5..8 rows
+        if (p.M > 16 || kbytes > 2048) return false;
+        // 9..16 rows: the MFMA kernel, rows quantized by every workgroup
+        constexpr int W = DUQ_DEC_MFMA_FUSEQ_WAVES;
+        p.tiles_per_wg = decode_tiles_per_workgroup((p.N + 15) / 16);
+        if (kbytes <= 1024) return launch_mfma_mode<W, 16 / W, 1, true, true>(p, epi, stream);
+        return launch_mfma_mode<W, 32 / W, 1, true, true>(p, epi, stream);
     } else {
         const uint32_t ntiles = (p.N + 15) / 16;
         p.tiles_per_wg = decode_tiles_per_workgroup(ntiles);

@@ -134,11 +134,19 @@ inline uint32_t decode_tiles_per_workgroup(uint32_t ntiles) { return (ntiles + 2
 // of at most 4096 elements, or 8192 on at most 4096 columns (the rows kernel with eight rows, one wavefront
 // quantizing each; measured against quantizer + MFMA decode kernel at 8 rows: N = K = 4096 6.3 against 7.2 us,
 // N = 11008 8.5 against 9.8, K = 2048 4.9 against 6.4, N = K = 8192 16.9 against 13.5); from two rows on only up to
-// 16384 output columns (every workgroup quantizes the rows again: measured slower than two launches beyond)
+// 16384 output columns (every workgroup quantizes the rows again: measured slower than two launches beyond).
+// 9..16 rows: the MFMA kernel with sixteen wavefronts, one quantizing each row, while the rows together hold at most
+// 32768 elements, 40960 on at most 4096 columns (measured against two launches, N = 4096: 16 rows of 2048 4.9 against
+// 6.0 us, of 1024 4.1 against 5.3, 10 of 3072 5.9 against 6.3, 9 of 4096 6.2 against 6.5; 16 of 3072 6.45 either way,
+// 16 of 4096 7.2 against 6.55: each CU then spends 2 us of vector work and 0.85 us of fetching on the rows.  16 rows
+// of 2048: N = 8192 5.9 against 6.6, N = 16384 8.4 against 8.9; 10 of 4096 on N = 11008 9.3 either way, 13 of 3072
+// on N = 11008 9.0 against 8.6).
 inline bool decode_fp16in_one_launch(uint32_t M, uint32_t N, uint32_t K)
 {
     const int kernel = select_gemm_kernel(M, N, K);
     if (kernel == kKernelDecodeRows) return M == 1 || N <= 16384;
+    if (M > 8)
+        return M <= 16 && K <= 4096 && M * K <= (N <= 4096 ? 40960u : 32768u) && N <= 16384 && kernel == kKernelDecodeMfma;
     return M <= 8 && N <= 16384 && (K <= 4096 || (K <= 8192 && N <= 4096)) && kernel == kKernelDecodeMfma;
 }
 // decode kernels (duq_decode.hip); the shape must be one select_gemm_kernel gives to them

@@ -48,7 +48,7 @@ class _Linear4bitBase(torch.nn.Module):
     def _finish(self, y):
         return y if self.bias is None else y + self.bias
 
-    # ---- decode: quantizer + GEMM + dequant as ONE launch (up to eight rows of binary16 activations) ----
+    # ---- decode: quantizer + GEMM + dequant as ONE launch (up to eight rows of binary16 activations, sixteen short ones) ----
     # _decode_spec: (epilogue mode, ((argument of _HIP.FusedDecode, buffer name), ...)) of a layer class that has a
     # one-launch form; the weight comes first.
     _decode_spec = None
@@ -79,8 +79,8 @@ class _Linear4bitBase(torch.nn.Module):
         return d
 
     def _decode_forward(self, x, clip=1.0, qmax=6, checked=False):
-        """y for binary16 rows ``x`` when the layer takes them in one library call (up to eight rows: one launch,
-        quantizer inside; up to 1024: quantizer launch + GEMM launch), else None."""
+        """y for binary16 rows ``x`` when the layer takes them in one library call (up to eight rows, or nine to sixteen
+        that hold at most 32768 elements together: one launch, quantizer inside; up to 1024: quantizer launch + GEMM launch), else None."""
         if not self.fused:
             return None
         d = self._decode_call()
@@ -332,7 +332,7 @@ class LinearQuant4bitDUASQRowSum(_Linear4bitBase):
     and each part gets the row-sum correction with its own pair:
         y = s_x * ( s_1 * corr(k < 10) + s_2 * corr(k >= 10) ),  corr = acc - z_x * (R_w - n_k * z_w) - z_w * R_x
     Codes and zero points are stored minus 8 (the signed GEMM reads them exactly), ``weight_rowsum_1/2`` hold
-    ``R_w - n_k * z_w`` of the two ranges.  The forward is one launch for up to eight rows, quantizer + GEMM with the
+    ``R_w - n_k * z_w`` of the two ranges.  The forward is one launch for up to eight rows (sixteen short ones), quantizer + GEMM with the
     epilogue inside for the shapes of the decode and prefill kernels, else quantizer, GEMM into int32, epilogue."""
 
     def __init__(self, in_features, out_features, bias=False, require_quantizer=True):

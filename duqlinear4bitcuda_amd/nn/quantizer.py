@@ -28,7 +28,7 @@ class SymQuantizer(torch.nn.Module):
     (include/common.h:53-54), 7 what its Python fake-quant path applies."""
 
     # Inputs of at most this many rows (decode) are handed on unquantized inside the PackedQuantizedTensor: a
-    # Linear4bitSQ / Linear4bitDUSQ that follows quantizes them inside its own library call (up to eight rows
+    # Linear4bitSQ / Linear4bitDUSQ that follows quantizes them inside its own library call (up to eight rows, sixteen short ones,
     # quantizer + GEMM + dequant are ONE launch; above, the quantizer launch and the GEMM launch of one call: at
     # these sizes a step costs more on the host than on the GPU, and a call less is most of it), and anything
     # else that reads quantized_x / scales_x triggers this quantizer's launch then, with the same bits.  Not for

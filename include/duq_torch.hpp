@@ -216,7 +216,7 @@ public:
     bool shadow;  // also write the 6-bit float shadow (inputs whose width is a multiple of 128)
     // defer_rows > 0 (at most 1024 is useful): inputs of at most that many rows are handed on unquantized
     // (PackedQuantizedTensor::deferred) and the linear layer behind quantizes them inside its own library call (one
-    // launch up to eight rows, the quantizer launch and the GEMM launch of one call above).  Off by default: the
+    // launch up to eight rows or sixteen short ones, the quantizer launch and the GEMM launch of one call above).  Off by default: the
     // fields quantized_x and scale of such a tensor are undefined until materialize(), and code written against the
     // reference reads them as plain members (test/test.cu:238-242).  A decode pipeline that only passes the tensor
     // on, torch::nn::Sequential(Quantizer4bit(clip, qmax, false, 64), Linear4bit) (test/pipeline.cu:107-110), turns it on.

@@ -35,6 +35,10 @@ SHAPES = [(1, 64, 64), (1, 20, 128), (2, 37, 4096), (3, 100, 2048), (4, 4096, 40
           (12, 40, 16384), (16, 24, 12352),
           # five to eight rows: from binary16 the rows kernel with eight rows (one launch), pre-quantized the MFMA kernel
           (5, 4096, 4096), (8, 11008, 4096), (6, 300, 2048), (7, 4100, 8192), (8, 16384, 64), (8, 8200, 8192), (8, 20000, 128),
+          # nine to sixteen rows of at most 32768 elements together (40960 on at most 4096 columns): from binary16 the MFMA
+          # kernel quantizes them itself
+          (16, 4090, 2048), (9, 300, 4096), (8, 11008, 4032), (12, 520, 3072), (16, 100, 2560), (13, 9000, 1984),
+          (16, 16384, 1024), (11, 4096, 3712),
           # MFMA decode kernel with two to four row tiles (17..64 rows of at most 4096 elements, 17..32 of at most
           # 8192), one to several column tiles per workgroup, tiles that end inside M and N
           (17, 4096, 4096), (32, 300, 4096), (33, 4099, 2048), (48, 1000, 4096), (64, 11008, 4096), (50, 72, 64),
@@ -100,7 +104,7 @@ def test_decode_rowsum_epilogue(hip, dev):
         assert cases.bits_equal(y.cpu().numpy(), want)
 
 
-@pytest.mark.parametrize("M", [1, 2, 4, 7])
+@pytest.mark.parametrize("M", [1, 2, 4, 7, 12, 16])
 def test_fp16_input_special_rows_and_clamps(hip, dev, M):
     """Rows of zeros, with an infinity, with a NaN, with subnormals only, clip 0.9 and both upper clamps: the
     one-launch path gives the stand-alone quantizer's codes and scales and the oracle's outputs."""

@@ -309,6 +309,9 @@ def test_asym_fp16_input_entry_point_validation_without_launch():
     assert g(1, 64, 4, 64) == 64 * 32 + 128 + 128 and g(4, 64, 4, 64) == 64 * 32 + 128 + 128 + 256
     assert g(5, 64, 4, 64) == 64 * 32 + 128 + 128 + 256 and g(5, 100, 8, 128) == 100 * 64 + 208 + 208 + 400 + 3200
     assert g(1, 8, 4096, 4096) == 0 and g(5, 8, 4096, 4096) == 0 and g(2, 64, 4, 64) == 0
+    # nine to sixteen rows are one launch while they hold at most 32768 elements together (40960 on at most 4096 columns)
+    assert g(1, 16, 4096, 2048) == 0 and g(4, 10, 4096, 4096) == 0 and g(1, 11, 4096, 4096) > 0 and g(1, 16, 20000, 2048) > 0
+    assert g(1, 16, 16384, 2048) == 0 and g(1, 10, 11008, 4096) > 0
     # the entry point that allocates nothing: slot and size limits are checked before anything else
     s = lib.duq_quantize_linear4bit_forward_static
     assert s(0, P, 1.0, 6, P, P, None, None, 8, 64, 64, P, None, None, 4, None) == -7   # no such slot
@@ -319,9 +322,9 @@ def test_asym_fp16_input_entry_point_validation_without_launch():
     # the prepared-layer form: a shape of two launches needs its workspace, checked before anything else is touched
     layer = _lib.FusedLayer(0, 1.0, 6, 4096, 4096, P, P, None, None, None, None, None, None)
     g = lib.duq_quantize_linear4bit_forward_layer
-    assert g(ctypes.addressof(layer), P, 9, P, None, 0, None) == -1 and g(None, P, 1, P, None, 0, None) == -1
-    assert g(ctypes.addressof(layer), P, 9, P, P, 100, None) == -2
-    assert g(ctypes.addressof(layer), P, 9, P, ctypes.c_void_p(4104), 1 << 20, None) == -5
+    assert g(ctypes.addressof(layer), P, 12, P, None, 0, None) == -1 and g(None, P, 1, P, None, 0, None) == -1
+    assert g(ctypes.addressof(layer), P, 12, P, P, 100, None) == -2
+    assert g(ctypes.addressof(layer), P, 12, P, ctypes.c_void_p(4104), 1 << 20, None) == -5
     assert g(ctypes.addressof(layer), P, 0, P, None, 0, None) == 0
     layer.mode = 9
     assert g(ctypes.addressof(layer), P, 1, P, None, 0, None) == -4
