@@ -325,7 +325,7 @@ def decode_section(dev, quick, eager=True):
     """HBM-bound decode at configuration 2 and around it.  Per shape, HIP-graph timed, with the weights rotated
     over more than 512 MB of distinct buffers so that no launch finds its weights in a cache:
       us            binary16 activations in -> per-token quantize -> GEMM -> fp16 out, the single entry point
-                    (one launch up to eight rows, quantizer + GEMM launches above)
+                    (one launch up to eight rows and for nine to sixteen short ones, quantizer + GEMM launches above)
       gemm_only_us  the GEMM + dequant launch alone on pre-quantized activations
       read_floor_us a kernel that only reads the same N*K/2 weight bytes with the decode access pattern
       module_graph_us  the same step through the drop-in modules, Sequential(SymQuantizer, Linear4bitSQ) on an input
@@ -344,7 +344,9 @@ def decode_section(dev, quick, eager=True):
     shapes = list(LLAMA7B_DECODE)
     if not quick:
         shapes += [(8, 4096, 4096), (32, 4096, 4096), (64, 11008, 4096), (1, 4096, 11008), (16, 4096, 11008), (1, 28672, 8192),
-                   (1, 8192, 28672), (16, 28672, 8192)]
+                   (1, 8192, 28672), (16, 28672, 8192),
+                   # sixteen rows of 2048 elements: one launch (the MFMA decode kernel quantizes the rows itself)
+                   (16, 2048, 2048), (16, 8192, 2048)]
     for (M, N, K) in shapes:
         wbytes = N * K // 2
         nbuf = min(96, max(3, int(600e6 // wbytes) + 1))
@@ -371,7 +373,7 @@ def decode_section(dev, quick, eager=True):
                     "launches": 1 if hip.quantize_linear4bit_one_launch(M, N, K) else 2,
                     "module_graph_us": round(us_mod_graph, 3), "module_eager_us": round(us_mod_eager, 3) if eager else None,
                     "module_launches": 1 if hip.quantize_linear4bit_one_launch(M, N, K) else 2,
-                    "module_library_calls": 1 if M <= 64 else 2,
+                    "module_library_calls": 1 if M <= 1024 else 2,
                     "gemm_only_us": round(us_gemm, 3),
                     "gemm_only_GBps": round((byts - 2 * M * K + M * K // 2 + 2 * M) / us_gemm / 1e3, 1),
                     "read_floor_us": round(us_read, 3), "read_floor_GBps": round(wbytes / us_read / 1e3, 1),
