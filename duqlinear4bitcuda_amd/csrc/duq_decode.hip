@@ -65,6 +65,10 @@
 #ifndef DUQ_DEC_WAVES
 #define DUQ_DEC_WAVES 8
 #endif
+// 8-element units whose quantization chains are interleaved in the kernels that quantize their rows themselves
+#ifndef DUQ_DEC_QUANT_GROUP
+#define DUQ_DEC_QUANT_GROUP 8
+#endif
 // wavefronts per workgroup of the MFMA kernel when it quantizes its 16 rows itself
 // (16 rows, N = 4096: sixteen against eight wavefronts K = 4096 7.2 against 7.9 us, K = 2048 4.9 against 5.4)
 #ifndef DUQ_DEC_MFMA_FUSEQ_WAVES
@@ -95,6 +99,24 @@ struct DecodeParams {
     int32_t *rs_out;     // FUSEQ with the row-sum epilogue, optional: the per-token sums of the shifted codes [M]
 };
 static_assert(offsetof(DecodeParams, y) + sizeof(uint16_t *) == kHeadBytes, "the fields delivered in registers");
+
+// The quantization step over N units, G at a time (RowQuant::quant_units: the path is chosen once per group and the
+// group's chains interleave; a group holds 4 G more registers than a single unit).
+template <int G, int S = 0, bool ASYM, int N>
+__device__ __forceinline__ void quant_in_groups(const RowQuant<ASYM> &rq, const v4u (&raw)[N], uint32_t (&out)[N])
+{
+    if constexpr (S < N) {
+        constexpr int L = N - S < G ? N - S : G;
+        v4u in[L];
+        uint32_t w[L];
+#pragma unroll
+        for (int j = 0; j < L; ++j) in[j] = raw[S + j];
+        rq.quant_units(in, w);
+#pragma unroll
+        for (int j = 0; j < L; ++j) out[S + j] = w[j];
+        quant_in_groups<G, S + L>(rq, raw, out);
+    }
+}
 
 template <int CTRL>
 __device__ __forceinline__ int dpp_add(int v)
@@ -323,11 +345,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_s4_rows_kernel(DUQ_HEAD_DECL,
             RowQuant<ASYMQ> rq;
             rq.init(m16, lo, hi, q_clip, q_qmax);
             const bool copy_out = blockIdx.x == 0;
+            uint32_t words[UPL];
+            quant_in_groups<(XS >= 8 ? 4 : DUQ_DEC_QUANT_GROUP)>(rq, raw, words);  // (long rows: registers)
 #pragma unroll
             for (int j = 0; j < UPL; ++j) {
                 const uint32_t c = qpart * 64 + lane + j * (64 * WPR);
                 if (c < nunits) {
-                    uint32_t word = rq.quant8(raw[j]);
+                    uint32_t word = words[j];
                     if (SHIFTQ) {
                         // eight unsigned codes: sum them, then u - 8 as a signed nibble is u with bit 3 flipped
                         const uint32_t pairs = (word & 0x0F0F0F0Fu) + ((word >> 4) & 0x0F0F0F0Fu);
@@ -586,11 +610,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_s4_decode_kernel(DUQ_HEAD_DEC
                 RowQuant<ASYMQ> rq;
                 rq.init(m16, lo, hi, q_clip, q_qmax);
                 int code_sum = 0;
+                uint32_t words[UPR];
+                quant_in_groups<DUQ_DEC_QUANT_GROUP>(rq, raw[r], words);
 #pragma unroll
                 for (int j = 0; j < UPR; ++j) {
                     const uint32_t c = lane + j * 64;
                     if (c < nunits) {
-                        uint32_t word = rq.quant8(raw[r][j]);
+                        uint32_t word = words[j];
                         if (SHIFTQ) {
                             const uint32_t pairs = (word & 0x0F0F0F0Fu) + ((word >> 4) & 0x0F0F0F0Fu);
                             code_sum = (int)__builtin_amdgcn_udot4(pairs, 0x01010101u, (uint32_t)code_sum, false);
@@ -804,7 +830,9 @@ bool launch_decode_any(DecodeParams &p, int epi, hipStream_t stream)
         return launch_rows_xs<4, FUSEQ>(p, epi, stream);
     }
     if constexpr (FUSEQ) {
+#ifndef DUQ_DEC_M8_MFMA
         if (p.M <= 8) return launch_rows_xs<8, true>(p, epi, stream);  // 5..8 rows
+#endif
         if (p.M > 16 || kbytes > 2048) return false;
         // 9..16 rows: the MFMA kernel, rows quantized by every workgroup
         constexpr int W = DUQ_DEC_MFMA_FUSEQ_WAVES;

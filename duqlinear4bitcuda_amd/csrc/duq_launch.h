@@ -145,8 +145,13 @@ inline bool decode_fp16in_one_launch(uint32_t M, uint32_t N, uint32_t K)
 {
     const int kernel = select_gemm_kernel(M, N, K);
     if (kernel == kKernelDecodeRows) return M == 1 || N <= 16384;
+#ifndef DUQ_DEC_FUSEQ16_ELEMS
+#define DUQ_DEC_FUSEQ16_ELEMS 32768u
+#define DUQ_DEC_FUSEQ16_ELEMS_NARROW 40960u
+#endif
     if (M > 8)
-        return M <= 16 && K <= 4096 && M * K <= (N <= 4096 ? 40960u : 32768u) && N <= 16384 && kernel == kKernelDecodeMfma;
+        return M <= 16 && K <= 4096 && M * K <= (N <= 4096 ? DUQ_DEC_FUSEQ16_ELEMS_NARROW : DUQ_DEC_FUSEQ16_ELEMS) && N <= 16384 &&
+               kernel == kKernelDecodeMfma;
     return M <= 8 && N <= 16384 && (K <= 4096 || (K <= 8192 && N <= 4096)) && kernel == kKernelDecodeMfma;
 }
 // decode kernels (duq_decode.hip); the shape must be one select_gemm_kernel gives to them

@@ -229,6 +229,27 @@ struct RowQuant {
         if (!ASYM && clamp_lo) return quant8_packed<true, true>(raw);
         return clamp_hi ? quant8_packed<false, true>(raw) : quant8_packed<false, false>(raw);
     }
+
+    // N units at once: the path is chosen once, so that the N independent chains of a path sit in one block of
+    // straight-line code and the scheduler can interleave them (a unit's chain is eight instructions deep).  Units
+    // a caller does not store may hold anything (zeros from loads past the row end): every path is total.
+    template <int N>
+    __device__ __forceinline__ void quant_units(const v4u (&raw)[N], uint32_t (&out)[N]) const
+    {
+        if (!fast) {
+#pragma unroll
+            for (int j = 0; j < N; ++j) out[j] = quant8_exact<ASYM>(raw[j], rcp, qmax, zi);
+        } else if (!ASYM && clamp_lo) {
+#pragma unroll
+            for (int j = 0; j < N; ++j) out[j] = quant8_packed<true, true>(raw[j]);
+        } else if (clamp_hi) {
+#pragma unroll
+            for (int j = 0; j < N; ++j) out[j] = quant8_packed<false, true>(raw[j]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < N; ++j) out[j] = quant8_packed<false, false>(raw[j]);
+        }
+    }
 };
 
 }  // namespace duq
