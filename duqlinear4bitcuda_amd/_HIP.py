@@ -623,7 +623,7 @@ class FusedDecode:
             ref = self._structs[key] = (ctypes.addressof(st), st)   # (the struct is kept alive beside its address)
         return ref[0]
 
-    # Rows up to which a module hands binary16 activations to this call.  Up to eight rows, sixteen short ones (and N <= 16384) it is one
+    # Rows up to which a module hands binary16 activations to this call.  Up to eight rows, sixteen short ones, it is one
     # launch; above, the quantizer launch and the GEMM launch of one library call: up to about 700 rows (N = K = 4096)
     # the two kernels take less time than two calls cost on the host (23 us).
     max_rows = 1024

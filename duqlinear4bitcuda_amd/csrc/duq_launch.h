@@ -132,9 +132,12 @@ inline bool decode_uses_rows_kernel(uint32_t M) { return M <= 4; }
 inline uint32_t decode_tiles_per_workgroup(uint32_t ntiles) { return (ntiles + 255) / 256; }
 // quantize + GEMM + dequant from binary16 activations in one launch: shapes of the rows kernel, and 5..8 rows
 // of at most 4096 elements, or 8192 on at most 4096 columns (the rows kernel with eight rows, one wavefront
-// quantizing each; measured against quantizer + MFMA decode kernel at 8 rows: N = K = 4096 6.3 against 7.2 us,
-// N = 11008 8.5 against 9.8, K = 2048 4.9 against 6.4, N = K = 8192 16.9 against 13.5); from two rows on only up to
-// 16384 output columns (every workgroup quantizes the rows again: measured slower than two launches beyond).
+// quantizing each; measured against quantizer + MFMA decode kernel at 8 rows: N = K = 4096 4.7 against 6.5 us,
+// N = 11008 7.2 against 9.3, N = 28672 13.0 against 16.0, N = 65536 K = 2048 18.7 against 21.5; K = 8192: N = 8192
+// 15.3 against 13.0, N = 11008 21.0 against 15.0).  Two to four rows longer than 8192 elements only up to 16384
+// output columns: every workgroup quantizes the rows again (4 rows: N = 28672 K = 8192 20.5 - 21.9 against 23.4 us,
+// N = 32000 K = 4096 12.6 against 14.1, N = 128256 K = 4096 41.3 against 42.4, but N = 20000 K = 16384 45.2 against
+// 36.3).
 // 9..16 rows: the MFMA kernel with sixteen wavefronts, one quantizing each row, while the rows together hold at most
 // 32768 elements, 40960 on at most 4096 columns (measured against two launches, N = 4096: 16 rows of 2048 4.9 against
 // 6.0 us, of 1024 4.1 against 5.3, 10 of 3072 5.9 against 6.3, 9 of 4096 6.2 against 6.5; 16 of 3072 6.45 either way,
@@ -144,7 +147,7 @@ inline uint32_t decode_tiles_per_workgroup(uint32_t ntiles) { return (ntiles + 2
 inline bool decode_fp16in_one_launch(uint32_t M, uint32_t N, uint32_t K)
 {
     const int kernel = select_gemm_kernel(M, N, K);
-    if (kernel == kKernelDecodeRows) return M == 1 || N <= 16384;
+    if (kernel == kKernelDecodeRows) return M == 1 || N <= 16384 || K <= 8192;
 #ifndef DUQ_DEC_FUSEQ16_ELEMS
 #define DUQ_DEC_FUSEQ16_ELEMS 32768u
 #define DUQ_DEC_FUSEQ16_ELEMS_NARROW 40960u
@@ -152,7 +155,7 @@ inline bool decode_fp16in_one_launch(uint32_t M, uint32_t N, uint32_t K)
     if (M > 8)
         return M <= 16 && K <= 4096 && M * K <= (N <= 4096 ? DUQ_DEC_FUSEQ16_ELEMS_NARROW : DUQ_DEC_FUSEQ16_ELEMS) && N <= 16384 &&
                kernel == kKernelDecodeMfma;
-    return M <= 8 && N <= 16384 && (K <= 4096 || (K <= 8192 && N <= 4096)) && kernel == kKernelDecodeMfma;
+    return M <= 8 && (K <= 4096 || (K <= 8192 && N <= 4096)) && kernel == kKernelDecodeMfma;
 }
 // decode kernels (duq_decode.hip); the shape must be one select_gemm_kernel gives to them
 int launch_decode_s4(const uint8_t *A, const uint8_t *B, uint32_t M, uint32_t N, uint32_t K, int32_t *out_acc,

@@ -238,8 +238,8 @@ int duq_probe_read(const void *src, uint64_t bytes, uint32_t *sink, duq_stream_t
  *   mode DUQ_EPI_SYM (w_scale_2 NULL) or DUQ_EPI_SYM_DUAL;  w, w_scale_1, w_scale_2, bias, y as duq_linear4bit_forward
  *   q_out [M,K/2] / scale_out [M]: optional (NULL): the packed codes and per-token scales, for callers that need
  *   them as well
- * Up to four rows (K <= 16384, N * K / 2 < 2^32 - 256; from two rows on N <= 16384), five to eight rows of at
- * most 4096 elements (8192 with N <= 4096) and nine to sixteen rows that hold at most 32768 elements together (40960
+ * Up to four rows (K <= 16384, N * K / 2 < 2^32 - 256; from two rows on K <= 8192 or N <= 16384), five to eight rows
+ * of at most 4096 elements (8192 with N <= 4096) and nine to sixteen rows that hold at most 32768 elements together (40960
  * with N <= 4096; K <= 4096, N <= 16384) run as ONE launch: every workgroup quantizes the rows itself while its
  * weights are in flight, and `workspace` is not touched.  Any other shape runs two launches
  * (quantizer, then GEMM) and stages the codes and scales in `workspace`, device memory of at least

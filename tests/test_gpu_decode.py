@@ -39,6 +39,9 @@ SHAPES = [(1, 64, 64), (1, 20, 128), (2, 37, 4096), (3, 100, 2048), (4, 4096, 40
           # kernel quantizes them itself
           (16, 4090, 2048), (9, 300, 4096), (8, 11008, 4032), (12, 520, 3072), (16, 100, 2560), (13, 9000, 1984),
           (16, 16384, 1024), (11, 4096, 3712),
+          # up to eight rows on more than 16384 columns: one launch from binary16 (rows of at most 8192 elements at
+          # two to four rows, of at most 4096 at five to eight)
+          (4, 20000, 8192), (2, 17000, 4096), (3, 30000, 256), (8, 20000, 4096), (5, 40000, 1024), (7, 17000, 2112),
           # MFMA decode kernel with two to four row tiles (17..64 rows of at most 4096 elements, 17..32 of at most
           # 8192), one to several column tiles per workgroup, tiles that end inside M and N
           (17, 4096, 4096), (32, 300, 4096), (33, 4099, 2048), (48, 1000, 4096), (64, 11008, 4096), (50, 72, 64),

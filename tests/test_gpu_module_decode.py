@@ -165,7 +165,8 @@ def _asym_weights(N, K, seed):
 
 @pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (4, 11008, 4096), (8, 4096, 4096), (3, 100, 2048), (2, 64, 8192),
                                     (7, 300, 1024), (4, 16000, 128), (16, 4096, 4096), (40, 1000, 1024), (64, 11008, 4096),
-                                    (12, 300, 2048), (16, 4104, 1024), (9, 520, 4096), (10, 8200, 3008)])
+                                    (12, 300, 2048), (16, 4104, 1024), (9, 520, 4096), (10, 8200, 3008),
+                                    (6, 20000, 1024), (3, 18000, 2048)])
 def test_asymmetric_layers_decode_in_one_library_call(dev, library_calls, M, N, K):
     """Linear4bitASQ, LinearQuant4bitDUASQ (qlinear4bit/nn/linear.py:104-115, 239-250) and the row-sum layer from
     binary16 rows: one library call (one launch up to eight rows and for sixteen short ones), the oracle's bits (activations ~U[0, 6] as in
@@ -281,7 +282,8 @@ def test_asym_fp16_input_two_launch_shapes_and_errors(dev):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (4, 11008, 4096), (8, 512, 2048), (3, 100, 8192), (16, 4096, 4096),
-                                    (40, 1000, 1024), (100, 1000, 512), (16, 1000, 2048), (9, 200, 4096), (12, 4500, 2560)])
+                                    (40, 1000, 1024), (100, 1000, 512), (16, 1000, 2048), (9, 200, 4096), (12, 4500, 2560),
+                                    (8, 17000, 512)])
 def test_dual_uniform_rowsum_layer_decode(dev, library_calls, M, N, K):
     """LinearQuant4bitDUASQRowSum from binary16 rows: one library call up to 1024 rows (one launch up to eight, the
     quantizer inside the rows kernel; quantizer + GEMM with the epilogue inside for the MFMA decode kernel's shapes;

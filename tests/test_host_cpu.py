@@ -284,7 +284,13 @@ def test_fp16_input_entry_point_validation_without_launch():
     assert f(0, None, 1.0, 6, None, None, None, None, 0, 4, 64, None, None, None, None, 0, None) == 0
     assert lib.duq_quantize_linear4bit_workspace_bytes(64, 4, 64) == 64 * 32 + 128
     assert lib.duq_quantize_linear4bit_workspace_bytes(4, 4096, 4096) == 0
-    assert lib.duq_quantize_linear4bit_workspace_bytes(4, 28672, 8192) == 4 * 4096 + 16
+    # two to four rows: one launch on any width up to 8192 elements, up to 16384 columns beyond
+    assert lib.duq_quantize_linear4bit_workspace_bytes(4, 28672, 8192) == 0
+    assert lib.duq_quantize_linear4bit_workspace_bytes(4, 20000, 16384) == 4 * 8192 + 16
+    assert lib.duq_quantize_linear4bit_workspace_bytes(1, 20000, 16384) == 0
+    # five to eight rows: any width up to 4096 elements, 8192 on at most 4096 columns
+    assert lib.duq_quantize_linear4bit_workspace_bytes(8, 28672, 4096) == 0
+    assert lib.duq_quantize_linear4bit_workspace_bytes(8, 4112, 8192) == 8 * 4096 + 16
 
 
 def test_asym_fp16_input_entry_point_validation_without_launch():
