@@ -84,3 +84,66 @@ def test_random_shapes_8bit(hip, dev, M, N, K):
     got = hip.linear8bit_forward(T(a), T(sr), T(zr), hip.weight_tile_8bit(T(b)), T(sc), T(zc), T(bias),
                                  tiled_rows=N).cpu().numpy()
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def _draw_decode(rng, n):
+    """Decode-sized shapes for the entry points that take binary16 rows: one launch or two depends on M, N and K
+    together, so the draws spread over all three (a few rows, narrow to very wide layers, short to long rows)."""
+    out = []
+    for i in range(n):
+        m = int(rng.integers(1, 18))
+        nn = int(np.exp(rng.uniform(np.log(8), np.log(40000))))
+        k = 64 * int(np.exp(rng.uniform(0, np.log(256))))
+        while m * nn * k > 2e9:
+            nn = max(1, nn // 2)
+        out.append((m, nn, k, i % 6))
+    return out
+
+
+SHAPES_FP16IN = _draw_decode(np.random.default_rng(2026), 42)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N,K,mode", SHAPES_FP16IN)
+def test_random_shapes_fp16_input(hip, dev, M, N, K, mode):
+    """quantizer + GEMM + dequant from binary16 rows (duq_quantize_linear4bit_forward / ..._forward_asym), every
+    epilogue mode, with a zero row and a row that holds an infinity now and then: the oracle's bits."""
+    print("fp16-in", M, N, K, "mode", mode, "one launch" if hip.quantize_linear4bit_one_launch(M, N, K) else "two", flush=True)
+    rng = np.random.default_rng(M * 13 + N * 3 + K + mode)
+    x = (cases.acts_outliers if mode in (0, 2) else cases.acts_uniform)(M, K, seed=int(rng.integers(1 << 30)))
+    if rng.random() < 0.3:
+        x[rng.integers(M)] = 0
+    if rng.random() < 0.2:
+        x[rng.integers(M), rng.integers(K)] = np.float16(np.inf)
+    wq = rng.integers(0, 256, (N, K // 2)).astype(np.uint8)
+    s1 = rng.uniform(0.001, 0.01, (N, 1)).astype(np.float16)
+    s2 = rng.uniform(0.001, 0.01, (N, 1)).astype(np.float16)
+    z1 = rng.integers(-8, 8, (N, 1)).astype(np.float16)
+    z2 = rng.integers(-8, 8, (N, 1)).astype(np.float16)
+    a1 = rng.integers(-8 * K, 8 * K, (N,)).astype(np.int32)
+    a2 = rng.integers(-8 * K, 8 * K, (N,)).astype(np.int32)
+    bias = rng.standard_normal(N).astype(np.float16) if rng.random() < 0.5 else None
+    T = lambda v: None if v is None else cases.t(v, dev)
+    X = T(x)
+    with np.errstate(invalid="ignore", over="ignore", divide="ignore"):
+        if mode == 0:
+            clip, qmax = (1.0, 6) if rng.random() < 0.6 else (0.9, 7)
+            got = hip.quantize_linear4bit_forward(X, T(wq), T(s1), None, T(bias), clip, qmax)
+            want = orc.linear4bit_sq_forward(x, wq, s1, bias, clip, qmax)[0]
+        elif mode == 2:
+            got = hip.quantize_linear4bit_forward(X, T(wq), T(s1), T(s2), T(bias))
+            want = orc.linear4bit_dusq_forward(x, wq, s1, s2, bias)[0]
+        elif mode == 1:
+            got = hip.quantize_linear4bit_forward_asym(hip.EPI_ASYM, X, T(wq), T(s1), T(z1 + 8), bias=T(bias))
+            want = orc.linear4bit_asq_forward(x, wq, s1, z1 + 8, bias)[0]
+        elif mode == 3:
+            got = hip.quantize_linear4bit_forward_asym(hip.EPI_ASYM_DUAL, X, T(wq), T(s1), T(z1 + 8), T(s2), T(z2 + 8), bias=T(bias))
+            want = orc.linear4bit_duasq_forward(x, wq, s1, z1 + 8, s2, z2 + 8, bias)[0]
+        elif mode == 4:
+            got = hip.quantize_linear4bit_forward_asym(hip.EPI_ASYM_ROWSUM, X, T(wq), T(s1), T(z1), None, None, T(a1), T(bias))
+            want = orc.linear4bit_asq_rowsum_forward(x, wq, s1, z1, a1, bias)[0]
+        else:
+            got = hip.quantize_linear4bit_forward_asym(hip.EPI_ASYM_DUAL_ROWSUM, X, T(wq), T(s1), T(z1), T(s2), T(z2), T(a1),
+                                                       T(bias), w_rowsum_adj_2=T(a2))
+            want = orc.linear4bit_duasq_rowsum_forward(x, wq, s1, z1, s2, z2, a1, a2, bias)[0]
+    assert cases.bits_equal(got.cpu().numpy().reshape(M, N), want)
